@@ -1,0 +1,214 @@
+#!/usr/bin/env python3
+"""Benchmark of the helium MI355X backend's hot path on ONE GPU.
+
+A "step" is one pass of the headline workload over one batch of synthetic, seeded input that is already
+resident in HBM when the timed region starts. Prints ONE JSON line (see README / DESIGN.md for the fields).
+The other BASELINE workloads are measured in the same run and reported under "kernels".
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--only] [--no-cpu]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "fused-GEMM TFLOP/s & permute/pointwise GB/s, % of MI355X roofline"
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+BF16_PEAK_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
+ROTATE_BYTES = 768 << 20     # rotate operand sets so repeated steps cannot live in the 256 MB Infinity Cache
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def bf16_rne(x):
+    """float32 -> bfloat16 bit patterns, round to nearest even."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+class PermuteWorkload:
+    """BASELINE config 2: bf16 N(0,1) tensors, bit-exact permutes. Algorithmic bytes = 2 * numel * 2."""
+
+    bound = "hbm"
+    unit = "GB/s"
+    dtype = "bf16"
+
+    def __init__(self, name, shape, perm, seed):
+        self.name, self.shape, self.perm, self.seed = name, shape, perm, seed
+        self.numel = int(np.prod(shape))
+        self.work = 2 * self.numel * 2  # bytes read + bytes written
+
+    def describe(self):
+        return f"{self.name}: bf16 {list(self.shape)} permute {self.perm}"
+
+    def setup(self):
+        import helium_amd as ha
+
+        rng = np.random.default_rng(self.seed)
+        self.host = bf16_rne(rng.standard_normal(size=self.shape, dtype=np.float32))
+        self.op = ha.PermuteDims(self.shape, "bf16", perm=self.perm)
+        nsets = max(2, min(16, ROTATE_BYTES // self.work + 1))
+        self.sets = []
+        for _ in range(nsets):
+            src = ha.DeviceBuffer.from_numpy(self.host)
+            dst = ha.DeviceBuffer(self.host.nbytes)
+            self.sets.append((src, dst))
+        log(f"[bench] {self.describe()} :: {self.op.description} :: {nsets} operand sets")
+
+    def step(self, stream, i):
+        src, dst = self.sets[i % len(self.sets)]
+        self.op.execute(src, dst, stream)
+
+    def check(self):
+        from oracle import permute as oracle
+
+        src, dst = self.sets[0]
+        got = dst.to_numpy(np.uint16, self.op.out_shape)
+        want = oracle.permute(self.host, self.perm)
+        if not np.array_equal(got, want):
+            raise SystemExit(f"[bench] PARITY FAILURE in {self.name}: output differs from the oracle")
+        return "bit-exact vs numpy oracle"
+
+    def cpu_baseline(self, budget_s=10.0):
+        from oracle import permute as oracle
+
+        oracle.permute(self.host, self.perm)
+        best, reps, t_all = 1e30, 0, time.perf_counter()
+        while reps < 3 or (time.perf_counter() - t_all < budget_s and reps < 20):
+            t0 = time.perf_counter()
+            oracle.permute(self.host, self.perm)
+            best = min(best, time.perf_counter() - t0)
+            reps += 1
+        return {"value": round(self.work / best / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"full {self.name} tensor, numpy transpose+copy (oracle), best of {reps} passes"}
+
+    def free(self):
+        for s, d in self.sets:
+            s.free()
+            d.free()
+        self.sets = []
+
+
+def make_workloads():
+    w = {
+        "C2a": PermuteWorkload("C2a", (64, 56, 56, 256), (0, 3, 1, 2), 21),
+        "C2b": PermuteWorkload("C2b", (4096, 4096), (1, 0), 22),
+        "C2c": PermuteWorkload("C2c", (32, 128, 28, 28), (0, 2, 3, 1), 23),
+    }
+    try:
+        import bench_workloads  # optional: further workloads (pointwise chain, fused GEMM) register here
+
+        bench_workloads.register(w)
+    except ImportError:
+        pass
+    return w
+
+
+def time_workload(wl, stream, steps, warmup):
+    """Returns (ms_per_step from HIP events on the launch stream, wall ms per step)."""
+    import helium_amd as ha
+
+    for i in range(warmup):
+        wl.step(stream, i)
+    stream.synchronize()
+    ha.device.synchronize()
+    start, stop = ha.Event(), ha.Event()
+    t0 = time.perf_counter()
+    start.record(stream)
+    for i in range(steps):
+        wl.step(stream, warmup + i)
+    stop.record(stream)
+    stop.synchronize()
+    ha.device.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    return start.elapsed_ms(stop) / steps, wall_ms
+
+
+def roofline(wl, ms):
+    if wl.bound == "hbm":
+        achieved = wl.work / (ms * 1e-3) / 1e9
+        peak, unit = HBM_PEAK_GBS, "GB/s"
+    else:
+        achieved = wl.work / (ms * 1e-3) / 1e12
+        peak, unit = BF16_PEAK_TFLOPS, "TFLOP/s"
+    return {"bound": wl.bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
+            "frac": round(achieved / peak, 4), "traffic": getattr(wl, "traffic", None)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default=None, help="headline workload (default: the best-covered BASELINE config)")
+    ap.add_argument("--only", action="store_true", help="measure the headline workload only")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import helium_amd as ha
+
+    ha.device.init(0)
+    arch = ha.device.device_arch(0)
+    cus = ha.device.device_attr(0)
+    log(f"[bench] device 0: {arch}, {cus} CUs; roofline constants: HBM {HBM_PEAK_GBS} GB/s, "
+        f"bf16 MFMA {BF16_PEAK_TFLOPS} TFLOP/s")
+    workloads = make_workloads()
+    headline = args.workload or getattr(sys.modules.get("bench_workloads"), "HEADLINE", "C2a")
+    if headline not in workloads:
+        raise SystemExit(f"unknown workload {headline}; have {sorted(workloads)}")
+    stream = ha.Stream()
+
+    kernels = {}
+    head = None
+    order = [headline] + ([] if args.only else [k for k in workloads if k != headline])
+    for name in order:
+        wl = workloads[name]
+        wl.setup()
+        wl.step(stream, 0)
+        stream.synchronize()
+        parity = wl.check()
+        ms, wall = time_workload(wl, stream, args.steps, args.warmup)
+        rl = roofline(wl, ms)
+        kernels[name] = {"workload": wl.describe(), "ms": round(ms, 5), "wall_ms": round(wall, 5), "parity": parity,
+                         "roofline": rl}
+        log(f"[bench] {name}: {ms * 1e3:.1f} us/step -> {rl['achieved']} {rl['unit']} ({rl['frac'] * 100:.1f}% of peak)")
+        if name == headline:
+            cpu = None if args.no_cpu else wl.cpu_baseline()
+            head = (wl, ms, rl, cpu)
+        wl.free()
+
+    wl, ms, rl, cpu = head
+    line = {
+        "metric": METRIC,
+        "value": rl["achieved"],
+        "unit": rl["unit"],
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": wl.dtype,
+        "data": "synthetic",
+        "config": {"workload": wl.describe(), "device": arch, "cus": cus,
+                   "host_cores": os.cpu_count()},
+        "roofline": rl,
+        "cpu_baseline": cpu,
+        "kernels": kernels,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

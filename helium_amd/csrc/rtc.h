@@ -1,0 +1,46 @@
+// hiprtc compilation with a memory + disk cache, and a loaded-kernel wrapper
+// (the counterpart of KernelBuilder::build_ptx / JitKernel in helium/src/cuda/kernel_jit.rs).
+#pragma once
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "common.h"
+
+namespace he {
+
+// Compiles HIP source for gfx950. Cached by (source, options): in memory, and as a code-object file under the
+// cache directory (HELIUM_HIP_CACHE_DIR, default <library dir>/_kcache) when that directory is usable.
+std::shared_ptr<const std::vector<char>> rtc_compile(const std::string& source, const std::string& name,
+                                                     const std::vector<std::string>& extra_options);
+void rtc_stats(uint64_t stats[3]);
+
+// Flags every generated kernel is compiled with.
+std::vector<std::string> default_kernel_options();
+
+// A compiled kernel: code object + entry name. The module is loaded lazily on first launch (so that
+// generation and compilation work on a machine without a GPU) and kept for the life of the object.
+class JitKernel {
+public:
+    JitKernel(std::string source, std::string entry, std::vector<std::string> options = {});
+    ~JitKernel();
+    JitKernel(const JitKernel&) = delete;
+    JitKernel& operator=(const JitKernel&) = delete;
+
+    const std::string& source() const { return source_; }
+    const std::string& entry() const { return entry_; }
+    void launch(const uint32_t grid[3], const uint32_t block[3], uint32_t lds_bytes, hipStream_t stream,
+                void** args);
+    // Number of scratch bytes per lane the compiler reported (0 == no spills); -1 before the module is loaded.
+    int private_bytes();
+    int vgprs();
+
+private:
+    void ensure_loaded();
+    std::string source_, entry_;
+    std::shared_ptr<const std::vector<char>> code_;
+    hipModule_t module_ = nullptr;
+    hipFunction_t func_ = nullptr;
+};
+
+}  // namespace he

@@ -1,0 +1,101 @@
+"""Runs a generated HIP kernel on the CPU for bounds and index checking (host AddressSanitizer).
+
+The kernel text is compiled as host C++ behind a small shim: every GPU thread of a block is an OS thread,
+__syncthreads() is a pthread barrier, __shared__ variables are function-static, blocks run one after another.
+Operand buffers are heap allocations of exactly the tensor's size, so any out-of-bounds access of the kernel's
+index arithmetic aborts the run. Only kernels without wave intrinsics can run this way.
+"""
+import os
+import subprocess
+import tempfile
+
+import numpy as np
+
+CLANG = "/opt/rocm/lib/llvm/bin/clang++"
+
+SHIM = r"""
+#include <pthread.h>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <utility>
+#include <vector>
+struct Dim3 { unsigned x = 0, y = 0, z = 0; };
+static thread_local Dim3 threadIdx, blockIdx;
+static Dim3 blockDim, gridDim;
+static pthread_barrier_t g_bar;
+#define __global__
+#define __device__
+#define __forceinline__ inline
+#define __launch_bounds__(...)
+#define __shared__ static
+#define __restrict__
+#define __syncthreads() pthread_barrier_wait(&g_bar)
+#define __builtin_nontemporal_load(p) (*(p))
+#define __builtin_nontemporal_store(v, p) (*(p) = (v))
+"""
+
+MAIN = r"""
+template <class... A, size_t... I>
+static void call_impl(void (*f)(A...), void** b, std::index_sequence<I...>) { f((A)b[I]...); }
+template <class... A>
+static void call(void (*f)(A...), void** b) { call_impl(f, b, std::index_sequence_for<A...>{}); }
+static void** g_bufs;
+static void* worker(void* arg) {
+    unsigned tid = (unsigned)(size_t)arg;
+    threadIdx.x = tid;
+    for (unsigned b = 0; b < gridDim.x; b++) {
+        blockIdx.x = b;
+        call(&ENTRY, g_bufs);
+        pthread_barrier_wait(&g_bar);
+    }
+    return nullptr;
+}
+int main(int argc, char** argv) {
+    // argv: grid threads (path bytes is_output)...
+    gridDim.x = atoi(argv[1]); blockDim.x = atoi(argv[2]);
+    int nb = (argc - 3) / 3;
+    std::vector<void*> bufs(nb); std::vector<size_t> sizes(nb); std::vector<int> isout(nb);
+    for (int i = 0; i < nb; i++) {
+        sizes[i] = strtoull(argv[4 + 3 * i], nullptr, 10); isout[i] = atoi(argv[5 + 3 * i]);
+        bufs[i] = malloc(sizes[i] ? sizes[i] : 1);
+        if (!isout[i]) { FILE* f = fopen(argv[3 + 3 * i], "rb"); if (fread(bufs[i], 1, sizes[i], f) != sizes[i]) return 3; fclose(f); }
+        else memset(bufs[i], 0xEE, sizes[i]);
+    }
+    g_bufs = bufs.data();
+    pthread_barrier_init(&g_bar, nullptr, blockDim.x);
+    std::vector<pthread_t> th(blockDim.x);
+    for (unsigned t = 0; t < blockDim.x; t++) pthread_create(&th[t], nullptr, worker, (void*)(size_t)t);
+    for (auto& t : th) pthread_join(t, nullptr);
+    for (int i = 0; i < nb; i++) if (isout[i]) { FILE* f = fopen(argv[3 + 3 * i], "wb"); fwrite(bufs[i], 1, sizes[i], f); fclose(f); }
+    for (auto p : bufs) free(p);
+    return 0;
+}
+"""
+
+
+def run_kernel(source, entry, grid, threads, buffers):
+    """buffers: list of (numpy array, is_output). Returns the output arrays (same dtype/shape as given)."""
+    with tempfile.TemporaryDirectory() as d:
+        src = os.path.join(d, "k.cpp")
+        with open(src, "w") as f:
+            f.write(SHIM + source + f"\n#define ENTRY {entry}\n" + MAIN)
+        exe = os.path.join(d, "k")
+        subprocess.check_call([CLANG, "-O1", "-g", "-std=c++17", "-fsanitize=address", "-fno-omit-frame-pointer",
+                               "-pthread", src, "-o", exe])
+        argv = [exe, str(grid), str(threads)]
+        paths = []
+        for i, (a, is_out) in enumerate(buffers):
+            p = os.path.join(d, f"b{i}.bin")
+            paths.append(p)
+            if not is_out:
+                np.ascontiguousarray(a).tofile(p)
+            argv += [p, str(a.nbytes), "1" if is_out else "0"]
+        res = subprocess.run(argv, capture_output=True, text=True, env={**os.environ, "ASAN_OPTIONS": "detect_leaks=0"})
+        if res.returncode != 0:
+            raise AssertionError(f"CPU emulation of {entry} failed (exit {res.returncode}):\n{res.stderr[-4000:]}")
+        outs = []
+        for p, (a, is_out) in zip(paths, buffers):
+            if is_out:
+                outs.append(np.fromfile(p, dtype=a.dtype).reshape(a.shape))
+        return outs
