@@ -1,0 +1,528 @@
+// HIP source emission for tile programs: the shared expression emitter and the pointwise/reduction kernel.
+#include <cmath>
+#include <cstring>
+#include <sstream>
+
+#include "tp.h"
+
+namespace he::tp {
+
+const char* c_type(int dtype) {
+    switch (dtype) {
+        case HE_F16: return "f16_t";
+        case HE_BF16: return "bf16_t";
+        case HE_F32: return "float";
+        case HE_U32: return "u32";
+        case HE_BOOL: return "u32";
+    }
+    return "?";
+}
+
+static const char* cls_type(Cls c) { return c == Cls::F ? "float" : c == Cls::I ? "u32" : "bool"; }
+
+// Types, vector loads/stores with conversion, wave/block reductions, float atomics.
+static const char* kPrelude = R"HIP(
+typedef unsigned short u16;
+typedef unsigned int u32;
+typedef unsigned long long u64;
+typedef __bf16 bf16_t;
+typedef _Float16 f16_t;
+template <class T, int N> struct Vec { typedef T type __attribute__((ext_vector_type(N))); };
+template <class T> struct Vec<T, 1> { typedef T type; };
+
+template <int NV> __device__ __forceinline__ void ld_vec(const float* p, float (&e)[NV]) {
+    typedef typename Vec<float, NV>::type V;
+    V v = *(const V*)p;
+    if constexpr (NV == 1) e[0] = v; else
+#pragma unroll
+    for (int k = 0; k < NV; k++) e[k] = v[k];
+}
+template <int NV> __device__ __forceinline__ void ld_vec(const u32* p, u32 (&e)[NV]) {
+    typedef typename Vec<u32, NV>::type V;
+    V v = *(const V*)p;
+    if constexpr (NV == 1) e[0] = v; else
+#pragma unroll
+    for (int k = 0; k < NV; k++) e[k] = v[k];
+}
+template <int NV> __device__ __forceinline__ void ld_vec(const bf16_t* p, float (&e)[NV]) {
+    typedef typename Vec<u16, NV>::type V;
+    V v = *(const V*)p;
+    if constexpr (NV == 1) e[0] = __builtin_bit_cast(float, (u32)v << 16); else
+#pragma unroll
+    for (int k = 0; k < NV; k++) e[k] = __builtin_bit_cast(float, (u32)v[k] << 16);
+}
+template <int NV> __device__ __forceinline__ void ld_vec(const f16_t* p, float (&e)[NV]) {
+    typedef typename Vec<f16_t, NV>::type V;
+    V v = *(const V*)p;
+    if constexpr (NV == 1) e[0] = (float)v; else
+#pragma unroll
+    for (int k = 0; k < NV; k++) e[k] = (float)v[k];
+}
+__device__ __forceinline__ float ld_one(const float* p) { return *p; }
+__device__ __forceinline__ u32 ld_one(const u32* p) { return *p; }
+__device__ __forceinline__ float ld_one(const bf16_t* p) { return __builtin_bit_cast(float, (u32)(*(const u16*)p) << 16); }
+__device__ __forceinline__ float ld_one(const f16_t* p) { return (float)*p; }
+
+template <int NV> __device__ __forceinline__ void st_vec(float* p, const float (&e)[NV]) {
+    typedef typename Vec<float, NV>::type V;
+    V v;
+    if constexpr (NV == 1) v = e[0]; else
+#pragma unroll
+    for (int k = 0; k < NV; k++) v[k] = e[k];
+    *(V*)p = v;
+}
+template <int NV> __device__ __forceinline__ void st_vec(u32* p, const u32 (&e)[NV]) {
+    typedef typename Vec<u32, NV>::type V;
+    V v;
+    if constexpr (NV == 1) v = e[0]; else
+#pragma unroll
+    for (int k = 0; k < NV; k++) v[k] = e[k];
+    *(V*)p = v;
+}
+template <int NV> __device__ __forceinline__ void st_vec(bf16_t* p, const float (&e)[NV]) {
+    typedef typename Vec<bf16_t, NV>::type V;
+    V v;
+    if constexpr (NV == 1) v = (bf16_t)e[0]; else
+#pragma unroll
+    for (int k = 0; k < NV; k++) v[k] = (bf16_t)e[k];   // round to nearest even
+    *(V*)p = v;
+}
+template <int NV> __device__ __forceinline__ void st_vec(f16_t* p, const float (&e)[NV]) {
+    typedef typename Vec<f16_t, NV>::type V;
+    V v;
+    if constexpr (NV == 1) v = (f16_t)e[0]; else
+#pragma unroll
+    for (int k = 0; k < NV; k++) v[k] = (f16_t)e[k];
+    *(V*)p = v;
+}
+__device__ __forceinline__ void st_one(float* p, float v) { *p = v; }
+__device__ __forceinline__ void st_one(u32* p, u32 v) { *p = v; }
+__device__ __forceinline__ void st_one(bf16_t* p, float v) { *p = (bf16_t)v; }
+__device__ __forceinline__ void st_one(f16_t* p, float v) { *p = (f16_t)v; }
+
+// Reduction operators: 0 Sum, 1 Mean (terms are pre-scaled), 2 Max, 3 Min.
+template <int OP> __device__ __forceinline__ float red_op(float a, float b) {
+    if constexpr (OP == 2) return fmaxf(a, b);
+    else if constexpr (OP == 3) return fminf(a, b);
+    else return a + b;
+}
+template <int OP> __device__ __forceinline__ float red_identity() {
+    if constexpr (OP == 2) return -__builtin_huge_valf();
+    else if constexpr (OP == 3) return __builtin_huge_valf();
+    else return 0.0f;
+}
+// Butterfly over the `WIDTH` consecutive lanes a value's group occupies (WIDTH a power of two <= 64).
+template <int OP, int WIDTH> __device__ __forceinline__ float wave_reduce(float v) {
+#pragma unroll
+    for (int off = WIDTH / 2; off > 0; off /= 2) v = red_op<OP>(v, __shfl_xor(v, off, 64));
+    return v;
+}
+template <int OP> __device__ __forceinline__ void atomic_red(float* addr, float v) {
+    if constexpr (OP == 2) {
+        // float max through integer atomics, split by sign (helium/src/cuda/instr/pointwise/jit.rs:40-56)
+        if (v >= 0) atomicMax((int*)addr, __float_as_int(v)); else atomicMin((unsigned int*)addr, __float_as_uint(v));
+    } else if constexpr (OP == 3) {
+        if (v >= 0) atomicMin((int*)addr, __float_as_int(v)); else atomicMax((unsigned int*)addr, __float_as_uint(v));
+    } else {
+        atomicAdd(addr, v);
+    }
+}
+__device__ __forceinline__ float fast_tanh(float x) {
+    float t = __expf(2.0f * x);
+    return 1.0f - __fdividef(2.0f, t + 1.0f);
+}
+)HIP";
+
+std::string emit_prelude(const Program&) { return kPrelude; }
+
+static std::string f32_literal(uint32_t bits) {
+    // Bit-exact constants, as the reference prints them (jit.rs:697-702).
+    return strfmt("__builtin_bit_cast(float, 0x%08xu)", bits);
+}
+
+static std::string unary_expr(const Expr& e, const std::string& x, bool fast) {
+    float cf;
+    memcpy(&cf, &e.bits, 4);
+    std::string c = f32_literal(e.bits);
+    switch ((UOp)e.op) {
+        case UOp::Recip: return fast ? "__fdividef(1.0f, " + x + ")" : "1.0f / " + x;
+        case UOp::Neg: return "-" + x;
+        case UOp::Exp: return (fast ? "__expf(" : "expf(") + x + ")";
+        case UOp::Sin: return (fast ? "__sinf(" : "sinf(") + x + ")";
+        case UOp::Cos: return (fast ? "__cosf(" : "cosf(") + x + ")";
+        case UOp::Tan: return (fast ? "__tanf(" : "tanf(") + x + ")";
+        case UOp::Sigmoid:
+            return fast ? "__fdividef(1.0f, 1.0f + __expf(-" + x + "))" : "1.0f / (1.0f + expf(-" + x + "))";
+        case UOp::Tanh: return (fast ? "fast_tanh(" : "tanhf(") + x + ")";
+        case UOp::Relu: return "fmaxf(" + x + ", 0.0f)";
+        case UOp::Sqrt: return (fast ? "__fsqrt_rn(" : "sqrtf(") + x + ")";
+        case UOp::Log: return (fast ? "__logf(" : "logf(") + x + ")";
+        case UOp::Gelu: return "0.5f * " + x + " * (1.0f + erff(" + x + " * 0.70710678118654752f))";
+        case UOp::AddC: return x + " + " + c;
+        case UOp::MulC: return x + " * " + c;
+        case UOp::PowC:
+            // x*x for an exponent of exactly 2, as the reference's generator special-cases
+            // (helium-playground/src/kernel_generator.rs:383-391); x**c otherwise (torch_synthesizer.rs:55).
+            if (cf == 2.0f) return x + " * " + x;
+            return (fast ? "__powf(" : "powf(") + x + ", " + c + ")";
+    }
+    fail(HE_ERR_INTERNAL, "bad unary op");
+}
+
+static std::string binary_expr(const Expr& e, Cls cls, const std::string& a, const std::string& b, bool fast) {
+    switch ((BOp)e.op) {
+        case BOp::Add: return cls == Cls::B ? a + " != " + b : a + " + " + b;
+        case BOp::Sub: return a + " - " + b;
+        case BOp::Mul: return cls == Cls::B ? a + " && " + b : a + " * " + b;
+        case BOp::Div: return fast ? "__fdividef(" + a + ", " + b + ")" : a + " / " + b;
+        case BOp::Pow: return (fast ? "__powf(" : "powf(") + a + ", " + b + ")";
+        case BOp::Min: return cls == Cls::F ? "fminf(" + a + ", " + b + ")" : "(" + a + " < " + b + " ? " + a + " : " + b + ")";
+        case BOp::Max: return cls == Cls::F ? "fmaxf(" + a + ", " + b + ")" : "(" + a + " > " + b + " ? " + a + " : " + b + ")";
+        case BOp::And: return cls == Cls::B ? a + " && " + b : a + " & " + b;
+        case BOp::Or: return cls == Cls::B ? a + " || " + b : a + " | " + b;
+        case BOp::Xor: return cls == Cls::B ? a + " != " + b : a + " ^ " + b;
+        case BOp::Drelu: return "(" + b + " > 0.0f) ? " + a + " : 0.0f";
+    }
+    fail(HE_ERR_INTERNAL, "bad binary op");
+}
+
+static const char* compare_sym(int op) {
+    static const char* s[] = {"==", "!=", "<", "<=", ">", ">="};
+    HE_REQUIRE(op >= 0 && op < 6, HE_ERR_INVALID, "bad compare op");
+    return s[op];
+}
+
+// One generic index map applied to the u32 variable `lin` (jit.rs:807-906).
+static void emit_generic_map(std::ostringstream& s, const GenericMap& g) {
+    if (g.kind == GenericMap::Swap) {
+        Shape out = g.in_shape;
+        std::swap(out[g.axis_a], out[g.axis_b]);
+        const int n = (int)out.size();
+        s << "{ u32 in_index = 0;";
+        int64_t ostride = 1;
+        for (int i = n - 1; i >= 0; i--) {
+            s << " u32 c" << i << " = (lin / " << ostride << "u) % " << out[i] << "u;";
+            ostride *= out[i];
+        }
+        int64_t istride = 1;
+        for (int j = n - 1; j >= 0; j--) {
+            int k = j == g.axis_a ? (int)g.axis_b : j == g.axis_b ? (int)g.axis_a : j;
+            s << " in_index += c" << k << " * " << istride << "u;";
+            istride *= g.in_shape[j];
+        }
+        s << " lin = in_index; }";
+    } else {
+        const int n = (int)g.out_shape.size(), r = (int)g.in_shape.size();
+        s << "{ u32 in_index = 0;";
+        int64_t ostride = 1, istride = 1;
+        for (int i = 0; i < n; i++) {  // i counts dims from the last
+            int od = n - 1 - i, id = r - 1 - i;
+            s << " u32 co" << i << " = (lin / " << ostride << "u) % " << g.out_shape[od] << "u;";
+            ostride *= g.out_shape[od];
+            bool zero = id < 0 || g.bcast[od];
+            if (!zero) s << " in_index += co" << i << " * " << istride << "u;";
+            istride *= id >= 0 ? g.in_shape[id] : 1;
+        }
+        s << " lin = in_index; }";
+    }
+}
+
+int pick_nv(const Program& p, int max_bytes) {
+    const int n = (int)p.dims.size();
+    const int64_t N = p.N();
+    int widest = 1;  // bytes of the widest element moved along full rows
+    auto consider = [&](int dtype) {
+        if (dtype != HE_BOOL) widest = std::max(widest, (int)dtype_bits(dtype) / 8);
+    };
+    for (auto& e : p.exprs)
+        if (e.kind == Expr::Load && e.access.chain.empty() && e.access.stride[n - 1] == 1) consider(e.access.dtype);
+    for (auto& o : p.outs)
+        if (!o.reduce) consider(o.dtype);
+    if (p.acc_expr >= 0) widest = std::max(widest, 4);
+    int nv = std::max(1, max_bytes / widest);
+    auto ok = [&](int v) {
+        if (N % v) return false;
+        for (auto& e : p.exprs) {
+            if (e.kind != Expr::Load || !e.access.chain.empty()) continue;
+            if (e.access.stride[n - 1] != 1) continue;
+            if (e.access.dtype == HE_BOOL) return false;
+            for (int d = 0; d + 1 < n; d++)
+                if (e.access.stride[d] % v) return false;
+        }
+        for (auto& o : p.outs)
+            if (!o.reduce && o.dtype == HE_BOOL) return false;
+        return true;
+    };
+    while (nv > 1 && !ok(nv)) nv /= 2;
+    return nv;
+}
+
+std::string emit_exprs(const Program& p, const EmitCtx& cx) {
+    const int n = (int)p.dims.size();
+    const int NV = cx.nv;
+    std::ostringstream s;
+    auto coord_sum = [&](const std::vector<int64_t>& stride) {
+        // Linear index of the first of the NV columns.
+        std::ostringstream o;
+        o << "(size_t)0";
+        for (int d = 0; d < n; d++) {
+            if (stride[d] == 0 || p.dims[d] <= 1) continue;
+            std::string c = d == n - 1 ? "n0" : d == n - 2 ? "m" : "cB" + std::to_string(d);
+            o << " + (size_t)" << c << " * " << stride[d] << "ull";
+        }
+        return o.str();
+    };
+    for (size_t i = 0; i < p.exprs.size(); i++) {
+        const Expr& e = p.exprs[i];
+        const std::string v = "e" + std::to_string(i);
+        const char* T = cls_type(e.cls);
+        auto each = [&](const std::string& rhs_k) {
+            s << T << " " << v << "[" << NV << "];\n#pragma unroll\nfor (int k = 0; k < " << NV << "; k++) " << v
+              << "[k] = " << rhs_k << ";\n";
+        };
+        auto ref = [&](int id) { return "e" + std::to_string(id) + "[k]"; };
+        switch (e.kind) {
+            case Expr::Load: {
+                const Access& a = e.access;
+                const int64_t sn = p.dims[n - 1] > 1 ? a.stride[n - 1] : 0;
+                const std::string ptr = "a" + std::to_string(a.arg);
+                s << T << " " << v << "[" << NV << "];\n{ const size_t o = " << coord_sum(a.stride) << ";\n";
+                if (!a.chain.empty()) {
+                    s << "#pragma unroll\nfor (int k = 0; k < " << NV << "; k++) { u32 lin = (u32)(o + (size_t)k * " << sn
+                      << "ull);\n";
+                    for (auto& g : a.chain) emit_generic_map(s, g);
+                    if (a.dtype == HE_BOOL)
+                        s << "\n" << v << "[k] = ((" << ptr << "[lin >> 5] >> (lin & 31u)) & 1u) != 0; }\n";
+                    else
+                        s << "\n" << v << "[k] = ld_one(" << ptr << " + lin); }\n";
+                } else if (a.dtype == HE_BOOL) {
+                    s << "#pragma unroll\nfor (int k = 0; k < " << NV << "; k++) { const size_t l = o + (size_t)k * " << sn
+                      << "ull; " << v << "[k] = ((" << ptr << "[l >> 5] >> (l & 31)) & 1u) != 0; }\n";
+                } else if (sn == 1 && NV > 1) {
+                    s << "ld_vec<" << NV << ">(" << ptr << " + o, " << v << ");\n";
+                } else if (sn == 0) {
+                    s << "const " << T << " t = ld_one(" << ptr << " + o);\n#pragma unroll\nfor (int k = 0; k < " << NV
+                      << "; k++) " << v << "[k] = t;\n";
+                } else {
+                    s << "#pragma unroll\nfor (int k = 0; k < " << NV << "; k++) " << v << "[k] = ld_one(" << ptr
+                      << " + o + (size_t)k * " << sn << "ull);\n";
+                }
+                s << "}\n";
+                break;
+            }
+            case Expr::Acc: each("acc[k]"); break;
+            case Expr::Const:
+                if (e.cls == Cls::F) each(f32_literal(e.bits));
+                else if (e.cls == Cls::I) each(strfmt("0x%xu", e.bits));
+                else each(e.bits ? "true" : "false");
+                break;
+            case Expr::Unary: each(unary_expr(e, ref(e.a), p.fast_math)); break;
+            case Expr::Binary: each(binary_expr(e, e.cls, ref(e.a), ref(e.b), p.fast_math)); break;
+            case Expr::Compare: each(ref(e.a) + " " + compare_sym(e.op) + " " + ref(e.b)); break;
+            case Expr::Select: each(ref(e.c) + " ? " + ref(e.b) + " : " + ref(e.a)); break;  // rhs when true (jit.rs:583-586)
+            case Expr::Cast: {
+                Cls from = p.exprs[e.a].cls;
+                std::string x = ref(e.a);
+                if (from == Cls::F && e.cls == Cls::B) each(x + " != 0.0f");
+                else if (from == Cls::B && e.cls == Cls::F) each(x + " ? 1.0f : 0.0f");
+                else if (from == Cls::F && e.cls == Cls::I) each("(u32)" + x);
+                else if (from == Cls::I && e.cls == Cls::F) each("(float)" + x);
+                else if (from == Cls::B && e.cls == Cls::I) each(x + " ? 1u : 0u");
+                else if (from == Cls::I && e.cls == Cls::B) each(x + " != 0u");
+                else fail(HE_ERR_INTERNAL, "cast within one data class");
+                break;
+            }
+        }
+    }
+    return s.str();
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Pointwise / reduction kernel.
+//
+// The iteration space is viewed as [B][M][N]. A block of 256 threads owns one b, TR = TY*RPT rows and
+// TC = TX*NV columns; a thread owns NV consecutive columns (one 16-byte access per operand) and walks RPT rows.
+//   * reductions that keep the row (fold N only) finish per row: butterfly over the row's TX lanes, then one
+//     store or atomic per row segment;
+//   * reductions that keep the column (fold M only) accumulate NV partial sums per thread over its rows, are
+//     combined across the block's TY row-groups through LDS and issue one atomic per column per block;
+//   * reductions that fold both accumulate one scalar per thread, reduced per wave (shuffles), per block (LDS)
+//     and finished with one atomic per block.
+// ---------------------------------------------------------------------------------------------------------
+static int pow2_ceil(int64_t x) {
+    int p = 1;
+    while (p < x) p *= 2;
+    return p;
+}
+
+PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
+    HE_REQUIRE(p.acc_expr < 0, HE_ERR_INVALID, "program reads a GEMM accumulator");
+    const int n = (int)p.dims.size();
+    const int64_t N = p.N(), M = p.M(), B = p.B();
+    HE_REQUIRE(ir::num_elements(p.dims) < (1ll << 32), HE_ERR_INVALID, "pointwise kernels index with 32 bits");
+    PointwiseLaunch L;
+    L.entry = entry;
+    if (ir::num_elements(p.dims) == 0) {
+        L.grid = 0;
+        L.source = "";
+        return L;
+    }
+    const int NV = pick_nv(p, 16);
+    const int threads = 256;
+    int TX = (int)std::min<int64_t>(threads, pow2_ceil((N + NV - 1) / NV));
+    int TY = threads / TX;
+    const int64_t gx = (N + (int64_t)TX * NV - 1) / ((int64_t)TX * NV);
+    const int64_t gy1 = (M + TY - 1) / TY;
+    int64_t blocks1 = gx * gy1 * B;
+    int RPT = 1;
+    if (const char* env = getenv("HELIUM_HIP_POINTWISE_RPT")) {
+        RPT = std::max(1, atoi(env));
+    } else {
+        while (RPT < 16 && blocks1 / (RPT * 2) >= 2048) RPT *= 2;
+    }
+    RPT = (int)std::min<int64_t>(RPT, std::max<int64_t>(1, gy1));
+    const int TR = TY * RPT;
+    const int64_t gy = (M + TR - 1) / TR;
+    const int64_t grid = gx * gy * B;
+    HE_REQUIRE(grid < (1ll << 31), HE_ERR_INVALID, "pointwise grid too large");
+    L.grid = (uint32_t)grid;
+    L.threads = threads;
+    L.nv = NV;
+    L.tx = TX;
+    L.ty = TY;
+    L.rpt = RPT;
+    L.options = {p.fast_math ? "-ffp-contract=fast" : "-ffp-contract=off", "-munsafe-fp-atomics"};
+
+    bool any_col = false, any_scalar = false;
+    for (auto& o : p.outs) {
+        if (!o.reduce) continue;
+        if (o.fold_m && !o.fold_n) any_col = true;
+        if (o.fold_m && o.fold_n) any_scalar = true;
+    }
+
+    std::ostringstream s;
+    s << "// pointwise kernel generated for gfx950: dims=[";
+    for (int d = 0; d < n; d++) s << (d ? "," : "") << p.dims[d];
+    s << "] NV=" << NV << " TX=" << TX << " TY=" << TY << " RPT=" << RPT << "\n";
+    s << kPrelude;
+    s << "#define NV " << NV << "\n#define TX " << TX << "\n#define TY " << TY << "\n#define RPT " << RPT
+      << "\n#define TR " << TR << "\n#define DIM_N " << N << "u\n#define DIM_M " << M << "u\n";
+    s << "extern \"C\" __global__ __launch_bounds__(" << threads << ") void " << entry << "(";
+    for (size_t a = 0; a < p.args.size(); a++)
+        s << (a ? ", " : "") << (p.args[a].is_output ? "" : "const ") << c_type(p.args[a].dtype) << "* __restrict__ a" << a;
+    s << ") {\n";
+    if (any_col && TY > 1) s << "__shared__ float col_red[TY * TX * NV];\n";
+    if (any_scalar) s << "__shared__ float blk_red[" << threads / 64 << "];\n";
+    s << "u32 t = blockIdx.x;\nconst u32 tile_x = t % " << gx << "u; t /= " << gx << "u;\nconst u32 tile_y = t % " << gy
+      << "u; t /= " << gy << "u;\nconst u32 b = t;\n";
+    {
+        // coordinates of the dims that flatten into b
+        s << "u32 brem = b; (void)brem;\n";
+        for (int d = n - 3; d >= 0; d--)
+            s << "const u32 cB" << d << " = brem % " << p.dims[d] << "u; brem /= " << p.dims[d] << "u; (void)cB" << d << ";\n";
+    }
+    s << "const u32 tx = threadIdx.x % TX, ty = threadIdx.x / TX;\n";
+    s << "const u32 n0 = (tile_x * TX + tx) * NV;\nconst bool col_ok = n0 < DIM_N;\n";
+    // reduction partials
+    for (size_t oi = 0; oi < p.outs.size(); oi++) {
+        const Out& o = p.outs[oi];
+        if (!o.reduce) continue;
+        if (o.fold_m && !o.fold_n)
+            s << "float rc" << oi << "[NV];\n#pragma unroll\nfor (int k = 0; k < NV; k++) rc" << oi << "[k] = red_identity<"
+              << (int)o.rop << ">();\n";
+        else if (o.fold_m && o.fold_n)
+            s << "float rs" << oi << " = red_identity<" << (int)o.rop << ">();\n";
+    }
+    s << "#pragma unroll\nfor (u32 i = 0; i < RPT; i++) {\nconst u32 m = tile_y * TR + i * TY + ty;\nconst bool ok = col_ok && m < DIM_M;\n";
+    for (size_t oi = 0; oi < p.outs.size(); oi++)
+        if (p.outs[oi].reduce && p.outs[oi].fold_n && !p.outs[oi].fold_m)
+            s << "float rr" << oi << " = red_identity<" << (int)p.outs[oi].rop << ">();\n";
+    s << "if (ok) {\n";
+    EmitCtx cx;
+    cx.nv = NV;
+    s << emit_exprs(p, cx);
+    // outputs
+    Shape pst = ir::packed_strides(p.dims);
+    for (size_t oi = 0; oi < p.outs.size(); oi++) {
+        const Out& o = p.outs[oi];
+        const std::string v = "e" + std::to_string(o.expr);
+        if (!o.reduce) {
+            s << "{ const size_t o = (size_t)b * " << (M * N) << "ull + (size_t)m * " << N << "ull + n0;\n";
+            if (o.dtype == HE_BOOL) {
+                // bit k of word o/32; the buffer is cleared before the launch (jit.rs:293-301)
+                s << "#pragma unroll\nfor (int k = 0; k < NV; k++) { const size_t l = o + k; if (" << v
+                  << "[k]) atomicOr(a" << o.arg << " + (l >> 5), 1u << (l & 31)); }\n";
+            } else {
+                s << "st_vec<NV>(a" << o.arg << " + o, " << v << ");\n";
+            }
+            s << "}\n";
+            continue;
+        }
+        std::string term = v + "[k]";
+        if (o.rop == ROp::Mean) term = strfmt("(float)((double)%s[k] * %.17g)", v.c_str(), o.mean_scale);
+        if (o.fold_m && !o.fold_n)
+            s << "#pragma unroll\nfor (int k = 0; k < NV; k++) rc" << oi << "[k] = red_op<" << (int)o.rop << ">(rc" << oi
+              << "[k], " << term << ");\n";
+        else if (o.fold_m && o.fold_n)
+            s << "#pragma unroll\nfor (int k = 0; k < NV; k++) rs" << oi << " = red_op<" << (int)o.rop << ">(rs" << oi << ", "
+              << term << ");\n";
+        else
+            s << "#pragma unroll\nfor (int k = 0; k < NV; k++) rr" << oi << " = red_op<" << (int)o.rop << ">(rr" << oi << ", "
+              << term << ");\n";
+    }
+    s << "}\n";  // if (ok)
+    // per-row reductions: every lane takes part in the butterfly
+    for (size_t oi = 0; oi < p.outs.size(); oi++) {
+        const Out& o = p.outs[oi];
+        if (!(o.reduce && o.fold_n && !o.fold_m)) continue;
+        const int width = std::min(TX, 64);
+        s << "{ float r = wave_reduce<" << (int)o.rop << ", " << width << ">(rr" << oi << ");\n";
+        s << "if ((threadIdx.x % " << width << ") == 0 && m < DIM_M && col_ok) atomic_red<" << (int)o.rop << ">(a" << o.arg
+          << " + (size_t)b * " << M << "ull + m, r); }\n";
+    }
+    s << "}\n";  // row loop
+    // column reductions
+    for (size_t oi = 0; oi < p.outs.size(); oi++) {
+        const Out& o = p.outs[oi];
+        if (!(o.reduce && o.fold_m && !o.fold_n)) continue;
+        if (TY > 1) {
+            s << "__syncthreads();\n#pragma unroll\nfor (int k = 0; k < NV; k++) col_red[(ty * TX + tx) * NV + k] = rc" << oi
+              << "[k];\n__syncthreads();\nif (ty == 0) {\n#pragma unroll\nfor (int k = 0; k < NV; k++) { float r = rc" << oi
+              << "[k];\nfor (u32 y = 1; y < TY; y++) r = red_op<" << (int)o.rop << ">(r, col_red[(y * TX + tx) * NV + k]);\nrc"
+              << oi << "[k] = r; } }\n";
+        }
+        s << "if (ty == 0 && col_ok) {\n#pragma unroll\nfor (int k = 0; k < NV; k++) atomic_red<" << (int)o.rop << ">(a" << o.arg
+          << " + (size_t)b * " << N << "ull + n0 + k, rc" << oi << "[k]); }\n";
+    }
+    // scalar reductions
+    for (size_t oi = 0; oi < p.outs.size(); oi++) {
+        const Out& o = p.outs[oi];
+        if (!(o.reduce && o.fold_m && o.fold_n)) continue;
+        s << "{ float r = wave_reduce<" << (int)o.rop << ", 64>(rs" << oi << ");\n__syncthreads();\nif ((threadIdx.x & 63) == 0) blk_red[threadIdx.x >> 6] = r;\n__syncthreads();\n";
+        s << "if (threadIdx.x == 0) { r = blk_red[0];\nfor (int w = 1; w < " << threads / 64 << "; w++) r = red_op<"
+          << (int)o.rop << ">(r, blk_red[w]);\natomic_red<" << (int)o.rop << ">(a" << o.arg << " + (size_t)(b / " << o.b_div
+          << "u), r); } }\n";
+    }
+    s << "}\n";
+    L.source = s.str();
+
+    for (auto& o : p.outs) {
+        if (o.reduce) {
+            uint32_t bits = 0;
+            float f = o.rop == ROp::Max ? -INFINITY : o.rop == ROp::Min ? INFINITY : 0.0f;
+            memcpy(&bits, &f, 4);
+            L.fills.push_back({o.arg, bits});
+        } else if (o.dtype == HE_BOOL) {
+            L.fills.push_back({o.arg, 0u});
+        }
+    }
+    std::ostringstream d;
+    d << "dims=[";
+    for (int i = 0; i < n; i++) d << (i ? "x" : "") << p.dims[i];
+    d << "] NV=" << NV << " TX=" << TX << " TY=" << TY << " RPT=" << RPT << " grid=" << L.grid << " threads=" << threads
+      << " exprs=" << p.exprs.size() << " outs=" << p.outs.size();
+    L.describe = d.str();
+    return L;
+}
+
+}  // namespace he::tp

@@ -1,0 +1,290 @@
+#include "ir.h"
+
+#include <sstream>
+
+namespace he::ir {
+
+int64_t num_elements(const Shape& s) {
+    int64_t n = 1;
+    for (int64_t d : s) n *= d;
+    return n;
+}
+
+Shape packed_strides(const Shape& s) {
+    Shape st(s.size(), 1);
+    for (int i = (int)s.size() - 2; i >= 0; i--) st[i] = st[i + 1] * s[i + 1];
+    return st;
+}
+
+int accumulator_type(Precision p) {
+    switch (p) {
+        case Precision::MulF16AccumF16:
+        case Precision::MulF8AccumF16: return HE_F16;
+        default: return HE_F32;
+    }
+}
+
+bool Op::operator==(const Op& o) const {
+    return kind == o.kind && inputs == o.inputs && sub_op == o.sub_op && precision == o.precision &&
+           f8_modes == o.f8_modes && target_type == o.target_type && depth == o.depth &&
+           new_dim_count == o.new_dim_count && broadcast_axes == o.broadcast_axes && shape == o.shape &&
+           axis_a == o.axis_a && axis_b == o.axis_b && const_bits == o.const_bits && const_dtype == o.const_dtype;
+}
+
+uint64_t Op::hash() const {
+    uint64_t h = fnv1a(&kind, sizeof kind);
+    auto mix = [&](const void* p, size_t n) { h = fnv1a(p, n, h); };
+    if (!inputs.empty()) mix(inputs.data(), inputs.size() * sizeof(NodeId));
+    mix(&sub_op, sizeof sub_op);
+    mix(&precision, sizeof precision);
+    mix(&target_type, sizeof target_type);
+    mix(&depth, sizeof depth);
+    mix(&new_dim_count, sizeof new_dim_count);
+    for (auto& a : broadcast_axes) mix(&a, sizeof a);
+    if (!shape.empty()) mix(shape.data(), shape.size() * sizeof(int64_t));
+    mix(&axis_a, sizeof axis_a);
+    mix(&axis_b, sizeof axis_b);
+    mix(&const_bits, sizeof const_bits);
+    mix(&const_dtype, sizeof const_dtype);
+    return h;
+}
+
+NodeId OpGraph::push(Node n) {
+    nodes_.push_back(std::move(n));
+    in_.emplace_back();
+    out_.emplace_back();
+    return (NodeId)(nodes_.size() - 1);
+}
+
+static void push_if_absent(std::vector<NodeId>& v, NodeId x) {
+    if (std::find(v.begin(), v.end(), x) == v.end()) v.push_back(x);
+}
+static void remove_element(std::vector<NodeId>& v, NodeId x) {
+    auto it = std::find(v.begin(), v.end(), x);
+    if (it != v.end()) v.erase(it);
+}
+
+NodeId OpGraph::new_input(const Descriptor& d) {
+    for (int64_t e : d.shape) HE_REQUIRE(e >= 0, HE_ERR_INVALID, "negative extent in input shape");
+    Node n;
+    n.kind = Node::Input;
+    n.desc = d;
+    NodeId id = push(std::move(n));
+    inputs_.push_back(id);
+    return id;
+}
+
+Shape OpGraph::broadcast_output_shape(const Op& op, const Shape& in) {
+    // op.rs:376-390: left-pad with 1s up to new_dim_count, then overwrite every listed axis.
+    Shape s = in;
+    while ((int64_t)s.size() < op.new_dim_count) s.insert(s.begin(), 1);
+    for (auto& a : op.broadcast_axes) {
+        HE_REQUIRE(a.axis >= 0 && a.axis < (int64_t)s.size(), HE_ERR_INVALID, "broadcast axis %lld out of range",
+                   (long long)a.axis);
+        s[a.axis] = a.new_size;
+    }
+    return s;
+}
+
+Descriptor OpGraph::infer(const Op& op, const OpGraph& g) {
+    auto in = [&](size_t i) -> const Descriptor& {
+        HE_REQUIRE(i < op.inputs.size(), HE_ERR_INVALID, "op is missing input %zu", i);
+        return g.get(op.inputs[i]).desc;
+    };
+    switch (op.kind) {
+        case OpKind::ChangeDataType: return {in(0).shape, op.target_type};
+        case OpKind::Matmul: {
+            // op.rs:61-73: A's shape with the last extent replaced by B's last extent; accumulator dtype.
+            Descriptor d{in(0).shape, accumulator_type(op.precision)};
+            HE_REQUIRE(d.shape.size() >= 2 && in(1).shape.size() >= 2, HE_ERR_INVALID, "matmul needs rank >= 2");
+            d.shape.back() = in(1).shape.back();
+            return d;
+        }
+        case OpKind::UnaryPointwise:
+        case OpKind::BinaryPointwise: return in(0);
+        case OpKind::Reduce: {
+            // op.rs:78-89: drop the last `depth` dims, append a single 1; always F32.
+            Shape s = in(0).shape;
+            HE_REQUIRE(op.depth >= 1 && op.depth <= s.size(), HE_ERR_INVALID, "reduce depth %u for rank %zu", op.depth,
+                       s.size());
+            s.resize(s.size() - op.depth + 1);
+            s.back() = 1;
+            return {s, HE_F32};
+        }
+        case OpKind::Reshape:
+            HE_REQUIRE(num_elements(op.shape) == num_elements(in(0).shape), HE_ERR_INVALID,
+                       "reshape changes the element count");
+            return {op.shape, in(0).dtype};
+        case OpKind::Broadcast: return {broadcast_output_shape(op, in(0).shape), in(0).dtype};
+        case OpKind::SwapDims: {
+            Shape s = in(0).shape;
+            HE_REQUIRE(op.axis_a >= 0 && op.axis_b >= 0 && op.axis_a < (int64_t)s.size() && op.axis_b < (int64_t)s.size(),
+                       HE_ERR_INVALID, "swap axis out of range");
+            std::swap(s[op.axis_a], s[op.axis_b]);
+            return {s, in(0).dtype};
+        }
+        case OpKind::Compare: return {in(0).shape, HE_BOOL};
+        case OpKind::Select: return in(0);
+        case OpKind::Constant: return {op.shape, op.const_dtype};
+        case OpKind::Conv:
+        case OpKind::ConvBackwardData:
+        case OpKind::ConvBackwardFilter:
+            fail(HE_ERR_UNSUPPORTED, "convolution ops are outside this backend's path");
+    }
+    fail(HE_ERR_INVALID, "bad op kind");
+}
+
+NodeId OpGraph::new_op(Op op) {
+    for (NodeId i : op.inputs) HE_REQUIRE(alive(i) && get(i).kind != Node::Output, HE_ERR_INVALID, "bad input node %u", i);
+    Node n;
+    n.kind = Node::Intermediate;
+    n.desc = infer(op, *this);
+    std::vector<NodeId> inputs = op.inputs;
+    n.op = std::move(op);
+    NodeId id = push(std::move(n));
+    for (NodeId i : inputs) push_if_absent(out_[i], id);
+    in_[id] = inputs;
+    return id;
+}
+
+NodeId OpGraph::new_output(NodeId from) {
+    HE_REQUIRE(alive(from), HE_ERR_INVALID, "bad node %u", from);
+    Node n;
+    n.kind = Node::Output;
+    n.desc = get(from).desc;
+    NodeId id = push(std::move(n));
+    outputs_.push_back(id);
+    in_[id] = {from};
+    push_if_absent(out_[from], id);
+    return id;
+}
+
+void OpGraph::remove(NodeId id) {
+    HE_REQUIRE(alive(id), HE_ERR_INVALID, "bad node %u", id);
+    for (NodeId p : in_[id]) remove_element(out_[p], id);
+    for (NodeId s : out_[id]) remove_element(in_[s], id);
+    in_[id].clear();
+    out_[id].clear();
+    remove_element(inputs_, id);
+    remove_element(outputs_, id);
+    nodes_[id] = Node{};
+}
+
+void OpGraph::optimize() {
+    std::vector<char> visited(nodes_.size(), 0);
+    std::vector<NodeId> stack = outputs_;
+    while (!stack.empty()) {
+        NodeId n = stack.back();
+        stack.pop_back();
+        visited[n] = 1;
+        for (NodeId p : in_[n])
+            if (!visited[p]) stack.push_back(p);
+    }
+    for (NodeId id = 0; id < nodes_.size(); id++)
+        if (nodes_[id].kind != Node::Removed && !visited[id]) remove(id);
+}
+
+const Node& OpGraph::get(NodeId id) const {
+    HE_REQUIRE(alive(id), HE_ERR_INVALID, "node %u does not exist", id);
+    return nodes_[id];
+}
+
+std::vector<NodeId> OpGraph::nodes() const {
+    std::vector<NodeId> v;
+    for (NodeId id = 0; id < nodes_.size(); id++)
+        if (nodes_[id].kind != Node::Removed) v.push_back(id);
+    return v;
+}
+
+size_t OpGraph::num_nodes() const {
+    size_t n = 0;
+    for (auto& x : nodes_) n += x.kind != Node::Removed;
+    return n;
+}
+
+bool OpGraph::feeds_output(NodeId id) const {
+    for (NodeId s : out_[id])
+        if (nodes_[s].kind == Node::Output) return true;
+    return false;
+}
+
+uint64_t OpGraph::structural_hash() const {
+    uint64_t h = 1469598103934665603ull;
+    for (NodeId id = 0; id < nodes_.size(); id++) {
+        const Node& n = nodes_[id];
+        if (n.kind == Node::Removed) continue;
+        h = fnv1a(&id, sizeof id, h);
+        h = fnv1a(&n.kind, sizeof n.kind, h);
+        h = fnv1a(&n.desc.dtype, sizeof n.desc.dtype, h);
+        if (!n.desc.shape.empty()) h = fnv1a(n.desc.shape.data(), n.desc.shape.size() * 8, h);
+        if (n.kind == Node::Intermediate) {
+            uint64_t oh = n.op.hash();
+            h = fnv1a(&oh, sizeof oh, h);
+        }
+    }
+    return h;
+}
+
+bool OpGraph::structurally_equal(const OpGraph& o) const {
+    // opgraph.rs:205-216: same nodes in the same slots with the same edges.
+    if (nodes_.size() != o.nodes_.size()) return false;
+    for (NodeId id = 0; id < nodes_.size(); id++) {
+        const Node &a = nodes_[id], &b = o.nodes_[id];
+        if (a.kind != b.kind) return false;
+        if (a.kind == Node::Removed) continue;
+        if (!(a.desc == b.desc)) return false;
+        if (a.kind == Node::Intermediate && !(a.op == b.op)) return false;
+        if (in_[id] != o.in_[id] || out_[id] != o.out_[id]) return false;
+    }
+    return true;
+}
+
+OpSubgraph::OpSubgraph(std::shared_ptr<const OpGraph> g, std::vector<NodeId> nodes) : graph_(std::move(g)) {
+    std::sort(nodes.begin(), nodes.end());
+    nodes.erase(std::unique(nodes.begin(), nodes.end()), nodes.end());
+    nodes_ = std::move(nodes);
+    for (NodeId n : nodes_) {
+        HE_REQUIRE(graph_->alive(n) && graph_->get(n).kind == Node::Intermediate, HE_ERR_INVALID,
+                   "subgraph node %u is not an intermediate node", n);
+        bool root = false;
+        for (NodeId i : graph_->inbound(n))
+            if (!contains(i)) {
+                push_if_absent(inputs_, i);
+                root = true;
+            }
+        if (root) roots_.push_back(n);
+        for (NodeId s : graph_->outbound(n))
+            if (!contains(s)) {
+                leafs_.push_back(n);
+                break;
+            }
+    }
+    std::sort(inputs_.begin(), inputs_.end());
+}
+
+OpSubgraph OpSubgraph::merge_with(const OpSubgraph& o) const {
+    HE_REQUIRE(graph_ == o.graph_, HE_ERR_INVALID, "subgraphs of different graphs");
+    std::vector<NodeId> n = nodes_;
+    n.insert(n.end(), o.nodes_.begin(), o.nodes_.end());
+    return OpSubgraph(graph_, std::move(n));
+}
+
+std::string OpSubgraph::cache_key() const {
+    std::ostringstream s;
+    for (NodeId n : nodes_) {
+        const Node& node = graph_->get(n);
+        s << n << ':' << node.op.hash() << ':' << node.desc.dtype << '[';
+        for (int64_t d : node.desc.shape) s << d << ',';
+        s << "];";
+    }
+    s << '|';
+    for (NodeId n : inputs_) {
+        const Node& node = graph_->get(n);
+        s << n << ':' << node.desc.dtype << '[';
+        for (int64_t d : node.desc.shape) s << d << ',';
+        s << "];";
+    }
+    return s.str();
+}
+
+}  // namespace he::ir

@@ -1,0 +1,128 @@
+// The helium-ir operation graph (helium-ir/src/opgraph.rs, opgraph/op.rs, opgraph/subgraph.rs, shape.rs),
+// restated in C++ so that plan generation and the kernel generators consume the same structure the Rust
+// front-end records.
+#pragma once
+#include <algorithm>
+#include <cstdint>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "common.h"
+
+namespace he::ir {
+
+using NodeId = uint32_t;  // index into the graph's node table; ids are never reused within a graph
+constexpr NodeId kNoNode = 0xffffffffu;
+
+using Shape = std::vector<int64_t>;
+int64_t num_elements(const Shape& s);
+Shape packed_strides(const Shape& s);
+
+enum class OpKind : int {
+    Matmul = 0, UnaryPointwise, BinaryPointwise, ChangeDataType, Reduce, Broadcast, Reshape, SwapDims, Compare,
+    Select, Conv, ConvBackwardData, ConvBackwardFilter, Constant
+};
+// opgraph/op.rs:291-304
+enum class UnaryOp : int { Recip = 0, Neg, Exp, Sin, Cos, Tan, Sigmoid, Tanh, Relu, Sqrt, Log };
+// opgraph/op.rs:315-328
+enum class BinaryOp : int { Add = 0, Mul, Pow, Min, Max, And, Or, Xor };
+// opgraph/op.rs:360-367
+enum class ReduceOp : int { Sum = 0, Mean, Max, Min };
+// opgraph/op.rs:429-437
+enum class CompareOp : int { Equal = 0, NotEqual, LessThan, LessThanOrEqual, GreaterThan, GreaterThanOrEqual };
+// opgraph/op/precision.rs:36-81 (the two FP8 variants carry their modes in `f8_modes`)
+enum class Precision : int { MulF32AccumF32 = 0, MulTf32AccumF32, MulBf16AccumF32, MulF16AccumF32, MulF16AccumF16,
+                             MulF8AccumF32, MulF8AccumF16 };
+int accumulator_type(Precision p);  // precision.rs:87-96
+
+struct BroadcastAxis {
+    int64_t axis, new_size;
+    bool operator==(const BroadcastAxis& o) const { return axis == o.axis && new_size == o.new_size; }
+};
+
+struct Op {
+    OpKind kind = OpKind::Constant;
+    std::vector<NodeId> inputs;  // Matmul: a,b; Binary/Compare: lhs,rhs; Select: lhs,rhs,selector
+    int sub_op = 0;              // UnaryOp / BinaryOp / ReduceOp / CompareOp
+    Precision precision = Precision::MulBf16AccumF32;
+    int f8_modes = 0;
+    int target_type = HE_F32;    // ChangeDataType
+    uint32_t depth = 0;          // Reduce
+    int64_t new_dim_count = 0;   // Broadcast
+    std::vector<BroadcastAxis> broadcast_axes;
+    Shape shape;                 // Reshape target / Constant shape
+    int64_t axis_a = 0, axis_b = 0;
+    uint32_t const_bits = 0;     // Constant scalar, bit pattern in its own dtype
+    int const_dtype = HE_F32;
+    bool operator==(const Op& o) const;
+    uint64_t hash() const;
+};
+
+struct Descriptor {
+    Shape shape;
+    int dtype = HE_F32;
+    bool operator==(const Descriptor& o) const { return shape == o.shape && dtype == o.dtype; }
+};
+
+struct Node {
+    enum Kind { Input, Intermediate, Output, Removed } kind = Removed;
+    Descriptor desc;
+    Op op;  // Intermediate only
+};
+
+class OpGraph {
+public:
+    NodeId new_input(const Descriptor& d);
+    NodeId new_op(Op op);  // infers the output descriptor (op.rs:52-179)
+    NodeId new_output(NodeId from);
+    void remove(NodeId id);
+    void optimize();  // prune_unused (opgraph.rs:165-191)
+
+    const Node& get(NodeId id) const;
+    bool alive(NodeId id) const { return id < nodes_.size() && nodes_[id].kind != Node::Removed; }
+    std::vector<NodeId> nodes() const;  // live nodes in id order
+    size_t capacity() const { return nodes_.size(); }
+    size_t num_nodes() const;
+    const std::vector<NodeId>& inputs() const { return inputs_; }
+    const std::vector<NodeId>& outputs() const { return outputs_; }
+    const std::vector<NodeId>& inbound(NodeId id) const { return in_[id]; }
+    const std::vector<NodeId>& outbound(NodeId id) const { return out_[id]; }
+    bool feeds_output(NodeId id) const;
+    uint64_t structural_hash() const;
+    bool structurally_equal(const OpGraph& o) const;
+
+    static Descriptor infer(const Op& op, const OpGraph& g);
+    static Shape broadcast_output_shape(const Op& op, const Shape& in);
+
+private:
+    NodeId push(Node n);
+    std::vector<Node> nodes_;
+    std::vector<NodeId> inputs_, outputs_;
+    std::vector<std::vector<NodeId>> in_, out_;
+};
+
+// Subset of an OpGraph (opgraph/subgraph.rs): nodes sorted by id; `inputs` = outside producers feeding it,
+// `roots` = members with an outside input, `leafs` = members with an outside consumer.
+class OpSubgraph {
+public:
+    OpSubgraph() = default;
+    OpSubgraph(std::shared_ptr<const OpGraph> g, std::vector<NodeId> nodes);
+    OpSubgraph merge_with(const OpSubgraph& o) const;
+    const std::shared_ptr<const OpGraph>& graph() const { return graph_; }
+    const std::vector<NodeId>& nodes() const { return nodes_; }
+    const std::vector<NodeId>& inputs() const { return inputs_; }
+    const std::vector<NodeId>& roots() const { return roots_; }
+    const std::vector<NodeId>& leafs() const { return leafs_; }
+    bool contains(NodeId id) const { return std::binary_search(nodes_.begin(), nodes_.end(), id); }
+    bool is_input(NodeId id) const { return std::find(inputs_.begin(), inputs_.end(), id) != inputs_.end(); }
+    bool is_leaf(NodeId id) const { return std::find(leafs_.begin(), leafs_.end(), id) != leafs_.end(); }
+    // Structural key used by the kernel caches (subgraph.rs:203-233): ops, descriptors and input descriptors.
+    std::string cache_key() const;
+
+private:
+    std::shared_ptr<const OpGraph> graph_;
+    std::vector<NodeId> nodes_, inputs_, roots_, leafs_;
+};
+
+}  // namespace he::ir

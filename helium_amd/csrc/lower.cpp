@@ -1,0 +1,585 @@
+// Lowering of the two front-end IRs to tile programs.
+#include <cstring>
+#include <map>
+
+#include "tp.h"
+
+namespace he::tp {
+
+namespace {
+
+// How the linear index of the node being visited depends on the iteration coordinates: an affine part
+// (weights per iteration dim, in the node's packed layout) followed by reference-style generic maps.
+struct Mapping {
+    std::vector<int64_t> w;
+    std::vector<GenericMap> chain;
+    bool operator==(const Mapping& o) const { return w == o.w && chain == o.chain; }
+};
+
+// For every dim of `shape`, the iteration dim its coordinate equals (-1: coordinate 0). Fails when an iteration
+// dim does not land on exactly one dim of `shape` (a Reshape regrouped it).
+bool try_align(const std::vector<int64_t>& w, const Shape& iter_dims, const Shape& shape, std::vector<int>& src) {
+    Shape st = ir::packed_strides(shape);
+    src.assign(shape.size(), -1);
+    for (size_t d = 0; d < w.size(); d++) {
+        if (iter_dims[d] <= 1 || w[d] == 0) continue;
+        int found = -1;
+        for (size_t j = 0; j < shape.size(); j++)
+            if (st[j] == w[d] && shape[j] >= iter_dims[d] && shape[j] > 1) {
+                found = (int)j;
+                break;
+            }
+        if (found < 0 || src[found] != -1) return false;
+        src[found] = (int)d;
+    }
+    return true;
+}
+
+Mapping through_swap(const Mapping& mp, const Shape& iter_dims, const Shape& out_shape, const Shape& in_shape,
+                     int64_t a, int64_t b) {
+    Mapping r = mp;
+    std::vector<int> src;
+    if (mp.chain.empty() && try_align(mp.w, iter_dims, out_shape, src)) {
+        Shape st = ir::packed_strides(in_shape);
+        std::fill(r.w.begin(), r.w.end(), 0);
+        for (size_t j = 0; j < out_shape.size(); j++) {
+            if (src[j] < 0) continue;
+            size_t k = (int64_t)j == a ? (size_t)b : (int64_t)j == b ? (size_t)a : j;
+            r.w[src[j]] += st[k];
+        }
+        return r;
+    }
+    GenericMap g;
+    g.kind = GenericMap::Swap;
+    g.in_shape = in_shape;
+    g.axis_a = a;
+    g.axis_b = b;
+    r.chain.push_back(g);
+    return r;
+}
+
+Mapping through_broadcast(const Mapping& mp, const Shape& iter_dims, const Shape& out_shape, const Shape& in_shape,
+                          const std::vector<char>& bcast) {
+    Mapping r = mp;
+    std::vector<int> src;
+    const size_t pad = out_shape.size() - in_shape.size();
+    if (mp.chain.empty() && try_align(mp.w, iter_dims, out_shape, src)) {
+        Shape st = ir::packed_strides(in_shape);
+        std::fill(r.w.begin(), r.w.end(), 0);
+        for (size_t j = pad; j < out_shape.size(); j++) {
+            if (src[j] < 0 || bcast[j]) continue;
+            r.w[src[j]] += st[j - pad];
+        }
+        return r;
+    }
+    GenericMap g;
+    g.kind = GenericMap::Bcast;
+    g.in_shape = in_shape;
+    g.out_shape = out_shape;
+    g.bcast = bcast;
+    r.chain.push_back(g);
+    return r;
+}
+
+Cls cls_of(int dtype) {
+    switch (dtype_class(dtype)) {
+        case DataClass::Float: return Cls::F;
+        case DataClass::Int: return Cls::I;
+        case DataClass::Bool: return Cls::B;
+    }
+    return Cls::F;
+}
+
+float bf16_bits_to_f32(uint32_t b) {
+    uint32_t u = b << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+float f16_bits_to_f32(uint32_t h) {
+    uint32_t sign = (h >> 15) & 1, exp = (h >> 10) & 0x1f, man = h & 0x3ff, u;
+    if (exp == 0) {
+        if (man == 0) {
+            u = sign << 31;
+        } else {
+            int e = -1;
+            do {
+                e++;
+                man <<= 1;
+            } while (!(man & 0x400));
+            u = (sign << 31) | ((uint32_t)(127 - 15 - e) << 23) | ((man & 0x3ff) << 13);
+        }
+    } else if (exp == 31) {
+        u = (sign << 31) | 0x7f800000u | (man << 13);
+    } else {
+        u = (sign << 31) | ((exp + 127 - 15) << 23) | (man << 13);
+    }
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+uint32_t f32_bits(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    return u;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// helium-ir pointwise subgraphs
+// ---------------------------------------------------------------------------------------------------------
+class PointwiseLowering {
+public:
+    explicit PointwiseLowering(const ir::OpSubgraph& sg) : sg_(sg), g_(*sg.graph()) {}
+
+    Program run() {
+        HE_REQUIRE(!sg_.leafs().empty(), HE_ERR_INVALID, "pointwise subgraph has no output");
+        // Iteration space: the (pre-reduction) shape of the first leaf, as compute_output_shape picks it
+        // (jit.rs:350-362).
+        ir::NodeId first = sg_.leafs()[0];
+        const ir::Node& fn = g_.get(first);
+        p_.dims = fn.op.kind == ir::OpKind::Reduce ? g_.get(fn.op.inputs[0]).desc.shape : fn.desc.shape;
+        if (p_.dims.empty()) p_.dims = {1};
+        const int64_t numel = ir::num_elements(p_.dims);
+
+        for (ir::NodeId in : sg_.inputs()) {
+            const ir::Descriptor& d = g_.get(in).desc;
+            input_arg_[in] = (int)p_.args.size();
+            p_.args.push_back({d.dtype, ir::num_elements(d.shape), false, in});
+        }
+        Mapping ident;
+        ident.w = ir::packed_strides(p_.dims);
+        for (ir::NodeId leaf : sg_.leafs()) {
+            const ir::Node& n = g_.get(leaf);
+            Out o;
+            o.arg = (int)p_.args.size();
+            if (n.op.kind == ir::OpKind::Reduce) {
+                const Shape& rs = g_.get(n.op.inputs[0]).desc.shape;
+                HE_REQUIRE(ir::num_elements(rs) == numel, HE_ERR_UNSUPPORTED,
+                           "reduction input has a different element count than the other outputs");
+                Shape rdims = rs.empty() ? Shape{1} : rs;
+                HE_REQUIRE(rdims == p_.dims, HE_ERR_UNSUPPORTED, "all reductions of a kernel must share one input shape");
+                const size_t rank = rdims.size();
+                const size_t depth = n.op.depth;
+                HE_REQUIRE(depth >= 1 && depth <= rank, HE_ERR_INVALID, "bad reduce depth");
+                o.reduce = true;
+                o.rop = (ROp)n.op.sub_op;
+                o.fold_n = true;
+                o.fold_m = depth >= 2;
+                o.b_div = 1;
+                for (size_t k = rank - depth; k + 2 < rank; k++) o.b_div *= rdims[k];
+                int64_t group = 1;
+                for (size_t k = rank - depth; k < rank; k++) group *= rdims[k];
+                o.mean_scale = 1.0 / (double)group;
+                o.dtype = HE_F32;
+                o.expr = eval(n.op.inputs[0], ident);
+                HE_REQUIRE(p_.exprs[o.expr].cls == Cls::F, HE_ERR_UNSUPPORTED, "reductions take float operands");
+                p_.args.push_back({HE_F32, ir::num_elements(n.desc.shape), true, leaf});
+            } else {
+                HE_REQUIRE(ir::num_elements(n.desc.shape) == numel, HE_ERR_UNSUPPORTED,
+                           "all outputs of a pointwise kernel must have the same element count");
+                o.dtype = n.desc.dtype;
+                o.expr = eval(leaf, ident);
+                p_.args.push_back({n.desc.dtype, numel, true, leaf});
+            }
+            p_.outs.push_back(o);
+        }
+        return std::move(p_);
+    }
+
+private:
+    int push(Expr e) {
+        p_.exprs.push_back(std::move(e));
+        return (int)p_.exprs.size() - 1;
+    }
+
+    int eval(ir::NodeId node, const Mapping& mp) {
+        for (auto& m : memo_)
+            if (m.node == node && m.mp == mp) return m.expr;
+        int id = eval_uncached(node, mp);
+        memo_.push_back({node, mp, id});
+        return id;
+    }
+
+    int eval_uncached(ir::NodeId node, const Mapping& mp) {
+        const ir::Node& n = g_.get(node);
+        if (sg_.is_input(node)) {
+            Expr e;
+            e.kind = Expr::Load;
+            e.cls = cls_of(n.desc.dtype);
+            e.access.arg = input_arg_.at(node);
+            e.access.dtype = n.desc.dtype;
+            e.access.stride = mp.w;
+            e.access.chain = mp.chain;
+            return push(e);
+        }
+        HE_REQUIRE(sg_.contains(node) && n.kind == ir::Node::Intermediate, HE_ERR_INVALID,
+                   "node %u is outside the subgraph", node);
+        const ir::Op& op = n.op;
+        auto in_shape = [&](size_t i) -> const Shape& { return g_.get(op.inputs[i]).desc.shape; };
+        switch (op.kind) {
+            case ir::OpKind::SwapDims:
+                return eval(op.inputs[0], through_swap(mp, p_.dims, n.desc.shape, in_shape(0), op.axis_a, op.axis_b));
+            case ir::OpKind::Broadcast: {
+                std::vector<char> flags(n.desc.shape.size(), 0);
+                for (auto& a : op.broadcast_axes) flags[a.axis] = 1;
+                return eval(op.inputs[0], through_broadcast(mp, p_.dims, n.desc.shape, in_shape(0), flags));
+            }
+            case ir::OpKind::Reshape: return eval(op.inputs[0], mp);
+            case ir::OpKind::ChangeDataType: {
+                int x = eval(op.inputs[0], mp);
+                Cls to = cls_of(op.target_type);
+                if (p_.exprs[x].cls == to) return x;  // same class: only loads and stores change (jit.rs:674-690)
+                Expr e;
+                e.kind = Expr::Cast;
+                e.cls = to;
+                e.a = x;
+                return push(e);
+            }
+            case ir::OpKind::UnaryPointwise: {
+                Expr e;
+                e.kind = Expr::Unary;
+                e.a = eval(op.inputs[0], mp);
+                e.cls = p_.exprs[e.a].cls;
+                HE_REQUIRE(e.cls == Cls::F, HE_ERR_UNSUPPORTED, "unary pointwise ops take float operands");
+                static const UOp map[] = {UOp::Recip, UOp::Neg, UOp::Exp, UOp::Sin, UOp::Cos, UOp::Tan,
+                                          UOp::Sigmoid, UOp::Tanh, UOp::Relu, UOp::Sqrt, UOp::Log};
+                HE_REQUIRE(op.sub_op >= 0 && op.sub_op < 11, HE_ERR_INVALID, "bad unary op");
+                e.op = (int)map[op.sub_op];
+                return push(e);
+            }
+            case ir::OpKind::BinaryPointwise: {
+                Expr e;
+                e.kind = Expr::Binary;
+                e.a = eval(op.inputs[0], mp);
+                e.b = eval(op.inputs[1], mp);
+                e.cls = p_.exprs[e.a].cls;
+                HE_REQUIRE(p_.exprs[e.b].cls == e.cls, HE_ERR_UNSUPPORTED, "binary operands differ in data class");
+                static const BOp map[] = {BOp::Add, BOp::Mul, BOp::Pow, BOp::Min, BOp::Max, BOp::And, BOp::Or, BOp::Xor};
+                HE_REQUIRE(op.sub_op >= 0 && op.sub_op < 8, HE_ERR_INVALID, "bad binary op");
+                e.op = (int)map[op.sub_op];
+                return push(e);
+            }
+            case ir::OpKind::Compare: {
+                Expr e;
+                e.kind = Expr::Compare;
+                e.cls = Cls::B;
+                e.a = eval(op.inputs[0], mp);
+                e.b = eval(op.inputs[1], mp);
+                e.op = op.sub_op;
+                return push(e);
+            }
+            case ir::OpKind::Select: {
+                Expr e;
+                e.kind = Expr::Select;
+                e.a = eval(op.inputs[0], mp);
+                e.b = eval(op.inputs[1], mp);
+                e.c = eval(op.inputs[2], mp);
+                e.cls = p_.exprs[e.a].cls;
+                HE_REQUIRE(p_.exprs[e.c].cls == Cls::B, HE_ERR_UNSUPPORTED, "select needs a bool selector");
+                return push(e);
+            }
+            case ir::OpKind::Constant: {
+                Expr e;
+                e.kind = Expr::Const;
+                e.cls = cls_of(op.const_dtype);
+                switch (op.const_dtype) {
+                    case HE_F32: e.bits = op.const_bits; break;
+                    case HE_BF16: e.bits = f32_bits(bf16_bits_to_f32(op.const_bits & 0xffff)); break;
+                    case HE_F16: e.bits = f32_bits(f16_bits_to_f32(op.const_bits & 0xffff)); break;
+                    case HE_U32: e.bits = op.const_bits; break;
+                    case HE_BOOL: e.bits = op.const_bits ? 1 : 0; break;
+                }
+                return push(e);
+            }
+            case ir::OpKind::Reduce: fail(HE_ERR_UNSUPPORTED, "a reduction must be an output of its kernel");
+            default: fail(HE_ERR_UNSUPPORTED, "op kind is not handled by the pointwise instruction");
+        }
+    }
+
+    struct Memo {
+        ir::NodeId node;
+        Mapping mp;
+        int expr;
+    };
+    const ir::OpSubgraph& sg_;
+    const ir::OpGraph& g_;
+    Program p_;
+    std::map<ir::NodeId, int> input_arg_;
+    std::vector<Memo> memo_;
+};
+
+// ---------------------------------------------------------------------------------------------------------
+// fusion-IR graphs (aux fusions and GEMM epilogues)
+// ---------------------------------------------------------------------------------------------------------
+class FusionLowering {
+public:
+    FusionLowering(const fir::OpGraph& g, fir::OpNode anchor) : g_(g), anchor_(anchor) {}
+
+    Program run() {
+        // Outputs: every leaf; a Consumer stands for the node it reads (kernel_generator.rs:157-167).
+        std::vector<std::pair<fir::OpNode, fir::OpNode>> outs;  // (leaf id, value node)
+        for (fir::OpNode leaf : g_.leaves()) {
+            const fir::Op& op = g_.get(leaf);
+            fir::OpNode x = op.kind == fir::OpKind::Consumer ? op.a : leaf;
+            if (anchor_ != fir::kNoOpNode && !downstream_of_anchor(x)) continue;
+            outs.push_back({leaf, x});
+        }
+        HE_REQUIRE(!outs.empty(), HE_ERR_INVALID, "fusion has no output");
+
+        // Iteration space: the anchor's output, else the largest root (kernel_generator.rs:98-106).
+        fir::Shape3 s;
+        if (anchor_ != fir::kNoOpNode) {
+            s = g_.shape(anchor_);
+        } else {
+            fir::OpNode best = fir::kNoOpNode;
+            uint64_t best_n = 0;
+            for (fir::OpNode r : g_.roots()) {
+                const fir::Shape3& rs = g_.shape(r);
+                uint64_t n = (uint64_t)rs[0] * rs[1] * rs[2];
+                if (best == fir::kNoOpNode || n > best_n) {
+                    best = r;
+                    best_n = n;
+                }
+            }
+            HE_REQUIRE(best != fir::kNoOpNode, HE_ERR_INVALID, "fusion has no input");
+            s = g_.shape(best);
+            // An output may be larger than every input (a broadcast of a small producer): take the value shape.
+            for (auto& o : outs) {
+                const fir::Op& vop = g_.get(o.second);
+                fir::Shape3 vs = vop.kind == fir::OpKind::Reduction ? g_.shape(vop.a) : g_.shape(o.second);
+                if ((uint64_t)vs[0] * vs[1] * vs[2] > (uint64_t)s[0] * s[1] * s[2]) s = vs;
+            }
+        }
+        p_.dims = {s[0], s[1], s[2]};
+
+        // Arguments: producers reachable from the outputs (in id order), then outputs (in leaf order).
+        std::vector<fir::OpNode> producers;
+        {
+            std::vector<fir::OpNode> stack;
+            std::map<fir::OpNode, char> seen;
+            for (auto& o : outs) stack.push_back(o.second);
+            while (!stack.empty()) {
+                fir::OpNode n = stack.back();
+                stack.pop_back();
+                if (seen[n]++) continue;
+                if (n == anchor_) continue;  // the mainloop side is not part of this program
+                if (g_.get(n).kind == fir::OpKind::Producer) producers.push_back(n);
+                for (fir::OpNode i : g_.inbound(n)) stack.push_back(i);
+            }
+            std::sort(producers.begin(), producers.end());
+        }
+        for (fir::OpNode pnode : producers) {
+            const fir::Shape3& ps = g_.shape(pnode);
+            input_arg_[pnode] = (int)p_.args.size();
+            p_.args.push_back({g_.get(pnode).dtype, (int64_t)ps[0] * ps[1] * ps[2], false, pnode});
+        }
+        Mapping ident;
+        ident.w = ir::packed_strides(p_.dims);
+        for (auto& [leaf, x] : outs) {
+            const fir::Op& vop = g_.get(x);
+            Out o;
+            o.arg = (int)p_.args.size();
+            if (vop.kind == fir::OpKind::Reduction) {
+                const fir::Shape3& rs = g_.shape(vop.a);
+                HE_REQUIRE(Shape({rs[0], rs[1], rs[2]}) == p_.dims, HE_ERR_UNSUPPORTED,
+                           "reduction input shape differs from the fusion's tile space");
+                o.reduce = true;
+                o.rop = ROp::Sum;
+                switch (vop.depth) {
+                    case fir::ReductionDepth::Rows: o.fold_n = true; break;
+                    case fir::ReductionDepth::Columns: o.fold_m = true; break;
+                    case fir::ReductionDepth::Item: o.fold_n = o.fold_m = true; break;
+                    case fir::ReductionDepth::Batch:
+                        o.fold_n = o.fold_m = true;
+                        o.b_div = rs[0];
+                        break;
+                }
+                o.dtype = HE_F32;  // reductions accumulate and are stored in f32
+                o.expr = eval(vop.a, ident);
+                const fir::Shape3& os = g_.shape(x);
+                p_.args.push_back({HE_F32, (int64_t)os[0] * os[1] * os[2], true, leaf});
+            } else {
+                const fir::Shape3& vs = g_.shape(x);
+                HE_REQUIRE(Shape({vs[0], vs[1], vs[2]}) == p_.dims, HE_ERR_UNSUPPORTED,
+                           "full-size outputs must have the fusion's tile-space shape (transposed outputs are not fused)");
+                o.dtype = g_.get(leaf).kind == fir::OpKind::Consumer ? g_.get(leaf).dtype : HE_BF16;
+                o.expr = eval(x, ident);
+                p_.args.push_back({o.dtype, ir::num_elements(p_.dims), true, leaf});
+            }
+            p_.outs.push_back(o);
+        }
+        return std::move(p_);
+    }
+
+private:
+    bool downstream_of_anchor(fir::OpNode n) {
+        auto it = down_.find(n);
+        if (it != down_.end()) return it->second;
+        bool r = n == anchor_;
+        if (!r)
+            for (fir::OpNode i : g_.inbound(n)) r = r || downstream_of_anchor(i);
+        return down_[n] = r;
+    }
+
+    int push(Expr e) {
+        p_.exprs.push_back(std::move(e));
+        return (int)p_.exprs.size() - 1;
+    }
+
+    int eval(fir::OpNode node, const Mapping& mp) {
+        for (auto& m : memo_)
+            if (m.node == node && m.mp == mp) return m.expr;
+        int id = eval_uncached(node, mp);
+        memo_.push_back({node, mp, id});
+        return id;
+    }
+
+    int eval_uncached(fir::OpNode node, const Mapping& mp) {
+        const fir::Op& op = g_.get(node);
+        auto shape_of = [&](fir::OpNode n) {
+            const fir::Shape3& s = g_.shape(n);
+            return Shape{s[0], s[1], s[2]};
+        };
+        if (node == anchor_) {
+            HE_REQUIRE(mp.chain.empty() && mp.w == ir::packed_strides(p_.dims), HE_ERR_UNSUPPORTED,
+                       "the anchor's tile can only be read in place (no transpose/broadcast of the GEMM result)");
+            if (p_.acc_expr < 0) {
+                Expr e;
+                e.kind = Expr::Acc;
+                e.cls = Cls::F;
+                p_.acc_expr = push(e);
+            }
+            return p_.acc_expr;
+        }
+        switch (op.kind) {
+            case fir::OpKind::Producer: {
+                Expr e;
+                e.kind = Expr::Load;
+                e.cls = cls_of(op.dtype);
+                HE_REQUIRE(e.cls == Cls::F, HE_ERR_UNSUPPORTED, "fusion-IR tensors are float tensors");
+                e.access.arg = input_arg_.at(node);
+                e.access.dtype = op.dtype;
+                e.access.stride = mp.w;
+                e.access.chain = mp.chain;
+                return push(e);
+            }
+            case fir::OpKind::Constant: {
+                Expr e;
+                e.kind = Expr::Const;
+                e.cls = Cls::F;
+                e.bits = f32_bits(op.value);
+                return push(e);
+            }
+            case fir::OpKind::UnaryPointwise: {
+                Expr e;
+                e.kind = Expr::Unary;
+                e.cls = Cls::F;
+                e.a = eval(op.a, mp);
+                static const UOp map[] = {UOp::Neg, UOp::Relu, UOp::Gelu, UOp::Tanh, UOp::Exp, UOp::Log, UOp::Sqrt,
+                                          UOp::AddC, UOp::MulC, UOp::PowC};
+                HE_REQUIRE(op.sub_op >= 0 && op.sub_op < 10, HE_ERR_INVALID, "bad unary op");
+                e.op = (int)map[op.sub_op];
+                e.bits = f32_bits(op.constant);
+                return push(e);
+            }
+            case fir::OpKind::BinaryPointwise: {
+                Expr e;
+                e.kind = Expr::Binary;
+                e.cls = Cls::F;
+                e.a = eval(op.a, mp);
+                e.b = eval(op.b, mp);
+                static const BOp map[] = {BOp::Add, BOp::Sub, BOp::Mul, BOp::Div, BOp::Pow, BOp::Drelu};
+                HE_REQUIRE(op.sub_op >= 0 && op.sub_op < 6, HE_ERR_INVALID, "bad binary op");
+                e.op = (int)map[op.sub_op];
+                return push(e);
+            }
+            case fir::OpKind::Broadcast: {
+                std::vector<char> flags(3, 0);
+                flags[op.axis] = 1;
+                return eval(op.a, through_broadcast(mp, p_.dims, shape_of(node), shape_of(op.a), flags));
+            }
+            case fir::OpKind::Transpose:
+                return eval(op.a, through_swap(mp, p_.dims, shape_of(node), shape_of(op.a), 1, 2));
+            case fir::OpKind::Consumer: return eval(op.a, mp);
+            case fir::OpKind::Reduction: fail(HE_ERR_UNSUPPORTED, "a reduction terminates its fusion");
+            case fir::OpKind::Matmul: fail(HE_ERR_UNSUPPORTED, "a fusion holds at most one Matmul");
+        }
+        fail(HE_ERR_INVALID, "bad fusion-IR op");
+    }
+
+    struct Memo {
+        fir::OpNode node;
+        Mapping mp;
+        int expr;
+    };
+    const fir::OpGraph& g_;
+    fir::OpNode anchor_;
+    Program p_;
+    std::map<fir::OpNode, int> input_arg_;
+    std::map<fir::OpNode, bool> down_;
+    std::vector<Memo> memo_;
+};
+
+}  // namespace
+
+bool pointwise_supports(const ir::OpSubgraph& sg) {
+    // helium/src/cuda/instr/pointwise.rs:121-186, statement for statement: `x` counts Broadcasts as well as
+    // SwapDims, and only a SwapDims checks it.
+    const ir::OpGraph& g = *sg.graph();
+    int64_t output_size = -1;
+    bool have_red = false;
+    Shape red_shape;
+    uint32_t red_depth = 0;
+    int x = 0;
+    for (ir::NodeId node : sg.nodes()) {
+        const ir::Op& op = g.get(node).op;
+        ir::NodeId check = op.kind == ir::OpKind::Reduce ? op.inputs[0] : node;
+        if (sg.is_leaf(node)) {
+            int64_t n = ir::num_elements(g.get(check).desc.shape);
+            if (output_size < 0)
+                output_size = n;
+            else if (output_size != n)
+                return false;
+        }
+        switch (op.kind) {
+            case ir::OpKind::Select:
+            case ir::OpKind::Reshape:
+            case ir::OpKind::Compare:
+            case ir::OpKind::UnaryPointwise:
+            case ir::OpKind::BinaryPointwise:
+            case ir::OpKind::ChangeDataType: continue;
+            case ir::OpKind::Broadcast: x += 1; break;
+            case ir::OpKind::SwapDims:
+                x += 1;
+                if (x > 1) return false;
+                break;
+            case ir::OpKind::Reduce: {
+                if (!sg.is_leaf(node)) return false;
+                const Shape& s = g.get(op.inputs[0]).desc.shape;
+                if (!have_red) {
+                    have_red = true;
+                    red_shape = s;
+                    red_depth = op.depth;
+                } else if (red_shape != s || red_depth != op.depth) {
+                    return false;
+                }
+                break;
+            }
+            default: return false;  // includes Constant, exactly as the reference's `_ => return false`
+        }
+    }
+    return true;
+}
+
+Program lower_pointwise(const ir::OpSubgraph& sg) { return PointwiseLowering(sg).run(); }
+Program lower_aux(const fir::OpGraph& g) {
+    HE_REQUIRE(g.anchor() == fir::kNoOpNode, HE_ERR_INVALID, "an auxiliary fusion holds no Matmul");
+    return FusionLowering(g, fir::kNoOpNode).run();
+}
+Program lower_epilogue(const fir::OpGraph& g, fir::OpNode anchor) {
+    Program p = FusionLowering(g, anchor).run();
+    p.fast_math = true;
+    return p;
+}
+
+}  // namespace he::tp

@@ -135,6 +135,121 @@ const char* he_permute_describe(he_permute_t permute);
 int he_permute_reference_output_strides(const int64_t* shape, int rank, const int32_t* swaps, int num_swaps,
                                         int64_t* strides_out);
 
+
+/* ==================================================================================================
+ * 3. helium-ir operation graph — the structure helium/src/raw_tensor.rs records and hands to the backend
+ *    (helium-ir/src/opgraph.rs, opgraph/op.rs, opgraph/subgraph.rs). Node ids are indices in creation order.
+ * ================================================================================================== */
+typedef struct he_graph_s* he_graph_t;
+
+/* OpKind, same order as helium-ir/src/opgraph/op.rs:15-30. */
+enum {
+    HE_OP_MATMUL = 0, HE_OP_UNARY, HE_OP_BINARY, HE_OP_CHANGE_DTYPE, HE_OP_REDUCE, HE_OP_BROADCAST, HE_OP_RESHAPE,
+    HE_OP_SWAP_DIMS, HE_OP_COMPARE, HE_OP_SELECT, HE_OP_CONV, HE_OP_CONV_BWD_DATA, HE_OP_CONV_BWD_FILTER,
+    HE_OP_CONSTANT
+};
+/* UnaryPointwiseOp (op.rs:291-304) */
+enum { HE_UN_RECIP = 0, HE_UN_NEG, HE_UN_EXP, HE_UN_SIN, HE_UN_COS, HE_UN_TAN, HE_UN_SIGMOID, HE_UN_TANH,
+       HE_UN_RELU, HE_UN_SQRT, HE_UN_LOG };
+/* BinaryPointwiseOp (op.rs:315-328) */
+enum { HE_BIN_ADD = 0, HE_BIN_MUL, HE_BIN_POW, HE_BIN_MIN, HE_BIN_MAX, HE_BIN_AND, HE_BIN_OR, HE_BIN_XOR };
+/* ReduceOp (op.rs:360-367) */
+enum { HE_RED_SUM = 0, HE_RED_MEAN, HE_RED_MAX, HE_RED_MIN };
+/* CompareOp (op.rs:429-437) */
+enum { HE_CMP_EQ = 0, HE_CMP_NE, HE_CMP_LT, HE_CMP_LE, HE_CMP_GT, HE_CMP_GE };
+/* Precision (op/precision.rs:36-81) */
+enum { HE_PREC_F32_F32 = 0, HE_PREC_TF32_F32, HE_PREC_BF16_F32, HE_PREC_F16_F32, HE_PREC_F16_F16,
+       HE_PREC_F8_F32, HE_PREC_F8_F16 };
+
+/* One `Op` value (op.rs:15-30 and the structs below it). Only the fields of the given kind are read.
+ *   inputs: Matmul a,b | Unary x | Binary/Compare lhs,rhs | Select lhs,rhs,selector | others x          */
+typedef struct he_op_desc {
+    int32_t kind;
+    uint32_t inputs[3];
+    int32_t num_inputs;
+    int32_t sub_op;         /* HE_UN_* / HE_BIN_* / HE_RED_* / HE_CMP_* */
+    int32_t precision;      /* Matmul: HE_PREC_* */
+    int32_t target_type;    /* ChangeDataType */
+    uint32_t depth;         /* Reduce: number of trailing dims folded */
+    int64_t new_dim_count;  /* Broadcast */
+    const int64_t* broadcast_axes; /* Broadcast: (axis, new_size) pairs */
+    int32_t num_broadcast_axes;
+    const int64_t* shape;   /* Reshape target shape / Constant shape */
+    int32_t shape_rank;
+    int64_t axis_a, axis_b; /* SwapDims */
+    uint32_t const_bits;    /* Constant: the scalar's bit pattern in const_dtype */
+    int32_t const_dtype;
+} he_op_desc;
+
+int he_graph_create(he_graph_t* graph);                                       /* OpGraph::new (opgraph.rs:21-23) */
+int he_graph_destroy(he_graph_t graph);
+int he_graph_new_input(he_graph_t graph, const int64_t* shape, int rank, int dtype, uint32_t* node); /* :66-70 */
+int he_graph_new_op(he_graph_t graph, const he_op_desc* op, uint32_t* node);  /* new_op + shape inference :73-86 */
+int he_graph_new_output(he_graph_t graph, uint32_t from_node, uint32_t* node); /* :89-100 */
+int he_graph_optimize(he_graph_t graph);                                      /* prune_unused :165-191 */
+int he_graph_num_nodes(he_graph_t graph, uint32_t* count);
+/* Descriptor of a node (opgraph.rs:240-246). shape_out must hold 16 entries. kind: 0 input, 1 intermediate, 2 output. */
+int he_graph_node_info(he_graph_t graph, uint32_t node, int32_t* kind, int32_t* dtype, int32_t* rank, int64_t* shape_out);
+
+/* ==================================================================================================
+ * 4. Pointwise / reduction instruction — helium/src/cuda/instr/pointwise.rs + pointwise/jit.rs (kernels K2, K3).
+ * ================================================================================================== */
+typedef struct he_tile_kernel_s* he_tile_kernel_t;
+
+/* supports_subgraph (pointwise.rs:121-186) for the subgraph made of `nodes`. */
+int he_pointwise_supports(he_graph_t graph, const uint32_t* nodes, int num_nodes, int* supported);
+/* PointwiseGraph::new + precompile (pointwise.rs:35-54): lowers the subgraph, generates and compiles its kernel. */
+int he_pointwise_create(he_tile_kernel_t* kernel, he_graph_t graph, const uint32_t* nodes, int num_nodes);
+/* Kernel arguments: the subgraph's inputs in id order, then its leafs in id order. */
+int he_tile_kernel_num_args(he_tile_kernel_t kernel, int* count);
+int he_tile_kernel_arg_info(he_tile_kernel_t kernel, int index, uint64_t* node, int32_t* is_output, int32_t* dtype,
+                            int64_t* numel);
+/* PointwiseGraph::execute (pointwise.rs:57-86): fills reduction / bitset outputs, then one launch. */
+int he_tile_kernel_execute(he_tile_kernel_t kernel, void* const* arg_ptrs, int num_args, he_stream_t stream);
+const char* he_tile_kernel_source(he_tile_kernel_t kernel);
+const char* he_tile_kernel_describe(he_tile_kernel_t kernel);
+int he_tile_kernel_destroy(he_tile_kernel_t kernel);
+
+/* ==================================================================================================
+ * 5. Fusion IR — helium-playground/src/opgraph.rs: 3-d [batch, rows, cols] shapes, Core = Matmul with Mainloop
+ *    and Epilogue op lists, or anchor-less auxiliary fusions.
+ * ================================================================================================== */
+typedef struct he_fgraph_s* he_fgraph_t;
+
+/* Op variants (opgraph.rs:264-301) */
+enum { HE_FOP_PRODUCER = 0, HE_FOP_CONSTANT, HE_FOP_MATMUL, HE_FOP_UNARY, HE_FOP_REDUCTION, HE_FOP_BINARY,
+       HE_FOP_BROADCAST, HE_FOP_TRANSPOSE, HE_FOP_CONSUMER };
+/* UnaryPointwiseOp (opgraph.rs:317-328) */
+enum { HE_FUN_NEG = 0, HE_FUN_RELU, HE_FUN_GELU, HE_FUN_TANH, HE_FUN_EXP, HE_FUN_LN, HE_FUN_SQRT, HE_FUN_ADD_CONSTANT,
+       HE_FUN_MUL_CONSTANT, HE_FUN_POW_CONSTANT };
+/* BinaryPointwiseOp (opgraph.rs:330-338) */
+enum { HE_FBIN_ADD = 0, HE_FBIN_SUB, HE_FBIN_MUL, HE_FBIN_DIV, HE_FBIN_POW, HE_FBIN_DRELU };
+/* ReductionDepth (opgraph.rs:309-314) */
+enum { HE_FRED_ROWS = 0, HE_FRED_COLUMNS, HE_FRED_ITEM, HE_FRED_BATCH };
+
+typedef struct he_fop_desc {
+    int32_t kind;          /* HE_FOP_* */
+    uint32_t shape[3];     /* Producer / Constant */
+    float value;           /* Constant */
+    uint64_t a, b;         /* Matmul a,b | Binary lhs,rhs | Unary/Reduction/Broadcast/Transpose/Consumer x in a */
+    int32_t sub_op;        /* HE_FUN_* / HE_FBIN_* */
+    float constant;        /* AddConstant / MulConstant / PowConstant */
+    int32_t depth;         /* Reduction: HE_FRED_* (the op is always Sum, opgraph.rs:303-306) */
+    uint32_t axis, amount; /* Broadcast */
+    int32_t dtype;         /* Producer / Consumer storage type (the reference's kernels assume bf16) */
+} he_fop_desc;
+
+int he_fgraph_create(he_fgraph_t* graph);                                  /* OpGraph::new (opgraph.rs:29-31) */
+int he_fgraph_destroy(he_fgraph_t graph);
+/* OpGraph::insert (opgraph.rs:33-57). With *node == UINT64_MAX on entry the id is assigned in insertion order,
+ * otherwise the given id is used (to rebuild a printed fusion with its own numbering). */
+int he_fgraph_insert(he_fgraph_t graph, const he_fop_desc* op, uint64_t* node);
+int he_fgraph_shape(he_fgraph_t graph, uint64_t node, uint32_t shape_out[3]);
+
+/* KernelGenerator::new + generate for an anchor-less fusion (kernel_generator.rs:22-49,98-115; template
+ * templates/auxiliary.cu). Arguments: producers in id order, then leaves in id order (:52-63,138-148). */
+int he_aux_kernel_create(he_tile_kernel_t* kernel, he_fgraph_t graph);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,236 @@
+"""Oracle for helium-ir graphs: shape/dtype inference and op-by-op evaluation. Test infrastructure only.
+
+Follows helium-ir/src/opgraph/op.rs (inference), helium/src/cuda/instr/pointwise/jit.rs (arithmetic: every float
+op is computed in f32 whatever the storage type; same-class casts are transparent inside a kernel; stores round
+to the storage type) and helium/src/raw_tensor.rs (front-end lowerings, in `lower_*` helpers used by the tests).
+
+Pinned by tests/golden/tensor_ops.json (helium/tests/tensor_ops.rs: add/mul/div/recip/scalar ops, op chain = 0.4,
+reduce sum/mean/max/min incl. 200k elements, broadcast, reshape, swaps, relu, constant, max/min, matmul small
+cases) and by closed forms in tests/test_oracle.py. Transcendentals (`expf`, `tanhf`, `powf`, ...) are evaluated
+in float64 and rounded once to float32; the reference uses CUDA libdevice for them, whose last-bit behaviour is
+"parity unpinned" beyond the exact-answer cases.
+
+The graph is plain data: a list of dicts as recorded by helium_amd.ir.OpGraph.nodes
+  {"id", "node": "input", "shape", "dtype"} | {"id", "node": "output", "from"} |
+  {"id", "node": "op", "op": kind, "inputs": [...], ...op fields}.
+"""
+import numpy as np
+
+from . import numerics as nm
+
+FLOATS = ("f32", "bf16", "f16")
+
+
+def accumulator_type(precision):
+    """helium-ir/src/opgraph/op/precision.rs:87-96"""
+    return "f16" if precision in ("f16_f16", "f8_f16") else "f32"
+
+
+def infer(node, desc):
+    """Output (shape, dtype) of an op node given `desc[id] = (shape, dtype)` (op.rs:52-179)."""
+    op, ins = node["op"], node["inputs"]
+    s0, t0 = desc[ins[0]] if ins else (None, None)
+    if op == "change_dtype":
+        return list(s0), node["target"]
+    if op == "matmul":
+        return list(s0[:-1]) + [desc[ins[1]][0][-1]], accumulator_type(node["precision"])
+    if op in ("unary", "binary", "select"):
+        return list(s0), t0
+    if op == "reduce":
+        return list(s0[: len(s0) - node["depth"]]) + [1], "f32"
+    if op == "reshape":
+        return list(node["new_shape"]), t0
+    if op == "broadcast":
+        shape = [1] * max(0, node["new_dim_count"] - len(s0)) + list(s0)
+        for axis, size in node["axes"]:
+            shape[axis] = size
+        return shape, t0
+    if op == "swap_dims":
+        shape = list(s0)
+        a, b = node["axis_a"], node["axis_b"]
+        shape[a], shape[b] = shape[b], shape[a]
+        return shape, t0
+    if op == "compare":
+        return list(s0), "bool"
+    if op == "constant":
+        return list(node["shape"]), node["const_dtype"]
+    raise ValueError(op)
+
+
+def _f64(fn, x):
+    with np.errstate(all="ignore"):
+        return fn(x.astype(np.float64)).astype(np.float32)
+
+
+def unary(fn, x):
+    """jit.rs:718-732, in f32."""
+    one = np.float32(1.0)
+    with np.errstate(all="ignore"):
+        if fn == "recip":
+            return one / x
+        if fn == "neg":
+            return -x
+        if fn == "exp":
+            return _f64(np.exp, x)
+        if fn == "sin":
+            return _f64(np.sin, x)
+        if fn == "cos":
+            return _f64(np.cos, x)
+        if fn == "tan":
+            return _f64(np.tan, x)
+        if fn == "sigmoid":
+            return one / (one + _f64(np.exp, -x))
+        if fn == "tanh":
+            return _f64(np.tanh, x)
+        if fn == "relu":
+            return np.fmax(x, np.float32(0.0))
+        if fn == "sqrt":
+            return np.sqrt(x)
+        if fn == "log":
+            return _f64(np.log, x)
+    raise ValueError(fn)
+
+
+def binary(fn, a, b):
+    """jit.rs:734-747"""
+    with np.errstate(all="ignore"):
+        if a.dtype == np.bool_:
+            return {"and": a & b, "or": a | b, "xor": a ^ b}[fn]
+        if fn == "add":
+            return a + b
+        if fn == "mul":
+            return a * b
+        if fn == "pow":
+            return np.power(a.astype(np.float64), b.astype(np.float64)).astype(np.float32)
+        if fn == "min":
+            return np.fmin(a, b)
+        if fn == "max":
+            return np.fmax(a, b)
+        if fn in ("and", "or", "xor"):
+            return {"and": a & b, "or": a | b, "xor": a ^ b}[fn]
+    raise ValueError(fn)
+
+
+def compare(fn, a, b):
+    return {"eq": a == b, "ne": a != b, "lt": a < b, "le": a <= b, "gt": a > b, "ge": a >= b}[fn]
+
+
+def cast_class(x, src, dst):
+    """jit.rs:663-672. Same-class casts do nothing to the math-domain value."""
+    sf, df = src in FLOATS, dst in FLOATS
+    if sf and df or src == dst:
+        return x
+    if sf and dst == "bool":
+        return x != np.float32(0.0)
+    if src == "bool" and df:
+        return np.where(x, np.float32(1.0), np.float32(0.0)).astype(np.float32)
+    if sf and dst == "u32":
+        with np.errstate(all="ignore"):
+            return np.clip(np.trunc(x.astype(np.float64)), 0, 0xFFFFFFFF).astype(np.uint32)
+    if src == "u32" and df:
+        return x.astype(np.float32)
+    if src == "bool" and dst == "u32":
+        return x.astype(np.uint32)
+    if src == "u32" and dst == "bool":
+        return x != 0
+    raise ValueError((src, dst))
+
+
+def reduce(fn, x, depth):
+    """jit.rs:588-644 + op.rs:78-89: fold the last `depth` dims into one of extent 1; result is f32.
+    Summation runs in float64 (the reference's order is unspecified: block tree + atomics)."""
+    shape = list(x.shape)
+    keep = shape[: len(shape) - depth]
+    flat = x.reshape(keep + [-1])
+    group = flat.shape[-1]
+    if fn == "sum":
+        r = flat.astype(np.float64).sum(axis=-1)
+    elif fn == "mean":
+        # every term is scaled by the double 1/group first, in double, then narrowed to float (jit.rs:599-604)
+        r = (flat.astype(np.float64) * (1.0 / group)).astype(np.float32).astype(np.float64).sum(axis=-1)
+    elif fn == "max":
+        r = flat.max(axis=-1)
+    elif fn == "min":
+        r = flat.min(axis=-1)
+    else:
+        raise ValueError(fn)
+    return r.astype(np.float32).reshape(keep + [1])
+
+
+def matmul(a, b, precision, a_dtype, b_dtype):
+    """Batched row-major A[..,M,K] x B[..,K,N] with operands rounded to the multiplicand type and f32
+    accumulation, evaluated in float64 (helium-ir op.rs:61-73; precision.rs:3-35: actual precision may exceed the
+    one asked for, never fall below)."""
+    def to_mul(x):
+        if precision in ("bf16_f32",):
+            return nm.bf16_bits_to_f32(nm.f32_to_bf16_bits(x)).reshape(x.shape)
+        if precision in ("f16_f32", "f16_f16"):
+            return x.astype(np.float16).astype(np.float32)
+        return x
+    r = np.matmul(to_mul(a).astype(np.float64), to_mul(b).astype(np.float64)).astype(np.float32)
+    if accumulator_type(precision) == "f16":
+        r = r.astype(np.float16).astype(np.float32)
+    return r
+
+
+def evaluate(nodes, inputs, materialize=False):
+    """Evaluates the graph. `inputs`: {input id: storage array}. Returns {node id: math-domain array} for every
+    node plus the descriptors. With materialize=True every intermediate is rounded to its storage dtype (what
+    happens when each op runs as its own kernel); with False none is (one fused kernel)."""
+    desc, val = {}, {}
+    for n in nodes:
+        i = n["id"]
+        if n["node"] == "input":
+            desc[i] = (list(n["shape"]), n["dtype"])
+            val[i] = nm.from_storage(inputs[i], n["dtype"], n["shape"])
+        elif n["node"] == "output":
+            desc[i] = desc[n["from"]]
+            val[i] = val[n["from"]]
+        else:
+            desc[i] = infer(n, desc)
+            val[i] = _eval_op(n, desc, val)
+            shape, dtype = desc[i]
+            assert list(val[i].shape) == list(shape), (n, val[i].shape, shape)
+            if materialize:
+                val[i] = nm.from_storage(nm.to_storage(val[i], dtype), dtype, shape)
+    return val, desc
+
+
+def _eval_op(n, desc, val):
+    op, ins = n["op"], n["inputs"]
+    if op == "unary":
+        return unary(n["fn"], val[ins[0]])
+    if op == "binary":
+        return binary(n["fn"], val[ins[0]], val[ins[1]])
+    if op == "change_dtype":
+        return cast_class(val[ins[0]], desc[ins[0]][1], n["target"])
+    if op == "reduce":
+        return reduce(n["fn"], val[ins[0]], n["depth"])
+    if op == "broadcast":
+        shape, _ = infer(n, desc)
+        x = val[ins[0]]
+        x = x.reshape([1] * (len(shape) - x.ndim) + list(x.shape))
+        # a listed axis always reads coordinate 0 of the input (jit.rs:877-879)
+        index = tuple(slice(0, 1) if any(a == ax for ax, _ in n["axes"]) else slice(None) for a in range(len(shape)))
+        return np.ascontiguousarray(np.broadcast_to(x[index], shape))
+    if op == "reshape":
+        return val[ins[0]].reshape(n["new_shape"])
+    if op == "swap_dims":
+        return np.ascontiguousarray(np.swapaxes(val[ins[0]], n["axis_a"], n["axis_b"]))
+    if op == "compare":
+        return compare(n["fn"], val[ins[0]], val[ins[1]])
+    if op == "select":
+        return np.where(val[ins[2]], val[ins[1]], val[ins[0]])  # rhs where the selector is true
+    if op == "constant":
+        dt = n["const_dtype"]
+        math = nm.from_storage(nm.to_storage(np.array([n["value"]]), dt), dt, [1]) if dt != "bool" else np.array([bool(n["value"])])
+        return np.ascontiguousarray(np.broadcast_to(math.reshape([1] * len(n["shape"])), n["shape"]))
+    if op == "matmul":
+        return matmul(val[ins[0]], val[ins[1]], n["precision"], desc[ins[0]][1], desc[ins[1]][1])
+    raise ValueError(op)
+
+
+def kernel_outputs(nodes, inputs, leaf_ids):
+    """Storage-domain outputs of ONE fused kernel whose leaves are `leaf_ids`."""
+    val, desc = evaluate(nodes, inputs, materialize=False)
+    return {i: nm.to_storage(val[i], desc[i][1]) for i in leaf_ids}

@@ -33,6 +33,45 @@ static pthread_barrier_t g_bar;
 #define __syncthreads() pthread_barrier_wait(&g_bar)
 #define __builtin_nontemporal_load(p) (*(p))
 #define __builtin_nontemporal_store(v, p) (*(p) = (v))
+#include <cmath>
+// wave shuffles: every thread of the block calls in lockstep, so a block-wide exchange through memory works
+static float g_shfl[1024];
+static inline float __shfl_xor(float v, int mask, int width) {
+    unsigned tid = threadIdx.x;
+    g_shfl[tid] = v;
+    pthread_barrier_wait(&g_bar);
+    float r = g_shfl[(tid & ~63u) | ((tid & 63u) ^ (unsigned)mask)];
+    pthread_barrier_wait(&g_bar);
+    return r;
+}
+static inline int __float_as_int(float f) { int i; memcpy(&i, &f, 4); return i; }
+static inline unsigned __float_as_uint(float f) { unsigned i; memcpy(&i, &f, 4); return i; }
+static inline float atomicAdd(float* a, float v) {
+    unsigned* ua = (unsigned*)a; unsigned old = __atomic_load_n(ua, __ATOMIC_RELAXED), nw;
+    float f;
+    do { memcpy(&f, &old, 4); f += v; memcpy(&nw, &f, 4); } while (!__atomic_compare_exchange_n(ua, &old, nw, false, __ATOMIC_SEQ_CST, __ATOMIC_RELAXED));
+    return f;
+}
+template <class T> static inline T atomicMax(T* a, T v) {
+    T old = __atomic_load_n(a, __ATOMIC_RELAXED);
+    while (old < v && !__atomic_compare_exchange_n(a, &old, v, false, __ATOMIC_SEQ_CST, __ATOMIC_RELAXED)) {}
+    return old;
+}
+template <class T> static inline T atomicMin(T* a, T v) {
+    T old = __atomic_load_n(a, __ATOMIC_RELAXED);
+    while (old > v && !__atomic_compare_exchange_n(a, &old, v, false, __ATOMIC_SEQ_CST, __ATOMIC_RELAXED)) {}
+    return old;
+}
+static inline unsigned atomicOr(unsigned* a, unsigned v) { return __atomic_fetch_or(a, v, __ATOMIC_SEQ_CST); }
+#define __expf expf
+#define __logf logf
+#define __sinf sinf
+#define __cosf cosf
+#define __tanf tanf
+#define __powf powf
+static inline float he_fdividef(float x, float y) { return x / y; }
+#define __fdividef he_fdividef
+#define __fsqrt_rn sqrtf
 """
 
 MAIN = r"""
@@ -59,7 +98,7 @@ int main(int argc, char** argv) {
     for (int i = 0; i < nb; i++) {
         sizes[i] = strtoull(argv[4 + 3 * i], nullptr, 10); isout[i] = atoi(argv[5 + 3 * i]);
         bufs[i] = malloc(sizes[i] ? sizes[i] : 1);
-        if (!isout[i]) { FILE* f = fopen(argv[3 + 3 * i], "rb"); if (fread(bufs[i], 1, sizes[i], f) != sizes[i]) return 3; fclose(f); }
+        if (isout[i] != 1) { FILE* f = fopen(argv[3 + 3 * i], "rb"); if (fread(bufs[i], 1, sizes[i], f) != sizes[i]) return 3; fclose(f); }
         else memset(bufs[i], 0xEE, sizes[i]);
     }
     g_bufs = bufs.data();
@@ -74,23 +113,24 @@ int main(int argc, char** argv) {
 """
 
 
-def run_kernel(source, entry, grid, threads, buffers):
-    """buffers: list of (numpy array, is_output). Returns the output arrays (same dtype/shape as given)."""
+def run_kernel(source, entry, grid, threads, buffers, flags=()):
+    """buffers: list of (numpy array, mode) with mode False/0 = input, True/1 = output (starts as 0xEE bytes),
+    2 = in-out (starts from the array's contents). Returns the output arrays (same dtype/shape as given)."""
     with tempfile.TemporaryDirectory() as d:
         src = os.path.join(d, "k.cpp")
         with open(src, "w") as f:
             f.write(SHIM + source + f"\n#define ENTRY {entry}\n" + MAIN)
         exe = os.path.join(d, "k")
         subprocess.check_call([CLANG, "-O1", "-g", "-std=c++17", "-fsanitize=address", "-fno-omit-frame-pointer",
-                               "-pthread", src, "-o", exe])
+                               "-pthread", *flags, src, "-o", exe])
         argv = [exe, str(grid), str(threads)]
         paths = []
         for i, (a, is_out) in enumerate(buffers):
             p = os.path.join(d, f"b{i}.bin")
             paths.append(p)
-            if not is_out:
+            if int(is_out) != 1:
                 np.ascontiguousarray(a).tofile(p)
-            argv += [p, str(a.nbytes), "1" if is_out else "0"]
+            argv += [p, str(a.nbytes), str(int(is_out))]
         res = subprocess.run(argv, capture_output=True, text=True, env={**os.environ, "ASAN_OPTIONS": "detect_leaks=0"})
         if res.returncode != 0:
             raise AssertionError(f"CPU emulation of {entry} failed (exit {res.returncode}):\n{res.stderr[-4000:]}")

@@ -1,0 +1,140 @@
+"""Shared test helpers: front-end lowerings (as helium/src/raw_tensor.rs writes them), runners that execute one
+tile kernel either on the GPU through the C ABI or on the CPU under the emulation shim, and comparison helpers."""
+import re
+
+import numpy as np
+
+from oracle import helium_ir as oracle_ir
+from oracle import numerics as nm
+
+
+# ---- front-end lowerings (helium/src/raw_tensor.rs) ---------------------------------------------------------
+def scalar_tensor(g, value, like_shape):
+    """`x op f32`: a 1-element f32 input broadcast to x's shape (raw_tensor.rs:638-645, broadcast_to :389-414).
+    Returns (broadcast node, scalar input node, scalar storage)."""
+    s = g.new_input([1], "f32")
+    rank = len(like_shape)
+    axes = []
+    if like_shape[-1] != 1:
+        axes.append((rank - 1, like_shape[-1]))
+    for i in range(rank - 1):
+        axes.append((i, like_shape[i]))
+    b = g.broadcast(s, rank, axes)
+    return b, s, np.array([value], dtype=np.float32)
+
+
+def broadcast_to(g, x, x_shape, new_shape):
+    """RawTensor::broadcast_to (raw_tensor.rs:370-424)."""
+    d, d2 = len(x_shape), len(new_shape)
+    axes = []
+    for rev, (old, new) in enumerate(zip(reversed(x_shape), reversed(new_shape))):
+        index = d2 - rev - 1
+        if old != 1:
+            assert old == new
+        if old == 1 and new != 1:
+            axes.append((index, new))
+    for i in range(d2 - d):
+        axes.append((i, new_shape[i]))
+    return g.broadcast(x, d2, axes)
+
+
+def sub(g, a, b):
+    return g.binary(a, g.unary(b, "neg"), "add")  # a - b = a + (-b), raw_tensor.rs:647-653
+
+
+def div(g, a, b):
+    return g.binary(a, g.unary(b, "recip"), "mul")  # a / b = a * recip(b), raw_tensor.rs:679-686
+
+
+# ---- runners -----------------------------------------------------------------------------------------------
+def _launch_numbers(desc):
+    return int(re.search(r"grid=(\d+)", desc).group(1)), int(re.search(r"threads=(\d+)", desc).group(1))
+
+
+def run_tile_kernel_gpu(kernel, inputs_by_node):
+    """Executes on the GPU; returns {leaf node: storage array}."""
+    from helium_amd import DeviceBuffer
+
+    bufs, outs = [], {}
+    for a in kernel.args:
+        nbytes = _storage_bytes(a)
+        if a["is_output"]:
+            b = DeviceBuffer(max(nbytes, 4))
+            b.fill_u8(0xEE)
+            outs[a["node"]] = (b, a)
+        else:
+            host = np.ascontiguousarray(inputs_by_node[a["node"]])
+            assert host.nbytes == nbytes, (a, host.nbytes, nbytes)
+            b = DeviceBuffer.from_numpy(host) if nbytes else DeviceBuffer(4)
+        bufs.append(b)
+    kernel.execute(bufs)
+    return {node: b.to_numpy(nm.NP_STORAGE[a["dtype"]])[: _storage_elems(a)] for node, (b, a) in outs.items()}
+
+
+def _storage_bytes(a):
+    if a["dtype"] == "bool":
+        return (a["numel"] + 31) // 32 * 4
+    return a["numel"] * np.dtype(nm.NP_STORAGE[a["dtype"]]).itemsize
+
+
+def _storage_elems(a):
+    return (a["numel"] + 31) // 32 if a["dtype"] == "bool" else a["numel"]
+
+
+def run_tile_kernel_cpu(kernel, inputs_by_node, entry, fills):
+    """Executes the generated source on the CPU (tests/cpu_emul.py). `fills`: {leaf node: 32-bit pattern} for the
+    outputs the launch pre-fills (reduction identities, zeroed bitsets)."""
+    from cpu_emul import run_kernel
+
+    grid, threads = _launch_numbers(kernel.description)
+    buffers, order = [], []
+    for a in kernel.args:
+        dt = nm.NP_STORAGE[a["dtype"]]
+        if a["is_output"]:
+            if a["node"] in fills:  # pre-filled outputs are 32-bit typed (f32 reductions, u32 bitsets)
+                buffers.append((np.full(_storage_elems(a), fills[a["node"]], dtype=np.uint32).view(dt), 2))
+            else:
+                buffers.append((np.empty(_storage_elems(a), dtype=dt), 1))
+            order.append(a["node"])
+        else:
+            buffers.append((np.ascontiguousarray(inputs_by_node[a["node"]]), 0))
+    outs = run_kernel(kernel.source, entry, grid, threads, buffers)
+    return dict(zip(order, outs))
+
+
+def reduction_fills(graph_nodes, leaf_ids):
+    """32-bit fill pattern per reduction / bitset leaf, as PointwiseGraph::execute initialises them
+    (helium/src/cuda/instr/pointwise.rs:62-74,113-119)."""
+    by_id = {n["id"]: n for n in graph_nodes}
+    fills = {}
+    for leaf in leaf_ids:
+        n = by_id[leaf]
+        if n.get("op") == "reduce":
+            ident = {"sum": 0.0, "mean": 0.0, "max": -np.inf, "min": np.inf}[n["fn"]]
+            fills[leaf] = int(np.array([ident], dtype=np.float32).view(np.uint32)[0])
+        elif n.get("dtype") == "bool":
+            fills[leaf] = 0
+    return fills
+
+
+# ---- comparison --------------------------------------------------------------------------------------------
+def assert_storage_close(got, want, dtype, what="", max_ulps=2, reduce_rel=None):
+    """Float outputs: the reference tests' ulps criterion on the f32 value (bf16/f16 outputs: at most one step of
+    the storage format apart). `reduce_rel`: relative tolerance for reductions (summation order is free)."""
+    if dtype in ("u32", "bool"):
+        assert np.array_equal(got, want), what
+        return
+    if dtype == "f32":
+        g, w = np.asarray(got, np.float32), np.asarray(want, np.float32)
+        if reduce_rel is not None:
+            ok = np.isclose(g.astype(np.float64), w.astype(np.float64), rtol=reduce_rel, atol=1e-6) | (g == w)
+        else:
+            ok = nm.ulps_close(g, w, max_ulps=max_ulps)
+    else:
+        conv = nm.bf16_bits_to_f32 if dtype == "bf16" else nm.f16_bits_to_f32
+        diff = np.abs(np.asarray(got, np.uint16).astype(np.int32) - np.asarray(want, np.uint16).astype(np.int32))
+        ok = (diff <= 1) | (np.isnan(conv(got)) & np.isnan(conv(want)))
+    if not ok.all():
+        bad = np.flatnonzero(~ok.reshape(-1))[:5]
+        raise AssertionError(f"{what}: {(~ok).sum()} of {ok.size} elements differ, e.g. at {bad}: got "
+                             f"{np.asarray(got).reshape(-1)[bad]} want {np.asarray(want).reshape(-1)[bad]}")
