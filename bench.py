@@ -21,6 +21,7 @@ sys.path.insert(0, ROOT)
 METRIC = "fused-GEMM TFLOP/s & permute/pointwise GB/s, % of MI355X roofline"
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 BF16_PEAK_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
+HEADLINE = "C2a"             # the workload `value` is quoted on
 ROTATE_BYTES = 768 << 20     # rotate operand sets so repeated steps cannot live in the 256 MB Infinity Cache
 
 
@@ -97,18 +98,90 @@ class PermuteWorkload:
         self.sets = []
 
 
-def make_workloads():
-    w = {
-        "C2a": PermuteWorkload("C2a", (64, 56, 56, 256), (0, 3, 1, 2), 21),
-        "C2b": PermuteWorkload("C2b", (4096, 4096), (1, 0), 22),
-        "C2c": PermuteWorkload("C2c", (32, 128, 28, 28), (0, 2, 3, 1), 23),
-    }
-    try:
-        import bench_workloads  # optional: further workloads (pointwise chain, fused GEMM) register here
+class AuxChainWorkload:
+    """BASELINE config 3: the 10-op f32 pointwise chain ending in Sum(batch) and Sum(columns), one fused kernel.
+    Algorithmic bytes: four [1,4096,4096] f32 inputs + the bias + both outputs = 268,468,228."""
 
-        bench_workloads.register(w)
-    except ImportError:
-        pass
+    bound = "hbm"
+    unit = "GB/s"
+    dtype = "f32"
+    name = "C3"
+
+    def __init__(self):
+        self.work = 4 * 4096 * 4096 * 4 + 4096 * 4 + (4096 + 1) * 4
+
+    def describe(self):
+        return "C3: f32 [1,4096,4096] 10-op chain + Sum(batch) + Sum(columns), one kernel"
+
+    def setup(self):
+        import helium_amd as ha
+        from helium_amd import configs
+
+        self.graph, self.inputs, self.outs = configs.c3_chain()
+        self.kernel = ha.TileKernel.auxiliary(self.graph)
+        nsets = 4  # 4 x 268 MB of operands rotate through the caches
+        self.sets = []
+        for s in range(nsets):
+            bufs = []
+            for a in self.kernel.args:
+                if a["is_output"]:
+                    bufs.append(ha.DeviceBuffer(a["numel"] * 4))
+                else:
+                    bufs.append(ha.DeviceBuffer.from_numpy(self.inputs[a["node"]]))
+            self.sets.append(bufs)
+        log(f"[bench] {self.describe()} :: {self.kernel.description} :: {nsets} operand sets")
+
+    def step(self, stream, i):
+        self.kernel.execute(self.sets[i % len(self.sets)], stream)
+
+    def check(self):
+        from oracle import fusion_ir as oracle
+
+        want = oracle.outputs(self.graph.nodes, self.inputs)
+        for a, buf in zip(self.kernel.args, self.sets[0]):
+            if not a["is_output"]:
+                continue
+            got = buf.to_numpy(np.float32)[: a["numel"]]
+            w = want[a["node"]].reshape(-1)
+            err = np.max(np.abs(got.astype(np.float64) - w) / np.maximum(np.abs(w), 1e-30))
+            if not err <= 1e-3:
+                raise SystemExit(f"[bench] PARITY FAILURE in C3 output {a['node']}: max rel err {err}")
+        return "reductions within 1e-3 relative of the f64-summed oracle"
+
+    def cpu_baseline(self, budget_s=20.0):
+        from oracle import fusion_ir as oracle
+
+        rows = 512  # bounded sample: the first 512 of 4096 rows of every operand
+        sample = {k: np.ascontiguousarray(v[:, :rows]) if v.shape[1] == 4096 else v for k, v in self.inputs.items()}
+        nodes = [dict(n) for n in self.graph.nodes]
+        for n in nodes:
+            if n["op"] == "producer" and n["shape"][1] == 4096:
+                n["shape"] = [1, rows, n["shape"][2]]
+            if n["op"] == "broadcast" and n["axis"] == 1:
+                n["amount"] = rows
+        best, reps, t_all = 1e30, 0, time.perf_counter()
+        while reps < 2 or (time.perf_counter() - t_all < budget_s and reps < 5):
+            t0 = time.perf_counter()
+            oracle.evaluate(nodes, sample)
+            best = min(best, time.perf_counter() - t0)
+            reps += 1
+        work = self.work * rows / 4096
+        return {"value": round(work / best / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"first {rows} of 4096 rows of the C3 operands, numpy oracle, best of {reps} passes"}
+
+    def free(self):
+        for bufs in self.sets:
+            for b in bufs:
+                b.free()
+        self.sets = []
+
+
+def make_workloads():
+    from helium_amd import configs
+
+    w = {name: PermuteWorkload(name, shape, perm, {"C2a": 21, "C2b": 22, "C2c": 23}[name])
+         for name, (shape, perm) in configs.PERMUTES.items()}
+    w["C3"] = AuxChainWorkload()
     return w
 
 
@@ -163,7 +236,7 @@ def main():
     log(f"[bench] device 0: {arch}, {cus} CUs; roofline constants: HBM {HBM_PEAK_GBS} GB/s, "
         f"bf16 MFMA {BF16_PEAK_TFLOPS} TFLOP/s")
     workloads = make_workloads()
-    headline = args.workload or getattr(sys.modules.get("bench_workloads"), "HEADLINE", "C2a")
+    headline = args.workload or HEADLINE
     if headline not in workloads:
         raise SystemExit(f"unknown workload {headline}; have {sorted(workloads)}")
     stream = ha.Stream()

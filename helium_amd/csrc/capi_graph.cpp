@@ -12,8 +12,7 @@ struct he_fgraph_s {
     he::fir::OpGraph g;
 };
 struct he_tile_kernel_s {
-    std::unique_ptr<he::TileKernel> k;
-    std::string describe;
+    std::unique_ptr<he::KernelBase> k;
 };
 
 namespace he {
@@ -113,13 +112,24 @@ int he_aux_kernel_create(he_tile_kernel_t* kernel, he_fgraph_t graph) {
         *kernel = k.release();
     });
 }
+int he_fused_kernel_create(he_tile_kernel_t* kernel, he_fgraph_t graph) {
+    return he::guard([&] {
+        HE_REQUIRE(kernel && graph, HE_ERR_INVALID, "bad argument");
+        auto k = std::make_unique<he_tile_kernel_s>();
+        if (graph->g.anchor() == he::fir::kNoOpNode)
+            k->k.reset(new he::TileKernel(he::tp::lower_aux(graph->g), "fused_auxiliary"));
+        else
+            k->k.reset(new he::GemmKernel(he::gemm_problem_from_fusion(graph->g)));
+        *kernel = k.release();
+    });
+}
 int he_tile_kernel_num_args(he_tile_kernel_t kernel, int* count) {
-    return he::guard([&] { *count = (int)kernel->k->program().args.size(); });
+    return he::guard([&] { *count = (int)kernel->k->args().size(); });
 }
 int he_tile_kernel_arg_info(he_tile_kernel_t kernel, int index, uint64_t* node, int32_t* is_output, int32_t* dtype,
                             int64_t* numel) {
     return he::guard([&] {
-        const auto& args = kernel->k->program().args;
+        const auto& args = kernel->k->args();
         HE_REQUIRE(index >= 0 && index < (int)args.size(), HE_ERR_INVALID, "argument index out of range");
         *node = args[index].node;
         *is_output = args[index].is_output;
@@ -130,14 +140,14 @@ int he_tile_kernel_arg_info(he_tile_kernel_t kernel, int index, uint64_t* node, 
 int he_tile_kernel_execute(he_tile_kernel_t kernel, void* const* arg_ptrs, int num_args, he_stream_t stream) {
     return he::guard([&] {
         HE_REQUIRE(kernel && arg_ptrs, HE_ERR_INVALID, "bad argument");
-        HE_REQUIRE(num_args == (int)kernel->k->program().args.size(), HE_ERR_INVALID, "kernel takes %zu arguments, got %d",
-                   kernel->k->program().args.size(), num_args);
+        HE_REQUIRE(num_args == (int)kernel->k->args().size(), HE_ERR_INVALID, "kernel takes %zu arguments, got %d",
+                   kernel->k->args().size(), num_args);
         kernel->k->execute(arg_ptrs, stream ? stream->s : nullptr);
     });
 }
 const char* he_tile_kernel_source(he_tile_kernel_t kernel) { return kernel ? kernel->k->source().c_str() : ""; }
 const char* he_tile_kernel_describe(he_tile_kernel_t kernel) {
-    return kernel ? kernel->k->launch_info().describe.c_str() : "";
+    return kernel ? kernel->k->describe().c_str() : "";
 }
 int he_tile_kernel_destroy(he_tile_kernel_t kernel) {
     delete kernel;

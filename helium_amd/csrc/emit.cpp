@@ -369,7 +369,17 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
     }
     const int NV = pick_nv(p, 16);
     const int threads = 256;
-    int TX = (int)std::min<int64_t>(threads, pow2_ceil((N + NV - 1) / NV));
+    bool any_col = false, any_scalar = false;
+    for (auto& o : p.outs) {
+        if (!o.reduce) continue;
+        if (o.fold_m && !o.fold_n) any_col = true;
+        if (o.fold_m && o.fold_n) any_scalar = true;
+    }
+    // Threads along a row. With a column reduction a block should be tall rather than wide: its TY row groups are
+    // combined in LDS, so every block issues one atomic per column it spans, not one per column per row group.
+    int tx_cap = any_col ? 64 : threads;
+    if (const char* env = getenv("HELIUM_HIP_POINTWISE_TX")) tx_cap = std::max(1, atoi(env));
+    int TX = (int)std::min<int64_t>(tx_cap, pow2_ceil((N + NV - 1) / NV));
     int TY = threads / TX;
     const int64_t gx = (N + (int64_t)TX * NV - 1) / ((int64_t)TX * NV);
     const int64_t gy1 = (M + TY - 1) / TY;
@@ -392,13 +402,6 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
     L.ty = TY;
     L.rpt = RPT;
     L.options = {p.fast_math ? "-ffp-contract=fast" : "-ffp-contract=off", "-munsafe-fp-atomics"};
-
-    bool any_col = false, any_scalar = false;
-    for (auto& o : p.outs) {
-        if (!o.reduce) continue;
-        if (o.fold_m && !o.fold_n) any_col = true;
-        if (o.fold_m && o.fold_n) any_scalar = true;
-    }
 
     std::ostringstream s;
     s << "// pointwise kernel generated for gfx950: dims=[";

@@ -1,0 +1,472 @@
+// Fused GEMM generator for gfx950: bf16/f16 MFMA (v_mfma_f32_32x32x16) with f32 accumulators.
+//
+//   * Operand tiles are staged global -> registers -> LDS. Mainloop op chains (e.g. Relu, Mul by a tensor) run in
+//     f32 on the staged registers and are rounded to the multiplicand type before they reach LDS, so every
+//     element is computed once per workgroup and the MFMA loop reads finished operands.
+//   * A tiles sit in LDS as [m][k] (k contiguous, 16-byte chunks XOR-swizzled by m), read with one 128-bit LDS
+//     load per MFMA operand. B tiles sit as [k][n] exactly as they are in memory and are read with the
+//     transposing LDS load of gfx950 (ds_read_b64_tr_b16), which hands every lane the 4 consecutive k it needs.
+//   * The epilogue program runs on the f32 accumulators: each wave passes its accumulators through a private LDS
+//     strip to get row-major vectors of NV consecutive columns, so auxiliary tensors are read and outputs written
+//     with coalesced 16-byte accesses; column / row / scalar reductions are folded per lane, combined with wave
+//     shuffles and finished with one atomic per wave and output element.
+#include <cmath>
+#include <cstring>
+#include <sstream>
+
+#include "kernels.h"
+
+namespace he {
+
+namespace {
+
+struct Tile {
+    int bm = 256, bn = 256, bk = 64;  // workgroup tile
+    int wm = 2, wn = 2;               // waves along m / n (wm * wn * 64 threads)
+};
+
+const char* kGemmPrelude = R"HIP(
+typedef u32 u32x4 __attribute__((ext_vector_type(4)));
+typedef u32 u32x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+#ifndef LDS_AS
+#define LDS_AS __attribute__((address_space(3)))
+#endif
+)HIP";
+
+// Helpers that depend on the problem constants.
+const char* kGemmHelpers = R"HIP(
+__device__ __forceinline__ u32x4 pack8(const float (&v)[8]) {
+#if MMA_BF16
+    bf16x8 r;
+#pragma unroll
+    for (int j = 0; j < 8; j++) r[j] = (__bf16)v[j];
+#else
+    f16x8 r;
+#pragma unroll
+    for (int j = 0; j < 8; j++) r[j] = (_Float16)v[j];
+#endif
+    return __builtin_bit_cast(u32x4, r);
+}
+)HIP";
+
+// Kernel body; problem and tile constants are #defines in front of it.
+const char* kGemmBody = R"HIP(
+#define NTHREADS (WAVES_M * WAVES_N * 64)
+#define WTM (BM / WAVES_M)        /* wave tile */
+#define WTN (BN / WAVES_N)
+#define MB (WTM / 32)             /* 32x32 MFMA blocks per wave tile */
+#define NB (WTN / 32)
+#define A_CHUNKS (BK / 8)         /* 16-byte chunks per A row */
+#define B_CHUNKS (BN / 8)
+#define A_TILE_BYTES (BM * BK * 2)
+#define B_TILE_BYTES (BK * BN * 2)
+#define STAGE_BYTES (A_TILE_BYTES + B_TILE_BYTES)
+#define A_PER_THREAD (BM * A_CHUNKS / NTHREADS)
+#define B_PER_THREAD (BK * B_CHUNKS / NTHREADS)
+#define EP (WTN + 4)              /* float pitch of the epilogue strip */
+#define KT ((GK + BK - 1) / BK)
+
+__device__ __forceinline__ u32 a_off(u32 m, u32 kc) { return m * (BK * 2) + ((kc ^ (m & (A_CHUNKS - 1))) << 4); }
+__device__ __forceinline__ u32 b_off(u32 k, u32 n) {
+    return k * (BN * 2) + ((((n >> 3) ^ ((k & 3) << 2))) << 4) + ((n & 7) << 1);
+}
+
+#ifndef KERNEL_ATTRS
+#define KERNEL_ATTRS __attribute__((amdgpu_waves_per_eu(1, 1)))  /* one wave per SIMD: the full 512-register budget */
+#endif
+extern "C" __global__ __launch_bounds__(NTHREADS) KERNEL_ATTRS
+void fused_matmul(KERNEL_PARAMS) {
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * STAGE_BYTES];
+    const u32 tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const u32 wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+    // Tile order: consecutive workgroups walk down a column of tiles, so the workgroups resident at the same time
+    // share B panels (and, through the XCD round-robin, spread A panels over all L2s).
+    const u32 tiles_m = (GM + BM - 1) / BM;
+    const u32 tile_m = blockIdx.x % tiles_m, tile_n = blockIdx.x / tiles_m;
+    const u32 bz = blockIdx.y;
+    const u32 m0 = tile_m * BM, n0 = tile_n * BN;
+
+    f32x16 acc[MB][NB];
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+#pragma unroll
+        for (int j = 0; j < NB; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
+
+    u32x4 sa[A_PER_THREAD], sb[B_PER_THREAD];
+    auto stage_load = [&](u32 kt) {
+        const u32 k0 = kt * BK;
+#pragma unroll
+        for (int i = 0; i < A_PER_THREAD; i++) {
+            const u32 idx = tid + i * NTHREADS;
+            const u32 row = idx / A_CHUNKS, kc = idx % A_CHUNKS;
+            sa[i] = fetch_a(FETCH_A_ARGS bz, m0 + row, k0 + kc * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < B_PER_THREAD; i++) {
+            const u32 idx = tid + i * NTHREADS;
+            const u32 krow = idx / B_CHUNKS, nc = idx % B_CHUNKS;
+            sb[i] = fetch_b(FETCH_B_ARGS bz, k0 + krow, n0 + nc * 8);
+        }
+    };
+    auto stage_store = [&](u32 buf) {
+        unsigned char* la = lds + buf * STAGE_BYTES;
+        unsigned char* lb = la + A_TILE_BYTES;
+#pragma unroll
+        for (int i = 0; i < A_PER_THREAD; i++) {
+            const u32 idx = tid + i * NTHREADS;
+            *(u32x4*)(la + a_off(idx / A_CHUNKS, idx % A_CHUNKS)) = sa[i];
+        }
+#pragma unroll
+        for (int i = 0; i < B_PER_THREAD; i++) {
+            const u32 idx = tid + i * NTHREADS;
+            *(u32x4*)(lb + b_off(idx / B_CHUNKS, (idx % B_CHUNKS) * 8)) = sb[i];
+        }
+    };
+    auto compute = [&](u32 buf) {
+        const unsigned char* la = lds + buf * STAGE_BYTES;
+        const unsigned char* lb = la + A_TILE_BYTES;
+        const u32 g = lane >> 4, r = lane & 15;
+#pragma unroll
+        for (int kk = 0; kk < BK / 16; kk++) {
+            s16x8 af[MB], bf[NB];
+#pragma unroll
+            for (int i = 0; i < MB; i++) {
+                const u32 row = wave_m * WTM + i * 32 + (lane & 31);
+                af[i] = *(const s16x8*)(la + a_off(row, kk * 2 + (lane >> 5)));
+            }
+#pragma unroll
+            for (int j = 0; j < NB; j++) {
+                const u32 k = kk * 16 + (g >> 1) * 8 + (r >> 2);
+                const u32 n = wave_n * WTN + j * 32 + (g & 1) * 16 + (r & 3) * 4;
+                s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(lb + b_off(k, n)));
+                s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(lb + b_off(k + 4, n)));
+                bf[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+#pragma unroll
+            for (int i = 0; i < MB; i++)
+#pragma unroll
+                for (int j = 0; j < NB; j++) {
+#if MMA_BF16
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[i]),
+                                                                       __builtin_bit_cast(bf16x8, bf[j]), acc[i][j], 0, 0, 0);
+#else
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, af[i]),
+                                                                      __builtin_bit_cast(f16x8, bf[j]), acc[i][j], 0, 0, 0);
+#endif
+                }
+        }
+    };
+
+    stage_load(0);
+    stage_store(0);
+    __syncthreads();
+    for (u32 kt = 0; kt < KT; kt++) {
+        const bool more = kt + 1 < KT;
+        if (more) stage_load(kt + 1);
+        compute(kt & 1);
+        if (more) stage_store((kt + 1) & 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: accumulators -> wave-private LDS strip -> row-major NV-wide vectors -----------------------
+    float* strip = (float*)lds + wave * (32 * EP);
+    EPILOGUE_SETUP
+#pragma unroll
+    for (int i = 0; i < MB; i++) {
+#pragma unroll
+        for (int j = 0; j < NB; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const u32 row = (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3), col = j * 32 + (lane & 31);
+                strip[row * EP + col] = acc[i][j][e];
+            }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int step = 0; step < (32 * WTN) / (64 * NVE); step++) {
+            const u32 idx = (step * 64 + lane) * NVE;
+            const u32 row = idx / WTN, col = idx % WTN;
+            const u32 m = m0 + wave_m * WTM + i * 32 + row;
+            const u32 nn = n0 + wave_n * WTN + col;
+            float acc_v[NVE];
+#pragma unroll
+            for (int k = 0; k < NVE; k++) acc_v[k] = strip[row * EP + col + k];
+            const bool ok = m < GM && nn < GN;
+            EPILOGUE_BODY
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    EPILOGUE_FINISH
+}
+)HIP";
+
+bool is_raw_copy(const tp::Program& p, int root, int mma_dtype) {
+    const tp::Expr& e = p.exprs[root];
+    if (e.kind != tp::Expr::Load || !e.access.chain.empty() || e.access.dtype != mma_dtype) return false;
+    return e.access.stride == ir::packed_strides(p.dims);
+}
+
+// A __device__ function that evaluates an operand program for NV consecutive columns at (b, row, col).
+std::string emit_operand_fn(const tp::Program& p, int root, const std::string& name, int nv) {
+    std::ostringstream s;
+    s << "__device__ __forceinline__ void " << name << "(";
+    for (size_t a = 0; a < p.args.size(); a++) s << "const " << tp::c_type(p.args[a].dtype) << "* __restrict__ a" << a << ", ";
+    s << "u32 cB0, u32 m, u32 n0, float* out) {\n(void)cB0;\n";
+    tp::EmitCtx cx;
+    cx.nv = nv;
+    s << tp::emit_exprs(p, cx);
+    s << "#pragma unroll\nfor (int k = 0; k < " << nv << "; k++) out[k] = e" << root << "[k];\n}\n";
+    return s.str();
+}
+
+}  // namespace
+
+GemmProblem gemm_problem_from_fusion(const fir::OpGraph& g) {
+    GemmProblem pr;
+    fir::OpNode anchor = g.anchor();
+    HE_REQUIRE(anchor != fir::kNoOpNode, HE_ERR_UNSUPPORTED, "fusion has no Matmul anchor");
+    int anchors = 0;
+    for (fir::OpNode n : g.nodes()) anchors += g.get(n).is_anchor();
+    HE_REQUIRE(anchors == 1, HE_ERR_UNSUPPORTED, "a Core fusion holds exactly one Matmul");
+    const fir::Op& mm = g.get(anchor);
+    const fir::Shape3 &sa = g.shape(mm.a), &sc = g.shape(anchor);
+    pr.batch = sc[0];
+    pr.M = sc[1];
+    pr.N = sc[2];
+    pr.K = sa[2];
+    pr.op_a = tp::lower_operand(g, mm.a, &pr.root_a);
+    pr.op_b = tp::lower_operand(g, mm.b, &pr.root_b);
+    pr.epi = tp::lower_epilogue(g, anchor);
+    // Multiplicand type: f16 when every operand source is f16, bf16 otherwise (f32 sources are rounded to bf16,
+    // the reference's MulBf16AccumF32).
+    bool all_f16 = true;
+    for (auto* p : {&pr.op_a, &pr.op_b})
+        for (auto& a : p->args) all_f16 = all_f16 && a.dtype == HE_F16;
+    pr.mma_dtype = all_f16 ? HE_F16 : HE_BF16;
+
+    // Kernel arguments: every distinct producer in id order, then every output in leaf order.
+    std::vector<tp::Arg> inputs, outputs;
+    auto add_input = [&](const tp::Arg& a) {
+        for (auto& x : inputs)
+            if (x.node == a.node) return;
+        inputs.push_back(a);
+    };
+    for (auto* p : {&pr.op_a, &pr.op_b, &pr.epi})
+        for (auto& a : p->args) {
+            if (a.is_output) outputs.push_back(a);
+            else add_input(a);
+        }
+    std::sort(inputs.begin(), inputs.end(), [](const tp::Arg& x, const tp::Arg& y) { return x.node < y.node; });
+    pr.args = inputs;
+    pr.args.insert(pr.args.end(), outputs.begin(), outputs.end());
+    auto map_of = [&](const tp::Program& p) {
+        std::vector<int> m;
+        for (auto& a : p.args)
+            for (size_t k = 0; k < pr.args.size(); k++)
+                if (pr.args[k].node == a.node && pr.args[k].is_output == a.is_output) {
+                    m.push_back((int)k);
+                    break;
+                }
+        HE_REQUIRE(m.size() == p.args.size(), HE_ERR_INTERNAL, "argument mapping failed");
+        return m;
+    };
+    pr.map_a = map_of(pr.op_a);
+    pr.map_b = map_of(pr.op_b);
+    pr.map_e = map_of(pr.epi);
+    return pr;
+}
+
+GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
+    const GemmProblem& pr = prob_;
+    HE_REQUIRE(pr.M > 0 && pr.N > 0 && pr.K > 0 && pr.batch > 0, HE_ERR_INVALID, "empty GEMM");
+    HE_REQUIRE(pr.M < (1ll << 31) && pr.N < (1ll << 31) && pr.K < (1ll << 31) &&
+                   pr.batch * pr.M * std::max(pr.N, pr.K) < (1ll << 40),
+               HE_ERR_INVALID, "GEMM too large");
+    HE_REQUIRE(pr.mma_dtype == HE_BF16 || pr.mma_dtype == HE_F16, HE_ERR_UNSUPPORTED, "unsupported multiplicand type");
+    Tile t;
+    if (const char* env = getenv("HELIUM_HIP_GEMM_TILE")) {
+        int a, b, c, d, e;
+        if (sscanf(env, "%d,%d,%d,%d,%d", &a, &b, &c, &d, &e) == 5) t = {a, b, c, d, e};
+    } else {
+        // Smaller problems take smaller tiles so that every CU gets work.
+        if (pr.M <= 128 || pr.N <= 128 || ((pr.M + 255) / 256) * ((pr.N + 255) / 256) * pr.batch < 128) {
+            t.bm = t.bn = 128;
+        }
+    }
+    HE_REQUIRE(t.bm % (t.wm * 32) == 0 && t.bn % (t.wn * 32) == 0 && t.bk == 64, HE_ERR_INVALID, "bad GEMM tile");
+    const int threads = t.wm * t.wn * 64;
+    HE_REQUIRE((t.bm * t.bk / 8) % threads == 0 && (t.bk * t.bn / 8) % threads == 0, HE_ERR_INVALID, "bad GEMM tile");
+    const int wtn = t.bn / t.wn;
+
+    const bool raw_a = is_raw_copy(pr.op_a, pr.root_a, pr.mma_dtype) && pr.K % 8 == 0;
+    const bool raw_b = is_raw_copy(pr.op_b, pr.root_b, pr.mma_dtype) && pr.N % 8 == 0;
+    const int nva = tp::pick_nv(pr.op_a, 16), nvb = tp::pick_nv(pr.op_b, 16);
+    int nve = tp::pick_nv(pr.epi, 32);
+    while (nve > 1 && ((32 * wtn) % (64 * nve) != 0)) nve /= 2;
+    nve = std::min(nve, 8);
+    const int lanes_per_row = wtn / nve;           // lanes that share one row of the strip in one step
+    const int colsets = std::max(1, lanes_per_row / 64);  // distinct column sets a lane visits
+
+    std::ostringstream s;
+    s << "// fused_matmul generated for gfx950: [" << pr.batch << "," << pr.M << "," << pr.K << "] x [" << pr.batch << ","
+      << pr.K << "," << pr.N << "], tile " << t.bm << "x" << t.bn << "x" << t.bk << "\n";
+    s << tp::emit_prelude(pr.epi) << kGemmPrelude;
+    s << "#define GM " << pr.M << "u\n#define GN " << pr.N << "u\n#define GK " << pr.K << "u\n";
+    s << "#define BM " << t.bm << "\n#define BN " << t.bn << "\n#define BK " << t.bk << "\n#define WAVES_M " << t.wm
+      << "\n#define WAVES_N " << t.wn << "\n#define NVE " << nve << "\n#define MMA_BF16 " << (pr.mma_dtype == HE_BF16 ? 1 : 0)
+      << "\n";
+
+    s << kGemmHelpers;
+    // kernel parameters
+    {
+        std::ostringstream ps;
+        for (size_t a = 0; a < pr.args.size(); a++)
+            ps << (a ? ", " : "") << (pr.args[a].is_output ? "" : "const ") << tp::c_type(pr.args[a].dtype) << "* __restrict__ p" << a;
+        s << "#define KERNEL_PARAMS " << ps.str() << "\n";
+    }
+    // operand fetchers
+    auto emit_fetch = [&](const char* which, const tp::Program& p, int root, const std::vector<int>& map, bool raw, int nv,
+                          const char* rows, const char* cols) {
+        // rows/cols: extents of the operand matrix ("GM","GK" for A; "GK","GN" for B)
+        std::ostringstream args, params;
+        for (size_t a = 0; a < p.args.size(); a++) {
+            args << "p" << map[a] << ", ";
+            params << "const " << tp::c_type(p.args[a].dtype) << "* __restrict__ q" << a << ", ";
+        }
+        std::string W = which;
+        s << "#define FETCH_" << (W == "a" ? "A" : "B") << "_ARGS " << args.str() << "\n";
+        if (!raw) s << emit_operand_fn(p, root, "operand_" + W, nv);
+        s << "__device__ __forceinline__ u32x4 fetch_" << W << "(" << params.str() << "u32 b, u32 row, u32 col) {\n";
+        if (raw) {
+            s << "u32x4 v = {0u, 0u, 0u, 0u};\nif (row < " << rows << " && col < " << cols << ") v = *(const u32x4*)(q0 + ((size_t)b * "
+              << rows << " + row) * " << cols << " + col);\nreturn v;\n}\n";
+        } else {
+            s << "float v[8];\n#pragma unroll\nfor (int j = 0; j < 8; j += " << nv << ") {\nif (row < " << rows << " && col + j < " << cols
+              << ") operand_" << W << "(";
+            for (size_t a = 0; a < p.args.size(); a++) s << "q" << a << ", ";
+            s << "b, row, col + j, v + j);\nelse {\n#pragma unroll\nfor (int k = 0; k < " << nv << "; k++) v[j + k] = 0.0f; }\n}\nreturn pack8(v);\n}\n";
+        }
+    };
+    emit_fetch("a", pr.op_a, pr.root_a, pr.map_a, raw_a, nva, "GM", "GK");
+    emit_fetch("b", pr.op_b, pr.root_b, pr.map_b, raw_b, nvb, "GK", "GN");
+
+    // epilogue pieces
+    std::ostringstream setup, body, finish;
+    for (size_t a = 0; a < pr.epi.args.size(); a++)
+        setup << "auto* a" << a << " = p" << pr.map_e[a] << "; (void)a" << a << ";\n";
+    setup << "const u32 cB0 = bz; (void)cB0;\n";
+    for (size_t oi = 0; oi < pr.epi.outs.size(); oi++) {
+        const tp::Out& o = pr.epi.outs[oi];
+        if (!o.reduce) continue;
+        HE_REQUIRE(o.rop == tp::ROp::Sum, HE_ERR_UNSUPPORTED, "GEMM epilogues reduce with Sum only");
+        if (o.fold_m && !o.fold_n)
+            setup << "float rc" << oi << "[" << colsets << "][NVE];\n#pragma unroll\nfor (int c = 0; c < " << colsets
+                  << "; c++)\n#pragma unroll\nfor (int k = 0; k < NVE; k++) rc" << oi << "[c][k] = 0.0f;\n";
+        else if (o.fold_m && o.fold_n)
+            setup << "float rs" << oi << " = 0.0f;\n";
+    }
+    {
+        // body: runs once per (row, NVE columns) of the strip
+        for (size_t oi = 0; oi < pr.epi.outs.size(); oi++)
+            if (pr.epi.outs[oi].reduce && pr.epi.outs[oi].fold_n && !pr.epi.outs[oi].fold_m) body << "float rr" << oi << " = 0.0f;\n";
+        body << "if (ok) {\nconst u32 n0 = nn; (void)n0;\nfloat (&acc)[NVE] = acc_v;\n";
+        tp::EmitCtx cx;
+        cx.nv = nve;
+        // the emitter names the first of the NV columns `n0`; the tile origin of the same name is shadowed here
+        body << tp::emit_exprs(pr.epi, cx);
+        for (size_t oi = 0; oi < pr.epi.outs.size(); oi++) {
+            const tp::Out& o = pr.epi.outs[oi];
+            const std::string v = "e" + std::to_string(o.expr);
+            if (!o.reduce) {
+                body << "st_vec<NVE>(a" << o.arg << " + ((size_t)bz * GM + m) * GN + nn, " << v << ");\n";
+            } else if (o.fold_m && !o.fold_n) {
+                body << "#pragma unroll\nfor (int k = 0; k < NVE; k++) rc" << oi << "[step % " << colsets << "][k] += " << v << "[k];\n";
+            } else if (o.fold_m && o.fold_n) {
+                body << "#pragma unroll\nfor (int k = 0; k < NVE; k++) rs" << oi << " += " << v << "[k];\n";
+            } else {
+                body << "#pragma unroll\nfor (int k = 0; k < NVE; k++) rr" << oi << " += " << v << "[k];\n";
+            }
+        }
+        body << "}\n";
+        // per-row sums: combine the lanes that share the row, one atomic per row segment
+        for (size_t oi = 0; oi < pr.epi.outs.size(); oi++) {
+            const tp::Out& o = pr.epi.outs[oi];
+            if (!(o.reduce && o.fold_n && !o.fold_m)) continue;
+            const int width = std::min(lanes_per_row, 64);
+            body << "{ float r = wave_reduce<0, " << width << ">(rr" << oi << ");\nif ((lane % " << width
+                 << ") == 0 && m < GM && nn < GN) atomicAdd(a" << o.arg << " + (size_t)bz * GM + m, r); }\n";
+        }
+    }
+    for (size_t oi = 0; oi < pr.epi.outs.size(); oi++) {
+        const tp::Out& o = pr.epi.outs[oi];
+        if (!o.reduce) continue;
+        if (o.fold_m && !o.fold_n) {
+            // lanes that hold the same columns differ by multiples of lanes_per_row
+            finish << "#pragma unroll\nfor (int c = 0; c < " << colsets << "; c++) {\n#pragma unroll\nfor (int k = 0; k < NVE; k++) {\nfloat r = rc"
+                   << oi << "[c][k];\n";
+            for (int off = lanes_per_row; off < 64; off *= 2) finish << "r += __shfl_xor(r, " << off << ", 64);\n";
+            finish << "const u32 col = ((c * 64 + lane) * NVE) % WTN + k;\nconst u32 nn = n0 + wave_n * WTN + col;\n";
+            finish << "if (lane < " << std::min(lanes_per_row, 64) << " && nn < GN) atomicAdd(a" << o.arg << " + (size_t)bz * GN + nn, r);\n}\n}\n";
+        } else if (o.fold_m && o.fold_n) {
+            finish << "{ float r = wave_reduce<0, 64>(rs" << oi << ");\nif (lane == 0) atomicAdd(a" << o.arg << " + (size_t)(bz / " << o.b_div
+                   << "u), r); }\n";
+        }
+    }
+    // splice the generated pieces into the body
+    std::string body_text = kGemmBody;
+    auto splice = [&](const std::string& marker, const std::string& text) {
+        size_t pos = body_text.find(marker);
+        HE_REQUIRE(pos != std::string::npos, HE_ERR_INTERNAL, "kernel template lacks %s", marker.c_str());
+        body_text.replace(pos, marker.size(), text);
+    };
+    splice("EPILOGUE_SETUP", setup.str());
+    splice("EPILOGUE_BODY", body.str());
+    splice("EPILOGUE_FINISH", finish.str());
+    s << body_text;
+    source_ = s.str();
+
+    const int64_t tiles = ((pr.M + t.bm - 1) / t.bm) * ((pr.N + t.bn - 1) / t.bn);
+    HE_REQUIRE(tiles < (1ll << 31) && pr.batch < 65536, HE_ERR_INVALID, "GEMM grid too large");
+    grid_[0] = (uint32_t)tiles;
+    grid_[1] = (uint32_t)pr.batch;
+    threads_ = (uint32_t)threads;
+    for (auto& o : pr.epi.outs)
+        if (o.reduce) fills_.push_back({pr.map_e[o.arg], 0u});
+    describe_ = strfmt("gemm [%lld,%lld,%lld]x[%lld] tile=%dx%dx%d waves=%dx%d threads=%d grid=%ux%u rawA=%d rawB=%d NVA=%d NVB=%d NVE=%d "
+                       "mma=%s epilogue_exprs=%zu outs=%zu",
+                       (long long)pr.batch, (long long)pr.M, (long long)pr.K, (long long)pr.N, t.bm, t.bn, t.bk, t.wm, t.wn, threads,
+                       grid_[0], grid_[1], (int)raw_a, (int)raw_b, nva, nvb, nve, dtype_name(pr.mma_dtype), pr.epi.exprs.size(),
+                       pr.epi.outs.size());
+    kernel_.reset(new JitKernel(source_, "fused_matmul", {"-ffp-contract=fast", "-munsafe-fp-atomics"}));
+}
+
+void GemmKernel::execute(void* const* ptrs, hipStream_t stream) {
+    const size_t nargs = prob_.args.size();
+    for (size_t i = 0; i < nargs; i++) {
+        HE_REQUIRE(ptrs[i] != nullptr, HE_ERR_INVALID, "kernel argument %zu is null", i);
+        HE_REQUIRE(((uintptr_t)ptrs[i] & 15) == 0, HE_ERR_INVALID, "kernel argument %zu is not 16-byte aligned", i);
+    }
+    std::vector<std::pair<void*, std::pair<uint32_t, uint32_t>>> fills;
+    for (auto& f : fills_) {
+        const tp::Arg& a = prob_.args[f.first];
+        fills.push_back({ptrs[f.first], {(uint32_t)(storage_bytes(a.dtype, (size_t)a.numel) / 4), f.second}});
+    }
+    if (!fills.empty()) fill_buffers(fills, stream);
+    std::vector<void*> holders(ptrs, ptrs + nargs), argv(nargs);
+    for (size_t i = 0; i < nargs; i++) argv[i] = &holders[i];
+    const uint32_t block[3] = {threads_, 1, 1};
+    kernel_->launch(grid_, block, 0, stream, argv.data());
+}
+
+}  // namespace he

@@ -1,4 +1,5 @@
-// Executable kernels built from tile programs: the pointwise/reduction instruction and fused fusion-IR kernels.
+// Executable kernels built from tile programs: the pointwise/reduction instruction, anchor-less fusion-IR kernels
+// and the fused GEMM.
 #pragma once
 #include <memory>
 
@@ -7,20 +8,66 @@
 
 namespace he {
 
+// Fills each (pointer, (32-bit words, pattern)) buffer on `stream` with one kernel launch per 8 buffers.
+void fill_buffers(const std::vector<std::pair<void*, std::pair<uint32_t, uint32_t>>>& fills, hipStream_t stream);
+
+// What every generated kernel offers the C ABI: an ordered argument list, its source and a launch.
+class KernelBase {
+public:
+    virtual ~KernelBase() = default;
+    virtual const std::vector<tp::Arg>& args() const = 0;
+    virtual const std::string& source() const = 0;
+    virtual const std::string& describe() const = 0;
+    // `ptrs[i]` is the device address of argument i.
+    virtual void execute(void* const* ptrs, hipStream_t stream) = 0;
+};
+
 // A tile program compiled into one kernel launch (plus the fills its reduction / bitset outputs need).
-class TileKernel {
+class TileKernel : public KernelBase {
 public:
     TileKernel(tp::Program prog, const std::string& entry);
     const tp::Program& program() const { return prog_; }
     const tp::PointwiseLaunch& launch_info() const { return launch_; }
-    const std::string& source() const { return launch_.source; }
-    // `ptrs[i]` is the device address of program argument i.
-    void execute(void* const* ptrs, hipStream_t stream);
+    const std::vector<tp::Arg>& args() const override { return prog_.args; }
+    const std::string& source() const override { return launch_.source; }
+    const std::string& describe() const override { return launch_.describe; }
+    void execute(void* const* ptrs, hipStream_t stream) override;
 
 private:
     tp::Program prog_;
     tp::PointwiseLaunch launch_;
     std::unique_ptr<JitKernel> kernel_;
+};
+
+// Fused GEMM: C = f(A) g(B) with mainloop op chains applied while tiles are staged into LDS and the epilogue
+// program applied to the f32 accumulators (helium-kernel-generator/src/generators/matmul.rs,
+// helium-playground/src/kernel_generator.rs + templates/matmul.cu).
+struct GemmProblem {
+    int64_t batch = 1, M = 0, N = 0, K = 0;
+    int mma_dtype = HE_BF16;       // multiplicand type: HE_BF16, HE_F16 or HE_F32
+    tp::Program op_a, op_b, epi;   // dims [batch,M,K], [batch,K,N], [batch,M,N]
+    int root_a = -1, root_b = -1;  // expression ids of the operand values in op_a / op_b
+    std::vector<tp::Arg> args;     // the kernel's arguments: inputs in node order, then outputs in node order
+    std::vector<int> map_a, map_b, map_e;  // program argument -> kernel argument
+};
+GemmProblem gemm_problem_from_fusion(const fir::OpGraph& g);
+
+class GemmKernel : public KernelBase {
+public:
+    explicit GemmKernel(GemmProblem prob);
+    const std::vector<tp::Arg>& args() const override { return prob_.args; }
+    const std::string& source() const override { return source_; }
+    const std::string& describe() const override { return describe_; }
+    void execute(void* const* ptrs, hipStream_t stream) override;
+    const GemmProblem& problem() const { return prob_; }
+
+private:
+    GemmProblem prob_;
+    std::string source_, describe_;
+    std::unique_ptr<JitKernel> kernel_;
+    uint32_t grid_[3] = {1, 1, 1};
+    uint32_t threads_ = 256;
+    std::vector<std::pair<int, uint32_t>> fills_;
 };
 
 }  // namespace he

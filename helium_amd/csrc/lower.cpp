@@ -326,29 +326,15 @@ public:
         }
         HE_REQUIRE(!outs.empty(), HE_ERR_INVALID, "fusion has no output");
 
-        // Iteration space: the anchor's output, else the largest root (kernel_generator.rs:98-106).
+        // Iteration space: the anchor's output; without an anchor, the (pre-reduction) shape of the first output.
+        // (The reference takes M and N from its largest root, kernel_generator.rs:98-106, which only agrees with
+        // the outputs when no input is transposed.)
         fir::Shape3 s;
         if (anchor_ != fir::kNoOpNode) {
             s = g_.shape(anchor_);
         } else {
-            fir::OpNode best = fir::kNoOpNode;
-            uint64_t best_n = 0;
-            for (fir::OpNode r : g_.roots()) {
-                const fir::Shape3& rs = g_.shape(r);
-                uint64_t n = (uint64_t)rs[0] * rs[1] * rs[2];
-                if (best == fir::kNoOpNode || n > best_n) {
-                    best = r;
-                    best_n = n;
-                }
-            }
-            HE_REQUIRE(best != fir::kNoOpNode, HE_ERR_INVALID, "fusion has no input");
-            s = g_.shape(best);
-            // An output may be larger than every input (a broadcast of a small producer): take the value shape.
-            for (auto& o : outs) {
-                const fir::Op& vop = g_.get(o.second);
-                fir::Shape3 vs = vop.kind == fir::OpKind::Reduction ? g_.shape(vop.a) : g_.shape(o.second);
-                if ((uint64_t)vs[0] * vs[1] * vs[2] > (uint64_t)s[0] * s[1] * s[2]) s = vs;
-            }
+            const fir::Op& vop = g_.get(outs[0].second);
+            s = vop.kind == fir::OpKind::Reduction ? g_.shape(vop.a) : g_.shape(outs[0].second);
         }
         p_.dims = {s[0], s[1], s[2]};
 
@@ -408,6 +394,33 @@ public:
             }
             p_.outs.push_back(o);
         }
+        return std::move(p_);
+    }
+
+    // The value of one node (a Matmul operand with its mainloop ops) over that node's own shape.
+    Program run_value(fir::OpNode value, int* root) {
+        const fir::Shape3& s = g_.shape(value);
+        p_.dims = {s[0], s[1], s[2]};
+        std::vector<fir::OpNode> producers, stack{value};
+        std::map<fir::OpNode, char> seen;
+        while (!stack.empty()) {
+            fir::OpNode n = stack.back();
+            stack.pop_back();
+            if (seen[n]++) continue;
+            HE_REQUIRE(g_.get(n).kind != fir::OpKind::Matmul && g_.get(n).kind != fir::OpKind::Reduction,
+                       HE_ERR_UNSUPPORTED, "a mainloop fusion holds pointwise, broadcast and transpose ops only");
+            if (g_.get(n).kind == fir::OpKind::Producer) producers.push_back(n);
+            for (fir::OpNode i : g_.inbound(n)) stack.push_back(i);
+        }
+        std::sort(producers.begin(), producers.end());
+        for (fir::OpNode pnode : producers) {
+            const fir::Shape3& ps = g_.shape(pnode);
+            input_arg_[pnode] = (int)p_.args.size();
+            p_.args.push_back({g_.get(pnode).dtype, (int64_t)ps[0] * ps[1] * ps[2], false, pnode});
+        }
+        Mapping ident;
+        ident.w = ir::packed_strides(p_.dims);
+        *root = eval(value, ident);
         return std::move(p_);
     }
 
@@ -575,6 +588,9 @@ Program lower_pointwise(const ir::OpSubgraph& sg) { return PointwiseLowering(sg)
 Program lower_aux(const fir::OpGraph& g) {
     HE_REQUIRE(g.anchor() == fir::kNoOpNode, HE_ERR_INVALID, "an auxiliary fusion holds no Matmul");
     return FusionLowering(g, fir::kNoOpNode).run();
+}
+Program lower_operand(const fir::OpGraph& g, fir::OpNode value, int* root_expr) {
+    return FusionLowering(g, fir::kNoOpNode).run_value(value, root_expr);
 }
 Program lower_epilogue(const fir::OpGraph& g, fir::OpNode anchor) {
     Program p = FusionLowering(g, anchor).run();

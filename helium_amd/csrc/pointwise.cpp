@@ -3,6 +3,46 @@
 
 namespace he {
 
+// One launch that fills up to 8 buffers with 32-bit patterns (reduction identities, cleared bitsets): a single
+// small kernel instead of one memset per output.
+namespace {
+struct FillArgs {
+    uint32_t* ptr[8];
+    uint32_t words[8];
+    uint32_t value[8];
+    int32_t count;
+};
+const char* kFillSource = R"HIP(
+struct FillArgs { unsigned* ptr[8]; unsigned words[8]; unsigned value[8]; int count; };
+extern "C" __global__ __launch_bounds__(256) void fill_many(FillArgs a) {
+    for (int k = 0; k < a.count; k++)
+        for (unsigned i = blockIdx.x * 256u + threadIdx.x; i < a.words[k]; i += gridDim.x * 256u) a.ptr[k][i] = a.value[k];
+}
+)HIP";
+JitKernel& fill_kernel() {
+    static JitKernel k(kFillSource, "fill_many");
+    return k;
+}
+}  // namespace
+
+void fill_buffers(const std::vector<std::pair<void*, std::pair<uint32_t, uint32_t>>>& fills, hipStream_t stream) {
+    for (size_t base = 0; base < fills.size(); base += 8) {
+        FillArgs a{};
+        uint32_t max_words = 0;
+        a.count = (int)std::min<size_t>(8, fills.size() - base);
+        for (int k = 0; k < a.count; k++) {
+            a.ptr[k] = (uint32_t*)fills[base + k].first;
+            a.words[k] = fills[base + k].second.first;
+            a.value[k] = fills[base + k].second.second;
+            max_words = std::max(max_words, a.words[k]);
+        }
+        if (!max_words) continue;
+        const uint32_t grid[3] = {std::min<uint32_t>((max_words + 1023) / 1024, 1024), 1, 1}, block[3] = {256, 1, 1};
+        void* argv[] = {&a};
+        fill_kernel().launch(grid, block, 0, stream, argv);
+    }
+}
+
 TileKernel::TileKernel(tp::Program prog, const std::string& entry) : prog_(std::move(prog)) {
     launch_ = tp::emit_pointwise(prog_, entry);
     if (launch_.grid > 0) kernel_.reset(new JitKernel(launch_.source, launch_.entry, launch_.options));
@@ -12,13 +52,15 @@ void TileKernel::execute(void* const* ptrs, hipStream_t stream) {
     const size_t nargs = prog_.args.size();
     for (size_t i = 0; i < nargs; i++)
         HE_REQUIRE(ptrs[i] != nullptr || prog_.args[i].numel == 0, HE_ERR_INVALID, "kernel argument %zu is null", i);
+    // Reduction outputs start from the operator's identity and bitset outputs from zero
+    // (helium/src/cuda/instr/pointwise.rs:62-74).
+    std::vector<std::pair<void*, std::pair<uint32_t, uint32_t>>> fills;
     for (auto& f : launch_.fills) {
         const tp::Arg& a = prog_.args[f.first];
         size_t words = storage_bytes(a.dtype, (size_t)a.numel) / 4;
-        // Reduction outputs start from the operator's identity and bitset outputs from zero
-        // (helium/src/cuda/instr/pointwise.rs:62-74).
-        if (words) HE_HIP(hipMemsetD32Async((hipDeviceptr_t)ptrs[f.first], (int)f.second, words, stream));
+        if (words) fills.push_back({ptrs[f.first], {(uint32_t)words, f.second}});
     }
+    if (!fills.empty()) fill_buffers(fills, stream);
     if (launch_.grid == 0) return;
     for (size_t i = 0; i < nargs; i++)
         HE_REQUIRE(((uintptr_t)ptrs[i] & 15) == 0, HE_ERR_INVALID, "kernel argument %zu is not 16-byte aligned", i);

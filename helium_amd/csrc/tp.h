@@ -103,6 +103,9 @@ Program lower_aux(const fir::OpGraph& g);
 // The epilogue of a Core fusion: everything downstream of `anchor`. Producers that feed only the mainloop are not
 // arguments of the program. `arg_nodes` receives the producer / consumer node behind every program argument.
 Program lower_epilogue(const fir::OpGraph& g, fir::OpNode anchor);
+// One Matmul operand together with the mainloop ops that produce it, evaluated over the operand's own shape
+// ([batch, M, K] for a, [batch, K, N] for b). `root_expr` receives the id of the operand's value.
+Program lower_operand(const fir::OpGraph& g, fir::OpNode value, int* root_expr);
 
 // ---- emission -----------------------------------------------------------------------------------------------
 struct PointwiseLaunch {

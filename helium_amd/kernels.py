@@ -9,6 +9,7 @@ from .device import _h
 _ffi._sig("he_pointwise_supports", C.c_void_p, C.POINTER(C.c_uint32), C.c_int, C.POINTER(C.c_int))
 _ffi._sig("he_pointwise_create", C.POINTER(C.c_void_p), C.c_void_p, C.POINTER(C.c_uint32), C.c_int)
 _ffi._sig("he_aux_kernel_create", C.POINTER(C.c_void_p), C.c_void_p)
+_ffi._sig("he_fused_kernel_create", C.POINTER(C.c_void_p), C.c_void_p)
 _ffi._sig("he_tile_kernel_num_args", C.c_void_p, C.POINTER(C.c_int))
 _ffi._sig("he_tile_kernel_arg_info", C.c_void_p, C.c_int, C.POINTER(C.c_uint64), C.POINTER(C.c_int32),
           C.POINTER(C.c_int32), C.POINTER(C.c_int64))
@@ -50,6 +51,14 @@ class TileKernel:
         """KernelGenerator for an anchor-less fusion-IR graph."""
         h = C.c_void_p()
         check(lib.he_aux_kernel_create(C.byref(h), fgraph.handle))
+        return cls(h)
+
+    @classmethod
+    def fused(cls, fgraph):
+        """KernelGenerator for any fusion-IR graph: the fused GEMM when it holds a Matmul anchor (its mainloop ops
+        run while operand tiles are staged, its epilogue ops on the accumulators), else the auxiliary kernel."""
+        h = C.c_void_p()
+        check(lib.he_fused_kernel_create(C.byref(h), fgraph.handle))
         return cls(h)
 
     @property

@@ -249,6 +249,10 @@ int he_fgraph_shape(he_fgraph_t graph, uint64_t node, uint32_t shape_out[3]);
 /* KernelGenerator::new + generate for an anchor-less fusion (kernel_generator.rs:22-49,98-115; template
  * templates/auxiliary.cu). Arguments: producers in id order, then leaves in id order (:52-63,138-148). */
 int he_aux_kernel_create(he_tile_kernel_t* kernel, he_fgraph_t graph);
+/* KernelGenerator::new + generate for any fusion (kernel_generator.rs:22-117): with a Matmul anchor the fused
+ * GEMM (templates/matmul.cu's role: mainloop ops while tiles are staged, epilogue ops and reductions on the
+ * accumulators), otherwise the auxiliary kernel. Arguments: producers in id order, then leaves in id order. */
+int he_fused_kernel_create(he_tile_kernel_t* kernel, he_fgraph_t graph);
 
 #ifdef __cplusplus
 }

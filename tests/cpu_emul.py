@@ -63,6 +63,50 @@ template <class T> static inline T atomicMin(T* a, T v) {
     return old;
 }
 static inline unsigned atomicOr(unsigned* a, unsigned v) { return __atomic_fetch_or(a, v, __ATOMIC_SEQ_CST); }
+// matrix-core and transposing-LDS-load stand-ins: whole waves call them in lockstep, lanes meet in memory
+typedef short emu_s16x8 __attribute__((ext_vector_type(8)));
+typedef short emu_s16x4 __attribute__((ext_vector_type(4)));
+typedef float emu_f32x16 __attribute__((ext_vector_type(16)));
+static emu_s16x8 g_mfa[1024], g_mfb[1024];
+static inline float emu_bf16(short h) { unsigned u = ((unsigned)(unsigned short)h) << 16; float f; memcpy(&f, &u, 4); return f; }
+static inline float emu_f16(short h) { _Float16 x; memcpy(&x, &h, 2); return (float)x; }
+template <class V, bool BF> static inline emu_f32x16 emu_mfma(V a, V b, emu_f32x16 c) {
+    // v_mfma_f32_32x32x16: lane l holds A[l%32][(l/32)*8+j] and B[(l/32)*8+j][l%32]; c[i] is row (i/4)*8+(l/32)*4+i%4
+    unsigned tid = threadIdx.x, base = tid & ~63u, lane = tid & 63u;
+    g_mfa[tid] = __builtin_bit_cast(emu_s16x8, a);
+    g_mfb[tid] = __builtin_bit_cast(emu_s16x8, b);
+    pthread_barrier_wait(&g_bar);
+    for (int i = 0; i < 16; i++) {
+        unsigned row = (i / 4) * 8 + (lane / 32) * 4 + i % 4, col = lane % 32;
+        float sum = 0;
+        for (int k = 0; k < 16; k++) {
+            short av = g_mfa[base + row + 32 * (k / 8)][k % 8], bv = g_mfb[base + col + 32 * (k / 8)][k % 8];
+            sum += BF ? emu_bf16(av) * emu_bf16(bv) : emu_f16(av) * emu_f16(bv);
+        }
+        c[i] += sum;
+    }
+    pthread_barrier_wait(&g_bar);
+    return c;
+}
+#define __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, x, y, z) emu_mfma<decltype(a), true>(a, b, c)
+#define __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, x, y, z) emu_mfma<decltype(a), false>(a, b, c)
+static const short* g_traddr[1024];
+static inline emu_s16x4 emu_tr16(const emu_s16x4* p) {
+    // ds_read_b64_tr_b16, as measured on gfx950: within each group of 16 lanes, lane L gets element L%4 of the
+    // four source lanes 4e + L/4 (e = 0..3)
+    unsigned tid = threadIdx.x, gbase = tid & ~15u, L = tid & 15u;
+    g_traddr[tid] = (const short*)p;
+    pthread_barrier_wait(&g_bar);
+    emu_s16x4 r;
+    for (int e = 0; e < 4; e++) r[e] = g_traddr[gbase + 4 * e + L / 4][L % 4];
+    pthread_barrier_wait(&g_bar);
+    return r;
+}
+#define __builtin_amdgcn_ds_read_tr16_b64_v4i16(p) emu_tr16(p)
+#define LDS_AS
+#define KERNEL_ATTRS
+#define __builtin_amdgcn_fence(...)
+#define __builtin_amdgcn_wave_barrier() pthread_barrier_wait(&g_bar)
 #define __expf expf
 #define __logf logf
 #define __sinf sinf
@@ -83,8 +127,8 @@ static void** g_bufs;
 static void* worker(void* arg) {
     unsigned tid = (unsigned)(size_t)arg;
     threadIdx.x = tid;
-    for (unsigned b = 0; b < gridDim.x; b++) {
-        blockIdx.x = b;
+    for (unsigned b = 0; b < gridDim.x * gridDim.y; b++) {
+        blockIdx.x = b % gridDim.x; blockIdx.y = b / gridDim.x;
         call(&ENTRY, g_bufs);
         pthread_barrier_wait(&g_bar);
     }
@@ -93,6 +137,8 @@ static void* worker(void* arg) {
 int main(int argc, char** argv) {
     // argv: grid threads (path bytes is_output)...
     gridDim.x = atoi(argv[1]); blockDim.x = atoi(argv[2]);
+    gridDim.y = 1;
+    if (const char* gy = getenv("EMUL_GRID_Y")) gridDim.y = atoi(gy);
     int nb = (argc - 3) / 3;
     std::vector<void*> bufs(nb); std::vector<size_t> sizes(nb); std::vector<int> isout(nb);
     for (int i = 0; i < nb; i++) {
@@ -113,7 +159,7 @@ int main(int argc, char** argv) {
 """
 
 
-def run_kernel(source, entry, grid, threads, buffers, flags=()):
+def run_kernel(source, entry, grid, threads, buffers, flags=(), grid_y=1):
     """buffers: list of (numpy array, mode) with mode False/0 = input, True/1 = output (starts as 0xEE bytes),
     2 = in-out (starts from the array's contents). Returns the output arrays (same dtype/shape as given)."""
     with tempfile.TemporaryDirectory() as d:
@@ -131,7 +177,7 @@ def run_kernel(source, entry, grid, threads, buffers, flags=()):
             if int(is_out) != 1:
                 np.ascontiguousarray(a).tofile(p)
             argv += [p, str(a.nbytes), str(int(is_out))]
-        res = subprocess.run(argv, capture_output=True, text=True, env={**os.environ, "ASAN_OPTIONS": "detect_leaks=0"})
+        res = subprocess.run(argv, capture_output=True, text=True, env={**os.environ, "ASAN_OPTIONS": "detect_leaks=0", "EMUL_GRID_Y": str(grid_y)})
         if res.returncode != 0:
             raise AssertionError(f"CPU emulation of {entry} failed (exit {res.returncode}):\n{res.stderr[-4000:]}")
         outs = []

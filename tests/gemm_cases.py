@@ -1,0 +1,59 @@
+"""Fused-GEMM cases shared by the CPU-emulation and GPU parity tests (fusion IR built through the C ABI)."""
+import numpy as np
+
+import helium_amd as ha
+from helium_amd import configs
+
+
+def bf16_normal(rng, shape, scale=1.0):
+    return configs.bf16_rne((rng.standard_normal(shape) * scale).astype(np.float32))
+
+
+def plain(m, n, k, batch=1, seed=0, dtype="bf16", out_dtype="f32", scale=0.5):
+    g = ha.fusion.OpGraph()
+    rng = np.random.default_rng(seed)
+    a = g.producer([batch, m, k], dtype); b = g.producer([batch, k, n], dtype)
+    out = g.consumer(g.matmul(a, b), out_dtype)
+    if dtype == "bf16":
+        inputs = {a: bf16_normal(rng, (batch, m, k), scale), b: bf16_normal(rng, (batch, k, n), scale)}
+    elif dtype == "f16":
+        inputs = {a: (rng.standard_normal((batch, m, k)) * scale).astype(np.float16).view(np.uint16),
+                  b: (rng.standard_normal((batch, k, n)) * scale).astype(np.float16).view(np.uint16)}
+    else:
+        inputs = {a: (rng.standard_normal((batch, m, k)) * scale).astype(np.float32),
+                  b: (rng.standard_normal((batch, k, n)) * scale).astype(np.float32)}
+    return g, inputs, [out]
+
+
+def bias_relu_colsum(m, n, k, batch=1, seed=1, bias_axis=1, mainloop=False):
+    """Config 5a's shape of fusion: optional mainloop relu(A0) * T on the A operand, bias + Relu epilogue, the
+    full-size result and its column sums as outputs."""
+    g = ha.fusion.OpGraph()
+    rng = np.random.default_rng(seed)
+    a0 = g.producer([batch, m, k], "bf16")
+    inputs = {a0: bf16_normal(rng, (batch, m, k))}
+    a = a0
+    if mainloop:
+        t = g.producer([batch, m, k], "bf16")
+        inputs[t] = bf16_normal(rng, (batch, m, k))
+        a = g.binary(g.unary(a0, "relu"), t, "mul")
+    b = g.producer([batch, k, n], "bf16")
+    inputs[b] = bf16_normal(rng, (batch, k, n), 0.25)
+    bshape = [batch, 1, n] if bias_axis == 1 else [batch, m, 1]
+    bias = g.producer(bshape, "f32")
+    inputs[bias] = rng.standard_normal(bshape).astype(np.float32)
+    mm = g.matmul(a, b)
+    y = g.unary(g.binary(mm, g.broadcast(bias, bias_axis, m if bias_axis == 1 else n), "add"), "relu")
+    outs = [g.consumer(y, "bf16"), g.consumer(g.reduction(y, "columns"), "f32")]
+    return g, inputs, outs
+
+
+def all_reductions(m, n, k, batch=2, seed=2):
+    g = ha.fusion.OpGraph()
+    rng = np.random.default_rng(seed)
+    a = g.producer([batch, m, k], "bf16"); b = g.producer([batch, k, n], "bf16"); aux = g.producer([batch, m, n], "bf16")
+    inputs = {a: bf16_normal(rng, (batch, m, k), 0.5), b: bf16_normal(rng, (batch, k, n), 0.5), aux: bf16_normal(rng, (batch, m, n))}
+    v = g.binary(g.unary(g.matmul(a, b), "tanh"), aux, "mul")
+    outs = [g.consumer(g.reduction(v, d), "f32") for d in ("rows", "columns", "item", "batch")]
+    outs.append(g.consumer(v, "f32"))
+    return g, inputs, outs

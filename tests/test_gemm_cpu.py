@@ -1,0 +1,70 @@
+"""The generated fused-GEMM kernel run on the CPU (threads + barriers, MFMA and transposing-LDS-load stand-ins,
+AddressSanitizer) against the oracle: index arithmetic, edge predication, mainloop and epilogue fusion."""
+import os
+import re
+
+import numpy as np
+import pytest
+
+import helium_amd as ha
+from oracle import fusion_ir as oracle
+from oracle import numerics as nm
+
+import gemm_cases
+from cpu_emul import run_kernel
+
+
+def run_emulated(g, inputs, tile):
+    os.environ["HELIUM_HIP_GEMM_TILE"] = tile
+    try:
+        k = ha.TileKernel.fused(g)
+    finally:
+        del os.environ["HELIUM_HIP_GEMM_TILE"]
+    gx, gy = map(int, re.search(r"grid=(\d+)x(\d+)", k.description).groups())
+    threads = int(re.search(r"threads=(\d+)", k.description).group(1))
+    bufs = []
+    for a in k.args:
+        dt = nm.NP_STORAGE[a["dtype"]]
+        bufs.append((np.zeros(a["numel"], dtype=dt), 2) if a["is_output"] else (inputs[a["node"]], 0))
+    res = run_kernel(k.source, "fused_matmul", gx, threads, bufs, grid_y=gy)
+    outs = [a for a in k.args if a["is_output"]]
+    return k, {a["node"]: (r, a["dtype"]) for a, r in zip(outs, res)}
+
+
+def compare(got, want, rel=1e-2, eps=1e-3):
+    for node, (g, dtype) in got.items():
+        w = want[node].reshape(-1)
+        if dtype == "bf16":
+            g, w = nm.bf16_bits_to_f32(g), nm.bf16_bits_to_f32(w)
+        g, w = g.astype(np.float64), w.astype(np.float64)
+        # approx::relative_eq(epsilon 1e-3, max_relative 1e-2), helium-kernel-generator/tests/matmul.rs:140-147
+        ok = (np.abs(g - w) <= eps) | (np.abs(g - w) <= rel * np.maximum(np.abs(g), np.abs(w)))
+        assert ok.all(), (node, np.abs(g - w).max())
+
+
+CASES = [
+    ("plain_2x2_tiles", lambda: gemm_cases.plain(160, 136, 72), "128,128,64,2,2"),
+    ("ragged_scalar_paths", lambda: gemm_cases.plain(97, 131, 67), "128,128,64,2,2"),
+    ("mainloop_bias_relu_colsum", lambda: gemm_cases.bias_relu_colsum(130, 136, 80, mainloop=True), "128,128,64,2,2"),
+    ("row_bias", lambda: gemm_cases.bias_relu_colsum(64, 72, 64, bias_axis=2), "128,128,64,2,2"),
+    ("all_reductions_batched", lambda: gemm_cases.all_reductions(70, 72, 64), "128,128,64,2,2"),
+    ("f16_operands", lambda: gemm_cases.plain(64, 64, 64, dtype="f16"), "128,128,64,2,2"),
+    ("f32_operands_rounded_to_bf16", lambda: gemm_cases.plain(40, 48, 40, dtype="f32"), "128,128,64,2,2"),
+    ("big_tile_256", lambda: gemm_cases.plain(256, 256, 64), "256,256,64,2,2"),
+]
+
+
+@pytest.mark.parametrize("name,build,tile", CASES, ids=[c[0] for c in CASES])
+def test_fused_gemm_on_cpu(name, build, tile):
+    g, inputs, outs = build()
+    k, got = run_emulated(g, inputs, tile)
+    assert sorted(got) == sorted(outs), k.description
+    want = oracle.outputs(g.nodes, inputs, round_mainloop_to="f16" if name == "f16_operands" else "bf16")
+    compare(got, want)
+
+
+def test_argument_order_is_producers_then_leaves():
+    g, inputs, outs = gemm_cases.bias_relu_colsum(64, 64, 64, mainloop=True)
+    k = ha.TileKernel.fused(g)
+    ins = [a["node"] for a in k.args if not a["is_output"]]
+    assert ins == sorted(inputs) and [a["node"] for a in k.args if a["is_output"]] == outs
