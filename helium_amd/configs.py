@@ -57,3 +57,91 @@ def c3_chain(rows=4096, cols=4096, bias_axis=2, seed=31, make_inputs=True):
         inputs = {n: rng.uniform(-1, 1, size=full).astype(np.float32) for n in (a, b, c, d)}
         inputs[bias] = rng.uniform(-1, 1, size=bshape).astype(np.float32)
     return g, inputs, {"batch": out_batch, "columns": out_cols, "r": r}
+
+
+def c4_graph(size=4096, mainloop=False, full_size_outputs=False):
+    """Config 4: the reference README's fusion (README.md:33-79), node ids as printed there.
+
+    Core = Matmul{a: n1, b: n2} is node 12; n13, n24, n26 are the other GEMM results of the LSTM-cell-like graph
+    and arrive as bf16 tensors, n9 is the previous state, n11 the target, n6 / n8 the f32 biases [1,1,size]
+    broadcast along axis 1. 39 epilogue ops follow the anchor; the leaves are the three reductions n39 (Batch),
+    n58 and n87 (Columns). With mainloop=True the anchor's A operand is n25 = Relu(n22) * n9 (README.md:36-38).
+    With full_size_outputs=True n57 and n86 (the gradients the backward GEMMs would read) are also stored, as bf16.
+    """
+    g = fusion.OpGraph()
+    full = [1, size, size]
+    P = lambda i, shape=full, dt="bf16": g.producer(shape, dt, node_id=i)  # noqa: E731
+    n1 = P(22) if mainloop else P(1)
+    n2 = P(2)
+    n6, n8 = P(6, [1, 1, size], "f32"), P(8, [1, 1, size], "f32")
+    n9, n11, n13, n24, n26 = P(9), P(11), P(13), P(24), P(26)
+    a_operand = n1
+    if mainloop:
+        g.unary(22, "relu", node_id=23)
+        a_operand = g.binary(23, n9, "mul", node_id=25)
+    g.matmul(a_operand, n2, node_id=12)
+    U = lambda i, x, fn, c=0.0: g.unary(x, fn, c, node_id=i)  # noqa: E731
+    B = lambda i, lhs, rhs, fn: g.binary(lhs, rhs, fn, node_id=i)  # noqa: E731
+    inv = np.float32(0.00024414063)
+    B(14, 12, n13, "add"); g.broadcast(n6, 1, size, node_id=15); B(16, 14, 15, "add"); U(17, 16, "relu")
+    B(27, n24, n26, "add"); g.broadcast(n8, 1, size, node_id=28); B(29, 27, 28, "add"); U(30, 29, "tanh")
+    U(31, 17, "neg"); U(32, 31, "add_constant", 1.0); B(33, 32, n9, "mul"); B(34, 17, 30, "mul"); B(35, 33, 34, "add")
+    B(36, 35, n11, "sub"); U(37, 36, "pow_constant", 2.0); U(38, 37, "mul_constant", inv)
+    g.reduction(38, "batch", node_id=39)
+    g.constant([1, 1, 1], 1.0, node_id=41)
+    g.broadcast(41, 1, size, node_id=42); g.broadcast(42, 2, size, node_id=43); g.broadcast(43, 0, 1, node_id=44)
+    U(45, 44, "mul_constant", inv)
+    g.constant(full, 2.0, node_id=46); g.constant(full, 1.0, node_id=47)
+    B(48, 36, 47, "pow"); B(49, 48, 46, "mul"); B(50, 49, 45, "mul")
+    B(52, 50, 30, "mul"); B(53, 17, 50, "mul"); U(54, 30, "pow_constant", 2.0); U(55, 54, "neg")
+    U(56, 55, "add_constant", 1.0); B(57, 53, 56, "mul")
+    g.reduction(57, "columns", node_id=58)
+    B(81, 50, n9, "mul"); U(84, 81, "neg"); B(85, 52, 84, "add"); B(86, 85, 16, "drelu")
+    g.reduction(86, "columns", node_id=87)
+    outs = {"loss": 39, "db8": 58, "db6": 87}
+    if full_size_outputs:
+        outs["dpre_c"] = g.consumer(57, "bf16", node_id=90)
+        outs["dpre_z"] = g.consumer(86, "bf16", node_id=91)
+    return g, outs
+
+
+def c4_inputs(g, size=4096, seed=41):
+    """A, B ~ N(0, 0.02) (bf16); the other GEMM results ~ N(0, 0.02 * 0.02 * sqrt(size)) like a product of two
+    such matrices; previous state and target ~ N(0,1); biases ~ N(0,1) f32."""
+    rng = np.random.default_rng(seed)
+    inputs = {}
+    for n in g.nodes:
+        if n["op"] != "producer":
+            continue
+        shape = n["shape"]
+        if n["dtype"] == "f32":
+            inputs[n["id"]] = rng.standard_normal(shape).astype(np.float32)
+        elif n["id"] in (1, 2, 22):
+            inputs[n["id"]] = bf16_rne((rng.standard_normal(shape) * 0.02).astype(np.float32))
+        elif n["id"] in (13, 24, 26):
+            inputs[n["id"]] = bf16_rne((rng.standard_normal(shape) * (0.02 * 0.02 * np.sqrt(size))).astype(np.float32))
+        else:
+            inputs[n["id"]] = bf16_rne(rng.standard_normal(shape).astype(np.float32))
+    return inputs
+
+
+def c5a_graph(size=4096):
+    """Config 5a: Y = relu(A' B + bias) with A' = Relu(A0) * T applied to the A tiles before the MFMA; bf16
+    operands, f32 bias [1,1,size], bf16 output."""
+    g = fusion.OpGraph()
+    full = [1, size, size]
+    a0, t, b = g.producer(full, "bf16"), g.producer(full, "bf16"), g.producer(full, "bf16")
+    bias = g.producer([1, 1, size], "f32")
+    a = g.binary(g.unary(a0, "relu"), t, "mul")
+    y = g.unary(g.binary(g.matmul(a, b), g.broadcast(bias, 1, size), "add"), "relu")
+    out = g.consumer(y, "bf16")
+    return g, {"a0": a0, "t": t, "b": b, "bias": bias, "y": out}
+
+
+def c5a_inputs(names, size=4096, seed=51):
+    rng = np.random.default_rng(seed)
+    full = (1, size, size)
+    return {names["a0"]: bf16_rne(rng.standard_normal(full).astype(np.float32)),
+            names["t"]: bf16_rne(rng.standard_normal(full).astype(np.float32)),
+            names["b"]: bf16_rne((rng.standard_normal(full) * 0.02).astype(np.float32)),
+            names["bias"]: rng.standard_normal((1, 1, size)).astype(np.float32)}

@@ -164,7 +164,7 @@ static std::string unary_expr(const Expr& e, const std::string& x, bool fast) {
             // x*x for an exponent of exactly 2, as the reference's generator special-cases
             // (helium-playground/src/kernel_generator.rs:383-391); x**c otherwise (torch_synthesizer.rs:55).
             if (cf == 2.0f) return x + " * " + x;
-            return (fast ? "__powf(" : "powf(") + x + ", " + c + ")";
+            return "powf(" + x + ", " + c + ")";
     }
     fail(HE_ERR_INTERNAL, "bad unary op");
 }
@@ -175,7 +175,7 @@ static std::string binary_expr(const Expr& e, Cls cls, const std::string& a, con
         case BOp::Sub: return a + " - " + b;
         case BOp::Mul: return cls == Cls::B ? a + " && " + b : a + " * " + b;
         case BOp::Div: return fast ? "__fdividef(" + a + ", " + b + ")" : a + " / " + b;
-        case BOp::Pow: return (fast ? "__powf(" : "powf(") + a + ", " + b + ")";
+        case BOp::Pow: return "powf(" + a + ", " + b + ")";
         case BOp::Min: return cls == Cls::F ? "fminf(" + a + ", " + b + ")" : "(" + a + " < " + b + " ? " + a + " : " + b + ")";
         case BOp::Max: return cls == Cls::F ? "fmaxf(" + a + ", " + b + ")" : "(" + a + " > " + b + " ? " + a + " : " + b + ")";
         case BOp::And: return cls == Cls::B ? a + " && " + b : a + " & " + b;
@@ -317,7 +317,19 @@ std::string emit_exprs(const Program& p, const EmitCtx& cx) {
                 else each(e.bits ? "true" : "false");
                 break;
             case Expr::Unary: each(unary_expr(e, ref(e.a), p.fast_math)); break;
-            case Expr::Binary: each(binary_expr(e, e.cls, ref(e.a), ref(e.b), p.fast_math)); break;
+            case Expr::Binary: {
+                const Expr& rhs = p.exprs[e.b];
+                if ((BOp)e.op == BOp::Pow && rhs.kind == Expr::Const && rhs.cls == Cls::F) {
+                    // x ** 1 and x ** 2 are exact products; any other exponent takes the precise powf (the fast
+                    // exp2(y * log2(x)) form is undefined for negative bases).
+                    float y;
+                    memcpy(&y, &rhs.bits, 4);
+                    if (y == 1.0f) { each(ref(e.a)); break; }
+                    if (y == 2.0f) { each(ref(e.a) + " * " + ref(e.a)); break; }
+                }
+                each(binary_expr(e, e.cls, ref(e.a), ref(e.b), p.fast_math));
+                break;
+            }
             case Expr::Compare: each(ref(e.a) + " " + compare_sym(e.op) + " " + ref(e.b)); break;
             case Expr::Select: each(ref(e.c) + " ? " + ref(e.b) + " : " + ref(e.a)); break;  // rhs when true (jit.rs:583-586)
             case Expr::Cast: {

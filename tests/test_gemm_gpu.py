@@ -86,3 +86,38 @@ def test_reference_test_shape_4097_cubed_is_predicated(gpu):
 def test_4096_cubed_plain(gpu):
     g, inputs, outs = gemm_cases.plain(4096, 4096, 4096, seed=3, scale=0.02)
     check(g, inputs, outs, eps=1e-4)
+
+
+def check_reductions_and_full(g, inputs, rel_full=1e-2, rel_red=1e-3):
+    k = ha.TileKernel.fused(g)
+    print(k.description, flush=True)
+    got = run_tile_kernel_gpu(k, inputs)
+    want = oracle.outputs(g.nodes, inputs, round_mainloop_to="bf16")
+    for a in k.args:
+        if not a["is_output"]:
+            continue
+        gv, wv = got[a["node"]], want[a["node"]].reshape(-1)
+        if a["dtype"] == "bf16":
+            gv, wv = nm.bf16_bits_to_f32(gv).astype(np.float64), nm.bf16_bits_to_f32(wv).astype(np.float64)
+            ok = (np.abs(gv - wv) <= 1e-3) | (np.abs(gv - wv) <= rel_full * np.maximum(np.abs(gv), np.abs(wv)))
+            assert ok.all(), (a["node"], float(np.abs(gv - wv).max()))
+        else:
+            gv, wv = gv.astype(np.float64), wv.astype(np.float64)
+            assert np.abs(gv - wv).max() <= rel_red * np.abs(wv).max(), (a["node"], float(np.abs(gv - wv).max()), float(np.abs(wv).max()))
+
+
+@pytest.mark.parametrize("size,mainloop,full", [(256, False, False), (384, True, True), (1024, True, True), (4096, False, False),
+                                                (4096, True, True)])
+def test_c4_readme_fusion(gpu, size, mainloop, full):
+    from helium_amd import configs
+
+    g, outs = configs.c4_graph(size, mainloop=mainloop, full_size_outputs=full)
+    check_reductions_and_full(g, configs.c4_inputs(g, size))
+
+
+@pytest.mark.parametrize("size", [512, 4096])
+def test_c5a_mainloop_and_epilogue(gpu, size):
+    from helium_amd import configs
+
+    g, names = configs.c5a_graph(size)
+    check_reductions_and_full(g, configs.c5a_inputs(names, size))
