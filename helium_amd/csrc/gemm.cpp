@@ -22,7 +22,8 @@ namespace {
 
 struct Tile {
     int bm = 256, bn = 256, bk = 64;  // workgroup tile
-    int wm = 2, wn = 2;               // waves along m / n (wm * wn * 64 threads)
+    int wm = 2, wn = 4;               // waves along m / n (wm * wn * 64 threads)
+    int stages = 2;                   // LDS stages (direct global->LDS loads use a deeper ring)
 };
 
 const char* kGemmPrelude = R"HIP(
@@ -36,6 +37,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 #ifndef LDS_AS
 #define LDS_AS __attribute__((address_space(3)))
+#define GLOBAL_AS __attribute__((address_space(1)))
 #endif
 )HIP";
 
@@ -57,11 +59,13 @@ __device__ __forceinline__ u32x4 pack8(const float (&v)[8]) {
 
 // Kernel body; problem and tile constants are #defines in front of it.
 const char* kGemmBody = R"HIP(
-#define NTHREADS (WAVES_M * WAVES_N * 64)
+#define NWAVES (WAVES_M * WAVES_N)
+#define NTHREADS (NWAVES * 64)
 #define WTM (BM / WAVES_M)        /* wave tile */
 #define WTN (BN / WAVES_N)
 #define MB (WTM / 32)             /* 32x32 MFMA blocks per wave tile */
 #define NB (WTN / 32)
+#define KK (BK / 16)              /* MFMA k-steps per tile */
 #define A_CHUNKS (BK / 8)         /* 16-byte chunks per A row */
 #define B_CHUNKS (BN / 8)
 #define A_TILE_BYTES (BM * BK * 2)
@@ -70,27 +74,33 @@ const char* kGemmBody = R"HIP(
 #define A_PER_THREAD (BM * A_CHUNKS / NTHREADS)
 #define B_PER_THREAD (BK * B_CHUNKS / NTHREADS)
 #define EP (WTN + 4)              /* float pitch of the epilogue strip */
+#if NSTAGES * STAGE_BYTES < NWAVES * 32 * EP * 4
+#error "the epilogue strip does not fit in the operand stages"
+#endif
 #define KT ((GK + BK - 1) / BK)
 
-__device__ __forceinline__ u32 a_off(u32 m, u32 kc) { return m * (BK * 2) + ((kc ^ (m & (A_CHUNKS - 1))) << 4); }
+__device__ __forceinline__ u32 a_off(u32 m, u32 kc) { return m * (BK * 2) + ((kc ^ ((m >> A_SWZ_SHIFT) & (A_CHUNKS - 1))) << 4); }
 __device__ __forceinline__ u32 b_off(u32 k, u32 n) {
     return k * (BN * 2) + ((((n >> 3) ^ ((k & 3) << 2))) << 4) + ((n & 7) << 1);
 }
 
 #ifndef KERNEL_ATTRS
-#define KERNEL_ATTRS __attribute__((amdgpu_waves_per_eu(1, 1)))  /* one wave per SIMD: the full 512-register budget */
+/* NWAVES / 4 waves per SIMD: with four waves each one owns the full 512-register budget */
+#define KERNEL_ATTRS __attribute__((amdgpu_waves_per_eu(NWAVES / 4, NWAVES / 4)))
 #endif
 extern "C" __global__ __launch_bounds__(NTHREADS) KERNEL_ATTRS
 void fused_matmul(KERNEL_PARAMS) {
-    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * STAGE_BYTES];
+    __shared__ __attribute__((aligned(16))) unsigned char lds[NSTAGES * STAGE_BYTES];
     const u32 tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const u32 wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
-    // Tile order: consecutive workgroups walk down a column of tiles, so the workgroups resident at the same time
-    // share B panels (and, through the XCD round-robin, spread A panels over all L2s).
-    const u32 tiles_m = (GM + BM - 1) / BM;
-    const u32 tile_m = blockIdx.x % tiles_m, tile_n = blockIdx.x / tiles_m;
+    u32 tile_m, tile_n;
+    TILE_ORDER
     const u32 bz = blockIdx.y;
     const u32 m0 = tile_m * BM, n0 = tile_n * BN;
+    // Optional rotation of the k loop per workgroup (tuning knob, off by default: workgroups that share an A or B
+    // panel read the same k range at the same time, which is what lets them share it through L2).
+    const u32 k_shift = (STAGGER_EXPR) % KT;
+    auto k_tile = [&](u32 kt) { u32 x = kt + k_shift; return x >= KT ? x - KT : x; };
 
     f32x16 acc[MB][NB];
 #pragma unroll
@@ -102,7 +112,7 @@ void fused_matmul(KERNEL_PARAMS) {
 
     u32x4 sa[A_PER_THREAD], sb[B_PER_THREAD];
     auto stage_load = [&](u32 kt) {
-        const u32 k0 = kt * BK;
+        const u32 k0 = k_tile(kt) * BK;
 #pragma unroll
         for (int i = 0; i < A_PER_THREAD; i++) {
             const u32 idx = tid + i * NTHREADS;
@@ -130,51 +140,148 @@ void fused_matmul(KERNEL_PARAMS) {
             *(u32x4*)(lb + b_off(idx / B_CHUNKS, (idx % B_CHUNKS) * 8)) = sb[i];
         }
     };
-    auto compute = [&](u32 buf) {
+    const u32 grp = lane >> 4, sub = lane & 15;
+    auto load_frags = [&](u32 buf, int kk, s16x8 (&af)[MB], s16x8 (&bf)[NB]) {
         const unsigned char* la = lds + buf * STAGE_BYTES;
         const unsigned char* lb = la + A_TILE_BYTES;
-        const u32 g = lane >> 4, r = lane & 15;
 #pragma unroll
-        for (int kk = 0; kk < BK / 16; kk++) {
-            s16x8 af[MB], bf[NB];
+        for (int i = 0; i < MB; i++) {
+            const u32 row = wave_m * WTM + i * 32 + (lane & 31);
+            af[i] = *(const s16x8*)(la + a_off(row, kk * 2 + (lane >> 5)));
+        }
 #pragma unroll
-            for (int i = 0; i < MB; i++) {
-                const u32 row = wave_m * WTM + i * 32 + (lane & 31);
-                af[i] = *(const s16x8*)(la + a_off(row, kk * 2 + (lane >> 5)));
-            }
-#pragma unroll
-            for (int j = 0; j < NB; j++) {
-                const u32 k = kk * 16 + (g >> 1) * 8 + (r >> 2);
-                const u32 n = wave_n * WTN + j * 32 + (g & 1) * 16 + (r & 3) * 4;
-                s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(lb + b_off(k, n)));
-                s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(lb + b_off(k + 4, n)));
-                bf[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            }
-#pragma unroll
-            for (int i = 0; i < MB; i++)
-#pragma unroll
-                for (int j = 0; j < NB; j++) {
-#if MMA_BF16
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[i]),
-                                                                       __builtin_bit_cast(bf16x8, bf[j]), acc[i][j], 0, 0, 0);
-#else
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, af[i]),
-                                                                      __builtin_bit_cast(f16x8, bf[j]), acc[i][j], 0, 0, 0);
-#endif
-                }
+        for (int j = 0; j < NB; j++) {
+            const u32 k = kk * 16 + (grp >> 1) * 8 + (sub >> 2);
+            const u32 n = wave_n * WTN + j * 32 + (grp & 1) * 16 + (sub & 3) * 4;
+            s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(lb + b_off(k, n)));
+            s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(lb + b_off(k + 4, n)));
+            bf[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         }
     };
+    auto mma = [&](const s16x8 (&af)[MB], const s16x8 (&bf)[NB]) {
+#pragma unroll
+        for (int i = 0; i < MB; i++)
+#pragma unroll
+            for (int j = 0; j < NB; j++) {
+#if MMA_BF16
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[i]),
+                                                                   __builtin_bit_cast(bf16x8, bf[j]), acc[i][j], 0, 0, 0);
+#else
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, af[i]),
+                                                                  __builtin_bit_cast(f16x8, bf[j]), acc[i][j], 0, 0, 0);
+#endif
+            }
+    };
+    // One k-tile: operands for step kk+1 are fetched from LDS while the MFMAs of step kk run.
+    auto compute = [&](u32 buf, auto&& per_step) {
+        s16x8 af[2][MB], bf[2][NB];
+        load_frags(buf, 0, af[0], bf[0]);
+#pragma unroll
+        for (int kk = 0; kk < KK; kk++) {
+            per_step(kk);  // a slice of the next tile's global->LDS traffic, spread over the MFMA steps
+#if GEMM_SKIP & 2
+            if (kk + 1 < KK) { for (int i = 0; i < MB; i++) af[(kk + 1) & 1][i] = af[kk & 1][i]; for (int j = 0; j < NB; j++) bf[(kk + 1) & 1][j] = bf[kk & 1][j]; }
+#else
+            if (kk + 1 < KK) load_frags(buf, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+#endif
+#if !(GEMM_SKIP & 4)
+            mma(af[kk & 1], bf[kk & 1]);
+#else
+            acc[0][0][0] += (float)af[kk & 1][0][0] + (float)bf[kk & 1][0][0];
+#endif
+            SCHED_HINT
+        }
+        SCHED_PLAN
+    };
 
+#if DIRECT_LOADS
+    // Operand tiles go from global memory straight into LDS (global_load_lds_dwordx4): a wave instruction fills
+    // 1 KB of LDS in lane order, so each lane fetches the global chunk whose swizzled LDS slot is lane * 16.
+/* s_waitcnt immediate: vmcnt lives in bits [3:0] and [15:14] */
+#define WAITCNT_VM(n) ((((n) & 15) | (((n) >> 4) << 14)))
+#define A_DPW (A_TILE_BYTES / 1024 / NWAVES)  /* direct-load instructions per wave and tile */
+#define B_DPW (B_TILE_BYTES / 1024 / NWAVES)
+    auto direct_issue = [&](u32 kt, u32 buf, int i) {
+#if GEMM_SKIP & 1
+        return;
+#endif
+        unsigned char* la = lds + buf * STAGE_BYTES;
+        unsigned char* lb = la + A_TILE_BYTES;
+        const u32 k0 = k_tile(kt) * BK;
+        if (i < A_DPW) {
+            const u32 blk = wave * A_DPW + i;
+            const u32 row = blk * (64 / A_CHUNKS) + lane / A_CHUNKS, pc = lane % A_CHUNKS;
+            const u32 kc = pc ^ ((row >> A_SWZ_SHIFT) & (A_CHUNKS - 1));
+            const bf16_t* gp = (const bf16_t*)DIRECT_A_PTR + ((size_t)bz * GM + m0 + row) * GK + k0 + kc * 8;
+            __builtin_amdgcn_global_load_lds((GLOBAL_AS const void*)gp, (LDS_AS void*)(la + blk * 1024), 16, 0, 0);
+        } else {
+            const u32 blk = wave * B_DPW + (i - A_DPW);
+            const u32 krow = blk * (64 / B_CHUNKS) + lane / B_CHUNKS, pc = lane % B_CHUNKS;
+            const u32 nc = pc ^ ((krow & 3) << 2);
+            const bf16_t* gp = (const bf16_t*)DIRECT_B_PTR + ((size_t)bz * GK + k0 + krow) * GN + n0 + nc * 8;
+            __builtin_amdgcn_global_load_lds((GLOBAL_AS const void*)gp, (LDS_AS void*)(lb + blk * 1024), 16, 0, 0);
+        }
+    };
+    // NSTAGES-deep ring of LDS stages: tile kt + NSTAGES - 1 is requested while tile kt is multiplied, so a
+    // wave only ever waits for loads issued NSTAGES - 2 tiles earlier.
+#pragma unroll
+    for (int st = 0; st < NSTAGES - 1; st++)
+        if (st < KT) {
+#pragma unroll
+            for (int i = 0; i < A_DPW + B_DPW; i++) direct_issue(st, st, i);
+        }
+#if GEMM_TIMING
+    unsigned long long t_load = 0, t_compute = 0, t_wait = 0, t_barrier = 0, t0, t1;
+#define TICK(var) t1 = __builtin_readcyclecounter(); var += t1 - t0; t0 = t1;
+    t0 = __builtin_readcyclecounter();
+#else
+#define TICK(var)
+#endif
+    for (u32 kt = 0; kt < KT; kt++) {
+        // tile kt must have landed; up to NSTAGES - 2 younger tiles may still be in flight
+        const u32 younger = KT - 1 - kt < NSTAGES - 2 ? KT - 1 - kt : NSTAGES - 2;
+        if (younger >= 2) __builtin_amdgcn_s_waitcnt(0x0F70 | WAITCNT_VM(2 * (A_DPW + B_DPW)));
+        else if (younger == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | WAITCNT_VM(A_DPW + B_DPW));
+        else __builtin_amdgcn_s_waitcnt(0x0F70);
+        TICK(t_wait)
+        __syncthreads();
+        TICK(t_barrier)
+        const u32 next = kt + NSTAGES - 1;
+        const bool more = next < KT;
+        compute(kt % NSTAGES, [&](int kk) {
+            constexpr int per = (A_DPW + B_DPW + KK - 1) / KK;
+            if (more) {
+#pragma unroll
+                for (int i = kk * per; i < (kk + 1) * per && i < A_DPW + B_DPW; i++) direct_issue(next, next % NSTAGES, i);
+            }
+        });
+        __builtin_amdgcn_sched_barrier(0);
+        TICK(t_compute)
+    }
+    __syncthreads();
+#if GEMM_TIMING
+    if (blockIdx.x == 0 && tid == 64) {
+        unsigned long long* dbg = (unsigned long long*)GEMM_TIMING_PTR;
+        dbg[0] = t_load; dbg[1] = t_compute; dbg[2] = t_wait; dbg[3] = t_barrier;
+    }
+    __syncthreads();
+    if (blockIdx.x == 0) return;
+#endif
+#else
     stage_load(0);
     stage_store(0);
     __syncthreads();
     for (u32 kt = 0; kt < KT; kt++) {
         const bool more = kt + 1 < KT;
+        // The next tile's global loads are issued before any MFMA of this tile and consumed after the last one.
         if (more) stage_load(kt + 1);
-        compute(kt & 1);
+        STAGE_SCHED_BARRIER
+        compute(kt & 1, [](int) {});
+        STAGE_SCHED_BARRIER
         if (more) stage_store((kt + 1) & 1);
         __syncthreads();
     }
+#endif
 
     // ---- epilogue: accumulators -> wave-private LDS strip -> row-major NV-wide vectors -----------------------
     float* strip = (float*)lds + wave * (32 * EP);
@@ -295,23 +402,38 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
                HE_ERR_INVALID, "GEMM too large");
     HE_REQUIRE(pr.mma_dtype == HE_BF16 || pr.mma_dtype == HE_F16, HE_ERR_UNSUPPORTED, "unsupported multiplicand type");
     Tile t;
+    const bool raw_a0 = is_raw_copy(pr.op_a, pr.root_a, pr.mma_dtype) && pr.K % 8 == 0;
+    const bool raw_b0 = is_raw_copy(pr.op_b, pr.root_b, pr.mma_dtype) && pr.N % 8 == 0;
+    bool want_direct = raw_a0 && raw_b0 && !getenv("HELIUM_HIP_GEMM_NO_DIRECT");
     if (const char* env = getenv("HELIUM_HIP_GEMM_TILE")) {
-        int a, b, c, d, e;
-        if (sscanf(env, "%d,%d,%d,%d,%d", &a, &b, &c, &d, &e) == 5) t = {a, b, c, d, e};
+        int v[6] = {256, 256, 64, 2, 4, 2};
+        int n = sscanf(env, "%d,%d,%d,%d,%d,%d", &v[0], &v[1], &v[2], &v[3], &v[4], &v[5]);
+        HE_REQUIRE(n >= 5, HE_ERR_INVALID, "HELIUM_HIP_GEMM_TILE wants bm,bn,bk,wm,wn[,stages]");
+        t = {v[0], v[1], v[2], v[3], v[4], v[5]};
     } else {
         // Smaller problems take smaller tiles so that every CU gets work.
         if (pr.M <= 128 || pr.N <= 128 || ((pr.M + 255) / 256) * ((pr.N + 255) / 256) * pr.batch < 128) {
             t.bm = t.bn = 128;
+            t.wm = t.wn = 2;
         }
     }
-    HE_REQUIRE(t.bm % (t.wm * 32) == 0 && t.bn % (t.wn * 32) == 0 && t.bk == 64, HE_ERR_INVALID, "bad GEMM tile");
+    HE_REQUIRE(t.bm % (t.wm * 32) == 0 && t.bn % (t.wn * 32) == 0 && (t.bk == 64 || t.bk == 32), HE_ERR_INVALID, "bad GEMM tile");
     const int threads = t.wm * t.wn * 64;
+    HE_REQUIRE(threads == 256 || threads == 512, HE_ERR_INVALID, "GEMM workgroups have 4 or 8 waves");
     HE_REQUIRE((t.bm * t.bk / 8) % threads == 0 && (t.bk * t.bn / 8) % threads == 0, HE_ERR_INVALID, "bad GEMM tile");
+    HE_REQUIRE(t.stages >= 2 && t.stages <= 4 && t.stages * (t.bm + t.bn) * t.bk * 2 <= 160 * 1024, HE_ERR_INVALID,
+               "GEMM tile exceeds LDS");
     const int wtn = t.bn / t.wn;
 
     const bool raw_a = is_raw_copy(pr.op_a, pr.root_a, pr.mma_dtype) && pr.K % 8 == 0;
     const bool raw_b = is_raw_copy(pr.op_b, pr.root_b, pr.mma_dtype) && pr.N % 8 == 0;
     const int nva = tp::pick_nv(pr.op_a, 16), nvb = tp::pick_nv(pr.op_b, 16);
+    // Direct global->LDS loads need unpredicated, unmodified 16-byte chunks: raw operands and full tiles everywhere.
+    const bool direct = want_direct && raw_a && raw_b && pr.M % t.bm == 0 && pr.N % t.bn == 0 && pr.K % t.bk == 0 &&
+                        (t.bm * t.bk * 2 / 1024) % (threads / 64) == 0 && (t.bk * t.bn * 2 / 1024) % (threads / 64) == 0 &&
+                        64 % (t.bn / 8) == 0;
+    if (!direct) t.stages = 2;
+    if (!direct) t.stages = 2;
     int nve = tp::pick_nv(pr.epi, 32);
     while (nve > 1 && ((32 * wtn) % (64 * nve) != 0)) nve /= 2;
     nve = std::min(nve, 8);
@@ -324,8 +446,13 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     s << tp::emit_prelude(pr.epi) << kGemmPrelude;
     s << "#define GM " << pr.M << "u\n#define GN " << pr.N << "u\n#define GK " << pr.K << "u\n";
     s << "#define BM " << t.bm << "\n#define BN " << t.bn << "\n#define BK " << t.bk << "\n#define WAVES_M " << t.wm
-      << "\n#define WAVES_N " << t.wn << "\n#define NVE " << nve << "\n#define MMA_BF16 " << (pr.mma_dtype == HE_BF16 ? 1 : 0)
-      << "\n";
+      << "\n#define WAVES_N " << t.wn << "\n#define NSTAGES " << t.stages << "\n#define NVE " << nve << "\n#define MMA_BF16 " << (pr.mma_dtype == HE_BF16 ? 1 : 0)
+      << "\n#define STAGGER_EXPR " << (getenv("HELIUM_HIP_GEMM_STAGGER") ? getenv("HELIUM_HIP_GEMM_STAGGER") : "0u")
+      << "\n#define GEMM_SKIP " << (getenv("HELIUM_HIP_GEMM_SKIP") ? atoi(getenv("HELIUM_HIP_GEMM_SKIP")) : 0)
+      << "\n#define GEMM_TIMING " << (getenv("HELIUM_HIP_GEMM_TIMING") ? 1 : 0) << "\n#define GEMM_TIMING_PTR p" << (pr.args.size() - 1)
+      << "\n#define DIRECT_LOADS " << (direct ? 1 : 0) << "\n#define DIRECT_A_PTR p" << (direct ? pr.map_a[0] : 0)
+      << "\n#define DIRECT_B_PTR p" << (direct ? pr.map_b[0] : 0) << "\n#define STAGE_SCHED_BARRIER "
+      << (getenv("HELIUM_HIP_GEMM_PIN") ? "__builtin_amdgcn_sched_barrier(0);" : "") << "\n#define A_SWZ_SHIFT " << (getenv("HELIUM_HIP_GEMM_ASWZ") ? atoi(getenv("HELIUM_HIP_GEMM_ASWZ")) : (t.bk == 64 ? 1 : 2)) << "\n";
 
     s << kGemmHelpers;
     // kernel parameters
@@ -337,7 +464,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     }
     // operand fetchers
     auto emit_fetch = [&](const char* which, const tp::Program& p, int root, const std::vector<int>& map, bool raw, int nv,
-                          const char* rows, const char* cols) {
+                          const char* rows, const char* cols, bool aligned) {
         // rows/cols: extents of the operand matrix ("GM","GK" for A; "GK","GN" for B)
         std::ostringstream args, params;
         for (size_t a = 0; a < p.args.size(); a++) {
@@ -348,7 +475,10 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         s << "#define FETCH_" << (W == "a" ? "A" : "B") << "_ARGS " << args.str() << "\n";
         if (!raw) s << emit_operand_fn(p, root, "operand_" + W, nv);
         s << "__device__ __forceinline__ u32x4 fetch_" << W << "(" << params.str() << "u32 b, u32 row, u32 col) {\n";
-        if (raw) {
+        if (raw && aligned) {
+            // every tile is full: no predication on the operand loads
+            s << "return *(const u32x4*)(q0 + ((size_t)b * " << rows << " + row) * " << cols << " + col);\n}\n";
+        } else if (raw) {
             s << "u32x4 v = {0u, 0u, 0u, 0u};\nif (row < " << rows << " && col < " << cols << ") v = *(const u32x4*)(q0 + ((size_t)b * "
               << rows << " + row) * " << cols << " + col);\nreturn v;\n}\n";
         } else {
@@ -358,8 +488,8 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
             s << "b, row, col + j, v + j);\nelse {\n#pragma unroll\nfor (int k = 0; k < " << nv << "; k++) v[j + k] = 0.0f; }\n}\nreturn pack8(v);\n}\n";
         }
     };
-    emit_fetch("a", pr.op_a, pr.root_a, pr.map_a, raw_a, nva, "GM", "GK");
-    emit_fetch("b", pr.op_b, pr.root_b, pr.map_b, raw_b, nvb, "GK", "GN");
+    emit_fetch("a", pr.op_a, pr.root_a, pr.map_a, raw_a, nva, "GM", "GK", pr.M % t.bm == 0 && pr.K % t.bk == 0);
+    emit_fetch("b", pr.op_b, pr.root_b, pr.map_b, raw_b, nvb, "GK", "GN", pr.K % t.bk == 0 && pr.N % t.bn == 0);
 
     // epilogue pieces
     std::ostringstream setup, body, finish;
@@ -430,6 +560,59 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         HE_REQUIRE(pos != std::string::npos, HE_ERR_INTERNAL, "kernel template lacks %s", marker.c_str());
         body_text.replace(pos, marker.size(), text);
     };
+    {
+        // Tile order. Workgroups are dealt round-robin to the 8 XCDs, each with its own L2: when the tile count
+        // allows, XCD x takes the x-th eighth of a sequence in which groups of 4 tile rows are walked column by
+        // column, so the tiles resident on one XCD form a compact block sharing few A and B panels.
+        const int64_t tm = (pr.M + t.bm - 1) / t.bm, tn = (pr.N + t.bn - 1) / t.bn;
+        std::ostringstream o;
+        const bool xcd = (tm * tn) % 8 == 0 && !getenv("HELIUM_HIP_GEMM_NO_XCD");
+        o << "{ u32 b = blockIdx.x;\n";
+        if (xcd) o << "b = (b % 8u) * " << (tm * tn / 8) << "u + b / 8u;\n";
+        const int G = getenv("HELIUM_HIP_GEMM_GROUP") ? atoi(getenv("HELIUM_HIP_GEMM_GROUP")) : 4;
+        o << "const u32 gsize = " << G * tn << "u, group = b / gsize, first = group * " << G << "u;\n";
+        o << "const u32 rows = (" << tm << "u - first) < " << G << "u ? (" << tm << "u - first) : " << G << "u;\n";
+        o << "tile_m = first + (b % gsize) % rows; tile_n = (b % gsize) / rows; }\n";
+        splice("TILE_ORDER", o.str());
+        std::ostringstream h;
+        if (getenv("HELIUM_HIP_GEMM_SCHED")) {
+            // ask the scheduler to alternate LDS reads with MFMAs instead of batching either
+            h << "_Pragma(\"unroll\") for (int q = 0; q < MB + 2 * NB; q++) { __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); "
+                 "__builtin_amdgcn_sched_group_barrier(0x008, 1, 0); }\n";
+            h << "__builtin_amdgcn_sched_group_barrier(0x008, MB * NB - (MB + 2 * NB) > 0 ? MB * NB - (MB + 2 * NB) : 0, 0);\n";
+        }
+        splice("SCHED_HINT", h.str());
+        std::ostringstream plan;
+        const int mode = getenv("HELIUM_HIP_GEMM_PLAN") ? atoi(getenv("HELIUM_HIP_GEMM_PLAN")) : 2;
+        const int mb = t.bm / t.wm / 32, nb = t.bn / t.wn / 32, kk_steps = t.bk / 16;
+        const int nr = mb + 2 * nb, nm = mb * nb;
+        if (mode == 1) {
+            // all operand reads of step kk+1 are issued ahead of the MFMAs of step kk
+            plan << "__builtin_amdgcn_sched_group_barrier(0x100, " << nr << ", 0);\n";
+            for (int kk = 0; kk < kk_steps; kk++) {
+                if (kk + 1 < kk_steps) plan << "__builtin_amdgcn_sched_group_barrier(0x100, " << nr << ", 0);\n";
+                plan << "__builtin_amdgcn_sched_group_barrier(0x008, " << nm << ", 0);\n";
+            }
+        } else if (mode == 2) {
+            // reads of step kk+1 are spread between the MFMAs of step kk
+            plan << "__builtin_amdgcn_sched_group_barrier(0x100, " << nr << ", 0);\n";
+            const int waves = threads / 64;
+            const int dl = direct ? (t.bm * t.bk * 2 / 1024 + t.bk * t.bn * 2 / 1024) / waves : 0;
+            const int per = (dl + kk_steps - 1) / kk_steps;
+            for (int kk = 0; kk < kk_steps; kk++) {
+                int issue = std::max(0, std::min(per, dl - kk * per));
+                if (issue) plan << "__builtin_amdgcn_sched_group_barrier(0x020, " << issue << ", 0);\n";
+                int reads = kk + 1 < kk_steps ? nr : 0, done_r = 0;
+                for (int m = 0; m < nm; m++) {
+                    int want_r = reads * (m + 1) / nm;
+                    if (want_r > done_r) plan << "__builtin_amdgcn_sched_group_barrier(0x100, " << (want_r - done_r) << ", 0);\n";
+                    done_r = want_r;
+                    plan << "__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);\n";
+                }
+            }
+        }
+        splice("SCHED_PLAN", plan.str());
+    }
     splice("EPILOGUE_SETUP", setup.str());
     splice("EPILOGUE_BODY", body.str());
     splice("EPILOGUE_FINISH", finish.str());
@@ -443,10 +626,10 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     threads_ = (uint32_t)threads;
     for (auto& o : pr.epi.outs)
         if (o.reduce) fills_.push_back({pr.map_e[o.arg], 0u});
-    describe_ = strfmt("gemm [%lld,%lld,%lld]x[%lld] tile=%dx%dx%d waves=%dx%d threads=%d grid=%ux%u rawA=%d rawB=%d NVA=%d NVB=%d NVE=%d "
-                       "mma=%s epilogue_exprs=%zu outs=%zu",
-                       (long long)pr.batch, (long long)pr.M, (long long)pr.K, (long long)pr.N, t.bm, t.bn, t.bk, t.wm, t.wn, threads,
-                       grid_[0], grid_[1], (int)raw_a, (int)raw_b, nva, nvb, nve, dtype_name(pr.mma_dtype), pr.epi.exprs.size(),
+    describe_ = strfmt("gemm [%lld,%lld,%lld]x[%lld] tile=%dx%dx%d stages=%d waves=%dx%d threads=%d grid=%ux%u rawA=%d rawB=%d NVA=%d NVB=%d NVE=%d "
+                       "direct=%d mma=%s epilogue_exprs=%zu outs=%zu",
+                       (long long)pr.batch, (long long)pr.M, (long long)pr.K, (long long)pr.N, t.bm, t.bn, t.bk, t.stages, t.wm, t.wn, threads,
+                       grid_[0], grid_[1], (int)raw_a, (int)raw_b, nva, nvb, nve, (int)direct, dtype_name(pr.mma_dtype), pr.epi.exprs.size(),
                        pr.epi.outs.size());
     kernel_.reset(new JitKernel(source_, "fused_matmul", {"-ffp-contract=fast", "-munsafe-fp-atomics"}));
 }
