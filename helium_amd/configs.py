@@ -29,6 +29,36 @@ def permute_input(name, seed=None):
     return bf16_rne(rng.standard_normal(size=shape, dtype=np.float32))
 
 
+def c1_graph(rows=256, inner=512, cols=512):
+    """Config 1 as one Core fusion: Y = relu(X W + b) and the sum of Y over columns (fold of the row axis), all f32."""
+    g = fusion.OpGraph()
+    x, w = g.producer([1, rows, inner], "f32"), g.producer([1, inner, cols], "f32")
+    b = g.producer([1, 1, cols], "f32")
+    y = g.unary(g.binary(g.matmul(x, w), g.broadcast(b, 1, rows), "add"), "relu")
+    return g, {"x": x, "w": w, "b": b, "y": g.consumer(y, "f32"),
+               "colsum": g.consumer(g.reduction(y, "columns"), "f32")}
+
+
+def c1_ir_graph(rows=256, inner=512, cols=512):
+    """Config 1 as the lazy-tensor front end records it (helium-ir): Matmul, broadcast-add, Relu, and the column
+    sum as swap_dims + Reduce(depth 1); execute_graph plans it as a GEMM and two pointwise kernels."""
+    from . import ir
+
+    g = ir.OpGraph()
+    x, w, b = g.new_input([rows, inner], "f32"), g.new_input([inner, cols], "f32"), g.new_input([cols], "f32")
+    y = g.unary(g.binary(g.matmul(x, w, "f32_f32"), g.broadcast(b, 2, [(0, rows)]), "add"), "relu")
+    colsum = g.reduce(g.swap_dims(y, 0, 1), "sum", 1)
+    return g, {"x": x, "w": w, "b": b, "y": g.new_output(y), "colsum": g.new_output(colsum)}
+
+
+def c1_inputs(names, rows=256, inner=512, cols=512, seed=11, batched=True):
+    rng = np.random.default_rng(seed)
+    lead = (1,) if batched else ()
+    return {names["x"]: rng.uniform(-1, 1, lead + (rows, inner)).astype(np.float32),
+            names["w"]: rng.uniform(-1, 1, lead + (inner, cols)).astype(np.float32),
+            names["b"]: rng.uniform(-1, 1, (lead + (1, cols)) if batched else (cols,)).astype(np.float32)}
+
+
 def c3_chain(rows=4096, cols=4096, bias_axis=2, seed=31, make_inputs=True):
     """Config 3: Add, broadcast-add of a bias, Relu, Tanh, Neg, AddConstant(1.0), Mul, Sub, PowConstant(2.0),
     MulConstant(1/4096), then Sum over batch and over columns; f32, U(-1,1).

@@ -5,15 +5,7 @@
 #include "ir.h"
 #include "kernels.h"
 
-struct he_graph_s {
-    std::shared_ptr<he::ir::OpGraph> g = std::make_shared<he::ir::OpGraph>();
-};
-struct he_fgraph_s {
-    he::fir::OpGraph g;
-};
-struct he_tile_kernel_s {
-    std::unique_ptr<he::KernelBase> k;
-};
+#include "capi_types.h"
 
 namespace he {
 ir::Op op_from_desc(const he_op_desc& d) {

@@ -1,0 +1,319 @@
+#include "exec.h"
+
+#include <algorithm>
+#include <cstring>
+#include <future>
+#include <set>
+
+namespace he::exec {
+
+// ---------------------------------------------------------------------------------------------------------
+// Device pool
+// ---------------------------------------------------------------------------------------------------------
+DevicePool& DevicePool::global() {
+    static DevicePool* pool = new DevicePool();  // never destroyed: tensors may outlive static destruction order
+    return *pool;
+}
+
+size_t DevicePool::size_class(size_t bytes) {
+    // 256-byte granules up to 1 MiB, then 2 MiB granules: few distinct sizes, so freed blocks get reused
+    if (bytes == 0) bytes = 1;
+    if (bytes <= (1u << 20)) {
+        size_t c = 256;
+        while (c < bytes) c *= 2;
+        return c;
+    }
+    const size_t g = 2u << 20;
+    return (bytes + g - 1) / g * g;
+}
+
+uint64_t DevicePool::begin_scope() {
+    std::lock_guard<std::mutex> lk(mu_);
+    uint64_t s = next_scope_++;
+    free_scoped_[s];
+    return s;
+}
+
+void DevicePool::end_scope(uint64_t scope) {
+    std::lock_guard<std::mutex> lk(mu_);
+    auto it = free_scoped_.find(scope);
+    if (it == free_scoped_.end()) return;
+    for (auto& kv : it->second) free_global_.insert(kv);
+    free_scoped_.erase(it);
+    for (size_t i = 0; i < deferred_.size();) {
+        auto& w = deferred_[i].waiting;
+        w.erase(std::remove(w.begin(), w.end(), scope), w.end());
+        if (w.empty()) {
+            free_global_.insert({deferred_[i].cls, deferred_[i].ptr});
+            deferred_[i] = deferred_.back();
+            deferred_.pop_back();
+        } else {
+            i++;
+        }
+    }
+}
+
+void DevicePool::note_use(Tensor& t, uint64_t scope) {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (std::find(t.used.begin(), t.used.end(), scope) == t.used.end()) t.used.push_back(scope);
+}
+
+void* DevicePool::allocate(size_t bytes, uint64_t scope) {
+    const size_t cls = size_class(bytes);
+    {
+        std::lock_guard<std::mutex> lk(mu_);
+        auto take = [&](std::multimap<size_t, void*>& m) -> void* {
+            auto it = m.find(cls);
+            if (it == m.end()) return nullptr;
+            void* p = it->second;
+            m.erase(it);
+            reuses_++;
+            return p;
+        };
+        auto sc = free_scoped_.find(scope);
+        if (sc != free_scoped_.end())
+            if (void* p = take(sc->second)) return p;
+        if (void* p = take(free_global_)) return p;
+        driver_bytes_ += cls;
+        driver_allocs_++;
+    }
+    void* p = nullptr;
+    HE_HIP(hipMalloc(&p, cls));
+    return p;
+}
+
+void DevicePool::release(void* ptr, size_t bytes, uint64_t owner, const std::vector<uint64_t>& used) {
+    if (!ptr) return;
+    std::lock_guard<std::mutex> lk(mu_);
+    const size_t cls = size_class(bytes);
+    std::vector<uint64_t> live;
+    for (uint64_t s : used)
+        if (s != owner && free_scoped_.count(s)) live.push_back(s);
+    auto own = free_scoped_.find(owner);
+    if (live.empty()) {
+        if (own != free_scoped_.end()) own->second.insert({cls, ptr});
+        else free_global_.insert({cls, ptr});
+        return;
+    }
+    if (own != free_scoped_.end()) live.push_back(owner);
+    deferred_.push_back({ptr, cls, std::move(live)});
+}
+
+void DevicePool::stats(uint64_t* driver_bytes, uint64_t* driver_allocs, uint64_t* reuses) {
+    std::lock_guard<std::mutex> lk(mu_);
+    *driver_bytes = driver_bytes_;
+    *driver_allocs = driver_allocs_;
+    *reuses = reuses_;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Tensors
+// ---------------------------------------------------------------------------------------------------------
+Tensor::~Tensor() {
+    if (ready) {
+        if (uploaded) (void)hipEventSynchronize(ready);  // the copy that fills the block may still be queued
+        (void)hipEventDestroy(ready);
+    }
+    DevicePool::global().release(ptr, bytes, scope, used);
+}
+
+TensorRef allocate_tensor(int dtype, size_t len, uint64_t scope) {
+    auto t = std::make_shared<Tensor>();
+    t->dtype = dtype;
+    t->len = len;
+    t->bytes = storage_bytes(dtype, len);
+    t->scope = scope;
+    t->ptr = DevicePool::global().allocate(t->bytes, scope);
+    HE_HIP(hipEventCreateWithFlags(&t->ready, hipEventDisableTiming));
+    return t;
+}
+
+namespace {
+struct Staging {
+    void* host = nullptr;
+    size_t capacity = 0;
+    hipEvent_t done = nullptr;
+};
+struct Streams {
+    std::vector<hipStream_t> s;
+    hipStream_t h2d = nullptr, d2h = nullptr;
+    std::vector<Staging> staging;  // pinned upload buffers, reused once their copy has finished
+};
+// A pinned buffer of at least `bytes` whose previous copy (if any) has completed.
+Staging& staging_buffer(Streams& st, size_t bytes) {
+    for (Staging& b : st.staging)
+        if (b.capacity >= bytes && hipEventQuery(b.done) == hipSuccess) return b;
+    // drop finished buffers that are too small before growing: keeps at most a few per thread
+    for (size_t i = 0; i < st.staging.size();) {
+        if (hipEventQuery(st.staging[i].done) == hipSuccess) {
+            (void)hipHostFree(st.staging[i].host);
+            (void)hipEventDestroy(st.staging[i].done);
+            st.staging[i] = st.staging.back();
+            st.staging.pop_back();
+        } else {
+            i++;
+        }
+    }
+    Staging b;
+    b.capacity = std::max<size_t>(bytes, 1u << 20);
+    HE_HIP(hipHostMalloc(&b.host, b.capacity, hipHostMallocDefault));
+    HE_HIP(hipEventCreateWithFlags(&b.done, hipEventDisableTiming));
+    st.staging.push_back(b);
+    return st.staging.back();
+}
+Streams& thread_streams() {
+    // a small pool of non-blocking streams per host thread (helium/src/cuda/context.rs:112-125)
+    static thread_local Streams st;
+    if (st.s.empty()) {
+        const int n = 4;
+        for (int i = 0; i < n; i++) {
+            hipStream_t x;
+            HE_HIP(hipStreamCreateWithFlags(&x, hipStreamNonBlocking));
+            st.s.push_back(x);
+        }
+        HE_HIP(hipStreamCreateWithFlags(&st.h2d, hipStreamNonBlocking));
+        HE_HIP(hipStreamCreateWithFlags(&st.d2h, hipStreamNonBlocking));
+    }
+    return st;
+}
+}  // namespace
+
+TensorRef create_tensor_with_data(const void* data, int dtype, size_t len) {
+    TensorRef t = allocate_tensor(dtype, len, 0);
+    Streams& st = thread_streams();
+    if (t->bytes) {
+        // staged through pinned memory so that the copy is asynchronous (tensor_storage.rs:83-110)
+        Staging& b = staging_buffer(st, t->bytes);
+        memcpy(b.host, data, t->bytes);
+        HE_HIP(hipMemcpyAsync(t->ptr, b.host, t->bytes, hipMemcpyHostToDevice, st.h2d));
+        HE_HIP(hipEventRecord(b.done, st.h2d));
+    }
+    t->uploaded = true;
+    HE_HIP(hipEventRecord(t->ready, st.h2d));
+    return t;
+}
+
+void download_tensor(const TensorRef& t, void* dst) {
+    Streams& st = thread_streams();
+    HE_HIP(hipStreamWaitEvent(st.d2h, t->ready, 0));
+    if (t->bytes) HE_HIP(hipMemcpyAsync(dst, t->ptr, t->bytes, hipMemcpyDeviceToHost, st.d2h));
+    HE_HIP(hipStreamSynchronize(st.d2h));
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// execute_graph
+// ---------------------------------------------------------------------------------------------------------
+std::map<NodeId, TensorRef> execute_graph(const ir::OpGraph& graph_in, const std::map<NodeId, TensorRef>& inputs,
+                                          ExecStats* stats) {
+    auto graph = std::make_shared<ir::OpGraph>(graph_in);
+    graph->optimize();
+    std::shared_ptr<const plan::Plan> plan = plan::generate_cached_plan(graph);
+
+    // begin_execute (cuda.rs:98-139): compile every kernel of the plan up front, in parallel (cuda.rs:262-270)
+    {
+        std::vector<std::future<void>> jobs;
+        for (auto& step : plan->steps)
+            for (auto& instr : step.instrs)
+                if (!instr->compiled()) jobs.push_back(std::async(std::launch::async, [instr] { instr->precompile(); }));
+        for (auto& j : jobs) j.get();
+    }
+    DevicePool& pool = DevicePool::global();
+    const uint64_t scope = pool.begin_scope();
+    Streams& st = thread_streams();
+    std::map<NodeId, TensorRef> tensors = inputs;
+    for (NodeId in : graph->inputs())
+        HE_REQUIRE(tensors.count(in), HE_ERR_INVALID, "missing storage for input node %u", in);
+    for (auto& kv : tensors) pool.note_use(*kv.second, scope);
+
+    // tensors that survive the plan get their ready event recorded (enumerate_output_tensors, cuda.rs:142-153)
+    std::set<NodeId> alive;
+    for (auto& step : plan->steps) {
+        for (auto& instr : step.instrs)
+            for (NodeId o : instr->outputs()) alive.insert(o);
+        for (NodeId r : step.tensors_to_release) alive.erase(r);
+    }
+
+    ExecStats local;
+    std::set<const Tensor*> synced;           // input tensors whose ready event a stream already waited on
+    std::vector<hipEvent_t> prev_events;      // one per stream used by the previous step
+    std::vector<hipEvent_t> all_events;
+    std::set<size_t> used_streams;
+    for (auto& step : plan->steps) {
+        for (NodeId r : step.tensors_to_release) tensors.erase(r);
+        if (step.instrs.empty()) continue;
+        local.steps++;
+        std::vector<const Tensor*> waited;
+        // Instructions of one step are independent: they fan out over the stream pool. Every stream used by this
+        // step first waits for every stream used by the previous one.
+        const size_t width = std::min(step.instrs.size(), st.s.size());
+        for (size_t w = 0; w < width; w++)
+            for (hipEvent_t e : prev_events) {
+                HE_HIP(hipStreamWaitEvent(st.s[w], e, 0));
+                local.event_waits++;
+            }
+        for (size_t i = 0; i < step.instrs.size(); i++) {
+            const plan::Instr& instr = *step.instrs[i];
+            hipStream_t stream = st.s[i % width];
+            used_streams.insert(i % width);
+            for (NodeId out : instr.outputs()) {
+                const ir::Descriptor& d = graph->get(out).desc;
+                tensors[out] = allocate_tensor(d.dtype, (size_t)ir::num_elements(d.shape), scope);
+            }
+            for (NodeId in : instr.inputs()) {
+                auto it = tensors.find(in);
+                HE_REQUIRE(it != tensors.end(), HE_ERR_INTERNAL, "missing storage for node %u", in);
+                // tensors made outside this execution carry a ready event (uploads, earlier graphs)
+                if (inputs.count(in) && !synced.count(it->second.get())) {
+                    HE_HIP(hipStreamWaitEvent(stream, it->second->ready, 0));
+                    local.event_waits++;
+                    waited.push_back(it->second.get());
+                }
+            }
+            instr.execute([&](NodeId n) -> void* { return tensors.at(n)->ptr; }, stream);
+            local.instrs++;
+            for (NodeId out : instr.outputs())
+                if (alive.count(out)) HE_HIP(hipEventRecord(tensors.at(out)->ready, stream));
+        }
+        // every stream of the next steps is ordered after this step's streams, so one wait per tensor is enough
+        synced.insert(waited.begin(), waited.end());
+        prev_events.clear();
+        for (size_t w = 0; w < width; w++) {
+            hipEvent_t e;
+            HE_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+            HE_HIP(hipEventRecord(e, st.s[w]));
+            prev_events.push_back(e);
+            all_events.push_back(e);
+        }
+    }
+    // Drop of the executor (cuda.rs:232-260): when everything queued above has run, the scope's freed blocks
+    // become available to everyone.
+    for (hipEvent_t e : prev_events) HE_HIP(hipStreamWaitEvent(st.s[0], e, 0));
+    struct Done {
+        uint64_t scope;
+        std::vector<hipEvent_t> events;
+    };
+    Done* done = new Done{scope, all_events};
+    HE_HIP(hipLaunchHostFunc(st.s[0], [](void* p) {
+        Done* d = static_cast<Done*>(p);
+        DevicePool::global().end_scope(d->scope);
+        delete d;  // events are destroyed by the next executor of this thread (not from a callback thread)
+    }, done));
+    {
+        static thread_local std::vector<hipEvent_t> garbage;
+        for (hipEvent_t e : garbage) (void)hipEventDestroy(e);  // recorded long ago; destruction is deferred by HIP
+        garbage = all_events;
+    }
+    local.streams_used = (int)used_streams.size();
+    if (stats) *stats = local;
+
+    std::map<NodeId, TensorRef> result;
+    for (NodeId out : graph->outputs()) {
+        NodeId from = graph->inbound(out)[0];
+        auto it = tensors.find(from);
+        HE_REQUIRE(it != tensors.end(), HE_ERR_INTERNAL, "output node %u has no storage", out);
+        result[out] = it->second;
+    }
+    return result;
+}
+
+}  // namespace he::exec

@@ -1,0 +1,71 @@
+// Graph executor for the HIP backend: tensor storage, pooled device memory with execution scopes, and the step
+// loop of helium/src/backend.rs:40-80 driven over a pool of HIP streams (helium/src/cuda.rs:98-260).
+#pragma once
+#include <map>
+#include <memory>
+#include <mutex>
+#include <vector>
+
+#include "plan.h"
+
+namespace he::exec {
+
+using ir::NodeId;
+
+// Pooling device allocator (helium/src/cuda/allocator/device.rs): memory is never returned to the driver; a block
+// freed inside an execution scope is reusable by that scope at once and by everyone else when the scope has ended
+// on the device (device.rs:60-89, block.rs:216-244).
+class DevicePool {
+public:
+    static DevicePool& global();
+    uint64_t begin_scope();
+    void end_scope(uint64_t scope);  // called once the scope's device work has finished
+    void* allocate(size_t bytes, uint64_t scope);
+    // `owner`: the scope the block was allocated in (0: none); `used`: every scope whose device work touches it.
+    // The block goes to the owner's free list while only the owner can still touch it, to the global list when no
+    // live scope can, and otherwise waits until the last such scope has ended on the device.
+    void release(void* ptr, size_t bytes, uint64_t owner, const std::vector<uint64_t>& used);
+    void note_use(struct Tensor& t, uint64_t scope);
+    void stats(uint64_t* driver_bytes, uint64_t* driver_allocs, uint64_t* reuses);
+
+private:
+    static size_t size_class(size_t bytes);
+    std::mutex mu_;
+    std::multimap<size_t, void*> free_global_;
+    std::map<uint64_t, std::multimap<size_t, void*>> free_scoped_;  // one entry per live scope
+    struct Deferred {
+        void* ptr;
+        size_t cls;
+        std::vector<uint64_t> waiting;
+    };
+    std::vector<Deferred> deferred_;
+    uint64_t next_scope_ = 1, driver_bytes_ = 0, driver_allocs_ = 0, reuses_ = 0;
+};
+
+// TensorStorage (helium/src/cuda/tensor_storage.rs:31-42): device buffer + ready event; shared by reference count.
+struct Tensor {
+    void* ptr = nullptr;
+    size_t bytes = 0, len = 0;
+    int dtype = HE_F32;
+    uint64_t scope = 0;
+    std::vector<uint64_t> used;  // execution scopes that read or wrote the tensor (guarded by the pool's mutex)
+    bool uploaded = false;       // filled by an asynchronous host-to-device copy
+    hipEvent_t ready = nullptr;
+    ~Tensor();
+};
+using TensorRef = std::shared_ptr<Tensor>;
+
+TensorRef allocate_tensor(int dtype, size_t len, uint64_t scope);            // TensorStorage::new (:45-73)
+TensorRef create_tensor_with_data(const void* data, int dtype, size_t len);  // Backend::create_tensor_with_data (cuda.rs:62-79)
+void download_tensor(const TensorRef& t, void* dst);                         // Backend::download_tensor (cuda.rs:81-96), blocking
+
+struct ExecStats {
+    int steps = 0, instrs = 0, streams_used = 0, event_waits = 0;
+};
+
+// BackendExt::execute_graph (backend.rs:40-80). `inputs`: storage for every Input node. Returns the storage of
+// every node that feeds an Output node, keyed by the Output node's id.
+std::map<NodeId, TensorRef> execute_graph(const ir::OpGraph& graph, const std::map<NodeId, TensorRef>& inputs,
+                                          ExecStats* stats = nullptr);
+
+}  // namespace he::exec

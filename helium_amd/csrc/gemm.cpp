@@ -43,7 +43,13 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
 // Helpers that depend on the problem constants.
 const char* kGemmHelpers = R"HIP(
-__device__ __forceinline__ u32x4 pack8(const float (&v)[8]) {
+#if MMA_F32
+__device__ __forceinline__ u32x4 pack_chunk(const float (&v)[4]) {
+    return u32x4{__builtin_bit_cast(u32, v[0]), __builtin_bit_cast(u32, v[1]), __builtin_bit_cast(u32, v[2]),
+                 __builtin_bit_cast(u32, v[3])};
+}
+#else
+__device__ __forceinline__ u32x4 pack_chunk(const float (&v)[8]) {
 #if MMA_BF16
     bf16x8 r;
 #pragma unroll
@@ -55,6 +61,7 @@ __device__ __forceinline__ u32x4 pack8(const float (&v)[8]) {
 #endif
     return __builtin_bit_cast(u32x4, r);
 }
+#endif
 )HIP";
 
 // Kernel body; problem and tile constants are #defines in front of it.
@@ -65,11 +72,13 @@ const char* kGemmBody = R"HIP(
 #define WTN (BN / WAVES_N)
 #define MB (WTM / 32)             /* 32x32 MFMA blocks per wave tile */
 #define NB (WTN / 32)
-#define KK (BK / 16)              /* MFMA k-steps per tile */
-#define A_CHUNKS (BK / 8)         /* 16-byte chunks per A row */
-#define B_CHUNKS (BN / 8)
-#define A_TILE_BYTES (BM * BK * 2)
-#define B_TILE_BYTES (BK * BN * 2)
+#define ESZ (MMA_F32 ? 4 : 2)     /* bytes per multiplicand */
+#define EPC (16 / ESZ)            /* multiplicands per 16-byte chunk */
+#define KK (BK / (2 * EPC))       /* k-steps per tile: one 16-byte chunk per lane half */
+#define A_CHUNKS (BK / EPC)       /* 16-byte chunks per A row */
+#define B_CHUNKS (BN / EPC)
+#define A_TILE_BYTES (BM * BK * ESZ)
+#define B_TILE_BYTES (BK * BN * ESZ)
 #define STAGE_BYTES (A_TILE_BYTES + B_TILE_BYTES)
 #define A_PER_THREAD (BM * A_CHUNKS / NTHREADS)
 #define B_PER_THREAD (BK * B_CHUNKS / NTHREADS)
@@ -79,10 +88,11 @@ const char* kGemmBody = R"HIP(
 #endif
 #define KT ((GK + BK - 1) / BK)
 
-__device__ __forceinline__ u32 a_off(u32 m, u32 kc) { return m * (BK * 2) + ((kc ^ ((m >> A_SWZ_SHIFT) & (A_CHUNKS - 1))) << 4); }
-__device__ __forceinline__ u32 b_off(u32 k, u32 n) {
-    return k * (BN * 2) + ((((n >> 3) ^ ((k & 3) << 2))) << 4) + ((n & 7) << 1);
-}
+__device__ __forceinline__ u32 a_off(u32 m, u32 kc) { return m * (BK * ESZ) + ((kc ^ ((m >> A_SWZ_SHIFT) & (A_CHUNKS - 1))) << 4); }
+// B rows keep their memory order; the chunk index is XORed with 4 * (k % 4) for the transposing 16-bit reads
+// (f32 operands are read one word per lane along n and need no swizzle).
+__device__ __forceinline__ u32 b_chunk_off(u32 k, u32 nc) { return k * (BN * ESZ) + ((nc ^ (MMA_F32 ? 0u : ((k & 3) << 2))) << 4); }
+__device__ __forceinline__ u32 b_off(u32 k, u32 n) { return b_chunk_off(k, (n * ESZ) >> 4) + ((n * ESZ) & 15); }
 
 #ifndef KERNEL_ATTRS
 /* NWAVES / 4 waves per SIMD: with four waves each one owns the full 512-register budget */
@@ -117,13 +127,13 @@ void fused_matmul(KERNEL_PARAMS) {
         for (int i = 0; i < A_PER_THREAD; i++) {
             const u32 idx = tid + i * NTHREADS;
             const u32 row = idx / A_CHUNKS, kc = idx % A_CHUNKS;
-            sa[i] = fetch_a(FETCH_A_ARGS bz, m0 + row, k0 + kc * 8);
+            sa[i] = fetch_a(FETCH_A_ARGS bz, m0 + row, k0 + kc * EPC);
         }
 #pragma unroll
         for (int i = 0; i < B_PER_THREAD; i++) {
             const u32 idx = tid + i * NTHREADS;
             const u32 krow = idx / B_CHUNKS, nc = idx % B_CHUNKS;
-            sb[i] = fetch_b(FETCH_B_ARGS bz, k0 + krow, n0 + nc * 8);
+            sb[i] = fetch_b(FETCH_B_ARGS bz, k0 + krow, n0 + nc * EPC);
         }
     };
     auto stage_store = [&](u32 buf) {
@@ -137,10 +147,43 @@ void fused_matmul(KERNEL_PARAMS) {
 #pragma unroll
         for (int i = 0; i < B_PER_THREAD; i++) {
             const u32 idx = tid + i * NTHREADS;
-            *(u32x4*)(lb + b_off(idx / B_CHUNKS, (idx % B_CHUNKS) * 8)) = sb[i];
+            *(u32x4*)(lb + b_chunk_off(idx / B_CHUNKS, idx % B_CHUNKS)) = sb[i];
         }
     };
     const u32 grp = lane >> 4, sub = lane & 15;
+    (void)grp; (void)sub;
+#if MMA_F32
+    // v_mfma_f32_32x32x2_f32: lane l supplies A[l % 32][l / 32] and B[l / 32][l % 32]. One k-step covers 8 k: each
+    // lane half owns 4 consecutive k (one 16-byte chunk of its A row) and issues 4 MFMAs per output block.
+    typedef f32x4 afrag_t;
+    typedef f32x4 bfrag_t;
+    auto load_frags = [&](u32 buf, int kk, afrag_t (&af)[MB], bfrag_t (&bf)[NB]) {
+        const unsigned char* la = lds + buf * STAGE_BYTES;
+        const unsigned char* lb = la + A_TILE_BYTES;
+#pragma unroll
+        for (int i = 0; i < MB; i++) {
+            const u32 row = wave_m * WTM + i * 32 + (lane & 31);
+            af[i] = *(const f32x4*)(la + a_off(row, kk * 2 + (lane >> 5)));
+        }
+#pragma unroll
+        for (int j = 0; j < NB; j++) {
+            const u32 n = wave_n * WTN + j * 32 + (lane & 31);
+#pragma unroll
+            for (int e = 0; e < 4; e++) bf[j][e] = *(const float*)(lb + b_off(kk * 8 + (lane >> 5) * 4 + e, n));
+        }
+    };
+    auto mma = [&](const afrag_t (&af)[MB], const bfrag_t (&bf)[NB]) {
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+#pragma unroll
+            for (int i = 0; i < MB; i++)
+#pragma unroll
+                for (int j = 0; j < NB; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][e], bf[j][e], acc[i][j], 0, 0, 0);
+    };
+#else
+    typedef s16x8 afrag_t;
+    typedef s16x8 bfrag_t;
     auto load_frags = [&](u32 buf, int kk, s16x8 (&af)[MB], s16x8 (&bf)[NB]) {
         const unsigned char* la = lds + buf * STAGE_BYTES;
         const unsigned char* lb = la + A_TILE_BYTES;
@@ -172,9 +215,11 @@ void fused_matmul(KERNEL_PARAMS) {
 #endif
             }
     };
+#endif
     // One k-tile: operands for step kk+1 are fetched from LDS while the MFMAs of step kk run.
     auto compute = [&](u32 buf, auto&& per_step) {
-        s16x8 af[2][MB], bf[2][NB];
+        afrag_t af[2][MB];
+        bfrag_t bf[2][NB];
         load_frags(buf, 0, af[0], bf[0]);
 #pragma unroll
         for (int kk = 0; kk < KK; kk++) {
@@ -355,12 +400,15 @@ GemmProblem gemm_problem_from_fusion(const fir::OpGraph& g) {
     pr.op_a = tp::lower_operand(g, mm.a, &pr.root_a);
     pr.op_b = tp::lower_operand(g, mm.b, &pr.root_b);
     pr.epi = tp::lower_epilogue(g, anchor);
-    // Multiplicand type: f16 when every operand source is f16, bf16 otherwise (f32 sources are rounded to bf16,
-    // the reference's MulBf16AccumF32).
-    bool all_f16 = true;
+    // Multiplicand type (the fusion IR carries no Precision): f16 when every operand source is f16, f32 when every
+    // one is f32, bf16 otherwise (mixed sources are rounded to bf16, the reference's MulBf16AccumF32).
+    bool all_f16 = true, all_f32 = true;
     for (auto* p : {&pr.op_a, &pr.op_b})
-        for (auto& a : p->args) all_f16 = all_f16 && a.dtype == HE_F16;
-    pr.mma_dtype = all_f16 ? HE_F16 : HE_BF16;
+        for (auto& a : p->args) {
+            all_f16 = all_f16 && a.dtype == HE_F16;
+            all_f32 = all_f32 && a.dtype == HE_F32;
+        }
+    pr.mma_dtype = all_f16 ? HE_F16 : all_f32 ? HE_F32 : HE_BF16;
 
     // Kernel arguments: every distinct producer in id order, then every output in leaf order.
     std::vector<tp::Arg> inputs, outputs;
@@ -400,34 +448,37 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     HE_REQUIRE(pr.M < (1ll << 31) && pr.N < (1ll << 31) && pr.K < (1ll << 31) &&
                    pr.batch * pr.M * std::max(pr.N, pr.K) < (1ll << 40),
                HE_ERR_INVALID, "GEMM too large");
-    HE_REQUIRE(pr.mma_dtype == HE_BF16 || pr.mma_dtype == HE_F16, HE_ERR_UNSUPPORTED, "unsupported multiplicand type");
+    HE_REQUIRE(pr.mma_dtype == HE_BF16 || pr.mma_dtype == HE_F16 || pr.mma_dtype == HE_F32, HE_ERR_UNSUPPORTED,
+               "unsupported multiplicand type");
+    const bool f32 = pr.mma_dtype == HE_F32;
+    const int epc = f32 ? 4 : 8;  // multiplicands per 16-byte chunk
     Tile t;
-    const bool raw_a0 = is_raw_copy(pr.op_a, pr.root_a, pr.mma_dtype) && pr.K % 8 == 0;
-    const bool raw_b0 = is_raw_copy(pr.op_b, pr.root_b, pr.mma_dtype) && pr.N % 8 == 0;
-    bool want_direct = raw_a0 && raw_b0 && !getenv("HELIUM_HIP_GEMM_NO_DIRECT");
+    const bool raw_a0 = is_raw_copy(pr.op_a, pr.root_a, pr.mma_dtype) && pr.K % epc == 0;
+    const bool raw_b0 = is_raw_copy(pr.op_b, pr.root_b, pr.mma_dtype) && pr.N % epc == 0;
+    bool want_direct = raw_a0 && raw_b0 && !f32 && !getenv("HELIUM_HIP_GEMM_NO_DIRECT");
     if (const char* env = getenv("HELIUM_HIP_GEMM_TILE")) {
         int v[6] = {256, 256, 64, 2, 4, 2};
         int n = sscanf(env, "%d,%d,%d,%d,%d,%d", &v[0], &v[1], &v[2], &v[3], &v[4], &v[5]);
         HE_REQUIRE(n >= 5, HE_ERR_INVALID, "HELIUM_HIP_GEMM_TILE wants bm,bn,bk,wm,wn[,stages]");
         t = {v[0], v[1], v[2], v[3], v[4], v[5]};
     } else {
+        if (f32) t.bk = 32;  // same bytes per tile row as 64 two-byte multiplicands
         // Smaller problems take smaller tiles so that every CU gets work.
         if (pr.M <= 128 || pr.N <= 128 || ((pr.M + 255) / 256) * ((pr.N + 255) / 256) * pr.batch < 128) {
             t.bm = t.bn = 128;
             t.wm = t.wn = 2;
         }
     }
-    HE_REQUIRE(t.bm % (t.wm * 32) == 0 && t.bn % (t.wn * 32) == 0 && (t.bk == 64 || t.bk == 32), HE_ERR_INVALID, "bad GEMM tile");
+    HE_REQUIRE(t.bm % (t.wm * 32) == 0 && t.bn % (t.wn * 32) == 0 && (t.bk == 64 || t.bk == 32) && (!f32 || t.bk == 32), HE_ERR_INVALID, "bad GEMM tile");
     const int threads = t.wm * t.wn * 64;
     HE_REQUIRE(threads == 256 || threads == 512, HE_ERR_INVALID, "GEMM workgroups have 4 or 8 waves");
-    HE_REQUIRE((t.bm * t.bk / 8) % threads == 0 && (t.bk * t.bn / 8) % threads == 0, HE_ERR_INVALID, "bad GEMM tile");
-    HE_REQUIRE(t.stages >= 2 && t.stages <= 4 && t.stages * (t.bm + t.bn) * t.bk * 2 <= 160 * 1024, HE_ERR_INVALID,
+    HE_REQUIRE((t.bm * t.bk / epc) % threads == 0 && (t.bk * t.bn / epc) % threads == 0, HE_ERR_INVALID, "bad GEMM tile");
+    HE_REQUIRE(t.stages >= 2 && t.stages <= 4 && t.stages * (t.bm + t.bn) * t.bk * (16 / epc) <= 160 * 1024, HE_ERR_INVALID,
                "GEMM tile exceeds LDS");
     const int wtn = t.bn / t.wn;
 
-    const bool raw_a = is_raw_copy(pr.op_a, pr.root_a, pr.mma_dtype) && pr.K % 8 == 0;
-    const bool raw_b = is_raw_copy(pr.op_b, pr.root_b, pr.mma_dtype) && pr.N % 8 == 0;
-    const int nva = tp::pick_nv(pr.op_a, 16), nvb = tp::pick_nv(pr.op_b, 16);
+    const bool raw_a = raw_a0, raw_b = raw_b0;
+    const int nva = std::min(epc, tp::pick_nv(pr.op_a, 16)), nvb = std::min(epc, tp::pick_nv(pr.op_b, 16));
     // Direct global->LDS loads need unpredicated, unmodified 16-byte chunks: raw operands and full tiles everywhere.
     const bool direct = want_direct && raw_a && raw_b && pr.M % t.bm == 0 && pr.N % t.bn == 0 && pr.K % t.bk == 0 &&
                         (t.bm * t.bk * 2 / 1024) % (threads / 64) == 0 && (t.bk * t.bn * 2 / 1024) % (threads / 64) == 0 &&
@@ -446,7 +497,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     s << tp::emit_prelude(pr.epi) << kGemmPrelude;
     s << "#define GM " << pr.M << "u\n#define GN " << pr.N << "u\n#define GK " << pr.K << "u\n";
     s << "#define BM " << t.bm << "\n#define BN " << t.bn << "\n#define BK " << t.bk << "\n#define WAVES_M " << t.wm
-      << "\n#define WAVES_N " << t.wn << "\n#define NSTAGES " << t.stages << "\n#define NVE " << nve << "\n#define MMA_BF16 " << (pr.mma_dtype == HE_BF16 ? 1 : 0)
+      << "\n#define WAVES_N " << t.wn << "\n#define NSTAGES " << t.stages << "\n#define NVE " << nve << "\n#define MMA_BF16 " << (pr.mma_dtype == HE_BF16 ? 1 : 0) << "\n#define MMA_F32 " << (f32 ? 1 : 0)
       << "\n#define STAGGER_EXPR " << (getenv("HELIUM_HIP_GEMM_STAGGER") ? getenv("HELIUM_HIP_GEMM_STAGGER") : "0u")
       << "\n#define GEMM_SKIP " << (getenv("HELIUM_HIP_GEMM_SKIP") ? atoi(getenv("HELIUM_HIP_GEMM_SKIP")) : 0)
       << "\n#define GEMM_TIMING " << (getenv("HELIUM_HIP_GEMM_TIMING") ? 1 : 0) << "\n#define GEMM_TIMING_PTR p" << (pr.args.size() - 1)
@@ -482,10 +533,10 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
             s << "u32x4 v = {0u, 0u, 0u, 0u};\nif (row < " << rows << " && col < " << cols << ") v = *(const u32x4*)(q0 + ((size_t)b * "
               << rows << " + row) * " << cols << " + col);\nreturn v;\n}\n";
         } else {
-            s << "float v[8];\n#pragma unroll\nfor (int j = 0; j < 8; j += " << nv << ") {\nif (row < " << rows << " && col + j < " << cols
+            s << "float v[" << epc << "];\n#pragma unroll\nfor (int j = 0; j < " << epc << "; j += " << nv << ") {\nif (row < " << rows << " && col + j < " << cols
               << ") operand_" << W << "(";
             for (size_t a = 0; a < p.args.size(); a++) s << "q" << a << ", ";
-            s << "b, row, col + j, v + j);\nelse {\n#pragma unroll\nfor (int k = 0; k < " << nv << "; k++) v[j + k] = 0.0f; }\n}\nreturn pack8(v);\n}\n";
+            s << "b, row, col + j, v + j);\nelse {\n#pragma unroll\nfor (int k = 0; k < " << nv << "; k++) v[j + k] = 0.0f; }\n}\nreturn pack_chunk(v);\n}\n";
         }
     };
     emit_fetch("a", pr.op_a, pr.root_a, pr.map_a, raw_a, nva, "GM", "GK", pr.M % t.bm == 0 && pr.K % t.bk == 0);
@@ -584,8 +635,8 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         splice("SCHED_HINT", h.str());
         std::ostringstream plan;
         const int mode = getenv("HELIUM_HIP_GEMM_PLAN") ? atoi(getenv("HELIUM_HIP_GEMM_PLAN")) : 2;
-        const int mb = t.bm / t.wm / 32, nb = t.bn / t.wn / 32, kk_steps = t.bk / 16;
-        const int nr = mb + 2 * nb, nm = mb * nb;
+        const int mb = t.bm / t.wm / 32, nb = t.bn / t.wn / 32, kk_steps = t.bk / (2 * epc);
+        const int nr = f32 ? mb + 4 * nb : mb + 2 * nb, nm = f32 ? 4 * mb * nb : mb * nb;
         if (mode == 1) {
             // all operand reads of step kk+1 are issued ahead of the MFMAs of step kk
             plan << "__builtin_amdgcn_sched_group_barrier(0x100, " << nr << ", 0);\n";

@@ -284,6 +284,9 @@ std::string OpSubgraph::cache_key() const {
         for (int64_t d : node.desc.shape) s << d << ',';
         s << "];";
     }
+    // which values leave the kernel depends on the consumers outside the node set
+    s << "|L";
+    for (NodeId n : leafs_) s << n << ',';
     return s.str();
 }
 

@@ -1,0 +1,492 @@
+#include "plan.h"
+
+#include <future>
+#include <list>
+#include <map>
+#include <set>
+#include <sstream>
+#include <unordered_map>
+
+namespace he::plan {
+
+// ---------------------------------------------------------------------------------------------------------
+// Instructions
+// ---------------------------------------------------------------------------------------------------------
+bool enumerate_swaps(const ir::OpSubgraph& sg, std::vector<std::pair<int, int>>* swaps) {
+    swaps->clear();
+    if (sg.inputs().size() != 1) return false;
+    const ir::OpGraph& g = *sg.graph();
+    // entry_node (permute_dims.rs:144-153): the member that consumes the single input
+    NodeId current = ir::kNoNode;
+    for (NodeId c : g.outbound(sg.inputs()[0]))
+        if (sg.contains(c)) {
+            current = c;
+            break;
+        }
+    if (current == ir::kNoNode) return false;
+    std::vector<NodeId> visited{current};
+    for (;;) {
+        const ir::Node& n = g.get(current);
+        if (n.kind != ir::Node::Intermediate || n.op.kind != ir::OpKind::SwapDims) return false;
+        swaps->emplace_back((int)n.op.axis_a, (int)n.op.axis_b);
+        const auto& next = g.outbound(current);
+        if (next.size() == 1 && sg.contains(next[0])) {
+            current = next[0];
+            visited.push_back(current);
+        } else {
+            break;
+        }
+    }
+    for (NodeId n : sg.nodes())
+        if (std::find(visited.begin(), visited.end(), n) == visited.end()) return false;
+    return true;
+}
+
+bool Instr::can_fuse_with(const Instr& next) const {
+    if (kind_ != next.kind_) return false;  // only instructions of one kind fuse (instr.rs:71-84)
+    switch (kind_) {
+        case InstrKind::Gemm: return false;  // the reference's matmul instruction never fuses (cudnn_graph.rs:319-321)
+        case InstrKind::Pointwise: return tp::pointwise_supports(sg_.merge_with(next.sg_));
+        case InstrKind::Permute: {
+            std::vector<std::pair<int, int>> swaps;
+            return enumerate_swaps(sg_.merge_with(next.sg_), &swaps);
+        }
+    }
+    return false;
+}
+
+Instr Instr::fuse_with(const Instr& next) const { return Instr(kind_, sg_.merge_with(next.sg_)); }
+
+Instr make_instr_for_op(const std::shared_ptr<const ir::OpGraph>& g, NodeId node) {
+    const ir::Node& n = g->get(node);
+    HE_REQUIRE(n.kind == ir::Node::Intermediate, HE_ERR_INVALID, "node %u is not an op", node);
+    ir::OpSubgraph sg(g, {node});
+    switch (n.op.kind) {
+        case ir::OpKind::SwapDims:
+            // Heuristic of the reference: the tiled permute kernel for large tensors, the pointwise kernel (which
+            // can fuse) for small ones.
+            if (ir::num_elements(n.desc.shape) > kPermuteThreshold) return Instr(InstrKind::Permute, sg);
+            return Instr(InstrKind::Pointwise, sg);
+        case ir::OpKind::Constant:
+        case ir::OpKind::UnaryPointwise:
+        case ir::OpKind::BinaryPointwise:
+        case ir::OpKind::ChangeDataType:
+        case ir::OpKind::Reduce:
+        case ir::OpKind::Broadcast:
+        case ir::OpKind::Reshape:
+        case ir::OpKind::Compare:
+        case ir::OpKind::Select: return Instr(InstrKind::Pointwise, sg);
+        case ir::OpKind::Matmul: return Instr(InstrKind::Gemm, sg);
+        default: fail(HE_ERR_UNSUPPORTED, "convolution ops have no instruction in this backend");
+    }
+}
+
+namespace {
+template <class V>
+class KernelCache {
+public:
+    explicit KernelCache(size_t cap) : cap_(cap) {}
+    template <class F>
+    std::shared_ptr<V> get_or_insert(const std::string& key, F&& make) {
+        {
+            std::lock_guard<std::mutex> lk(mu_);
+            auto it = map_.find(key);
+            if (it != map_.end()) return it->second;
+        }
+        // built outside the lock: a redundant build by a racing thread is an accepted cost (cache.rs:40-49)
+        std::shared_ptr<V> v = make();
+        std::lock_guard<std::mutex> lk(mu_);
+        if (map_.size() >= cap_) map_.erase(map_.begin());
+        return map_.emplace(key, v).first->second;
+    }
+
+private:
+    size_t cap_;
+    std::mutex mu_;
+    std::unordered_map<std::string, std::shared_ptr<V>> map_;
+};
+KernelCache<KernelBase> g_tile_kernels(1024);  // pointwise.rs:45, permute_dims.rs:61 use 1024 entries
+KernelCache<Permute> g_permutes(1024);
+}  // namespace
+
+void Instr::precompile() const {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (kernel_ || permute_) return;
+    switch (kind_) {
+        case InstrKind::Pointwise:
+            kernel_ = g_tile_kernels.get_or_insert("pw:" + sg_.cache_key(), [&] {
+                return std::shared_ptr<KernelBase>(new TileKernel(tp::lower_pointwise(sg_), "pointwise_kernel"));
+            });
+            break;
+        case InstrKind::Gemm:
+            kernel_ = g_tile_kernels.get_or_insert("mm:" + sg_.cache_key(), [&] {
+                return std::shared_ptr<KernelBase>(new GemmKernel(gemm_problem_from_ir(sg_)));
+            });
+            break;
+        case InstrKind::Permute: {
+            std::vector<std::pair<int, int>> swaps;
+            HE_REQUIRE(enumerate_swaps(sg_, &swaps), HE_ERR_INTERNAL, "permute instruction is not a chain of swaps");
+            const ir::Descriptor& d = sg_.graph()->get(sg_.inputs()[0]).desc;
+            std::vector<int> perm = perm_from_swaps((int)d.shape.size(), swaps);
+            std::ostringstream key;
+            key << d.dtype << ':';
+            for (int64_t e : d.shape) key << e << ',';
+            key << ':';
+            for (int p : perm) key << p << ',';
+            permute_ = g_permutes.get_or_insert(key.str(), [&] { return std::make_shared<Permute>(d.shape, perm, d.dtype); });
+            break;
+        }
+    }
+}
+
+void Instr::execute(const std::function<void*(NodeId)>& storage, hipStream_t stream) const {
+    precompile();
+    if (kind_ == InstrKind::Permute) {
+        permute_->execute(storage(sg_.inputs()[0]), storage(sg_.leafs()[0]), stream);
+        return;
+    }
+    const auto& args = kernel_->args();
+    std::vector<void*> ptrs(args.size());
+    for (size_t i = 0; i < args.size(); i++) ptrs[i] = storage((NodeId)args[i].node);
+    kernel_->execute(ptrs.data(), stream);
+}
+
+std::string Instr::describe() const {
+    std::ostringstream s;
+    s << (kind_ == InstrKind::Gemm ? "gemm" : kind_ == InstrKind::Pointwise ? "pointwise" : "permute") << "{";
+    for (size_t i = 0; i < sg_.nodes().size(); i++) s << (i ? "," : "") << sg_.nodes()[i];
+    s << "}";
+    return s.str();
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Instruction graph (plan_generation.rs:87-236)
+// ---------------------------------------------------------------------------------------------------------
+namespace {
+struct InstrGraph {
+    std::map<uint64_t, std::shared_ptr<Instr>> instrs;
+    uint64_t next_id = 0;
+    std::map<NodeId, uint64_t> producers;
+    std::map<NodeId, std::set<uint64_t>> consumers;
+    std::map<uint64_t, std::set<uint64_t>> dependencies, dependents;
+
+    // Ids order the greedy fusion and the steps. The reference keeps instructions in a slotmap (slotmap 1.0.7),
+    // whose keys compare by slot index first and whose free list is last-in-first-out: the instruction made by
+    // fusing a into b therefore takes b's slot, and `slot` lets fuse() say so.
+    uint64_t insert(std::shared_ptr<Instr> instr, int64_t slot = -1) {
+        const uint64_t id = slot >= 0 ? (uint64_t)slot : next_id++;
+        const auto inputs = instr->inputs(), outputs = instr->outputs();
+        instrs[id] = std::move(instr);
+        for (NodeId in : inputs) {
+            consumers[in].insert(id);
+            auto p = producers.find(in);
+            if (p != producers.end()) dependents[p->second].insert(id);
+        }
+        for (NodeId out : outputs) {
+            HE_REQUIRE(!producers.count(out), HE_ERR_INTERNAL, "node %u has two producers", out);
+            producers[out] = id;
+            for (uint64_t c : consumers[out]) dependencies[c].insert(id);
+        }
+        std::set<uint64_t>& dts = dependents[id];
+        for (NodeId out : outputs)
+            for (uint64_t c : consumers[out]) dts.insert(c);
+        std::set<uint64_t>& dps = dependencies[id];
+        for (NodeId in : inputs) {
+            auto p = producers.find(in);
+            if (p != producers.end()) dps.insert(p->second);
+        }
+        return id;
+    }
+
+    std::shared_ptr<Instr> remove(uint64_t id) {
+        std::shared_ptr<Instr> instr = instrs.at(id);
+        instrs.erase(id);
+        for (NodeId in : instr->inputs()) {
+            consumers[in].erase(id);
+            auto p = producers.find(in);
+            if (p != producers.end()) dependents[p->second].erase(id);
+        }
+        for (NodeId out : instr->outputs()) {
+            producers.erase(out);
+            for (uint64_t c : consumers[out]) dependencies[c].erase(id);
+        }
+        dependencies.erase(id);
+        dependents.erase(id);
+        return instr;
+    }
+
+    // Is there a path a -> ... -> b besides the direct edge? Fusing across one would create a cycle.
+    bool exist_multiple_paths(uint64_t a, uint64_t b) const {
+        std::vector<uint64_t> stack;
+        std::set<uint64_t> visited;
+        for (uint64_t d : dependents.at(a))
+            if (d != b) {
+                stack.push_back(d);
+                visited.insert(d);
+            }
+        while (!stack.empty()) {
+            uint64_t cur = stack.back();
+            stack.pop_back();
+            if (cur == b) return true;
+            for (uint64_t n : dependents.at(cur))
+                if (visited.insert(n).second) stack.push_back(n);
+        }
+        return false;
+    }
+
+    bool can_fuse(uint64_t a, uint64_t b) const {
+        return instrs.at(a)->can_fuse_with(*instrs.at(b)) && !exist_multiple_paths(a, b);
+    }
+
+    uint64_t fuse(uint64_t a, uint64_t b) {
+        std::shared_ptr<Instr> ia = remove(a), ib = remove(b);
+        return insert(std::make_shared<Instr>(ia->fuse_with(*ib)), (int64_t)b);
+    }
+};
+
+bool intersects(const std::vector<NodeId>& a, const std::vector<NodeId>& b) {
+    for (NodeId x : a)
+        for (NodeId y : b)
+            if (x == y) return true;
+    return false;
+}
+}  // namespace
+
+std::shared_ptr<const Plan> generate_plan(const std::shared_ptr<const ir::OpGraph>& g) {
+    // make_instr_graph (:259-270): one instruction per intermediate node, in node order
+    InstrGraph ig;
+    for (NodeId n : g->nodes())
+        if (g->get(n).kind == ir::Node::Intermediate) ig.insert(std::make_shared<Instr>(make_instr_for_op(g, n)));
+
+    // do_fusions (:243-256)
+    {
+        std::set<uint64_t> work;
+        for (auto& kv : ig.instrs) work.insert(kv.first);
+        while (!work.empty()) {
+            const uint64_t cur = *work.begin();
+            work.erase(work.begin());
+            std::vector<uint64_t> nexts(ig.dependents.at(cur).begin(), ig.dependents.at(cur).end());
+            for (uint64_t nxt : nexts)
+                if (ig.can_fuse(cur, nxt)) {
+                    uint64_t merged = ig.fuse(cur, nxt);
+                    work.erase(nxt);
+                    work.insert(merged);
+                    break;
+                }
+        }
+    }
+
+    // generate_plan_from_graph (:275-321): Kahn levels
+    auto plan = std::make_shared<Plan>();
+    {
+        const size_t total = ig.instrs.size();
+        std::map<uint64_t, size_t> indeg;
+        std::vector<uint64_t> stack;
+        for (auto& kv : ig.instrs) {
+            indeg[kv.first] = ig.dependencies.at(kv.first).size();
+            if (indeg[kv.first] == 0) stack.push_back(kv.first);
+        }
+        size_t placed = 0;
+        while (!stack.empty()) {
+            std::vector<uint64_t> step;
+            step.swap(stack);
+            for (uint64_t id : step)
+                for (uint64_t nxt : ig.dependents.at(id)) {
+                    HE_REQUIRE(indeg[nxt] > 0, HE_ERR_INTERNAL, "indegree underflow");
+                    if (--indeg[nxt] == 0) stack.push_back(nxt);
+                }
+            Step s;
+            for (uint64_t id : step) s.instrs.push_back(ig.instrs.at(id));
+            placed += s.instrs.size();
+            plan->steps.push_back(std::move(s));
+        }
+        HE_REQUIRE(placed == total, HE_ERR_INTERNAL, "cycle detected in instruction graph?");
+    }
+
+    // delay_computations (:325-353): push every instruction to the step before its first reader
+    for (int i = (int)plan->steps.size() - 1; i >= 0; i--) {
+        std::vector<std::shared_ptr<Instr>> kept;
+        std::vector<std::shared_ptr<Instr>> here;
+        here.swap(plan->steps[i].instrs);
+        for (auto& instr : here) {
+            const auto outs = instr->outputs();
+            int target = -1;
+            for (size_t j = i + 1; j < plan->steps.size(); j++) {
+                bool reads = false;
+                for (auto& other : plan->steps[j].instrs) reads = reads || intersects(other->inputs(), outs);
+                if (reads) {
+                    target = (int)j - 1;
+                    break;
+                }
+            }
+            if (target >= 0 && target != i) plan->steps[target].instrs.push_back(instr);
+            else kept.push_back(instr);
+        }
+        plan->steps[i].instrs = kept;
+    }
+
+    // analyze_tensor_lifetimes (:360-416)
+    {
+        std::vector<std::vector<NodeId>> releases;
+        releases.emplace_back();  // nothing is freed at the first step
+        for (size_t i = 0; i < plan->steps.size(); i++) {
+            std::vector<NodeId> used;
+            for (auto& instr : plan->steps[i].instrs)
+                for (NodeId in : instr->inputs()) used.push_back(in);
+            std::sort(used.begin(), used.end());
+            used.erase(std::unique(used.begin(), used.end()), used.end());
+            std::vector<NodeId> rel;
+            for (NodeId t : used) {
+                if (g->feeds_output(t)) continue;
+                bool later = false;
+                for (size_t j = i + 1; j < plan->steps.size() && !later; j++)
+                    for (auto& instr : plan->steps[j].instrs) {
+                        const auto ins = instr->inputs();
+                        if (std::find(ins.begin(), ins.end(), t) != ins.end()) {
+                            later = true;
+                            break;
+                        }
+                    }
+                if (!later) rel.push_back(t);
+            }
+            releases.push_back(std::move(rel));
+        }
+        plan->steps.emplace_back();  // a last, empty step that frees the final temporaries
+        for (size_t i = 0; i < plan->steps.size(); i++) plan->steps[i].tensors_to_release = releases[i];
+    }
+    return plan;
+}
+
+std::string Plan::describe() const {
+    std::ostringstream s;
+    for (size_t i = 0; i < steps.size(); i++) {
+        s << "step " << i << ":";
+        for (auto& instr : steps[i].instrs) s << " " << instr->describe();
+        s << " | release";
+        for (NodeId t : steps[i].tensors_to_release) s << " " << t;
+        s << "\n";
+    }
+    return s.str();
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Plan cache (plan_generation.rs:29-50)
+// ---------------------------------------------------------------------------------------------------------
+namespace {
+struct CacheEntry {
+    uint64_t hash;
+    std::shared_ptr<const ir::OpGraph> graph;
+    std::shared_ptr<const Plan> plan;
+};
+std::mutex g_plan_mu;
+std::list<CacheEntry> g_plans;  // most recently used first
+uint64_t g_plan_hits = 0, g_plan_misses = 0;
+constexpr size_t kPlanCacheCapacity = 256;
+}  // namespace
+
+std::shared_ptr<const Plan> generate_cached_plan(const std::shared_ptr<const ir::OpGraph>& g) {
+    const uint64_t h = g->structural_hash();
+    {
+        std::lock_guard<std::mutex> lk(g_plan_mu);
+        for (auto it = g_plans.begin(); it != g_plans.end(); ++it)
+            if (it->hash == h && it->graph->structurally_equal(*g)) {
+                g_plans.splice(g_plans.begin(), g_plans, it);
+                g_plan_hits++;
+                return g_plans.front().plan;
+            }
+        g_plan_misses++;
+    }
+    // The cached plan refers to the graph object it was generated from; node ids are equal by construction.
+    std::shared_ptr<const Plan> plan = generate_plan(g);
+    std::lock_guard<std::mutex> lk(g_plan_mu);
+    g_plans.push_front({h, g, plan});
+    if (g_plans.size() > kPlanCacheCapacity) g_plans.pop_back();
+    return plan;
+}
+
+void plan_cache_stats(uint64_t* hits, uint64_t* misses) {
+    std::lock_guard<std::mutex> lk(g_plan_mu);
+    *hits = g_plan_hits;
+    *misses = g_plan_misses;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// helium-ir Matmul -> GEMM problem
+// ---------------------------------------------------------------------------------------------------------
+GemmProblem gemm_problem_from_ir(const ir::OpSubgraph& sg) {
+    const ir::OpGraph& g = *sg.graph();
+    NodeId mm = ir::kNoNode;
+    for (NodeId n : sg.nodes())
+        if (g.get(n).op.kind == ir::OpKind::Matmul) {
+            HE_REQUIRE(mm == ir::kNoNode, HE_ERR_UNSUPPORTED, "a GEMM fusion holds one Matmul");
+            mm = n;
+        }
+    HE_REQUIRE(mm != ir::kNoNode, HE_ERR_UNSUPPORTED, "no Matmul in the subgraph");  // find_matmul (matmul.rs:222-233)
+    HE_REQUIRE(sg.nodes().size() == 1, HE_ERR_UNSUPPORTED,
+               "mainloop / epilogue fusion of helium-ir ops around a Matmul is expressed through the fusion IR");
+    const ir::Op& op = g.get(mm).op;
+    const ir::Descriptor &da = g.get(op.inputs[0]).desc, &db = g.get(op.inputs[1]).desc, &dc = g.get(mm).desc;
+    HE_REQUIRE(da.shape.size() >= 2 && da.shape.size() == db.shape.size(), HE_ERR_UNSUPPORTED, "matmul operand ranks differ");
+    const size_t r = da.shape.size();
+    int64_t batch = 1;
+    for (size_t i = 0; i + 2 < r; i++) {
+        HE_REQUIRE(da.shape[i] == db.shape[i], HE_ERR_UNSUPPORTED, "matmul batch extents differ");
+        batch *= da.shape[i];
+    }
+    HE_REQUIRE(da.shape[r - 1] == db.shape[r - 2], HE_ERR_INVALID, "matmul inner extents differ");
+    HE_REQUIRE(dtype_class(da.dtype) == DataClass::Float && dtype_class(db.dtype) == DataClass::Float, HE_ERR_UNSUPPORTED,
+               "matmul takes float operands");
+    GemmProblem pr;
+    pr.batch = batch;
+    pr.M = da.shape[r - 2];
+    pr.K = da.shape[r - 1];
+    pr.N = db.shape[r - 1];
+    // Multiplicand type by Precision (precision.rs:36-81): never less precise than asked for. TF32 and F8 have no
+    // matrix-core form here; TF32 runs as f32, F8 as bf16.
+    switch (op.precision) {
+        case ir::Precision::MulF32AccumF32:
+        case ir::Precision::MulTf32AccumF32: pr.mma_dtype = HE_F32; break;
+        case ir::Precision::MulF16AccumF32:
+        case ir::Precision::MulF16AccumF16: pr.mma_dtype = HE_F16; break;
+        default: pr.mma_dtype = HE_BF16; break;
+    }
+    auto operand = [&](tp::Program& p, const ir::Descriptor& d, NodeId node, int64_t rows, int64_t cols) {
+        p.dims = {batch, rows, cols};
+        p.args.push_back({d.dtype, ir::num_elements(d.shape), false, node});
+        tp::Expr e;
+        e.kind = tp::Expr::Load;
+        e.cls = tp::Cls::F;
+        e.access.arg = 0;
+        e.access.dtype = d.dtype;
+        e.access.stride = ir::packed_strides(p.dims);
+        p.exprs.push_back(e);
+    };
+    operand(pr.op_a, da, op.inputs[0], pr.M, pr.K);
+    operand(pr.op_b, db, op.inputs[1], pr.K, pr.N);
+    pr.root_a = pr.root_b = 0;
+    pr.epi.dims = {batch, pr.M, pr.N};
+    pr.epi.fast_math = true;
+    tp::Expr acc;
+    acc.kind = tp::Expr::Acc;
+    acc.cls = tp::Cls::F;
+    pr.epi.exprs.push_back(acc);
+    pr.epi.acc_expr = 0;
+    tp::Out o;
+    o.expr = 0;
+    o.arg = 0;
+    o.dtype = dc.dtype;  // the accumulator type (op.rs:61-73)
+    pr.epi.outs.push_back(o);
+    pr.epi.args.push_back({dc.dtype, ir::num_elements(dc.shape), true, mm});
+    pr.args = {pr.op_a.args[0], pr.op_b.args[0], pr.epi.args[0]};
+    pr.map_a = {0};
+    pr.map_b = {1};
+    pr.map_e = {2};
+    if (op.inputs[0] == op.inputs[1]) {  // A x A: one kernel argument read twice
+        pr.args = {pr.op_a.args[0], pr.epi.args[0]};
+        pr.map_b = {0};
+        pr.map_e = {1};
+    }
+    return pr;
+}
+
+}  // namespace he::plan

@@ -1,0 +1,78 @@
+// Plan generation for a helium-ir graph: one instruction per op, greedy pairwise fusion, level-ised steps, late
+// scheduling and tensor lifetimes — helium/src/backend/plan_generation.rs, with the HIP backend's op -> instruction
+// mapping (helium/src/cuda.rs:33-60) and its instruction kinds (helium/src/cuda/instr.rs).
+#pragma once
+#include <functional>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "ir.h"
+#include "kernels.h"
+#include "permute.h"
+
+namespace he::plan {
+
+using ir::NodeId;
+
+enum class InstrKind : int { Gemm = 0, Pointwise = 1, Permute = 2 };
+
+// SwapDims nodes with more elements than this become Permute instructions (cuda.rs:38-41).
+constexpr int64_t kPermuteThreshold = 1000000;
+
+class Instr {
+public:
+    Instr(InstrKind kind, ir::OpSubgraph sg) : kind_(kind), sg_(std::move(sg)) {}
+    Instr(const Instr& o) : kind_(o.kind_), sg_(o.sg_), kernel_(o.kernel_), permute_(o.permute_) {}
+    InstrKind kind() const { return kind_; }
+    const ir::OpSubgraph& subgraph() const { return sg_; }
+    std::vector<NodeId> inputs() const { return sg_.inputs(); }   // Instruction::inputs (backend.rs:86)
+    std::vector<NodeId> outputs() const { return sg_.leafs(); }   // Instruction::outputs (backend.rs:87)
+    bool can_fuse_with(const Instr& next) const;                   // instr.rs:71-84
+    Instr fuse_with(const Instr& next) const;                      // instr.rs:86-99
+
+    // precompile (instr.rs:44-51): builds (or fetches from the kernel cache) the compiled kernel.
+    void precompile() const;
+    bool compiled() const {
+        std::lock_guard<std::mutex> lk(mu_);
+        return kernel_ || permute_;
+    }
+    // execute (instr.rs:27-42): `storage(node)` returns the device address of a tensor.
+    void execute(const std::function<void*(NodeId)>& storage, hipStream_t stream) const;
+    std::string describe() const;
+
+private:
+    InstrKind kind_;
+    ir::OpSubgraph sg_;
+    mutable std::shared_ptr<KernelBase> kernel_;   // Gemm / Pointwise
+    mutable std::shared_ptr<Permute> permute_;     // Permute
+    mutable std::mutex mu_;
+};
+
+// enumerate_swaps (permute_dims.rs:112-142): the chain of (axis_a, axis_b) when the subgraph is a linear chain of
+// SwapDims on one input; empty optional-like flag otherwise.
+bool enumerate_swaps(const ir::OpSubgraph& sg, std::vector<std::pair<int, int>>* swaps);
+
+Instr make_instr_for_op(const std::shared_ptr<const ir::OpGraph>& g, NodeId node);  // cuda.rs:33-60
+
+struct Step {
+    std::vector<std::shared_ptr<Instr>> instrs;
+    std::vector<NodeId> tensors_to_release;
+};
+struct Plan {
+    std::vector<Step> steps;
+    std::string describe() const;  // one line per step: instruction kinds, node sets, releases
+};
+
+// generate_plan (plan_generation.rs:22-26).
+std::shared_ptr<const Plan> generate_plan(const std::shared_ptr<const ir::OpGraph>& g);
+// generate_cached_plan (:16-19): LRU of 256 plans keyed by the graph's structure.
+std::shared_ptr<const Plan> generate_cached_plan(const std::shared_ptr<const ir::OpGraph>& g);
+void plan_cache_stats(uint64_t* hits, uint64_t* misses);
+
+// GEMM problem of a Matmul-anchored helium-ir subgraph (MatmulGenerator::new,
+// helium-kernel-generator/src/generators/matmul.rs:88-130). Throws HE_ERR_UNSUPPORTED for an UnsupportedFusion.
+GemmProblem gemm_problem_from_ir(const ir::OpSubgraph& sg);
+
+}  // namespace he::plan

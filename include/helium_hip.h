@@ -254,6 +254,47 @@ int he_aux_kernel_create(he_tile_kernel_t* kernel, he_fgraph_t graph);
  * accumulators), otherwise the auxiliary kernel. Arguments: producers in id order, then leaves in id order. */
 int he_fused_kernel_create(he_tile_kernel_t* kernel, he_fgraph_t graph);
 
+
+/* MatmulGenerator::new + generate (helium-kernel-generator/src/generators/matmul.rs:88-153) for the Matmul-anchored
+ * subgraph made of `nodes` of a helium-ir graph; HE_ERR_UNSUPPORTED stands for Err(UnsupportedFusion). The kernel's
+ * arguments are A, B, then the output, the order CompiledKernel::execute passes them (:181-219). */
+int he_matmul_kernel_create(he_tile_kernel_t* kernel, he_graph_t graph, const uint32_t* nodes, int num_nodes);
+
+/* ==================================================================================================
+ * 6. Backend: tensors, plan generation and graph execution — helium/src/backend.rs, backend/plan_generation.rs,
+ *    helium/src/cuda.rs, cuda/tensor_storage.rs, cuda/allocator/.
+ * ================================================================================================== */
+typedef struct he_tensor_s* he_tensor_t;
+typedef struct he_plan_s* he_plan_t;
+
+/* Backend::create_tensor_with_data (backend.rs:21-22, cuda.rs:62-79): asynchronous upload through pinned memory on
+ * a dedicated stream; the tensor's ready event is recorded behind it. `len` counts elements (bits for Bool). */
+int he_tensor_create_with_data(he_tensor_t* tensor, const void* data, int dtype, size_t len);
+/* Backend::download_tensor (backend.rs:24-29, cuda.rs:81-96), blocking form: waits for the ready event, copies
+ * the tensor's storage to `dst` and returns when the copy is done. */
+int he_tensor_download(he_tensor_t tensor, void* dst);
+int he_tensor_info(he_tensor_t tensor, int32_t* dtype, uint64_t* len, uint64_t* bytes, void** device_ptr);
+/* Drops one reference (TensorStorage is reference counted, tensor_storage.rs:30-42). */
+int he_tensor_free(he_tensor_t tensor);
+
+/* generate_plan (plan_generation.rs:22-26) for the graph as it stands; the graph must outlive the plan. */
+int he_plan_generate(he_graph_t graph, he_plan_t* plan);
+int he_plan_num_steps(he_plan_t plan, int* steps);
+/* One line per step: "step i: kind{node,node,...} ... | release node ...". */
+const char* he_plan_describe(he_plan_t plan);
+int he_plan_destroy(he_plan_t plan);
+
+/* BackendExt::execute_graph (backend.rs:40-80): prunes a copy of the graph, takes the cached plan, compiles its
+ * kernels, and runs the steps over a pool of streams. input_tensors[i] is the storage of Input node input_nodes[i].
+ * On return output_nodes / output_tensors hold one (Output node, tensor) pair per Output node of the graph; each
+ * tensor is a new reference the caller frees. */
+int he_execute_graph(he_graph_t graph, const uint32_t* input_nodes, const he_tensor_t* input_tensors, int num_inputs,
+                     uint32_t* output_nodes, he_tensor_t* output_tensors, int max_outputs, int* num_outputs);
+/* Counters of the last he_execute_graph on this thread: [0] steps run, [1] instructions, [2] streams used,
+ * [3] event waits; and of the process: [4] plan-cache hits, [5] misses, [6] bytes held from the driver,
+ * [7] driver allocations, [8] pooled reuses. */
+int he_backend_stats(uint64_t stats[9]);
+
 #ifdef __cplusplus
 }
 #endif

@@ -176,7 +176,8 @@ def matmul(a, b, precision, a_dtype, b_dtype):
 def evaluate(nodes, inputs, materialize=False):
     """Evaluates the graph. `inputs`: {input id: storage array}. Returns {node id: math-domain array} for every
     node plus the descriptors. With materialize=True every intermediate is rounded to its storage dtype (what
-    happens when each op runs as its own kernel); with False none is (one fused kernel)."""
+    happens when each op runs as its own kernel); with False none is (one fused kernel); with a set of node ids
+    exactly those are (the tensors that cross kernel boundaries of a plan)."""
     desc, val = {}, {}
     for n in nodes:
         i = n["id"]
@@ -191,7 +192,7 @@ def evaluate(nodes, inputs, materialize=False):
             val[i] = _eval_op(n, desc, val)
             shape, dtype = desc[i]
             assert list(val[i].shape) == list(shape), (n, val[i].shape, shape)
-            if materialize:
+            if materialize is True or (materialize is not False and i in materialize):
                 val[i] = nm.from_storage(nm.to_storage(val[i], dtype), dtype, shape)
     return val, desc
 
@@ -234,3 +235,20 @@ def kernel_outputs(nodes, inputs, leaf_ids):
     """Storage-domain outputs of ONE fused kernel whose leaves are `leaf_ids`."""
     val, desc = evaluate(nodes, inputs, materialize=False)
     return {i: nm.to_storage(val[i], desc[i][1]) for i in leaf_ids}
+
+
+def plan_outputs(nodes, inputs, plan_steps):
+    """Storage-domain value of every Output node when the graph runs as the kernels of `plan_steps`
+    ([(instrs, released)], instrs = [(kind, [node ids])]): a value is rounded to its storage dtype exactly where it
+    leaves the kernel that computes it. Returns {output node id: storage array}."""
+    consumers = {}
+    for n in nodes:
+        for p in (n.get("inputs") or ([n["from"]] if n["node"] == "output" else [])):
+            consumers.setdefault(p, []).append(n["id"])
+    boundary = set()
+    for instrs, _ in plan_steps:
+        for _, members in instrs:
+            inside = set(members)
+            boundary |= {m for m in members if any(c not in inside for c in consumers.get(m, []))}
+    val, desc = evaluate(nodes, inputs, materialize=boundary)
+    return {n["id"]: nm.to_storage(val[n["id"]], desc[n["id"]][1]) for n in nodes if n["node"] == "output"}

@@ -90,6 +90,20 @@ template <class V, bool BF> static inline emu_f32x16 emu_mfma(V a, V b, emu_f32x
 }
 #define __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, x, y, z) emu_mfma<decltype(a), true>(a, b, c)
 #define __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, x, y, z) emu_mfma<decltype(a), false>(a, b, c)
+static float g_mfa32[1024], g_mfb32[1024];
+static inline emu_f32x16 emu_mfma_f32(float a, float b, emu_f32x16 c) {
+    // v_mfma_f32_32x32x2_f32: lane l holds A[l%32][l/32] and B[l/32][l%32]
+    unsigned tid = threadIdx.x, base = tid & ~63u, lane = tid & 63u;
+    g_mfa32[tid] = a; g_mfb32[tid] = b;
+    pthread_barrier_wait(&g_bar);
+    for (int i = 0; i < 16; i++) {
+        unsigned row = (i / 4) * 8 + (lane / 32) * 4 + i % 4, col = lane % 32;
+        c[i] += g_mfa32[base + row] * g_mfb32[base + col] + g_mfa32[base + 32 + row] * g_mfb32[base + 32 + col];
+    }
+    pthread_barrier_wait(&g_bar);
+    return c;
+}
+#define __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, x, y, z) emu_mfma_f32(a, b, c)
 static const short* g_traddr[1024];
 static inline emu_s16x4 emu_tr16(const emu_s16x4* p) {
     // ds_read_b64_tr_b16, as measured on gfx950: within each group of 16 lanes, lane L gets element L%4 of the

@@ -25,13 +25,21 @@ def plain(m, n, k, batch=1, seed=0, dtype="bf16", out_dtype="f32", scale=0.5):
     return g, inputs, [out]
 
 
-def bias_relu_colsum(m, n, k, batch=1, seed=1, bias_axis=1, mainloop=False):
+def linear_layer(m, k, n):
+    """Config 1 at a small size: f32 Y = relu(X W + b) and its column sums."""
+    from helium_amd import configs
+
+    g, names = configs.c1_graph(m, k, n)
+    return g, configs.c1_inputs(names, m, k, n), [names["y"], names["colsum"]]
+
+
+def bias_relu_colsum(m, n, k, batch=1, seed=1, bias_axis=1, mainloop=False, a_dtype="bf16"):
     """Config 5a's shape of fusion: optional mainloop relu(A0) * T on the A operand, bias + Relu epilogue, the
     full-size result and its column sums as outputs."""
     g = ha.fusion.OpGraph()
     rng = np.random.default_rng(seed)
-    a0 = g.producer([batch, m, k], "bf16")
-    inputs = {a0: bf16_normal(rng, (batch, m, k))}
+    a0 = g.producer([batch, m, k], a_dtype)
+    inputs = {a0: bf16_normal(rng, (batch, m, k)) if a_dtype == "bf16" else rng.standard_normal((batch, m, k)).astype(np.float32)}
     a = a0
     if mainloop:
         t = g.producer([batch, m, k], "bf16")

@@ -1,0 +1,175 @@
+"""GPU parity tests of the backend slice through the C ABI: tensors, plans and execute_graph
+(helium/src/backend.rs:40-80, helium/src/cuda.rs:155-260) against the oracle on the same seeded inputs."""
+import threading
+
+import numpy as np
+import pytest
+
+import helium_amd as ha
+from helium_amd import configs
+from helium_amd.backend import Plan, Tensor, execute_graph, stats
+from oracle import helium_ir as oracle_ir
+from oracle import numerics as nm
+
+import test_plan_cpu as plans
+from helpers import assert_storage_close
+
+pytestmark = pytest.mark.gpu
+
+
+def run_graph(g, host_inputs):
+    """Uploads, executes, downloads. Returns ({output node: storage array}, plan steps)."""
+    by_id = {n["id"]: n for n in g.nodes}
+    tensors = {i: Tensor.from_numpy(a, by_id[i]["dtype"], int(np.prod(by_id[i]["shape"]))) for i, a in host_inputs.items()}
+    outs = execute_graph(g, tensors)
+    return {o: t.to_numpy() for o, t in outs.items()}, Plan(g).steps
+
+
+def check_against_oracle(g, host_inputs, got, steps, max_ulps=2, rel=1e-3, matmul_rel=None):
+    want = oracle_ir.plan_outputs(g.nodes, host_inputs, steps)
+    _, desc = oracle_ir.evaluate(g.nodes, host_inputs)
+    by_id = {n["id"]: n for n in g.nodes}
+    assert sorted(got) == sorted(want)
+    for o in want:
+        src = by_id[by_id[o]["from"]]
+        dtype = desc[o][1]
+        if matmul_rel is not None:
+            a = nm.from_storage(got[o], dtype, [got[o].size]).astype(np.float64)
+            b = nm.from_storage(want[o].reshape(-1), dtype, [want[o].size]).astype(np.float64)
+            scale = np.maximum(np.abs(b), np.abs(b).mean())
+            assert (np.abs(a - b) <= matmul_rel * scale + 1e-6).all(), (o, np.abs(a - b).max())
+        else:
+            is_sum = src.get("op") == "reduce" and src["fn"] in ("sum", "mean")
+            assert_storage_close(got[o], want[o].reshape(-1), dtype, f"output {o}", max_ulps=max_ulps,
+                                 reduce_rel=rel if is_sum else None)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "f16", "u32", "bool"])
+def test_tensor_upload_download_round_trip(gpu, dtype):
+    rng = np.random.default_rng(5)
+    n = 100_003
+    if dtype == "bool":
+        host = rng.integers(0, 2**32, (n + 31) // 32, dtype=np.uint32)
+    elif dtype == "u32":
+        host = rng.integers(0, 2**32, n, dtype=np.uint32)
+    elif dtype == "f32":
+        host = rng.standard_normal(n).astype(np.float32)
+    else:
+        host = rng.integers(0, 2**16, n).astype(np.uint16)
+    t = Tensor.from_numpy(host, dtype, n)
+    assert t.len == n and t.dtype == dtype
+    assert np.array_equal(t.to_numpy(), host)
+
+
+def seeded_inputs(g, seed):
+    rng = np.random.default_rng(seed)
+    return {n["id"]: nm.to_storage(rng.uniform(-1, 1, n["shape"]).astype(np.float32), n["dtype"])
+            for n in g.nodes if n["node"] == "input"}
+
+
+@pytest.mark.parametrize("make", [plans.linear_layer, plans.second_path_blocks_fusion, plans.constant_is_delayed,
+                                  plans.two_reduction_depths], ids=lambda f: f.__name__)
+def test_named_plans_execute(gpu, make):
+    g, _ = make()
+    host = seeded_inputs(g, 7)
+    got, steps = run_graph(g, host)
+    has_mm = any(n.get("op") == "matmul" for n in g.nodes)
+    check_against_oracle(g, host, got, steps, matmul_rel=1e-4 if has_mm else None)
+
+
+def test_large_swap_chain_runs_as_one_permute_and_is_bit_exact(gpu):
+    g, want_plan = plans.large_swaps_chain()
+    x = configs.permute_input("C2a")
+    got, steps = run_graph(g, {0: x})
+    assert steps == want_plan
+    (out,) = got.values()
+    assert np.array_equal(out.reshape(64, 256, 56, 56), np.transpose(x, (0, 3, 1, 2)))
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_graphs_execute(gpu, seed):
+    g = plans.random_graph(seed)
+    if g.nodes[0]["shape"][0] != 8:
+        pytest.skip("large-extent variants are plan-only cases")
+    if not any(n["node"] == "output" for n in g.nodes):
+        pytest.skip("graph without outputs")
+    host = seeded_inputs(g, seed)
+    got, steps = run_graph(g, host)
+    # chains of exp/tanh over matmuls amplify 1-ulp differences; the bound here is on the whole graph
+    want = oracle_ir.plan_outputs(g.nodes, host, steps)
+    _, desc = oracle_ir.evaluate(g.nodes, host)
+    for o in want:
+        a = nm.from_storage(got[o], desc[o][1], [got[o].size]).astype(np.float64)
+        b = nm.from_storage(want[o].reshape(-1), desc[o][1], [want[o].size]).astype(np.float64)
+        fin = np.isfinite(b)
+        assert np.array_equal(np.isfinite(a), fin)
+        assert np.allclose(a[fin], b[fin], rtol=2e-2 if desc[o][1] == "bf16" else 1e-3, atol=1e-5), (o, steps)
+
+
+def test_config1_linear_layer(gpu):
+    g, names = configs.c1_ir_graph()
+    host = configs.c1_inputs(names, batched=False)
+    got, steps = run_graph(g, host)
+    assert [k for instrs, _ in steps for k, _ in instrs] == ["gemm", "pointwise", "pointwise"]
+    val, _ = oracle_ir.evaluate(g.nodes, host)
+    y = got[names["y"]].reshape(256, 512).astype(np.float64)
+    want = val[names["y"]].astype(np.float64)
+    assert (np.abs(y - want) <= 1e-4 * np.maximum(np.abs(want), 1.0)).all()
+    cs = got[names["colsum"]].astype(np.float64)
+    want_cs = want.sum(axis=0)
+    assert (np.abs(cs - want_cs) <= 1e-3 * np.abs(want_cs) + 1e-4).all()
+
+
+@pytest.mark.parametrize("precision,dtype,rel", [("f32_f32", "f32", 1e-4), ("tf32_f32", "f32", 1e-4),
+                                                 ("bf16_f32", "bf16", 1e-2), ("f16_f32", "f16", 1e-2),
+                                                 ("f16_f16", "f16", 1e-2), ("bf16_f32", "f32", 1e-2)])
+def test_matmul_precisions(gpu, precision, dtype, rel):
+    rng = np.random.default_rng(9)
+    m, k, n = 384, 520, 264
+    g = ha.ir.OpGraph()
+    a, b = g.new_input([m, k], dtype), g.new_input([k, n], dtype)
+    g.new_output(g.matmul(a, b, precision))
+    host = {a: nm.to_storage(rng.uniform(-1, 1, (m, k)).astype(np.float32), dtype),
+            b: nm.to_storage(rng.uniform(-1, 1, (k, n)).astype(np.float32), dtype)}
+    got, steps = run_graph(g, host)
+    check_against_oracle(g, host, got, steps, matmul_rel=rel)
+
+
+def test_outputs_feed_the_next_graph_and_inputs_stay_intact(gpu):
+    rng = np.random.default_rng(3)
+    x = rng.uniform(-1, 1, (300, 70)).astype(np.float32)
+    g1 = ha.ir.OpGraph(); i1 = g1.new_input([300, 70], "f32"); o1 = g1.new_output(g1.unary(i1, "exp"))
+    g2 = ha.ir.OpGraph(); i2 = g2.new_input([300, 70], "f32"); o2 = g2.new_output(g2.reduce(g2.unary(i2, "neg"), "sum", 1))
+    tx = Tensor.from_numpy(x, "f32")
+    mid = execute_graph(g1, {i1: tx})[o1]
+    out = execute_graph(g2, {i2: mid})[o2].to_numpy()
+    assert np.array_equal(tx.to_numpy(), x)
+    want = -np.exp(x.astype(np.float64)).sum(axis=1)
+    assert np.allclose(out, want, rtol=1e-5)
+
+
+def test_four_threads_execute_concurrently(gpu):
+    # helium/tests/stress_test.rs:16-17: any thread may call execute_graph
+    g, names = configs.c1_ir_graph(64, 96, 80)
+    host = configs.c1_inputs(names, 64, 96, 80, batched=False)
+    ref, _ = run_graph(g, host)
+    errors = []
+
+    def worker():
+        try:
+            for _ in range(20):
+                got, _ = run_graph(g, host)
+                for o in ref:
+                    if o == names["y"]:
+                        assert np.array_equal(got[o], ref[o])
+                    else:
+                        assert np.allclose(got[o], ref[o], rtol=1e-5)
+        except Exception as e:  # noqa: BLE001
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker) for _ in range(4)]
+    [t.start() for t in threads]
+    [t.join() for t in threads]
+    assert not errors, errors[0]
+    s = stats()
+    assert s["plan_cache_hits"] > 0 and s["pool_reuses"] > 0

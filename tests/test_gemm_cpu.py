@@ -49,7 +49,9 @@ CASES = [
     ("row_bias", lambda: gemm_cases.bias_relu_colsum(64, 72, 64, bias_axis=2), "128,128,64,2,2"),
     ("all_reductions_batched", lambda: gemm_cases.all_reductions(70, 72, 64), "128,128,64,2,2"),
     ("f16_operands", lambda: gemm_cases.plain(64, 64, 64, dtype="f16"), "128,128,64,2,2"),
-    ("f32_operands_rounded_to_bf16", lambda: gemm_cases.plain(40, 48, 40, dtype="f32"), "128,128,64,2,2"),
+    ("f32_operands", lambda: gemm_cases.plain(40, 48, 40, dtype="f32"), "128,128,32,2,2"),
+    ("f32_mainloop_and_bf16_source_round_to_bf16", lambda: gemm_cases.bias_relu_colsum(64, 72, 40, mainloop=True, a_dtype="f32"), "128,128,64,2,2"),
+    ("f32_linear_layer", lambda: gemm_cases.linear_layer(48, 40, 72), "128,128,32,2,2"),
     ("big_tile_256", lambda: gemm_cases.plain(256, 256, 64), "256,256,64,2,2"),
     ("eight_tiles_xcd_order", lambda: gemm_cases.plain(256, 512, 64), "128,128,64,2,2"),
     ("twelve_tiles_grouped_order", lambda: gemm_cases.plain(768, 260, 64), "128,128,64,2,2"),
@@ -66,8 +68,12 @@ def test_fused_gemm_on_cpu(name, build, tile):
     g, inputs, outs = build()
     k, got = run_emulated(g, inputs, tile)
     assert sorted(got) == sorted(outs), k.description
-    want = oracle.outputs(g.nodes, inputs, round_mainloop_to="f16" if name == "f16_operands" else "bf16")
-    compare(got, want)
+    rounding = "f16" if name == "f16_operands" else None if name in ("f32_operands", "f32_linear_layer") else "bf16"
+    want = oracle.outputs(g.nodes, inputs, round_mainloop_to=rounding)
+    if rounding is None:
+        compare(got, want, rel=1e-4, eps=1e-5)  # f32 multiplicands: 1e-4 relative
+    else:
+        compare(got, want)
 
 
 def test_argument_order_is_producers_then_leaves():
@@ -75,3 +81,46 @@ def test_argument_order_is_producers_then_leaves():
     k = ha.TileKernel.fused(g)
     ins = [a["node"] for a in k.args if not a["is_output"]]
     assert ins == sorted(inputs) and [a["node"] for a in k.args if a["is_output"]] == outs
+
+
+# ---- helium-ir Matmul nodes (the GEMM instruction of the backend) -------------------------------------------
+def ir_matmul_case(shape_a, shape_b, precision, dtype, seed=3):
+    rng = np.random.default_rng(seed)
+    g = ha.ir.OpGraph()
+    a = g.new_input(shape_a, dtype); b = g.new_input(shape_b, dtype)
+    mm = g.matmul(a, b, precision)
+    g.new_output(mm)
+    inputs = {a: nm.to_storage(rng.uniform(-1, 1, shape_a).astype(np.float32), dtype),
+              b: nm.to_storage(rng.uniform(-1, 1, shape_b).astype(np.float32), dtype)}
+    return g, mm, inputs
+
+
+IR_CASES = [
+    # name, A shape, B shape, precision, storage dtype, max |err|
+    ("f32_exact_products", [70, 40], [40, 72], "f32_f32", "f32", 1e-4),
+    ("tf32_runs_as_f32", [33, 64], [64, 31], "tf32_f32", "f32", 1e-4),
+    ("bf16_multiplicands_of_f32_tensors", [64, 48], [48, 64], "bf16_f32", "f32", 1e-3),
+    ("f16_accumulator_type", [64, 64], [64, 64], "f16_f16", "f16", 2e-2),
+    ("batched_f32", [2, 40, 24], [2, 24, 36], "f32_f32", "f32", 1e-4),
+]
+
+
+@pytest.mark.parametrize("name,sa,sb,precision,dtype,tol", IR_CASES, ids=[c[0] for c in IR_CASES])
+def test_ir_matmul_on_cpu(name, sa, sb, precision, dtype, tol):
+    from oracle import helium_ir as oracle_ir
+
+    g, mm, inputs = ir_matmul_case(sa, sb, precision, dtype)
+    k = ha.backend.matmul_kernel(g, [mm])
+    gx, gy = map(int, re.search(r"grid=(\d+)x(\d+)", k.description).groups())
+    threads = int(re.search(r"threads=(\d+)", k.description).group(1))
+    bufs = []
+    for a in k.args:
+        dt = nm.NP_STORAGE[a["dtype"]]
+        bufs.append((np.zeros(a["numel"], dtype=dt), 2) if a["is_output"] else (inputs[a["node"]], 0))
+    res = run_kernel(k.source, "fused_matmul", gx, threads, bufs, grid_y=gy)
+    out = [a for a in k.args if a["is_output"]]
+    assert [a["node"] for a in out] == [mm]
+    want = oracle_ir.kernel_outputs(g.nodes, inputs, [mm])[mm]
+    got = nm.from_storage(res[0], out[0]["dtype"], [res[0].size]).astype(np.float64)
+    want = nm.from_storage(want.reshape(-1), out[0]["dtype"], [want.size]).astype(np.float64)
+    assert np.abs(got - want).max() <= tol, (k.description, np.abs(got - want).max())

@@ -1,0 +1,160 @@
+"""Plan generation (helium/src/backend/plan_generation.rs) through the C ABI.
+
+The expected plans of the named cases are worked out by hand from the reference text (slot order of the greedy
+fusion, Kahn levels, delay_computations, release lists); the same cases then pin oracle/plan.py, which in turn
+checks the library on seeded random graphs together with the invariants the reference asserts in debug builds
+(plan_generation.rs:418-445)."""
+import numpy as np
+import pytest
+
+import helium_amd as ha
+from helium_amd.backend import Plan, stats
+from oracle import plan as oracle_plan
+
+
+def linear_layer():
+    g = ha.ir.OpGraph()
+    x = g.new_input([256, 512], "f32"); w = g.new_input([512, 512], "f32"); b = g.new_input([512], "f32")
+    mm = g.matmul(x, w, "tf32_f32")
+    bb = g.broadcast(b, 2, [(0, 256)])
+    y = g.unary(g.binary(mm, bb, "add"), "relu")
+    r = g.reduce(g.swap_dims(y, 0, 1), "sum", 1)
+    g.new_output(y); g.new_output(r)
+    # broadcast+add+relu fuse; the swap cannot join them (a Broadcast was counted first, pointwise.rs:156-162) and
+    # starts a second kernel that takes the reduction
+    return g, [([("gemm", [3])], []), ([("pointwise", [4, 5, 6])], [0, 1]), ([("pointwise", [7, 8])], [2, 3]), ([], [])]
+
+
+def second_path_blocks_fusion():
+    g = ha.ir.OpGraph()
+    a = g.new_input([64, 64], "f32"); w = g.new_input([64, 64], "f32")
+    u = g.unary(a, "exp"); m = g.matmul(u, w, "f32_f32"); v = g.binary(u, m, "add")
+    g.new_output(v)
+    # exp and add are fusible, but exp -> matmul -> add is a second path (plan_generation.rs:195-217)
+    return g, [([("pointwise", [2])], []), ([("gemm", [3])], [0]), ([("pointwise", [4])], [1]), ([], [2, 3])]
+
+
+def constant_is_delayed():
+    g = ha.ir.OpGraph()
+    x = g.new_input([32, 32], "f32"); w = g.new_input([32, 32], "f32")
+    m1 = g.matmul(x, w, "f32_f32"); m2 = g.matmul(m1, w, "f32_f32")
+    c = g.constant(1.0, "f32", [32, 32])
+    g.new_output(g.binary(m2, c, "add"))
+    # the constant is ready at step 0 but first read at step 2, so it moves to step 1 (:325-353)
+    return g, [([("gemm", [2])], []), ([("gemm", [3]), ("pointwise", [4])], [0]), ([("pointwise", [5])], [1, 2]),
+               ([], [3, 4])]
+
+
+def large_swaps_chain():
+    g = ha.ir.OpGraph()
+    x = g.new_input([64, 56, 56, 256], "bf16")
+    g.new_output(g.swap_dims(g.swap_dims(x, 2, 3), 1, 2))
+    return g, [([("permute", [1, 2])], []), ([], [0])]
+
+
+def two_reduction_depths():
+    g = ha.ir.OpGraph()
+    a = g.new_input([64, 64], "f32")
+    t = g.unary(a, "tanh")
+    r1 = g.reduce(t, "sum", 2)
+    r2 = g.reduce(g.swap_dims(t, 0, 1), "sum", 1)
+    g.new_output(r1); g.new_output(r2)
+    # the chain takes the first reduction and the swap; the second reduction has another depth (pointwise.rs:163-179)
+    return g, [([("pointwise", [1, 2, 3])], []), ([("pointwise", [4])], [0]), ([], [3])]
+
+
+NAMED = [linear_layer, second_path_blocks_fusion, constant_is_delayed, large_swaps_chain, two_reduction_depths]
+
+
+@pytest.mark.parametrize("make", NAMED, ids=lambda f: f.__name__)
+def test_hand_derived_plans(make):
+    g, want = make()
+    assert oracle_plan.generate_plan(g.nodes) == want
+    assert Plan(g).steps == want
+
+
+def random_graph(seed):
+    rng = np.random.default_rng(seed)
+    n = int(rng.choice([8, 1024, 1100]))  # 1100² > 1,000,000: swaps become permute instructions
+    g = ha.ir.OpGraph()
+    vals = [(g.new_input([n, n], "f32"), [n, n]) for _ in range(int(rng.integers(1, 4)))]
+    for _ in range(int(rng.integers(3, 22))):
+        kind = rng.choice(["unary", "binary", "swap", "reduce", "matmul", "constant", "broadcast", "cast"],
+                          p=[0.3, 0.25, 0.12, 0.1, 0.06, 0.04, 0.08, 0.05])
+        x, shape = vals[int(rng.integers(len(vals)))]
+        if kind == "unary":
+            vals.append((g.unary(x, str(rng.choice(["exp", "relu", "neg", "tanh"]))), shape))
+        elif kind == "binary":
+            same = [v for v in vals if v[1] == shape]
+            y, _ = same[int(rng.integers(len(same)))]
+            vals.append((g.binary(x, y, str(rng.choice(["add", "mul", "max"]))), shape))
+        elif kind == "swap" and len(shape) == 2:
+            vals.append((g.swap_dims(x, 0, 1), shape[::-1]))
+        elif kind == "reduce" and len(shape) >= 1:
+            d = int(rng.integers(1, len(shape) + 1))
+            vals.append((g.reduce(x, str(rng.choice(["sum", "max"])), d), shape[: len(shape) - d] or [1]))
+        elif kind == "matmul" and shape == [n, n] and n <= 1024:
+            sq = [v for v in vals if v[1] == [n, n]]
+            y, _ = sq[int(rng.integers(len(sq)))]
+            vals.append((g.matmul(x, y, "f32_f32"), [n, n]))
+        elif kind == "constant":
+            vals.append((g.constant(2.0, "f32", [n, n]), [n, n]))
+        elif kind == "broadcast" and shape == [n]:
+            vals.append((g.broadcast(x, 2, [(0, n)]), [n, n]))
+        elif kind == "cast":
+            vals.append((g.unary(g.change_data_type(x, "bf16"), "neg"), shape))
+    consumed = {i for nd in g.nodes if nd["node"] == "op" for i in nd["inputs"]}
+    ops = [nd["id"] for nd in g.nodes if nd["node"] == "op"]
+    for i in ops:
+        if i not in consumed and rng.random() < 0.85 or rng.random() < 0.1:  # a few sinks stay dead on purpose
+            g.new_output(i)
+    return g
+
+
+def check_invariants(g, steps):
+    og = oracle_plan.Graph(g.nodes)
+    ops = [nd["id"] for nd in g.nodes if nd["node"] == "op"]
+    placed = [n for instrs, _ in steps for _, nodes in instrs for n in nodes]
+    assert sorted(placed) == sorted(ops), "every op belongs to exactly one instruction"
+    assert steps[-1][0] == [] and steps[0][1] == []
+    ready = {nd["id"] for nd in g.nodes if nd["node"] == "input"}
+    freed = set()
+    for instrs, released in steps:
+        for t in released:
+            assert t in ready and t not in freed and not og.feeds_output(t)
+            freed.add(t)
+        produced = set()
+        for _, nodes in instrs:
+            inside = set(nodes)
+            for n in nodes:
+                for p in og.inbound[n]:
+                    if p not in inside:
+                        assert p in ready and p not in freed, f"node {n} reads {p} before it exists / after its release"
+            produced |= inside
+        ready |= produced
+    # every tensor some instruction reads from outside is freed at some step unless it feeds an output
+    for instrs, _ in steps:
+        for _, nodes in instrs:
+            inside = set(nodes)
+            for n in nodes:
+                for p in og.inbound[n]:
+                    if p not in inside:
+                        assert p in freed or og.feeds_output(p), f"tensor {p} is never released"
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_graphs_match_the_restatement(seed):
+    g = random_graph(seed)
+    got = Plan(g).steps
+    assert got == oracle_plan.generate_plan(g.nodes)
+    check_invariants(g, got)
+
+
+def test_plan_cache_returns_the_same_plan_for_an_equal_graph():
+    before = stats()
+    a, _ = linear_layer()
+    b, _ = linear_layer()
+    pa, pb = Plan(a), Plan(b)
+    after = stats()
+    assert pa.text == pb.text
+    assert after["plan_cache_hits"] + after["plan_cache_misses"] >= before["plan_cache_hits"] + before["plan_cache_misses"]
