@@ -143,7 +143,7 @@ def test_outputs_feed_the_next_graph_and_inputs_stay_intact(gpu):
     tx = Tensor.from_numpy(x, "f32")
     mid = execute_graph(g1, {i1: tx})[o1]
     out = execute_graph(g2, {i2: mid})[o2].to_numpy()
-    assert np.array_equal(tx.to_numpy(), x)
+    assert np.array_equal(tx.to_numpy(), x.reshape(-1))
     want = -np.exp(x.astype(np.float64)).sum(axis=1)
     assert np.allclose(out, want, rtol=1e-5)
 

@@ -60,8 +60,17 @@ def test_reference_small_cases(gpu):
 def test_f16_and_f32_operands(gpu):
     g, inputs, outs = gemm_cases.plain(192, 200, 136, dtype="f16")
     check(g, inputs, outs, mma="f16")
+    # all-f32 sources multiply as f32: 1e-4 relative
     g, inputs, outs = gemm_cases.plain(192, 200, 136, dtype="f32")
-    check(g, inputs, outs, mma="bf16")
+    check(g, inputs, outs, mma=None, rel=1e-4, eps=1e-5)
+
+
+def test_config1_linear_layer_as_one_fusion(gpu):
+    from helium_amd import configs
+
+    g, names = configs.c1_graph()
+    k = check(g, configs.c1_inputs(names), [names["y"], names["colsum"]], mma=None, rel=1e-4, eps=1e-4)
+    assert "mma=f32" in k.description
 
 
 @pytest.mark.parametrize("mainloop", [False, True])
