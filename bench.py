@@ -21,6 +21,10 @@ sys.path.insert(0, ROOT)
 METRIC = "fused-GEMM TFLOP/s & permute/pointwise GB/s, % of MI355X roofline"
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 BF16_PEAK_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
+# Bytes that left the XCD L2s per launch of each workload's dominant kernel: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE,
+# each scaled by what the same counter reads for the COPY workload (profiles/<kernel>_<workload>.txt).
+TRAFFIC_BYTES = {"COPY": 268435456, "C2a": 205565287, "C2b": 67153057, "C2c": 17587641, "C3": 277275033,
+                 "C4": 378277232, "C5a": 302136294, "GEMM": 234913614}
 HEADLINE = "C4"              # the workload `value` is quoted on
 ROTATE_BYTES = 768 << 20     # rotate operand sets so repeated steps cannot live in the 256 MB Infinity Cache
 
@@ -310,6 +314,9 @@ def make_workloads():
 
     w = {name: PermuteWorkload(name, shape, perm, {"C2a": 21, "C2b": 22, "C2c": 23}[name])
          for name, (shape, perm) in configs.PERMUTES.items()}
+    # a plain copy of known size (identity permute): the measured ceiling the permute kernels are read against and
+    # the scale for the FETCH_SIZE / WRITE_SIZE counters
+    w["COPY"] = PermuteWorkload("COPY", (8192, 8192), (0, 1), 24)
     w["C3"] = AuxChainWorkload()
     for name in ("C4", "C5a", "C4m", "GEMM"):
         w[name] = FusedGemmWorkload(name)
@@ -344,7 +351,7 @@ def roofline(wl, ms):
         achieved = wl.work / (ms * 1e-3) / 1e12
         peak, unit = BF16_PEAK_TFLOPS, "TFLOP/s"
     return {"bound": wl.bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
-            "frac": round(achieved / peak, 4), "traffic": getattr(wl, "traffic", None)}
+            "frac": round(achieved / peak, 4), "traffic": TRAFFIC_BYTES.get(wl.name)}
 
 
 def main():
