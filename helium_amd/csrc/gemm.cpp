@@ -94,6 +94,145 @@ __device__ __forceinline__ u32 a_off(u32 m, u32 kc) { return m * (BK * ESZ) + ((
 __device__ __forceinline__ u32 b_chunk_off(u32 k, u32 nc) { return k * (BN * ESZ) + ((nc ^ (MMA_F32 ? 0u : ((k & 3) << 2))) << 4); }
 __device__ __forceinline__ u32 b_off(u32 k, u32 n) { return b_chunk_off(k, (n * ESZ) >> 4) + ((n * ESZ) & 15); }
 
+#if MMA_F32
+typedef f32x4 afrag_t;
+typedef f32x4 bfrag_t;
+#else
+typedef s16x8 afrag_t;
+typedef s16x8 bfrag_t;
+#endif
+struct WavePos { u32 lane, wave, wave_m, wave_n; };
+
+// Operand fragments of k-step kk from one LDS stage. `st` is __restrict__ on purpose: after inlining, every LDS
+// read carries alias-scope information that separates it from the direct global->LDS writes into the *other*
+// stage, so the compiler does not make the reads wait for those writes (vmcnt) before the MFMAs can start.
+__device__ __forceinline__ void load_frags(const unsigned char* __restrict__ st, int kk, const WavePos& w,
+                                           afrag_t (&af)[MB], bfrag_t (&bf)[NB]) {
+    const unsigned char* la = st;
+    const unsigned char* lb = st + A_TILE_BYTES;
+    const u32 lane = w.lane;
+#if MMA_F32
+    // v_mfma_f32_32x32x2_f32: lane l supplies A[l % 32][l / 32] and B[l / 32][l % 32]. One k-step covers 8 k: each
+    // lane half owns 4 consecutive k (one 16-byte chunk of its A row) and issues 4 MFMAs per output block.
+#pragma unroll
+    for (int i = 0; i < MB; i++) {
+        const u32 row = w.wave_m * WTM + i * 32 + (lane & 31);
+        af[i] = *(const f32x4*)(la + a_off(row, kk * 2 + (lane >> 5)));
+    }
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+        const u32 n = w.wave_n * WTN + j * 32 + (lane & 31);
+#pragma unroll
+        for (int e = 0; e < 4; e++) bf[j][e] = *(const float*)(lb + b_off(kk * 8 + (lane >> 5) * 4 + e, n));
+    }
+#else
+    const u32 grp = lane >> 4, sub = lane & 15;
+#pragma unroll
+    for (int i = 0; i < MB; i++) {
+        const u32 row = w.wave_m * WTM + i * 32 + (lane & 31);
+        af[i] = *(const s16x8*)(la + a_off(row, kk * 2 + (lane >> 5)));
+    }
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+        const u32 k = kk * 16 + (grp >> 1) * 8 + (sub >> 2);
+        const u32 n = w.wave_n * WTN + j * 32 + (grp & 1) * 16 + (sub & 3) * 4;
+        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(lb + b_off(k, n)));
+        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(lb + b_off(k + 4, n)));
+        bf[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+#endif
+}
+
+__device__ __forceinline__ void mma_step(f32x16 (&acc)[MB][NB], const afrag_t (&af)[MB], const bfrag_t (&bf)[NB]) {
+#if MMA_F32
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+#pragma unroll
+        for (int i = 0; i < MB; i++)
+#pragma unroll
+            for (int j = 0; j < NB; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][e], bf[j][e], acc[i][j], 0, 0, 0);
+#else
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+#pragma unroll
+        for (int j = 0; j < NB; j++) {
+#if MMA_BF16
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[i]),
+                                                               __builtin_bit_cast(bf16x8, bf[j]), acc[i][j], 0, 0, 0);
+#else
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, af[i]),
+                                                              __builtin_bit_cast(f16x8, bf[j]), acc[i][j], 0, 0, 0);
+#endif
+        }
+#endif
+}
+
+// One k-tile: operands for step kk+1 are fetched from LDS while the MFMAs of step kk run.
+template <class PerStep>
+__device__ __forceinline__ void compute_tile(const unsigned char* __restrict__ st, f32x16 (&acc)[MB][NB], const WavePos& w,
+                                             PerStep&& per_step) {
+    afrag_t af[2][MB];
+    bfrag_t bf[2][NB];
+    load_frags(st, 0, w, af[0], bf[0]);
+#pragma unroll
+    for (int kk = 0; kk < KK; kk++) {
+        per_step(kk);  // a slice of the next tile's global->LDS traffic
+#if GEMM_SKIP & 2
+        if (kk + 1 < KK) { for (int i = 0; i < MB; i++) af[(kk + 1) & 1][i] = af[kk & 1][i]; for (int j = 0; j < NB; j++) bf[(kk + 1) & 1][j] = bf[kk & 1][j]; }
+#else
+        if (kk + 1 < KK) load_frags(st, kk + 1, w, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+#endif
+#if !(GEMM_SKIP & 4)
+        mma_step(acc, af[kk & 1], bf[kk & 1]);
+#else
+        acc[0][0][0] += (float)af[kk & 1][0][0] + (float)bf[kk & 1][0][0];
+#endif
+        SCHED_HINT
+    }
+    SCHED_PLAN
+}
+
+#if DIRECT_LOADS
+// Operand tiles go from global memory straight into LDS (global_load_lds_dwordx4): a wave instruction fills
+// 1 KB of LDS in lane order, so each lane fetches the global chunk whose swizzled LDS slot is lane * 16.
+// `ga` / `gb` point at the tile's first A row / first B k-row (at this workgroup's columns).
+#define A_DPW (A_TILE_BYTES / 1024 / NWAVES)  /* direct-load instructions per wave and tile */
+#define B_DPW (B_TILE_BYTES / 1024 / NWAVES)
+__device__ __forceinline__ void direct_issue(unsigned char* __restrict__ st, const bf16_t* __restrict__ ga,
+                                             const bf16_t* __restrict__ gb, const WavePos& w, int i) {
+#if GEMM_SKIP & 1
+    return;
+#endif
+    const u32 lane = w.lane, wave = w.wave;
+    if (i < A_DPW) {
+        const u32 blk = wave * A_DPW + i;
+        const u32 row = blk * (64 / A_CHUNKS) + lane / A_CHUNKS, pc = lane % A_CHUNKS;
+        const u32 kc = pc ^ ((row >> A_SWZ_SHIFT) & (A_CHUNKS - 1));
+        const bf16_t* gp = ga + (size_t)row * GK + kc * 8;
+        __builtin_amdgcn_global_load_lds((GLOBAL_AS const void*)gp, (LDS_AS void*)(st + blk * 1024), 16, 0, 0);
+    } else {
+        const u32 blk = wave * B_DPW + (i - A_DPW);
+        const u32 krow = blk * (64 / B_CHUNKS) + lane / B_CHUNKS, pc = lane % B_CHUNKS;
+        const u32 nc = pc ^ ((krow & 3) << 2);
+        const bf16_t* gp = gb + (size_t)krow * GN + nc * 8;
+        __builtin_amdgcn_global_load_lds((GLOBAL_AS const void*)gp, (LDS_AS void*)(st + A_TILE_BYTES + blk * 1024), 16, 0, 0);
+    }
+}
+// Multiplies the tile in stage `rd` while requesting the tile that goes into stage `wr`.
+__device__ __forceinline__ void direct_tile(const unsigned char* __restrict__ rd, unsigned char* __restrict__ wr,
+                                            const bf16_t* __restrict__ ga, const bf16_t* __restrict__ gb, bool more,
+                                            f32x16 (&acc)[MB][NB], const WavePos& w) {
+    compute_tile(rd, acc, w, [&](int kk) {
+        constexpr int per = ISSUE_FRONT ? (A_DPW + B_DPW) : (A_DPW + B_DPW + KK - 1) / KK;
+        if (more) {
+#pragma unroll
+            for (int i = kk * per; i < (kk + 1) * per && i < A_DPW + B_DPW; i++) direct_issue(wr, ga, gb, w, i);
+        }
+    });
+}
+#endif
+
 #ifndef KERNEL_ATTRS
 /* NWAVES / 4 waves per SIMD: with four waves each one owns the full 512-register budget */
 #define KERNEL_ATTRS __attribute__((amdgpu_waves_per_eu(NWAVES / 4, NWAVES / 4)))
@@ -150,142 +289,35 @@ void fused_matmul(KERNEL_PARAMS) {
             *(u32x4*)(lb + b_chunk_off(idx / B_CHUNKS, idx % B_CHUNKS)) = sb[i];
         }
     };
-    const u32 grp = lane >> 4, sub = lane & 15;
-    (void)grp; (void)sub;
-#if MMA_F32
-    // v_mfma_f32_32x32x2_f32: lane l supplies A[l % 32][l / 32] and B[l / 32][l % 32]. One k-step covers 8 k: each
-    // lane half owns 4 consecutive k (one 16-byte chunk of its A row) and issues 4 MFMAs per output block.
-    typedef f32x4 afrag_t;
-    typedef f32x4 bfrag_t;
-    auto load_frags = [&](u32 buf, int kk, afrag_t (&af)[MB], bfrag_t (&bf)[NB]) {
-        const unsigned char* la = lds + buf * STAGE_BYTES;
-        const unsigned char* lb = la + A_TILE_BYTES;
-#pragma unroll
-        for (int i = 0; i < MB; i++) {
-            const u32 row = wave_m * WTM + i * 32 + (lane & 31);
-            af[i] = *(const f32x4*)(la + a_off(row, kk * 2 + (lane >> 5)));
-        }
-#pragma unroll
-        for (int j = 0; j < NB; j++) {
-            const u32 n = wave_n * WTN + j * 32 + (lane & 31);
-#pragma unroll
-            for (int e = 0; e < 4; e++) bf[j][e] = *(const float*)(lb + b_off(kk * 8 + (lane >> 5) * 4 + e, n));
-        }
-    };
-    auto mma = [&](const afrag_t (&af)[MB], const bfrag_t (&bf)[NB]) {
-#pragma unroll
-        for (int e = 0; e < 4; e++)
-#pragma unroll
-            for (int i = 0; i < MB; i++)
-#pragma unroll
-                for (int j = 0; j < NB; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][e], bf[j][e], acc[i][j], 0, 0, 0);
-    };
-#else
-    typedef s16x8 afrag_t;
-    typedef s16x8 bfrag_t;
-    auto load_frags = [&](u32 buf, int kk, s16x8 (&af)[MB], s16x8 (&bf)[NB]) {
-        const unsigned char* la = lds + buf * STAGE_BYTES;
-        const unsigned char* lb = la + A_TILE_BYTES;
-#pragma unroll
-        for (int i = 0; i < MB; i++) {
-            const u32 row = wave_m * WTM + i * 32 + (lane & 31);
-            af[i] = *(const s16x8*)(la + a_off(row, kk * 2 + (lane >> 5)));
-        }
-#pragma unroll
-        for (int j = 0; j < NB; j++) {
-            const u32 k = kk * 16 + (grp >> 1) * 8 + (sub >> 2);
-            const u32 n = wave_n * WTN + j * 32 + (grp & 1) * 16 + (sub & 3) * 4;
-            s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(lb + b_off(k, n)));
-            s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(lb + b_off(k + 4, n)));
-            bf[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        }
-    };
-    auto mma = [&](const s16x8 (&af)[MB], const s16x8 (&bf)[NB]) {
-#pragma unroll
-        for (int i = 0; i < MB; i++)
-#pragma unroll
-            for (int j = 0; j < NB; j++) {
-#if MMA_BF16
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[i]),
-                                                                   __builtin_bit_cast(bf16x8, bf[j]), acc[i][j], 0, 0, 0);
-#else
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, af[i]),
-                                                                  __builtin_bit_cast(f16x8, bf[j]), acc[i][j], 0, 0, 0);
-#endif
-            }
-    };
-#endif
-    // One k-tile: operands for step kk+1 are fetched from LDS while the MFMAs of step kk run.
-    auto compute = [&](u32 buf, auto&& per_step) {
-        afrag_t af[2][MB];
-        bfrag_t bf[2][NB];
-        load_frags(buf, 0, af[0], bf[0]);
-#pragma unroll
-        for (int kk = 0; kk < KK; kk++) {
-            per_step(kk);  // a slice of the next tile's global->LDS traffic, spread over the MFMA steps
-#if GEMM_SKIP & 2
-            if (kk + 1 < KK) { for (int i = 0; i < MB; i++) af[(kk + 1) & 1][i] = af[kk & 1][i]; for (int j = 0; j < NB; j++) bf[(kk + 1) & 1][j] = bf[kk & 1][j]; }
-#else
-            if (kk + 1 < KK) load_frags(buf, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
-#endif
-#if !(GEMM_SKIP & 4)
-            mma(af[kk & 1], bf[kk & 1]);
-#else
-            acc[0][0][0] += (float)af[kk & 1][0][0] + (float)bf[kk & 1][0][0];
-#endif
-            SCHED_HINT
-        }
-        SCHED_PLAN
-    };
+    const WavePos wpos = {lane, wave, wave_m, wave_n};
 
 #if DIRECT_LOADS
-    // Operand tiles go from global memory straight into LDS (global_load_lds_dwordx4): a wave instruction fills
-    // 1 KB of LDS in lane order, so each lane fetches the global chunk whose swizzled LDS slot is lane * 16.
 /* s_waitcnt immediate: vmcnt lives in bits [3:0] and [15:14] */
 #define WAITCNT_VM(n) ((((n) & 15) | (((n) >> 4) << 14)))
-#define A_DPW (A_TILE_BYTES / 1024 / NWAVES)  /* direct-load instructions per wave and tile */
-#define B_DPW (B_TILE_BYTES / 1024 / NWAVES)
-    auto direct_issue = [&](u32 kt, u32 buf, int i) {
-#if GEMM_SKIP & 1
-        return;
-#endif
-        unsigned char* la = lds + buf * STAGE_BYTES;
-        unsigned char* lb = la + A_TILE_BYTES;
-        const u32 k0 = k_tile(kt) * BK;
-        if (i < A_DPW) {
-            const u32 blk = wave * A_DPW + i;
-            const u32 row = blk * (64 / A_CHUNKS) + lane / A_CHUNKS, pc = lane % A_CHUNKS;
-            const u32 kc = pc ^ ((row >> A_SWZ_SHIFT) & (A_CHUNKS - 1));
-            const bf16_t* gp = (const bf16_t*)DIRECT_A_PTR + ((size_t)bz * GM + m0 + row) * GK + k0 + kc * 8;
-            __builtin_amdgcn_global_load_lds((GLOBAL_AS const void*)gp, (LDS_AS void*)(la + blk * 1024), 16, 0, 0);
-        } else {
-            const u32 blk = wave * B_DPW + (i - A_DPW);
-            const u32 krow = blk * (64 / B_CHUNKS) + lane / B_CHUNKS, pc = lane % B_CHUNKS;
-            const u32 nc = pc ^ ((krow & 3) << 2);
-            const bf16_t* gp = (const bf16_t*)DIRECT_B_PTR + ((size_t)bz * GK + k0 + krow) * GN + n0 + nc * 8;
-            __builtin_amdgcn_global_load_lds((GLOBAL_AS const void*)gp, (LDS_AS void*)(lb + blk * 1024), 16, 0, 0);
-        }
-    };
+    const bf16_t* const ga0 = (const bf16_t*)DIRECT_A_PTR + ((size_t)bz * GM + m0) * GK;
+    const bf16_t* const gb0 = (const bf16_t*)DIRECT_B_PTR + (size_t)bz * GK * GN + n0;
     // NSTAGES-deep ring of LDS stages: tile kt + NSTAGES - 1 is requested while tile kt is multiplied, so a
     // wave only ever waits for loads issued NSTAGES - 2 tiles earlier.
 #pragma unroll
     for (int st = 0; st < NSTAGES - 1; st++)
         if (st < KT) {
 #pragma unroll
-            for (int i = 0; i < A_DPW + B_DPW; i++) direct_issue(st, st, i);
+            for (int i = 0; i < A_DPW + B_DPW; i++)
+                direct_issue(lds + st * STAGE_BYTES, ga0 + k_tile(st) * BK, gb0 + (size_t)(k_tile(st) * BK) * GN, wpos, i);
         }
 #if GEMM_TIMING
     unsigned long long t_load = 0, t_compute = 0, t_wait = 0, t_barrier = 0, t0, t1;
 #define TICK(var) t1 = __builtin_readcyclecounter(); var += t1 - t0; t0 = t1;
     t0 = __builtin_readcyclecounter();
+    const unsigned long long wall0 = __builtin_amdgcn_s_memrealtime();
 #else
 #define TICK(var)
 #endif
     for (u32 kt = 0; kt < KT; kt++) {
         // tile kt must have landed; up to NSTAGES - 2 younger tiles may still be in flight
         const u32 younger = KT - 1 - kt < NSTAGES - 2 ? KT - 1 - kt : NSTAGES - 2;
-        if (younger >= 2) __builtin_amdgcn_s_waitcnt(0x0F70 | WAITCNT_VM(2 * (A_DPW + B_DPW)));
+        if (younger >= 3) __builtin_amdgcn_s_waitcnt(0x0F70 | WAITCNT_VM(3 * (A_DPW + B_DPW)));
+        else if (younger == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | WAITCNT_VM(2 * (A_DPW + B_DPW)));
         else if (younger == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | WAITCNT_VM(A_DPW + B_DPW));
         else __builtin_amdgcn_s_waitcnt(0x0F70);
         TICK(t_wait)
@@ -293,13 +325,9 @@ void fused_matmul(KERNEL_PARAMS) {
         TICK(t_barrier)
         const u32 next = kt + NSTAGES - 1;
         const bool more = next < KT;
-        compute(kt % NSTAGES, [&](int kk) {
-            constexpr int per = (A_DPW + B_DPW + KK - 1) / KK;
-            if (more) {
-#pragma unroll
-                for (int i = kk * per; i < (kk + 1) * per && i < A_DPW + B_DPW; i++) direct_issue(next, next % NSTAGES, i);
-            }
-        });
+        const u32 knext = more ? k_tile(next) * BK : 0u;
+        direct_tile(lds + (kt % NSTAGES) * STAGE_BYTES, lds + (next % NSTAGES) * STAGE_BYTES, ga0 + knext,
+                    gb0 + (size_t)knext * GN, more, acc, wpos);
         __builtin_amdgcn_sched_barrier(0);
         TICK(t_compute)
     }
@@ -308,6 +336,7 @@ void fused_matmul(KERNEL_PARAMS) {
     if (blockIdx.x == 0 && tid == 64) {
         unsigned long long* dbg = (unsigned long long*)GEMM_TIMING_PTR;
         dbg[0] = t_load; dbg[1] = t_compute; dbg[2] = t_wait; dbg[3] = t_barrier;
+        dbg[4] = __builtin_amdgcn_s_memrealtime() - wall0;  // 100 MHz ticks
     }
     __syncthreads();
     if (blockIdx.x == 0) return;
@@ -321,7 +350,7 @@ void fused_matmul(KERNEL_PARAMS) {
         // The next tile's global loads are issued before any MFMA of this tile and consumed after the last one.
         if (more) stage_load(kt + 1);
         STAGE_SCHED_BARRIER
-        compute(kt & 1, [](int) {});
+        compute_tile(lds + (kt & 1) * STAGE_BYTES, acc, wpos, [](int) {});
         STAGE_SCHED_BARRIER
         if (more) stage_store((kt + 1) & 1);
         __syncthreads();
@@ -473,7 +502,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     const int threads = t.wm * t.wn * 64;
     HE_REQUIRE(threads == 256 || threads == 512, HE_ERR_INVALID, "GEMM workgroups have 4 or 8 waves");
     HE_REQUIRE((t.bm * t.bk / epc) % threads == 0 && (t.bk * t.bn / epc) % threads == 0, HE_ERR_INVALID, "bad GEMM tile");
-    HE_REQUIRE(t.stages >= 2 && t.stages <= 4 && t.stages * (t.bm + t.bn) * t.bk * (16 / epc) <= 160 * 1024, HE_ERR_INVALID,
+    HE_REQUIRE(t.stages >= 2 && t.stages <= 5 && t.stages * (t.bm + t.bn) * t.bk * (16 / epc) <= 160 * 1024, HE_ERR_INVALID,
                "GEMM tile exceeds LDS");
     const int wtn = t.bn / t.wn;
 
@@ -483,7 +512,6 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     const bool direct = want_direct && raw_a && raw_b && pr.M % t.bm == 0 && pr.N % t.bn == 0 && pr.K % t.bk == 0 &&
                         (t.bm * t.bk * 2 / 1024) % (threads / 64) == 0 && (t.bk * t.bn * 2 / 1024) % (threads / 64) == 0 &&
                         64 % (t.bn / 8) == 0;
-    if (!direct) t.stages = 2;
     if (!direct) t.stages = 2;
     int nve = tp::pick_nv(pr.epi, 32);
     while (nve > 1 && ((32 * wtn) % (64 * nve) != 0)) nve /= 2;
@@ -499,6 +527,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     s << "#define BM " << t.bm << "\n#define BN " << t.bn << "\n#define BK " << t.bk << "\n#define WAVES_M " << t.wm
       << "\n#define WAVES_N " << t.wn << "\n#define NSTAGES " << t.stages << "\n#define NVE " << nve << "\n#define MMA_BF16 " << (pr.mma_dtype == HE_BF16 ? 1 : 0) << "\n#define MMA_F32 " << (f32 ? 1 : 0)
       << "\n#define STAGGER_EXPR " << (getenv("HELIUM_HIP_GEMM_STAGGER") ? getenv("HELIUM_HIP_GEMM_STAGGER") : "0u")
+      << "\n#define ISSUE_FRONT " << (getenv("HELIUM_HIP_GEMM_ISSUE") ? atoi(getenv("HELIUM_HIP_GEMM_ISSUE")) : 0)
       << "\n#define GEMM_SKIP " << (getenv("HELIUM_HIP_GEMM_SKIP") ? atoi(getenv("HELIUM_HIP_GEMM_SKIP")) : 0)
       << "\n#define GEMM_TIMING " << (getenv("HELIUM_HIP_GEMM_TIMING") ? 1 : 0) << "\n#define GEMM_TIMING_PTR p" << (pr.args.size() - 1)
       << "\n#define DIRECT_LOADS " << (direct ? 1 : 0) << "\n#define DIRECT_A_PTR p" << (direct ? pr.map_a[0] : 0)
@@ -649,7 +678,8 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
             plan << "__builtin_amdgcn_sched_group_barrier(0x100, " << nr << ", 0);\n";
             const int waves = threads / 64;
             const int dl = direct ? (t.bm * t.bk * 2 / 1024 + t.bk * t.bn * 2 / 1024) / waves : 0;
-            const int per = (dl + kk_steps - 1) / kk_steps;
+            const bool front = getenv("HELIUM_HIP_GEMM_ISSUE") && atoi(getenv("HELIUM_HIP_GEMM_ISSUE"));
+            const int per = front ? dl : (dl + kk_steps - 1) / kk_steps;
             for (int kk = 0; kk < kk_steps; kk++) {
                 int issue = std::max(0, std::min(per, dl - kk * per));
                 if (issue) plan << "__builtin_amdgcn_sched_group_barrier(0x020, " << issue << ", 0);\n";
