@@ -257,6 +257,22 @@ int pick_nv(const Program& p, int max_bytes) {
     return nv;
 }
 
+static bool is_deferred_load(const Program& p, const Expr& e, int nv) {
+    if (e.kind != Expr::Load || nv < 2 || !e.access.chain.empty() || e.access.dtype == HE_BOOL) return false;
+    const int n = (int)p.dims.size();
+    return p.dims[n - 1] > 1 && e.access.stride[n - 1] == 1;
+}
+static std::string raw_type(int dtype, int nv) {
+    const char* elem = dtype == HE_BF16 ? "u16" : dtype == HE_F16 ? "f16_t" : dtype == HE_U32 ? "u32" : "float";
+    return strfmt("typename Vec<%s, %d>::type", elem, nv);
+}
+std::string emit_raw_members(const Program& p, int nv) {
+    std::ostringstream s;
+    for (size_t i = 0; i < p.exprs.size(); i++)
+        if (is_deferred_load(p, p.exprs[i], nv)) s << raw_type(p.exprs[i].access.dtype, nv) << " raw" << i << ";\n";
+    return s.str();
+}
+
 std::string emit_exprs(const Program& p, const EmitCtx& cx) {
     const int n = (int)p.dims.size();
     const int NV = cx.nv;
@@ -276,6 +292,22 @@ std::string emit_exprs(const Program& p, const EmitCtx& cx) {
         const Expr& e = p.exprs[i];
         const std::string v = "e" + std::to_string(i);
         const char* T = cls_type(e.cls);
+        if (cx.phase != 0) {
+            const bool deferred = is_deferred_load(p, e, NV);
+            if (cx.phase == 1) {
+                if (deferred)
+                    s << "{ const size_t o = " << coord_sum(e.access.stride) << ";\nR.raw" << i << " = *(const " << raw_type(e.access.dtype, NV)
+                      << "*)(a" << e.access.arg << " + o); }\n";
+                continue;
+            }
+            if (deferred) {
+                s << T << " " << v << "[" << NV << "];\n#pragma unroll\nfor (int k = 0; k < " << NV << "; k++) " << v << "[k] = ";
+                if (e.access.dtype == HE_BF16) s << "__builtin_bit_cast(float, (u32)R.raw" << i << "[k] << 16);\n";
+                else if (e.access.dtype == HE_F16) s << "(float)R.raw" << i << "[k];\n";
+                else s << "R.raw" << i << "[k];\n";
+                continue;
+            }
+        }
         auto each = [&](const std::string& rhs_k) {
             s << T << " " << v << "[" << NV << "];\n#pragma unroll\nfor (int k = 0; k < " << NV << "; k++) " << v
               << "[k] = " << rhs_k << ";\n";

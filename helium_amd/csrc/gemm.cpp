@@ -197,8 +197,8 @@ __device__ __forceinline__ void compute_tile(const unsigned char* __restrict__ s
 // Operand tiles go from global memory straight into LDS (global_load_lds_dwordx4): a wave instruction fills
 // 1 KB of LDS in lane order, so each lane fetches the global chunk whose swizzled LDS slot is lane * 16.
 // `ga` / `gb` point at the tile's first A row / first B k-row (at this workgroup's columns).
-#define A_DPW (A_TILE_BYTES / 1024 / NWAVES)  /* direct-load instructions per wave and tile */
-#define B_DPW (B_TILE_BYTES / 1024 / NWAVES)
+#define A_DPW (DIRECT_A ? A_TILE_BYTES / 1024 / NWAVES : 0)  /* direct-load instructions per wave and tile */
+#define B_DPW (DIRECT_B ? B_TILE_BYTES / 1024 / NWAVES : 0)
 __device__ __forceinline__ void direct_issue(unsigned char* __restrict__ st, const bf16_t* __restrict__ ga,
                                              const bf16_t* __restrict__ gb, const WavePos& w, int i) {
 #if GEMM_SKIP & 1
@@ -259,41 +259,85 @@ void fused_matmul(KERNEL_PARAMS) {
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
-    u32x4 sa[A_PER_THREAD], sb[B_PER_THREAD];
+    // Register staging of the operands that do not travel by direct global->LDS loads. A raw operand waits in
+    // registers as the 16-byte chunk it was loaded as; a mainloop-fused one as its undecoded source vectors, which
+    // stage_store turns into multiplicands after the tile's MFMAs.
+#if !DIRECT_A
+#if RAW_A
+    u32x4 sa[A_PER_THREAD];
+#else
+    raw_a_t sa[A_PER_THREAD][SPLIT_A];
+#endif
+#endif
+#if !DIRECT_B
+#if RAW_B
+    u32x4 sb[B_PER_THREAD];
+#else
+    raw_b_t sb[B_PER_THREAD][SPLIT_B];
+#endif
+#endif
     auto stage_load = [&](u32 kt) {
-        const u32 k0 = k_tile(kt) * BK;
+        const u32 k0 = k_tile(kt) * BK; (void)k0;
+#if !DIRECT_A
 #pragma unroll
         for (int i = 0; i < A_PER_THREAD; i++) {
             const u32 idx = tid + i * NTHREADS;
             const u32 row = idx / A_CHUNKS, kc = idx % A_CHUNKS;
+#if RAW_A
             sa[i] = fetch_a(FETCH_A_ARGS bz, m0 + row, k0 + kc * EPC);
+#else
+            fetch_a_load(FETCH_A_ARGS bz, m0 + row, k0 + kc * EPC, sa[i]);
+#endif
         }
+#endif
+#if !DIRECT_B
 #pragma unroll
         for (int i = 0; i < B_PER_THREAD; i++) {
             const u32 idx = tid + i * NTHREADS;
             const u32 krow = idx / B_CHUNKS, nc = idx % B_CHUNKS;
+#if RAW_B
             sb[i] = fetch_b(FETCH_B_ARGS bz, k0 + krow, n0 + nc * EPC);
+#else
+            fetch_b_load(FETCH_B_ARGS bz, k0 + krow, n0 + nc * EPC, sb[i]);
+#endif
         }
+#endif
     };
-    auto stage_store = [&](u32 buf) {
+    auto stage_store = [&](u32 kt, u32 buf) {
+        const u32 k0 = k_tile(kt) * BK; (void)k0;
         unsigned char* la = lds + buf * STAGE_BYTES;
         unsigned char* lb = la + A_TILE_BYTES;
+        (void)la; (void)lb;
+#if !DIRECT_A
 #pragma unroll
         for (int i = 0; i < A_PER_THREAD; i++) {
             const u32 idx = tid + i * NTHREADS;
-            *(u32x4*)(la + a_off(idx / A_CHUNKS, idx % A_CHUNKS)) = sa[i];
+            const u32 row = idx / A_CHUNKS, kc = idx % A_CHUNKS;
+#if RAW_A
+            *(u32x4*)(la + a_off(row, kc)) = sa[i];
+#else
+            *(u32x4*)(la + a_off(row, kc)) = fetch_a_eval(FETCH_A_ARGS bz, m0 + row, k0 + kc * EPC, sa[i]);
+#endif
         }
+#endif
+#if !DIRECT_B
 #pragma unroll
         for (int i = 0; i < B_PER_THREAD; i++) {
             const u32 idx = tid + i * NTHREADS;
-            *(u32x4*)(lb + b_chunk_off(idx / B_CHUNKS, idx % B_CHUNKS)) = sb[i];
+            const u32 krow = idx / B_CHUNKS, nc = idx % B_CHUNKS;
+#if RAW_B
+            *(u32x4*)(lb + b_chunk_off(krow, nc)) = sb[i];
+#else
+            *(u32x4*)(lb + b_chunk_off(krow, nc)) = fetch_b_eval(FETCH_B_ARGS bz, k0 + krow, n0 + nc * EPC, sb[i]);
+#endif
         }
+#endif
     };
     const WavePos wpos = {lane, wave, wave_m, wave_n};
 
-#if DIRECT_LOADS
 /* s_waitcnt immediate: vmcnt lives in bits [3:0] and [15:14] */
 #define WAITCNT_VM(n) ((((n) & 15) | (((n) >> 4) << 14)))
+#if DIRECT_LOADS
     const bf16_t* const ga0 = (const bf16_t*)DIRECT_A_PTR + ((size_t)bz * GM + m0) * GK;
     const bf16_t* const gb0 = (const bf16_t*)DIRECT_B_PTR + (size_t)bz * GK * GN + n0;
     // NSTAGES-deep ring of LDS stages: tile kt + NSTAGES - 1 is requested while tile kt is multiplied, so a
@@ -305,6 +349,11 @@ void fused_matmul(KERNEL_PARAMS) {
             for (int i = 0; i < A_DPW + B_DPW; i++)
                 direct_issue(lds + st * STAGE_BYTES, ga0 + k_tile(st) * BK, gb0 + (size_t)(k_tile(st) * BK) * GN, wpos, i);
         }
+#endif
+#if STAGED
+    stage_load(0);
+    stage_store(0, 0);
+#endif
 #if GEMM_TIMING
     unsigned long long t_load = 0, t_compute = 0, t_wait = 0, t_barrier = 0, t0, t1;
 #define TICK(var) t1 = __builtin_readcyclecounter(); var += t1 - t0; t0 = t1;
@@ -314,20 +363,37 @@ void fused_matmul(KERNEL_PARAMS) {
 #define TICK(var)
 #endif
     for (u32 kt = 0; kt < KT; kt++) {
+#if DIRECT_LOADS
         // tile kt must have landed; up to NSTAGES - 2 younger tiles may still be in flight
         const u32 younger = KT - 1 - kt < NSTAGES - 2 ? KT - 1 - kt : NSTAGES - 2;
         if (younger >= 3) __builtin_amdgcn_s_waitcnt(0x0F70 | WAITCNT_VM(3 * (A_DPW + B_DPW)));
         else if (younger == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | WAITCNT_VM(2 * (A_DPW + B_DPW)));
         else if (younger == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | WAITCNT_VM(A_DPW + B_DPW));
         else __builtin_amdgcn_s_waitcnt(0x0F70);
+#endif
         TICK(t_wait)
+        // every wave's share of tile kt is in LDS (direct loads waited for above, staged stores made before the
+        // barrier) and nobody still reads the stage that this iteration refills
         __syncthreads();
         TICK(t_barrier)
         const u32 next = kt + NSTAGES - 1;
         const bool more = next < KT;
+#if STAGED
+        // The next tile's global loads are issued before any MFMA of this tile and consumed after the last one.
+        if (more) stage_load(next);
+        STAGE_SCHED_BARRIER
+#endif
+#if DIRECT_LOADS
         const u32 knext = more ? k_tile(next) * BK : 0u;
         direct_tile(lds + (kt % NSTAGES) * STAGE_BYTES, lds + (next % NSTAGES) * STAGE_BYTES, ga0 + knext,
                     gb0 + (size_t)knext * GN, more, acc, wpos);
+#else
+        compute_tile(lds + (kt % NSTAGES) * STAGE_BYTES, acc, wpos, [](int) {});
+#endif
+#if STAGED
+        STAGE_SCHED_BARRIER
+        if (more) stage_store(next, next % NSTAGES);
+#endif
         __builtin_amdgcn_sched_barrier(0);
         TICK(t_compute)
     }
@@ -340,21 +406,6 @@ void fused_matmul(KERNEL_PARAMS) {
     }
     __syncthreads();
     if (blockIdx.x == 0) return;
-#endif
-#else
-    stage_load(0);
-    stage_store(0);
-    __syncthreads();
-    for (u32 kt = 0; kt < KT; kt++) {
-        const bool more = kt + 1 < KT;
-        // The next tile's global loads are issued before any MFMA of this tile and consumed after the last one.
-        if (more) stage_load(kt + 1);
-        STAGE_SCHED_BARRIER
-        compute_tile(lds + (kt & 1) * STAGE_BYTES, acc, wpos, [](int) {});
-        STAGE_SCHED_BARRIER
-        if (more) stage_store((kt + 1) & 1);
-        __syncthreads();
-    }
 #endif
 
     // ---- epilogue: accumulators -> wave-private LDS strip -> row-major NV-wide vectors -----------------------
@@ -398,16 +449,21 @@ bool is_raw_copy(const tp::Program& p, int root, int mma_dtype) {
     return e.access.stride == ir::packed_strides(p.dims);
 }
 
-// A __device__ function that evaluates an operand program for NV consecutive columns at (b, row, col).
-std::string emit_operand_fn(const tp::Program& p, int root, const std::string& name, int nv) {
+// The same program in two halves: `<name>_load` issues the full-vector loads into a Raw struct, `<name>_eval`
+// turns them into the operand's NV values. A kernel calls the first before a tile's MFMAs and the second after.
+std::string emit_operand_split(const tp::Program& p, int root, const std::string& name, int nv) {
     std::ostringstream s;
-    s << "__device__ __forceinline__ void " << name << "(";
-    for (size_t a = 0; a < p.args.size(); a++) s << "const " << tp::c_type(p.args[a].dtype) << "* __restrict__ a" << a << ", ";
-    s << "u32 cB0, u32 m, u32 n0, float* out) {\n(void)cB0;\n";
+    std::string sig;
+    for (size_t a = 0; a < p.args.size(); a++) sig += std::string("const ") + tp::c_type(p.args[a].dtype) + "* __restrict__ a" + std::to_string(a) + ", ";
+    s << "struct Raw_" << name << " {\n" << tp::emit_raw_members(p, nv) << "};\n";
     tp::EmitCtx cx;
     cx.nv = nv;
-    s << tp::emit_exprs(p, cx);
-    s << "#pragma unroll\nfor (int k = 0; k < " << nv << "; k++) out[k] = e" << root << "[k];\n}\n";
+    cx.phase = 1;
+    s << "__device__ __forceinline__ void " << name << "_load(" << sig << "u32 cB0, u32 m, u32 n0, Raw_" << name << "& R) {\n(void)cB0; (void)m; (void)n0; (void)R;\n"
+      << tp::emit_exprs(p, cx) << "}\n";
+    cx.phase = 2;
+    s << "__device__ __forceinline__ void " << name << "_eval(" << sig << "u32 cB0, u32 m, u32 n0, const Raw_" << name << "& R, float* out) {\n(void)cB0; (void)R;\n"
+      << tp::emit_exprs(p, cx) << "#pragma unroll\nfor (int k = 0; k < " << nv << "; k++) out[k] = e" << root << "[k];\n}\n";
     return s.str();
 }
 
@@ -484,7 +540,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     Tile t;
     const bool raw_a0 = is_raw_copy(pr.op_a, pr.root_a, pr.mma_dtype) && pr.K % epc == 0;
     const bool raw_b0 = is_raw_copy(pr.op_b, pr.root_b, pr.mma_dtype) && pr.N % epc == 0;
-    bool want_direct = raw_a0 && raw_b0 && !f32 && !getenv("HELIUM_HIP_GEMM_NO_DIRECT");
+    const bool want_direct = !f32 && !getenv("HELIUM_HIP_GEMM_NO_DIRECT");
     if (const char* env = getenv("HELIUM_HIP_GEMM_TILE")) {
         int v[6] = {256, 256, 64, 2, 4, 2};
         int n = sscanf(env, "%d,%d,%d,%d,%d,%d", &v[0], &v[1], &v[2], &v[3], &v[4], &v[5]);
@@ -509,10 +565,15 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     const bool raw_a = raw_a0, raw_b = raw_b0;
     const int nva = std::min(epc, tp::pick_nv(pr.op_a, 16)), nvb = std::min(epc, tp::pick_nv(pr.op_b, 16));
     // Direct global->LDS loads need unpredicated, unmodified 16-byte chunks: raw operands and full tiles everywhere.
-    const bool direct = want_direct && raw_a && raw_b && pr.M % t.bm == 0 && pr.N % t.bn == 0 && pr.K % t.bk == 0 &&
-                        (t.bm * t.bk * 2 / 1024) % (threads / 64) == 0 && (t.bk * t.bn * 2 / 1024) % (threads / 64) == 0 &&
-                        64 % (t.bn / 8) == 0;
-    if (!direct) t.stages = 2;
+    // Each operand qualifies on its own; the other one then goes through registers.
+    const bool direct_a = want_direct && raw_a && pr.M % t.bm == 0 && pr.K % t.bk == 0 && (t.bm * t.bk * 2 / 1024) % (threads / 64) == 0 &&
+                          !getenv("HELIUM_HIP_GEMM_NO_DIRECT_A");
+    const bool direct_b = want_direct && raw_b && pr.N % t.bn == 0 && pr.K % t.bk == 0 && (t.bk * t.bn * 2 / 1024) % (threads / 64) == 0 &&
+                          64 % (t.bn / 8) == 0 && !getenv("HELIUM_HIP_GEMM_NO_DIRECT_B");
+    if (!(direct_a && direct_b)) t.stages = 2;  // register staging is double-buffered only
+    // All direct loads of the next tile are issued at the start of a tile's MFMAs (the round trip needs the whole
+    // tile to hide); HELIUM_HIP_GEMM_ISSUE=0 spreads them over the k-steps instead.
+    const bool issue_front = getenv("HELIUM_HIP_GEMM_ISSUE") ? atoi(getenv("HELIUM_HIP_GEMM_ISSUE")) != 0 : true;
     int nve = tp::pick_nv(pr.epi, 32);
     while (nve > 1 && ((32 * wtn) % (64 * nve) != 0)) nve /= 2;
     nve = std::min(nve, 8);
@@ -527,11 +588,13 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     s << "#define BM " << t.bm << "\n#define BN " << t.bn << "\n#define BK " << t.bk << "\n#define WAVES_M " << t.wm
       << "\n#define WAVES_N " << t.wn << "\n#define NSTAGES " << t.stages << "\n#define NVE " << nve << "\n#define MMA_BF16 " << (pr.mma_dtype == HE_BF16 ? 1 : 0) << "\n#define MMA_F32 " << (f32 ? 1 : 0)
       << "\n#define STAGGER_EXPR " << (getenv("HELIUM_HIP_GEMM_STAGGER") ? getenv("HELIUM_HIP_GEMM_STAGGER") : "0u")
-      << "\n#define ISSUE_FRONT " << (getenv("HELIUM_HIP_GEMM_ISSUE") ? atoi(getenv("HELIUM_HIP_GEMM_ISSUE")) : 0)
+      << "\n#define ISSUE_FRONT " << (issue_front ? 1 : 0)
       << "\n#define GEMM_SKIP " << (getenv("HELIUM_HIP_GEMM_SKIP") ? atoi(getenv("HELIUM_HIP_GEMM_SKIP")) : 0)
       << "\n#define GEMM_TIMING " << (getenv("HELIUM_HIP_GEMM_TIMING") ? 1 : 0) << "\n#define GEMM_TIMING_PTR p" << (pr.args.size() - 1)
-      << "\n#define DIRECT_LOADS " << (direct ? 1 : 0) << "\n#define DIRECT_A_PTR p" << (direct ? pr.map_a[0] : 0)
-      << "\n#define DIRECT_B_PTR p" << (direct ? pr.map_b[0] : 0) << "\n#define STAGE_SCHED_BARRIER "
+      << "\n#define DIRECT_A " << (direct_a ? 1 : 0) << "\n#define DIRECT_B " << (direct_b ? 1 : 0)
+      << "\n#define DIRECT_LOADS (DIRECT_A || DIRECT_B)\n#define STAGED (!DIRECT_A || !DIRECT_B)"
+      << "\n#define DIRECT_A_PTR p" << (direct_a ? pr.map_a[0] : 0)
+      << "\n#define DIRECT_B_PTR p" << (direct_b ? pr.map_b[0] : 0) << "\n#define STAGE_SCHED_BARRIER "
       << (getenv("HELIUM_HIP_GEMM_PIN") ? "__builtin_amdgcn_sched_barrier(0);" : "") << "\n#define A_SWZ_SHIFT " << (getenv("HELIUM_HIP_GEMM_ASWZ") ? atoi(getenv("HELIUM_HIP_GEMM_ASWZ")) : (t.bk == 64 ? 1 : 2)) << "\n";
 
     s << kGemmHelpers;
@@ -553,20 +616,31 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         }
         std::string W = which;
         s << "#define FETCH_" << (W == "a" ? "A" : "B") << "_ARGS " << args.str() << "\n";
-        if (!raw) s << emit_operand_fn(p, root, "operand_" + W, nv);
-        s << "__device__ __forceinline__ u32x4 fetch_" << W << "(" << params.str() << "u32 b, u32 row, u32 col) {\n";
-        if (raw && aligned) {
-            // every tile is full: no predication on the operand loads
-            s << "return *(const u32x4*)(q0 + ((size_t)b * " << rows << " + row) * " << cols << " + col);\n}\n";
-        } else if (raw) {
-            s << "u32x4 v = {0u, 0u, 0u, 0u};\nif (row < " << rows << " && col < " << cols << ") v = *(const u32x4*)(q0 + ((size_t)b * "
-              << rows << " + row) * " << cols << " + col);\nreturn v;\n}\n";
-        } else {
-            s << "float v[" << epc << "];\n#pragma unroll\nfor (int j = 0; j < " << epc << "; j += " << nv << ") {\nif (row < " << rows << " && col + j < " << cols
-              << ") operand_" << W << "(";
-            for (size_t a = 0; a < p.args.size(); a++) s << "q" << a << ", ";
-            s << "b, row, col + j, v + j);\nelse {\n#pragma unroll\nfor (int k = 0; k < " << nv << "; k++) v[j + k] = 0.0f; }\n}\nreturn pack_chunk(v);\n}\n";
+        const std::string X = (W == "a" ? "A" : "B");
+        s << "#define RAW_" << X << " " << (raw ? 1 : 0) << "\n#define SPLIT_" << X << " " << epc / nv << "\n";
+        if (raw) {
+            s << "__device__ __forceinline__ u32x4 fetch_" << W << "(" << params.str() << "u32 b, u32 row, u32 col) {\n";
+            if (aligned)  // every tile is full: no predication on the operand loads
+                s << "return *(const u32x4*)(q0 + ((size_t)b * " << rows << " + row) * " << cols << " + col);\n}\n";
+            else
+                s << "u32x4 v = {0u, 0u, 0u, 0u};\nif (row < " << rows << " && col < " << cols << ") v = *(const u32x4*)(q0 + ((size_t)b * "
+                  << rows << " + row) * " << cols << " + col);\nreturn v;\n}\n";
+            return;
         }
+        // Mainloop-fused operand: loads first (fetch_x_load), arithmetic and rounding to the multiplicand type later
+        // (fetch_x_eval), so that the memory latency is covered by the MFMAs in between.
+        s << emit_operand_split(p, root, "operand_" + W, nv);
+        std::string pass;
+        for (size_t a = 0; a < p.args.size(); a++) pass += "q" + std::to_string(a) + ", ";
+        const std::string guard = aligned ? "" : "if (row < " + std::string(rows) + " && col + j < " + cols + ") ";
+        s << "typedef Raw_operand_" << W << " raw_" << W << "_t;\n";
+        s << "__device__ __forceinline__ void fetch_" << W << "_load(" << params.str() << "u32 b, u32 row, u32 col, raw_" << W << "_t (&R)[" << epc / nv << "]) {\n"
+          << "#pragma unroll\nfor (int j = 0; j < " << epc << "; j += " << nv << ") " << guard << "operand_" << W << "_load(" << pass << "b, row, col + j, R[j / " << nv << "]);\n}\n";
+        s << "__device__ __forceinline__ u32x4 fetch_" << W << "_eval(" << params.str() << "u32 b, u32 row, u32 col, const raw_" << W << "_t (&R)[" << epc / nv << "]) {\n"
+          << "float v[" << epc << "];\n#pragma unroll\nfor (int j = 0; j < " << epc << "; j += " << nv << ") {\n";
+        if (aligned) s << "operand_" << W << "_eval(" << pass << "b, row, col + j, R[j / " << nv << "], v + j);\n}\n";
+        else s << guard << "operand_" << W << "_eval(" << pass << "b, row, col + j, R[j / " << nv << "], v + j);\nelse {\n#pragma unroll\nfor (int k = 0; k < " << nv << "; k++) v[j + k] = 0.0f; }\n}\n";
+        s << "return pack_chunk(v);\n}\n";
     };
     emit_fetch("a", pr.op_a, pr.root_a, pr.map_a, raw_a, nva, "GM", "GK", pr.M % t.bm == 0 && pr.K % t.bk == 0);
     emit_fetch("b", pr.op_b, pr.root_b, pr.map_b, raw_b, nvb, "GK", "GN", pr.K % t.bk == 0 && pr.N % t.bn == 0);
@@ -663,7 +737,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         }
         splice("SCHED_HINT", h.str());
         std::ostringstream plan;
-        const int mode = getenv("HELIUM_HIP_GEMM_PLAN") ? atoi(getenv("HELIUM_HIP_GEMM_PLAN")) : 2;
+        const int mode = getenv("HELIUM_HIP_GEMM_PLAN") ? atoi(getenv("HELIUM_HIP_GEMM_PLAN")) : 3;
         const int mb = t.bm / t.wm / 32, nb = t.bn / t.wn / 32, kk_steps = t.bk / (2 * epc);
         const int nr = f32 ? mb + 4 * nb : mb + 2 * nb, nm = f32 ? 4 * mb * nb : mb * nb;
         if (mode == 1) {
@@ -673,13 +747,32 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
                 if (kk + 1 < kk_steps) plan << "__builtin_amdgcn_sched_group_barrier(0x100, " << nr << ", 0);\n";
                 plan << "__builtin_amdgcn_sched_group_barrier(0x008, " << nm << ", 0);\n";
             }
+        } else if (mode == 3 || mode == 4) {
+            // reads of step kk+1 go between the first MFMAs of step kk (two per MFMA in mode 3, all before the second
+            // MFMA in mode 4), so that they have landed when the step ends: while direct loads are in flight the
+            // compiler can only wait for *all* outstanding LDS reads at once
+            plan << "__builtin_amdgcn_sched_group_barrier(0x100, " << nr << ", 0);\n";
+            const int waves = threads / 64;
+            const int dl = ((direct_a ? t.bm * t.bk * 2 / 1024 : 0) + (direct_b ? t.bk * t.bn * 2 / 1024 : 0)) / waves;
+            const int per = issue_front ? dl : (dl + kk_steps - 1) / kk_steps;
+            const int rate = mode == 3 ? 2 : nr;
+            for (int kk = 0; kk < kk_steps; kk++) {
+                int issue = std::max(0, std::min(per, dl - kk * per));
+                if (issue) plan << "__builtin_amdgcn_sched_group_barrier(0x020, " << issue << ", 0);\n";
+                int left = kk + 1 < kk_steps ? nr : 0;
+                for (int m = 0; m < nm; m++) {
+                    plan << "__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);\n";
+                    const int r = std::min(left, rate);
+                    if (r) plan << "__builtin_amdgcn_sched_group_barrier(0x100, " << r << ", 0);\n";
+                    left -= r;
+                }
+            }
         } else if (mode == 2) {
             // reads of step kk+1 are spread between the MFMAs of step kk
             plan << "__builtin_amdgcn_sched_group_barrier(0x100, " << nr << ", 0);\n";
             const int waves = threads / 64;
-            const int dl = direct ? (t.bm * t.bk * 2 / 1024 + t.bk * t.bn * 2 / 1024) / waves : 0;
-            const bool front = getenv("HELIUM_HIP_GEMM_ISSUE") && atoi(getenv("HELIUM_HIP_GEMM_ISSUE"));
-            const int per = front ? dl : (dl + kk_steps - 1) / kk_steps;
+            const int dl = ((direct_a ? t.bm * t.bk * 2 / 1024 : 0) + (direct_b ? t.bk * t.bn * 2 / 1024 : 0)) / waves;
+            const int per = issue_front ? dl : (dl + kk_steps - 1) / kk_steps;
             for (int kk = 0; kk < kk_steps; kk++) {
                 int issue = std::max(0, std::min(per, dl - kk * per));
                 if (issue) plan << "__builtin_amdgcn_sched_group_barrier(0x020, " << issue << ", 0);\n";
@@ -708,9 +801,9 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     for (auto& o : pr.epi.outs)
         if (o.reduce) fills_.push_back({pr.map_e[o.arg], 0u});
     describe_ = strfmt("gemm [%lld,%lld,%lld]x[%lld] tile=%dx%dx%d stages=%d waves=%dx%d threads=%d grid=%ux%u rawA=%d rawB=%d NVA=%d NVB=%d NVE=%d "
-                       "direct=%d mma=%s epilogue_exprs=%zu outs=%zu",
+                       "direct=%d%d mma=%s epilogue_exprs=%zu outs=%zu",
                        (long long)pr.batch, (long long)pr.M, (long long)pr.K, (long long)pr.N, t.bm, t.bn, t.bk, t.stages, t.wm, t.wn, threads,
-                       grid_[0], grid_[1], (int)raw_a, (int)raw_b, nva, nvb, nve, (int)direct, dtype_name(pr.mma_dtype), pr.epi.exprs.size(),
+                       grid_[0], grid_[1], (int)raw_a, (int)raw_b, nva, nvb, nve, (int)direct_a, (int)direct_b, dtype_name(pr.mma_dtype), pr.epi.exprs.size(),
                        pr.epi.outs.size());
     kernel_.reset(new JitKernel(source_, "fused_matmul", {"-ffp-contract=fast", "-munsafe-fp-atomics"}));
 }

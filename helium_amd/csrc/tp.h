@@ -126,7 +126,12 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry);
 struct EmitCtx {
     int nv = 1;
     bool guard_vector_loads = false;  // when set, full-width loads are only legal if `vec_ok` is true
+    // 0: everything. 1: only the full-vector loads, left undecoded in members raw<expr id> of a struct named `R`.
+    // 2: everything else, reading those members. Splitting lets a kernel issue the loads long before it needs them.
+    int phase = 0;
 };
+// Members of the struct phase 1 fills: one native vector per full-vector Load of the program.
+std::string emit_raw_members(const Program& p, int nv);
 std::string emit_exprs(const Program& p, const EmitCtx& cx);
 // Largest vector width (elements) legal for every full-row access and store of the program.
 int pick_nv(const Program& p, int max_bytes);

@@ -57,6 +57,7 @@ CASES = [
     ("twelve_tiles_grouped_order", lambda: gemm_cases.plain(768, 260, 64), "128,128,64,2,2"),
     ("eight_waves_2x4", lambda: gemm_cases.bias_relu_colsum(140, 264, 72, mainloop=True), "128,256,64,2,4"),
     ("four_stage_ring_bk32", lambda: gemm_cases.plain(256, 256, 192), "256,256,32,2,4,4"),
+    ("mainloop_in_registers_b_direct", lambda: gemm_cases.bias_relu_colsum(256, 256, 128, mainloop=True), "128,128,64,2,2"),
     ("five_stage_ring_bk32", lambda: gemm_cases.plain(256, 256, 288), "256,256,32,2,4,5"),
     ("three_stage_ring_short_k", lambda: gemm_cases.plain(128, 256, 32), "128,128,32,2,2,3"),
     ("three_stage_ring_bk64", lambda: gemm_cases.bias_relu_colsum(128, 128, 320), "128,128,64,2,2,3"),
