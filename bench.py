@@ -2,7 +2,7 @@
 """Benchmark of the helium MI355X backend's hot path on ONE GPU.
 
 A "step" is one pass of the headline workload over one batch of synthetic, seeded input that is already
-resident in HBM when the timed region starts. Prints ONE JSON line (see README / DESIGN.md for the fields).
+resident in HBM when the timed region starts. Prints ONE JSON line.
 The other BASELINE workloads are measured in the same run and reported under "kernels".
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--only] [--no-cpu]

@@ -27,6 +27,9 @@ typedef unsigned int u32;
 typedef unsigned long long u64;
 typedef __bf16 bf16_t;
 typedef _Float16 f16_t;
+#ifndef TANH_RCP
+#define TANH_RCP(x) __builtin_amdgcn_rcpf(x)
+#endif
 template <class T, int N> struct Vec { typedef T type __attribute__((ext_vector_type(N))); };
 template <class T> struct Vec<T, 1> { typedef T type; };
 
@@ -127,6 +130,26 @@ template <int OP> __device__ __forceinline__ void atomic_red(float* addr, float 
         atomicAdd(addr, v);
     }
 }
+// tanh to within 2 ulp without branches (lanes of a wave rarely agree on which side of a branch they are):
+// x + x^3 P(x^2) below 1, 1 - 2 / (exp(2|x|) + 1) from there on; measured against double tanh over every float in
+// (0, 10] with exp off by one ulp either way the worst error is 1.21 ulp.
+__device__ __forceinline__ float tanh_2ulp(float x) {
+    const float ax = __builtin_fabsf(x);
+    const float u = ax * ax;
+    float p = __builtin_fmaf(u, -0.0003552270936779678f, 0.002289985306560993f);
+    p = __builtin_fmaf(u, p, -0.007930326275527477f);
+    p = __builtin_fmaf(u, p, 0.021475814282894135f);
+    p = __builtin_fmaf(u, p, -0.05387599393725395f);
+    p = __builtin_fmaf(u, p, 0.1333228200674057f);
+    p = __builtin_fmaf(u, p, -0.33333292603492737f);
+    const float small = __builtin_fmaf(ax * u, p, ax);
+    const float d = expf(2.0f * ax) + 1.0f;            // +inf for large |x|: the quotient is 0 and tanh is 1
+    float r = TANH_RCP(d);
+    r = __builtin_isinf(d) ? 0.0f : __builtin_fmaf(__builtin_fmaf(-d, r, 1.0f), r, r);  // one Newton step
+    const float big = __builtin_fmaf(-2.0f, r, 1.0f);
+    const float t = ax < 1.0f ? small : big;           // NaN falls through to `big`, which is NaN
+    return __builtin_copysignf(t, x);
+}
 __device__ __forceinline__ float fast_tanh(float x) {
     float t = __expf(2.0f * x);
     return 1.0f - __fdividef(2.0f, t + 1.0f);
@@ -153,7 +176,7 @@ static std::string unary_expr(const Expr& e, const std::string& x, bool fast) {
         case UOp::Tan: return (fast ? "__tanf(" : "tanf(") + x + ")";
         case UOp::Sigmoid:
             return fast ? "__fdividef(1.0f, 1.0f + __expf(-" + x + "))" : "1.0f / (1.0f + expf(-" + x + "))";
-        case UOp::Tanh: return (fast ? "fast_tanh(" : "tanhf(") + x + ")";
+        case UOp::Tanh: return (fast ? "fast_tanh(" : "tanh_2ulp(") + x + ")";
         case UOp::Relu: return "fmaxf(" + x + ", 0.0f)";
         case UOp::Sqrt: return (fast ? "__fsqrt_rn(" : "sqrtf(") + x + ")";
         case UOp::Log: return (fast ? "__logf(" : "logf(") + x + ")";
@@ -432,7 +455,10 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
     if (const char* env = getenv("HELIUM_HIP_POINTWISE_RPT")) {
         RPT = std::max(1, atoi(env));
     } else {
-        while (RPT < 16 && blocks1 / (RPT * 2) >= 2048) RPT *= 2;
+        // Blocks that end in per-column or scalar atomics are worth making tall: 32 rows per thread and about two
+        // blocks per CU measured 20% faster on a 4096^2 chain than 8 rows and eight blocks per CU.
+        const bool tall = any_col || any_scalar;
+        while (RPT < (tall ? 32 : 16) && blocks1 / (RPT * 2) >= (tall ? 512 : 2048)) RPT *= 2;
     }
     RPT = (int)std::min<int64_t>(RPT, std::max<int64_t>(1, gy1));
     const int TR = TY * RPT;
