@@ -21,6 +21,12 @@ _ffi._sig("he_plan_destroy", C.c_void_p)
 _ffi._sig("he_execute_graph", C.c_void_p, C.POINTER(C.c_uint32), C.POINTER(C.c_void_p), C.c_int, C.POINTER(C.c_uint32),
           C.POINTER(C.c_void_p), C.c_int, C.POINTER(C.c_int))
 _ffi._sig("he_backend_stats", C.POINTER(C.c_uint64))
+_ffi._sig("he_backend_set_option", C.c_int, C.c_int64)
+OPT_FUSE_MATMUL_EPILOGUE = 0
+
+
+def set_option(option, value):
+    check(lib.he_backend_set_option(option, int(value)))
 
 
 class Tensor:

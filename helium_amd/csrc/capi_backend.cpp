@@ -100,6 +100,15 @@ int he_execute_graph(he_graph_t graph, const uint32_t* input_nodes, const he_ten
     });
 }
 
+int he_backend_set_option(int option, int64_t value) {
+    return he::guard([&] {
+        switch (option) {
+            case HE_OPT_FUSE_MATMUL_EPILOGUE: he::plan::set_fuse_matmul_epilogue(value != 0); break;
+            default: he::fail(HE_ERR_INVALID, "unknown backend option");
+        }
+    });
+}
+
 int he_backend_stats(uint64_t stats[9]) {
     return he::guard([&] {
         stats[0] = g_last_stats.steps;

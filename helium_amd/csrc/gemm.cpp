@@ -495,7 +495,12 @@ GemmProblem gemm_problem_from_fusion(const fir::OpGraph& g) {
         }
     pr.mma_dtype = all_f16 ? HE_F16 : all_f32 ? HE_F32 : HE_BF16;
 
-    // Kernel arguments: every distinct producer in id order, then every output in leaf order.
+    assemble_gemm_args(pr);
+    return pr;
+}
+
+void assemble_gemm_args(GemmProblem& pr) {
+    // Kernel arguments: every distinct input in id order, then every output in leaf order.
     std::vector<tp::Arg> inputs, outputs;
     auto add_input = [&](const tp::Arg& a) {
         for (auto& x : inputs)
@@ -524,7 +529,16 @@ GemmProblem gemm_problem_from_fusion(const fir::OpGraph& g) {
     pr.map_a = map_of(pr.op_a);
     pr.map_b = map_of(pr.op_b);
     pr.map_e = map_of(pr.epi);
-    return pr;
+}
+
+void validate_gemm_epilogue(const tp::Program& epi) {
+    HE_REQUIRE(epi.dims.size() <= 3, HE_ERR_UNSUPPORTED, "GEMM epilogues run over [batch, rows, cols]");
+    HE_REQUIRE(!epi.outs.empty(), HE_ERR_UNSUPPORTED, "GEMM fusion without an output");
+    for (auto& o : epi.outs) {
+        HE_REQUIRE(epi.exprs[o.expr].cls == tp::Cls::F, HE_ERR_UNSUPPORTED, "GEMM epilogues store float values");
+        if (o.reduce) HE_REQUIRE(o.rop == tp::ROp::Sum, HE_ERR_UNSUPPORTED, "GEMM epilogues reduce with Sum only");
+        else HE_REQUIRE(o.dtype == HE_F32 || o.dtype == HE_BF16 || o.dtype == HE_F16, HE_ERR_UNSUPPORTED, "GEMM epilogues store float tensors");
+    }
 }
 
 GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
@@ -535,6 +549,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
                HE_ERR_INVALID, "GEMM too large");
     HE_REQUIRE(pr.mma_dtype == HE_BF16 || pr.mma_dtype == HE_F16 || pr.mma_dtype == HE_F32, HE_ERR_UNSUPPORTED,
                "unsupported multiplicand type");
+    validate_gemm_epilogue(pr.epi);
     const bool f32 = pr.mma_dtype == HE_F32;
     const int epc = f32 ? 4 : 8;  // multiplicands per 16-byte chunk
     Tile t;

@@ -51,6 +51,10 @@ struct GemmProblem {
     std::vector<int> map_a, map_b, map_e;  // program argument -> kernel argument
 };
 GemmProblem gemm_problem_from_fusion(const fir::OpGraph& g);
+// Fills args / map_a / map_b / map_e from the three programs: distinct inputs in node order, then outputs.
+void assemble_gemm_args(GemmProblem& pr);
+// Throws HE_ERR_UNSUPPORTED for an epilogue program the GEMM kernel cannot run.
+void validate_gemm_epilogue(const tp::Program& epi);
 
 class GemmKernel : public KernelBase {
 public:

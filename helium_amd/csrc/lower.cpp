@@ -129,7 +129,9 @@ uint32_t f32_bits(float f) {
 // ---------------------------------------------------------------------------------------------------------
 class PointwiseLowering {
 public:
-    explicit PointwiseLowering(const ir::OpSubgraph& sg) : sg_(sg), g_(*sg.graph()) {}
+    // With `anchor` set the subgraph is a Matmul plus the ops that follow it: the program is the epilogue, iterates
+    // over the Matmul's output and reads the anchor's value as the accumulator.
+    explicit PointwiseLowering(const ir::OpSubgraph& sg, ir::NodeId anchor = ir::kNoNode) : sg_(sg), g_(*sg.graph()), anchor_(anchor) {}
 
     Program run() {
         HE_REQUIRE(!sg_.leafs().empty(), HE_ERR_INVALID, "pointwise subgraph has no output");
@@ -138,6 +140,10 @@ public:
         ir::NodeId first = sg_.leafs()[0];
         const ir::Node& fn = g_.get(first);
         p_.dims = fn.op.kind == ir::OpKind::Reduce ? g_.get(fn.op.inputs[0]).desc.shape : fn.desc.shape;
+        if (anchor_ != ir::kNoNode) {
+            p_.dims = g_.get(anchor_).desc.shape;
+            p_.fast_math = true;
+        }
         if (p_.dims.empty()) p_.dims = {1};
         const int64_t numel = ir::num_elements(p_.dims);
 
@@ -183,10 +189,29 @@ public:
             }
             p_.outs.push_back(o);
         }
+        if (anchor_ != ir::kNoNode) drop_unused_inputs();
         return std::move(p_);
     }
 
 private:
+    // The Matmul's own operands are inputs of the subgraph but not of the epilogue unless an epilogue op reads them.
+    void drop_unused_inputs() {
+        std::vector<char> used(p_.args.size(), 0);
+        for (auto& e : p_.exprs)
+            if (e.kind == Expr::Load) used[e.access.arg] = 1;
+        std::vector<int> remap(p_.args.size(), -1);
+        std::vector<Arg> kept;
+        for (size_t a = 0; a < p_.args.size(); a++)
+            if (p_.args[a].is_output || used[a]) {
+                remap[a] = (int)kept.size();
+                kept.push_back(p_.args[a]);
+            }
+        for (auto& e : p_.exprs)
+            if (e.kind == Expr::Load) e.access.arg = remap[e.access.arg];
+        for (auto& o : p_.outs) o.arg = remap[o.arg];
+        p_.args = kept;
+    }
+
     int push(Expr e) {
         p_.exprs.push_back(std::move(e));
         return (int)p_.exprs.size() - 1;
@@ -214,6 +239,17 @@ private:
         }
         HE_REQUIRE(sg_.contains(node) && n.kind == ir::Node::Intermediate, HE_ERR_INVALID,
                    "node %u is outside the subgraph", node);
+        if (node == anchor_) {
+            // the accumulator exists only at the coordinate a thread owns: the path from the outputs back to the
+            // Matmul must not move or repeat elements
+            HE_REQUIRE(mp.chain.empty() && mp.w == ir::packed_strides(p_.dims), HE_ERR_UNSUPPORTED,
+                       "the epilogue reads the Matmul result through a transposition or broadcast");
+            Expr e;
+            e.kind = Expr::Acc;
+            e.cls = Cls::F;
+            p_.acc_expr = push(e);
+            return p_.acc_expr;
+        }
         const ir::Op& op = n.op;
         auto in_shape = [&](size_t i) -> const Shape& { return g_.get(op.inputs[i]).desc.shape; };
         switch (op.kind) {
@@ -303,6 +339,7 @@ private:
     };
     const ir::OpSubgraph& sg_;
     const ir::OpGraph& g_;
+    ir::NodeId anchor_;
     Program p_;
     std::map<ir::NodeId, int> input_arg_;
     std::vector<Memo> memo_;
@@ -585,6 +622,7 @@ bool pointwise_supports(const ir::OpSubgraph& sg) {
 }
 
 Program lower_pointwise(const ir::OpSubgraph& sg) { return PointwiseLowering(sg).run(); }
+Program lower_ir_epilogue(const ir::OpSubgraph& sg, ir::NodeId anchor) { return PointwiseLowering(sg, anchor).run(); }
 Program lower_aux(const fir::OpGraph& g) {
     HE_REQUIRE(g.anchor() == fir::kNoOpNode, HE_ERR_INVALID, "an auxiliary fusion holds no Matmul");
     return FusionLowering(g, fir::kNoOpNode).run();

@@ -1,5 +1,6 @@
 #include "plan.h"
 
+#include <atomic>
 #include <future>
 #include <list>
 #include <map>
@@ -42,7 +43,26 @@ bool enumerate_swaps(const ir::OpSubgraph& sg, std::vector<std::pair<int, int>>*
     return true;
 }
 
+namespace {
+std::atomic<bool> g_fuse_matmul_epilogue{true};
+}
+void set_fuse_matmul_epilogue(bool on) { g_fuse_matmul_epilogue.store(on); }
+bool fuse_matmul_epilogue() { return g_fuse_matmul_epilogue.load(); }
+
 bool Instr::can_fuse_with(const Instr& next) const {
+    const bool gemm_and_pointwise = (kind_ == InstrKind::Gemm && next.kind_ == InstrKind::Pointwise) ||
+                                    (kind_ == InstrKind::Pointwise && next.kind_ == InstrKind::Gemm);
+    if (gemm_and_pointwise && fuse_matmul_epilogue()) {
+        // Beyond the reference, whose matmul instruction never fuses: pointwise and reduce ops that follow a Matmul
+        // join it when they can run on the accumulators as the fused GEMM's epilogue; so do the ops that only prepare
+        // epilogue operands (a bias broadcast), whichever of the two the greedy pass visits first.
+        try {
+            (void)gemm_problem_from_ir(sg_.merge_with(next.sg_));
+            return true;
+        } catch (const Error&) {
+            return false;
+        }
+    }
     if (kind_ != next.kind_) return false;  // only instructions of one kind fuse (instr.rs:71-84)
     switch (kind_) {
         case InstrKind::Gemm: return false;  // the reference's matmul instruction never fuses (cudnn_graph.rs:319-321)
@@ -55,7 +75,10 @@ bool Instr::can_fuse_with(const Instr& next) const {
     return false;
 }
 
-Instr Instr::fuse_with(const Instr& next) const { return Instr(kind_, sg_.merge_with(next.sg_)); }
+Instr Instr::fuse_with(const Instr& next) const {
+    const InstrKind kind = (kind_ == InstrKind::Gemm || next.kind_ == InstrKind::Gemm) ? InstrKind::Gemm : kind_;
+    return Instr(kind, sg_.merge_with(next.sg_));
+}
 
 Instr make_instr_for_op(const std::shared_ptr<const ir::OpGraph>& g, NodeId node) {
     const ir::Node& n = g->get(node);
@@ -374,6 +397,7 @@ std::string Plan::describe() const {
 // ---------------------------------------------------------------------------------------------------------
 namespace {
 struct CacheEntry {
+    bool fused_epilogues;
     uint64_t hash;
     std::shared_ptr<const ir::OpGraph> graph;
     std::shared_ptr<const Plan> plan;
@@ -389,7 +413,7 @@ std::shared_ptr<const Plan> generate_cached_plan(const std::shared_ptr<const ir:
     {
         std::lock_guard<std::mutex> lk(g_plan_mu);
         for (auto it = g_plans.begin(); it != g_plans.end(); ++it)
-            if (it->hash == h && it->graph->structurally_equal(*g)) {
+            if (it->hash == h && it->fused_epilogues == fuse_matmul_epilogue() && it->graph->structurally_equal(*g)) {
                 g_plans.splice(g_plans.begin(), g_plans, it);
                 g_plan_hits++;
                 return g_plans.front().plan;
@@ -399,7 +423,7 @@ std::shared_ptr<const Plan> generate_cached_plan(const std::shared_ptr<const ir:
     // The cached plan refers to the graph object it was generated from; node ids are equal by construction.
     std::shared_ptr<const Plan> plan = generate_plan(g);
     std::lock_guard<std::mutex> lk(g_plan_mu);
-    g_plans.push_front({h, g, plan});
+    g_plans.push_front({fuse_matmul_epilogue(), h, g, plan});
     if (g_plans.size() > kPlanCacheCapacity) g_plans.pop_back();
     return plan;
 }
@@ -422,8 +446,6 @@ GemmProblem gemm_problem_from_ir(const ir::OpSubgraph& sg) {
             mm = n;
         }
     HE_REQUIRE(mm != ir::kNoNode, HE_ERR_UNSUPPORTED, "no Matmul in the subgraph");  // find_matmul (matmul.rs:222-233)
-    HE_REQUIRE(sg.nodes().size() == 1, HE_ERR_UNSUPPORTED,
-               "mainloop / epilogue fusion of helium-ir ops around a Matmul is expressed through the fusion IR");
     const ir::Op& op = g.get(mm).op;
     const ir::Descriptor &da = g.get(op.inputs[0]).desc, &db = g.get(op.inputs[1]).desc, &dc = g.get(mm).desc;
     HE_REQUIRE(da.shape.size() >= 2 && da.shape.size() == db.shape.size(), HE_ERR_UNSUPPORTED, "matmul operand ranks differ");
@@ -464,28 +486,29 @@ GemmProblem gemm_problem_from_ir(const ir::OpSubgraph& sg) {
     operand(pr.op_a, da, op.inputs[0], pr.M, pr.K);
     operand(pr.op_b, db, op.inputs[1], pr.K, pr.N);
     pr.root_a = pr.root_b = 0;
-    pr.epi.dims = {batch, pr.M, pr.N};
-    pr.epi.fast_math = true;
-    tp::Expr acc;
-    acc.kind = tp::Expr::Acc;
-    acc.cls = tp::Cls::F;
-    pr.epi.exprs.push_back(acc);
-    pr.epi.acc_expr = 0;
-    tp::Out o;
-    o.expr = 0;
-    o.arg = 0;
-    o.dtype = dc.dtype;  // the accumulator type (op.rs:61-73)
-    pr.epi.outs.push_back(o);
-    pr.epi.args.push_back({dc.dtype, ir::num_elements(dc.shape), true, mm});
-    pr.args = {pr.op_a.args[0], pr.op_b.args[0], pr.epi.args[0]};
-    pr.map_a = {0};
-    pr.map_b = {1};
-    pr.map_e = {2};
-    if (op.inputs[0] == op.inputs[1]) {  // A x A: one kernel argument read twice
-        pr.args = {pr.op_a.args[0], pr.epi.args[0]};
-        pr.map_b = {0};
-        pr.map_e = {1};
+    HE_REQUIRE(sg.is_input(op.inputs[0]) && sg.is_input(op.inputs[1]), HE_ERR_UNSUPPORTED,
+               "ops that feed a Matmul operand are fused through the fusion IR only");
+    if (sg.nodes().size() == 1) {
+        pr.epi.dims = {batch, pr.M, pr.N};
+        pr.epi.fast_math = true;
+        tp::Expr acc;
+        acc.kind = tp::Expr::Acc;
+        acc.cls = tp::Cls::F;
+        pr.epi.exprs.push_back(acc);
+        pr.epi.acc_expr = 0;
+        tp::Out o;
+        o.expr = 0;
+        o.arg = 0;
+        o.dtype = dc.dtype;  // the accumulator type (op.rs:61-73)
+        pr.epi.outs.push_back(o);
+        pr.epi.args.push_back({dc.dtype, ir::num_elements(dc.shape), true, mm});
+    } else {
+        // Matmul + the pointwise / reduce ops after it: the epilogue runs on the accumulators
+        // (MatmulGenerator's leaves, matmul.rs:88-130).
+        pr.epi = tp::lower_ir_epilogue(sg, mm);
     }
+    validate_gemm_epilogue(pr.epi);
+    assemble_gemm_args(pr);
     return pr;
 }
 

@@ -65,6 +65,11 @@ struct Plan {
     std::string describe() const;  // one line per step: instruction kinds, node sets, releases
 };
 
+// Whether pointwise / reduce ops downstream of a Matmul may join its instruction (on by default). Off gives the
+// reference's grouping, where a matmul instruction never fuses.
+void set_fuse_matmul_epilogue(bool on);
+bool fuse_matmul_epilogue();
+
 // generate_plan (plan_generation.rs:22-26).
 std::shared_ptr<const Plan> generate_plan(const std::shared_ptr<const ir::OpGraph>& g);
 // generate_cached_plan (:16-19): LRU of 256 plans keyed by the graph's structure.

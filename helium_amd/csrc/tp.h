@@ -94,6 +94,9 @@ struct Program {
 // per leaf in id order (the parameter order of jit.rs:213-221,285-286 is inputs, then outputs as they are stored;
 // here outputs are always in leaf order).
 Program lower_pointwise(const ir::OpSubgraph& sg);
+// A Matmul node (`anchor`) and the pointwise / reduce ops downstream of it -> the GEMM epilogue program over the
+// Matmul's output shape. Throws HE_ERR_UNSUPPORTED when the ops cannot run on the accumulator in place.
+Program lower_ir_epilogue(const ir::OpSubgraph& sg, ir::NodeId anchor);
 // supports_subgraph of helium/src/cuda/instr/pointwise.rs:121-186.
 bool pointwise_supports(const ir::OpSubgraph& sg);
 

@@ -290,6 +290,12 @@ int he_plan_destroy(he_plan_t plan);
  * tensor is a new reference the caller frees. */
 int he_execute_graph(he_graph_t graph, const uint32_t* input_nodes, const he_tensor_t* input_tensors, int num_inputs,
                      uint32_t* output_nodes, he_tensor_t* output_tensors, int max_outputs, int* num_outputs);
+/* Backend options. HE_OPT_FUSE_MATMUL_EPILOGUE (default 1): pointwise / reduce ops that follow a Matmul join its
+ * instruction and run as the fused GEMM's epilogue (the MatmulGenerator path, matmul.rs:88-130); 0 restores the
+ * grouping of helium/src/cuda/instr/cudnn_graph.rs:319-321, where a matmul instruction never fuses. */
+enum { HE_OPT_FUSE_MATMUL_EPILOGUE = 0 };
+int he_backend_set_option(int option, int64_t value);
+
 /* Counters of the last he_execute_graph on this thread: [0] steps run, [1] instructions, [2] streams used,
  * [3] event waits; and of the process: [4] plan-cache hits, [5] misses, [6] bytes held from the driver,
  * [7] driver allocations, [8] pooled reuses. */

@@ -66,9 +66,12 @@ class Instr:
         self.outputs = [n for n in self.nodes if any(o not in inside for o in graph.outbound[n])]
 
     def merged(self, other):
-        return Instr(self.g, self.kind, self.nodes + other.nodes)
+        kind = GEMM if GEMM in (self.kind, other.kind) else self.kind
+        return Instr(self.g, kind, self.nodes + other.nodes)
 
-    def can_fuse_with(self, nxt):
+    def can_fuse_with(self, nxt, gemm_epilogue=None):
+        if gemm_epilogue is not None and {self.kind, nxt.kind} == {GEMM, POINTWISE}:
+            return bool(gemm_epilogue(self.merged(nxt)))
         if self.kind != nxt.kind:
             return False
         if self.kind == GEMM:
@@ -192,8 +195,12 @@ class _InstrGraph:
         return False
 
 
-def generate_plan(nodes):
-    """Returns [(instrs, tensors_to_release)], instrs = [(kind, [node ids])] in the reference's order."""
+def generate_plan(nodes, gemm_epilogue=None):
+    """Returns [(instrs, tensors_to_release)], instrs = [(kind, [node ids])] in the reference's order.
+
+    `gemm_epilogue`: None for the reference's rule (a matmul instruction never fuses). The backend's extension lets
+    a matmul instruction and a pointwise one merge when the ops can run as the fused GEMM's epilogue; a test passes
+    the predicate (merged Instr -> bool) that states which merges it expects to be admitted."""
     g = Graph(nodes)
     ig = _InstrGraph()
     for i in g.order:
@@ -205,7 +212,7 @@ def generate_plan(nodes):
         cur = min(work)
         work.discard(cur)
         for nxt in sorted(ig.dependents[cur]):
-            if ig.instrs[cur].can_fuse_with(ig.instrs[nxt]) and not ig.exist_multiple_paths(cur, nxt):
+            if ig.instrs[cur].can_fuse_with(ig.instrs[nxt], gemm_epilogue) and not ig.exist_multiple_paths(cur, nxt):
                 a, b = ig.remove(cur), ig.remove(nxt)
                 new = ig.insert(a.merged(b), slot=nxt)
                 work.discard(nxt)

@@ -106,11 +106,18 @@ def test_random_graphs_execute(gpu, seed):
         assert np.allclose(a[fin], b[fin], rtol=2e-2 if desc[o][1] == "bf16" else 1e-3, atol=1e-5), (o, steps)
 
 
-def test_config1_linear_layer(gpu):
+@pytest.mark.parametrize("fuse", [1, 0], ids=["matmul_takes_its_epilogue", "reference_grouping"])
+def test_config1_linear_layer(gpu, fuse):
+    from helium_amd.backend import OPT_FUSE_MATMUL_EPILOGUE, set_option
+
     g, names = configs.c1_ir_graph()
     host = configs.c1_inputs(names, batched=False)
-    got, steps = run_graph(g, host)
-    assert [k for instrs, _ in steps for k, _ in instrs] == ["gemm", "pointwise", "pointwise"]
+    set_option(OPT_FUSE_MATMUL_EPILOGUE, fuse)
+    try:
+        got, steps = run_graph(g, host)
+    finally:
+        set_option(OPT_FUSE_MATMUL_EPILOGUE, 1)
+    assert [k for instrs, _ in steps for k, _ in instrs] == (["gemm", "pointwise"] if fuse else ["gemm", "pointwise", "pointwise"])
     val, _ = oracle_ir.evaluate(g.nodes, host)
     y = got[names["y"]].reshape(256, 512).astype(np.float64)
     want = val[names["y"]].astype(np.float64)

@@ -126,3 +126,46 @@ def test_ir_matmul_on_cpu(name, sa, sb, precision, dtype, tol):
     got = nm.from_storage(res[0], out[0]["dtype"], [res[0].size]).astype(np.float64)
     want = nm.from_storage(want.reshape(-1), out[0]["dtype"], [want.size]).astype(np.float64)
     assert np.abs(got - want).max() <= tol, (k.description, np.abs(got - want).max())
+
+
+def run_ir_kernel_on_cpu(g, nodes, inputs):
+    k = ha.backend.matmul_kernel(g, nodes)
+    gx, gy = map(int, re.search(r"grid=(\d+)x(\d+)", k.description).groups())
+    threads = int(re.search(r"threads=(\d+)", k.description).group(1))
+    bufs = []
+    for a in k.args:
+        dt = nm.NP_STORAGE[a["dtype"]]
+        bufs.append((np.zeros(a["numel"], dtype=dt), 2) if a["is_output"] else (inputs[a["node"]], 0))
+    res = run_kernel(k.source, "fused_matmul", gx, threads, bufs, grid_y=gy)
+    outs = [a for a in k.args if a["is_output"]]
+    return k, {a["node"]: nm.from_storage(r, a["dtype"], [r.size]).astype(np.float64) for a, r in zip(outs, res)}
+
+
+def test_ir_matmul_with_epilogue_on_cpu():
+    """Matmul + bias broadcast + add + relu of a helium-ir graph as one fused GEMM (config 1 at a small size)."""
+    from helium_amd import configs
+    from oracle import helium_ir as oracle_ir
+
+    g, names = configs.c1_ir_graph(40, 24, 72)
+    host = configs.c1_inputs(names, 40, 24, 72, batched=False)
+    k, got = run_ir_kernel_on_cpu(g, [3, 4, 5, 6], host)
+    assert [a["node"] for a in k.args] == [0, 1, 2, 6], k.args
+    val, _ = oracle_ir.evaluate(g.nodes, host)
+    assert np.abs(got[6] - val[6].reshape(-1)).max() <= 1e-4
+
+
+def test_ir_matmul_with_row_sums_on_cpu():
+    from oracle import helium_ir as oracle_ir
+
+    rng = np.random.default_rng(4)
+    g = ha.ir.OpGraph()
+    a = g.new_input([2, 40, 24], "bf16"); b = g.new_input([2, 24, 36], "bf16")
+    y = g.unary(g.matmul(a, b, "bf16_f32"), "relu")
+    oy = g.new_output(y); r = g.reduce(y, "sum", 1); g.new_output(r)
+    host = {a: nm.to_storage(rng.uniform(-1, 1, (2, 40, 24)).astype(np.float32), "bf16"),
+            b: nm.to_storage(rng.uniform(-1, 1, (2, 24, 36)).astype(np.float32), "bf16")}
+    k, got = run_ir_kernel_on_cpu(g, [2, 3, r], host)
+    val, desc = oracle_ir.evaluate(g.nodes, host)
+    want_y = nm.from_storage(nm.to_storage(val[y], desc[y][1]), desc[y][1], val[y].shape).astype(np.float64).reshape(-1)
+    assert np.abs(got[y] - want_y).max() <= 2e-2 * np.abs(want_y).max(), k.description
+    assert np.abs(got[r] - val[r].reshape(-1)).max() <= 1e-3 * np.abs(val[r]).max()

@@ -8,8 +8,16 @@ import numpy as np
 import pytest
 
 import helium_amd as ha
-from helium_amd.backend import Plan, stats
+from helium_amd.backend import OPT_FUSE_MATMUL_EPILOGUE, Plan, set_option, stats
 from oracle import plan as oracle_plan
+
+
+@pytest.fixture
+def reference_grouping():
+    """The reference's rule: a matmul instruction never fuses (cudnn_graph.rs:319-321)."""
+    set_option(OPT_FUSE_MATMUL_EPILOGUE, 0)
+    yield
+    set_option(OPT_FUSE_MATMUL_EPILOGUE, 1)
 
 
 def linear_layer():
@@ -67,7 +75,7 @@ NAMED = [linear_layer, second_path_blocks_fusion, constant_is_delayed, large_swa
 
 
 @pytest.mark.parametrize("make", NAMED, ids=lambda f: f.__name__)
-def test_hand_derived_plans(make):
+def test_hand_derived_plans(reference_grouping, make):
     g, want = make()
     assert oracle_plan.generate_plan(g.nodes) == want
     assert Plan(g).steps == want
@@ -143,11 +151,37 @@ def check_invariants(g, steps):
 
 
 @pytest.mark.parametrize("seed", range(60))
-def test_random_graphs_match_the_restatement(seed):
+def test_random_graphs_match_the_restatement(reference_grouping, seed):
     g = random_graph(seed)
     got = Plan(g).steps
     assert got == oracle_plan.generate_plan(g.nodes)
     check_invariants(g, got)
+
+
+def test_matmul_takes_the_ops_that_can_run_on_its_accumulators():
+    # default grouping of this backend. Worked out by hand: the matmul (slot 1) takes the add, the bias broadcast
+    # (slot 2) then joins as an epilogue operand, the relu follows; the swap cannot run in place on accumulators and
+    # starts the second kernel, which takes the reduction.
+    g, _ = linear_layer()
+    want = [([("gemm", [3, 4, 5, 6])], []), ([("pointwise", [7, 8])], [0, 1, 2]), ([], [])]
+    assert Plan(g).steps == want
+    in_place = lambda instr: not any(instr.g.nodes[n]["op"] == "swap_dims" for n in instr.nodes)  # noqa: E731
+    assert oracle_plan.generate_plan(g.nodes, gemm_epilogue=in_place) == want
+
+
+def test_ops_feeding_a_matmul_operand_stay_outside_it():
+    g, want = second_path_blocks_fusion()
+    # exp feeds the Matmul's A operand: no merge with it; the add after the Matmul reads exp's tensor and joins
+    assert Plan(g).steps == [([("pointwise", [2])], []), ([("gemm", [3, 4])], [0]), ([], [1, 2])]
+
+
+def test_row_sums_join_the_matmul():
+    g = ha.ir.OpGraph()
+    a = g.new_input([3, 64, 32], "bf16"); b = g.new_input([3, 32, 48], "bf16")
+    y = g.unary(g.matmul(a, b, "bf16_f32"), "relu")
+    g.new_output(y); g.new_output(g.reduce(y, "sum", 1)); g.new_output(g.reduce(y, "max", 1))
+    # the Sum folds into the epilogue; Max is not a reduction the GEMM epilogue offers and stays a kernel of its own
+    assert Plan(g).steps == [([("gemm", [2, 3, 5])], []), ([("pointwise", [7])], [0, 1]), ([], [])]
 
 
 def test_plan_cache_returns_the_same_plan_for_an_equal_graph():
