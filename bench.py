@@ -21,6 +21,7 @@ sys.path.insert(0, ROOT)
 METRIC = "fused-GEMM TFLOP/s & permute/pointwise GB/s, % of MI355X roofline"
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 BF16_PEAK_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
+F32_PEAK_TFLOPS = 157.3      # MI355X dense fp32 matrix, published
 # Bytes that left the XCD L2s per launch of each workload's dominant kernel: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE,
 # each scaled by what the same counter reads for the COPY workload (profiles/<kernel>_<workload>.txt).
 TRAFFIC_BYTES = {"COPY": 268435456, "C2a": 205565287, "C2b": 67153057, "C2c": 17587641, "C3": 277275033,
@@ -180,6 +181,71 @@ class AuxChainWorkload:
         self.sets = []
 
 
+class LinearLayerWorkload:
+    """BASELINE config 1 through the whole backend path: execute_graph on the lazy-graph form of
+    Y = relu(X W + b) plus the column sums (plan generation from cache, pooled allocation, a fused f32 GEMM with
+    its epilogue and one pointwise/reduction kernel). 0.13 GFLOP: latency-bound, reported as time per graph.
+    The executor owns its streams, so the time is the host's wall clock around K executions and one device sync."""
+
+    bound = "mfma"
+    unit = "TFLOP/s"
+    dtype = "f32"
+    name = "C1"
+    peak = F32_PEAK_TFLOPS
+    wall_timed = True
+
+    def __init__(self):
+        self.work = 2.0 * 256 * 512 * 512
+
+    def describe(self):
+        return "C1: f32 X[256,512] W[512,512] + b, relu, column sums via execute_graph (2 kernels)"
+
+    def setup(self):
+        from helium_amd import configs
+        from helium_amd.backend import Plan, Tensor
+
+        self.graph, self.names = configs.c1_ir_graph()
+        self.host = configs.c1_inputs(self.names, batched=False)
+        self.tensors = {i: Tensor.from_numpy(a, "f32") for i, a in self.host.items()}
+        self.plan = Plan(self.graph)
+        self.last = None
+        log(f"[bench] {self.describe()} :: plan: " + self.plan.text.replace("\n", " ; "))
+
+    def step(self, stream, i):
+        from helium_amd.backend import execute_graph
+
+        self.last = execute_graph(self.graph, self.tensors)
+
+    def check(self):
+        from oracle import helium_ir as oracle
+
+        val, _ = oracle.evaluate(self.graph.nodes, self.host)
+        y = self.last[self.names["y"]].to_numpy().astype(np.float64)
+        want = val[self.names["y"]].astype(np.float64).reshape(-1)
+        if not (np.abs(y - want) <= 1e-4 * np.maximum(np.abs(want), 1.0)).all():
+            raise SystemExit("[bench] PARITY FAILURE in C1: Y differs from the oracle")
+        cs = self.last[self.names["colsum"]].to_numpy().astype(np.float64)
+        want_cs = val[self.names["y"]].astype(np.float64).sum(axis=0)
+        if not (np.abs(cs - want_cs) <= 1e-3 * np.abs(want_cs) + 1e-4).all():
+            raise SystemExit("[bench] PARITY FAILURE in C1: column sums differ from the oracle")
+        return "Y within 1e-4, column sums within 1e-3 relative of the f64 oracle"
+
+    def cpu_baseline(self, budget_s=5.0):
+        from oracle import helium_ir as oracle
+
+        best, reps, t_all = 1e30, 0, time.perf_counter()
+        while reps < 3 or (time.perf_counter() - t_all < budget_s and reps < 50):
+            t0 = time.perf_counter()
+            oracle.evaluate(self.graph.nodes, self.host)
+            best = min(best, time.perf_counter() - t0)
+            reps += 1
+        return {"value": round(self.work / best / 1e12, 5), "unit": "TFLOP/s", "cores": os.cpu_count(), "kind": "port",
+                "sample": f"the whole C1 graph, numpy oracle (float64 BLAS matmul), best of {reps} passes"}
+
+    def free(self):
+        self.tensors, self.last = {}, None
+
+
 class FusedGemmWorkload:
     """BASELINE configs 4 / 5a: 4096^3 bf16 GEMM with fused mainloop / epilogue. Work = 2*M*N*K FLOP."""
 
@@ -317,6 +383,7 @@ def make_workloads():
     # a plain copy of known size (identity permute): the measured ceiling the permute kernels are read against and
     # the scale for the FETCH_SIZE / WRITE_SIZE counters
     w["COPY"] = PermuteWorkload("COPY", (8192, 8192), (0, 1), 24)
+    w["C1"] = LinearLayerWorkload()
     w["C3"] = AuxChainWorkload()
     for name in ("C4", "C5a", "C4m", "GEMM"):
         w[name] = FusedGemmWorkload(name)
@@ -349,7 +416,7 @@ def roofline(wl, ms):
         peak, unit = HBM_PEAK_GBS, "GB/s"
     else:
         achieved = wl.work / (ms * 1e-3) / 1e12
-        peak, unit = BF16_PEAK_TFLOPS, "TFLOP/s"
+        peak, unit = getattr(wl, "peak", BF16_PEAK_TFLOPS), "TFLOP/s"
     return {"bound": wl.bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
             "frac": round(achieved / peak, 4), "traffic": TRAFFIC_BYTES.get(wl.name)}
 
@@ -389,6 +456,8 @@ def main():
         stream.synchronize()
         parity = wl.check()
         ms, wall = time_workload(wl, stream, args.steps, args.warmup)
+        if getattr(wl, "wall_timed", False):
+            ms = wall  # launched on the executor's own streams: only the host clock brackets them
         rl = roofline(wl, ms)
         kernels[name] = {"workload": wl.describe(), "ms": round(ms, 5), "wall_ms": round(wall, 5), "parity": parity,
                          "roofline": rl}

@@ -27,7 +27,27 @@ size_t DevicePool::size_class(size_t bytes) {
     return (bytes + g - 1) / g * g;
 }
 
+void DevicePool::end_scope_after(uint64_t scope, hipEvent_t done) {
+    std::lock_guard<std::mutex> lk(mu_);
+    pending_.push_back({scope, done});
+}
+
+void DevicePool::poll() {
+    std::lock_guard<std::mutex> lk(mu_);
+    for (size_t i = 0; i < pending_.size();) {
+        if (hipEventQuery(pending_[i].second) == hipSuccess) {
+            end_scope_locked(pending_[i].first);
+            (void)hipEventDestroy(pending_[i].second);
+            pending_[i] = pending_.back();
+            pending_.pop_back();
+        } else {
+            i++;
+        }
+    }
+}
+
 uint64_t DevicePool::begin_scope() {
+    poll();
     std::lock_guard<std::mutex> lk(mu_);
     uint64_t s = next_scope_++;
     free_scoped_[s];
@@ -36,6 +56,10 @@ uint64_t DevicePool::begin_scope() {
 
 void DevicePool::end_scope(uint64_t scope) {
     std::lock_guard<std::mutex> lk(mu_);
+    end_scope_locked(scope);
+}
+
+void DevicePool::end_scope_locked(uint64_t scope) {
     auto it = free_scoped_.find(scope);
     if (it == free_scoped_.end()) return;
     for (auto& kv : it->second) free_global_.insert(kv);
@@ -74,6 +98,17 @@ void* DevicePool::allocate(size_t bytes, uint64_t scope) {
         if (sc != free_scoped_.end())
             if (void* p = take(sc->second)) return p;
         if (void* p = take(free_global_)) return p;
+    }
+    poll();  // blocks of executions that have finished since become available
+    {
+        std::lock_guard<std::mutex> lk(mu_);
+        auto it = free_global_.find(cls);
+        if (it != free_global_.end()) {
+            void* p = it->second;
+            free_global_.erase(it);
+            reuses_++;
+            return p;
+        }
         driver_bytes_ += cls;
         driver_allocs_++;
     }
@@ -234,23 +269,38 @@ std::map<NodeId, TensorRef> execute_graph(const ir::OpGraph& graph_in, const std
     }
 
     ExecStats local;
-    std::set<const Tensor*> synced;           // input tensors whose ready event a stream already waited on
-    std::vector<hipEvent_t> prev_events;      // one per stream used by the previous step
-    std::vector<hipEvent_t> all_events;
+    std::set<const Tensor*> synced;        // input tensors whose ready event a stream already waited on
+    std::vector<size_t> prev_streams;      // streams the previous step ran on
+    std::vector<hipEvent_t> events;        // join events of this execution
     std::set<size_t> used_streams;
+    // Every stream in `cur` waits for the end of the previous step on every other stream it ran on. The events are
+    // recorded here, before the new step enqueues anything, so they mark exactly the end of that step.
+    auto join = [&](const std::vector<size_t>& cur) {
+        for (size_t p : prev_streams) {
+            bool needed = false;
+            for (size_t w : cur) needed = needed || w != p;
+            if (!needed) continue;
+            hipEvent_t e;
+            HE_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+            events.push_back(e);
+            HE_HIP(hipEventRecord(e, st.s[p]));
+            for (size_t w : cur)
+                if (w != p) {
+                    HE_HIP(hipStreamWaitEvent(st.s[w], e, 0));
+                    local.event_waits++;
+                }
+        }
+    };
     for (auto& step : plan->steps) {
         for (NodeId r : step.tensors_to_release) tensors.erase(r);
         if (step.instrs.empty()) continue;
         local.steps++;
         std::vector<const Tensor*> waited;
-        // Instructions of one step are independent: they fan out over the stream pool. Every stream used by this
-        // step first waits for every stream used by the previous one.
+        // Instructions of one step are independent: they fan out over the stream pool.
         const size_t width = std::min(step.instrs.size(), st.s.size());
-        for (size_t w = 0; w < width; w++)
-            for (hipEvent_t e : prev_events) {
-                HE_HIP(hipStreamWaitEvent(st.s[w], e, 0));
-                local.event_waits++;
-            }
+        std::vector<size_t> cur(width);
+        for (size_t w = 0; w < width; w++) cur[w] = w;
+        join(cur);
         for (size_t i = 0; i < step.instrs.size(); i++) {
             const plan::Instr& instr = *step.instrs[i];
             hipStream_t stream = st.s[i % width];
@@ -276,32 +326,20 @@ std::map<NodeId, TensorRef> execute_graph(const ir::OpGraph& graph_in, const std
         }
         // every stream of the next steps is ordered after this step's streams, so one wait per tensor is enough
         synced.insert(waited.begin(), waited.end());
-        prev_events.clear();
-        for (size_t w = 0; w < width; w++) {
-            hipEvent_t e;
-            HE_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
-            HE_HIP(hipEventRecord(e, st.s[w]));
-            prev_events.push_back(e);
-            all_events.push_back(e);
-        }
+        prev_streams = cur;
     }
     // Drop of the executor (cuda.rs:232-260): when everything queued above has run, the scope's freed blocks
-    // become available to everyone.
-    for (hipEvent_t e : prev_events) HE_HIP(hipStreamWaitEvent(st.s[0], e, 0));
-    struct Done {
-        uint64_t scope;
-        std::vector<hipEvent_t> events;
-    };
-    Done* done = new Done{scope, all_events};
-    HE_HIP(hipLaunchHostFunc(st.s[0], [](void* p) {
-        Done* d = static_cast<Done*>(p);
-        DevicePool::global().end_scope(d->scope);
-        delete d;  // events are destroyed by the next executor of this thread (not from a callback thread)
-    }, done));
+    // become available to everyone. Stream 0 joins the last step and carries the event the pool polls.
+    join({0});
+    hipEvent_t done;
+    HE_HIP(hipEventCreateWithFlags(&done, hipEventDisableTiming));
+    HE_HIP(hipEventRecord(done, st.s[0]));
+    pool.end_scope_after(scope, done);
     {
+        // join events of the previous execution on this thread: recorded and waited on long ago
         static thread_local std::vector<hipEvent_t> garbage;
-        for (hipEvent_t e : garbage) (void)hipEventDestroy(e);  // recorded long ago; destruction is deferred by HIP
-        garbage = all_events;
+        for (hipEvent_t e : garbage) (void)hipEventDestroy(e);
+        garbage = events;
     }
     local.streams_used = (int)used_streams.size();
     if (stats) *stats = local;

@@ -20,6 +20,10 @@ public:
     static DevicePool& global();
     uint64_t begin_scope();
     void end_scope(uint64_t scope);  // called once the scope's device work has finished
+    // Ends the scope once `done` (recorded after all of its device work) has completed; polled from begin_scope and
+    // from allocate, so no host callback sits in any stream. The pool takes the event over.
+    void end_scope_after(uint64_t scope, hipEvent_t done);
+    void poll();
     void* allocate(size_t bytes, uint64_t scope);
     // `owner`: the scope the block was allocated in (0: none); `used`: every scope whose device work touches it.
     // The block goes to the owner's free list while only the owner can still touch it, to the global list when no
@@ -39,6 +43,8 @@ private:
         std::vector<uint64_t> waiting;
     };
     std::vector<Deferred> deferred_;
+    std::vector<std::pair<uint64_t, hipEvent_t>> pending_;  // scopes whose device work may still be running
+    void end_scope_locked(uint64_t scope);
     uint64_t next_scope_ = 1, driver_bytes_ = 0, driver_allocs_ = 0, reuses_ = 0;
 };
 
