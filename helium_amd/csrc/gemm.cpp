@@ -91,7 +91,8 @@ const char* kGemmBody = R"HIP(
 __device__ __forceinline__ u32 a_off(u32 m, u32 kc) { return m * (BK * ESZ) + ((kc ^ ((m >> A_SWZ_SHIFT) & (A_CHUNKS - 1))) << 4); }
 // B rows keep their memory order; the chunk index is XORed with 4 * (k % 4) for the transposing 16-bit reads
 // (f32 operands are read one word per lane along n and need no swizzle).
-__device__ __forceinline__ u32 b_chunk_off(u32 k, u32 nc) { return k * (BN * ESZ) + ((nc ^ (MMA_F32 ? 0u : ((k & 3) << 2))) << 4); }
+#define B_SWZ(k) (MMA_F32 ? 0u : (((k) & 3) << 2) & (B_CHUNKS - 1))
+__device__ __forceinline__ u32 b_chunk_off(u32 k, u32 nc) { return k * (BN * ESZ) + ((nc ^ B_SWZ(k)) << 4); }
 __device__ __forceinline__ u32 b_off(u32 k, u32 n) { return b_chunk_off(k, (n * ESZ) >> 4) + ((n * ESZ) & 15); }
 
 #if MMA_F32
@@ -102,6 +103,11 @@ typedef s16x8 afrag_t;
 typedef s16x8 bfrag_t;
 #endif
 struct WavePos { u32 lane, wave, wave_m, wave_n; };
+#if MMA_F32
+typedef float mul_t;   /* multiplicand as stored in global memory */
+#else
+typedef bf16_t mul_t;  /* any two-byte multiplicand: only the element size matters to the address arithmetic */
+#endif
 
 // Operand fragments of k-step kk from one LDS stage. `st` is __restrict__ on purpose: after inlining, every LDS
 // read carries alias-scope information that separates it from the direct global->LDS writes into the *other*
@@ -199,8 +205,8 @@ __device__ __forceinline__ void compute_tile(const unsigned char* __restrict__ s
 // `ga` / `gb` point at the tile's first A row / first B k-row (at this workgroup's columns).
 #define A_DPW (DIRECT_A ? A_TILE_BYTES / 1024 / NWAVES : 0)  /* direct-load instructions per wave and tile */
 #define B_DPW (DIRECT_B ? B_TILE_BYTES / 1024 / NWAVES : 0)
-__device__ __forceinline__ void direct_issue(unsigned char* __restrict__ st, const bf16_t* __restrict__ ga,
-                                             const bf16_t* __restrict__ gb, const WavePos& w, int i) {
+__device__ __forceinline__ void direct_issue(unsigned char* __restrict__ st, const mul_t* __restrict__ ga,
+                                             const mul_t* __restrict__ gb, const WavePos& w, int i) {
 #if GEMM_SKIP & 1
     return;
 #endif
@@ -209,19 +215,19 @@ __device__ __forceinline__ void direct_issue(unsigned char* __restrict__ st, con
         const u32 blk = wave * A_DPW + i;
         const u32 row = blk * (64 / A_CHUNKS) + lane / A_CHUNKS, pc = lane % A_CHUNKS;
         const u32 kc = pc ^ ((row >> A_SWZ_SHIFT) & (A_CHUNKS - 1));
-        const bf16_t* gp = ga + (size_t)row * GK + kc * 8;
+        const mul_t* gp = ga + (size_t)row * GK + kc * EPC;
         __builtin_amdgcn_global_load_lds((GLOBAL_AS const void*)gp, (LDS_AS void*)(st + blk * 1024), 16, 0, 0);
     } else {
         const u32 blk = wave * B_DPW + (i - A_DPW);
         const u32 krow = blk * (64 / B_CHUNKS) + lane / B_CHUNKS, pc = lane % B_CHUNKS;
-        const u32 nc = pc ^ ((krow & 3) << 2);
-        const bf16_t* gp = gb + (size_t)krow * GN + nc * 8;
+        const u32 nc = pc ^ B_SWZ(krow);
+        const mul_t* gp = gb + (size_t)krow * GN + nc * EPC;
         __builtin_amdgcn_global_load_lds((GLOBAL_AS const void*)gp, (LDS_AS void*)(st + A_TILE_BYTES + blk * 1024), 16, 0, 0);
     }
 }
 // Multiplies the tile in stage `rd` while requesting the tile that goes into stage `wr`.
 __device__ __forceinline__ void direct_tile(const unsigned char* __restrict__ rd, unsigned char* __restrict__ wr,
-                                            const bf16_t* __restrict__ ga, const bf16_t* __restrict__ gb, bool more,
+                                            const mul_t* __restrict__ ga, const mul_t* __restrict__ gb, bool more,
                                             f32x16 (&acc)[MB][NB], const WavePos& w) {
     compute_tile(rd, acc, w, [&](int kk) {
         constexpr int per = ISSUE_FRONT ? (A_DPW + B_DPW) : (A_DPW + B_DPW + KK - 1) / KK;
@@ -338,8 +344,8 @@ void fused_matmul(KERNEL_PARAMS) {
 /* s_waitcnt immediate: vmcnt lives in bits [3:0] and [15:14] */
 #define WAITCNT_VM(n) ((((n) & 15) | (((n) >> 4) << 14)))
 #if DIRECT_LOADS
-    const bf16_t* const ga0 = (const bf16_t*)DIRECT_A_PTR + ((size_t)bz * GM + m0) * GK;
-    const bf16_t* const gb0 = (const bf16_t*)DIRECT_B_PTR + (size_t)bz * GK * GN + n0;
+    const mul_t* const ga0 = (const mul_t*)DIRECT_A_PTR + ((size_t)bz * GM + m0) * GK;
+    const mul_t* const gb0 = (const mul_t*)DIRECT_B_PTR + (size_t)bz * GK * GN + n0;
     // NSTAGES-deep ring of LDS stages: tile kt + NSTAGES - 1 is requested while tile kt is multiplied, so a
     // wave only ever waits for loads issued NSTAGES - 2 tiles earlier.
 #pragma unroll
@@ -553,9 +559,11 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     const bool f32 = pr.mma_dtype == HE_F32;
     const int epc = f32 ? 4 : 8;  // multiplicands per 16-byte chunk
     Tile t;
+    bool small = false;
     const bool raw_a0 = is_raw_copy(pr.op_a, pr.root_a, pr.mma_dtype) && pr.K % epc == 0;
     const bool raw_b0 = is_raw_copy(pr.op_b, pr.root_b, pr.mma_dtype) && pr.N % epc == 0;
-    const bool want_direct = !f32 && !getenv("HELIUM_HIP_GEMM_NO_DIRECT");
+    const bool want_direct = !getenv("HELIUM_HIP_GEMM_NO_DIRECT");
+    const int esz = 16 / epc;  // bytes per multiplicand
     if (const char* env = getenv("HELIUM_HIP_GEMM_TILE")) {
         int v[6] = {256, 256, 64, 2, 4, 2};
         int n = sscanf(env, "%d,%d,%d,%d,%d,%d", &v[0], &v[1], &v[2], &v[3], &v[4], &v[5]);
@@ -567,6 +575,9 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         if (pr.M <= 128 || pr.N <= 128 || ((pr.M + 255) / 256) * ((pr.N + 255) / 256) * pr.batch < 128) {
             t.bm = t.bn = 128;
             t.wm = t.wn = 2;
+            small = true;
+            // still fewer workgroups than half the CUs: 64x64 tiles (one MFMA block per wave) spread the work
+            if (pr.M > 64 && pr.N > 64 && ((pr.M + 127) / 128) * ((pr.N + 127) / 128) * pr.batch < 128) t.bm = t.bn = 64;
         }
     }
     HE_REQUIRE(t.bm % (t.wm * 32) == 0 && t.bn % (t.wn * 32) == 0 && (t.bk == 64 || t.bk == 32) && (!f32 || t.bk == 32), HE_ERR_INVALID, "bad GEMM tile");
@@ -581,11 +592,15 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     const int nva = std::min(epc, tp::pick_nv(pr.op_a, 16)), nvb = std::min(epc, tp::pick_nv(pr.op_b, 16));
     // Direct global->LDS loads need unpredicated, unmodified 16-byte chunks: raw operands and full tiles everywhere.
     // Each operand qualifies on its own; the other one then goes through registers.
-    const bool direct_a = want_direct && raw_a && pr.M % t.bm == 0 && pr.K % t.bk == 0 && (t.bm * t.bk * 2 / 1024) % (threads / 64) == 0 &&
+    const bool direct_a = want_direct && raw_a && pr.M % t.bm == 0 && pr.K % t.bk == 0 && (t.bm * t.bk * esz / 1024) % (threads / 64) == 0 &&
                           !getenv("HELIUM_HIP_GEMM_NO_DIRECT_A");
-    const bool direct_b = want_direct && raw_b && pr.N % t.bn == 0 && pr.K % t.bk == 0 && (t.bk * t.bn * 2 / 1024) % (threads / 64) == 0 &&
-                          64 % (t.bn / 8) == 0 && !getenv("HELIUM_HIP_GEMM_NO_DIRECT_B");
+    const bool direct_b = want_direct && raw_b && pr.N % t.bn == 0 && pr.K % t.bk == 0 && (t.bk * t.bn * esz / 1024) % (threads / 64) == 0 &&
+                          64 % (t.bn / epc) == 0 && !getenv("HELIUM_HIP_GEMM_NO_DIRECT_B");
     if (!(direct_a && direct_b)) t.stages = 2;  // register staging is double-buffered only
+    else if (!getenv("HELIUM_HIP_GEMM_TILE") && small) {
+        // A grid that leaves CUs idle is bound by the latency of its k-loop: keep as many tiles in flight as LDS holds.
+        while (t.stages < 4 && (t.stages + 1) * (t.bm + t.bn) * t.bk * esz <= 128 * 1024) t.stages++;
+    }
     // All direct loads of the next tile are issued at the start of a tile's MFMAs (the round trip needs the whole
     // tile to hide); HELIUM_HIP_GEMM_ISSUE=0 spreads them over the k-steps instead.
     const bool issue_front = getenv("HELIUM_HIP_GEMM_ISSUE") ? atoi(getenv("HELIUM_HIP_GEMM_ISSUE")) != 0 : true;
@@ -768,7 +783,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
             // compiler can only wait for *all* outstanding LDS reads at once
             plan << "__builtin_amdgcn_sched_group_barrier(0x100, " << nr << ", 0);\n";
             const int waves = threads / 64;
-            const int dl = ((direct_a ? t.bm * t.bk * 2 / 1024 : 0) + (direct_b ? t.bk * t.bn * 2 / 1024 : 0)) / waves;
+            const int dl = ((direct_a ? t.bm * t.bk * esz / 1024 : 0) + (direct_b ? t.bk * t.bn * esz / 1024 : 0)) / waves;
             const int per = issue_front ? dl : (dl + kk_steps - 1) / kk_steps;
             const int rate = mode == 3 ? 2 : nr;
             for (int kk = 0; kk < kk_steps; kk++) {
@@ -786,7 +801,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
             // reads of step kk+1 are spread between the MFMAs of step kk
             plan << "__builtin_amdgcn_sched_group_barrier(0x100, " << nr << ", 0);\n";
             const int waves = threads / 64;
-            const int dl = ((direct_a ? t.bm * t.bk * 2 / 1024 : 0) + (direct_b ? t.bk * t.bn * 2 / 1024 : 0)) / waves;
+            const int dl = ((direct_a ? t.bm * t.bk * esz / 1024 : 0) + (direct_b ? t.bk * t.bn * esz / 1024 : 0)) / waves;
             const int per = issue_front ? dl : (dl + kk_steps - 1) / kk_steps;
             for (int kk = 0; kk < kk_steps; kk++) {
                 int issue = std::max(0, std::min(per, dl - kk * per));

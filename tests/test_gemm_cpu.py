@@ -58,6 +58,8 @@ CASES = [
     ("eight_waves_2x4", lambda: gemm_cases.bias_relu_colsum(140, 264, 72, mainloop=True), "128,256,64,2,4"),
     ("four_stage_ring_bk32", lambda: gemm_cases.plain(256, 256, 192), "256,256,32,2,4,4"),
     ("mainloop_in_registers_b_direct", lambda: gemm_cases.bias_relu_colsum(256, 256, 128, mainloop=True), "128,128,64,2,2"),
+    ("tile_64x64_staged", lambda: gemm_cases.bias_relu_colsum(100, 72, 136), "64,64,64,2,2"),
+    ("tile_64x64_direct", lambda: gemm_cases.plain(128, 192, 128), "64,64,64,2,2,3"),
     ("five_stage_ring_bk32", lambda: gemm_cases.plain(256, 256, 288), "256,256,32,2,4,5"),
     ("three_stage_ring_short_k", lambda: gemm_cases.plain(128, 256, 32), "128,128,32,2,2,3"),
     ("three_stage_ring_bk64", lambda: gemm_cases.bias_relu_colsum(128, 128, 320), "128,128,64,2,2,3"),
@@ -104,6 +106,7 @@ IR_CASES = [
     ("bf16_multiplicands_of_f32_tensors", [64, 48], [48, 64], "bf16_f32", "f32", 1e-3),
     ("f16_accumulator_type", [64, 64], [64, 64], "f16_f16", "f16", 2e-2),
     ("batched_f32", [2, 40, 24], [2, 24, 36], "f32_f32", "f32", 1e-4),
+    ("f32_direct_loads_four_stage_ring", [128, 160], [160, 256], "f32_f32", "f32", 1e-4),
 ]
 
 
