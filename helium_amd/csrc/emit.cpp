@@ -282,19 +282,20 @@ int pick_nv(const Program& p, int max_bytes) {
     return nv;
 }
 
-static bool is_deferred_load(const Program& p, const Expr& e, int nv) {
+static bool is_deferred_load(const Program& p, const Expr& e, int nv, bool row_varying_only = false) {
     if (e.kind != Expr::Load || nv < 2 || !e.access.chain.empty() || e.access.dtype == HE_BOOL) return false;
     const int n = (int)p.dims.size();
+    if (row_varying_only && (n < 2 || p.dims[n - 2] <= 1 || e.access.stride[n - 2] == 0)) return false;
     return p.dims[n - 1] > 1 && e.access.stride[n - 1] == 1;
 }
 static std::string raw_type(int dtype, int nv) {
     const char* elem = dtype == HE_BF16 ? "u16" : dtype == HE_F16 ? "f16_t" : dtype == HE_U32 ? "u32" : "float";
     return strfmt("typename Vec<%s, %d>::type", elem, nv);
 }
-std::string emit_raw_members(const Program& p, int nv) {
+std::string emit_raw_members(const Program& p, int nv, bool row_varying_only) {
     std::ostringstream s;
     for (size_t i = 0; i < p.exprs.size(); i++)
-        if (is_deferred_load(p, p.exprs[i], nv)) s << raw_type(p.exprs[i].access.dtype, nv) << " raw" << i << ";\n";
+        if (is_deferred_load(p, p.exprs[i], nv, row_varying_only)) s << raw_type(p.exprs[i].access.dtype, nv) << " raw" << i << ";\n";
     return s.str();
 }
 
@@ -318,7 +319,7 @@ std::string emit_exprs(const Program& p, const EmitCtx& cx) {
         const std::string v = "e" + std::to_string(i);
         const char* T = cls_type(e.cls);
         if (cx.phase != 0) {
-            const bool deferred = is_deferred_load(p, e, NV);
+            const bool deferred = is_deferred_load(p, e, NV, cx.defer_row_varying_only);
             if (cx.phase == 1) {
                 if (deferred)
                     s << "{ const size_t o = " << coord_sum(e.access.stride) << ";\nR.raw" << i << " = *(const " << raw_type(e.access.dtype, NV)

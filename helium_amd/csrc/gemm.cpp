@@ -83,6 +83,7 @@ const char* kGemmBody = R"HIP(
 #define A_PER_THREAD (BM * A_CHUNKS / NTHREADS)
 #define B_PER_THREAD (BK * B_CHUNKS / NTHREADS)
 #define EP (WTN + 4)              /* float pitch of the epilogue strip */
+#define EPI_STEPS ((32 * WTN) / (64 * NVE))  /* NVE-wide steps a lane takes through one 32-row block */
 #if NSTAGES * STAGE_BYTES < NWAVES * 32 * EP * 4
 #error "the epilogue strip does not fit in the operand stages"
 #endif
@@ -431,6 +432,7 @@ void fused_matmul(KERNEL_PARAMS) {
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
         for (int step = 0; step < (32 * WTN) / (64 * NVE); step++) {
+            EPILOGUE_PREFETCH
             const u32 idx = (step * 64 + lane) * NVE;
             const u32 row = idx / WTN, col = idx % WTN;
             const u32 m = m0 + wave_m * WTM + i * 32 + row;
@@ -677,10 +679,35 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     emit_fetch("b", pr.op_b, pr.root_b, pr.map_b, raw_b, nvb, "GK", "GN", pr.K % t.bk == 0 && pr.N % t.bn == 0);
 
     // epilogue pieces
-    std::ostringstream setup, body, finish;
+    std::ostringstream setup, body, finish, prefetch;
+    // Optional (HELIUM_HIP_GEMM_EPIPIPE=1): full-size tensors the epilogue reads are requested one step ahead of the
+    // step that uses them. Measured no faster than the compiler's own placement on the 40-op epilogue, so off.
+    const std::string raw_members = tp::emit_raw_members(pr.epi, nve, true);
+    const bool pipelined = !raw_members.empty() && getenv("HELIUM_HIP_GEMM_EPIPIPE");
+    if (pipelined) {
+        tp::EmitCtx lx;
+        lx.nv = nve;
+        lx.phase = 1;
+        lx.defer_row_varying_only = true;
+        s << "struct RawE {\n" << raw_members << "};\n__device__ __forceinline__ void epi_load(";
+        for (size_t a = 0; a < pr.epi.args.size(); a++)
+            s << (pr.epi.args[a].is_output ? "" : "const ") << tp::c_type(pr.epi.args[a].dtype) << "* __restrict__ a" << a << ", ";
+        s << "u32 cB0, u32 m, u32 n0, RawE& R) {\n(void)cB0; (void)m; (void)n0;\n" << tp::emit_exprs(pr.epi, lx) << "}\n";
+        std::string pass;
+        for (size_t a = 0; a < pr.epi.args.size(); a++) pass += "a" + std::to_string(a) + ", ";
+        prefetch << "{ const int q1 = i * EPI_STEPS + step + 1;\nif (q1 < MB * EPI_STEPS) {\nconst int i1 = q1 / EPI_STEPS, s1 = q1 % EPI_STEPS;\n"
+                 << "const u32 idx1 = (s1 * 64 + lane) * NVE;\nconst u32 m1 = m0 + wave_m * WTM + i1 * 32 + idx1 / WTN, nn1 = n0 + wave_n * WTN + idx1 % WTN;\n"
+                 << "if (m1 < GM && nn1 < GN) epi_load(" << pass << "bz, m1, nn1, Rb[q1 & 1]);\n} }\n";
+    }
     for (size_t a = 0; a < pr.epi.args.size(); a++)
         setup << "auto* a" << a << " = p" << pr.map_e[a] << "; (void)a" << a << ";\n";
     setup << "const u32 cB0 = bz; (void)cB0;\n";
+    if (pipelined) {
+        std::string pass;
+        for (size_t a = 0; a < pr.epi.args.size(); a++) pass += "a" + std::to_string(a) + ", ";
+        setup << "RawE Rb[2];\n{ const u32 idx1 = lane * NVE;\nconst u32 m1 = m0 + wave_m * WTM + idx1 / WTN, nn1 = n0 + wave_n * WTN + idx1 % WTN;\n"
+              << "if (m1 < GM && nn1 < GN) epi_load(" << pass << "bz, m1, nn1, Rb[0]);\n}\n";
+    }
     for (size_t oi = 0; oi < pr.epi.outs.size(); oi++) {
         const tp::Out& o = pr.epi.outs[oi];
         if (!o.reduce) continue;
@@ -698,6 +725,11 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         body << "if (ok) {\nconst u32 n0 = nn; (void)n0;\nfloat (&acc)[NVE] = acc_v;\n";
         tp::EmitCtx cx;
         cx.nv = nve;
+        if (pipelined) {
+            cx.phase = 2;
+            cx.defer_row_varying_only = true;
+            body << "const RawE& R = Rb[(i * EPI_STEPS + step) & 1]; (void)R;\n";
+        }
         // the emitter names the first of the NV columns `n0`; the tile origin of the same name is shadowed here
         body << tp::emit_exprs(pr.epi, cx);
         for (size_t oi = 0; oi < pr.epi.outs.size(); oi++) {
@@ -819,6 +851,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         splice("SCHED_PLAN", plan.str());
     }
     splice("EPILOGUE_SETUP", setup.str());
+    splice("EPILOGUE_PREFETCH", prefetch.str());
     splice("EPILOGUE_BODY", body.str());
     splice("EPILOGUE_FINISH", finish.str());
     s << body_text;

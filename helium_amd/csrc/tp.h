@@ -132,9 +132,10 @@ struct EmitCtx {
     // 0: everything. 1: only the full-vector loads, left undecoded in members raw<expr id> of a struct named `R`.
     // 2: everything else, reading those members. Splitting lets a kernel issue the loads long before it needs them.
     int phase = 0;
+    bool defer_row_varying_only = false;  // phases 1/2: loads whose address ignores the row stay in phase 2
 };
-// Members of the struct phase 1 fills: one native vector per full-vector Load of the program.
-std::string emit_raw_members(const Program& p, int nv);
+// Members of the struct phase 1 fills: one native vector per deferred Load of the program.
+std::string emit_raw_members(const Program& p, int nv, bool row_varying_only = false);
 std::string emit_exprs(const Program& p, const EmitCtx& cx);
 // Largest vector width (elements) legal for every full-row access and store of the program.
 int pick_nv(const Program& p, int max_bytes);

@@ -14,12 +14,16 @@ import gemm_cases
 from cpu_emul import run_kernel
 
 
-def run_emulated(g, inputs, tile):
+def run_emulated(g, inputs, tile, env=()):
     os.environ["HELIUM_HIP_GEMM_TILE"] = tile
+    for name in env:
+        os.environ[name] = "1"
     try:
         k = ha.TileKernel.fused(g)
     finally:
         del os.environ["HELIUM_HIP_GEMM_TILE"]
+        for name in env:
+            del os.environ[name]
     gx, gy = map(int, re.search(r"grid=(\d+)x(\d+)", k.description).groups())
     threads = int(re.search(r"threads=(\d+)", k.description).group(1))
     bufs = []
@@ -42,7 +46,16 @@ def compare(got, want, rel=1e-2, eps=1e-3):
         assert ok.all(), (node, np.abs(g - w).max())
 
 
+def readme_fusion(size, mainloop, full):
+    from helium_amd import configs
+
+    g, outs = configs.c4_graph(size, mainloop=mainloop, full_size_outputs=full)
+    return g, configs.c4_inputs(g, size), sorted(outs.values())
+
+
 CASES = [
+    ("readme_epilogue_with_prefetched_aux_tensors", lambda: readme_fusion(128, False, False), "128,128,64,2,2"),
+    ("readme_epilogue_ragged_with_mainloop", lambda: readme_fusion(72, True, True), "128,128,64,2,2"),
     ("plain_2x2_tiles", lambda: gemm_cases.plain(160, 136, 72), "128,128,64,2,2"),
     ("ragged_scalar_paths", lambda: gemm_cases.plain(97, 131, 67), "128,128,64,2,2"),
     ("mainloop_bias_relu_colsum", lambda: gemm_cases.bias_relu_colsum(130, 136, 80, mainloop=True), "128,128,64,2,2"),
@@ -70,7 +83,7 @@ CASES = [
 @pytest.mark.parametrize("name,build,tile", CASES, ids=[c[0] for c in CASES])
 def test_fused_gemm_on_cpu(name, build, tile):
     g, inputs, outs = build()
-    k, got = run_emulated(g, inputs, tile)
+    k, got = run_emulated(g, inputs, tile, env=("HELIUM_HIP_GEMM_EPIPIPE",) if "prefetched" in name else ())
     assert sorted(got) == sorted(outs), k.description
     rounding = "f16" if name == "f16_operands" else None if name in ("f32_operands", "f32_linear_layer") else "bf16"
     want = oracle.outputs(g.nodes, inputs, round_mainloop_to=rounding)
