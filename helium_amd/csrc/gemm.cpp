@@ -175,30 +175,54 @@ __device__ __forceinline__ void mma_step(f32x16 (&acc)[MB][NB], const afrag_t (&
 #endif
 }
 
-// One k-tile: operands for step kk+1 are fetched from LDS while the MFMAs of step kk run.
+// Fragment registers: double-buffered over the k-steps and carried from one k-tile to the next.
+struct Frags {
+    afrag_t a[2][MB];
+    bfrag_t b[2][NB];
+};
+__device__ __forceinline__ void mma_or_skip(f32x16 (&acc)[MB][NB], const afrag_t (&af)[MB], const bfrag_t (&bf)[NB]) {
+#if !(GEMM_SKIP & 4)
+    mma_step(acc, af, bf);
+#else
+    acc[0][0][0] += (float)af[0][0] + (float)bf[0][0];
+#endif
+}
+// One k-tile, rotated by one k-step: the MFMAs of the previous tile's last step run right after this tile's first
+// fragment reads have been issued, so the LDS latency that follows the workgroup barrier hides behind them; this
+// tile's own last step is left in `fr` for the next call (or for finish_tiles after the last tile).
 template <class PerStep>
 __device__ __forceinline__ void compute_tile(const unsigned char* __restrict__ st, f32x16 (&acc)[MB][NB], const WavePos& w,
-                                             PerStep&& per_step) {
-    afrag_t af[2][MB];
-    bfrag_t bf[2][NB];
-    load_frags(st, 0, w, af[0], bf[0]);
+                                             Frags& fr, PerStep&& per_step) {
+    static_assert(KK % 2 == 0, "the fragment double buffer assumes an even number of k-steps per tile");
+#if !(GEMM_SKIP & 2)
+    load_frags(st, 0, w, fr.a[0], fr.b[0]);
+#endif
+    // A slice (or all) of the next tile's global->LDS traffic. Issuing a direct load takes tens of cycles; the MFMAs
+    // of the previous tile's step KK-1 (zero fragments before the first tile) need nothing from memory and are
+    // scheduled between the loads, so the matrix pipes work while the address unit does.
+    per_step(0);
+    mma_or_skip(acc, fr.a[1], fr.b[1]);
 #pragma unroll
-    for (int kk = 0; kk < KK; kk++) {
-        per_step(kk);  // a slice of the next tile's global->LDS traffic
+    for (int kk = 0; kk + 1 < KK; kk++) {
+        per_step(kk + 1);
 #if GEMM_SKIP & 2
-        if (kk + 1 < KK) { for (int i = 0; i < MB; i++) af[(kk + 1) & 1][i] = af[kk & 1][i]; for (int j = 0; j < NB; j++) bf[(kk + 1) & 1][j] = bf[kk & 1][j]; }
+        for (int i = 0; i < MB; i++) fr.a[(kk + 1) & 1][i] = fr.a[kk & 1][i];
+        for (int j = 0; j < NB; j++) fr.b[(kk + 1) & 1][j] = fr.b[kk & 1][j];
 #else
-        if (kk + 1 < KK) load_frags(st, kk + 1, w, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+        load_frags(st, kk + 1, w, fr.a[(kk + 1) & 1], fr.b[(kk + 1) & 1]);
 #endif
-#if !(GEMM_SKIP & 4)
-        mma_step(acc, af[kk & 1], bf[kk & 1]);
-#else
-        acc[0][0][0] += (float)af[kk & 1][0][0] + (float)bf[kk & 1][0][0];
-#endif
+        mma_or_skip(acc, fr.a[kk & 1], fr.b[kk & 1]);
         SCHED_HINT
     }
     SCHED_PLAN
 }
+__device__ __forceinline__ void init_frags(Frags& fr) {
+#pragma unroll
+    for (int i = 0; i < MB; i++) fr.a[0][i] = fr.a[1][i] = afrag_t{};
+#pragma unroll
+    for (int j = 0; j < NB; j++) fr.b[0][j] = fr.b[1][j] = bfrag_t{};
+}
+__device__ __forceinline__ void finish_tiles(f32x16 (&acc)[MB][NB], const Frags& fr) { mma_or_skip(acc, fr.a[1], fr.b[1]); }
 
 #if DIRECT_LOADS
 // Operand tiles go from global memory straight into LDS (global_load_lds_dwordx4): a wave instruction fills
@@ -229,8 +253,8 @@ __device__ __forceinline__ void direct_issue(unsigned char* __restrict__ st, con
 // Multiplies the tile in stage `rd` while requesting the tile that goes into stage `wr`.
 __device__ __forceinline__ void direct_tile(const unsigned char* __restrict__ rd, unsigned char* __restrict__ wr,
                                             const mul_t* __restrict__ ga, const mul_t* __restrict__ gb, bool more,
-                                            f32x16 (&acc)[MB][NB], const WavePos& w) {
-    compute_tile(rd, acc, w, [&](int kk) {
+                                            f32x16 (&acc)[MB][NB], const WavePos& w, Frags& fr) {
+    compute_tile(rd, acc, w, fr, [&](int kk) {
         constexpr int per = ISSUE_FRONT ? (A_DPW + B_DPW) : (A_DPW + B_DPW + KK - 1) / KK;
         if (more) {
 #pragma unroll
@@ -369,6 +393,8 @@ void fused_matmul(KERNEL_PARAMS) {
 #else
 #define TICK(var)
 #endif
+    Frags frags;
+    init_frags(frags);
     for (u32 kt = 0; kt < KT; kt++) {
 #if DIRECT_LOADS
         // tile kt must have landed; up to NSTAGES - 2 younger tiles may still be in flight
@@ -393,9 +419,9 @@ void fused_matmul(KERNEL_PARAMS) {
 #if DIRECT_LOADS
         const u32 knext = more ? k_tile(next) * BK : 0u;
         direct_tile(lds + (kt % NSTAGES) * STAGE_BYTES, lds + (next % NSTAGES) * STAGE_BYTES, ga0 + knext,
-                    gb0 + (size_t)knext * GN, more, acc, wpos);
+                    gb0 + (size_t)knext * GN, more, acc, wpos, frags);
 #else
-        compute_tile(lds + (kt % NSTAGES) * STAGE_BYTES, acc, wpos, [](int) {});
+        compute_tile(lds + (kt % NSTAGES) * STAGE_BYTES, acc, wpos, frags, [](int) {});
 #endif
 #if STAGED
         STAGE_SCHED_BARRIER
@@ -404,6 +430,7 @@ void fused_matmul(KERNEL_PARAMS) {
         __builtin_amdgcn_sched_barrier(0);
         TICK(t_compute)
     }
+    finish_tiles(acc, frags);
     __syncthreads();
 #if GEMM_TIMING
     if (blockIdx.x == 0 && tid == 64) {
@@ -811,18 +838,31 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
                 plan << "__builtin_amdgcn_sched_group_barrier(0x008, " << nm << ", 0);\n";
             }
         } else if (mode == 3 || mode == 4) {
-            // reads of step kk+1 go between the first MFMAs of step kk (two per MFMA in mode 3, all before the second
-            // MFMA in mode 4), so that they have landed when the step ends: while direct loads are in flight the
-            // compiler can only wait for *all* outstanding LDS reads at once
-            plan << "__builtin_amdgcn_sched_group_barrier(0x100, " << nr << ", 0);\n";
+            // Rotated tile: direct loads, the first k-step's reads, the MFMAs left over from the previous tile, then
+            // per k-step the next step's reads between the first MFMAs (two per MFMA in mode 3, all before the
+            // second MFMA in mode 4) so that they have landed when the step ends: while direct loads are in flight
+            // the compiler can only wait for *all* outstanding LDS reads at once.
             const int waves = threads / 64;
             const int dl = ((direct_a ? t.bm * t.bk * esz / 1024 : 0) + (direct_b ? t.bk * t.bn * esz / 1024 : 0)) / waves;
             const int per = issue_front ? dl : (dl + kk_steps - 1) / kk_steps;
             const int rate = mode == 3 ? 2 : nr;
-            for (int kk = 0; kk < kk_steps; kk++) {
-                int issue = std::max(0, std::min(per, dl - kk * per));
-                if (issue) plan << "__builtin_amdgcn_sched_group_barrier(0x020, " << issue << ", 0);\n";
-                int left = kk + 1 < kk_steps ? nr : 0;
+            for (int g = 0; g < kk_steps; g++) {
+                int issue = std::max(0, std::min(per, dl - g * per));
+                if (g == 0) {
+                    plan << "__builtin_amdgcn_sched_group_barrier(0x100, " << nr << ", 0);\n";
+                    int done = 0;
+                    for (int m = 0; m < nm; m++) {  // direct loads spread evenly between the carried MFMAs
+                        const int upto = issue * (m + 1) / nm;
+                        if (upto > done) plan << "__builtin_amdgcn_sched_group_barrier(0x020, " << (upto - done) << ", 0);\n";
+                        done = upto;
+                        plan << "__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);\n";
+                    }
+                } else if (issue) {
+                    plan << "__builtin_amdgcn_sched_group_barrier(0x020, " << issue << ", 0);\n";
+                }
+                if (g + 1 == kk_steps) break;
+                // MFMAs of step g with the reads of step g + 1
+                int left = nr;
                 for (int m = 0; m < nm; m++) {
                     plan << "__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);\n";
                     const int r = std::min(left, rate);
