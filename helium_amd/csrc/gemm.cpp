@@ -655,7 +655,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
       << "\n#define DIRECT_LOADS (DIRECT_A || DIRECT_B)\n#define STAGED (!DIRECT_A || !DIRECT_B)"
       << "\n#define DIRECT_A_PTR p" << (direct_a ? pr.map_a[0] : 0)
       << "\n#define DIRECT_B_PTR p" << (direct_b ? pr.map_b[0] : 0) << "\n#define STAGE_SCHED_BARRIER "
-      << (getenv("HELIUM_HIP_GEMM_PIN") ? "__builtin_amdgcn_sched_barrier(0);" : "") << "\n#define A_SWZ_SHIFT " << (getenv("HELIUM_HIP_GEMM_ASWZ") ? atoi(getenv("HELIUM_HIP_GEMM_ASWZ")) : (t.bk == 64 ? 1 : 2)) << "\n";
+      << ((getenv("HELIUM_HIP_GEMM_PIN") ? atoi(getenv("HELIUM_HIP_GEMM_PIN")) != 0 : true) ? "__builtin_amdgcn_sched_barrier(0);" : "") << "\n#define A_SWZ_SHIFT " << (getenv("HELIUM_HIP_GEMM_ASWZ") ? atoi(getenv("HELIUM_HIP_GEMM_ASWZ")) : (t.bk == 64 ? 1 : 2)) << "\n";
 
     s << kGemmHelpers;
     // kernel parameters
@@ -827,7 +827,9 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         }
         splice("SCHED_HINT", h.str());
         std::ostringstream plan;
-        const int mode = getenv("HELIUM_HIP_GEMM_PLAN") ? atoi(getenv("HELIUM_HIP_GEMM_PLAN")) : 3;
+        // The instruction-order plan is written for tiles whose operands both arrive by direct loads; with an operand
+        // staged through registers the compiler's own order, fenced off from the staging code, measured 1.9x faster.
+        const int mode = getenv("HELIUM_HIP_GEMM_PLAN") ? atoi(getenv("HELIUM_HIP_GEMM_PLAN")) : (direct_a && direct_b) ? 3 : 0;
         const int mb = t.bm / t.wm / 32, nb = t.bn / t.wn / 32, kk_steps = t.bk / (2 * epc);
         const int nr = f32 ? mb + 4 * nb : mb + 2 * nb, nm = f32 ? 4 * mb * nb : mb * nb;
         if (mode == 1) {
