@@ -27,6 +27,12 @@ typedef unsigned int u32;
 typedef unsigned long long u64;
 typedef __bf16 bf16_t;
 typedef _Float16 f16_t;
+#ifndef HE_OPAQUE
+// Hides where a value came from. Negating a just-widened bf16 and narrowing it again makes this compiler (with
+// packed FP32 off) build an integer xor it then cannot select; the barrier keeps the three steps apart.
+__device__ __forceinline__ float he_opaque(float x) { asm volatile("" : "+v"(x)); return x; }
+#define HE_OPAQUE(x) he_opaque(x)
+#endif
 #ifndef HE_FAST_RCP
 #define HE_FAST_RCP(x) __builtin_amdgcn_rcpf(x)
 #endif
@@ -171,7 +177,7 @@ static std::string unary_expr(const Expr& e, const std::string& x, bool fast) {
     std::string c = f32_literal(e.bits);
     switch ((UOp)e.op) {
         case UOp::Recip: return fast ? "HE_FAST_RCP(" + x + ")" : "1.0f / " + x;
-        case UOp::Neg: return "-" + x;
+        case UOp::Neg: return "-HE_OPAQUE(" + x + ")";
         case UOp::Exp: return (fast ? "__expf(" : "expf(") + x + ")";
         case UOp::Sin: return (fast ? "__sinf(" : "sinf(") + x + ")";
         case UOp::Cos: return (fast ? "__cosf(" : "cosf(") + x + ")";

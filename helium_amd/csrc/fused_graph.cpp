@@ -1,0 +1,790 @@
+#include "fused_graph.h"
+
+#include <algorithm>
+#include <functional>
+#include <sstream>
+
+namespace he::fsearch {
+
+namespace {
+using fir::OpKind;
+bool is_pointwise(const fir::Op& op) {
+    return op.kind == OpKind::UnaryPointwise || op.kind == OpKind::BinaryPointwise || op.kind == OpKind::Constant;
+}
+// opgraph.rs:452-470
+bool is_terminator(const fir::Op& op) { return op.kind == OpKind::Reduction || op.kind == OpKind::Transpose; }
+bool is_epilogue_fusible(const fir::Op& op) {
+    return is_pointwise(op) || op.kind == OpKind::Reduction || op.kind == OpKind::Transpose || op.kind == OpKind::Broadcast;
+}
+bool is_mainloop_fusible(const fir::Op& op) { return is_pointwise(op) || op.kind == OpKind::Transpose || op.kind == OpKind::Broadcast; }
+bool is_input_output(const fir::Op& op) { return op.kind == OpKind::Producer || op.kind == OpKind::Consumer; }
+
+template <class T>
+bool has(const std::vector<T>& v, const T& x) {
+    return std::find(v.begin(), v.end(), x) != v.end();
+}
+template <class T>
+void erase_item(std::vector<T>& v, const T& x) {
+    auto it = std::find(v.begin(), v.end(), x);
+    if (it != v.end()) v.erase(it);
+}
+void insert_sorted(std::vector<OpNode>& v, OpNode n) { v.insert(std::lower_bound(v.begin(), v.end(), n), n); }
+constexpr size_t kMaxNodeRecomputations = 3;  // fused_graph.rs:423
+}  // namespace
+
+// ---------------------------------------------------------------------------------------------------------
+// Fusion
+// ---------------------------------------------------------------------------------------------------------
+std::vector<OpNode> Fusion::nodes() const {
+    if (!core) return fused;
+    std::vector<OpNode> n = mainloop;
+    n.insert(n.end(), epilogue.begin(), epilogue.end());
+    n.push_back(anchor);
+    return n;
+}
+bool Fusion::contains(OpNode n) const {
+    if (!core) return has(fused, n);
+    return n == anchor || has(mainloop, n) || has(epilogue, n);
+}
+void Fusion::remove_node(OpNode n) {
+    erase_item(mainloop, n);
+    erase_item(epilogue, n);
+    erase_item(fused, n);
+}
+bool Fusion::is_input_output(const fir::OpGraph& g) const {
+    for (OpNode n : nodes())
+        if (!he::fsearch::is_input_output(g.get(n))) return false;
+    return true;
+}
+std::string Fusion::key() const {
+    std::ostringstream s;
+    s << (core ? 'C' : 'A') << anchor << "|m";
+    for (OpNode n : mainloop) s << n << ',';
+    s << "|e";
+    for (OpNode n : epilogue) s << n << ',';
+    s << "|f";
+    for (OpNode n : fused) s << n << ',';
+    s << "|d";
+    for (auto& kv : dependencies) s << kv.first << '<' << kv.second << ',';
+    s << "|u";
+    for (auto& kv : dependents) s << kv.first << '>' << kv.second << ',';
+    return s.str();
+}
+
+std::string Action::describe() const {
+    static const char* names[] = {"CoreFuseIntoEpilogue", "CoreFuseIntoMainloop", "AuxFuse", "TransitionEdge"};
+    std::ostringstream s;
+    s << names[kind] << "{node " << node << ", fusion " << fusion;
+    if (kind == TransitionEdge) s << ", new_provider " << new_provider;
+    else
+        for (auto& kv : providers) s << ", " << kv.first << "<-" << kv.second;
+    s << "}";
+    return s.str();
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// FusedGraph
+// ---------------------------------------------------------------------------------------------------------
+FusedGraph FusedGraph::identity(std::shared_ptr<const fir::OpGraph> g) {
+    FusedGraph fg;
+    fg.g_ = g;
+    FusionId next = 0;
+    for (OpNode n : g->nodes()) {
+        Fusion f;
+        if (g->get(n).is_anchor()) {
+            f.core = true;
+            f.anchor = n;
+        } else {
+            f.fused = {n};
+        }
+        fg.fusions_[next] = f;
+        fg.node_fusions_[n] = {next};
+        next++;
+    }
+    for (OpNode n : g->nodes()) {
+        Fusion& f = fg.fusions_[fg.node_fusions_[n][0]];
+        for (OpNode in : g->inbound(n)) f.dependencies[in] = fg.node_fusions_[in][0];
+        for (OpNode out : g->outbound(n)) f.dependents.insert({n, fg.node_fusions_[out][0]});
+    }
+    fg.assert_invariants();
+    return fg;
+}
+
+bool FusedGraph::would_create_cycle(FusionId from, FusionId to) const {
+    std::vector<FusionId> stack{to};
+    std::set<FusionId> visited;
+    while (!stack.empty()) {
+        FusionId cur = stack.back();
+        stack.pop_back();
+        if (cur == from) return true;
+        for (auto& d : fusions_.at(cur).dependents)
+            if (visited.insert(d.second).second) stack.push_back(d.second);
+    }
+    return false;
+}
+
+std::vector<FusionId> FusedGraph::dependency_providers(OpNode dep, FusionId fusion,
+                                                      std::map<std::pair<FusionId, FusionId>, bool>& cache) const {
+    // a fusion that already reads `dep` keeps its provider (fused_graph.rs:539-544)
+    auto have = fusions_.at(fusion).dependencies.find(dep);
+    if (have != fusions_.at(fusion).dependencies.end()) return {have->second};
+    std::vector<FusionId> out;
+    for (FusionId p : node_fusions_.at(dep)) {
+        const Fusion& pf = fusions_.at(p);
+        if (pf.core && has(pf.mainloop, dep)) continue;  // mainloop values never leave their kernel
+        auto key = std::make_pair(p, fusion);
+        auto it = cache.find(key);
+        if (it == cache.end()) it = cache.emplace(key, would_create_cycle(p, fusion)).first;
+        if (!it->second) out.push_back(p);
+    }
+    return out;
+}
+
+namespace {
+// itertools' multi_cartesian_product over (dependency, provider) choices: the last dependency varies fastest; no
+// dependencies at all give one empty choice, a dependency nobody can provide gives none.
+void for_each_choice(const std::vector<OpNode>& deps, const std::vector<std::vector<FusionId>>& options,
+                     const std::function<void(const std::map<OpNode, FusionId>&)>& fn) {
+    for (auto& o : options)
+        if (o.empty()) return;
+    std::vector<size_t> idx(deps.size(), 0);
+    for (;;) {
+        std::map<OpNode, FusionId> choice;
+        for (size_t i = 0; i < deps.size(); i++) choice[deps[i]] = options[i][idx[i]];
+        fn(choice);
+        size_t k = deps.size();
+        while (k > 0) {
+            k--;
+            if (++idx[k] < options[k].size()) break;
+            idx[k] = 0;
+            if (k == 0) return;
+        }
+        if (deps.empty()) return;
+    }
+}
+}  // namespace
+
+void FusedGraph::epilogue_expansions(FusionId id, bool has_core, OpNode core, const std::vector<OpNode>& existing_epilogue,
+                                     const std::vector<OpNode>& existing_mainloop, std::vector<Action>& out,
+                                     std::map<std::pair<FusionId, FusionId>, bool>& cache) const {
+    std::vector<OpNode> existing = existing_epilogue;
+    if (has_core) existing.push_back(core);
+    std::set<OpNode> visited;
+    for (OpNode ex : existing) {
+        if (is_terminator(g_->get(ex))) continue;
+        std::vector<std::pair<OpNode, bool>> candidates;
+        for (OpNode n : g_->outbound(ex)) candidates.push_back({n, false});
+        for (OpNode n : g_->inbound(ex)) candidates.push_back({n, true});
+        for (auto& entry : candidates) {
+            const OpNode cand = entry.first;
+            const bool is_pred = entry.second;
+            if (!visited.insert(cand).second) continue;
+            if (is_pred && has_core && ex == core) continue;
+            if (has(existing_epilogue, cand) || has(existing_mainloop, cand) || (has_core && cand == core)) continue;
+            const fir::Op& cop = g_->get(cand);
+            if (!is_epilogue_fusible(cop)) continue;
+            if (is_pred && is_terminator(cop)) continue;
+            if (node_fusions_.at(cand).size() >= kMaxNodeRecomputations) continue;
+            // every dependency the node brings along must come from inside or from a fusion that can feed this
+            // one without closing a cycle
+            std::vector<OpNode> unmet;
+            for (OpNode d : g_->inbound(cand))
+                if (!(has_core && d == core) && !has(existing_epilogue, d)) unmet.push_back(d);
+            std::vector<std::vector<FusionId>> options;
+            for (OpNode d : unmet) options.push_back(dependency_providers(d, id, cache));
+            for_each_choice(unmet, options, [&](const std::map<OpNode, FusionId>& choice) {
+                Action a;
+                a.kind = has_core ? Action::CoreFuseIntoEpilogue : Action::AuxFuse;
+                a.node = cand;
+                a.fusion = id;
+                a.providers = choice;
+                out.push_back(a);
+            });
+        }
+    }
+}
+
+void FusedGraph::mainloop_expansions(FusionId id, OpNode core, const std::vector<OpNode>& existing_mainloop,
+                                     std::vector<Action>& out, std::map<std::pair<FusionId, FusionId>, bool>& cache) const {
+    std::vector<OpNode> existing = existing_mainloop;
+    existing.push_back(core);
+    std::set<OpNode> visited;
+    for (OpNode ex : existing)
+        for (OpNode pred : g_->inbound(ex)) {
+            if (!visited.insert(pred).second) continue;
+            if (has(existing_mainloop, pred)) continue;
+            if (node_fusions_.at(pred).size() >= kMaxNodeRecomputations) continue;
+            if (!is_mainloop_fusible(g_->get(pred))) continue;
+            std::vector<OpNode> unmet;
+            for (OpNode d : g_->inbound(pred))
+                if (!has(existing_mainloop, d)) unmet.push_back(d);
+            std::vector<std::vector<FusionId>> options;
+            for (OpNode d : unmet) options.push_back(dependency_providers(d, id, cache));
+            for_each_choice(unmet, options, [&](const std::map<OpNode, FusionId>& choice) {
+                Action a;
+                a.kind = Action::CoreFuseIntoMainloop;
+                a.node = pred;
+                a.fusion = id;
+                a.providers = choice;
+                out.push_back(a);
+            });
+        }
+}
+
+std::vector<Action> FusedGraph::enumerate_possible_actions() const {
+    std::vector<Action> out;
+    std::map<std::pair<FusionId, FusionId>, bool> cache;
+    for (auto& [id, f] : fusions_) {
+        // edge transitions: read an input from another fusion that also computes it
+        for (auto& [dep, provider] : f.dependencies)
+            for (FusionId alt : node_fusions_.at(dep)) {
+                if (alt == provider) continue;
+                const Fusion& af = fusions_.at(alt);
+                if (af.core && has(af.mainloop, dep)) continue;
+                auto key = std::make_pair(alt, id);
+                auto it = cache.find(key);
+                if (it == cache.end()) it = cache.emplace(key, would_create_cycle(alt, id)).first;
+                if (!it->second) {
+                    Action a;
+                    a.kind = Action::TransitionEdge;
+                    a.fusion = id;
+                    a.node = dep;
+                    a.new_provider = alt;
+                    out.push_back(a);
+                }
+            }
+        if (!f.core && f.fused.size() == 1 && is_input_output(g_->get(f.fused[0]))) continue;
+        if (f.core) {
+            epilogue_expansions(id, true, f.anchor, f.epilogue, f.mainloop, out, cache);
+            mainloop_expansions(id, f.anchor, f.mainloop, out, cache);
+        } else {
+            epilogue_expansions(id, false, fir::kNoOpNode, f.fused, {}, out, cache);
+        }
+    }
+    return out;
+}
+
+void FusedGraph::maybe_remove_collapsed(FusionId id) {
+    auto it = fusions_.find(id);
+    if (it == fusions_.end() || !it->second.dependents.empty()) return;
+    for (OpNode n : it->second.nodes())
+        if (node_fusions_.at(n).size() == 1) return;  // the only place the node is computed
+    Fusion f = it->second;
+    fusions_.erase(it);
+    for (OpNode n : f.nodes()) erase_item(node_fusions_[n], id);
+    for (auto& [dep, provider] : f.dependencies) {
+        auto p = fusions_.find(provider);
+        if (p != fusions_.end()) p->second.dependents.erase({dep, id});
+    }
+}
+
+void FusedGraph::remove_edge(OpNode node, FusionId provider, FusionId consumer) {
+    fusions_.at(provider).dependents.erase({node, consumer});
+    fusions_.at(consumer).dependencies.erase(node);
+    // A provider that no longer hands `node` to anyone, while someone else computes it too, sheds what only
+    // served that output.
+    bool still_provides = false;
+    for (auto& d : fusions_.at(provider).dependents) still_provides = still_provides || d.first == node;
+    if (node_fusions_.at(node).size() > 1 && !still_provides) {
+        Fusion& pf = fusions_.at(provider);
+        std::vector<OpNode> stack;
+        std::set<OpNode> visited;
+        for (auto& d : pf.dependents)
+            if (visited.insert(d.first).second) stack.push_back(d.first);
+        while (!stack.empty()) {
+            OpNode cur = stack.back();
+            stack.pop_back();
+            for (OpNode prev : g_->inbound(cur))
+                if (visited.insert(prev).second && pf.contains(prev)) stack.push_back(prev);
+        }
+        for (OpNode n : pf.nodes())
+            if (!visited.count(n) && !g_->get(n).is_anchor()) {
+                pf.remove_node(n);
+                erase_item(node_fusions_[n], provider);
+            }
+        const auto deps = pf.dependencies;
+        for (auto& [dep, provider2] : deps)
+            if (!visited.count(dep) && fusions_.count(provider) && fusions_.at(provider).dependencies.count(dep))
+                remove_edge(dep, provider2, provider);
+    }
+    maybe_remove_collapsed(provider);
+}
+
+void FusedGraph::apply_action(const Action& a) {
+    if (a.kind == Action::TransitionEdge) {
+        Fusion& f = fusions_.at(a.fusion);
+        const FusionId prev = f.dependencies.at(a.node);
+        f.dependencies.erase(a.node);
+        fusions_.at(prev).dependents.erase({a.node, a.fusion});
+        f.dependencies[a.node] = a.new_provider;
+        fusions_.at(a.new_provider).dependents.insert({a.node, a.fusion});
+        maybe_remove_collapsed(prev);
+        return;
+    }
+    bool had_provider = false;
+    FusionId previous_provider = 0;
+    {
+        auto it = fusions_.at(a.fusion).dependencies.find(a.node);
+        if (it != fusions_.at(a.fusion).dependencies.end()) {
+            had_provider = true;
+            previous_provider = it->second;
+        }
+    }
+    for (auto& [dep, provider] : a.providers) {
+        fusions_.at(a.fusion).dependencies[dep] = provider;
+        fusions_.at(provider).dependents.insert({dep, a.fusion});
+    }
+    if (had_provider) remove_edge(a.node, previous_provider, a.fusion);
+    node_fusions_[a.node].push_back(a.fusion);
+    Fusion& f = fusions_.at(a.fusion);
+    switch (a.kind) {
+        case Action::CoreFuseIntoEpilogue:
+            HE_REQUIRE(f.core, HE_ERR_INVALID, "epilogue fusion into an Aux fusion");
+            insert_sorted(f.epilogue, a.node);
+            break;
+        case Action::CoreFuseIntoMainloop:
+            HE_REQUIRE(f.core, HE_ERR_INVALID, "mainloop fusion into an Aux fusion");
+            insert_sorted(f.mainloop, a.node);
+            break;
+        default:
+            HE_REQUIRE(!f.core, HE_ERR_INVALID, "Aux fusion into a Core fusion");
+            insert_sorted(f.fused, a.node);
+            break;
+    }
+    const std::vector<FusionId> others = node_fusions_.at(a.node);
+    for (FusionId o : others)
+        if (o != a.fusion) maybe_remove_collapsed(o);
+}
+
+// One pass of produce_maximal_fusions for one action kind: a node that lives alone in its fusion moves into a
+// neighbouring fusion when every reader of it can be switched over to the new home (fused_graph.rs:116-155,180-218).
+bool FusedGraph::try_fuse_singletons(Action::Kind kind) {
+    const std::vector<Action> actions = enumerate_possible_actions();
+    for (const Action& a : actions) {
+        if (a.kind != kind) continue;
+        const auto& homes = node_fusions_.at(a.node);
+        if (homes.size() != 1) continue;
+        const FusionId old_home = homes[0];
+        if (fusions_.at(old_home).nodes().size() > 1) continue;
+        std::set<FusionId> readers;
+        for (auto& d : fusions_.at(old_home).dependents) readers.insert(d.second);
+        FusedGraph trial = *this;
+        trial.apply_action(a);
+        bool ok = true;
+        for (FusionId r : readers) {
+            Action want;
+            want.kind = Action::TransitionEdge;
+            want.fusion = r;
+            want.new_provider = a.fusion;
+            want.node = a.node;
+            const std::vector<Action> legal = trial.enumerate_possible_actions();
+            if (std::find(legal.begin(), legal.end(), want) == legal.end()) {
+                ok = false;
+                break;
+            }
+            trial.apply_action(want);
+        }
+        if (!ok) continue;
+        *this = std::move(trial);
+        return true;
+    }
+    return false;
+}
+
+void FusedGraph::produce_maximal_fusions() {
+    for (;;) {
+        if (try_fuse_singletons(Action::CoreFuseIntoEpilogue)) continue;
+        if (try_fuse_singletons(Action::AuxFuse)) continue;
+        break;
+    }
+    assert_invariants();
+}
+
+void FusedGraph::clean() {
+    assert_invariants(false);
+    // keep what some Consumer transitively reads
+    std::vector<FusionId> stack;
+    std::set<FusionId> visited;
+    for (auto& [id, f] : fusions_)
+        if (f.is_input_output(*g_) && g_->get(f.nodes()[0]).kind == OpKind::Consumer) {
+            stack.push_back(id);
+            visited.insert(id);
+        }
+    while (!stack.empty()) {
+        FusionId cur = stack.back();
+        stack.pop_back();
+        for (auto& d : fusions_.at(cur).dependencies)
+            if (visited.insert(d.second).second) stack.push_back(d.second);
+    }
+    std::vector<FusionId> remove;
+    for (auto& kv : fusions_)
+        if (!visited.count(kv.first)) remove.push_back(kv.first);
+    for (FusionId id : remove) {
+        fusions_.erase(id);
+        for (auto& kv : node_fusions_) erase_item(kv.second, id);
+        for (auto& kv : fusions_) {
+            for (auto it = kv.second.dependencies.begin(); it != kv.second.dependencies.end();)
+                it = it->second == id ? kv.second.dependencies.erase(it) : std::next(it);
+            for (auto it = kv.second.dependents.begin(); it != kv.second.dependents.end();)
+                it = it->second == id ? kv.second.dependents.erase(it) : std::next(it);
+        }
+    }
+    // Fusion::clean (fused_graph.rs:1089-1132): drop recomputed members nothing downstream of the fusion needs
+    for (auto& entry : fusions_) {
+        const FusionId id = entry.first;
+        Fusion& f = entry.second;
+        std::vector<OpNode> st;
+        std::set<OpNode> seen;
+        for (auto& d : f.dependents)
+            if (seen.insert(d.first).second) st.push_back(d.first);
+        while (!st.empty()) {
+            OpNode cur = st.back();
+            st.pop_back();
+            for (OpNode pred : g_->inbound(cur))
+                if (seen.insert(pred).second && f.contains(pred)) st.push_back(pred);
+        }
+        auto prune = [&](std::vector<OpNode>& v) {
+            std::vector<OpNode> kept;
+            for (OpNode n : v) {
+                if (!seen.count(n) && node_fusions_.at(n).size() > 1) erase_item(node_fusions_[n], id);
+                else kept.push_back(n);
+            }
+            v = kept;
+        };
+        if (f.core) prune(f.epilogue);
+        else prune(f.fused);
+    }
+}
+
+std::vector<FusionId> FusedGraph::topo_sort() const {
+    std::vector<FusionId> result, stack;
+    std::set<FusionId> visited;
+    for (auto& [id, f] : fusions_)
+        if (f.dependencies.empty()) {
+            stack.push_back(id);
+            visited.insert(id);
+        }
+    while (!stack.empty()) {
+        FusionId cur = stack.back();
+        stack.pop_back();
+        result.push_back(cur);
+        for (auto& d : fusions_.at(cur).dependents) {
+            bool ready = true;
+            for (auto& dep : fusions_.at(d.second).dependencies) ready = ready && has(result, dep.second);
+            if (ready && visited.insert(d.second).second) stack.push_back(d.second);
+        }
+    }
+    return result;
+}
+
+void FusedGraph::assert_invariants(bool every_node_placed) const {
+    for (auto& [id, f] : fusions_)
+        for (OpNode n : f.nodes()) {
+            HE_REQUIRE(has(node_fusions_.at(n), id), HE_ERR_INTERNAL, "node %llu does not list fusion %llu", (unsigned long long)n,
+                       (unsigned long long)id);
+            for (OpNode dep : g_->inbound(n)) {
+                if (f.contains(dep)) continue;
+                auto it = f.dependencies.find(dep);
+                HE_REQUIRE(it != f.dependencies.end(), HE_ERR_INTERNAL, "fusion %llu reads node %llu from nowhere", (unsigned long long)id,
+                           (unsigned long long)dep);
+                const Fusion& p = fusions_.at(it->second);
+                HE_REQUIRE(p.contains(dep), HE_ERR_INTERNAL, "provider %llu does not compute node %llu", (unsigned long long)it->second,
+                           (unsigned long long)dep);
+                HE_REQUIRE(p.dependents.count({dep, id}), HE_ERR_INTERNAL, "provider %llu does not list reader %llu of node %llu",
+                           (unsigned long long)it->second, (unsigned long long)id, (unsigned long long)dep);
+            }
+        }
+    for (auto& [n, fs] : node_fusions_)
+        for (FusionId f : fs) HE_REQUIRE(fusions_.at(f).contains(n), HE_ERR_INTERNAL, "stale fusion list of node %llu", (unsigned long long)n);
+    if (every_node_placed)
+        for (OpNode n : g_->nodes()) HE_REQUIRE(!node_fusions_.at(n).empty(), HE_ERR_INTERNAL, "node %llu is in no fusion", (unsigned long long)n);
+}
+
+uint64_t FusedGraph::state_hash() const {
+    uint64_t h = 0;
+    for (auto& kv : fusions_) {
+        const std::string k = kv.second.key();
+        h ^= fnv1a(k.data(), k.size());
+    }  // ids stay out: equal partitions are one state
+    return h;
+}
+
+namespace {
+std::string op_text(const fir::Op& op) {
+    static const char* un[] = {"Neg", "Relu", "Gelu", "Tanh", "Exp", "Ln", "Sqrt", "AddConstant", "MulConstant", "PowConstant"};
+    static const char* bin[] = {"Add", "Sub", "Mul", "Div", "Pow", "Drelu"};
+    static const char* dep[] = {"Rows", "Columns", "Item", "Batch"};
+    std::ostringstream s;
+    switch (op.kind) {
+        case OpKind::Producer: s << "Producer"; break;
+        case OpKind::Consumer: s << "Consumer { x: n" << op.a << " }"; break;
+        case OpKind::Constant: s << "Constant { value: " << op.value << " }"; break;
+        case OpKind::Matmul: s << "Matmul { a: n" << op.a << ", b: n" << op.b << " }"; break;
+        case OpKind::UnaryPointwise:
+            s << "UnaryPointwise { x: n" << op.a << ", op: " << un[op.sub_op];
+            if (op.sub_op >= (int)fir::UnaryOp::AddConstant) s << "(" << op.constant << ")";
+            s << " }";
+            break;
+        case OpKind::BinaryPointwise: s << "BinaryPointwise { lhs: n" << op.a << ", rhs: n" << op.b << ", op: " << bin[op.sub_op] << " }"; break;
+        case OpKind::Reduction: s << "Reduction { x: n" << op.a << ", depth: " << dep[(int)op.depth] << " }"; break;
+        case OpKind::Broadcast: s << "Broadcast { x: n" << op.a << ", axis: " << op.axis << ", amount: " << op.amount << " }"; break;
+        case OpKind::Transpose: s << "Transpose { x: n" << op.a << " }"; break;
+    }
+    return s.str();
+}
+}  // namespace
+
+std::string FusedGraph::describe() const {
+    std::ostringstream s;
+    for (FusionId id : topo_sort()) {
+        const Fusion& f = fusions_.at(id);
+        if (f.is_input_output(*g_)) continue;
+        s << "FusionId(" << id << "):\n";
+        for (auto& d : f.dependents) s << "Dependent: FusionId(" << d.second << ") uses n" << d.first << "\n";
+        if (!f.core) {
+            s << "---Aux---\n";
+            for (OpNode n : f.fused) s << "\tn" << n << " = " << op_text(g_->get(n)) << "\n";
+        } else {
+            const fir::Op& mm = g_->get(f.anchor);
+            s << "---Core(n" << f.anchor << " = matmul(n" << mm.a << ", n" << mm.b << "))---\n\tMainloop:\n";
+            for (OpNode n : f.mainloop) s << "\t\tn" << n << " = " << op_text(g_->get(n)) << "\n";
+            s << "\tEpilogue:\n";
+            for (OpNode n : f.epilogue) s << "\t\tn" << n << " = " << op_text(g_->get(n)) << "\n";
+        }
+        s << "\n";
+    }
+    return s.str();
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Cost models
+// ---------------------------------------------------------------------------------------------------------
+namespace {
+uint64_t elements(const fir::OpGraph& g, OpNode n) {
+    const fir::Shape3& s = g.shape(n);
+    return (uint64_t)s[0] * s[1] * s[2];
+}
+}  // namespace
+
+double naive_cost(const FusedGraph& fg, const CostParams& p) {
+    const fir::OpGraph& g = fg.opgraph();
+    const double mem = 1.0 / p.memory_elements_per_s, tflop = 1.0 / p.tensor_flops, rflop = 1.0 / p.regular_flops;
+    double cost = 0;
+    for (auto& [id, f] : fg.fusions()) {
+        if (f.is_input_output(g)) continue;
+        std::vector<OpNode> stack;
+        std::set<OpNode> visited;
+        for (auto& d : f.dependents)
+            if (visited.insert(d.first).second) stack.push_back(d.first);
+        std::sort(stack.begin(), stack.end());
+        uint64_t tensor = 0, regular = 0;
+        while (!stack.empty()) {
+            OpNode cur = stack.back();
+            stack.pop_back();
+            bool saved = false;
+            for (auto& d : f.dependents) saved = saved || d.first == cur;
+            if (saved) cost += mem * (double)elements(g, cur);
+            const fir::Op& op = g.get(cur);
+            switch (op.kind) {
+                case OpKind::Matmul: tensor += 2 * elements(g, op.a) * g.shape(op.b)[1]; break;  // as written: dim(1) of b
+                case OpKind::UnaryPointwise:
+                case OpKind::Reduction: regular += 2 * elements(g, op.a); break;
+                case OpKind::BinaryPointwise: regular += 3 * elements(g, op.a); break;
+                default: break;
+            }
+            for (OpNode prev : g.inbound(cur)) {
+                if (!visited.insert(prev).second) continue;
+                if (f.contains(prev)) stack.push_back(prev);
+                else if (f.dependencies.count(prev)) cost += mem * (double)elements(g, prev);
+            }
+        }
+        cost += (double)tensor * tflop + (double)regular * rflop;
+    }
+    return cost;
+}
+
+namespace {
+std::vector<OpNode> ancestors_in_fusion(const Fusion& f, const fir::OpGraph& g, OpNode node) {
+    std::vector<OpNode> out{node}, stack{node};
+    std::set<OpNode> visited{node};
+    while (!stack.empty()) {
+        OpNode cur = stack.back();
+        stack.pop_back();
+        for (OpNode pred : g.inbound(cur))
+            if (f.contains(pred) && visited.insert(pred).second) {
+                out.push_back(pred);
+                stack.push_back(pred);
+            }
+    }
+    return out;
+}
+}  // namespace
+
+double analytical_cost(const FusedGraph& fg) {
+    const fir::OpGraph& g = fg.opgraph();
+    double cost = 0;
+    for (auto& [id, f] : fg.fusions()) {
+        if (f.is_input_output(g)) continue;
+        std::vector<OpNode> stack;
+        std::set<OpNode> visited;
+        for (auto& d : f.dependents)
+            if (visited.insert(d.first).second) stack.push_back(d.first);
+        std::sort(stack.begin(), stack.end());
+        uint64_t e_c = 0, e_m = 0, m_ca = 0, m_cb = 0, r_a = 0, r_b = 0;
+        std::vector<OpNode> ma, mb;
+        if (f.core) {
+            const fir::Op& mm = g.get(f.anchor);
+            ma = ancestors_in_fusion(f, g, mm.a);
+            mb = ancestors_in_fusion(f, g, mm.b);
+            r_a = (g.shape(mm.a)[1] + 255) / 256;
+            r_b = (g.shape(mm.b)[2] + 127) / 128;
+        }
+        while (!stack.empty()) {
+            OpNode cur = stack.back();
+            stack.pop_back();
+            bool saved = false;
+            for (auto& d : f.dependents) saved = saved || d.first == cur;
+            if (saved) e_m += 2;
+            uint64_t& target = has(ma, cur) ? m_ca : has(mb, cur) ? m_cb : e_c;
+            const fir::Op& op = g.get(cur);
+            if (op.kind == OpKind::UnaryPointwise) {
+                switch ((fir::UnaryOp)op.sub_op) {
+                    case fir::UnaryOp::Neg:
+                    case fir::UnaryOp::Relu:
+                    case fir::UnaryOp::AddConstant:
+                    case fir::UnaryOp::MulConstant: target += 1; break;
+                    case fir::UnaryOp::PowConstant: target += op.constant == 2.0f ? 1 : 10; break;
+                    case fir::UnaryOp::Exp: target += 15; break;
+                    case fir::UnaryOp::Gelu: target += 8; break;
+                    case fir::UnaryOp::Ln: target += 12; break;
+                    case fir::UnaryOp::Sqrt: target += 13; break;
+                    case fir::UnaryOp::Tanh: target += 23; break;
+                }
+            } else if (op.kind == OpKind::Reduction) {
+                target += 10;
+            } else if (op.kind == OpKind::BinaryPointwise) {
+                switch ((fir::BinaryOp)op.sub_op) {
+                    case fir::BinaryOp::Add:
+                    case fir::BinaryOp::Sub:
+                    case fir::BinaryOp::Mul: target += 1; break;
+                    case fir::BinaryOp::Div: target += 5; break;
+                    case fir::BinaryOp::Pow: target += 24; break;
+                    case fir::BinaryOp::Drelu: target += 2; break;
+                }
+            }
+            for (OpNode prev : g.inbound(cur)) {
+                if (!visited.insert(prev).second) continue;
+                if (f.contains(prev)) stack.push_back(prev);
+                else if (f.dependencies.count(prev)) e_m += 2;
+            }
+            // as the reference writes it, the fitted terms are added once per visited node (cost_model.rs:204-229)
+            const uint64_t m_c = r_a * m_ca + r_b * m_cb;
+            const double alpha_c = 1.32e-6, alpha_m = 2.30e-5, beta_0 = 0.0, beta_1 = 6.55e-5, alpha_1 = 3.37e-6, gamma = 4.0,
+                         alpha_2 = 6.60e-6, beta_2 = beta_1 + gamma * alpha_1 - alpha_2 * gamma;
+            const double c_epilogue = alpha_c * (double)e_c + alpha_m * (double)e_m;
+            const double c_mainloop = m_c == 0 ? beta_0 : (double)m_c < gamma ? beta_1 + alpha_1 * (double)m_c : beta_2 + alpha_2 * (double)m_c;
+            cost += c_epilogue + c_mainloop;
+        }
+    }
+    return cost;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Search
+// ---------------------------------------------------------------------------------------------------------
+SearchResult minimize_cost(std::shared_ptr<const fir::OpGraph> g, Objective objective, const CostParams& p, size_t max_states) {
+    FusedGraph initial = FusedGraph::identity(g);
+    initial.produce_maximal_fusions();
+    auto cost_of = [&](const FusedGraph& fg) { return objective == Objective::Analytical ? analytical_cost(fg) : naive_cost(fg, p); };
+    if (objective == Objective::Maximal) return {initial, naive_cost(initial, p), 1};
+
+    bool have_best = false, best_updated = false;
+    FusedGraph best = initial;
+    double best_cost = 0;
+    std::set<uint64_t> visited;
+    size_t states = 0, total_states = 0;
+    std::function<void(const FusedGraph&, int)> visit = [&](const FusedGraph& cur, int depth) {
+        const double c = cost_of(cur);
+        if (!have_best) {
+            best = cur;
+            best_cost = c;
+            have_best = true;
+        } else if (c < best_cost) {
+            best = cur;
+            best_cost = c;
+            best_updated = true;
+        }
+        if (depth == 7 || states >= max_states) return;
+        for (const Action& a : cur.enumerate_possible_actions()) {
+            FusedGraph next = cur;
+            next.apply_action(a);
+            if (visited.insert(next.state_hash()).second) {
+                states++;
+                visit(next, depth + 1);
+                if (states >= max_states) return;
+            }
+        }
+    };
+    for (;;) {
+        states = 0;
+        visit(initial, 0);
+        total_states += states;
+        initial = best;
+        initial.clean();
+        if (!best_updated) break;
+        best_updated = false;
+        visited.clear();
+    }
+    best.clean();
+    return {best, best_cost, total_states};
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Subdivision
+// ---------------------------------------------------------------------------------------------------------
+std::vector<std::set<std::pair<OpNode, NodePortion>>> subdivide(const fir::OpGraph& g) {
+    std::vector<std::set<std::pair<OpNode, NodePortion>>> out;
+    std::set<OpNode> nonanchor, anchor_mainloop, anchor_epilogue;
+    for (;;) {
+        OpNode start = fir::kNoOpNode;
+        for (OpNode n : g.nodes()) {
+            if (is_input_output(g.get(n))) continue;
+            const bool open = g.get(n).is_anchor() ? (!anchor_epilogue.count(n) || !anchor_mainloop.count(n)) : !nonanchor.count(n);
+            if (open) {
+                start = n;
+                break;
+            }
+        }
+        if (start == fir::kNoOpNode) break;
+        const NodePortion portion =
+            g.get(start).is_anchor() ? (!anchor_epilogue.count(start) ? NodePortion::Epilogue : NodePortion::Mainloop) : NodePortion::Full;
+        std::set<std::pair<OpNode, NodePortion>> sub{{start, portion}};
+        std::vector<std::pair<OpNode, NodePortion>> stack{{start, portion}};
+        while (!stack.empty()) {
+            auto [cur, cur_portion] = stack.back();
+            stack.pop_back();
+            std::vector<OpNode> neighbors;
+            if (cur_portion != NodePortion::Epilogue) neighbors = g.inbound(cur);
+            if (cur_portion != NodePortion::Mainloop) neighbors.insert(neighbors.end(), g.outbound(cur).begin(), g.outbound(cur).end());
+            for (OpNode nb : neighbors) {
+                if (is_input_output(g.get(nb))) continue;
+                NodePortion np = NodePortion::Full;
+                if (g.get(nb).is_anchor()) np = has(g.outbound(cur), nb) ? NodePortion::Mainloop : NodePortion::Epilogue;
+                if (sub.insert({nb, np}).second) stack.push_back({nb, np});
+            }
+        }
+        for (auto& [n, np] : sub) {
+            if (np == NodePortion::Mainloop) anchor_mainloop.insert(n);
+            else if (np == NodePortion::Epilogue) anchor_epilogue.insert(n);
+            else {
+                anchor_epilogue.insert(n);
+                anchor_mainloop.insert(n);
+                nonanchor.insert(n);
+            }
+        }
+        out.push_back(sub);
+    }
+    return out;
+}
+
+}  // namespace he::fsearch

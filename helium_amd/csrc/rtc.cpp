@@ -101,6 +101,15 @@ std::shared_ptr<const std::vector<char>> rtc_compile(const std::string& source, 
         }
     }
 
+    if (const char* dump = getenv("HELIUM_HIP_DUMP_DIR")) {
+        // Written before compiling, so that a source that crashes the compiler is still on disk. The counterpart
+        // of the reference's `cuda-debug` feature, which writes every JIT source to kernel/
+        // (helium/src/cuda/kernel_jit.rs:145-151).
+        static std::atomic<int> id{0};
+        mkdir(dump, 0755);
+        std::ofstream f(strfmt("%s/jit_%s_%d.hip", dump, name.c_str(), id++));
+        f << source;
+    }
     hiprtcProgram prog;
     hiprtcResult r = hiprtcCreateProgram(&prog, source.c_str(), (name + ".hip").c_str(), 0, nullptr, nullptr);
     HE_REQUIRE(r == HIPRTC_SUCCESS, HE_ERR_RTC, "hiprtcCreateProgram: %s", hiprtcGetErrorString(r));
@@ -137,15 +146,6 @@ std::shared_ptr<const std::vector<char>> rtc_compile(const std::string& source, 
         }
         rename(tmp.c_str(), path.c_str());
     }
-    if (const char* dump = getenv("HELIUM_HIP_DUMP_DIR")) {
-        // The counterpart of the reference's `cuda-debug` feature, which writes every JIT source to kernel/
-        // (helium/src/cuda/kernel_jit.rs:145-151).
-        static std::atomic<int> id{0};
-        mkdir(dump, 0755);
-        std::ofstream f(strfmt("%s/jit_%s_%d.hip", dump, name.c_str(), id++));
-        f << source;
-    }
-
     auto sp = std::make_shared<const std::vector<char>>(std::move(blob));
     std::lock_guard<std::mutex> lk(g_mu);
     g_cache[key] = sp;

@@ -290,6 +290,34 @@ int he_plan_destroy(he_plan_t plan);
  * tensor is a new reference the caller frees. */
 int he_execute_graph(he_graph_t graph, const uint32_t* input_nodes, const he_tensor_t* input_tensors, int num_inputs,
                      uint32_t* output_nodes, he_tensor_t* output_tensors, int max_outputs, int* num_outputs);
+/* ---- 7. Fusion search over a fusion-IR graph ------------------------------------------------------------
+ * helium-playground/src/fused_graph.rs (FusedGraph: identity, enumerate_possible_actions, apply_action,
+ * produce_maximal_fusions, clean, topo_sort), cost_model.rs (naive_cost_function, analytical_cost_function,
+ * minimize_cost_function) and subdivision.rs (subdivide). The plan holds the chosen Core(mainloop, anchor, epilogue)
+ * and Aux fusions; each becomes one kernel (he_fused_kernel_create's generators) and he_fusion_plan_execute runs
+ * them in dependency order with pooled temporaries. */
+typedef struct he_fusion_plan_s* he_fusion_plan_t;
+enum { HE_FUSE_MAXIMAL = 0, HE_FUSE_MIN_NAIVE_COST = 1, HE_FUSE_MIN_ANALYTICAL_COST = 2 };
+enum { HE_FUSION_ROLE_MAINLOOP = 0, HE_FUSION_ROLE_EPILOGUE = 1, HE_FUSION_ROLE_ANCHOR = 2, HE_FUSION_ROLE_AUX = 3 };
+/* objective HE_FUSE_MAXIMAL: produce_maximal_fusions only (fused_graph.rs:113-223); otherwise minimize_cost_function
+ * (cost_model.rs:256-343) with the naive model on MI355X rates or the analytical model. */
+int he_fusion_search(he_fgraph_t graph, int objective, he_fusion_plan_t* plan);
+int he_fusion_plan_num_fusions(he_fusion_plan_t plan, int* count);   /* kernels, in execution order */
+int he_fusion_plan_fusion_info(he_fusion_plan_t plan, int index, int32_t* is_core, uint64_t* anchor, uint64_t* nodes,
+                               int32_t* roles, int capacity, int* count);
+const char* he_fusion_plan_describe(he_fusion_plan_t plan);           /* FusedGraph::print (fused_graph.rs:1060-1068) */
+/* objective 1: naive model (reference_constants != 0: the constants of cost_model.rs:10-12), 2: analytical model */
+int he_fusion_plan_cost(he_fusion_plan_t plan, int objective, int reference_constants, double* cost, uint64_t* states_visited);
+int he_fusion_plan_precompile(he_fusion_plan_t plan);
+/* Producers and Consumers of the whole graph are bound by node id; values between kernels are bf16 (f32 for
+ * reductions) in pooled device memory. */
+int he_fusion_plan_execute(he_fusion_plan_t plan, const uint64_t* producer_nodes, void* const* producer_ptrs, int num_producers,
+                           const uint64_t* consumer_nodes, void* const* consumer_ptrs, int num_consumers, he_stream_t stream);
+int he_fusion_plan_destroy(he_fusion_plan_t plan);
+/* subdivide (subdivision.rs:24-113): entry k is node nodes[k] as portion portions[k] (0 mainloop, 1 epilogue, 2 full)
+ * of subdivision subdivision_of[k]. */
+int he_fgraph_subdivide(he_fgraph_t graph, uint64_t* nodes, int32_t* portions, int32_t* subdivision_of, int capacity, int* count);
+
 /* Backend options. HE_OPT_FUSE_MATMUL_EPILOGUE (default 1): pointwise / reduce ops that follow a Matmul join its
  * instruction and run as the fused GEMM's epilogue (the MatmulGenerator path, matmul.rs:88-130); 0 restores the
  * grouping of helium/src/cuda/instr/cudnn_graph.rs:319-321, where a matmul instruction never fuses. */

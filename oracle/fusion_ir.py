@@ -104,8 +104,10 @@ def matmul(a, b):
     return np.matmul(a.astype(np.float64), b.astype(np.float64)).astype(np.float32)
 
 
-def evaluate(nodes, inputs, round_mainloop_to=None):
+def evaluate(nodes, inputs, round_mainloop_to=None, materialize=None):
     """inputs: {producer id: storage array}. Returns ({id: f32 array}, {id: shape}).
+    materialize: {node id: storage dtype} of values that cross a kernel boundary when the graph runs as several
+    kernels; they are rounded to that dtype where they are produced.
     round_mainloop_to: storage dtype the Matmul operands are rounded to after mainloop ops (the fused GEMM casts
     the mainloop chain's result back to the load type before the MMA, helium-kernel-generator/src/generators/
     matmul/sm80.rs:418-437); None leaves them in f32."""
@@ -138,6 +140,8 @@ def evaluate(nodes, inputs, round_mainloop_to=None):
         else:
             raise ValueError(op)
         assert list(val[i].shape) == list(shapes[i]), (n, val[i].shape, shapes[i])
+        if materialize and i in materialize:
+            val[i] = nm.from_storage(nm.to_storage(val[i], materialize[i]), materialize[i], val[i].shape)
     return val, shapes
 
 

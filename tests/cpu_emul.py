@@ -130,6 +130,7 @@ static inline emu_s16x4 emu_tr16(const emu_s16x4* p) {
 #define __builtin_amdgcn_wave_barrier() pthread_barrier_wait(&g_bar)
 #define __expf expf
 #define HE_FAST_RCP(x) (1.0f / (x))
+#define HE_OPAQUE(x) (x)
 #define __logf logf
 #define __sinf sinf
 #define __cosf cosf
