@@ -36,6 +36,16 @@ __device__ __forceinline__ float he_opaque(float x) { asm volatile("" : "+v"(x))
 #ifndef HE_FAST_RCP
 #define HE_FAST_RCP(x) __builtin_amdgcn_rcpf(x)
 #endif
+#ifndef HE_WS_STORE
+// Cross-block exchange through scratch memory. Device-scope atomic accesses go past the per-XCD L2 caches, so a
+// partial result written this way and waited for (HE_WS_DRAIN: all of the wave's memory operations have completed)
+// before the block takes its ticket is in memory by the time any other block can see that ticket. A device-scope
+// fence would give the same guarantee by writing back and invalidating the whole L2, once per wave.
+#define HE_WS_STORE(p, v) __hip_atomic_store((p), (v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+#define HE_WS_LOAD(p) __hip_atomic_load((p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+#define HE_WS_TICKET(p) __hip_atomic_fetch_add((p), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+#define HE_WS_DRAIN() __builtin_amdgcn_s_waitcnt(0)
+#endif
 template <class T, int N> struct Vec { typedef T type __attribute__((ext_vector_type(N))); };
 template <class T> struct Vec<T, 1> { typedef T type; };
 
@@ -492,9 +502,63 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
     s << "extern \"C\" __global__ __launch_bounds__(" << threads << ") void " << entry << "(";
     for (size_t a = 0; a < p.args.size(); a++)
         s << (a ? ", " : "") << (p.args[a].is_output ? "" : "const ") << c_type(p.args[a].dtype) << "* __restrict__ a" << a;
+    // Reductions whose terms come from several blocks: each block parks its partial result in scratch and takes a
+    // ticket; the last one to arrive folds the partials in block order (same result on every run) and writes the
+    // output, so the output needs no initial value and sees one store instead of one atomic per block.
+    struct WsUse {
+        bool on = false;
+        uint64_t foff = 0, coff = 0, coff1 = 0;
+        int64_t group = 0, ngroups = 0;  // scalar reductions with many blocks: tickets in two levels
+    };
+    // Tickets on one address are served one after another (about 20 ns each), and so are those on neighbours within a
+    // cache line: every counter gets a line of its own, and a reduction over many blocks counts arrivals in groups
+    // of about sqrt(blocks), the last arrival of a group carrying the group's ticket to the second level.
+    //
+    // The last block's way out is a chain of memory round trips (partials land, ticket, partials back, result), a few
+    // microseconds that nothing overlaps when all blocks end together. A short launch still gains, because the fill
+    // kernel and its dependent launch cost more than that; a long one is better off with one atomic per block and
+    // the fill (measured: [1,4096,4096] f32 with two reductions 50 us with atomics, 54 us with tickets).
+    const uint64_t CS = 32;  // counter stride in u32
+    bool tickets = B * M * N <= (int64_t)1 << 21;
+    if (const char* env = getenv("HELIUM_HIP_REDUCE")) tickets = std::string(env) == "ticket";
+    std::vector<WsUse> ws(p.outs.size());
+    std::vector<char> atomics(p.outs.size(), 0);  // reductions over several blocks that accumulate with atomics
+    for (size_t oi = 0; oi < p.outs.size(); oi++) {
+        const Out& o = p.outs[oi];
+        if (!o.reduce) continue;
+        if (!tickets) {
+            atomics[oi] = o.fold_n ? (o.fold_m ? gx * gy * o.b_div > 1 : false) : gy > 1;
+            continue;
+        }
+        if (o.fold_m && !o.fold_n && gy > 1) {
+            ws[oi].on = true;
+            ws[oi].foff = L.ws_floats;
+            ws[oi].coff = L.ws_counters;
+            L.ws_floats += (uint64_t)grid * TX * NV;
+            L.ws_counters += (uint64_t)B * gx * CS;
+        } else if (o.fold_m && o.fold_n && gx * gy * o.b_div > 1) {
+            const int64_t per = gx * gy * o.b_div, outs_n = B / o.b_div;
+            ws[oi].on = true;
+            ws[oi].foff = L.ws_floats;
+            ws[oi].coff = L.ws_counters;
+            L.ws_floats += (uint64_t)grid;
+            L.ws_counters += (uint64_t)outs_n * CS;
+            if (per > 64) {
+                int64_t G = 8;
+                while (G * G < per) G *= 2;
+                ws[oi].group = G;
+                ws[oi].ngroups = (per + G - 1) / G;
+                ws[oi].coff1 = L.ws_counters;
+                L.ws_counters += (uint64_t)outs_n * ws[oi].ngroups * CS;
+            }
+        }
+    }
+    const bool any_ws = L.ws_counters > 0;
+    if (any_ws) s << ", float* wsf, u32* wsc";
     s << ") {\n";
     if (any_col && TY > 1) s << "__shared__ float col_red[TY * TX * NV];\n";
     if (any_scalar) s << "__shared__ float blk_red[" << threads / 64 << "];\n";
+    if (any_ws) s << "__shared__ u32 ticket_s[" << p.outs.size() << "];\n";
     s << "u32 t = blockIdx.x;\nconst u32 tile_x = t % " << gx << "u; t /= " << gx << "u;\nconst u32 tile_y = t % " << gy
       << "u; t /= " << gy << "u;\nconst u32 b = t;\n";
     {
@@ -559,11 +623,19 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
         if (!(o.reduce && o.fold_n && !o.fold_m)) continue;
         const int width = std::min(TX, 64);
         s << "{ float r = wave_reduce<" << (int)o.rop << ", " << width << ">(rr" << oi << ");\n";
-        s << "if ((threadIdx.x % " << width << ") == 0 && m < DIM_M && col_ok) atomic_red<" << (int)o.rop << ">(a" << o.arg
-          << " + (size_t)b * " << M << "ull + m, r); }\n";
+        if (gx == 1 && TX <= 64)  // one wave segment holds the whole row
+            s << "if ((threadIdx.x % " << width << ") == 0 && m < DIM_M && col_ok) a" << o.arg << "[(size_t)b * " << M << "ull + m] = r; }\n";
+        else
+            s << "if ((threadIdx.x % " << width << ") == 0 && m < DIM_M && col_ok) atomic_red<" << (int)o.rop << ">(a" << o.arg
+              << " + (size_t)b * " << M << "ull + m, r); }\n";
     }
     s << "}\n";  // row loop
-    // column reductions
+    // Phase 1: every block finishes its own partial of each reduction. What no other block contributes to is stored
+    // straight to the output; the rest is parked in scratch.
+    int n_tickets = 0;
+    std::vector<int> ticket_of(p.outs.size(), -1);
+    for (size_t oi = 0; oi < p.outs.size(); oi++)
+        if (ws[oi].on) ticket_of[oi] = n_tickets++;
     for (size_t oi = 0; oi < p.outs.size(); oi++) {
         const Out& o = p.outs[oi];
         if (!(o.reduce && o.fold_m && !o.fold_n)) continue;
@@ -573,23 +645,93 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
               << "[k];\nfor (u32 y = 1; y < TY; y++) r = red_op<" << (int)o.rop << ">(r, col_red[(y * TX + tx) * NV + k]);\nrc"
               << oi << "[k] = r; } }\n";
         }
-        s << "if (ty == 0 && col_ok) {\n#pragma unroll\nfor (int k = 0; k < NV; k++) atomic_red<" << (int)o.rop << ">(a" << o.arg
-          << " + (size_t)b * " << N << "ull + n0 + k, rc" << oi << "[k]); }\n";
+        if (atomics[oi])
+            s << "if (ty == 0 && col_ok) {\n#pragma unroll\nfor (int k = 0; k < NV; k++) if (n0 + k < DIM_N) atomic_red<" << (int)o.rop << ">(a" << o.arg
+              << " + (size_t)b * " << N << "ull + n0 + k, rc" << oi << "[k]); }\n";
+        else if (!ws[oi].on)
+            s << "if (ty == 0 && col_ok) {\n#pragma unroll\nfor (int k = 0; k < NV; k++) if (n0 + k < DIM_N) a" << o.arg << "[(size_t)b * " << N
+              << "ull + n0 + k] = rc" << oi << "[k]; }\n";
+        else
+            s << "if (ty == 0) {\n#pragma unroll\nfor (int k = 0; k < NV; k++) HE_WS_STORE(wsf + " << ws[oi].foff
+              << "ull + (size_t)blockIdx.x * (TX * NV) + tx * NV + k, rc" << oi << "[k]); }\n";
     }
-    // scalar reductions
     for (size_t oi = 0; oi < p.outs.size(); oi++) {
         const Out& o = p.outs[oi];
         if (!(o.reduce && o.fold_m && o.fold_n)) continue;
         s << "{ float r = wave_reduce<" << (int)o.rop << ", 64>(rs" << oi << ");\n__syncthreads();\nif ((threadIdx.x & 63) == 0) blk_red[threadIdx.x >> 6] = r;\n__syncthreads();\n";
         s << "if (threadIdx.x == 0) { r = blk_red[0];\nfor (int w = 1; w < " << threads / 64 << "; w++) r = red_op<"
-          << (int)o.rop << ">(r, blk_red[w]);\natomic_red<" << (int)o.rop << ">(a" << o.arg << " + (size_t)(b / " << o.b_div
-          << "u), r); } }\n";
+          << (int)o.rop << ">(r, blk_red[w]);\n";
+        if (atomics[oi])
+            s << "atomic_red<" << (int)o.rop << ">(a" << o.arg << " + (size_t)(b / " << o.b_div << "u), r); } }\n";
+        else if (!ws[oi].on)
+            s << "a" << o.arg << "[b / " << o.b_div << "u] = r; } }\n";
+        else
+            s << "HE_WS_STORE(wsf + " << ws[oi].foff << "ull + blockIdx.x, r); } }\n";
+    }
+    if (n_tickets) {
+        // Phase 2: once every wave's partials have landed, one thread takes the block's ticket of each reduction.
+        s << "HE_WS_DRAIN();\n__syncthreads();\nif (threadIdx.x == 0) {\n";
+        for (size_t oi = 0; oi < p.outs.size(); oi++) {
+            if (!ws[oi].on) continue;
+            const Out& o = p.outs[oi];
+            const int j = ticket_of[oi];
+            if (!o.fold_n) {
+                s << "const u32 tk" << j << " = HE_WS_TICKET(wsc + " << ws[oi].coff << "ull + (size_t)(b * " << gx << "u + tile_x) * " << CS << "u) == "
+                  << gy - 1 << "u;\n";
+                continue;
+            }
+            const int64_t per = gx * gy * o.b_div;
+            if (!ws[oi].group) {
+                s << "const u32 tk" << j << " = HE_WS_TICKET(wsc + " << ws[oi].coff << "ull + (size_t)(b / " << o.b_div << "u) * " << CS << "u) == "
+                  << per - 1 << "u;\n";
+                continue;
+            }
+            s << "u32 tk" << j << " = 0u;\n{ const u32 q = b / " << o.b_div << "u, lb = blockIdx.x - q * " << per << "u, grp = lb / " << ws[oi].group
+              << "u;\nconst u32 rest = " << per << "u - grp * " << ws[oi].group << "u, members = rest < " << ws[oi].group << "u ? rest : " << ws[oi].group << "u;\nu32* c1 = wsc + " << ws[oi].coff1
+              << "ull + (size_t)(q * " << ws[oi].ngroups << "u + grp) * " << CS << "u;\nif (HE_WS_TICKET(c1) == members - 1u) {\nHE_WS_STORE(c1, 0u);\n"
+              << "tk" << j << " = HE_WS_TICKET(wsc + " << ws[oi].coff << "ull + (size_t)q * " << CS << "u) == " << ws[oi].ngroups - 1 << "u; } }\n";
+        }
+        for (int j = 0; j < n_tickets; j++) s << "ticket_s[" << j << "] = tk" << j << ";\n";
+        s << "}\n__syncthreads();\n";
+    }
+    // Phase 3: the block that drew the last ticket of a reduction folds all partials, always in the same order. The
+    // loads are issued in batches of independent registers: one at a time they would cost a memory round trip each.
+    for (size_t oi = 0; oi < p.outs.size(); oi++) {
+        const Out& o = p.outs[oi];
+        if (!ws[oi].on) continue;
+        const int rop = (int)o.rop;
+        if (!o.fold_n) {
+            s << "if (ticket_s[" << ticket_of[oi] << "]) {\nfloat r[NV];\n#pragma unroll\nfor (int k = 0; k < NV; k++) r[k] = red_identity<"
+              << rop << ">();\nif (col_ok) {\nfor (u32 y0 = ty; y0 < " << gy << "u; y0 += TY * 8) {\nfloat pv[8][NV];\n#pragma unroll\nfor (u32 c = 0; c < 8; c++) {\n"
+              << "const u32 y = y0 + c * TY;\nconst float* part = wsf + " << ws[oi].foff << "ull + (size_t)((b * " << gy << "u + (y < " << gy
+              << "u ? y : 0u)) * " << gx << "u + tile_x) * (TX * NV) + tx * NV;\n#pragma unroll\nfor (int k = 0; k < NV; k++) pv[c][k] = y < " << gy
+              << "u ? HE_WS_LOAD(part + k) : red_identity<" << rop << ">();\n}\n#pragma unroll\nfor (u32 c = 0; c < 8; c++) {\n#pragma unroll\n"
+              << "for (int k = 0; k < NV; k++) r[k] = red_op<" << rop << ">(r[k], pv[c][k]);\n}\n}\n}\n";
+            if (TY > 1)
+                s << "__syncthreads();\n#pragma unroll\nfor (int k = 0; k < NV; k++) col_red[(ty * TX + tx) * NV + k] = r[k];\n__syncthreads();\n"
+                  << "if (ty == 0) {\n#pragma unroll\nfor (int k = 0; k < NV; k++) {\nfor (u32 y = 1; y < TY; y++) r[k] = red_op<" << rop
+                  << ">(r[k], col_red[(y * TX + tx) * NV + k]);\n} }\n";
+            s << "if (ty == 0 && col_ok) {\n#pragma unroll\nfor (int k = 0; k < NV; k++) if (n0 + k < DIM_N) a" << o.arg << "[(size_t)b * " << N
+              << "ull + n0 + k] = r[k];\n}\nif (threadIdx.x == 0) HE_WS_STORE(wsc + " << ws[oi].coff << "ull + (size_t)(b * " << gx << "u + tile_x) * " << CS << "u, 0u);\n}\n";
+        } else {
+            const int64_t per = gx * gy * o.b_div;  // blocks that feed one output element: consecutive block indices
+            s << "if (ticket_s[" << ticket_of[oi] << "]) {\nconst u32 q = b / " << o.b_div << "u;\nfloat acc = red_identity<" << rop
+              << ">();\nfor (u32 i0 = threadIdx.x; i0 < " << per << "u; i0 += " << threads * 8 << "u) {\nfloat pv[8];\n#pragma unroll\nfor (u32 c = 0; c < 8; c++) {\n"
+              << "const u32 i = i0 + c * " << threads << "u;\npv[c] = i < " << per << "u ? HE_WS_LOAD(wsf + " << ws[oi].foff << "ull + (size_t)q * " << per
+              << "ull + i) : red_identity<" << rop << ">();\n}\n#pragma unroll\nfor (u32 c = 0; c < 8; c++) acc = red_op<" << rop << ">(acc, pv[c]);\n}\n"
+              << "acc = wave_reduce<" << rop << ", 64>(acc);\n__syncthreads();\nif ((threadIdx.x & 63) == 0) blk_red[threadIdx.x >> 6] = acc;\n"
+              << "__syncthreads();\nif (threadIdx.x == 0) { acc = blk_red[0];\nfor (int w = 1; w < " << threads / 64 << "; w++) acc = red_op<"
+              << rop << ">(acc, blk_red[w]);\na" << o.arg << "[q] = acc;\nHE_WS_STORE(wsc + " << ws[oi].coff << "ull + (size_t)q * " << CS << "u, 0u); }\n}\n";
+        }
     }
     s << "}\n";
     L.source = s.str();
 
-    for (auto& o : p.outs) {
+    for (size_t oi = 0; oi < p.outs.size(); oi++) {
+        const Out& o = p.outs[oi];
         if (o.reduce) {
+            // what accumulates with atomics starts from the operator's identity
+            if (o.fold_n && !o.fold_m ? gx == 1 && TX <= 64 : !atomics[oi]) continue;
             uint32_t bits = 0;
             float f = o.rop == ROp::Max ? -INFINITY : o.rop == ROp::Min ? INFINITY : 0.0f;
             memcpy(&bits, &f, 4);
@@ -602,7 +744,9 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
     d << "dims=[";
     for (int i = 0; i < n; i++) d << (i ? "x" : "") << p.dims[i];
     d << "] NV=" << NV << " TX=" << TX << " TY=" << TY << " RPT=" << RPT << " grid=" << L.grid << " threads=" << threads
-      << " exprs=" << p.exprs.size() << " outs=" << p.outs.size();
+      << " exprs=" << p.exprs.size() << " outs=" << p.outs.size() << " ws_floats=" << L.ws_floats << " ws_counters=" << L.ws_counters << " fills=[";
+    for (size_t i = 0; i < L.fills.size(); i++) d << (i ? "," : "") << L.fills[i].first << ":" << L.fills[i].second;
+    d << "]";
     L.describe = d.str();
     return L;
 }

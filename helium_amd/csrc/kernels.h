@@ -1,6 +1,8 @@
 // Executable kernels built from tile programs: the pointwise/reduction instruction, anchor-less fusion-IR kernels
 // and the fused GEMM.
 #pragma once
+#include <map>
+#include <mutex>
 #include <memory>
 
 #include "rtc.h"
@@ -22,7 +24,25 @@ public:
     virtual void execute(void* const* ptrs, hipStream_t stream) = 0;
 };
 
-// A tile program compiled into one kernel launch (plus the fills its reduction / bitset outputs need).
+// Device scratch of a kernel whose reductions span several blocks: per-block partials (floats) followed by arrival
+// counters (u32). One buffer per stream the kernel has run on, because launches on one stream run in order and
+// launches on different streams may overlap. The counters are cleared once, by a fill kernel ahead of the first
+// launch on that stream; every launch leaves them at zero again.
+class ReduceScratch {
+public:
+    struct Buf {
+        float* floats;
+        uint32_t* counters;
+    };
+    Buf get(uint64_t n_floats, uint64_t n_counters, hipStream_t stream);
+    void release();
+
+private:
+    std::mutex mu_;
+    std::map<hipStream_t, void*> per_stream_;
+};
+
+// A tile program compiled into one kernel launch (plus the fills its row-reduction / bitset outputs need).
 class TileKernel : public KernelBase {
 public:
     TileKernel(tp::Program prog, const std::string& entry);
@@ -32,11 +52,13 @@ public:
     const std::string& source() const override { return launch_.source; }
     const std::string& describe() const override { return launch_.describe; }
     void execute(void* const* ptrs, hipStream_t stream) override;
+    ~TileKernel() override;
 
 private:
     tp::Program prog_;
     tp::PointwiseLaunch launch_;
     std::unique_ptr<JitKernel> kernel_;
+    ReduceScratch scratch_;
 };
 
 // Fused GEMM: C = f(A) g(B) with mainloop op chains applied while tiles are staged into LDS and the epilogue

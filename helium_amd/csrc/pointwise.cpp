@@ -43,6 +43,27 @@ void fill_buffers(const std::vector<std::pair<void*, std::pair<uint32_t, uint32_
     }
 }
 
+ReduceScratch::Buf ReduceScratch::get(uint64_t n_floats, uint64_t n_counters, hipStream_t stream) {
+    const uint64_t float_bytes = (n_floats * 4 + 255) & ~255ull;
+    std::lock_guard<std::mutex> lk(mu_);
+    auto it = per_stream_.find(stream);
+    if (it == per_stream_.end()) {
+        void* p = nullptr;
+        HE_HIP(hipMalloc(&p, float_bytes + n_counters * 4));
+        it = per_stream_.emplace(stream, p).first;
+        fill_buffers({{(char*)p + float_bytes, {(uint32_t)n_counters, 0u}}}, stream);
+    }
+    return {(float*)it->second, (uint32_t*)((char*)it->second + float_bytes)};
+}
+
+void ReduceScratch::release() {
+    std::lock_guard<std::mutex> lk(mu_);
+    for (auto& kv : per_stream_) (void)hipFree(kv.second);
+    per_stream_.clear();
+}
+
+TileKernel::~TileKernel() { scratch_.release(); }
+
 TileKernel::TileKernel(tp::Program prog, const std::string& entry) : prog_(std::move(prog)) {
     launch_ = tp::emit_pointwise(prog_, entry);
     if (launch_.grid > 0) kernel_.reset(new JitKernel(launch_.source, launch_.entry, launch_.options));
@@ -65,8 +86,13 @@ void TileKernel::execute(void* const* ptrs, hipStream_t stream) {
     for (size_t i = 0; i < nargs; i++)
         HE_REQUIRE(((uintptr_t)ptrs[i] & 15) == 0, HE_ERR_INVALID, "kernel argument %zu is not 16-byte aligned", i);
     std::vector<void*> holders(ptrs, ptrs + nargs);
-    std::vector<void*> argv(nargs);
-    for (size_t i = 0; i < nargs; i++) argv[i] = &holders[i];
+    if (launch_.ws_counters) {
+        ReduceScratch::Buf ws = scratch_.get(launch_.ws_floats, launch_.ws_counters, stream);
+        holders.push_back(ws.floats);
+        holders.push_back(ws.counters);
+    }
+    std::vector<void*> argv(holders.size());
+    for (size_t i = 0; i < holders.size(); i++) argv[i] = &holders[i];
     const uint32_t grid[3] = {launch_.grid, 1, 1}, block[3] = {launch_.threads, 1, 1};
     kernel_->launch(grid, block, 0, stream, argv.data());
 }

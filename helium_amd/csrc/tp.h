@@ -117,6 +117,10 @@ struct PointwiseLaunch {
     int nv = 1, tx = 1, ty = 1, rpt = 1;
     // Outputs that must be filled before the launch: (argument index, 32-bit fill pattern).
     std::vector<std::pair<int, uint32_t>> fills;
+    // Scratch the kernel takes as two trailing arguments (float* then u32*) when nonzero: per-block partial results
+    // and arrival counters of the reductions that span several blocks. Counters must be zero before the first
+    // launch; the block that arrives last combines the partials in block order and zeroes its counter again.
+    uint64_t ws_floats = 0, ws_counters = 0;
     std::vector<std::string> options;
     std::string describe;
 };

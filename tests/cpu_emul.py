@@ -62,6 +62,12 @@ template <class T> static inline T atomicMin(T* a, T v) {
     while (old > v && !__atomic_compare_exchange_n(a, &old, v, false, __ATOMIC_SEQ_CST, __ATOMIC_RELAXED)) {}
     return old;
 }
+static inline unsigned atomicAdd(unsigned* a, unsigned v) { return __atomic_fetch_add(a, v, __ATOMIC_SEQ_CST); }
+// blocks run one after another here, so the scratch exchange needs no atomicity
+#define HE_WS_STORE(p, v) (*(p) = (v))
+#define HE_WS_LOAD(p) (*(p))
+#define HE_WS_TICKET(p) __atomic_fetch_add((p), 1u, __ATOMIC_RELAXED)
+#define HE_WS_DRAIN()
 static inline unsigned atomicOr(unsigned* a, unsigned v) { return __atomic_fetch_or(a, v, __ATOMIC_SEQ_CST); }
 // matrix-core and transposing-LDS-load stand-ins: whole waves call them in lockstep, lanes meet in memory
 typedef short emu_s16x8 __attribute__((ext_vector_type(8)));

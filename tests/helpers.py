@@ -81,24 +81,38 @@ def _storage_elems(a):
     return (a["numel"] + 31) // 32 if a["dtype"] == "bool" else a["numel"]
 
 
-def run_tile_kernel_cpu(kernel, inputs_by_node, entry, fills):
-    """Executes the generated source on the CPU (tests/cpu_emul.py). `fills`: {leaf node: 32-bit pattern} for the
-    outputs the launch pre-fills (reduction identities, zeroed bitsets)."""
+def run_tile_kernel_cpu(kernel, inputs_by_node, entry, fills=None):
+    """Executes the generated source on the CPU (tests/cpu_emul.py). The outputs the kernel's description lists
+    under fills=[argument:pattern,...] start from that 32-bit pattern, as the launch pre-fills them; every other
+    output starts as garbage. `fills`: {leaf node: pattern} the caller expects for the pre-filled ones."""
     from cpu_emul import run_kernel
 
     grid, threads = _launch_numbers(kernel.description)
+    listed = re.search(r"fills=\[([^\]]*)\]", kernel.description)
+    prefill = {int(a): int(v) for a, v in (item.split(":") for item in listed.group(1).split(",") if item)} if listed else {}
     buffers, order = [], []
-    for a in kernel.args:
+    for i, a in enumerate(kernel.args):
         dt = nm.NP_STORAGE[a["dtype"]]
         if a["is_output"]:
-            if a["node"] in fills:  # pre-filled outputs are 32-bit typed (f32 reductions, u32 bitsets)
-                buffers.append((np.full(_storage_elems(a), fills[a["node"]], dtype=np.uint32).view(dt), 2))
+            if i in prefill:  # pre-filled outputs are 32-bit typed (f32 reductions, u32 bitsets)
+                if fills is not None:
+                    assert fills[a["node"]] == prefill[i], (a, prefill)
+                buffers.append((np.full(_storage_elems(a), prefill[i], dtype=np.uint32).view(dt), 2))
             else:
                 buffers.append((np.empty(_storage_elems(a), dtype=dt), 1))
             order.append(a["node"])
         else:
             buffers.append((np.ascontiguousarray(inputs_by_node[a["node"]]), 0))
+    # scratch of the cross-block reductions: partials, then arrival counters, which every launch must leave at zero
+    ws = re.search(r"ws_floats=(\d+) ws_counters=(\d+)", kernel.description)
+    n_ws = (int(ws.group(1)), int(ws.group(2))) if ws else (0, 0)
+    if n_ws[1]:
+        buffers.append((np.full(max(n_ws[0], 1), np.nan, dtype=np.float32), 2))
+        buffers.append((np.zeros(n_ws[1], dtype=np.uint32), 2))
     outs = run_kernel(kernel.source, entry, grid, threads, buffers)
+    if n_ws[1]:
+        assert not outs[-1].any(), "arrival counters not back at zero"
+        outs = outs[:-2]
     return dict(zip(order, outs))
 
 

@@ -83,3 +83,25 @@ def test_transposed_producer_and_broadcast_constant(gpu):
     got = run_tile_kernel_gpu(ha.TileKernel.auxiliary(g), inputs)[out]
     want = oracle.outputs(g.nodes, inputs)[out].reshape(-1)
     assert np.array_equal(got, want)
+
+
+def test_repeated_launches_reuse_the_scratch_and_agree_bit_for_bit(gpu):
+    """A short launch combines its blocks' partial sums through scratch memory in block order: the arrival
+    counters must be back at zero after every launch, and the sums do not depend on which block finished last."""
+    g = ha.fusion.OpGraph()
+    rng = np.random.default_rng(21)
+    shape = [2, 700, 520]
+    x = g.producer(shape, "f32")
+    v = g.unary(x, "tanh")
+    outs = [g.consumer(g.reduction(v, d), "f32") for d in ("columns", "item", "batch")]
+    inputs = {x: rng.standard_normal(shape).astype(np.float32)}
+    kernel = ha.TileKernel.auxiliary(g)
+    assert "fills=[]" in kernel.description, kernel.description
+    want = oracle.outputs(g.nodes, inputs)
+    first = run_tile_kernel_gpu(kernel, inputs)
+    for leaf in outs:
+        assert np.allclose(first[leaf], want[leaf].reshape(-1), rtol=1e-3, atol=1e-4), leaf
+    for _ in range(4):
+        again = run_tile_kernel_gpu(kernel, inputs)
+        for leaf in outs:
+            assert np.array_equal(first[leaf], again[leaf]), leaf
