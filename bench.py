@@ -24,8 +24,7 @@ BF16_PEAK_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
 F32_PEAK_TFLOPS = 157.3      # MI355X dense fp32 matrix, published
 # Bytes that left the XCD L2s per launch of each workload's dominant kernel: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE,
 # each scaled by what the same counter reads for the COPY workload (profiles/<kernel>_<workload>.txt).
-TRAFFIC_BYTES = {"COPY": 268435456, "C2a": 205553498, "C2b": 67190487, "C2c": 17587582, "C3": 271216399,
-                 "C4": 378292763, "C5a": 302129448, "GEMM": 234913542}
+TRAFFIC_BYTES = {"COPY": 268435456, "C2a": 205564225, "C2b": 67187497, "C2c": 17587559, "C3": 271193138, "C4": 378155062, "C5a": 302133899, "GEMM": 234914050}
 HEADLINE = "C4"              # the workload `value` is quoted on
 ROTATE_BYTES = 768 << 20     # rotate operand sets so repeated steps cannot live in the 256 MB Infinity Cache
 

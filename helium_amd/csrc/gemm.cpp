@@ -399,15 +399,22 @@ void fused_matmul(KERNEL_PARAMS) {
 #if DIRECT_LOADS
         // tile kt must have landed; up to NSTAGES - 2 younger tiles may still be in flight
         const u32 younger = KT - 1 - kt < NSTAGES - 2 ? KT - 1 - kt : NSTAGES - 2;
-        if (younger >= 3) __builtin_amdgcn_s_waitcnt(0x0F70 | WAITCNT_VM(3 * (A_DPW + B_DPW)));
-        else if (younger == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | WAITCNT_VM(2 * (A_DPW + B_DPW)));
-        else if (younger == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | WAITCNT_VM(A_DPW + B_DPW));
-        else __builtin_amdgcn_s_waitcnt(0x0F70);
+        // (0x0070: no wait on the export counter, lgkmcnt(0) so that this wave's LDS reads and staged LDS stores are done)
+        if (younger >= 3) __builtin_amdgcn_s_waitcnt(0x0070 | WAITCNT_VM(3 * (A_DPW + B_DPW)));
+        else if (younger == 2) __builtin_amdgcn_s_waitcnt(0x0070 | WAITCNT_VM(2 * (A_DPW + B_DPW)));
+        else if (younger == 1) __builtin_amdgcn_s_waitcnt(0x0070 | WAITCNT_VM(A_DPW + B_DPW));
+        else __builtin_amdgcn_s_waitcnt(0x0070);
 #endif
         TICK(t_wait)
         // every wave's share of tile kt is in LDS (direct loads waited for above, staged stores made before the
         // barrier) and nobody still reads the stage that this iteration refills
+#if DIRECT_LOADS
+        // The bare barrier: __syncthreads() carries a fence for which the compiler drains every outstanding load,
+        // the ones for younger stages included, and a ring deeper than two stages would gain nothing.
+        __builtin_amdgcn_s_barrier();
+#else
         __syncthreads();
+#endif
         TICK(t_barrier)
         const u32 next = kt + NSTAGES - 1;
         const bool more = next < KT;

@@ -128,6 +128,7 @@ static inline emu_s16x4 emu_tr16(const emu_s16x4* p) {
 // global_load_lds_dwordx4: lane L of the wave writes its 16 bytes at lds_base + L * 16
 #define __builtin_amdgcn_global_load_lds(g, l, size, off, aux) memcpy((char*)(l) + (threadIdx.x & 63u) * (size), (const void*)(g), (size))
 #define __builtin_amdgcn_s_waitcnt(x)
+#define __builtin_amdgcn_s_barrier() pthread_barrier_wait(&g_bar)
 #define KERNEL_ATTRS
 #define __builtin_amdgcn_fence(...)
 #define __builtin_amdgcn_sched_barrier(x)
