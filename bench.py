@@ -245,6 +245,81 @@ class LinearLayerWorkload:
         self.tensors, self.last = {}, None
 
 
+class BatchNormWorkload:
+    """The non-convolution part of BASELINE config 5b that dominates its memory traffic: BatchNorm2d::forward in
+    Train mode followed by Relu (helium/src/modules/batch_norm.rs:32-72) on an NHWC bf16 activation of
+    [64,56,56,256], through execute_graph. Algorithmic bytes: x is read for the statistics and again to normalise
+    (the second pass needs the first one's result), y is written once: 3 * 64*56*56*256 * 2 B."""
+
+    bound = "hbm"
+    unit = "GB/s"
+    dtype = "bf16 storage, f32 math"
+    name = "C5b-bn"
+    wall_timed = True
+    shape = (64, 56, 56, 256)
+
+    def __init__(self):
+        self.work = 3 * int(np.prod(self.shape)) * 2
+
+    def describe(self):
+        return "C5b-bn: bf16 [64,56,56,256] BatchNorm2d train forward + relu via execute_graph"
+
+    def setup(self):
+        import helium_amd as ha
+        from helium_amd import configs, frontend
+        from helium_amd.backend import Plan, Tensor
+
+        g = ha.ir.OpGraph()
+        rec = frontend.Recorder(g)
+        c = self.shape[3]
+        x = g.new_input(list(self.shape), "bf16")
+        params = [g.new_input([c], "f32") for _ in range(4)]
+        y, new_mean, new_var = frontend.batch_norm_train(rec, x, *params)
+        self.outs = {"y": g.new_output(y), "mean": g.new_output(new_mean), "var": g.new_output(new_var)}
+        rng = np.random.default_rng(52)
+        self.host = {x: configs.bf16_rne((rng.standard_normal(self.shape, dtype=np.float32) * 1.5 + 0.3)),
+                     params[0]: np.zeros(c, np.float32), params[1]: np.ones(c, np.float32),
+                     params[2]: rng.uniform(0.5, 1.5, c).astype(np.float32),
+                     params[3]: rng.standard_normal(c).astype(np.float32), **rec.scalars}
+        self.x, self.params, self.graph = x, params, g
+        by_id = {n["id"]: n for n in g.nodes}
+        self.tensors = {i: Tensor.from_numpy(a, by_id[i]["dtype"], int(np.prod(by_id[i]["shape"]))) for i, a in self.host.items()}
+        self.last = None
+        log(f"[bench] {self.describe()} :: plan: " + Plan(g).text.replace("\n", " ; "))
+
+    def step(self, stream, i):
+        from helium_amd.backend import execute_graph
+
+        self.last = execute_graph(self.graph, self.tensors)
+
+    def check(self):
+        """Closed form of the graph in float64: per-channel statistics over all of x, y on 4096 sampled pixels."""
+        from oracle import numerics as nm
+
+        c = self.shape[3]
+        x = nm.bf16_bits_to_f32(self.host[self.x]).reshape(-1, c)
+        mean = x.mean(axis=0, dtype=np.float64)
+        var = (x.astype(np.float64) ** 2).mean(axis=0) - mean ** 2
+        got_mean = self.last[self.outs["mean"]].to_numpy().astype(np.float64)
+        got_var = self.last[self.outs["var"]].to_numpy().astype(np.float64)
+        # running statistics start at 0 / 1 and move by a tenth of the batch statistics
+        if not np.allclose(got_mean, 0.1 * mean, rtol=1e-3, atol=1e-4) or not np.allclose(got_var, 0.9 + 0.1 * var, rtol=1e-3, atol=1e-4):
+            raise SystemExit("[bench] PARITY FAILURE in C5b-bn: running statistics differ from the closed form")
+        rows = np.random.default_rng(3).integers(0, x.shape[0], 4096)
+        scale, bias = self.host[self.params[2]].astype(np.float64), self.host[self.params[3]].astype(np.float64)
+        want = np.maximum((x[rows] - mean) / np.sqrt(var + 1e-3) * scale + bias, 0.0)
+        y = nm.bf16_bits_to_f32(self.last[self.outs["y"]].to_numpy()).reshape(-1, c)[rows].astype(np.float64)
+        if not np.allclose(y, want, rtol=2e-2, atol=2e-2):
+            raise SystemExit("[bench] PARITY FAILURE in C5b-bn: y differs from the closed form")
+        return "running statistics within 1e-3, y (4096 sampled pixels) within 2e-2 of the f64 closed form"
+
+    def cpu_baseline(self, budget_s=5.0):
+        return None
+
+    def free(self):
+        self.tensors, self.last = {}, None
+
+
 class FusedGemmWorkload:
     """BASELINE configs 4 / 5a: 4096^3 bf16 GEMM with fused mainloop / epilogue. Work = 2*M*N*K FLOP."""
 
@@ -384,6 +459,7 @@ def make_workloads():
     w["COPY"] = PermuteWorkload("COPY", (8192, 8192), (0, 1), 24)
     w["C1"] = LinearLayerWorkload()
     w["C3"] = AuxChainWorkload()
+    w["C5b-bn"] = BatchNormWorkload()
     for name in ("C4", "C5a", "C4m", "GEMM"):
         w[name] = FusedGemmWorkload(name)
     return w

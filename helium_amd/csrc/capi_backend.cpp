@@ -1,4 +1,5 @@
 // C ABI of the backend layer: tensors, plans, execute_graph.
+#include <future>
 #include "exec.h"
 
 #include "capi_types.h"
@@ -69,6 +70,16 @@ int he_plan_num_steps(he_plan_t plan, int* steps) {
     return he::guard([&] { *steps = (int)plan->plan->steps.size(); });
 }
 const char* he_plan_describe(he_plan_t plan) { return plan ? plan->text.c_str() : ""; }
+int he_plan_precompile(he_plan_t plan) {
+    return he::guard([&] {
+        HE_REQUIRE(plan, HE_ERR_INVALID, "bad argument");
+        std::vector<std::future<void>> jobs;
+        for (auto& step : plan->plan->steps)
+            for (auto& instr : step.instrs)
+                if (!instr->compiled()) jobs.push_back(std::async(std::launch::async, [instr] { instr->precompile(); }));
+        for (auto& j : jobs) j.get();
+    });
+}
 int he_plan_destroy(he_plan_t plan) {
     delete plan;
     return HE_OK;
@@ -104,6 +115,7 @@ int he_backend_set_option(int option, int64_t value) {
     return he::guard([&] {
         switch (option) {
             case HE_OPT_FUSE_MATMUL_EPILOGUE: he::plan::set_fuse_matmul_epilogue(value != 0); break;
+            case HE_OPT_FOLD_SWAP_INTO_REDUCE: he::plan::set_fold_swap_into_reduce(value != 0); break;
             default: he::fail(HE_ERR_INVALID, "unknown backend option");
         }
     });

@@ -1,4 +1,5 @@
 // HIP source emission for tile programs: the shared expression emitter and the pointwise/reduction kernel.
+#include <algorithm>
 #include <cmath>
 #include <cstring>
 #include <sstream>
@@ -168,6 +169,13 @@ __device__ __forceinline__ float tanh_2ulp(float x) {
 }
 // a / b as a * rcp(b): about 1 ulp, one quarter-rate instruction instead of the ten of an IEEE division
 __device__ __forceinline__ float fast_div(float a, float b) { return a * HE_FAST_RCP(b); }
+// powf whose exponent is one value for the whole launch (a broadcast 1-element operand, as `x.pow_scalar(2.0)`
+// reaches the kernel): the tests are the same in every lane, and squares skip the general routine.
+__device__ __forceinline__ float pow_uniform(float x, float y) {
+    if (y == 2.0f) return x * x;
+    if (y == 1.0f) return x;
+    return powf(x, y);
+}
 __device__ __forceinline__ float fast_tanh(float x) {
     float t = __expf(2.0f * x);
     return 1.0f - fast_div(2.0f, t + 1.0f);
@@ -315,6 +323,14 @@ std::string emit_raw_members(const Program& p, int nv, bool row_varying_only) {
     return s.str();
 }
 
+bool is_uniform_pow(const Program& p, int id) {
+    const Expr& e = p.exprs[id];
+    if (e.kind != Expr::Binary || (BOp)e.op != BOp::Pow) return false;
+    const Expr& rhs = p.exprs[e.b];
+    return rhs.kind == Expr::Load && rhs.cls == Cls::F && rhs.access.chain.empty() &&
+           std::all_of(rhs.access.stride.begin(), rhs.access.stride.end(), [](int64_t w) { return w == 0; });
+}
+
 std::string emit_exprs(const Program& p, const EmitCtx& cx) {
     const int n = (int)p.dims.size();
     const int NV = cx.nv;
@@ -401,6 +417,11 @@ std::string emit_exprs(const Program& p, const EmitCtx& cx) {
                     if (y == 1.0f) { each(ref(e.a)); break; }
                     if (y == 2.0f) { each(ref(e.a) + " * " + ref(e.a)); break; }
                 }
+                if (is_uniform_pow(p, (int)i)) {
+                    if (cx.uniform_pow_is_square) each(ref(e.a) + " * " + ref(e.a));
+                    else each("pow_uniform(" + ref(e.a) + ", " + ref(e.b) + ")");
+                    break;
+                }
                 each(binary_expr(e, e.cls, ref(e.a), ref(e.b), p.fast_math));
                 break;
             }
@@ -455,6 +476,12 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
     }
     const int NV = pick_nv(p, 16);
     const int threads = 256;
+    // A Mean is the sum scaled by 1/group. The reference scales every term (float * double literal,
+    // pointwise/jit.rs:413-418); scaling the finished sum once, also in double, differs from that by rounding only
+    // and takes three double-rate instructions per element out of the inner loop.
+    auto scaled = [](const Out& o, const std::string& x) {
+        return o.rop == ROp::Mean ? strfmt("(float)((double)(%s) * %.17g)", x.c_str(), o.mean_scale) : x;
+    };
     bool any_col = false, any_scalar = false;
     for (auto& o : p.outs) {
         if (!o.reduce) continue;
@@ -462,7 +489,7 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
         if (o.fold_m && o.fold_n) any_scalar = true;
     }
     // Threads along a row. With a column reduction a block should be tall rather than wide: its TY row groups are
-    // combined in LDS, so every block issues one atomic per column it spans, not one per column per row group.
+    // combined in LDS, so every block leaves one partial per column it spans, not one per column per row group.
     int tx_cap = any_col ? 64 : threads;
     if (const char* env = getenv("HELIUM_HIP_POINTWISE_TX")) tx_cap = std::max(1, atoi(env));
     int TX = (int)std::min<int64_t>(tx_cap, pow2_ceil((N + NV - 1) / NV));
@@ -474,10 +501,20 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
     if (const char* env = getenv("HELIUM_HIP_POINTWISE_RPT")) {
         RPT = std::max(1, atoi(env));
     } else {
-        // Blocks that end in per-column or scalar atomics are worth making tall: 32 rows per thread and about two
-        // blocks per CU measured 20% faster on a 4096^2 chain than 8 rows and eight blocks per CU.
+        // Blocks that end in a column or scalar reduction pay for it once per block (LDS exchange, partials) and are
+        // worth making tall, up to about 256 KB of operands per block and no fewer than two blocks per CU
+        // (measured: [1,4096,4096] f32 chain with four operands best at 16 rows per thread, a [200704,256] bf16
+        // column reduction at 32).
         const bool tall = any_col || any_scalar;
-        while (RPT < (tall ? 32 : 16) && blocks1 / (RPT * 2) >= (tall ? 512 : 2048)) RPT *= 2;
+        int64_t row_bytes = 0;  // bytes one row of a block moves
+        for (auto& e : p.exprs)
+            if (e.kind == Expr::Load && n >= 2 && e.access.chain.empty() && e.access.stride[n - 2] != 0 && e.access.stride[n - 1] != 0)
+                row_bytes += (int64_t)TX * NV * (int64_t)storage_bytes(e.access.dtype, 1);
+        for (auto& o : p.outs)
+            if (!o.reduce) row_bytes += (int64_t)TX * NV * (int64_t)storage_bytes(o.dtype == HE_BOOL ? HE_U32 : o.dtype, 1);
+        while (RPT < (tall ? 32 : 16) && blocks1 / (RPT * 2) >= (tall ? 512 : 2048) &&
+               (!tall || row_bytes * TY * RPT * 2 <= (256 << 10)))
+            RPT *= 2;
     }
     RPT = (int)std::min<int64_t>(RPT, std::max<int64_t>(1, gy1));
     const int TR = TY * RPT;
@@ -502,63 +539,71 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
     s << "extern \"C\" __global__ __launch_bounds__(" << threads << ") void " << entry << "(";
     for (size_t a = 0; a < p.args.size(); a++)
         s << (a ? ", " : "") << (p.args[a].is_output ? "" : "const ") << c_type(p.args[a].dtype) << "* __restrict__ a" << a;
-    // Reductions whose terms come from several blocks: each block parks its partial result in scratch and takes a
-    // ticket; the last one to arrive folds the partials in block order (same result on every run) and writes the
-    // output, so the output needs no initial value and sees one store instead of one atomic per block.
+    // Reductions whose terms come from several blocks: each block parks its partial result in scratch, and the
+    // partials are folded in block order (the same result on every run) into an output that needs no initial value:
+    //  - short launches: by the block that arrives last, which every block finds out from a ticket (one launch);
+    //  - long launches: by a second, small launch of `<entry>_finalize` (two launches, as many as fill + kernel).
+    // One float atomic per block and column onto a pre-filled output is only left for rows wider than a block:
+    // atomics on one address, or on neighbours within a cache line, are served one after another (about 20 ns
+    // each), which for a [200704 x 256] column sum is 25,000 per line and took 200 us.
     struct WsUse {
-        bool on = false;
+        bool on = false, ticket = false;
         uint64_t foff = 0, coff = 0, coff1 = 0;
         int64_t group = 0, ngroups = 0;  // scalar reductions with many blocks: tickets in two levels
     };
-    // Tickets on one address are served one after another (about 20 ns each), and so are those on neighbours within a
-    // cache line: every counter gets a line of its own, and a reduction over many blocks counts arrivals in groups
-    // of about sqrt(blocks), the last arrival of a group carrying the group's ticket to the second level.
+    // Every ticket counter gets a cache line of its own, and a scalar reduction over many blocks counts arrivals in
+    // groups of about sqrt(blocks), the last arrival of a group carrying the group's ticket to the second level.
     //
     // The last block's way out is a chain of memory round trips (partials land, ticket, partials back, result), a few
-    // microseconds that nothing overlaps when all blocks end together. A short launch still gains, because the fill
-    // kernel and its dependent launch cost more than that; a long one is better off with one atomic per block and
-    // the fill (measured: [1,4096,4096] f32 with two reductions 50 us with atomics, 54 us with tickets).
+    // microseconds that nothing overlaps when all blocks end together. A short launch still gains, because a second
+    // dependent launch costs more than that (measured: [1,4096,4096] f32 with two reductions 54 us with tickets,
+    // 50 us with two launches; a [256,512] f32 column sum inside a graph 29 us -> 26 us with tickets).
     const uint64_t CS = 32;  // counter stride in u32
     bool tickets = B * M * N <= (int64_t)1 << 21;
     if (const char* env = getenv("HELIUM_HIP_REDUCE")) tickets = std::string(env) == "ticket";
     std::vector<WsUse> ws(p.outs.size());
-    std::vector<char> atomics(p.outs.size(), 0);  // reductions over several blocks that accumulate with atomics
+    bool any_finalize = false;
     for (size_t oi = 0; oi < p.outs.size(); oi++) {
         const Out& o = p.outs[oi];
         if (!o.reduce) continue;
-        if (!tickets) {
-            atomics[oi] = o.fold_n ? (o.fold_m ? gx * gy * o.b_div > 1 : false) : gy > 1;
-            continue;
-        }
-        if (o.fold_m && !o.fold_n && gy > 1) {
+        if (o.fold_m && !o.fold_n && gy * o.b_div > 1) {
             ws[oi].on = true;
+            // a column's counter is one address: beyond a few dozen arrivals the tickets would queue up
+            ws[oi].ticket = tickets && gy * o.b_div <= 64;
             ws[oi].foff = L.ws_floats;
-            ws[oi].coff = L.ws_counters;
             L.ws_floats += (uint64_t)grid * TX * NV;
-            L.ws_counters += (uint64_t)B * gx * CS;
+            if (ws[oi].ticket) {
+                ws[oi].coff = L.ws_counters;
+                L.ws_counters += (uint64_t)(B / o.b_div) * gx * CS;
+            }
         } else if (o.fold_m && o.fold_n && gx * gy * o.b_div > 1) {
             const int64_t per = gx * gy * o.b_div, outs_n = B / o.b_div;
             ws[oi].on = true;
+            ws[oi].ticket = tickets;
             ws[oi].foff = L.ws_floats;
-            ws[oi].coff = L.ws_counters;
             L.ws_floats += (uint64_t)grid;
-            L.ws_counters += (uint64_t)outs_n * CS;
-            if (per > 64) {
-                int64_t G = 8;
-                while (G * G < per) G *= 2;
-                ws[oi].group = G;
-                ws[oi].ngroups = (per + G - 1) / G;
-                ws[oi].coff1 = L.ws_counters;
-                L.ws_counters += (uint64_t)outs_n * ws[oi].ngroups * CS;
+            if (ws[oi].ticket) {
+                ws[oi].coff = L.ws_counters;
+                L.ws_counters += (uint64_t)outs_n * CS;
+                if (per > 64) {
+                    int64_t G = 8;
+                    while (G * G < per) G *= 2;
+                    ws[oi].group = G;
+                    ws[oi].ngroups = (per + G - 1) / G;
+                    ws[oi].coff1 = L.ws_counters;
+                    L.ws_counters += (uint64_t)outs_n * ws[oi].ngroups * CS;
+                }
             }
         }
+        if (ws[oi].on && !ws[oi].ticket) any_finalize = true;
     }
-    const bool any_ws = L.ws_counters > 0;
+    const bool any_ws = L.ws_floats > 0;
+    const bool any_ticket = L.ws_counters > 0;
     if (any_ws) s << ", float* wsf, u32* wsc";
     s << ") {\n";
     if (any_col && TY > 1) s << "__shared__ float col_red[TY * TX * NV];\n";
     if (any_scalar) s << "__shared__ float blk_red[" << threads / 64 << "];\n";
-    if (any_ws) s << "__shared__ u32 ticket_s[" << p.outs.size() << "];\n";
+    if (any_ticket) s << "__shared__ u32 ticket_s[" << p.outs.size() << "];\n";
     s << "u32 t = blockIdx.x;\nconst u32 tile_x = t % " << gx << "u; t /= " << gx << "u;\nconst u32 tile_y = t % " << gy
       << "u; t /= " << gy << "u;\nconst u32 b = t;\n";
     {
@@ -579,13 +624,19 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
         else if (o.fold_m && o.fold_n)
             s << "float rs" << oi << " = red_identity<" << (int)o.rop << ">();\n";
     }
-    s << "#pragma unroll\nfor (u32 i = 0; i < RPT; i++) {\nconst u32 m = tile_y * TR + i * TY + ty;\nconst bool ok = col_ok && m < DIM_M;\n";
+    // The rows of a block whose tile lies wholly inside the tensor carry no bounds test: a load under a per-row
+    // predicate cannot be issued ahead of the previous row's work, and a streaming kernel then waits out one memory
+    // round trip per row.
+    std::ostringstream& main_stream = s;
+    auto row_body = [&](bool squares) {
+    std::ostringstream s;
     for (size_t oi = 0; oi < p.outs.size(); oi++)
         if (p.outs[oi].reduce && p.outs[oi].fold_n && !p.outs[oi].fold_m)
             s << "float rr" << oi << " = red_identity<" << (int)p.outs[oi].rop << ">();\n";
     s << "if (ok) {\n";
     EmitCtx cx;
     cx.nv = NV;
+    cx.uniform_pow_is_square = squares;
     s << emit_exprs(p, cx);
     // outputs
     Shape pst = ir::packed_strides(p.dims);
@@ -605,7 +656,6 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
             continue;
         }
         std::string term = v + "[k]";
-        if (o.rop == ROp::Mean) term = strfmt("(float)((double)%s[k] * %.17g)", v.c_str(), o.mean_scale);
         if (o.fold_m && !o.fold_n)
             s << "#pragma unroll\nfor (int k = 0; k < NV; k++) rc" << oi << "[k] = red_op<" << (int)o.rop << ">(rc" << oi
               << "[k], " << term << ");\n";
@@ -624,18 +674,54 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
         const int width = std::min(TX, 64);
         s << "{ float r = wave_reduce<" << (int)o.rop << ", " << width << ">(rr" << oi << ");\n";
         if (gx == 1 && TX <= 64)  // one wave segment holds the whole row
-            s << "if ((threadIdx.x % " << width << ") == 0 && m < DIM_M && col_ok) a" << o.arg << "[(size_t)b * " << M << "ull + m] = r; }\n";
+            s << "if ((threadIdx.x % " << width << ") == 0 && m < DIM_M && col_ok) a" << o.arg << "[(size_t)b * " << M << "ull + m] = " << scaled(o, "r") << "; }\n";
         else
             s << "if ((threadIdx.x % " << width << ") == 0 && m < DIM_M && col_ok) atomic_red<" << (int)o.rop << ">(a" << o.arg
-              << " + (size_t)b * " << M << "ull + m, r); }\n";
+              << " + (size_t)b * " << M << "ull + m, " << scaled(o, "r") << "); }\n";
     }
-    s << "}\n";  // row loop
+    return s.str();
+    };
+    {
+        std::ostringstream& s = main_stream;
+        const int64_t TRv = (int64_t)TY * RPT;
+        const bool ragged = M % TRv != 0 || N % ((int64_t)TX * NV) != 0;
+        // UNROLL rows are in flight at a time: all RPT at once would keep every row's operands in registers
+        int unroll = std::min(RPT, 2);
+        if (const char* env = getenv("HELIUM_HIP_POINTWISE_UNROLL")) unroll = std::max(1, std::min(RPT, atoi(env)));
+        while (RPT % unroll) unroll--;
+        const std::string head = "#pragma unroll 1\nfor (u32 i0 = 0; i0 < RPT; i0 += " + std::to_string(unroll) + ") {\n#pragma unroll\nfor (u32 iu = 0; iu < " +
+                                 std::to_string(unroll) + "; iu++) {\nconst u32 i = i0 + iu;\nconst u32 m = tile_y * TR + i * TY + ty;\n";
+        auto loops = [&](const std::string& body) {
+            if (ragged) s << "if ((tile_y + 1) * TR <= DIM_M && (tile_x + 1) * (TX * NV) <= DIM_N) {\n";
+            s << head << "const bool ok = true;\n" << body << "}\n}\n";
+            if (ragged) s << "} else {\n" << head << "const bool ok = col_ok && m < DIM_M;\n" << body << "}\n}\n}\n";
+        };
+        // `x.pow_scalar(2.0)` reaches the kernel as Pow with a broadcast 1-element operand. The exponents are read
+        // once; when all of them are 2 the loop that squares runs, and the general routine (a few hundred
+        // instructions per call site) stays out of the instruction stream of the common case.
+        std::vector<int> exps;
+        for (size_t i = 0; i < p.exprs.size(); i++)
+            if (is_uniform_pow(p, (int)i)) exps.push_back(p.exprs[p.exprs[i].b].access.arg);
+        std::sort(exps.begin(), exps.end());
+        exps.erase(std::unique(exps.begin(), exps.end()), exps.end());
+        if (exps.empty()) {
+            loops(row_body(false));
+        } else {
+            s << "bool all_squares = true;\n";
+            for (int a : exps) s << "all_squares = all_squares && ld_one(a" << a << ") == 2.0f;\n";
+            s << "if (all_squares) {\n";
+            loops(row_body(true));
+            s << "} else {\n";
+            loops(row_body(false));
+            s << "}\n";
+        }
+    }
     // Phase 1: every block finishes its own partial of each reduction. What no other block contributes to is stored
     // straight to the output; the rest is parked in scratch.
     int n_tickets = 0;
     std::vector<int> ticket_of(p.outs.size(), -1);
     for (size_t oi = 0; oi < p.outs.size(); oi++)
-        if (ws[oi].on) ticket_of[oi] = n_tickets++;
+        if (ws[oi].ticket) ticket_of[oi] = n_tickets++;
     for (size_t oi = 0; oi < p.outs.size(); oi++) {
         const Out& o = p.outs[oi];
         if (!(o.reduce && o.fold_m && !o.fold_n)) continue;
@@ -645,15 +731,15 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
               << "[k];\nfor (u32 y = 1; y < TY; y++) r = red_op<" << (int)o.rop << ">(r, col_red[(y * TX + tx) * NV + k]);\nrc"
               << oi << "[k] = r; } }\n";
         }
-        if (atomics[oi])
-            s << "if (ty == 0 && col_ok) {\n#pragma unroll\nfor (int k = 0; k < NV; k++) if (n0 + k < DIM_N) atomic_red<" << (int)o.rop << ">(a" << o.arg
-              << " + (size_t)b * " << N << "ull + n0 + k, rc" << oi << "[k]); }\n";
-        else if (!ws[oi].on)
+        if (!ws[oi].on)
             s << "if (ty == 0 && col_ok) {\n#pragma unroll\nfor (int k = 0; k < NV; k++) if (n0 + k < DIM_N) a" << o.arg << "[(size_t)b * " << N
-              << "ull + n0 + k] = rc" << oi << "[k]; }\n";
-        else
+              << "ull + n0 + k] = " << scaled(o, "rc" + std::to_string(oi) + "[k]") << "; }\n";
+        else if (ws[oi].ticket)
             s << "if (ty == 0) {\n#pragma unroll\nfor (int k = 0; k < NV; k++) HE_WS_STORE(wsf + " << ws[oi].foff
               << "ull + (size_t)blockIdx.x * (TX * NV) + tx * NV + k, rc" << oi << "[k]); }\n";
+        else
+            s << "if (ty == 0) {\n#pragma unroll\nfor (int k = 0; k < NV; k++) wsf[" << ws[oi].foff
+              << "ull + (size_t)blockIdx.x * (TX * NV) + tx * NV + k] = rc" << oi << "[k]; }\n";
     }
     for (size_t oi = 0; oi < p.outs.size(); oi++) {
         const Out& o = p.outs[oi];
@@ -661,23 +747,23 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
         s << "{ float r = wave_reduce<" << (int)o.rop << ", 64>(rs" << oi << ");\n__syncthreads();\nif ((threadIdx.x & 63) == 0) blk_red[threadIdx.x >> 6] = r;\n__syncthreads();\n";
         s << "if (threadIdx.x == 0) { r = blk_red[0];\nfor (int w = 1; w < " << threads / 64 << "; w++) r = red_op<"
           << (int)o.rop << ">(r, blk_red[w]);\n";
-        if (atomics[oi])
-            s << "atomic_red<" << (int)o.rop << ">(a" << o.arg << " + (size_t)(b / " << o.b_div << "u), r); } }\n";
-        else if (!ws[oi].on)
-            s << "a" << o.arg << "[b / " << o.b_div << "u] = r; } }\n";
-        else
+        if (!ws[oi].on)
+            s << "a" << o.arg << "[b / " << o.b_div << "u] = " << scaled(o, "r") << "; } }\n";
+        else if (ws[oi].ticket)
             s << "HE_WS_STORE(wsf + " << ws[oi].foff << "ull + blockIdx.x, r); } }\n";
+        else
+            s << "wsf[" << ws[oi].foff << "ull + blockIdx.x] = r; } }\n";
     }
     if (n_tickets) {
         // Phase 2: once every wave's partials have landed, one thread takes the block's ticket of each reduction.
         s << "HE_WS_DRAIN();\n__syncthreads();\nif (threadIdx.x == 0) {\n";
         for (size_t oi = 0; oi < p.outs.size(); oi++) {
-            if (!ws[oi].on) continue;
+            if (!ws[oi].ticket) continue;
             const Out& o = p.outs[oi];
             const int j = ticket_of[oi];
             if (!o.fold_n) {
-                s << "const u32 tk" << j << " = HE_WS_TICKET(wsc + " << ws[oi].coff << "ull + (size_t)(b * " << gx << "u + tile_x) * " << CS << "u) == "
-                  << gy - 1 << "u;\n";
+                s << "const u32 tk" << j << " = HE_WS_TICKET(wsc + " << ws[oi].coff << "ull + (size_t)((b / " << o.b_div << "u) * " << gx << "u + tile_x) * " << CS << "u) == "
+                  << gy * o.b_div - 1 << "u;\n";
                 continue;
             }
             const int64_t per = gx * gy * o.b_div;
@@ -698,21 +784,22 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
     // loads are issued in batches of independent registers: one at a time they would cost a memory round trip each.
     for (size_t oi = 0; oi < p.outs.size(); oi++) {
         const Out& o = p.outs[oi];
-        if (!ws[oi].on) continue;
+        if (!ws[oi].ticket) continue;
         const int rop = (int)o.rop;
         if (!o.fold_n) {
-            s << "if (ticket_s[" << ticket_of[oi] << "]) {\nfloat r[NV];\n#pragma unroll\nfor (int k = 0; k < NV; k++) r[k] = red_identity<"
-              << rop << ">();\nif (col_ok) {\nfor (u32 y0 = ty; y0 < " << gy << "u; y0 += TY * 8) {\nfloat pv[8][NV];\n#pragma unroll\nfor (u32 c = 0; c < 8; c++) {\n"
-              << "const u32 y = y0 + c * TY;\nconst float* part = wsf + " << ws[oi].foff << "ull + (size_t)((b * " << gy << "u + (y < " << gy
-              << "u ? y : 0u)) * " << gx << "u + tile_x) * (TX * NV) + tx * NV;\n#pragma unroll\nfor (int k = 0; k < NV; k++) pv[c][k] = y < " << gy
+            const int64_t arrivals = gy * o.b_div;  // blocks (b, tile_y) that feed one (output row, tile_x): consecutive b * gy + tile_y
+            s << "if (ticket_s[" << ticket_of[oi] << "]) {\nconst u32 q = b / " << o.b_div << "u;\nfloat r[NV];\n#pragma unroll\nfor (int k = 0; k < NV; k++) r[k] = red_identity<"
+              << rop << ">();\nif (col_ok) {\nfor (u32 y0 = ty; y0 < " << arrivals << "u; y0 += TY * 8) {\nfloat pv[8][NV];\n#pragma unroll\nfor (u32 c = 0; c < 8; c++) {\n"
+              << "const u32 y = y0 + c * TY;\nconst float* part = wsf + " << ws[oi].foff << "ull + (size_t)((q * " << arrivals << "u + (y < " << arrivals
+              << "u ? y : 0u)) * " << gx << "u + tile_x) * (TX * NV) + tx * NV;\n#pragma unroll\nfor (int k = 0; k < NV; k++) pv[c][k] = y < " << arrivals
               << "u ? HE_WS_LOAD(part + k) : red_identity<" << rop << ">();\n}\n#pragma unroll\nfor (u32 c = 0; c < 8; c++) {\n#pragma unroll\n"
               << "for (int k = 0; k < NV; k++) r[k] = red_op<" << rop << ">(r[k], pv[c][k]);\n}\n}\n}\n";
             if (TY > 1)
                 s << "__syncthreads();\n#pragma unroll\nfor (int k = 0; k < NV; k++) col_red[(ty * TX + tx) * NV + k] = r[k];\n__syncthreads();\n"
                   << "if (ty == 0) {\n#pragma unroll\nfor (int k = 0; k < NV; k++) {\nfor (u32 y = 1; y < TY; y++) r[k] = red_op<" << rop
                   << ">(r[k], col_red[(y * TX + tx) * NV + k]);\n} }\n";
-            s << "if (ty == 0 && col_ok) {\n#pragma unroll\nfor (int k = 0; k < NV; k++) if (n0 + k < DIM_N) a" << o.arg << "[(size_t)b * " << N
-              << "ull + n0 + k] = r[k];\n}\nif (threadIdx.x == 0) HE_WS_STORE(wsc + " << ws[oi].coff << "ull + (size_t)(b * " << gx << "u + tile_x) * " << CS << "u, 0u);\n}\n";
+            s << "if (ty == 0 && col_ok) {\n#pragma unroll\nfor (int k = 0; k < NV; k++) if (n0 + k < DIM_N) a" << o.arg << "[(size_t)q * " << N
+              << "ull + n0 + k] = " << scaled(o, "r[k]") << ";\n}\nif (threadIdx.x == 0) HE_WS_STORE(wsc + " << ws[oi].coff << "ull + (size_t)(q * " << gx << "u + tile_x) * " << CS << "u, 0u);\n}\n";
         } else {
             const int64_t per = gx * gy * o.b_div;  // blocks that feed one output element: consecutive block indices
             s << "if (ticket_s[" << ticket_of[oi] << "]) {\nconst u32 q = b / " << o.b_div << "u;\nfloat acc = red_identity<" << rop
@@ -721,17 +808,66 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
               << "ull + i) : red_identity<" << rop << ">();\n}\n#pragma unroll\nfor (u32 c = 0; c < 8; c++) acc = red_op<" << rop << ">(acc, pv[c]);\n}\n"
               << "acc = wave_reduce<" << rop << ", 64>(acc);\n__syncthreads();\nif ((threadIdx.x & 63) == 0) blk_red[threadIdx.x >> 6] = acc;\n"
               << "__syncthreads();\nif (threadIdx.x == 0) { acc = blk_red[0];\nfor (int w = 1; w < " << threads / 64 << "; w++) acc = red_op<"
-              << rop << ">(acc, blk_red[w]);\na" << o.arg << "[q] = acc;\nHE_WS_STORE(wsc + " << ws[oi].coff << "ull + (size_t)q * " << CS << "u, 0u); }\n}\n";
+              << rop << ">(acc, blk_red[w]);\na" << o.arg << "[q] = " << scaled(o, "acc") << ";\nHE_WS_STORE(wsc + " << ws[oi].coff << "ull + (size_t)q * " << CS << "u, 0u); }\n}\n";
         }
     }
     s << "}\n";
+    if (any_finalize) {
+        // The second launch: one block per 16 output columns (or per scalar output) folds that slice of the
+        // partials, 16 thread groups sharing the blocks of the first launch between them, always in the same order.
+        const int FW = 16, FG = threads / FW;
+        struct Job {
+            size_t oi;
+            uint32_t first, blocks;
+        };
+        std::vector<Job> jobs;
+        uint32_t total = 0;
+        for (size_t oi = 0; oi < p.outs.size(); oi++) {
+            if (!ws[oi].on || ws[oi].ticket) continue;
+            const Out& o = p.outs[oi];
+            const uint32_t nb = o.fold_n ? (uint32_t)(B / o.b_div) : (uint32_t)((B / o.b_div) * ((N + FW - 1) / FW));
+            jobs.push_back({oi, total, nb});
+            total += nb;
+        }
+        L.finalize_entry = entry + "_finalize";
+        L.finalize_grid = total;
+        s << "extern \"C\" __global__ __launch_bounds__(" << threads << ") void " << L.finalize_entry << "(";
+        for (size_t a = 0; a < p.args.size(); a++)
+            s << (a ? ", " : "") << (p.args[a].is_output ? "" : "const ") << c_type(p.args[a].dtype) << "* __restrict__ a" << a;
+        s << ", const float* __restrict__ wsf) {\n__shared__ float fin_red[" << threads << "];\n";
+        for (auto& jb : jobs) {
+            const Out& o = p.outs[jb.oi];
+            const int rop = (int)o.rop;
+            s << "if (blockIdx.x >= " << jb.first << "u && blockIdx.x < " << jb.first + jb.blocks << "u) {\nconst u32 job = blockIdx.x - " << jb.first
+              << "u;\nfloat acc = red_identity<" << rop << ">();\n";
+            if (!o.fold_n) {
+                const int64_t arrivals = gy * o.b_div, slices = (N + FW - 1) / FW;
+                s << "const u32 q = job / " << slices << "u, n = (job % " << slices << "u) * " << FW << "u + threadIdx.x % " << FW
+                  << "u, grp = threadIdx.x / " << FW << "u;\nconst u32 tile_x = n / (TX * NV), within = n % (TX * NV);\nif (n < DIM_N) {\n"
+                  << "for (u32 j0 = grp; j0 < " << arrivals << "u; j0 += " << FG * 8 << "u) {\nfloat pv[8];\n#pragma unroll\nfor (u32 c = 0; c < 8; c++) {\n"
+                  << "const u32 j = j0 + c * " << FG << "u;\npv[c] = j < " << arrivals << "u ? wsf[" << ws[jb.oi].foff << "ull + (size_t)((q * " << arrivals
+                  << "u + j) * " << gx << "u + tile_x) * (TX * NV) + within] : red_identity<" << rop << ">();\n}\n#pragma unroll\nfor (u32 c = 0; c < 8; c++) acc = red_op<"
+                  << rop << ">(acc, pv[c]);\n}\n}\nfin_red[threadIdx.x] = acc;\n__syncthreads();\nif (grp == 0 && n < DIM_N) {\nfor (u32 g = 1; g < " << FG
+                  << "u; g++) acc = red_op<" << rop << ">(acc, fin_red[g * " << FW << "u + threadIdx.x]);\na" << o.arg << "[(size_t)q * " << N << "ull + n] = " << scaled(o, "acc") << ";\n}\n";
+            } else {
+                const int64_t per = gx * gy * o.b_div;
+                s << "for (u32 i0 = threadIdx.x; i0 < " << per << "u; i0 += " << threads * 8 << "u) {\nfloat pv[8];\n#pragma unroll\nfor (u32 c = 0; c < 8; c++) {\n"
+                  << "const u32 i = i0 + c * " << threads << "u;\npv[c] = i < " << per << "u ? wsf[" << ws[jb.oi].foff << "ull + (size_t)job * " << per
+                  << "ull + i] : red_identity<" << rop << ">();\n}\n#pragma unroll\nfor (u32 c = 0; c < 8; c++) acc = red_op<" << rop << ">(acc, pv[c]);\n}\n"
+                  << "fin_red[threadIdx.x] = acc;\n__syncthreads();\nif (threadIdx.x == 0) {\nfor (u32 t = 1; t < " << threads << "u; t++) acc = red_op<" << rop
+                  << ">(acc, fin_red[t]);\na" << o.arg << "[job] = " << scaled(o, "acc") << ";\n}\n";
+            }
+            s << "return;\n}\n";
+        }
+        s << "}\n";
+    }
     L.source = s.str();
 
     for (size_t oi = 0; oi < p.outs.size(); oi++) {
         const Out& o = p.outs[oi];
         if (o.reduce) {
-            // what accumulates with atomics starts from the operator's identity
-            if (o.fold_n && !o.fold_m ? gx == 1 && TX <= 64 : !atomics[oi]) continue;
+            // rows wider than a block accumulate with atomics, from the operator's identity
+            if (!(o.fold_n && !o.fold_m) || (gx == 1 && TX <= 64)) continue;
             uint32_t bits = 0;
             float f = o.rop == ROp::Max ? -INFINITY : o.rop == ROp::Min ? INFINITY : 0.0f;
             memcpy(&bits, &f, 4);
@@ -744,7 +880,7 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
     d << "dims=[";
     for (int i = 0; i < n; i++) d << (i ? "x" : "") << p.dims[i];
     d << "] NV=" << NV << " TX=" << TX << " TY=" << TY << " RPT=" << RPT << " grid=" << L.grid << " threads=" << threads
-      << " exprs=" << p.exprs.size() << " outs=" << p.outs.size() << " ws_floats=" << L.ws_floats << " ws_counters=" << L.ws_counters << " fills=[";
+      << " exprs=" << p.exprs.size() << " outs=" << p.outs.size() << " ws_floats=" << L.ws_floats << " ws_counters=" << L.ws_counters << " finalize_grid=" << L.finalize_grid << " fills=[";
     for (size_t i = 0; i < L.fills.size(); i++) d << (i ? "," : "") << L.fills[i].first << ":" << L.fills[i].second;
     d << "]";
     L.describe = d.str();

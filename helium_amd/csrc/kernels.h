@@ -42,7 +42,8 @@ private:
     std::map<hipStream_t, void*> per_stream_;
 };
 
-// A tile program compiled into one kernel launch (plus the fills its row-reduction / bitset outputs need).
+// A tile program compiled into one kernel launch, plus the fills its bitset outputs (and rows wider than a block)
+// need and, for reductions of long launches, the small second launch that folds the blocks' partial results.
 class TileKernel : public KernelBase {
 public:
     TileKernel(tp::Program prog, const std::string& entry);
@@ -57,7 +58,7 @@ public:
 private:
     tp::Program prog_;
     tp::PointwiseLaunch launch_;
-    std::unique_ptr<JitKernel> kernel_;
+    std::unique_ptr<JitKernel> kernel_, finalize_;
     ReduceScratch scratch_;
 };
 

@@ -1,4 +1,5 @@
 // Lowering of the two front-end IRs to tile programs.
+#include <algorithm>
 #include <cstring>
 #include <map>
 
@@ -127,6 +128,12 @@ uint32_t f32_bits(float f) {
 // ---------------------------------------------------------------------------------------------------------
 // helium-ir pointwise subgraphs
 // ---------------------------------------------------------------------------------------------------------
+// Element count from which a reduction over leading dims is reordered into a column reduction.
+int64_t fold_columns_threshold() {
+    if (const char* env = getenv("HELIUM_HIP_FOLD_COLUMNS_MIN")) return atoll(env);
+    return 1 << 20;
+}
+
 class PointwiseLowering {
 public:
     // With `anchor` set the subgraph is a Matmul plus the ops that follow it: the program is the epilogue, iterates
@@ -176,6 +183,8 @@ public:
                 int64_t group = 1;
                 for (size_t k = rank - depth; k < rank; k++) group *= rdims[k];
                 o.mean_scale = 1.0 / (double)group;
+                out_depth_.resize(p_.outs.size() + 1, 0);
+                out_depth_[p_.outs.size()] = depth;
                 o.dtype = HE_F32;
                 o.expr = eval(n.op.inputs[0], ident);
                 HE_REQUIRE(p_.exprs[o.expr].cls == Cls::F, HE_ERR_UNSUPPORTED, "reductions take float operands");
@@ -190,10 +199,78 @@ public:
             p_.outs.push_back(o);
         }
         if (anchor_ != ir::kNoNode) drop_unused_inputs();
+        else fold_leading_dims_as_columns();
         return std::move(p_);
     }
 
 private:
+    // helium-ir's Reduce folds trailing dims only, so a reduction over leading dims reaches the kernel as
+    // SwapDims + Reduce (BatchNorm2d statistics over N, H, W of an NHWC tensor, helium/src/modules/batch_norm.rs:38-46;
+    // column sums). Iterated in the Reduce's own index space, the innermost coordinate then strides through memory.
+    // When every output is a reduction of one depth and the largest operand is contiguous along the last *kept* dim,
+    // the iteration space is reordered to [other kept dims, folded dims by decreasing stride, last kept dim] and
+    // mergeable folded dims are merged: the kernel then walks memory in order and folds rows (and part of the batch
+    // index) per column, which the emitter does with one pass over the operand.
+    void fold_leading_dims_as_columns() {
+        const size_t R = p_.dims.size();
+        if (p_.outs.empty() || R < 2) return;
+        // Small tensors stay as they are: they live in the caches whatever the order, and rows that one wave folds
+        // need no exchange between blocks, which at that size costs more than the strided reads.
+        if (ir::num_elements(p_.dims) < fold_columns_threshold()) return;
+        size_t depth = 0;
+        for (size_t i = 0; i < p_.outs.size(); i++) {
+            if (!p_.outs[i].reduce) return;
+            if (i && out_depth_[i] != out_depth_[0]) return;
+        }
+        depth = out_depth_[0];
+        if (depth >= R) return;
+        const size_t K = R - depth, kl = K - 1;
+        const Expr* big = nullptr;
+        for (auto& e : p_.exprs) {
+            if (e.kind != Expr::Load) continue;
+            if (!e.access.chain.empty() || e.access.stride.size() != R) return;
+            if (!big || p_.args[e.access.arg].numel > p_.args[big->access.arg].numel) big = &e;
+        }
+        if (!big || big->access.stride[kl] != 1 || p_.dims[kl] < 16 || big->access.stride[R - 1] == 1) return;
+        std::vector<size_t> perm;
+        for (size_t d = 0; d + 1 < K; d++) perm.push_back(d);
+        std::vector<size_t> folded;
+        for (size_t d = K; d < R; d++) folded.push_back(d);
+        const std::vector<int64_t> key = big->access.stride;
+        std::stable_sort(folded.begin(), folded.end(), [&](size_t a, size_t b) { return key[a] > key[b]; });
+        perm.insert(perm.end(), folded.begin(), folded.end());
+        perm.push_back(kl);
+        auto permute = [&](std::vector<int64_t>& v) {
+            std::vector<int64_t> r(R);
+            for (size_t i = 0; i < R; i++) r[i] = v[perm[i]];
+            v = r;
+        };
+        permute(p_.dims);
+        for (auto& e : p_.exprs)
+            if (e.kind == Expr::Load) permute(e.access.stride);
+        // merge neighbours among the folded dims (positions K-1 .. size-2) that every operand walks as one dim
+        for (size_t i = K - 1; i + 2 < p_.dims.size();) {
+            bool ok = true;
+            for (auto& e : p_.exprs)
+                if (e.kind == Expr::Load && e.access.stride[i] != e.access.stride[i + 1] * p_.dims[i + 1]) ok = false;
+            if (!ok) {
+                i++;
+                continue;
+            }
+            p_.dims[i + 1] *= p_.dims[i];
+            p_.dims.erase(p_.dims.begin() + i);
+            for (auto& e : p_.exprs)
+                if (e.kind == Expr::Load) e.access.stride.erase(e.access.stride.begin() + i);
+        }
+        int64_t b_div = 1;
+        for (size_t i = K - 1; i + 2 < p_.dims.size(); i++) b_div *= p_.dims[i];
+        for (auto& o : p_.outs) {
+            o.fold_n = false;
+            o.fold_m = true;
+            o.b_div = b_div;
+        }
+    }
+
     // The Matmul's own operands are inputs of the subgraph but not of the epilogue unless an epilogue op reads them.
     void drop_unused_inputs() {
         std::vector<char> used(p_.args.size(), 0);
@@ -343,6 +420,7 @@ private:
     Program p_;
     std::map<ir::NodeId, int> input_arg_;
     std::vector<Memo> memo_;
+    std::vector<size_t> out_depth_;  // per output: the Reduce's depth (0 for full-size outputs)
 };
 
 // ---------------------------------------------------------------------------------------------------------

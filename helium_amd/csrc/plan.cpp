@@ -45,9 +45,36 @@ bool enumerate_swaps(const ir::OpSubgraph& sg, std::vector<std::pair<int, int>>*
 
 namespace {
 std::atomic<bool> g_fuse_matmul_epilogue{true};
+std::atomic<bool> g_fold_swap_into_reduce{true};
+
+// True when every value computed from `node` inside the graph ends in a Reduce, through pointwise ops only: nothing
+// then needs the transposed tensor in memory.
+bool feeds_only_reductions(const ir::OpGraph& g, NodeId node, int budget = 64) {
+    const auto& users = g.outbound(node);
+    if (users.empty() || budget <= 0) return false;
+    for (NodeId u : users) {
+        const ir::Node& n = g.get(u);
+        if (n.kind != ir::Node::Intermediate) return false;
+        switch (n.op.kind) {
+            case ir::OpKind::Reduce: break;
+            case ir::OpKind::UnaryPointwise:
+            case ir::OpKind::BinaryPointwise:
+            case ir::OpKind::ChangeDataType:
+            case ir::OpKind::Compare:
+            case ir::OpKind::Select:
+                if (!feeds_only_reductions(g, u, budget - 1)) return false;
+                break;
+            default: return false;
+        }
+    }
+    return true;
 }
+}  // namespace
 void set_fuse_matmul_epilogue(bool on) { g_fuse_matmul_epilogue.store(on); }
 bool fuse_matmul_epilogue() { return g_fuse_matmul_epilogue.load(); }
+static unsigned option_mask() { return (fuse_matmul_epilogue() ? 1u : 0u) | (g_fold_swap_into_reduce.load() ? 2u : 0u); }
+void set_fold_swap_into_reduce(bool on) { g_fold_swap_into_reduce.store(on); }
+bool fold_swap_into_reduce() { return g_fold_swap_into_reduce.load(); }
 
 bool Instr::can_fuse_with(const Instr& next) const {
     const bool gemm_and_pointwise = (kind_ == InstrKind::Gemm && next.kind_ == InstrKind::Pointwise) ||
@@ -88,7 +115,10 @@ Instr make_instr_for_op(const std::shared_ptr<const ir::OpGraph>& g, NodeId node
         case ir::OpKind::SwapDims:
             // Heuristic of the reference: the tiled permute kernel for large tensors, the pointwise kernel (which
             // can fuse) for small ones.
-            if (ir::num_elements(n.desc.shape) > kPermuteThreshold) return Instr(InstrKind::Permute, sg);
+            // Beyond the reference: a transposition that only feeds reductions is never written to memory; the
+            // pointwise kernel folds the leading dims of the untransposed tensor in one pass over it.
+            if (ir::num_elements(n.desc.shape) > kPermuteThreshold && !(fold_swap_into_reduce() && feeds_only_reductions(*g, node)))
+                return Instr(InstrKind::Permute, sg);
             return Instr(InstrKind::Pointwise, sg);
         case ir::OpKind::Constant:
         case ir::OpKind::UnaryPointwise:
@@ -397,7 +427,7 @@ std::string Plan::describe() const {
 // ---------------------------------------------------------------------------------------------------------
 namespace {
 struct CacheEntry {
-    bool fused_epilogues;
+    unsigned options;
     uint64_t hash;
     std::shared_ptr<const ir::OpGraph> graph;
     std::shared_ptr<const Plan> plan;
@@ -413,7 +443,7 @@ std::shared_ptr<const Plan> generate_cached_plan(const std::shared_ptr<const ir:
     {
         std::lock_guard<std::mutex> lk(g_plan_mu);
         for (auto it = g_plans.begin(); it != g_plans.end(); ++it)
-            if (it->hash == h && it->fused_epilogues == fuse_matmul_epilogue() && it->graph->structurally_equal(*g)) {
+            if (it->hash == h && it->options == option_mask() && it->graph->structurally_equal(*g)) {
                 g_plans.splice(g_plans.begin(), g_plans, it);
                 g_plan_hits++;
                 return g_plans.front().plan;
@@ -423,7 +453,7 @@ std::shared_ptr<const Plan> generate_cached_plan(const std::shared_ptr<const ir:
     // The cached plan refers to the graph object it was generated from; node ids are equal by construction.
     std::shared_ptr<const Plan> plan = generate_plan(g);
     std::lock_guard<std::mutex> lk(g_plan_mu);
-    g_plans.push_front({fuse_matmul_epilogue(), h, g, plan});
+    g_plans.push_front({option_mask(), h, g, plan});
     if (g_plans.size() > kPlanCacheCapacity) g_plans.pop_back();
     return plan;
 }

@@ -69,6 +69,10 @@ struct Plan {
 // reference's grouping, where a matmul instruction never fuses.
 void set_fuse_matmul_epilogue(bool on);
 bool fuse_matmul_epilogue();
+// Whether a large SwapDims whose values all end in reductions stays in the pointwise instruction instead of becoming
+// a permute instruction of its own (on by default). Off gives the reference's choice by element count alone.
+void set_fold_swap_into_reduce(bool on);
+bool fold_swap_into_reduce();
 
 // generate_plan (plan_generation.rs:22-26).
 std::shared_ptr<const Plan> generate_plan(const std::shared_ptr<const ir::OpGraph>& g);

@@ -49,9 +49,9 @@ ReduceScratch::Buf ReduceScratch::get(uint64_t n_floats, uint64_t n_counters, hi
     auto it = per_stream_.find(stream);
     if (it == per_stream_.end()) {
         void* p = nullptr;
-        HE_HIP(hipMalloc(&p, float_bytes + n_counters * 4));
+        HE_HIP(hipMalloc(&p, float_bytes + std::max<uint64_t>(n_counters, 1) * 4));
         it = per_stream_.emplace(stream, p).first;
-        fill_buffers({{(char*)p + float_bytes, {(uint32_t)n_counters, 0u}}}, stream);
+        if (n_counters) fill_buffers({{(char*)p + float_bytes, {(uint32_t)n_counters, 0u}}}, stream);
     }
     return {(float*)it->second, (uint32_t*)((char*)it->second + float_bytes)};
 }
@@ -67,6 +67,8 @@ TileKernel::~TileKernel() { scratch_.release(); }
 TileKernel::TileKernel(tp::Program prog, const std::string& entry) : prog_(std::move(prog)) {
     launch_ = tp::emit_pointwise(prog_, entry);
     if (launch_.grid > 0) kernel_.reset(new JitKernel(launch_.source, launch_.entry, launch_.options));
+    if (launch_.grid > 0 && launch_.finalize_grid > 0)
+        finalize_.reset(new JitKernel(launch_.source, launch_.finalize_entry, launch_.options));
 }
 
 void TileKernel::execute(void* const* ptrs, hipStream_t stream) {
@@ -86,7 +88,7 @@ void TileKernel::execute(void* const* ptrs, hipStream_t stream) {
     for (size_t i = 0; i < nargs; i++)
         HE_REQUIRE(((uintptr_t)ptrs[i] & 15) == 0, HE_ERR_INVALID, "kernel argument %zu is not 16-byte aligned", i);
     std::vector<void*> holders(ptrs, ptrs + nargs);
-    if (launch_.ws_counters) {
+    if (launch_.ws_floats) {
         ReduceScratch::Buf ws = scratch_.get(launch_.ws_floats, launch_.ws_counters, stream);
         holders.push_back(ws.floats);
         holders.push_back(ws.counters);
@@ -95,6 +97,12 @@ void TileKernel::execute(void* const* ptrs, hipStream_t stream) {
     for (size_t i = 0; i < holders.size(); i++) argv[i] = &holders[i];
     const uint32_t grid[3] = {launch_.grid, 1, 1}, block[3] = {launch_.threads, 1, 1};
     kernel_->launch(grid, block, 0, stream, argv.data());
+    if (finalize_) {
+        // same arguments, then the float scratch
+        argv.resize(nargs + 1);
+        const uint32_t fgrid[3] = {launch_.finalize_grid, 1, 1};
+        finalize_->launch(fgrid, block, 0, stream, argv.data());
+    }
 }
 
 }  // namespace he

@@ -121,6 +121,10 @@ struct PointwiseLaunch {
     // and arrival counters of the reductions that span several blocks. Counters must be zero before the first
     // launch; the block that arrives last combines the partials in block order and zeroes its counter again.
     uint64_t ws_floats = 0, ws_counters = 0;
+    // Long launches fold the partials with a second launch instead: entry `finalize_entry` of the same source, with
+    // `finalize_grid` blocks of `threads` threads, taking the kernel's arguments followed by the float scratch.
+    std::string finalize_entry;
+    uint32_t finalize_grid = 0;
     std::vector<std::string> options;
     std::string describe;
 };
@@ -137,7 +141,11 @@ struct EmitCtx {
     // 2: everything else, reading those members. Splitting lets a kernel issue the loads long before it needs them.
     int phase = 0;
     bool defer_row_varying_only = false;  // phases 1/2: loads whose address ignores the row stay in phase 2
+    // Pow whose exponent is a launch-uniform operand: written as x * x (the caller has tested the exponents)
+    bool uniform_pow_is_square = false;
 };
+// Whether expression `id` is a Pow whose exponent is a float operand read at one address by the whole launch.
+bool is_uniform_pow(const Program& p, int id);
 // Members of the struct phase 1 fills: one native vector per deferred Load of the program.
 std::string emit_raw_members(const Program& p, int nv, bool row_varying_only = false);
 std::string emit_exprs(const Program& p, const EmitCtx& cx);

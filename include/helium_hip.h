@@ -282,6 +282,9 @@ int he_plan_generate(he_graph_t graph, he_plan_t* plan);
 int he_plan_num_steps(he_plan_t plan, int* steps);
 /* One line per step: "step i: kind{node,node,...} ... | release node ...". */
 const char* he_plan_describe(he_plan_t plan);
+/* Compiles the kernels of every instruction of the plan, in parallel, into the kernel caches: what begin_execute does
+ * on first sight of a plan (cuda.rs:98-139, parallel_compile_kernels :262-270). Needs no device. */
+int he_plan_precompile(he_plan_t plan);
 int he_plan_destroy(he_plan_t plan);
 
 /* BackendExt::execute_graph (backend.rs:40-80): prunes a copy of the graph, takes the cached plan, compiles its
@@ -320,8 +323,11 @@ int he_fgraph_subdivide(he_fgraph_t graph, uint64_t* nodes, int32_t* portions, i
 
 /* Backend options. HE_OPT_FUSE_MATMUL_EPILOGUE (default 1): pointwise / reduce ops that follow a Matmul join its
  * instruction and run as the fused GEMM's epilogue (the MatmulGenerator path, matmul.rs:88-130); 0 restores the
- * grouping of helium/src/cuda/instr/cudnn_graph.rs:319-321, where a matmul instruction never fuses. */
-enum { HE_OPT_FUSE_MATMUL_EPILOGUE = 0 };
+ * grouping of helium/src/cuda/instr/cudnn_graph.rs:319-321, where a matmul instruction never fuses.
+ * HE_OPT_FOLD_SWAP_INTO_REDUCE (default 1): a SwapDims above the 1M-element threshold of cuda.rs:38-41 whose values
+ * all end in Reduce ops (BatchNorm2d statistics, column sums) stays in the pointwise instruction, which then folds the
+ * leading dims of the untransposed tensor in one pass; 0 makes it a permute instruction as the reference does. */
+enum { HE_OPT_FUSE_MATMUL_EPILOGUE = 0, HE_OPT_FOLD_SWAP_INTO_REDUCE = 1 };
 int he_backend_set_option(int option, int64_t value);
 
 /* Counters of the last he_execute_graph on this thread: [0] steps run, [1] instructions, [2] streams used,

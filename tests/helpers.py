@@ -8,42 +8,8 @@ from oracle import helium_ir as oracle_ir
 from oracle import numerics as nm
 
 
-# ---- front-end lowerings (helium/src/raw_tensor.rs) ---------------------------------------------------------
-def scalar_tensor(g, value, like_shape):
-    """`x op f32`: a 1-element f32 input broadcast to x's shape (raw_tensor.rs:638-645, broadcast_to :389-414).
-    Returns (broadcast node, scalar input node, scalar storage)."""
-    s = g.new_input([1], "f32")
-    rank = len(like_shape)
-    axes = []
-    if like_shape[-1] != 1:
-        axes.append((rank - 1, like_shape[-1]))
-    for i in range(rank - 1):
-        axes.append((i, like_shape[i]))
-    b = g.broadcast(s, rank, axes)
-    return b, s, np.array([value], dtype=np.float32)
-
-
-def broadcast_to(g, x, x_shape, new_shape):
-    """RawTensor::broadcast_to (raw_tensor.rs:370-424)."""
-    d, d2 = len(x_shape), len(new_shape)
-    axes = []
-    for rev, (old, new) in enumerate(zip(reversed(x_shape), reversed(new_shape))):
-        index = d2 - rev - 1
-        if old != 1:
-            assert old == new
-        if old == 1 and new != 1:
-            axes.append((index, new))
-    for i in range(d2 - d):
-        axes.append((i, new_shape[i]))
-    return g.broadcast(x, d2, axes)
-
-
-def sub(g, a, b):
-    return g.binary(a, g.unary(b, "neg"), "add")  # a - b = a + (-b), raw_tensor.rs:647-653
-
-
-def div(g, a, b):
-    return g.binary(a, g.unary(b, "recip"), "mul")  # a / b = a * recip(b), raw_tensor.rs:679-686
+# ---- front-end lowerings (helium/src/raw_tensor.rs) live in the package; the tests use the same ones
+from helium_amd.frontend import broadcast_to, div, scalar_tensor, sub  # noqa: E402,F401
 
 
 # ---- runners -----------------------------------------------------------------------------------------------
@@ -104,15 +70,20 @@ def run_tile_kernel_cpu(kernel, inputs_by_node, entry, fills=None):
         else:
             buffers.append((np.ascontiguousarray(inputs_by_node[a["node"]]), 0))
     # scratch of the cross-block reductions: partials, then arrival counters, which every launch must leave at zero
-    ws = re.search(r"ws_floats=(\d+) ws_counters=(\d+)", kernel.description)
-    n_ws = (int(ws.group(1)), int(ws.group(2))) if ws else (0, 0)
-    if n_ws[1]:
-        buffers.append((np.full(max(n_ws[0], 1), np.nan, dtype=np.float32), 2))
-        buffers.append((np.zeros(n_ws[1], dtype=np.uint32), 2))
+    ws = re.search(r"ws_floats=(\d+) ws_counters=(\d+) finalize_grid=(\d+)", kernel.description)
+    n_floats, n_counters, finalize_grid = (int(v) for v in ws.groups()) if ws else (0, 0, 0)
+    if n_floats:
+        buffers.append((np.full(n_floats, np.nan, dtype=np.float32), 2))
+        buffers.append((np.zeros(max(n_counters, 1), dtype=np.uint32), 2))
     outs = run_kernel(kernel.source, entry, grid, threads, buffers)
-    if n_ws[1]:
+    if n_floats:
         assert not outs[-1].any(), "arrival counters not back at zero"
-        outs = outs[:-2]
+        partials, outs = outs[-2], outs[:-2]
+        if finalize_grid:
+            # the second launch: same arguments (outputs carried over), then the partials
+            it = iter(outs)
+            again = [(next(it), 2) if a["is_output"] else b for a, b in zip(kernel.args, buffers)]
+            outs = run_kernel(kernel.source, entry + "_finalize", finalize_grid, threads, again + [(partials, 0)])
     return dict(zip(order, outs))
 
 

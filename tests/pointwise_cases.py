@@ -22,6 +22,7 @@ class Case:
         self.expected = {}
         self.reduce_rel = None
         self.admitted_by_fusion_rule = True
+        self.env = {}  # environment overrides the kernel is generated under
 
     def inp(self, shape, dtype, values):
         i = self.g.new_input(list(shape), dtype)
@@ -240,6 +241,34 @@ def generated_cases():
     x = c.inp([70_001], "f32", rng.standard_normal(70_001))
     c.out(c.op(c.g.unary(x, "sigmoid")))
     cases.append(c)
+    # (the reordering starts at 1M elements; the override applies it to shapes the emulation can afford)
+    FOLD_SMALL = {"HELIUM_HIP_FOLD_COLUMNS_MIN": "0"}
+    # Reductions over leading dims arrive as SwapDims + Reduce; the kernel reorders its iteration space so that the
+    # untransposed operand is walked in memory order and rows (and part of the batch index) fold per column.
+    c = Case("batch_norm_statistics_nhwc"); c.env = FOLD_SMALL  # helium/src/modules/batch_norm.rs:38-46
+    x = c.inp([3, 5, 4, 32], "bf16", rng.standard_normal(3 * 5 * 4 * 32))
+    xt = c.op(c.g.swap_dims(x, 0, 3))
+    two = c.inp([1], "f32", [2.0])
+    c.out(c.op(c.g.reduce(xt, "mean", 3)))
+    c.out(c.op(c.g.reduce(c.op(c.g.binary(xt, c.op(c.g.broadcast(two, 4, [(3, 3), (0, 32), (1, 5), (2, 4)])), "pow")), "mean", 3)))
+    c.reduce_rel = 1e-3; cases.append(c)
+
+    c = Case("column_sum_via_swap"); c.env = FOLD_SMALL
+    x = c.inp([300, 48], "f32", rng.standard_normal(300 * 48))
+    c.out(c.op(c.g.reduce(c.op(c.g.swap_dims(x, 0, 1)), "sum", 1))); c.reduce_rel = 1e-3; cases.append(c)
+
+    c = Case("fold_middle_dim_keep_two"); c.env = FOLD_SMALL  # [P,Q,R] -> [P,R,Q], fold Q: outputs [P,R], R contiguous
+    x = c.inp([5, 70, 40], "f32", rng.standard_normal(5 * 70 * 40))
+    c.out(c.op(c.g.reduce(c.op(c.g.swap_dims(x, 1, 2)), "max", 1))); cases.append(c)
+
+    c = Case("fold_two_dims_keep_two"); c.env = FOLD_SMALL  # [A,B,C,D] -> [A,D,C,B], fold C and B: they merge into one row dim
+    x = c.inp([3, 6, 9, 32], "f32", rng.standard_normal(3 * 6 * 9 * 32))
+    c.out(c.op(c.g.reduce(c.op(c.g.swap_dims(x, 1, 3)), "sum", 2))); c.reduce_rel = 1e-3; cases.append(c)
+
+    c = Case("fold_leading_dims_second_operand_blocks_merge"); c.env = FOLD_SMALL  # the batch index keeps a folded dim (b_div > 1)
+    x = c.inp([6, 5, 4, 32], "f32", rng.standard_normal(6 * 5 * 4 * 32)); y = c.inp([32, 5, 4, 6], "f32", rng.standard_normal(6 * 5 * 4 * 32))
+    c.out(c.op(c.g.reduce(c.op(c.g.binary(c.op(c.g.swap_dims(x, 0, 3)), y, "mul")), "sum", 3))); c.reduce_rel = 1e-3; cases.append(c)
+
     return cases
 
 

@@ -37,14 +37,16 @@ def test_all_reduction_depths_across_blocks(shape):
     assert np.all(np.abs(got[full].astype(np.int32) - want[full].reshape(-1).astype(np.int32)) <= 1)
 
 
-@pytest.mark.parametrize("mode", ["ticket", "atomic"])
+@pytest.mark.parametrize("mode", ["ticket", "twopass"])
 def test_both_ways_of_combining_blocks(monkeypatch, mode):
-    """Short launches combine blocks through scratch and tickets, long ones with atomics onto a pre-filled output;
-    the override picks either for a shape the emulation can afford."""
+    """Short launches fold the blocks' partials in the block that arrives last (tickets), long ones in a second
+    small launch; the override picks either for a shape the emulation can afford. Neither needs a pre-filled
+    output."""
     monkeypatch.setenv("HELIUM_HIP_REDUCE", mode)
-    g, inputs, outs = all_reductions_graph([2, 300, 200], 9)
+    g, inputs, outs = all_reductions_graph([2, 200, 200], 9)
     kernel = ha.TileKernel.auxiliary(g)
-    assert ("fills=[]" in kernel.description) == (mode == "ticket"), kernel.description
+    assert "fills=[]" in kernel.description
+    assert ("finalize_grid=0" in kernel.description) == (mode == "ticket"), kernel.description
     got = run_tile_kernel_cpu(kernel, inputs, "fused_auxiliary")
     want = oracle.outputs(g.nodes, inputs)
     for leaf in outs[:4]:

@@ -180,3 +180,43 @@ def test_four_threads_execute_concurrently(gpu):
     assert not errors, errors[0]
     s = stats()
     assert s["plan_cache_hits"] > 0 and s["pool_reuses"] > 0
+
+
+@pytest.mark.parametrize("fold", [1, 0], ids=["statistics_without_permute", "reference_grouping"])
+def test_batch_norm_train_step(gpu, fold):
+    """BatchNorm2d::forward in Train mode + Relu (helium/src/modules/batch_norm.rs:32-72) above the 1M-element
+    SwapDims threshold, planned both ways: with the transposition folded into the statistics kernel and as the
+    reference plans it (permute, then two reductions)."""
+    from helium_amd import frontend
+    from helium_amd.backend import OPT_FOLD_SWAP_INTO_REDUCE, set_option
+
+    shape = [8, 36, 36, 128]  # 1.3M elements
+    g = ha.ir.OpGraph()
+    rec = frontend.Recorder(g)
+    x = g.new_input(shape, "bf16")
+    params = [g.new_input([shape[3]], "f32") for _ in range(4)]
+    y, new_mean, new_var = frontend.batch_norm_train(rec, x, *params)
+    for v in (y, new_mean, new_var):
+        g.new_output(v)
+    rng = np.random.default_rng(77)
+    host = {x: nm.to_storage((rng.standard_normal(shape) * 1.5 + 0.3).astype(np.float32), "bf16"),
+            params[0]: rng.standard_normal(shape[3]).astype(np.float32),
+            params[1]: rng.uniform(0.5, 2.0, shape[3]).astype(np.float32),
+            params[2]: rng.uniform(0.5, 1.5, shape[3]).astype(np.float32),
+            params[3]: rng.standard_normal(shape[3]).astype(np.float32), **rec.scalars}
+    set_option(OPT_FOLD_SWAP_INTO_REDUCE, fold)
+    try:
+        got, steps = run_graph(g, host)
+    finally:
+        set_option(OPT_FOLD_SWAP_INTO_REDUCE, 1)
+    kinds = [k for instrs, _ in steps for k, _ in instrs]
+    assert ("permute" in kinds) == (fold == 0), steps
+    want = oracle_ir.plan_outputs(g.nodes, host, steps)
+    _, desc = oracle_ir.evaluate(g.nodes, host)
+    for o in want:
+        a = nm.from_storage(got[o], desc[o][1], [got[o].size]).astype(np.float64)
+        b = nm.from_storage(want[o].reshape(-1), desc[o][1], [want[o].size]).astype(np.float64)
+        # statistics: f32 sums of 10k bf16 terms in a different order; y: bf16 output of a chain that divides by
+        # sqrt(variance), so one bf16 step of y (2^-8 relative) plus the statistics' error
+        tol = 2e-2 if desc[o][1] == "bf16" else 1e-3
+        assert np.allclose(a, b, rtol=tol, atol=tol), (o, np.abs(a - b).max())

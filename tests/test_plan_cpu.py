@@ -8,16 +8,19 @@ import numpy as np
 import pytest
 
 import helium_amd as ha
-from helium_amd.backend import OPT_FUSE_MATMUL_EPILOGUE, Plan, set_option, stats
+from helium_amd.backend import OPT_FOLD_SWAP_INTO_REDUCE, OPT_FUSE_MATMUL_EPILOGUE, Plan, set_option, stats
 from oracle import plan as oracle_plan
 
 
 @pytest.fixture
 def reference_grouping():
-    """The reference's rule: a matmul instruction never fuses (cudnn_graph.rs:319-321)."""
+    """The reference's rules: a matmul instruction never fuses (cudnn_graph.rs:319-321) and a SwapDims of more
+    than 1M elements is always a permute instruction (cuda.rs:38-41)."""
     set_option(OPT_FUSE_MATMUL_EPILOGUE, 0)
+    set_option(OPT_FOLD_SWAP_INTO_REDUCE, 0)
     yield
     set_option(OPT_FUSE_MATMUL_EPILOGUE, 1)
+    set_option(OPT_FOLD_SWAP_INTO_REDUCE, 1)
 
 
 def linear_layer():
@@ -192,3 +195,38 @@ def test_plan_cache_returns_the_same_plan_for_an_equal_graph():
     after = stats()
     assert pa.text == pb.text
     assert after["plan_cache_hits"] + after["plan_cache_misses"] >= before["plan_cache_hits"] + before["plan_cache_misses"]
+
+
+def batch_norm_graph(shape):
+    from helium_amd import frontend
+
+    g = ha.ir.OpGraph()
+    rec = frontend.Recorder(g)
+    c = shape[3]
+    x = g.new_input(list(shape), "bf16")
+    stats_in = [g.new_input([c], "f32") for _ in range(4)]
+    y, new_mean, new_var = frontend.batch_norm_train(rec, x, *stats_in)
+    for v in (y, new_mean, new_var):
+        g.new_output(v)
+    return g
+
+
+def test_batch_norm_statistics_skip_the_permute():
+    """BatchNorm2d::forward (batch_norm.rs:32-72) at [64,56,56,256]: the reference's plan transposes 51M elements
+    and reads the transposed tensor twice; with the transposition folded into the reductions, one kernel reads x
+    once for both statistics."""
+    g = batch_norm_graph([64, 56, 56, 256])
+    kinds = [[k for k, _ in instrs] for instrs, _ in Plan(g).steps]
+    assert kinds[0] == ["pointwise"] and "permute" not in sum(kinds, [])
+    swap = next(n["id"] for n in g.nodes if n.get("op") == "swap_dims")
+    reduces = [n["id"] for n in g.nodes if n.get("op") == "reduce"]
+    first = Plan(g).steps[0][0][0][1]
+    assert swap in first and all(r in first for r in reduces)
+
+
+def test_batch_norm_reference_plan_has_the_permute(reference_grouping):
+    g = batch_norm_graph([64, 56, 56, 256])
+    steps = Plan(g).steps
+    assert [k for k, _ in steps[0][0]] == ["permute"]
+    assert sorted(k for k, _ in steps[1][0]) == ["pointwise", "pointwise"]  # the two statistics read xt separately
+    assert oracle_plan.generate_plan(g.nodes) == steps

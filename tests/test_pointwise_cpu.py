@@ -25,7 +25,9 @@ def test_oracle_matches_reference_known_answers(case):
 
 
 @pytest.mark.parametrize("case", CASES, ids=lambda c: c.name)
-def test_generated_kernel_on_cpu_matches_oracle(case):
+def test_generated_kernel_on_cpu_matches_oracle(case, monkeypatch):
+    for name, value in case.env.items():
+        monkeypatch.setenv(name, value)
     # what the reference's fusion rule admits (pointwise.rs:121-186); the generator itself accepts more
     admitted = ha.kernels.pointwise_supports(case.g, case.nodes)
     has_constant = any(n.get("op") == "constant" for n in case.g.nodes if n["id"] in case.nodes)
@@ -44,3 +46,15 @@ def test_generated_kernel_on_cpu_matches_oracle(case):
         if leaf in case.expected:
             g32 = nm.from_storage(got[leaf], by_id[leaf]["dtype"], case.expected[leaf].shape)
             assert nm.ulps_close(g32, case.expected[leaf], max_ulps=4, epsilon=1e-6).all()
+
+
+@pytest.mark.parametrize("case", [c for c in CASES if c.env], ids=lambda c: c.name)
+def test_reordered_cases_also_run_in_the_reduce_own_index_space(case):
+    """Below 1M elements a SwapDims + Reduce kernel iterates in the Reduce's index space (strided reads, rows folded
+    by one wave): the same cases without the override."""
+    kernel = ha.TileKernel.pointwise(case.g, case.nodes)
+    want = oracle_ir.kernel_outputs(case.g.nodes, case.inputs, case.leaves)
+    got = run_tile_kernel_cpu(kernel, case.inputs, "pointwise_kernel", reduction_fills(case.g.nodes, case.leaves))
+    for leaf in case.leaves:
+        assert_storage_close(got[leaf], want[leaf].reshape(-1), "f32", f"{case.name} leaf {leaf}: {kernel.description}",
+                             reduce_rel=case.reduce_rel)
