@@ -99,7 +99,19 @@ int he_execute_graph(he_graph_t graph, const uint32_t* input_nodes, const he_ten
                        "tensor for input node %u does not match its descriptor", input_nodes[i]);
             inputs[input_nodes[i]] = input_tensors[i]->t;
         }
-        auto outs = he::exec::execute_graph(*graph->g, inputs, &g_last_stats);
+        // the optimised copy of the graph and its plan are made on the first call and kept with the handle
+        std::shared_ptr<const he::exec::Prepared> prepared;
+        {
+            std::lock_guard<std::mutex> lk(graph->mu);
+            const unsigned options = he::plan::option_mask();
+            if (!graph->prepared || graph->prepared_nodes != graph->g->num_nodes() || graph->prepared_options != options) {
+                graph->prepared = he::exec::prepare(*graph->g);
+                graph->prepared_nodes = graph->g->num_nodes();
+                graph->prepared_options = options;
+            }
+            prepared = graph->prepared;
+        }
+        auto outs = he::exec::execute_prepared(*prepared, inputs, &g_last_stats);
         HE_REQUIRE((int)outs.size() <= max_outputs, HE_ERR_INVALID, "graph has %zu outputs, room for %d", outs.size(), max_outputs);
         int k = 0;
         for (auto& kv : outs) {

@@ -65,7 +65,11 @@ int he_graph_new_output(he_graph_t graph, uint32_t from_node, uint32_t* node) {
     });
 }
 int he_graph_optimize(he_graph_t graph) {
-    return he::guard([&] { graph->g->optimize(); });
+    return he::guard([&] {
+        std::lock_guard<std::mutex> lk(graph->mu);
+        graph->prepared.reset();
+        graph->g->optimize();
+    });
 }
 int he_graph_num_nodes(he_graph_t graph, uint32_t* count) {
     return he::guard([&] { *count = (uint32_t)graph->g->num_nodes(); });

@@ -1,3 +1,4 @@
+#include <chrono>
 #include "exec.h"
 
 #include <algorithm>
@@ -34,23 +35,36 @@ void DevicePool::end_scope_after(uint64_t scope, hipEvent_t done) {
 
 void DevicePool::poll() {
     std::lock_guard<std::mutex> lk(mu_);
-    for (size_t i = 0; i < pending_.size();) {
-        if (hipEventQuery(pending_[i].second) == hipSuccess) {
-            end_scope_locked(pending_[i].first);
-            (void)hipEventDestroy(pending_[i].second);
-            pending_[i] = pending_.back();
-            pending_.pop_back();
-        } else {
-            i++;
-        }
+    // Oldest first, and no further than the first execution that is still running: a host that runs many
+    // executions ahead of the device would otherwise query every one of them on every allocation. Executions of
+    // one thread finish in order; another thread's younger ones wait for the next poll at worst.
+    while (!pending_.empty() && hipEventQuery(pending_.front().second) == hipSuccess) {
+        end_scope_locked(pending_.front().first);
+        spare_events_.push_back(pending_.front().second);
+        pending_.pop_front();
     }
 }
 
-uint64_t DevicePool::begin_scope() {
+hipEvent_t DevicePool::take_event() {
+    {
+        std::lock_guard<std::mutex> lk(mu_);
+        if (!spare_events_.empty()) {
+            hipEvent_t e = spare_events_.back();
+            spare_events_.pop_back();
+            return e;
+        }
+    }
+    hipEvent_t e;
+    HE_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+    return e;
+}
+
+uint64_t DevicePool::begin_scope(uint64_t thread) {
     poll();
     std::lock_guard<std::mutex> lk(mu_);
     uint64_t s = next_scope_++;
     free_scoped_[s];
+    scope_thread_[s] = thread;
     return s;
 }
 
@@ -64,6 +78,7 @@ void DevicePool::end_scope_locked(uint64_t scope) {
     if (it == free_scoped_.end()) return;
     for (auto& kv : it->second) free_global_.insert(kv);
     free_scoped_.erase(it);
+    scope_thread_.erase(scope);
     for (size_t i = 0; i < deferred_.size();) {
         auto& w = deferred_[i].waiting;
         w.erase(std::remove(w.begin(), w.end(), scope), w.end());
@@ -82,6 +97,14 @@ void DevicePool::note_use(Tensor& t, uint64_t scope) {
     if (std::find(t.used.begin(), t.used.end(), scope) == t.used.end()) t.used.push_back(scope);
 }
 
+void DevicePool::note_uses(const std::map<ir::NodeId, TensorRef>& tensors, uint64_t scope) {
+    std::lock_guard<std::mutex> lk(mu_);
+    for (auto& kv : tensors) {
+        Tensor& t = *kv.second;
+        if (std::find(t.used.begin(), t.used.end(), scope) == t.used.end()) t.used.push_back(scope);
+    }
+}
+
 void* DevicePool::allocate(size_t bytes, uint64_t scope) {
     const size_t cls = size_class(bytes);
     {
@@ -97,6 +120,12 @@ void* DevicePool::allocate(size_t bytes, uint64_t scope) {
         auto sc = free_scoped_.find(scope);
         if (sc != free_scoped_.end())
             if (void* p = take(sc->second)) return p;
+        // blocks freed by this thread's earlier executions that are still queued: this one runs after them
+        auto mine = scope_thread_.find(scope);
+        if (mine != scope_thread_.end() && mine->second != 0)
+            for (auto& other : scope_thread_)
+                if (other.second == mine->second && other.first != scope)
+                    if (void* p = take(free_scoped_[other.first])) return p;
         if (void* p = take(free_global_)) return p;
     }
     poll();  // blocks of executions that have finished since become available
@@ -171,6 +200,8 @@ struct Staging {
 };
 struct Streams {
     std::vector<hipStream_t> s;
+    hipEvent_t exec_end = nullptr;  // end of this thread's latest execution (recorded on s[0] after it joined the others)
+    bool has_run = false;
     hipStream_t h2d = nullptr, d2h = nullptr;
     std::vector<Staging> staging;  // pinned upload buffers, reused once their copy has finished
 };
@@ -238,36 +269,69 @@ void download_tensor(const TensorRef& t, void* dst) {
 // ---------------------------------------------------------------------------------------------------------
 // execute_graph
 // ---------------------------------------------------------------------------------------------------------
-std::map<NodeId, TensorRef> execute_graph(const ir::OpGraph& graph_in, const std::map<NodeId, TensorRef>& inputs,
-                                          ExecStats* stats) {
+namespace {
+// HELIUM_HIP_EXEC_TIMING=1: host time per section of execute_graph, averaged and printed every 100 calls.
+struct HostTimer {
+    static bool on() {
+        static const bool v = getenv("HELIUM_HIP_EXEC_TIMING") != nullptr;
+        return v;
+    }
+    std::chrono::steady_clock::time_point t = std::chrono::steady_clock::now();
+    double acc[8] = {0};
+    void lap(int i) {
+        if (!on()) return;
+        auto n = std::chrono::steady_clock::now();
+        acc[i] += std::chrono::duration<double, std::micro>(n - t).count();
+        t = n;
+    }
+    void restart() {
+        if (on()) t = std::chrono::steady_clock::now();
+    }
+};
+thread_local double g_host_acc[8] = {0};
+thread_local int g_host_calls = 0;
+}  // namespace
+
+std::shared_ptr<const Prepared> prepare(const ir::OpGraph& graph_in) {
+    auto pr = std::make_shared<Prepared>();
     auto graph = std::make_shared<ir::OpGraph>(graph_in);
     graph->optimize();
-    std::shared_ptr<const plan::Plan> plan = plan::generate_cached_plan(graph);
-
+    pr->graph = graph;
+    pr->plan = plan::generate_cached_plan(graph);
     // begin_execute (cuda.rs:98-139): compile every kernel of the plan up front, in parallel (cuda.rs:262-270)
-    {
-        std::vector<std::future<void>> jobs;
-        for (auto& step : plan->steps)
-            for (auto& instr : step.instrs)
-                if (!instr->compiled()) jobs.push_back(std::async(std::launch::async, [instr] { instr->precompile(); }));
-        for (auto& j : jobs) j.get();
+    std::vector<std::future<void>> jobs;
+    for (auto& step : pr->plan->steps)
+        for (auto& instr : step.instrs)
+            if (!instr->compiled()) jobs.push_back(std::async(std::launch::async, [instr] { instr->precompile(); }));
+    for (auto& j : jobs) j.get();
+    // tensors that survive the plan get their ready event recorded (enumerate_output_tensors, cuda.rs:142-153)
+    for (auto& step : pr->plan->steps) {
+        for (auto& instr : step.instrs)
+            for (NodeId o : instr->outputs()) pr->alive.insert(o);
+        for (NodeId r : step.tensors_to_release) pr->alive.erase(r);
     }
+    return pr;
+}
+
+std::map<NodeId, TensorRef> execute_graph(const ir::OpGraph& graph_in, const std::map<NodeId, TensorRef>& inputs,
+                                          ExecStats* stats) {
+    return execute_prepared(*prepare(graph_in), inputs, stats);
+}
+
+std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std::map<NodeId, TensorRef>& inputs,
+                                             ExecStats* stats) {
+    HostTimer ht;
+    const std::shared_ptr<const ir::OpGraph>& graph = prepared.graph;
+    const std::shared_ptr<const plan::Plan>& plan = prepared.plan;
+    const std::set<NodeId>& alive = prepared.alive;
     DevicePool& pool = DevicePool::global();
-    const uint64_t scope = pool.begin_scope();
     Streams& st = thread_streams();
+    const uint64_t scope = pool.begin_scope((uint64_t)(uintptr_t)&st);
     std::map<NodeId, TensorRef> tensors = inputs;
     for (NodeId in : graph->inputs())
         HE_REQUIRE(tensors.count(in), HE_ERR_INVALID, "missing storage for input node %u", in);
-    for (auto& kv : tensors) pool.note_use(*kv.second, scope);
-
-    // tensors that survive the plan get their ready event recorded (enumerate_output_tensors, cuda.rs:142-153)
-    std::set<NodeId> alive;
-    for (auto& step : plan->steps) {
-        for (auto& instr : step.instrs)
-            for (NodeId o : instr->outputs()) alive.insert(o);
-        for (NodeId r : step.tensors_to_release) alive.erase(r);
-    }
-
+    pool.note_uses(tensors, scope);
+    ht.lap(2);
     ExecStats local;
     std::set<const Tensor*> synced;        // input tensors whose ready event a stream already waited on
     std::vector<size_t> prev_streams;      // streams the previous step ran on
@@ -304,7 +368,10 @@ std::map<NodeId, TensorRef> execute_graph(const ir::OpGraph& graph_in, const std
         for (size_t i = 0; i < step.instrs.size(); i++) {
             const plan::Instr& instr = *step.instrs[i];
             hipStream_t stream = st.s[i % width];
-            used_streams.insert(i % width);
+            // a stream's first work of this execution comes after the end of the thread's previous execution
+            // (stream 0 carried that end itself)
+            if (used_streams.insert(i % width).second && i % width != 0 && st.has_run)
+                HE_HIP(hipStreamWaitEvent(stream, st.exec_end, 0));
             for (NodeId out : instr.outputs()) {
                 const ir::Descriptor& d = graph->get(out).desc;
                 tensors[out] = allocate_tensor(d.dtype, (size_t)ir::num_elements(d.shape), scope);
@@ -314,12 +381,22 @@ std::map<NodeId, TensorRef> execute_graph(const ir::OpGraph& graph_in, const std
                 HE_REQUIRE(it != tensors.end(), HE_ERR_INTERNAL, "missing storage for node %u", in);
                 // tensors made outside this execution carry a ready event (uploads, earlier graphs)
                 if (inputs.count(in) && !synced.count(it->second.get())) {
-                    HE_HIP(hipStreamWaitEvent(stream, it->second->ready, 0));
-                    local.event_waits++;
+                    Tensor& t = *it->second;
+                    // a producer seen finished once stays finished: no wait is queued for it again
+                    if (!t.ready_seen.load(std::memory_order_acquire)) {
+                        if (hipEventQuery(t.ready) == hipSuccess) {
+                            t.ready_seen.store(true, std::memory_order_release);
+                        } else {
+                            HE_HIP(hipStreamWaitEvent(stream, t.ready, 0));
+                            local.event_waits++;
+                        }
+                    }
                     waited.push_back(it->second.get());
                 }
             }
+            ht.lap(3);
             instr.execute([&](NodeId n) -> void* { return tensors.at(n)->ptr; }, stream);
+            ht.lap(4);
             local.instrs++;
             for (NodeId out : instr.outputs())
                 if (alive.count(out)) HE_HIP(hipEventRecord(tensors.at(out)->ready, stream));
@@ -328,12 +405,16 @@ std::map<NodeId, TensorRef> execute_graph(const ir::OpGraph& graph_in, const std
         synced.insert(waited.begin(), waited.end());
         prev_streams = cur;
     }
+    ht.lap(3);
     // Drop of the executor (cuda.rs:232-260): when everything queued above has run, the scope's freed blocks
     // become available to everyone. Stream 0 joins the last step and carries the event the pool polls.
     join({0});
-    hipEvent_t done;
-    HE_HIP(hipEventCreateWithFlags(&done, hipEventDisableTiming));
+    hipEvent_t done = pool.take_event();
     HE_HIP(hipEventRecord(done, st.s[0]));
+    // The same event orders this thread's next execution after this one. The pool may hand it to another execution
+    // once it has completed; waiting for that one instead would be a needless wait, never a wrong one.
+    st.exec_end = done;
+    st.has_run = true;
     pool.end_scope_after(scope, done);
     {
         // join events of the previous execution on this thread: recorded and waited on long ago
@@ -350,6 +431,15 @@ std::map<NodeId, TensorRef> execute_graph(const ir::OpGraph& graph_in, const std
         auto it = tensors.find(from);
         HE_REQUIRE(it != tensors.end(), HE_ERR_INTERNAL, "output node %u has no storage", out);
         result[out] = it->second;
+    }
+    ht.lap(5);
+    if (HostTimer::on()) {
+        for (int i = 0; i < 8; i++) g_host_acc[i] += ht.acc[i];
+        if (++g_host_calls % 100 == 0) {
+            fprintf(stderr, "[exec timing] per graph, us: copy+optimize %.1f, plan lookup %.1f, setup %.1f, alloc+waits %.1f, launches %.1f, finish %.1f\n",
+                    g_host_acc[0] / 100, g_host_acc[1] / 100, g_host_acc[2] / 100, g_host_acc[3] / 100, g_host_acc[4] / 100, g_host_acc[5] / 100);
+            for (double& v : g_host_acc) v = 0;
+        }
     }
     return result;
 }

@@ -1,6 +1,9 @@
 // Graph executor for the HIP backend: tensor storage, pooled device memory with execution scopes, and the step
 // loop of helium/src/backend.rs:40-80 driven over a pool of HIP streams (helium/src/cuda.rs:98-260).
 #pragma once
+#include <atomic>
+#include <deque>
+#include <set>
 #include <map>
 #include <memory>
 #include <mutex>
@@ -18,7 +21,9 @@ using ir::NodeId;
 class DevicePool {
 public:
     static DevicePool& global();
-    uint64_t begin_scope();
+    // `thread`: a token of the calling host thread. The executions of one thread are ordered on the device (each
+    // waits for the end of the one before), so a later one may take the blocks an earlier one has freed at once.
+    uint64_t begin_scope(uint64_t thread = 0);
     void end_scope(uint64_t scope);  // called once the scope's device work has finished
     // Ends the scope once `done` (recorded after all of its device work) has completed; polled from begin_scope and
     // from allocate, so no host callback sits in any stream. The pool takes the event over.
@@ -30,6 +35,8 @@ public:
     // live scope can, and otherwise waits until the last such scope has ended on the device.
     void release(void* ptr, size_t bytes, uint64_t owner, const std::vector<uint64_t>& used);
     void note_use(struct Tensor& t, uint64_t scope);
+    void note_uses(const std::map<ir::NodeId, std::shared_ptr<struct Tensor>>& tensors, uint64_t scope);
+    hipEvent_t take_event();  // an event nobody waits on any more, or a new one
     void stats(uint64_t* driver_bytes, uint64_t* driver_allocs, uint64_t* reuses);
 
 private:
@@ -37,13 +44,15 @@ private:
     std::mutex mu_;
     std::multimap<size_t, void*> free_global_;
     std::map<uint64_t, std::multimap<size_t, void*>> free_scoped_;  // one entry per live scope
+    std::map<uint64_t, uint64_t> scope_thread_;                     // live scope -> thread token
     struct Deferred {
         void* ptr;
         size_t cls;
         std::vector<uint64_t> waiting;
     };
     std::vector<Deferred> deferred_;
-    std::vector<std::pair<uint64_t, hipEvent_t>> pending_;  // scopes whose device work may still be running
+    std::deque<std::pair<uint64_t, hipEvent_t>> pending_;  // scopes whose device work may still be running, oldest first
+    std::vector<hipEvent_t> spare_events_;
     void end_scope_locked(uint64_t scope);
     uint64_t next_scope_ = 1, driver_bytes_ = 0, driver_allocs_ = 0, reuses_ = 0;
 };
@@ -56,6 +65,7 @@ struct Tensor {
     uint64_t scope = 0;
     std::vector<uint64_t> used;  // execution scopes that read or wrote the tensor (guarded by the pool's mutex)
     bool uploaded = false;       // filled by an asynchronous host-to-device copy
+    std::atomic<bool> ready_seen{false};  // `ready` has been observed complete (it is recorded once per tensor)
     hipEvent_t ready = nullptr;
     ~Tensor();
 };
@@ -68,6 +78,17 @@ void download_tensor(const TensorRef& t, void* dst);                         // 
 struct ExecStats {
     int steps = 0, instrs = 0, streams_used = 0, event_waits = 0;
 };
+
+// Everything about an execution that depends on the graph alone: the optimised copy, its plan and the tensors that
+// outlive the plan. Built once per graph by `prepare` and shared by every later execution.
+struct Prepared {
+    std::shared_ptr<const ir::OpGraph> graph;
+    std::shared_ptr<const plan::Plan> plan;
+    std::set<NodeId> alive;  // enumerate_output_tensors (cuda.rs:142-153)
+};
+std::shared_ptr<const Prepared> prepare(const ir::OpGraph& graph);
+std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std::map<NodeId, TensorRef>& inputs,
+                                             ExecStats* stats = nullptr);
 
 // BackendExt::execute_graph (backend.rs:40-80). `inputs`: storage for every Input node. Returns the storage of
 // every node that feeds an Output node, keyed by the Output node's id.

@@ -72,7 +72,7 @@ bool feeds_only_reductions(const ir::OpGraph& g, NodeId node, int budget = 64) {
 }  // namespace
 void set_fuse_matmul_epilogue(bool on) { g_fuse_matmul_epilogue.store(on); }
 bool fuse_matmul_epilogue() { return g_fuse_matmul_epilogue.load(); }
-static unsigned option_mask() { return (fuse_matmul_epilogue() ? 1u : 0u) | (g_fold_swap_into_reduce.load() ? 2u : 0u); }
+unsigned option_mask() { return (fuse_matmul_epilogue() ? 1u : 0u) | (g_fold_swap_into_reduce.load() ? 2u : 0u); }
 void set_fold_swap_into_reduce(bool on) { g_fold_swap_into_reduce.store(on); }
 bool fold_swap_into_reduce() { return g_fold_swap_into_reduce.load(); }
 

@@ -160,6 +160,7 @@ def test_four_threads_execute_concurrently(gpu):
     g, names = configs.c1_ir_graph(64, 96, 80)
     host = configs.c1_inputs(names, 64, 96, 80, batched=False)
     ref, _ = run_graph(g, host)
+    misses_before = stats()["plan_cache_misses"]
     errors = []
 
     def worker():
@@ -179,7 +180,8 @@ def test_four_threads_execute_concurrently(gpu):
     [t.join() for t in threads]
     assert not errors, errors[0]
     s = stats()
-    assert s["plan_cache_hits"] > 0 and s["pool_reuses"] > 0
+    # the plan made by the first execution is reused by all 80 later ones, and freed blocks go round
+    assert s["plan_cache_misses"] == misses_before and s["pool_reuses"] > 0
 
 
 @pytest.mark.parametrize("fold", [1, 0], ids=["statistics_without_permute", "reference_grouping"])
