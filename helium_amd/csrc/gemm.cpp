@@ -619,7 +619,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     }
     HE_REQUIRE(t.bm % (t.wm * 32) == 0 && t.bn % (t.wn * 32) == 0 && (t.bk == 64 || t.bk == 32) && (!f32 || t.bk == 32), HE_ERR_INVALID, "bad GEMM tile");
     const int threads = t.wm * t.wn * 64;
-    HE_REQUIRE(threads == 256 || threads == 512, HE_ERR_INVALID, "GEMM workgroups have 4 or 8 waves");
+    HE_REQUIRE(threads == 64 || threads == 128 || threads == 256 || threads == 512, HE_ERR_INVALID, "GEMM workgroups have 1, 2, 4 or 8 waves");
     HE_REQUIRE((t.bm * t.bk / epc) % threads == 0 && (t.bk * t.bn / epc) % threads == 0, HE_ERR_INVALID, "bad GEMM tile");
     HE_REQUIRE(t.stages >= 2 && t.stages <= 5 && t.stages * (t.bm + t.bn) * t.bk * (16 / epc) <= 160 * 1024, HE_ERR_INVALID,
                "GEMM tile exceeds LDS");

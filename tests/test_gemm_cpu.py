@@ -77,6 +77,8 @@ CASES = [
     ("three_stage_ring_short_k", lambda: gemm_cases.plain(128, 256, 32), "128,128,32,2,2,3"),
     ("three_stage_ring_bk64", lambda: gemm_cases.bias_relu_colsum(128, 128, 320), "128,128,64,2,2,3"),
     ("eight_waves_4x2", lambda: gemm_cases.all_reductions(256, 130, 64, batch=1), "256,128,64,4,2"),
+    ("one_wave_32x32_f32_direct", lambda: gemm_cases.plain(64, 96, 128, dtype="f32"), "32,32,32,1,1,4"),
+    ("two_waves_64x32_linear_layer", lambda: gemm_cases.linear_layer(48, 40, 72), "64,32,32,2,1,4"),
 ]
 
 
@@ -85,7 +87,8 @@ def test_fused_gemm_on_cpu(name, build, tile):
     g, inputs, outs = build()
     k, got = run_emulated(g, inputs, tile, env=("HELIUM_HIP_GEMM_EPIPIPE",) if "prefetched" in name else ())
     assert sorted(got) == sorted(outs), k.description
-    rounding = "f16" if name == "f16_operands" else None if name in ("f32_operands", "f32_linear_layer") else "bf16"
+    f32_cases = ("f32_operands", "f32_linear_layer", "one_wave_32x32_f32_direct", "two_waves_64x32_linear_layer")
+    rounding = "f16" if name == "f16_operands" else None if name in f32_cases else "bf16"
     want = oracle.outputs(g.nodes, inputs, round_mainloop_to=rounding)
     if rounding is None:
         compare(got, want, rel=1e-4, eps=1e-5)  # f32 multiplicands: 1e-4 relative
