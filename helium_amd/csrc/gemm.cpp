@@ -95,6 +95,8 @@ __device__ __forceinline__ u32 a_off(u32 m, u32 kc) { return m * (BK * ESZ) + ((
 #define B_SWZ(k) (MMA_F32 ? 0u : (((k) & 3) << 2) & (B_CHUNKS - 1))
 __device__ __forceinline__ u32 b_chunk_off(u32 k, u32 nc) { return k * (BN * ESZ) + ((nc ^ B_SWZ(k)) << 4); }
 __device__ __forceinline__ u32 b_off(u32 k, u32 n) { return b_chunk_off(k, (n * ESZ) >> 4) + ((n * ESZ) & 15); }
+// B_NK: B arrives with k contiguous ([n][k] in memory). Its tile is then [n][k] in LDS too, staged and read like
+// A's: the MFMA wants 8 consecutive k of one n per lane, which is one 16-byte chunk of row n.
 
 #if MMA_F32
 typedef f32x4 afrag_t;
@@ -129,8 +131,12 @@ __device__ __forceinline__ void load_frags(const unsigned char* __restrict__ st,
 #pragma unroll
     for (int j = 0; j < NB; j++) {
         const u32 n = w.wave_n * WTN + j * 32 + (lane & 31);
+#if B_NK
+        bf[j] = *(const f32x4*)(lb + a_off(n, kk * 2 + (lane >> 5)));
+#else
 #pragma unroll
         for (int e = 0; e < 4; e++) bf[j][e] = *(const float*)(lb + b_off(kk * 8 + (lane >> 5) * 4 + e, n));
+#endif
     }
 #else
     const u32 grp = lane >> 4, sub = lane & 15;
@@ -139,6 +145,14 @@ __device__ __forceinline__ void load_frags(const unsigned char* __restrict__ st,
         const u32 row = w.wave_m * WTM + i * 32 + (lane & 31);
         af[i] = *(const s16x8*)(la + a_off(row, kk * 2 + (lane >> 5)));
     }
+#if B_NK
+    (void)grp; (void)sub;
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+        const u32 n = w.wave_n * WTN + j * 32 + (lane & 31);
+        bf[j] = *(const s16x8*)(lb + a_off(n, kk * 2 + (lane >> 5)));
+    }
+#else
 #pragma unroll
     for (int j = 0; j < NB; j++) {
         const u32 k = kk * 16 + (grp >> 1) * 8 + (sub >> 2);
@@ -147,6 +161,7 @@ __device__ __forceinline__ void load_frags(const unsigned char* __restrict__ st,
         s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(lb + b_off(k + 4, n)));
         bf[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     }
+#endif
 #endif
 }
 
@@ -244,9 +259,15 @@ __device__ __forceinline__ void direct_issue(unsigned char* __restrict__ st, con
         __builtin_amdgcn_global_load_lds((GLOBAL_AS const void*)gp, (LDS_AS void*)(st + blk * 1024), 16, 0, 0);
     } else {
         const u32 blk = wave * B_DPW + (i - A_DPW);
+#if B_NK
+        const u32 row = blk * (64 / A_CHUNKS) + lane / A_CHUNKS, pc = lane % A_CHUNKS;
+        const u32 kc = pc ^ ((row >> A_SWZ_SHIFT) & (A_CHUNKS - 1));
+        const mul_t* gp = gb + (size_t)row * GK + kc * EPC;
+#else
         const u32 krow = blk * (64 / B_CHUNKS) + lane / B_CHUNKS, pc = lane % B_CHUNKS;
         const u32 nc = pc ^ B_SWZ(krow);
         const mul_t* gp = gb + (size_t)krow * GN + nc * EPC;
+#endif
         __builtin_amdgcn_global_load_lds((GLOBAL_AS const void*)gp, (LDS_AS void*)(st + A_TILE_BYTES + blk * 1024), 16, 0, 0);
     }
 }
@@ -325,11 +346,15 @@ void fused_matmul(KERNEL_PARAMS) {
 #pragma unroll
         for (int i = 0; i < B_PER_THREAD; i++) {
             const u32 idx = tid + i * NTHREADS;
-            const u32 krow = idx / B_CHUNKS, nc = idx % B_CHUNKS;
-#if RAW_B
-            sb[i] = fetch_b(FETCH_B_ARGS bz, k0 + krow, n0 + nc * EPC);
+#if B_NK
+            const u32 brow = n0 + idx / A_CHUNKS, bcol = k0 + (idx % A_CHUNKS) * EPC;
 #else
-            fetch_b_load(FETCH_B_ARGS bz, k0 + krow, n0 + nc * EPC, sb[i]);
+            const u32 brow = k0 + idx / B_CHUNKS, bcol = n0 + (idx % B_CHUNKS) * EPC;
+#endif
+#if RAW_B
+            sb[i] = fetch_b(FETCH_B_ARGS bz, brow, bcol);
+#else
+            fetch_b_load(FETCH_B_ARGS bz, brow, bcol, sb[i]);
 #endif
         }
 #endif
@@ -355,11 +380,18 @@ void fused_matmul(KERNEL_PARAMS) {
 #pragma unroll
         for (int i = 0; i < B_PER_THREAD; i++) {
             const u32 idx = tid + i * NTHREADS;
-            const u32 krow = idx / B_CHUNKS, nc = idx % B_CHUNKS;
-#if RAW_B
-            *(u32x4*)(lb + b_chunk_off(krow, nc)) = sb[i];
+#if B_NK
+            const u32 slot = a_off(idx / A_CHUNKS, idx % A_CHUNKS);
+            const u32 brow = n0 + idx / A_CHUNKS, bcol = k0 + (idx % A_CHUNKS) * EPC;
 #else
-            *(u32x4*)(lb + b_chunk_off(krow, nc)) = fetch_b_eval(FETCH_B_ARGS bz, k0 + krow, n0 + nc * EPC, sb[i]);
+            const u32 slot = b_chunk_off(idx / B_CHUNKS, idx % B_CHUNKS);
+            const u32 brow = k0 + idx / B_CHUNKS, bcol = n0 + (idx % B_CHUNKS) * EPC;
+#endif
+            (void)brow; (void)bcol;
+#if RAW_B
+            *(u32x4*)(lb + slot) = sb[i];
+#else
+            *(u32x4*)(lb + slot) = fetch_b_eval(FETCH_B_ARGS bz, brow, bcol, sb[i]);
 #endif
         }
 #endif
@@ -370,7 +402,13 @@ void fused_matmul(KERNEL_PARAMS) {
 #define WAITCNT_VM(n) ((((n) & 15) | (((n) >> 4) << 14)))
 #if DIRECT_LOADS
     const mul_t* const ga0 = (const mul_t*)DIRECT_A_PTR + ((size_t)bz * GM + m0) * GK;
+#if B_NK
+    const mul_t* const gb0 = (const mul_t*)DIRECT_B_PTR + ((size_t)bz * GN + n0) * GK;
+#define B_TILE_AT(k) (gb0 + (k))
+#else
     const mul_t* const gb0 = (const mul_t*)DIRECT_B_PTR + (size_t)bz * GK * GN + n0;
+#define B_TILE_AT(k) (gb0 + (size_t)(k) * GN)
+#endif
     // NSTAGES-deep ring of LDS stages: tile kt + NSTAGES - 1 is requested while tile kt is multiplied, so a
     // wave only ever waits for loads issued NSTAGES - 2 tiles earlier.
 #pragma unroll
@@ -378,7 +416,7 @@ void fused_matmul(KERNEL_PARAMS) {
         if (st < KT) {
 #pragma unroll
             for (int i = 0; i < A_DPW + B_DPW; i++)
-                direct_issue(lds + st * STAGE_BYTES, ga0 + k_tile(st) * BK, gb0 + (size_t)(k_tile(st) * BK) * GN, wpos, i);
+                direct_issue(lds + st * STAGE_BYTES, ga0 + k_tile(st) * BK, B_TILE_AT(k_tile(st) * BK), wpos, i);
         }
 #endif
 #if STAGED
@@ -426,7 +464,7 @@ void fused_matmul(KERNEL_PARAMS) {
 #if DIRECT_LOADS
         const u32 knext = more ? k_tile(next) * BK : 0u;
         direct_tile(lds + (kt % NSTAGES) * STAGE_BYTES, lds + (next % NSTAGES) * STAGE_BYTES, ga0 + knext,
-                    gb0 + (size_t)knext * GN, more, acc, wpos, frags);
+                    B_TILE_AT(knext), more, acc, wpos, frags);
 #else
         compute_tile(lds + (kt % NSTAGES) * STAGE_BYTES, acc, wpos, frags, [](int) {});
 #endif
@@ -489,7 +527,10 @@ void fused_matmul(KERNEL_PARAMS) {
 bool is_raw_copy(const tp::Program& p, int root, int mma_dtype) {
     const tp::Expr& e = p.exprs[root];
     if (e.kind != tp::Expr::Load || !e.access.chain.empty() || e.access.dtype != mma_dtype) return false;
-    return e.access.stride == ir::packed_strides(p.dims);
+    const ir::Shape packed = ir::packed_strides(p.dims);
+    for (size_t d = 0; d < p.dims.size(); d++)
+        if (p.dims[d] > 1 && e.access.stride[d] != packed[d]) return false;  // the stride of an extent-1 dim is never used
+    return true;
 }
 
 // The same program in two halves: `<name>_load` issues the full-vector loads into a Raw struct, `<name>_eval`
@@ -527,6 +568,10 @@ GemmProblem gemm_problem_from_fusion(const fir::OpGraph& g) {
     pr.K = sa[2];
     pr.op_a = tp::lower_operand(g, mm.a, &pr.root_a);
     pr.op_b = tp::lower_operand(g, mm.b, &pr.root_b);
+    if (operand_b_prefers_nk(pr.op_b) && !getenv("HELIUM_HIP_GEMM_NO_NK")) {
+        pr.op_b = tp::lower_operand(g, mm.b, &pr.root_b, true);
+        pr.b_nk = true;
+    }
     pr.epi = tp::lower_epilogue(g, anchor);
     // Multiplicand type (the fusion IR carries no Precision): f16 when every operand source is f16, f32 when every
     // one is f32, bf16 otherwise (mixed sources are rounded to bf16, the reference's MulBf16AccumF32).
@@ -540,6 +585,17 @@ GemmProblem gemm_problem_from_fusion(const fir::OpGraph& g) {
 
     assemble_gemm_args(pr);
     return pr;
+}
+
+bool operand_b_prefers_nk(const tp::Program& op_b) {
+    const tp::Expr* big = nullptr;
+    for (auto& e : op_b.exprs) {
+        if (e.kind != tp::Expr::Load) continue;
+        if (!e.access.chain.empty() || e.access.stride.size() != 3) return false;
+        if (!big || op_b.args[e.access.arg].numel > op_b.args[big->access.arg].numel) big = &e;
+    }
+    // dims are [batch, K, N]: stride[1] walks k, stride[2] walks n
+    return big && big->access.stride[1] == 1 && big->access.stride[2] > 1;
 }
 
 void assemble_gemm_args(GemmProblem& pr) {
@@ -598,7 +654,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     Tile t;
     bool small = false;
     const bool raw_a0 = is_raw_copy(pr.op_a, pr.root_a, pr.mma_dtype) && pr.K % epc == 0;
-    const bool raw_b0 = is_raw_copy(pr.op_b, pr.root_b, pr.mma_dtype) && pr.N % epc == 0;
+    const bool raw_b0 = is_raw_copy(pr.op_b, pr.root_b, pr.mma_dtype) && (pr.b_nk ? pr.K : pr.N) % epc == 0;
     const bool want_direct = !getenv("HELIUM_HIP_GEMM_NO_DIRECT");
     const int esz = 16 / epc;  // bytes per multiplicand
     if (const char* env = getenv("HELIUM_HIP_GEMM_TILE")) {
@@ -632,7 +688,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     const bool direct_a = want_direct && raw_a && pr.M % t.bm == 0 && pr.K % t.bk == 0 && (t.bm * t.bk * esz / 1024) % (threads / 64) == 0 &&
                           !getenv("HELIUM_HIP_GEMM_NO_DIRECT_A");
     const bool direct_b = want_direct && raw_b && pr.N % t.bn == 0 && pr.K % t.bk == 0 && (t.bk * t.bn * esz / 1024) % (threads / 64) == 0 &&
-                          64 % (t.bn / epc) == 0 && !getenv("HELIUM_HIP_GEMM_NO_DIRECT_B");
+                          (pr.b_nk || 64 % (t.bn / epc) == 0) && !getenv("HELIUM_HIP_GEMM_NO_DIRECT_B");
     if (!(direct_a && direct_b)) t.stages = 2;  // register staging is double-buffered only
     else if (!getenv("HELIUM_HIP_GEMM_TILE") && small) {
         // A grid that leaves CUs idle is bound by the latency of its k-loop: keep as many tiles in flight as LDS holds.
@@ -659,7 +715,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
       << "\n#define GEMM_SKIP " << (getenv("HELIUM_HIP_GEMM_SKIP") ? atoi(getenv("HELIUM_HIP_GEMM_SKIP")) : 0)
       << "\n#define GEMM_TIMING " << (getenv("HELIUM_HIP_GEMM_TIMING") ? 1 : 0) << "\n#define GEMM_TIMING_PTR p" << (pr.args.size() - 1)
       << "\n#define DIRECT_A " << (direct_a ? 1 : 0) << "\n#define DIRECT_B " << (direct_b ? 1 : 0)
-      << "\n#define DIRECT_LOADS (DIRECT_A || DIRECT_B)\n#define STAGED (!DIRECT_A || !DIRECT_B)"
+      << "\n#define B_NK " << (pr.b_nk ? 1 : 0) << "\n#define DIRECT_LOADS (DIRECT_A || DIRECT_B)\n#define STAGED (!DIRECT_A || !DIRECT_B)"
       << "\n#define DIRECT_A_PTR p" << (direct_a ? pr.map_a[0] : 0)
       << "\n#define DIRECT_B_PTR p" << (direct_b ? pr.map_b[0] : 0) << "\n#define STAGE_SCHED_BARRIER "
       << ((getenv("HELIUM_HIP_GEMM_PIN") ? atoi(getenv("HELIUM_HIP_GEMM_PIN")) != 0 : true) ? "__builtin_amdgcn_sched_barrier(0);" : "") << "\n#define A_SWZ_SHIFT " << (getenv("HELIUM_HIP_GEMM_ASWZ") ? atoi(getenv("HELIUM_HIP_GEMM_ASWZ")) : (t.bk == 64 ? 1 : 2)) << "\n";
@@ -710,7 +766,8 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         s << "return pack_chunk(v);\n}\n";
     };
     emit_fetch("a", pr.op_a, pr.root_a, pr.map_a, raw_a, nva, "GM", "GK", pr.M % t.bm == 0 && pr.K % t.bk == 0);
-    emit_fetch("b", pr.op_b, pr.root_b, pr.map_b, raw_b, nvb, "GK", "GN", pr.K % t.bk == 0 && pr.N % t.bn == 0);
+    if (pr.b_nk) emit_fetch("b", pr.op_b, pr.root_b, pr.map_b, raw_b, nvb, "GN", "GK", pr.K % t.bk == 0 && pr.N % t.bn == 0);
+    else emit_fetch("b", pr.op_b, pr.root_b, pr.map_b, raw_b, nvb, "GK", "GN", pr.K % t.bk == 0 && pr.N % t.bn == 0);
 
     // epilogue pieces
     std::ostringstream setup, body, finish, prefetch;

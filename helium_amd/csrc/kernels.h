@@ -68,7 +68,10 @@ private:
 struct GemmProblem {
     int64_t batch = 1, M = 0, N = 0, K = 0;
     int mma_dtype = HE_BF16;       // multiplicand type: HE_BF16, HE_F16 or HE_F32
-    tp::Program op_a, op_b, epi;   // dims [batch,M,K], [batch,K,N], [batch,M,N]
+    tp::Program op_a, op_b, epi;   // dims [batch,M,K], [batch,K,N] ([batch,N,K] when b_nk), [batch,M,N]
+    // B's source is contiguous along k (a transposed matrix, a convolution filter): its program iterates [batch,N,K],
+    // its tile is staged and read like A's, with 16-byte chunks along k.
+    bool b_nk = false;
     int root_a = -1, root_b = -1;  // expression ids of the operand values in op_a / op_b
     std::vector<tp::Arg> args;     // the kernel's arguments: inputs in node order, then outputs in node order
     std::vector<int> map_a, map_b, map_e;  // program argument -> kernel argument
@@ -76,6 +79,9 @@ struct GemmProblem {
 GemmProblem gemm_problem_from_fusion(const fir::OpGraph& g);
 // Fills args / map_a / map_b / map_e from the three programs: distinct inputs in node order, then outputs.
 void assemble_gemm_args(GemmProblem& pr);
+// True when the B operand program (over [batch,K,N]) reads its largest source with unit stride along k and a
+// larger one along n: lowering it over [batch,N,K] instead makes its accesses vectors.
+bool operand_b_prefers_nk(const tp::Program& op_b);
 // Throws HE_ERR_UNSUPPORTED for an epilogue program the GEMM kernel cannot run.
 void validate_gemm_epilogue(const tp::Program& epi);
 

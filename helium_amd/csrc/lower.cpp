@@ -513,9 +513,11 @@ public:
     }
 
     // The value of one node (a Matmul operand with its mainloop ops) over that node's own shape.
-    Program run_value(fir::OpNode value, int* root) {
+    // `transposed`: iterate the value as [batch, cols, rows], so that vectors run along its rows' direction
+    Program run_value(fir::OpNode value, int* root, bool transposed = false) {
         const fir::Shape3& s = g_.shape(value);
         p_.dims = {s[0], s[1], s[2]};
+        if (transposed) p_.dims = {s[0], s[2], s[1]};
         std::vector<fir::OpNode> producers, stack{value};
         std::map<fir::OpNode, char> seen;
         while (!stack.empty()) {
@@ -535,6 +537,7 @@ public:
         }
         Mapping ident;
         ident.w = ir::packed_strides(p_.dims);
+        if (transposed) ident.w = {(int64_t)s[1] * s[2], 1, (int64_t)s[2]};  // the value's own packed strides, per iteration dim
         *root = eval(value, ident);
         return std::move(p_);
     }
@@ -705,8 +708,8 @@ Program lower_aux(const fir::OpGraph& g) {
     HE_REQUIRE(g.anchor() == fir::kNoOpNode, HE_ERR_INVALID, "an auxiliary fusion holds no Matmul");
     return FusionLowering(g, fir::kNoOpNode).run();
 }
-Program lower_operand(const fir::OpGraph& g, fir::OpNode value, int* root_expr) {
-    return FusionLowering(g, fir::kNoOpNode).run_value(value, root_expr);
+Program lower_operand(const fir::OpGraph& g, fir::OpNode value, int* root_expr, bool transposed) {
+    return FusionLowering(g, fir::kNoOpNode).run_value(value, root_expr, transposed);
 }
 Program lower_epilogue(const fir::OpGraph& g, fir::OpNode anchor) {
     Program p = FusionLowering(g, anchor).run();

@@ -108,7 +108,8 @@ Program lower_aux(const fir::OpGraph& g);
 Program lower_epilogue(const fir::OpGraph& g, fir::OpNode anchor);
 // One Matmul operand together with the mainloop ops that produce it, evaluated over the operand's own shape
 // ([batch, M, K] for a, [batch, K, N] for b). `root_expr` receives the id of the operand's value.
-Program lower_operand(const fir::OpGraph& g, fir::OpNode value, int* root_expr);
+// `transposed`: the same values iterated as [batch, cols, rows] (vector accesses then run along the value's rows).
+Program lower_operand(const fir::OpGraph& g, fir::OpNode value, int* root_expr, bool transposed = false);
 
 // ---- emission -----------------------------------------------------------------------------------------------
 struct PointwiseLaunch {

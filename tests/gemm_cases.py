@@ -25,6 +25,26 @@ def plain(m, n, k, batch=1, seed=0, dtype="bf16", out_dtype="f32", scale=0.5):
     return g, inputs, [out]
 
 
+def transposed_b(m, n, k, batch=1, seed=4, dtype="bf16", out_dtype="f32", scale=0.5, scaled=False):
+    """C = A * Bt^T with Bt stored [batch, n, k] (k contiguous): the mainloop's Transpose op on the B operand.
+    `scaled`: Bt is also multiplied by a [batch, n, 1] column before the transposition (a fused mainloop)."""
+    g = ha.fusion.OpGraph()
+    rng = np.random.default_rng(seed)
+    a = g.producer([batch, m, k], dtype); bt = g.producer([batch, n, k], dtype)
+    if dtype == "bf16":
+        inputs = {a: bf16_normal(rng, (batch, m, k), scale), bt: bf16_normal(rng, (batch, n, k), scale)}
+    else:
+        inputs = {a: (rng.standard_normal((batch, m, k)) * scale).astype(np.float32),
+                  bt: (rng.standard_normal((batch, n, k)) * scale).astype(np.float32)}
+    b = bt
+    if scaled:
+        col = g.producer([batch, n, 1], "f32")
+        inputs[col] = rng.uniform(0.5, 1.5, (batch, n, 1)).astype(np.float32)
+        b = g.binary(bt, g.broadcast(col, 2, k), "mul")
+    out = g.consumer(g.matmul(a, g.transpose(b)), out_dtype)
+    return g, inputs, [out]
+
+
 def linear_layer(m, k, n):
     """Config 1 at a small size: f32 Y = relu(X W + b) and its column sums."""
     from helium_amd import configs

@@ -130,3 +130,18 @@ def test_c5a_mainloop_and_epilogue(gpu, size):
 
     g, names = configs.c5a_graph(size)
     check_reductions_and_full(g, configs.c5a_inputs(names, size))
+
+
+@pytest.mark.parametrize("m,n,k,batch,scaled", [(256, 256, 128, 1, False), (512, 768, 320, 1, False), (100, 100, 100, 2, False),
+                                                (257, 263, 129, 1, True), (1024, 1024, 1024, 1, True), (4096, 4096, 512, 1, False)])
+def test_b_operand_stored_transposed(gpu, m, n, k, batch, scaled):
+    """C = A * Bt^T with Bt stored [n][k]: the B tile is staged and read like A's (chunks along k), straight from
+    global memory into LDS when Bt is used as it is, through registers when a mainloop op works on it first."""
+    g, inputs, outs = gemm_cases.transposed_b(m, n, k, batch=batch, scaled=scaled)
+    kernel = check(g, inputs, outs)
+    assert "NVB=8" in kernel.description or k % 8, kernel.description
+
+
+def test_b_operand_stored_transposed_f32(gpu):
+    g, inputs, outs = gemm_cases.transposed_b(192, 200, 136, dtype="f32")
+    check(g, inputs, outs, mma=None, rel=1e-4, eps=1e-5)
