@@ -320,6 +320,73 @@ class BatchNormWorkload:
         self.tensors, self.last = {}, None
 
 
+class ConvWorkload:
+    """One convolution of BASELINE config 5b's network through execute_graph: the 3x3, stride-1 convolution of a
+    64-channel residual block on a bf16 NHWC activation of [64,56,56,64] (resnet-train/src/model.rs), run as an
+    implicit GEMM: M = 64*56*56 output pixels, N = 64 output channels, K = 3*3*64 filter taps."""
+
+    bound = "mfma"
+    unit = "TFLOP/s"
+    dtype = "bf16 x bf16 -> f32 accumulate, bf16 output"
+    name = "C5b-conv"
+    wall_timed = True
+    image = (64, 56, 56, 64)
+    out_channels = 64
+    kernel = (3, 3)
+
+    def __init__(self):
+        n, h, w, c = self.image
+        self.work = 2.0 * n * h * w * self.out_channels * self.kernel[0] * self.kernel[1] * c
+
+    def describe(self):
+        return "C5b-conv: bf16 [64,56,56,64] conv 3x3 -> 64 channels via execute_graph (implicit GEMM 200704 x 64 x 576)"
+
+    def setup(self):
+        import helium_amd as ha
+        from helium_amd import configs
+        from helium_amd.backend import Plan, Tensor
+
+        g = ha.ir.OpGraph()
+        c = self.image[3]
+        fshape = [self.out_channels, self.kernel[0], self.kernel[1], c]
+        x = g.new_input(list(self.image), "bf16")
+        w = g.new_input(fshape, "bf16")
+        self.params = {"in_channels": c, "out_channels": self.out_channels, "kernel_size": list(self.kernel)}
+        y = g.conv(x, w, self.params)
+        self.out = g.new_output(y)
+        rng = np.random.default_rng(53)
+        self.host = {x: configs.bf16_rne(rng.standard_normal(self.image, dtype=np.float32)),
+                     w: configs.bf16_rne(rng.standard_normal(fshape, dtype=np.float32) * 0.05)}
+        self.x, self.w, self.graph = x, w, g
+        self.tensors = {i: Tensor.from_numpy(a, "bf16", a.size) for i, a in self.host.items()}
+        self.last = None
+        log(f"[bench] {self.describe()} :: plan: " + Plan(g).text.replace("\n", " ; "))
+
+    def step(self, stream, i):
+        from helium_amd.backend import execute_graph
+
+        self.last = execute_graph(self.graph, self.tensors)
+
+    def check(self):
+        """The oracle's cross-correlation on the first two images of the batch."""
+        from oracle import helium_ir as oracle
+        from oracle import numerics as nm
+
+        img = nm.bf16_bits_to_f32(self.host[self.x]).reshape(self.image)[:2]
+        flt = nm.bf16_bits_to_f32(self.host[self.w]).reshape(self.out_channels, *self.kernel, self.image[3])
+        want = oracle.conv(img, flt, self.params, "bf16").astype(np.float64)
+        got = nm.bf16_bits_to_f32(self.last[self.out].to_numpy()).reshape(self.image[0], -1)[:2].reshape(want.shape).astype(np.float64)
+        if not (np.abs(got - want) <= 1e-2 * np.maximum(np.abs(want), 1.0)).all():
+            raise SystemExit("[bench] PARITY FAILURE in C5b-conv: output differs from the oracle")
+        return "first two images within 1e-2 of the oracle's float64 cross-correlation"
+
+    def cpu_baseline(self, budget_s=5.0):
+        return None
+
+    def free(self):
+        self.tensors, self.last = {}, None
+
+
 class FusedGemmWorkload:
     """BASELINE configs 4 / 5a: 4096^3 bf16 GEMM with fused mainloop / epilogue. Work = 2*M*N*K FLOP."""
 
@@ -460,6 +527,7 @@ def make_workloads():
     w["C1"] = LinearLayerWorkload()
     w["C3"] = AuxChainWorkload()
     w["C5b-bn"] = BatchNormWorkload()
+    w["C5b-conv"] = ConvWorkload()
     for name in ("C4", "C5a", "C4m", "GEMM"):
         w[name] = FusedGemmWorkload(name)
     return w

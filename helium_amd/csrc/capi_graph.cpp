@@ -30,6 +30,18 @@ ir::Op op_from_desc(const he_op_desc& d) {
     op.axis_b = d.axis_b;
     op.const_bits = d.const_bits;
     op.const_dtype = d.const_dtype;
+    if (op.kind == ir::OpKind::Conv || op.kind == ir::OpKind::ConvBackwardData || op.kind == ir::OpKind::ConvBackwardFilter) {
+        op.conv.in_channels = d.conv_in_channels;
+        op.conv.out_channels = d.conv_out_channels;
+        for (int i = 0; i < 2; i++) {
+            op.conv.kernel[i] = d.conv_kernel[i];
+            op.conv.stride[i] = d.conv_stride[i];
+            op.conv.dilation[i] = d.conv_dilation[i];
+            op.conv.input_size[i] = d.conv_input_size[i];
+        }
+        HE_REQUIRE(d.conv_padding_mode >= HE_PAD_SAME && d.conv_padding_mode <= HE_PAD_FULL, HE_ERR_INVALID, "bad padding mode");
+        op.conv.padding_mode = d.conv_padding_mode;
+    }
     if (op.kind == ir::OpKind::ChangeDataType || op.kind == ir::OpKind::Constant)
         (void)dtype_bits(op.kind == ir::OpKind::Constant ? op.const_dtype : op.target_type);
     return op;

@@ -653,7 +653,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     const int epc = f32 ? 4 : 8;  // multiplicands per 16-byte chunk
     Tile t;
     bool small = false;
-    const bool raw_a0 = is_raw_copy(pr.op_a, pr.root_a, pr.mma_dtype) && pr.K % epc == 0;
+    const bool raw_a0 = pr.conv_a.on || (is_raw_copy(pr.op_a, pr.root_a, pr.mma_dtype) && pr.K % epc == 0);
     const bool raw_b0 = is_raw_copy(pr.op_b, pr.root_b, pr.mma_dtype) && (pr.b_nk ? pr.K : pr.N) % epc == 0;
     const bool want_direct = !getenv("HELIUM_HIP_GEMM_NO_DIRECT");
     const int esz = 16 / epc;  // bytes per multiplicand
@@ -664,6 +664,16 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         t = {v[0], v[1], v[2], v[3], v[4], v[5]};
     } else {
         if (f32) t.bk = 32;  // same bytes per tile row as 64 two-byte multiplicands
+        // A skinny product (few output columns, many rows: a convolution with 64 output channels) takes tiles as
+        // narrow as N, so that no matrix-core work is spent on columns that do not exist; eight waves of 64x32
+        // (measured on [200704 x 576] x [576 x 64]: 71 us with 128x128 tiles, 44 us with 256x64).
+        const bool skinny = !f32 && pr.N <= 64 && pr.N > 32 && pr.M >= 256 * 256;
+        if (skinny) {
+            t.bm = 256;
+            t.bn = 64;
+            t.wm = 4;
+            t.wn = 2;
+        } else
         // Smaller problems take smaller tiles so that every CU gets work.
         if (pr.M <= 128 || pr.N <= 128 || ((pr.M + 255) / 256) * ((pr.N + 255) / 256) * pr.batch < 128) {
             t.bm = t.bn = 128;
@@ -685,7 +695,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     const int nva = std::min(epc, tp::pick_nv(pr.op_a, 16)), nvb = std::min(epc, tp::pick_nv(pr.op_b, 16));
     // Direct global->LDS loads need unpredicated, unmodified 16-byte chunks: raw operands and full tiles everywhere.
     // Each operand qualifies on its own; the other one then goes through registers.
-    const bool direct_a = want_direct && raw_a && pr.M % t.bm == 0 && pr.K % t.bk == 0 && (t.bm * t.bk * esz / 1024) % (threads / 64) == 0 &&
+    const bool direct_a = want_direct && !pr.conv_a.on && raw_a && pr.M % t.bm == 0 && pr.K % t.bk == 0 && (t.bm * t.bk * esz / 1024) % (threads / 64) == 0 &&
                           !getenv("HELIUM_HIP_GEMM_NO_DIRECT_A");
     const bool direct_b = want_direct && raw_b && pr.N % t.bn == 0 && pr.K % t.bk == 0 && (t.bk * t.bn * esz / 1024) % (threads / 64) == 0 &&
                           (pr.b_nk || 64 % (t.bn / epc) == 0) && !getenv("HELIUM_HIP_GEMM_NO_DIRECT_B");
@@ -765,7 +775,28 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         else s << guard << "operand_" << W << "_eval(" << pass << "b, row, col + j, R[j / " << nv << "], v + j);\nelse {\n#pragma unroll\nfor (int k = 0; k < " << nv << "; k++) v[j + k] = 0.0f; }\n}\n";
         s << "return pack_chunk(v);\n}\n";
     };
-    emit_fetch("a", pr.op_a, pr.root_a, pr.map_a, raw_a, nva, "GM", "GK", pr.M % t.bm == 0 && pr.K % t.bk == 0);
+    if (pr.conv_a.on) {
+        // The gather of an implicit-GEMM convolution in place of A's loads: one 16-byte chunk is EPC consecutive
+        // channels of one filter tap when the channel count allows, EPC separate taps otherwise (a 3-channel image).
+        const auto& cv = pr.conv_a;
+        const tp::Arg& img = pr.op_a.args[0];
+        s << "#define FETCH_A_ARGS p" << pr.map_a[0] << ", \n#define RAW_A 1\n#define SPLIT_A 1\n";
+        s << "__device__ __forceinline__ bool conv_tap(u32 row, u32 col, size_t& at) {\n"
+          << "const u32 n = row / " << cv.P * cv.Q << "u, pq = row % " << cv.P * cv.Q << "u, p = pq / " << cv.Q << "u, q = pq % " << cv.Q << "u;\n"
+          << "const u32 rs = col / " << cv.C << "u, c = col % " << cv.C << "u, r = rs / " << cv.S << "u, sx = rs % " << cv.S << "u;\n"
+          << "const int ih = (int)(p * " << cv.sh << "u + r * " << cv.dh << "u) - " << cv.ph << ", iw = (int)(q * " << cv.sw << "u + sx * " << cv.dw << "u) - " << cv.pw << ";\n"
+          << "at = (((size_t)n * " << cv.H << "u + (u32)ih) * " << cv.W << "u + (u32)iw) * " << cv.C << "u + c;\n"
+          << "return row < GM && col < GK && ih >= 0 && ih < " << cv.H << " && iw >= 0 && iw < " << cv.W << ";\n}\n";
+        s << "__device__ __forceinline__ u32x4 fetch_a(const " << tp::c_type(img.dtype) << "* __restrict__ q0, u32 b, u32 row, u32 col) {\n(void)b;\n";
+        if (cv.C % epc == 0) {
+            s << "u32x4 v = {0u, 0u, 0u, 0u};\nsize_t at;\nif (conv_tap(row, col, at)) v = *(const u32x4*)(q0 + at);\nreturn v;\n}\n";
+        } else {
+            s << "float v[" << epc << "];\n#pragma unroll\nfor (int j = 0; j < " << epc << "; j++) {\nsize_t at;\nv[j] = conv_tap(row, col + j, at) ? ld_one(q0 + at) : 0.0f;\n}\n"
+              << "return pack_chunk(v);\n}\n";
+        }
+    } else {
+        emit_fetch("a", pr.op_a, pr.root_a, pr.map_a, raw_a, nva, "GM", "GK", pr.M % t.bm == 0 && pr.K % t.bk == 0);
+    }
     if (pr.b_nk) emit_fetch("b", pr.op_b, pr.root_b, pr.map_b, raw_b, nvb, "GN", "GK", pr.K % t.bk == 0 && pr.N % t.bn == 0);
     else emit_fetch("b", pr.op_b, pr.root_b, pr.map_b, raw_b, nvb, "GK", "GN", pr.K % t.bk == 0 && pr.N % t.bn == 0);
 

@@ -24,8 +24,25 @@ int accumulator_type(Precision p) {
     }
 }
 
+bool ConvParams::operator==(const ConvParams& o) const {
+    return in_channels == o.in_channels && out_channels == o.out_channels && kernel[0] == o.kernel[0] && kernel[1] == o.kernel[1] &&
+           stride[0] == o.stride[0] && stride[1] == o.stride[1] && dilation[0] == o.dilation[0] && dilation[1] == o.dilation[1] &&
+           padding_mode == o.padding_mode && input_size[0] == o.input_size[0] && input_size[1] == o.input_size[1];
+}
+void ConvParams::output_size(const int64_t in[2], const int64_t kernel_size[2], int64_t out[2]) const {
+    for (int d = 0; d < 2; d++) {
+        int64_t v = in[d];
+        if (padding_mode == 2) v += kernel_size[d] / 2;
+        else if (padding_mode == 1) v = std::max<int64_t>(0, v - kernel_size[d] / 2);
+        out[d] = v / stride[d];
+    }
+}
+void ConvParams::padding(int64_t pad[2]) const {
+    for (int d = 0; d < 2; d++) pad[d] = padding_mode == 0 ? kernel[d] / 2 : padding_mode == 1 ? 0 : kernel[d] - 1;
+}
+
 bool Op::operator==(const Op& o) const {
-    return kind == o.kind && inputs == o.inputs && sub_op == o.sub_op && precision == o.precision &&
+    return conv == o.conv && kind == o.kind && inputs == o.inputs && sub_op == o.sub_op && precision == o.precision &&
            f8_modes == o.f8_modes && target_type == o.target_type && depth == o.depth &&
            new_dim_count == o.new_dim_count && broadcast_axes == o.broadcast_axes && shape == o.shape &&
            axis_a == o.axis_a && axis_b == o.axis_b && const_bits == o.const_bits && const_dtype == o.const_dtype;
@@ -46,6 +63,11 @@ uint64_t Op::hash() const {
     mix(&axis_b, sizeof axis_b);
     mix(&const_bits, sizeof const_bits);
     mix(&const_dtype, sizeof const_dtype);
+    if (kind == OpKind::Conv || kind == OpKind::ConvBackwardData || kind == OpKind::ConvBackwardFilter) {
+        const int64_t c[] = {conv.in_channels, conv.out_channels, conv.kernel[0], conv.kernel[1], conv.stride[0], conv.stride[1],
+                             conv.dilation[0], conv.dilation[1], conv.padding_mode, conv.input_size[0], conv.input_size[1]};
+        mix(c, sizeof c);
+    }
     return h;
 }
 
@@ -126,10 +148,22 @@ Descriptor OpGraph::infer(const Op& op, const OpGraph& g) {
         case OpKind::Compare: return {in(0).shape, HE_BOOL};
         case OpKind::Select: return in(0);
         case OpKind::Constant: return {op.shape, op.const_dtype};
-        case OpKind::Conv:
-        case OpKind::ConvBackwardData:
-        case OpKind::ConvBackwardFilter:
-            fail(HE_ERR_UNSUPPORTED, "convolution ops are outside this backend's path");
+        case OpKind::Conv: {
+            // op.rs:123-142: NHWC image, [out_channels, kh, kw, in_channels] filter; the image's dtype
+            const Descriptor &image = in(0), &filter = in(1);
+            HE_REQUIRE(image.shape.size() == 4 && filter.shape.size() == 4, HE_ERR_INVALID, "conv takes rank-4 image and filter");
+            HE_REQUIRE(op.conv.in_channels > 0 && op.conv.out_channels > 0 && op.conv.kernel[0] > 0 && op.conv.kernel[1] > 0 &&
+                           op.conv.stride[0] > 0 && op.conv.stride[1] > 0 && op.conv.dilation[0] > 0 && op.conv.dilation[1] > 0,
+                       HE_ERR_INVALID, "conv parameters must be positive (Conv2dParams::validate)");
+            const int64_t in_size[2] = {image.shape[1], image.shape[2]}, k_size[2] = {filter.shape[1], filter.shape[2]};
+            int64_t out[2];
+            op.conv.output_size(in_size, k_size, out);
+            return {{image.shape[0], out[0], out[1], op.conv.out_channels}, image.dtype};
+        }
+        case OpKind::ConvBackwardData:  // op.rs:143-158
+            return {{in(0).shape.at(0), op.conv.input_size[0], op.conv.input_size[1], op.conv.in_channels}, in(0).dtype};
+        case OpKind::ConvBackwardFilter:  // op.rs:159-173
+            return {{op.conv.out_channels, op.conv.kernel[0], op.conv.kernel[1], op.conv.in_channels}, in(0).dtype};
     }
     fail(HE_ERR_INVALID, "bad op kind");
 }

@@ -41,6 +41,18 @@ struct BroadcastAxis {
     bool operator==(const BroadcastAxis& o) const { return axis == o.axis && new_size == o.new_size; }
 };
 
+// Conv2dParams (opgraph/op/conv.rs:5-12) and ConvBackwardData::input_size (op.rs:462-468).
+struct ConvParams {
+    int64_t in_channels = 0, out_channels = 0;
+    int64_t kernel[2] = {1, 1}, stride[2] = {1, 1}, dilation[2] = {1, 1};
+    int padding_mode = 0;            // 0 Same, 1 Valid, 2 Full
+    int64_t input_size[2] = {0, 0};  // ConvBackwardData only
+    bool operator==(const ConvParams& o) const;
+    // compute_output_size (conv.rs:51-73) and compute_padding_amount (conv.rs:85-91)
+    void output_size(const int64_t in[2], const int64_t kernel_size[2], int64_t out[2]) const;
+    void padding(int64_t pad[2]) const;
+};
+
 struct Op {
     OpKind kind = OpKind::Constant;
     std::vector<NodeId> inputs;  // Matmul: a,b; Binary/Compare: lhs,rhs; Select: lhs,rhs,selector
@@ -55,6 +67,7 @@ struct Op {
     int64_t axis_a = 0, axis_b = 0;
     uint32_t const_bits = 0;     // Constant scalar, bit pattern in its own dtype
     int const_dtype = HE_F32;
+    ConvParams conv;             // Conv (image, filter), ConvBackwardData (flow, filter), ConvBackwardFilter (flow, image)
     bool operator==(const Op& o) const;
     uint64_t hash() const;
 };

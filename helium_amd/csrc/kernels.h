@@ -72,6 +72,13 @@ struct GemmProblem {
     // B's source is contiguous along k (a transposed matrix, a convolution filter): its program iterates [batch,N,K],
     // its tile is staged and read like A's, with 16-byte chunks along k.
     bool b_nk = false;
+    // Implicit-GEMM convolution: the A operand is never materialised. Row m of A is output pixel (n, p, q), column k
+    // is filter tap (r, s, c); the element is image[n][p*sh + r*dh - ph][q*sw + s*dw - pw][c], or zero outside the
+    // image. op_a then only names the image argument.
+    struct ConvGather {
+        bool on = false;
+        int64_t N = 0, H = 0, W = 0, C = 0, R = 0, S = 0, P = 0, Q = 0, sh = 1, sw = 1, dh = 1, dw = 1, ph = 0, pw = 0;
+    } conv_a;
     int root_a = -1, root_b = -1;  // expression ids of the operand values in op_a / op_b
     std::vector<tp::Arg> args;     // the kernel's arguments: inputs in node order, then outputs in node order
     std::vector<int> map_a, map_b, map_e;  // program argument -> kernel argument

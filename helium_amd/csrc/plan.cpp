@@ -130,7 +130,10 @@ Instr make_instr_for_op(const std::shared_ptr<const ir::OpGraph>& g, NodeId node
         case ir::OpKind::Compare:
         case ir::OpKind::Select: return Instr(InstrKind::Pointwise, sg);
         case ir::OpKind::Matmul: return Instr(InstrKind::Gemm, sg);
-        default: fail(HE_ERR_UNSUPPORTED, "convolution ops have no instruction in this backend");
+        // The reference hands convolutions to cuDNN (cuda.rs:55-58, cudnn_graph.rs:193-204); here the forward
+        // convolution is the fused GEMM with an implicit im2col gather as its A operand.
+        case ir::OpKind::Conv: return Instr(InstrKind::Gemm, sg);
+        default: fail(HE_ERR_UNSUPPORTED, "the convolution backward ops have no instruction in this backend");
     }
 }
 
@@ -467,8 +470,74 @@ void plan_cache_stats(uint64_t* hits, uint64_t* misses) {
 // ---------------------------------------------------------------------------------------------------------
 // helium-ir Matmul -> GEMM problem
 // ---------------------------------------------------------------------------------------------------------
+namespace {
+// Op::Conv as a GEMM: rows = output pixels (n, p, q), columns = output channels, k = filter taps (r, s, c). The
+// filter [out_channels, kh, kw, in_channels] is B with k contiguous; A is gathered from the NHWC image on the fly.
+GemmProblem conv_problem(const ir::OpSubgraph& sg, NodeId conv) {
+    const ir::OpGraph& g = *sg.graph();
+    HE_REQUIRE(sg.nodes().size() == 1, HE_ERR_UNSUPPORTED, "a convolution instruction holds the Conv alone");
+    const ir::Op& op = g.get(conv).op;
+    const ir::Descriptor &image = g.get(op.inputs[0]).desc, &filter = g.get(op.inputs[1]).desc, &out = g.get(conv).desc;
+    HE_REQUIRE(dtype_class(image.dtype) == DataClass::Float && filter.dtype == image.dtype, HE_ERR_UNSUPPORTED,
+               "conv takes a float image and a filter of the same type");
+    HE_REQUIRE(filter.shape[0] == op.conv.out_channels && filter.shape[3] == op.conv.in_channels && image.shape[3] == op.conv.in_channels &&
+                   filter.shape[1] == op.conv.kernel[0] && filter.shape[2] == op.conv.kernel[1],
+               HE_ERR_INVALID, "conv filter / image shapes do not match the parameters");
+    GemmProblem pr;
+    auto& cv = pr.conv_a;
+    cv.on = true;
+    cv.N = image.shape[0]; cv.H = image.shape[1]; cv.W = image.shape[2]; cv.C = image.shape[3];
+    cv.R = filter.shape[1]; cv.S = filter.shape[2];
+    cv.P = out.shape[1]; cv.Q = out.shape[2];
+    cv.sh = op.conv.stride[0]; cv.sw = op.conv.stride[1];
+    cv.dh = op.conv.dilation[0]; cv.dw = op.conv.dilation[1];
+    int64_t pad[2];
+    op.conv.padding(pad);
+    cv.ph = pad[0]; cv.pw = pad[1];
+    pr.batch = 1;
+    pr.M = cv.N * cv.P * cv.Q;
+    pr.N = op.conv.out_channels;
+    pr.K = cv.R * cv.S * cv.C;
+    HE_REQUIRE(pr.M > 0 && pr.M < (1ll << 31) && ir::num_elements(image.shape) < (1ll << 32), HE_ERR_UNSUPPORTED, "conv too large for 32-bit tile indices");
+    pr.mma_dtype = image.dtype == HE_F32 ? HE_F32 : image.dtype == HE_F16 ? HE_F16 : HE_BF16;
+    auto operand = [&](tp::Program& p, const ir::Descriptor& d, NodeId node, int64_t rows, int64_t cols) {
+        p.dims = {1, rows, cols};
+        p.args.push_back({d.dtype, ir::num_elements(d.shape), false, node});
+        tp::Expr e;
+        e.kind = tp::Expr::Load;
+        e.cls = tp::Cls::F;
+        e.access.arg = 0;
+        e.access.dtype = d.dtype;
+        e.access.stride = ir::packed_strides(p.dims);
+        p.exprs.push_back(e);
+    };
+    operand(pr.op_a, image, op.inputs[0], pr.M, pr.K);   // stands for the gathered matrix; only its argument is used
+    operand(pr.op_b, filter, op.inputs[1], pr.N, pr.K);  // [n][k]: k contiguous
+    pr.b_nk = true;
+    pr.root_a = pr.root_b = 0;
+    pr.epi.dims = {1, pr.M, pr.N};
+    pr.epi.fast_math = true;
+    tp::Expr acc;
+    acc.kind = tp::Expr::Acc;
+    acc.cls = tp::Cls::F;
+    pr.epi.exprs.push_back(acc);
+    pr.epi.acc_expr = 0;
+    tp::Out o;
+    o.expr = 0;
+    o.arg = 0;
+    o.dtype = out.dtype;
+    pr.epi.outs.push_back(o);
+    pr.epi.args.push_back({out.dtype, ir::num_elements(out.shape), true, conv});
+    validate_gemm_epilogue(pr.epi);
+    assemble_gemm_args(pr);
+    return pr;
+}
+}  // namespace
+
 GemmProblem gemm_problem_from_ir(const ir::OpSubgraph& sg) {
     const ir::OpGraph& g = *sg.graph();
+    for (NodeId n : sg.nodes())
+        if (g.get(n).op.kind == ir::OpKind::Conv) return conv_problem(sg, n);
     NodeId mm = ir::kNoNode;
     for (NodeId n : sg.nodes())
         if (g.get(n).op.kind == ir::OpKind::Matmul) {

@@ -17,6 +17,7 @@ UNARY = ["recip", "neg", "exp", "sin", "cos", "tan", "sigmoid", "tanh", "relu", 
 BINARY = ["add", "mul", "pow", "min", "max", "and", "or", "xor"]
 REDUCE = ["sum", "mean", "max", "min"]
 COMPARE = ["eq", "ne", "lt", "le", "gt", "ge"]
+PADDING = ["same", "valid", "full"]
 PRECISION = ["f32_f32", "tf32_f32", "bf16_f32", "f16_f32", "f16_f16", "f8_f32", "f8_f16"]
 
 
@@ -25,7 +26,10 @@ class OpDesc(C.Structure):
                 ("precision", C.c_int32), ("target_type", C.c_int32), ("depth", C.c_uint32),
                 ("new_dim_count", C.c_int64), ("broadcast_axes", C.POINTER(C.c_int64)),
                 ("num_broadcast_axes", C.c_int32), ("shape", C.POINTER(C.c_int64)), ("shape_rank", C.c_int32),
-                ("axis_a", C.c_int64), ("axis_b", C.c_int64), ("const_bits", C.c_uint32), ("const_dtype", C.c_int32)]
+                ("axis_a", C.c_int64), ("axis_b", C.c_int64), ("const_bits", C.c_uint32), ("const_dtype", C.c_int32),
+                ("conv_in_channels", C.c_int64), ("conv_out_channels", C.c_int64), ("conv_kernel", C.c_int64 * 2),
+                ("conv_stride", C.c_int64 * 2), ("conv_dilation", C.c_int64 * 2), ("conv_padding_mode", C.c_int32),
+                ("conv_input_size", C.c_int64 * 2)]
 
 
 _ffi._sig("he_graph_create", C.POINTER(C.c_void_p))
@@ -137,6 +141,25 @@ class OpGraph:
     def select(self, lhs, rhs, selector):
         """lhs where the selector is false, rhs where it is true (op.rs:439-445)."""
         return self._op("select", [lhs, rhs, selector], {})
+
+    def _conv_fields(self, params, input_size=(0, 0)):
+        """params: dict with in_channels, out_channels, kernel_size, stride, dilation, padding_mode (Conv2dParams)."""
+        two = C.c_int64 * 2
+        return dict(conv_in_channels=params["in_channels"], conv_out_channels=params["out_channels"],
+                    conv_kernel=two(*params["kernel_size"]), conv_stride=two(*params.get("stride", (1, 1))),
+                    conv_dilation=two(*params.get("dilation", (1, 1))),
+                    conv_padding_mode=PADDING.index(params.get("padding_mode", "same")), conv_input_size=two(*input_size))
+
+    def conv(self, image, filter_, params):
+        """Op::Conv: NHWC image, [out_channels, kh, kw, in_channels] filter (op.rs:447-452)."""
+        return self._op("conv", [image, filter_], {"params": dict(params)}, **self._conv_fields(params))
+
+    def conv_backward_data(self, flow, filter_, params, input_size):
+        return self._op("conv_bwd_data", [flow, filter_], {"params": dict(params), "input_size": list(input_size)},
+                        **self._conv_fields(params, input_size))
+
+    def conv_backward_filter(self, flow, image, params):
+        return self._op("conv_bwd_filter", [flow, image], {"params": dict(params)}, **self._conv_fields(params))
 
     def constant(self, value, dtype, shape):
         return self._op("constant", [], {"value": value, "const_dtype": dtype}, shape=list(shape),

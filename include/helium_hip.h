@@ -179,7 +179,15 @@ typedef struct he_op_desc {
     int64_t axis_a, axis_b; /* SwapDims */
     uint32_t const_bits;    /* Constant: the scalar's bit pattern in const_dtype */
     int32_t const_dtype;
+    /* Conv (inputs image, filter), ConvBackwardData (flow, filter), ConvBackwardFilter (flow, image): Conv2dParams
+     * (opgraph/op/conv.rs:5-12); images are NHWC, filters [out_channels, kh, kw, in_channels] (op.rs:123-173) */
+    int64_t conv_in_channels, conv_out_channels;
+    int64_t conv_kernel[2], conv_stride[2], conv_dilation[2];
+    int32_t conv_padding_mode;     /* HE_PAD_* */
+    int64_t conv_input_size[2];    /* ConvBackwardData::input_size */
 } he_op_desc;
+/* PaddingMode (conv.rs:76-81) */
+enum { HE_PAD_SAME = 0, HE_PAD_VALID = 1, HE_PAD_FULL = 2 };
 
 int he_graph_create(he_graph_t* graph);                                       /* OpGraph::new (opgraph.rs:21-23) */
 int he_graph_destroy(he_graph_t graph);

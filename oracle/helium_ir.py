@@ -6,7 +6,7 @@ to the storage type) and helium/src/raw_tensor.rs (front-end lowerings, in `lowe
 
 Pinned by tests/golden/tensor_ops.json (helium/tests/tensor_ops.rs: add/mul/div/recip/scalar ops, op chain = 0.4,
 reduce sum/mean/max/min incl. 200k elements, broadcast, reshape, swaps, relu, constant, max/min, matmul small
-cases) and by closed forms in tests/test_oracle.py. Transcendentals (`expf`, `tanhf`, `powf`, ...) are evaluated
+cases, conv_simple) and by closed forms in tests/test_oracle.py. Transcendentals (`expf`, `tanhf`, `powf`, ...) are evaluated
 in float64 and rounded once to float32; the reference uses CUDA libdevice for them, whose last-bit behaviour is
 "parity unpinned" beyond the exact-answer cases.
 
@@ -54,7 +54,62 @@ def infer(node, desc):
         return list(s0), "bool"
     if op == "constant":
         return list(node["shape"]), node["const_dtype"]
+    if op == "conv":  # op.rs:123-142
+        image, filt = desc[ins[0]][0], desc[ins[1]][0]
+        out = conv_output_size(node["params"], image[1:3], filt[1:3])
+        return [image[0], out[0], out[1], node["params"]["out_channels"]], t0
     raise ValueError(op)
+
+
+def conv_output_size(params, input_size, kernel_size):
+    """Conv2dParams::compute_output_size (helium-ir/src/opgraph/op/conv.rs:51-73): Full adds kernel/2, Valid
+    subtracts kernel/2 (saturating), then the stride divides."""
+    mode = params.get("padding_mode", "same")
+    stride = params.get("stride", (1, 1))
+    out = []
+    for d in range(2):
+        v = input_size[d]
+        if mode == "full":
+            v += kernel_size[d] // 2
+        elif mode == "valid":
+            v = max(0, v - kernel_size[d] // 2)
+        out.append(v // stride[d])
+    return out
+
+
+def conv_padding(params):
+    """PaddingMode::compute_padding_amount (conv.rs:85-91)."""
+    k = params["kernel_size"]
+    mode = params.get("padding_mode", "same")
+    return [k[0] // 2, k[1] // 2] if mode == "same" else [0, 0] if mode == "valid" else [k[0] - 1, k[1] - 1]
+
+
+def conv(image, filt, params, dtype):
+    """Cross-correlation of an NHWC image with a [out_channels, kh, kw, in_channels] filter, zero padding of
+    `conv_padding` on both sides, stride and dilation as given (the descriptor helium/src/cuda/instr/
+    cudnn_graph.rs:384-396 builds: CUDNN_CROSS_CORRELATION, pre = post padding, f32 compute). Output element
+    (n, p, q, o) = sum over (r, s, c) of image[n, p*sh + r*dh - ph, q*sw + s*dw - pw, c] * filter[o, r, s, c], taps
+    outside the image contributing zero; evaluated in float64 on the stored operand values."""
+    n, h, w, c = image.shape
+    o, kr, ks, _ = filt.shape
+    sh, sw = params.get("stride", (1, 1))
+    dh, dw = params.get("dilation", (1, 1))
+    ph, pw = conv_padding(params)
+    oh, ow = conv_output_size(params, (h, w), (kr, ks))
+    x = image.astype(np.float64)
+    f = filt.astype(np.float64)
+    out = np.zeros((n, oh, ow, o), dtype=np.float64)
+    for r in range(kr):
+        for s in range(ks):
+            # rows / columns of the output whose tap (r, s) falls inside the image
+            ih = np.arange(oh) * sh + r * dh - ph
+            iw = np.arange(ow) * sw + s * dw - pw
+            vh, vw = (ih >= 0) & (ih < h), (iw >= 0) & (iw < w)
+            if not vh.any() or not vw.any():
+                continue
+            patch = x[:, ih[vh]][:, :, iw[vw]]  # [n, oh', ow', c]
+            out[np.ix_(np.arange(n), np.nonzero(vh)[0], np.nonzero(vw)[0], np.arange(o))] += np.einsum("nhwc,oc->nhwo", patch, f[:, r, s, :])
+    return out.astype(np.float32)
 
 
 def _f64(fn, x):
@@ -228,6 +283,8 @@ def _eval_op(n, desc, val):
         return np.ascontiguousarray(np.broadcast_to(math.reshape([1] * len(n["shape"])), n["shape"]))
     if op == "matmul":
         return matmul(val[ins[0]], val[ins[1]], n["precision"], desc[ins[0]][1], desc[ins[1]][1])
+    if op == "conv":
+        return conv(val[ins[0]], val[ins[1]], n["params"], desc[ins[0]][1])
     raise ValueError(op)
 
 

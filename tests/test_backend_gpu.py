@@ -222,3 +222,31 @@ def test_batch_norm_train_step(gpu, fold):
         # sqrt(variance), so one bf16 step of y (2^-8 relative) plus the statistics' error
         tol = 2e-2 if desc[o][1] == "bf16" else 1e-3
         assert np.allclose(a, b, rtol=tol, atol=tol), (o, np.abs(a - b).max())
+
+
+@pytest.mark.parametrize("image,oc,kernel,stride,mode,dtype", [
+    ((4, 28, 28, 64), 64, (3, 3), (1, 1), "same", "bf16"),     # a resnet block convolution
+    ((2, 30, 30, 64), 128, (3, 3), (2, 2), "same", "bf16"),    # the strided first convolution of a stage
+    ((2, 30, 30, 64), 128, (1, 1), (2, 2), "same", "bf16"),    # its 1x1 shortcut
+    ((2, 33, 31, 3), 32, (7, 7), (2, 2), "same", "bf16"),      # three-channel input
+    ((1, 17, 19, 16), 24, (3, 3), (1, 1), "valid", "f32"),
+])
+def test_convolution_runs_as_an_implicit_gemm(gpu, image, oc, kernel, stride, mode, dtype):
+    """Op::Conv (NHWC image, [out, kh, kw, in] filter) through execute_graph: one GEMM instruction whose A operand
+    is gathered from the image; parity against the oracle's direct cross-correlation in float64."""
+    rng = np.random.default_rng(9)
+    g = ha.ir.OpGraph()
+    fshape = [oc, kernel[0], kernel[1], image[3]]
+    x = g.new_input(list(image), dtype); w = g.new_input(fshape, dtype)
+    y = g.conv(x, w, {"in_channels": image[3], "out_channels": oc, "kernel_size": list(kernel), "stride": list(stride),
+                      "padding_mode": mode})
+    out = g.new_output(g.unary(y, "relu"))
+    host = {x: nm.to_storage(rng.uniform(-1, 1, image).astype(np.float32), dtype),
+            w: nm.to_storage((rng.uniform(-1, 1, fshape) * 0.2).astype(np.float32), dtype)}
+    got, steps = run_graph(g, host)
+    assert [k for instrs, _ in steps for k, _ in instrs] == ["gemm", "pointwise"], steps
+    want = oracle_ir.plan_outputs(g.nodes, host, steps)[out]
+    a = nm.from_storage(got[out], dtype, [got[out].size]).astype(np.float64)
+    b = nm.from_storage(want.reshape(-1), dtype, [want.size]).astype(np.float64)
+    tol = 1e-4 if dtype == "f32" else 1e-2
+    assert (np.abs(a - b) <= tol * np.maximum(np.abs(b), 1.0)).all(), float(np.abs(a - b).max())

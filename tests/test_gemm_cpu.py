@@ -193,3 +193,57 @@ def test_ir_matmul_with_row_sums_on_cpu():
     want_y = nm.from_storage(nm.to_storage(val[y], desc[y][1]), desc[y][1], val[y].shape).astype(np.float64).reshape(-1)
     assert np.abs(got[y] - want_y).max() <= 2e-2 * np.abs(want_y).max(), k.description
     assert np.abs(got[r] - val[r].reshape(-1)).max() <= 1e-3 * np.abs(val[r]).max()
+
+
+# ---- Op::Conv as an implicit GEMM ---------------------------------------------------------------------------
+def conv_case(image_shape, out_channels, kernel, dtype="bf16", stride=(1, 1), dilation=(1, 1), mode="same", seed=8):
+    rng = np.random.default_rng(seed)
+    g = ha.ir.OpGraph()
+    filter_shape = [out_channels, kernel[0], kernel[1], image_shape[3]]
+    x = g.new_input(list(image_shape), dtype); w = g.new_input(filter_shape, dtype)
+    params = {"in_channels": image_shape[3], "out_channels": out_channels, "kernel_size": list(kernel),
+              "stride": list(stride), "dilation": list(dilation), "padding_mode": mode}
+    y = g.conv(x, w, params)
+    g.new_output(y)
+    inputs = {x: nm.to_storage(rng.uniform(-1, 1, image_shape).astype(np.float32), dtype),
+              w: nm.to_storage((rng.uniform(-1, 1, filter_shape) * 0.25).astype(np.float32), dtype)}
+    return g, y, inputs
+
+
+def test_conv_reference_known_answer_on_cpu():
+    """conv_simple (helium/tests/tensor_ops.rs:379-397): 1x1 kernel over two channels."""
+    g = ha.ir.OpGraph()
+    x = g.new_input([1, 1, 1, 2], "f32"); w = g.new_input([2, 1, 1, 2], "f32")
+    y = g.conv(x, w, {"in_channels": 2, "out_channels": 2, "kernel_size": [1, 1]})
+    g.new_output(y)
+    assert g.descriptor(y) == ([1, 1, 1, 2], "f32")
+    inputs = {x: np.array([1.0, 2.0], np.float32), w: np.array([10.0, 20.0, 30.0, 40.0], np.float32)}
+    _, got = run_ir_kernel_on_cpu(g, [y], inputs)
+    assert got[y].tolist() == [50.0, 110.0]
+
+
+CONV_CASES = [
+    # name, image NHWC, out channels, kernel, dtype, stride, dilation, padding mode, tile
+    ("3x3_same_bf16", (2, 9, 10, 16), 24, (3, 3), "bf16", (1, 1), (1, 1), "same", "128,128,64,2,2"),
+    ("3x3_stride2_bf16", (1, 12, 12, 8), 32, (3, 3), "bf16", (2, 2), (1, 1), "same", "64,64,64,2,2"),
+    ("1x1_stride2_shortcut", (2, 8, 8, 32), 64, (1, 1), "bf16", (2, 2), (1, 1), "same", "128,128,64,2,2"),
+    ("three_channel_image_7x7", (1, 10, 9, 3), 16, (7, 7), "bf16", (2, 2), (1, 1), "same", "128,128,64,2,2"),
+    ("valid_and_dilated_f32", (1, 9, 9, 4), 8, (3, 3), "f32", (1, 1), (2, 1), "valid", "64,64,32,2,2"),
+    ("full_padding_f16", (1, 6, 7, 8), 8, (3, 2), "f16", (1, 1), (1, 1), "full", "128,128,64,2,2"),
+]
+
+
+@pytest.mark.parametrize("name,image,oc,kernel,dtype,stride,dilation,mode,tile", CONV_CASES, ids=[c[0] for c in CONV_CASES])
+def test_conv_on_cpu(name, image, oc, kernel, dtype, stride, dilation, mode, tile):
+    from oracle import helium_ir as oracle_ir
+
+    g, y, inputs = conv_case(image, oc, kernel, dtype, stride, dilation, mode)
+    os.environ["HELIUM_HIP_GEMM_TILE"] = tile
+    try:
+        k, got = run_ir_kernel_on_cpu(g, [y], inputs)
+    finally:
+        del os.environ["HELIUM_HIP_GEMM_TILE"]
+    want = oracle_ir.kernel_outputs(g.nodes, inputs, [y])[y]
+    want = nm.from_storage(want.reshape(-1), dtype, [want.size]).astype(np.float64)
+    tol = 1e-4 if dtype == "f32" else 2e-2
+    assert np.abs(got[y] - want).max() <= tol * max(1.0, np.abs(want).max()), (k.description, np.abs(got[y] - want).max())
