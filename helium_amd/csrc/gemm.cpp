@@ -105,7 +105,15 @@ typedef f32x4 bfrag_t;
 typedef s16x8 afrag_t;
 typedef s16x8 bfrag_t;
 #endif
-struct WavePos { u32 lane, wave, wave_m, wave_n; };
+struct WavePos {
+    u32 lane, wave, wave_m, wave_n;
+    u32 m0;           /* first row of the workgroup's tile (the gather of a convolution needs absolute rows) */
+    const void* img;  /* CONV_A: the image the A operand is gathered from */
+};
+#if CONV_A
+// Where the taps that fall outside the image (or the matrix) are read from by the direct global->LDS loads.
+__device__ __attribute__((aligned(16))) const u32 conv_zeros[4] = {0u, 0u, 0u, 0u};
+#endif
 #if MMA_F32
 typedef float mul_t;   /* multiplicand as stored in global memory */
 #else
@@ -255,7 +263,15 @@ __device__ __forceinline__ void direct_issue(unsigned char* __restrict__ st, con
         const u32 blk = wave * A_DPW + i;
         const u32 row = blk * (64 / A_CHUNKS) + lane / A_CHUNKS, pc = lane % A_CHUNKS;
         const u32 kc = pc ^ ((row >> A_SWZ_SHIFT) & (A_CHUNKS - 1));
+#if CONV_A
+        // `ga` carries the tile's first k as an element offset from null: every lane computes the address of its
+        // own chunk of 8 (4) channels of one filter tap, or points at zeros when the tap is outside the image
+        size_t at;
+        const bool inside = conv_tap(w.m0 + row, (u32)(ga - (const mul_t*)nullptr) + kc * EPC, at);
+        const mul_t* gp = inside ? (const mul_t*)w.img + at : (const mul_t*)conv_zeros;
+#else
         const mul_t* gp = ga + (size_t)row * GK + kc * EPC;
+#endif
         __builtin_amdgcn_global_load_lds((GLOBAL_AS const void*)gp, (LDS_AS void*)(st + blk * 1024), 16, 0, 0);
     } else {
         const u32 blk = wave * B_DPW + (i - A_DPW);
@@ -396,12 +412,20 @@ void fused_matmul(KERNEL_PARAMS) {
         }
 #endif
     };
-    const WavePos wpos = {lane, wave, wave_m, wave_n};
+#if CONV_A
+    const WavePos wpos = {lane, wave, wave_m, wave_n, m0, (const void*)CONV_IMG};
+#else
+    const WavePos wpos = {lane, wave, wave_m, wave_n, m0, nullptr};
+#endif
 
 /* s_waitcnt immediate: vmcnt lives in bits [3:0] and [15:14] */
 #define WAITCNT_VM(n) ((((n) & 15) | (((n) >> 4) << 14)))
 #if DIRECT_LOADS
+#if CONV_A
+    const mul_t* const ga0 = (const mul_t*)nullptr;  // direct_issue reads the k offset back from it
+#else
     const mul_t* const ga0 = (const mul_t*)DIRECT_A_PTR + ((size_t)bz * GM + m0) * GK;
+#endif
 #if B_NK
     const mul_t* const gb0 = (const mul_t*)DIRECT_B_PTR + ((size_t)bz * GN + n0) * GK;
 #define B_TILE_AT(k) (gb0 + (k))
@@ -695,7 +719,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     const int nva = std::min(epc, tp::pick_nv(pr.op_a, 16)), nvb = std::min(epc, tp::pick_nv(pr.op_b, 16));
     // Direct global->LDS loads need unpredicated, unmodified 16-byte chunks: raw operands and full tiles everywhere.
     // Each operand qualifies on its own; the other one then goes through registers.
-    const bool direct_a = want_direct && !pr.conv_a.on && raw_a && pr.M % t.bm == 0 && pr.K % t.bk == 0 && (t.bm * t.bk * esz / 1024) % (threads / 64) == 0 &&
+    const bool direct_a = want_direct && raw_a && (pr.conv_a.on ? pr.conv_a.C % epc == 0 : pr.M % t.bm == 0 && pr.K % t.bk == 0) && (t.bm * t.bk * esz / 1024) % (threads / 64) == 0 &&
                           !getenv("HELIUM_HIP_GEMM_NO_DIRECT_A");
     const bool direct_b = want_direct && raw_b && pr.N % t.bn == 0 && pr.K % t.bk == 0 && (t.bk * t.bn * esz / 1024) % (threads / 64) == 0 &&
                           (pr.b_nk || 64 % (t.bn / epc) == 0) && !getenv("HELIUM_HIP_GEMM_NO_DIRECT_B");
@@ -725,7 +749,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
       << "\n#define GEMM_SKIP " << (getenv("HELIUM_HIP_GEMM_SKIP") ? atoi(getenv("HELIUM_HIP_GEMM_SKIP")) : 0)
       << "\n#define GEMM_TIMING " << (getenv("HELIUM_HIP_GEMM_TIMING") ? 1 : 0) << "\n#define GEMM_TIMING_PTR p" << (pr.args.size() - 1)
       << "\n#define DIRECT_A " << (direct_a ? 1 : 0) << "\n#define DIRECT_B " << (direct_b ? 1 : 0)
-      << "\n#define B_NK " << (pr.b_nk ? 1 : 0) << "\n#define DIRECT_LOADS (DIRECT_A || DIRECT_B)\n#define STAGED (!DIRECT_A || !DIRECT_B)"
+      << "\n#define B_NK " << (pr.b_nk ? 1 : 0) << "\n#define CONV_A " << (pr.conv_a.on ? 1 : 0) << "\n#define CONV_IMG p" << (pr.conv_a.on ? pr.map_a[0] : 0) << "\n#define DIRECT_LOADS (DIRECT_A || DIRECT_B)\n#define STAGED (!DIRECT_A || !DIRECT_B)"
       << "\n#define DIRECT_A_PTR p" << (direct_a ? pr.map_a[0] : 0)
       << "\n#define DIRECT_B_PTR p" << (direct_b ? pr.map_b[0] : 0) << "\n#define STAGE_SCHED_BARRIER "
       << ((getenv("HELIUM_HIP_GEMM_PIN") ? atoi(getenv("HELIUM_HIP_GEMM_PIN")) != 0 : true) ? "__builtin_amdgcn_sched_barrier(0);" : "") << "\n#define A_SWZ_SHIFT " << (getenv("HELIUM_HIP_GEMM_ASWZ") ? atoi(getenv("HELIUM_HIP_GEMM_ASWZ")) : (t.bk == 64 ? 1 : 2)) << "\n";
