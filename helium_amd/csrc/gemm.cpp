@@ -107,8 +107,9 @@ typedef s16x8 bfrag_t;
 #endif
 struct WavePos {
     u32 lane, wave, wave_m, wave_n;
-    u32 m0;           /* first row of the workgroup's tile (the gather of a convolution needs absolute rows) */
+    u32 m0, n0;       /* first row / column of the workgroup's tile (gathers need absolute coordinates) */
     const void* img;  /* CONV_A: the image the A operand is gathered from */
+    const void* bsrc; /* B_ROW_GATHER: the tensor B's rows are picked from */
 };
 #if CONV_A
 // Where the taps that fall outside the image (or the matrix) are read from by the direct global->LDS loads.
@@ -282,7 +283,12 @@ __device__ __forceinline__ void direct_issue(unsigned char* __restrict__ st, con
 #else
         const u32 krow = blk * (64 / B_CHUNKS) + lane / B_CHUNKS, pc = lane % B_CHUNKS;
         const u32 nc = pc ^ B_SWZ(krow);
+#if B_ROW_GATHER
+        // `gb` carries the tile's first k as an element offset from null; row k of B starts at b_row_addr(k)
+        const mul_t* gp = (const mul_t*)w.bsrc + b_row_addr((u32)(gb - (const mul_t*)nullptr) + krow) + w.n0 + nc * EPC;
+#else
         const mul_t* gp = gb + (size_t)krow * GN + nc * EPC;
+#endif
 #endif
         __builtin_amdgcn_global_load_lds((GLOBAL_AS const void*)gp, (LDS_AS void*)(st + A_TILE_BYTES + blk * 1024), 16, 0, 0);
     }
@@ -412,11 +418,7 @@ void fused_matmul(KERNEL_PARAMS) {
         }
 #endif
     };
-#if CONV_A
-    const WavePos wpos = {lane, wave, wave_m, wave_n, m0, (const void*)CONV_IMG};
-#else
-    const WavePos wpos = {lane, wave, wave_m, wave_n, m0, nullptr};
-#endif
+    const WavePos wpos = {lane, wave, wave_m, wave_n, m0, n0, (const void*)CONV_IMG_OR_NULL, (const void*)B_SRC_OR_NULL};
 
 /* s_waitcnt immediate: vmcnt lives in bits [3:0] and [15:14] */
 #define WAITCNT_VM(n) ((((n) & 15) | (((n) >> 4) << 14)))
@@ -428,6 +430,9 @@ void fused_matmul(KERNEL_PARAMS) {
 #endif
 #if B_NK
     const mul_t* const gb0 = (const mul_t*)DIRECT_B_PTR + ((size_t)bz * GN + n0) * GK;
+#define B_TILE_AT(k) (gb0 + (k))
+#elif B_ROW_GATHER
+    const mul_t* const gb0 = (const mul_t*)nullptr;  // direct_issue reads the k offset back from it
 #define B_TILE_AT(k) (gb0 + (k))
 #else
     const mul_t* const gb0 = (const mul_t*)DIRECT_B_PTR + (size_t)bz * GK * GN + n0;
@@ -678,7 +683,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     Tile t;
     bool small = false;
     const bool raw_a0 = pr.conv_a.on || (is_raw_copy(pr.op_a, pr.root_a, pr.mma_dtype) && pr.K % epc == 0);
-    const bool raw_b0 = is_raw_copy(pr.op_b, pr.root_b, pr.mma_dtype) && (pr.b_nk ? pr.K : pr.N) % epc == 0;
+    const bool raw_b0 = pr.b_rows.on ? pr.N % epc == 0 : is_raw_copy(pr.op_b, pr.root_b, pr.mma_dtype) && (pr.b_nk ? pr.K : pr.N) % epc == 0;
     const bool want_direct = !getenv("HELIUM_HIP_GEMM_NO_DIRECT");
     const int esz = 16 / epc;  // bytes per multiplicand
     if (const char* env = getenv("HELIUM_HIP_GEMM_TILE")) {
@@ -749,7 +754,9 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
       << "\n#define GEMM_SKIP " << (getenv("HELIUM_HIP_GEMM_SKIP") ? atoi(getenv("HELIUM_HIP_GEMM_SKIP")) : 0)
       << "\n#define GEMM_TIMING " << (getenv("HELIUM_HIP_GEMM_TIMING") ? 1 : 0) << "\n#define GEMM_TIMING_PTR p" << (pr.args.size() - 1)
       << "\n#define DIRECT_A " << (direct_a ? 1 : 0) << "\n#define DIRECT_B " << (direct_b ? 1 : 0)
-      << "\n#define B_NK " << (pr.b_nk ? 1 : 0) << "\n#define CONV_A " << (pr.conv_a.on ? 1 : 0) << "\n#define CONV_IMG p" << (pr.conv_a.on ? pr.map_a[0] : 0) << "\n#define DIRECT_LOADS (DIRECT_A || DIRECT_B)\n#define STAGED (!DIRECT_A || !DIRECT_B)"
+      << "\n#define B_NK " << (pr.b_nk ? 1 : 0) << "\n#define CONV_A " << (pr.conv_a.on ? 1 : 0) << "\n#define CONV_IMG p" << (pr.conv_a.on ? pr.map_a[0] : 0)
+      << "\n#define CONV_IMG_OR_NULL " << (pr.conv_a.on ? "p" + std::to_string(pr.map_a[0]) : std::string("nullptr"))
+      << "\n#define B_ROW_GATHER " << (pr.b_rows.on ? 1 : 0) << "\n#define B_SRC_OR_NULL " << (pr.b_rows.on ? "p" + std::to_string(pr.map_b[0]) : std::string("nullptr")) << "\n#define DIRECT_LOADS (DIRECT_A || DIRECT_B)\n#define STAGED (!DIRECT_A || !DIRECT_B)"
       << "\n#define DIRECT_A_PTR p" << (direct_a ? pr.map_a[0] : 0)
       << "\n#define DIRECT_B_PTR p" << (direct_b ? pr.map_b[0] : 0) << "\n#define STAGE_SCHED_BARRIER "
       << ((getenv("HELIUM_HIP_GEMM_PIN") ? atoi(getenv("HELIUM_HIP_GEMM_PIN")) != 0 : true) ? "__builtin_amdgcn_sched_barrier(0);" : "") << "\n#define A_SWZ_SHIFT " << (getenv("HELIUM_HIP_GEMM_ASWZ") ? atoi(getenv("HELIUM_HIP_GEMM_ASWZ")) : (t.bk == 64 ? 1 : 2)) << "\n";
@@ -808,9 +815,16 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         s << "__device__ __forceinline__ bool conv_tap(u32 row, u32 col, size_t& at) {\n"
           << "const u32 n = row / " << cv.P * cv.Q << "u, pq = row % " << cv.P * cv.Q << "u, p = pq / " << cv.Q << "u, q = pq % " << cv.Q << "u;\n"
           << "const u32 rs = col / " << cv.C << "u, c = col % " << cv.C << "u, r = rs / " << cv.S << "u, sx = rs % " << cv.S << "u;\n"
-          << "const int ih = (int)(p * " << cv.sh << "u + r * " << cv.dh << "u) - " << cv.ph << ", iw = (int)(q * " << cv.sw << "u + sx * " << cv.dw << "u) - " << cv.pw << ";\n"
-          << "at = (((size_t)n * " << cv.H << "u + (u32)ih) * " << cv.W << "u + (u32)iw) * " << cv.C << "u + c;\n"
-          << "return row < GM && col < GK && ih >= 0 && ih < " << cv.H << " && iw >= 0 && iw < " << cv.W << ";\n}\n";
+          ;
+        if (!cv.bwd)
+            s << "const int ih = (int)(p * " << cv.sh << "u + r * " << cv.dh << "u) - " << cv.ph << ", iw = (int)(q * " << cv.sw << "u + sx * " << cv.dw << "u) - " << cv.pw << ";\n"
+              << "const bool hit = true;\n";
+        else
+            s << "const int th = (int)p + " << cv.ph << " - (int)(r * " << cv.dh << "u), tw = (int)q + " << cv.pw << " - (int)(sx * " << cv.dw << "u);\n"
+              << "const bool hit = th >= 0 && tw >= 0 && th % " << cv.sh << " == 0 && tw % " << cv.sw << " == 0;\n"
+              << "const int ih = th / " << cv.sh << ", iw = tw / " << cv.sw << ";\n";
+        s << "at = (((size_t)n * " << cv.H << "u + (u32)ih) * " << cv.W << "u + (u32)iw) * " << cv.C << "u + c;\n"
+          << "return row < GM && col < GK && hit && ih >= 0 && ih < " << cv.H << " && iw >= 0 && iw < " << cv.W << ";\n}\n";
         s << "__device__ __forceinline__ u32x4 fetch_a(const " << tp::c_type(img.dtype) << "* __restrict__ q0, u32 b, u32 row, u32 col) {\n(void)b;\n";
         if (cv.C % epc == 0) {
             s << "u32x4 v = {0u, 0u, 0u, 0u};\nsize_t at;\nif (conv_tap(row, col, at)) v = *(const u32x4*)(q0 + at);\nreturn v;\n}\n";
@@ -821,7 +835,14 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     } else {
         emit_fetch("a", pr.op_a, pr.root_a, pr.map_a, raw_a, nva, "GM", "GK", pr.M % t.bm == 0 && pr.K % t.bk == 0);
     }
-    if (pr.b_nk) emit_fetch("b", pr.op_b, pr.root_b, pr.map_b, raw_b, nvb, "GN", "GK", pr.K % t.bk == 0 && pr.N % t.bn == 0);
+    if (pr.b_rows.on) {
+        const auto& br = pr.b_rows;
+        s << "__device__ __forceinline__ size_t b_row_addr(u32 k) { return (size_t)(k % " << br.group << "u) * " << br.o_stride << "ull + (size_t)(k / "
+          << br.group << "u) * " << br.rs_stride << "ull; }\n";
+        s << "#define FETCH_B_ARGS p" << pr.map_b[0] << ", \n#define RAW_B 1\n#define SPLIT_B 1\n";
+        s << "__device__ __forceinline__ u32x4 fetch_b(const " << tp::c_type(pr.op_b.args[0].dtype) << "* __restrict__ q0, u32 b, u32 row, u32 col) {\n(void)b;\n"
+          << "u32x4 v = {0u, 0u, 0u, 0u};\nif (row < GK && col < GN) v = *(const u32x4*)(q0 + b_row_addr(row) + col);\nreturn v;\n}\n";
+    } else if (pr.b_nk) emit_fetch("b", pr.op_b, pr.root_b, pr.map_b, raw_b, nvb, "GN", "GK", pr.K % t.bk == 0 && pr.N % t.bn == 0);
     else emit_fetch("b", pr.op_b, pr.root_b, pr.map_b, raw_b, nvb, "GK", "GN", pr.K % t.bk == 0 && pr.N % t.bn == 0);
 
     // epilogue pieces

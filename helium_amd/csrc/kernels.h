@@ -75,10 +75,19 @@ struct GemmProblem {
     // Implicit-GEMM convolution: the A operand is never materialised. Row m of A is output pixel (n, p, q), column k
     // is filter tap (r, s, c); the element is image[n][p*sh + r*dh - ph][q*sw + s*dw - pw][c], or zero outside the
     // image. op_a then only names the image argument.
+    // `bwd` (ConvBackwardData): rows are input pixels (n, p, q) of the gradient being computed, the gathered tensor
+    // is the incoming flow [N, H, W, C] (C = output channels of the forward op), and tap (r, s) of row (p, q) reads
+    // flow[n][(p + ph - r*dh) / sh][(q + pw - s*dw) / sw][c] where both divisions are exact and in range.
     struct ConvGather {
-        bool on = false;
+        bool on = false, bwd = false;
         int64_t N = 0, H = 0, W = 0, C = 0, R = 0, S = 0, P = 0, Q = 0, sh = 1, sw = 1, dh = 1, dw = 1, ph = 0, pw = 0;
     } conv_a;
+    // B rows that are not consecutive in memory: row k = rs * group + o lives at element o * o_stride + rs * rs_stride
+    // (the filter [o][r][s][c] seen as the [(r, s, o)][c] matrix of ConvBackwardData). Columns stay contiguous.
+    struct RowGather {
+        bool on = false;
+        int64_t group = 1, o_stride = 0, rs_stride = 0;
+    } b_rows;
     int root_a = -1, root_b = -1;  // expression ids of the operand values in op_a / op_b
     std::vector<tp::Arg> args;     // the kernel's arguments: inputs in node order, then outputs in node order
     std::vector<int> map_a, map_b, map_e;  // program argument -> kernel argument

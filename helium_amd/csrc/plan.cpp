@@ -132,8 +132,9 @@ Instr make_instr_for_op(const std::shared_ptr<const ir::OpGraph>& g, NodeId node
         case ir::OpKind::Matmul: return Instr(InstrKind::Gemm, sg);
         // The reference hands convolutions to cuDNN (cuda.rs:55-58, cudnn_graph.rs:193-204); here the forward
         // convolution is the fused GEMM with an implicit im2col gather as its A operand.
-        case ir::OpKind::Conv: return Instr(InstrKind::Gemm, sg);
-        default: fail(HE_ERR_UNSUPPORTED, "the convolution backward ops have no instruction in this backend");
+        case ir::OpKind::Conv:
+        case ir::OpKind::ConvBackwardData: return Instr(InstrKind::Gemm, sg);
+        default: fail(HE_ERR_UNSUPPORTED, "ConvBackwardFilter has no instruction in this backend");
     }
 }
 
@@ -534,10 +535,85 @@ GemmProblem conv_problem(const ir::OpSubgraph& sg, NodeId conv) {
 }
 }  // namespace
 
+namespace {
+// Op::ConvBackwardData as a GEMM: rows = pixels (n, h, w) of the image gradient, columns = input channels,
+// k = (r, s, o). A is gathered from the flow (the gradient of the forward output): tap (r, s) of pixel (h, w) reads
+// flow[n][(h + ph - r*dh) / sh][(w + pw - s*dw) / sw][o] where that pixel exists; B's row (r, s, o) is the filter's
+// [o][r][s][:] row of input channels, picked out of the [out, kh, kw, in] tensor where it lies.
+GemmProblem conv_backward_data_problem(const ir::OpSubgraph& sg, NodeId node) {
+    const ir::OpGraph& g = *sg.graph();
+    HE_REQUIRE(sg.nodes().size() == 1, HE_ERR_UNSUPPORTED, "a convolution instruction holds the op alone");
+    const ir::Op& op = g.get(node).op;
+    const ir::Descriptor &flow = g.get(op.inputs[0]).desc, &filter = g.get(op.inputs[1]).desc, &out = g.get(node).desc;
+    HE_REQUIRE(flow.shape.size() == 4 && filter.shape.size() == 4, HE_ERR_INVALID, "conv backward takes rank-4 tensors");
+    HE_REQUIRE(dtype_class(flow.dtype) == DataClass::Float && filter.dtype == flow.dtype, HE_ERR_UNSUPPORTED,
+               "conv backward takes a float flow and a filter of the same type");
+    HE_REQUIRE(filter.shape[0] == op.conv.out_channels && filter.shape[3] == op.conv.in_channels && flow.shape[3] == op.conv.out_channels &&
+                   filter.shape[1] == op.conv.kernel[0] && filter.shape[2] == op.conv.kernel[1],
+               HE_ERR_INVALID, "conv backward filter / flow shapes do not match the parameters");
+    GemmProblem pr;
+    auto& cv = pr.conv_a;
+    cv.on = cv.bwd = true;
+    cv.N = flow.shape[0]; cv.H = flow.shape[1]; cv.W = flow.shape[2]; cv.C = flow.shape[3];
+    cv.R = filter.shape[1]; cv.S = filter.shape[2];
+    cv.P = out.shape[1]; cv.Q = out.shape[2];
+    cv.sh = op.conv.stride[0]; cv.sw = op.conv.stride[1];
+    cv.dh = op.conv.dilation[0]; cv.dw = op.conv.dilation[1];
+    int64_t pad[2];
+    op.conv.padding(pad);
+    cv.ph = pad[0]; cv.pw = pad[1];
+    const int64_t in_channels = op.conv.in_channels;
+    pr.batch = 1;
+    pr.M = cv.N * cv.P * cv.Q;
+    pr.N = in_channels;
+    pr.K = cv.R * cv.S * cv.C;
+    HE_REQUIRE(pr.M > 0 && pr.M < (1ll << 31) && ir::num_elements(flow.shape) < (1ll << 32), HE_ERR_UNSUPPORTED, "conv too large for 32-bit tile indices");
+    pr.mma_dtype = flow.dtype == HE_F32 ? HE_F32 : flow.dtype == HE_F16 ? HE_F16 : HE_BF16;
+    HE_REQUIRE(in_channels % (pr.mma_dtype == HE_F32 ? 4 : 8) == 0, HE_ERR_UNSUPPORTED,
+               "conv backward data needs an input-channel count that fills 16-byte chunks");
+    pr.b_rows.on = true;
+    pr.b_rows.group = cv.C;                                 // k = (r*S + s) * out_channels + o
+    pr.b_rows.o_stride = cv.R * cv.S * in_channels;         // filter[o][..]
+    pr.b_rows.rs_stride = in_channels;                      // filter[.][r][s][..]
+    auto operand = [&](tp::Program& p, const ir::Descriptor& d, NodeId n, int64_t rows, int64_t cols) {
+        p.dims = {1, rows, cols};
+        p.args.push_back({d.dtype, ir::num_elements(d.shape), false, n});
+        tp::Expr e;
+        e.kind = tp::Expr::Load;
+        e.cls = tp::Cls::F;
+        e.access.arg = 0;
+        e.access.dtype = d.dtype;
+        e.access.stride = ir::packed_strides(p.dims);
+        p.exprs.push_back(e);
+    };
+    operand(pr.op_a, flow, op.inputs[0], pr.M, pr.K);    // stand-ins: only the arguments are used
+    operand(pr.op_b, filter, op.inputs[1], pr.K, pr.N);
+    pr.root_a = pr.root_b = 0;
+    pr.epi.dims = {1, pr.M, pr.N};
+    pr.epi.fast_math = true;
+    tp::Expr acc;
+    acc.kind = tp::Expr::Acc;
+    acc.cls = tp::Cls::F;
+    pr.epi.exprs.push_back(acc);
+    pr.epi.acc_expr = 0;
+    tp::Out o;
+    o.expr = 0;
+    o.arg = 0;
+    o.dtype = out.dtype;
+    pr.epi.outs.push_back(o);
+    pr.epi.args.push_back({out.dtype, ir::num_elements(out.shape), true, node});
+    validate_gemm_epilogue(pr.epi);
+    assemble_gemm_args(pr);
+    return pr;
+}
+}  // namespace
+
 GemmProblem gemm_problem_from_ir(const ir::OpSubgraph& sg) {
     const ir::OpGraph& g = *sg.graph();
-    for (NodeId n : sg.nodes())
+    for (NodeId n : sg.nodes()) {
         if (g.get(n).op.kind == ir::OpKind::Conv) return conv_problem(sg, n);
+        if (g.get(n).op.kind == ir::OpKind::ConvBackwardData) return conv_backward_data_problem(sg, n);
+    }
     NodeId mm = ir::kNoNode;
     for (NodeId n : sg.nodes())
         if (g.get(n).op.kind == ir::OpKind::Matmul) {

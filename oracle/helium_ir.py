@@ -58,6 +58,8 @@ def infer(node, desc):
         image, filt = desc[ins[0]][0], desc[ins[1]][0]
         out = conv_output_size(node["params"], image[1:3], filt[1:3])
         return [image[0], out[0], out[1], node["params"]["out_channels"]], t0
+    if op == "conv_bwd_data":  # op.rs:143-158
+        return [s0[0], node["input_size"][0], node["input_size"][1], node["params"]["in_channels"]], t0
     raise ValueError(op)
 
 
@@ -285,7 +287,35 @@ def _eval_op(n, desc, val):
         return matmul(val[ins[0]], val[ins[1]], n["precision"], desc[ins[0]][1], desc[ins[1]][1])
     if op == "conv":
         return conv(val[ins[0]], val[ins[1]], n["params"], desc[ins[0]][1])
+    if op == "conv_bwd_data":
+        return conv_backward_data(val[ins[0]], val[ins[1]], n["params"], n["input_size"])
     raise ValueError(op)
+
+
+def conv_backward_data(flow, filt, params, input_size):
+    """Gradient of `conv` with respect to its image (what cuDNN's CONVOLUTION_BACKWARD_DATA computes for the
+    descriptor of cudnn_graph.rs:205-216,384-396): the adjoint of the forward map, so every product
+    flow[n,p,q,o] * filter[o,r,s,c] lands on the image pixel (p*sh + r*dh - ph, q*sw + s*dw - pw) the forward op
+    read for it, if that pixel exists. Evaluated in float64."""
+    n, oh, ow, o = flow.shape
+    _, kr, ks, c = filt.shape
+    h, w = input_size
+    sh, sw = params.get("stride", (1, 1))
+    dh, dw = params.get("dilation", (1, 1))
+    ph, pw = conv_padding(params)
+    dy = flow.astype(np.float64)
+    f = filt.astype(np.float64)
+    out = np.zeros((n, h, w, c), dtype=np.float64)
+    for r in range(kr):
+        for s in range(ks):
+            ih = np.arange(oh) * sh + r * dh - ph
+            iw = np.arange(ow) * sw + s * dw - pw
+            vh, vw = (ih >= 0) & (ih < h), (iw >= 0) & (iw < w)
+            if not vh.any() or not vw.any():
+                continue
+            contrib = np.einsum("nhwo,oc->nhwc", dy[:, vh][:, :, vw], f[:, r, s, :])
+            out[np.ix_(np.arange(n), ih[vh], iw[vw], np.arange(c))] += contrib
+    return out.astype(np.float32)
 
 
 def kernel_outputs(nodes, inputs, leaf_ids):

@@ -247,3 +247,43 @@ def test_conv_on_cpu(name, image, oc, kernel, dtype, stride, dilation, mode, til
     want = nm.from_storage(want.reshape(-1), dtype, [want.size]).astype(np.float64)
     tol = 1e-4 if dtype == "f32" else 2e-2
     assert np.abs(got[y] - want).max() <= tol * max(1.0, np.abs(want).max()), (k.description, np.abs(got[y] - want).max())
+
+
+BWD_DATA_CASES = [
+    # name, image NHWC (the tensor whose gradient is computed), out channels, kernel, dtype, stride, dilation, mode, tile
+    ("3x3_same_bf16", (2, 9, 10, 16), 24, (3, 3), "bf16", (1, 1), (1, 1), "same", "128,128,64,2,2"),
+    ("3x3_stride2_bf16", (1, 12, 12, 8), 32, (3, 3), "bf16", (2, 2), (1, 1), "same", "64,64,64,2,2"),
+    ("1x1_stride2_shortcut", (2, 8, 8, 32), 64, (1, 1), "bf16", (2, 2), (1, 1), "same", "128,128,64,2,2"),
+    ("direct_loads_both_operands", (1, 16, 16, 128), 64, (3, 3), "bf16", (1, 1), (1, 1), "same", "128,128,64,2,2"),
+    ("valid_and_dilated_f32", (1, 9, 9, 4), 8, (3, 3), "f32", (1, 1), (2, 1), "valid", "64,64,32,2,2"),
+]
+
+
+@pytest.mark.parametrize("name,image,oc,kernel,dtype,stride,dilation,mode,tile", BWD_DATA_CASES, ids=[c[0] for c in BWD_DATA_CASES])
+def test_conv_backward_data_on_cpu(name, image, oc, kernel, dtype, stride, dilation, mode, tile):
+    """Op::ConvBackwardData as an implicit GEMM: the flow gathered as A (with the stride's divisibility test), the
+    filter's rows picked as B. The oracle is the adjoint of the forward convolution."""
+    from oracle import helium_ir as oracle_ir
+
+    rng = np.random.default_rng(10)
+    params = {"in_channels": image[3], "out_channels": oc, "kernel_size": list(kernel), "stride": list(stride),
+              "dilation": list(dilation), "padding_mode": mode}
+    out_hw = oracle_ir.conv_output_size(params, image[1:3], kernel)
+    flow_shape = [image[0], out_hw[0], out_hw[1], oc]
+    filter_shape = [oc, kernel[0], kernel[1], image[3]]
+    g = ha.ir.OpGraph()
+    dy = g.new_input(flow_shape, dtype); w = g.new_input(filter_shape, dtype)
+    dx = g.conv_backward_data(dy, w, params, image[1:3])
+    g.new_output(dx)
+    assert g.descriptor(dx) == (list(image), dtype)
+    inputs = {dy: nm.to_storage(rng.uniform(-1, 1, flow_shape).astype(np.float32), dtype),
+              w: nm.to_storage((rng.uniform(-1, 1, filter_shape) * 0.25).astype(np.float32), dtype)}
+    os.environ["HELIUM_HIP_GEMM_TILE"] = tile
+    try:
+        k, got = run_ir_kernel_on_cpu(g, [dx], inputs)
+    finally:
+        del os.environ["HELIUM_HIP_GEMM_TILE"]
+    want = oracle_ir.kernel_outputs(g.nodes, inputs, [dx])[dx]
+    want = nm.from_storage(want.reshape(-1), dtype, [want.size]).astype(np.float64)
+    tol = 1e-4 if dtype == "f32" else 2e-2
+    assert np.abs(got[dx] - want).max() <= tol * max(1.0, np.abs(want).max()), (k.description, np.abs(got[dx] - want).max())
