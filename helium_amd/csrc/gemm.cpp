@@ -95,6 +95,12 @@ __device__ __forceinline__ u32 a_off(u32 m, u32 kc) { return m * (BK * ESZ) + ((
 #define B_SWZ(k) (MMA_F32 ? 0u : (((k) & 3) << 2) & (B_CHUNKS - 1))
 __device__ __forceinline__ u32 b_chunk_off(u32 k, u32 nc) { return k * (BN * ESZ) + ((nc ^ B_SWZ(k)) << 4); }
 __device__ __forceinline__ u32 b_off(u32 k, u32 n) { return b_chunk_off(k, (n * ESZ) >> 4) + ((n * ESZ) & 15); }
+// A_KM: A arrives with m contiguous ([k][m] in memory, a transposed matrix). Its tile is then [k][m] in LDS, staged and
+// read like a [k][n] B tile: 16-byte chunks along m, transposing reads for the 16-bit fragments.
+#define AKM_CHUNKS (BM / EPC)
+#define AKM_SWZ(k) (MMA_F32 ? 0u : (((k) & 3) << 2) & (AKM_CHUNKS - 1))
+__device__ __forceinline__ u32 akm_chunk_off(u32 k, u32 mc) { return k * (BM * ESZ) + ((mc ^ AKM_SWZ(k)) << 4); }
+__device__ __forceinline__ u32 akm_off(u32 k, u32 m) { return akm_chunk_off(k, (m * ESZ) >> 4) + ((m * ESZ) & 15); }
 // B_NK: B arrives with k contiguous ([n][k] in memory). Its tile is then [n][k] in LDS too, staged and read like
 // A's: the MFMA wants 8 consecutive k of one n per lane, which is one 16-byte chunk of row n.
 
@@ -135,7 +141,12 @@ __device__ __forceinline__ void load_frags(const unsigned char* __restrict__ st,
 #pragma unroll
     for (int i = 0; i < MB; i++) {
         const u32 row = w.wave_m * WTM + i * 32 + (lane & 31);
+#if A_KM
+#pragma unroll
+        for (int e = 0; e < 4; e++) af[i][e] = *(const float*)(la + akm_off(kk * 8 + (lane >> 5) * 4 + e, row));
+#else
         af[i] = *(const f32x4*)(la + a_off(row, kk * 2 + (lane >> 5)));
+#endif
     }
 #pragma unroll
     for (int j = 0; j < NB; j++) {
@@ -149,11 +160,22 @@ __device__ __forceinline__ void load_frags(const unsigned char* __restrict__ st,
     }
 #else
     const u32 grp = lane >> 4, sub = lane & 15;
+#if A_KM
+#pragma unroll
+    for (int i = 0; i < MB; i++) {
+        const u32 k = kk * 16 + (grp >> 1) * 8 + (sub >> 2);
+        const u32 m = w.wave_m * WTM + i * 32 + (grp & 1) * 16 + (sub & 3) * 4;
+        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(la + akm_off(k, m)));
+        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(la + akm_off(k + 4, m)));
+        af[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+#else
 #pragma unroll
     for (int i = 0; i < MB; i++) {
         const u32 row = w.wave_m * WTM + i * 32 + (lane & 31);
         af[i] = *(const s16x8*)(la + a_off(row, kk * 2 + (lane >> 5)));
     }
+#endif
 #if B_NK
     (void)grp; (void)sub;
 #pragma unroll
@@ -262,6 +284,13 @@ __device__ __forceinline__ void direct_issue(unsigned char* __restrict__ st, con
     const u32 lane = w.lane, wave = w.wave;
     if (i < A_DPW) {
         const u32 blk = wave * A_DPW + i;
+#if A_KM
+        const u32 krow = blk * (64 / AKM_CHUNKS) + lane / AKM_CHUNKS, pcm = lane % AKM_CHUNKS;
+        const u32 mc = pcm ^ AKM_SWZ(krow);
+        const mul_t* gpm = ga + (size_t)krow * GM + mc * EPC;
+        __builtin_amdgcn_global_load_lds((GLOBAL_AS const void*)gpm, (LDS_AS void*)(st + blk * 1024), 16, 0, 0);
+        return;
+#endif
         const u32 row = blk * (64 / A_CHUNKS) + lane / A_CHUNKS, pc = lane % A_CHUNKS;
         const u32 kc = pc ^ ((row >> A_SWZ_SHIFT) & (A_CHUNKS - 1));
 #if CONV_A
@@ -356,11 +385,15 @@ void fused_matmul(KERNEL_PARAMS) {
 #pragma unroll
         for (int i = 0; i < A_PER_THREAD; i++) {
             const u32 idx = tid + i * NTHREADS;
-            const u32 row = idx / A_CHUNKS, kc = idx % A_CHUNKS;
-#if RAW_A
-            sa[i] = fetch_a(FETCH_A_ARGS bz, m0 + row, k0 + kc * EPC);
+#if A_KM
+            const u32 arow = k0 + idx / AKM_CHUNKS, acol = m0 + (idx % AKM_CHUNKS) * EPC;
 #else
-            fetch_a_load(FETCH_A_ARGS bz, m0 + row, k0 + kc * EPC, sa[i]);
+            const u32 arow = m0 + idx / A_CHUNKS, acol = k0 + (idx % A_CHUNKS) * EPC;
+#endif
+#if RAW_A
+            sa[i] = fetch_a(FETCH_A_ARGS bz, arow, acol);
+#else
+            fetch_a_load(FETCH_A_ARGS bz, arow, acol, sa[i]);
 #endif
         }
 #endif
@@ -390,11 +423,18 @@ void fused_matmul(KERNEL_PARAMS) {
 #pragma unroll
         for (int i = 0; i < A_PER_THREAD; i++) {
             const u32 idx = tid + i * NTHREADS;
-            const u32 row = idx / A_CHUNKS, kc = idx % A_CHUNKS;
-#if RAW_A
-            *(u32x4*)(la + a_off(row, kc)) = sa[i];
+#if A_KM
+            const u32 aslot = akm_chunk_off(idx / AKM_CHUNKS, idx % AKM_CHUNKS);
+            const u32 arow = k0 + idx / AKM_CHUNKS, acol = m0 + (idx % AKM_CHUNKS) * EPC;
 #else
-            *(u32x4*)(la + a_off(row, kc)) = fetch_a_eval(FETCH_A_ARGS bz, m0 + row, k0 + kc * EPC, sa[i]);
+            const u32 aslot = a_off(idx / A_CHUNKS, idx % A_CHUNKS);
+            const u32 arow = m0 + idx / A_CHUNKS, acol = k0 + (idx % A_CHUNKS) * EPC;
+#endif
+            (void)arow; (void)acol;
+#if RAW_A
+            *(u32x4*)(la + aslot) = sa[i];
+#else
+            *(u32x4*)(la + aslot) = fetch_a_eval(FETCH_A_ARGS bz, arow, acol, sa[i]);
 #endif
         }
 #endif
@@ -425,8 +465,13 @@ void fused_matmul(KERNEL_PARAMS) {
 #if DIRECT_LOADS
 #if CONV_A
     const mul_t* const ga0 = (const mul_t*)nullptr;  // direct_issue reads the k offset back from it
+#define A_TILE_AT(k) (ga0 + (k))
+#elif A_KM
+    const mul_t* const ga0 = (const mul_t*)DIRECT_A_PTR + (size_t)bz * GK * GM + m0;
+#define A_TILE_AT(k) (ga0 + (size_t)(k) * GM)
 #else
     const mul_t* const ga0 = (const mul_t*)DIRECT_A_PTR + ((size_t)bz * GM + m0) * GK;
+#define A_TILE_AT(k) (ga0 + (k))
 #endif
 #if B_NK
     const mul_t* const gb0 = (const mul_t*)DIRECT_B_PTR + ((size_t)bz * GN + n0) * GK;
@@ -445,7 +490,7 @@ void fused_matmul(KERNEL_PARAMS) {
         if (st < KT) {
 #pragma unroll
             for (int i = 0; i < A_DPW + B_DPW; i++)
-                direct_issue(lds + st * STAGE_BYTES, ga0 + k_tile(st) * BK, B_TILE_AT(k_tile(st) * BK), wpos, i);
+                direct_issue(lds + st * STAGE_BYTES, A_TILE_AT(k_tile(st) * BK), B_TILE_AT(k_tile(st) * BK), wpos, i);
         }
 #endif
 #if STAGED
@@ -492,7 +537,7 @@ void fused_matmul(KERNEL_PARAMS) {
 #endif
 #if DIRECT_LOADS
         const u32 knext = more ? k_tile(next) * BK : 0u;
-        direct_tile(lds + (kt % NSTAGES) * STAGE_BYTES, lds + (next % NSTAGES) * STAGE_BYTES, ga0 + knext,
+        direct_tile(lds + (kt % NSTAGES) * STAGE_BYTES, lds + (next % NSTAGES) * STAGE_BYTES, A_TILE_AT(knext),
                     B_TILE_AT(knext), more, acc, wpos, frags);
 #else
         compute_tile(lds + (kt % NSTAGES) * STAGE_BYTES, acc, wpos, frags, [](int) {});
@@ -596,6 +641,11 @@ GemmProblem gemm_problem_from_fusion(const fir::OpGraph& g) {
     pr.N = sc[2];
     pr.K = sa[2];
     pr.op_a = tp::lower_operand(g, mm.a, &pr.root_a);
+    if (operand_b_prefers_nk(pr.op_a) && !getenv("HELIUM_HIP_GEMM_NO_KM")) {
+        // the same test on A's [batch, M, K] program asks whether A's source is contiguous along m
+        pr.op_a = tp::lower_operand(g, mm.a, &pr.root_a, true);
+        pr.a_km = true;
+    }
     pr.op_b = tp::lower_operand(g, mm.b, &pr.root_b);
     if (operand_b_prefers_nk(pr.op_b) && !getenv("HELIUM_HIP_GEMM_NO_NK")) {
         pr.op_b = tp::lower_operand(g, mm.b, &pr.root_b, true);
@@ -682,7 +732,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     const int epc = f32 ? 4 : 8;  // multiplicands per 16-byte chunk
     Tile t;
     bool small = false;
-    const bool raw_a0 = pr.conv_a.on || (is_raw_copy(pr.op_a, pr.root_a, pr.mma_dtype) && pr.K % epc == 0);
+    const bool raw_a0 = pr.conv_a.on || (is_raw_copy(pr.op_a, pr.root_a, pr.mma_dtype) && (pr.a_km ? pr.M : pr.K) % epc == 0);
     const bool raw_b0 = pr.b_rows.on ? pr.N % epc == 0 : is_raw_copy(pr.op_b, pr.root_b, pr.mma_dtype) && (pr.b_nk ? pr.K : pr.N) % epc == 0;
     const bool want_direct = !getenv("HELIUM_HIP_GEMM_NO_DIRECT");
     const int esz = 16 / epc;  // bytes per multiplicand
@@ -724,7 +774,8 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     const int nva = std::min(epc, tp::pick_nv(pr.op_a, 16)), nvb = std::min(epc, tp::pick_nv(pr.op_b, 16));
     // Direct global->LDS loads need unpredicated, unmodified 16-byte chunks: raw operands and full tiles everywhere.
     // Each operand qualifies on its own; the other one then goes through registers.
-    const bool direct_a = want_direct && raw_a && (pr.conv_a.on ? pr.conv_a.C % epc == 0 : pr.M % t.bm == 0 && pr.K % t.bk == 0) && (t.bm * t.bk * esz / 1024) % (threads / 64) == 0 &&
+    const bool direct_a = want_direct && raw_a && (pr.conv_a.on ? pr.conv_a.C % epc == 0 : pr.M % t.bm == 0 && pr.K % t.bk == 0) &&
+                          (!pr.a_km || 64 % (t.bm / epc) == 0) && (t.bm * t.bk * esz / 1024) % (threads / 64) == 0 &&
                           !getenv("HELIUM_HIP_GEMM_NO_DIRECT_A");
     const bool direct_b = want_direct && raw_b && pr.N % t.bn == 0 && pr.K % t.bk == 0 && (t.bk * t.bn * esz / 1024) % (threads / 64) == 0 &&
                           (pr.b_nk || 64 % (t.bn / epc) == 0) && !getenv("HELIUM_HIP_GEMM_NO_DIRECT_B");
@@ -754,7 +805,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
       << "\n#define GEMM_SKIP " << (getenv("HELIUM_HIP_GEMM_SKIP") ? atoi(getenv("HELIUM_HIP_GEMM_SKIP")) : 0)
       << "\n#define GEMM_TIMING " << (getenv("HELIUM_HIP_GEMM_TIMING") ? 1 : 0) << "\n#define GEMM_TIMING_PTR p" << (pr.args.size() - 1)
       << "\n#define DIRECT_A " << (direct_a ? 1 : 0) << "\n#define DIRECT_B " << (direct_b ? 1 : 0)
-      << "\n#define B_NK " << (pr.b_nk ? 1 : 0) << "\n#define CONV_A " << (pr.conv_a.on ? 1 : 0) << "\n#define CONV_IMG p" << (pr.conv_a.on ? pr.map_a[0] : 0)
+      << "\n#define A_KM " << (pr.a_km ? 1 : 0) << "\n#define B_NK " << (pr.b_nk ? 1 : 0) << "\n#define CONV_A " << (pr.conv_a.on ? 1 : 0) << "\n#define CONV_IMG p" << (pr.conv_a.on ? pr.map_a[0] : 0)
       << "\n#define CONV_IMG_OR_NULL " << (pr.conv_a.on ? "p" + std::to_string(pr.map_a[0]) : std::string("nullptr"))
       << "\n#define B_ROW_GATHER " << (pr.b_rows.on ? 1 : 0) << "\n#define B_SRC_OR_NULL " << (pr.b_rows.on ? "p" + std::to_string(pr.map_b[0]) : std::string("nullptr")) << "\n#define DIRECT_LOADS (DIRECT_A || DIRECT_B)\n#define STAGED (!DIRECT_A || !DIRECT_B)"
       << "\n#define DIRECT_A_PTR p" << (direct_a ? pr.map_a[0] : 0)
@@ -832,6 +883,8 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
             s << "float v[" << epc << "];\n#pragma unroll\nfor (int j = 0; j < " << epc << "; j++) {\nsize_t at;\nv[j] = conv_tap(row, col + j, at) ? ld_one(q0 + at) : 0.0f;\n}\n"
               << "return pack_chunk(v);\n}\n";
         }
+    } else if (pr.a_km) {
+        emit_fetch("a", pr.op_a, pr.root_a, pr.map_a, raw_a, nva, "GK", "GM", pr.M % t.bm == 0 && pr.K % t.bk == 0);
     } else {
         emit_fetch("a", pr.op_a, pr.root_a, pr.map_a, raw_a, nva, "GM", "GK", pr.M % t.bm == 0 && pr.K % t.bk == 0);
     }

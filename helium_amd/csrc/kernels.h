@@ -72,6 +72,9 @@ struct GemmProblem {
     // B's source is contiguous along k (a transposed matrix, a convolution filter): its program iterates [batch,N,K],
     // its tile is staged and read like A's, with 16-byte chunks along k.
     bool b_nk = false;
+    // A's source is contiguous along m (a transposed matrix): its program iterates [batch,K,M], its tile is staged
+    // and read like a [k][n] B tile, with 16-byte chunks along m.
+    bool a_km = false;
     // Implicit-GEMM convolution: the A operand is never materialised. Row m of A is output pixel (n, p, q), column k
     // is filter tap (r, s, c); the element is image[n][p*sh + r*dh - ph][q*sw + s*dw - pw][c], or zero outside the
     // image. op_a then only names the image argument.

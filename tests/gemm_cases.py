@@ -45,6 +45,21 @@ def transposed_b(m, n, k, batch=1, seed=4, dtype="bf16", out_dtype="f32", scale=
     return g, inputs, [out]
 
 
+def transposed_a(m, n, k, batch=1, seed=5, dtype="bf16", out_dtype="f32", scale=0.5, both=False):
+    """C = At^T * B with At stored [batch, k, m] (m contiguous); `both`: B is stored transposed as well."""
+    g = ha.fusion.OpGraph()
+    rng = np.random.default_rng(seed)
+    bshape = (batch, n, k) if both else (batch, k, n)
+    at = g.producer([batch, k, m], dtype); b = g.producer(list(bshape), dtype)
+    if dtype == "bf16":
+        inputs = {at: bf16_normal(rng, (batch, k, m), scale), b: bf16_normal(rng, bshape, scale)}
+    else:
+        inputs = {at: (rng.standard_normal((batch, k, m)) * scale).astype(np.float32),
+                  b: (rng.standard_normal(bshape) * scale).astype(np.float32)}
+    out = g.consumer(g.matmul(g.transpose(at), g.transpose(b) if both else b), out_dtype)
+    return g, inputs, [out]
+
+
 def linear_layer(m, k, n):
     """Config 1 at a small size: f32 Y = relu(X W + b) and its column sums."""
     from helium_amd import configs

@@ -82,6 +82,11 @@ CASES = [
     ("nt_mainloop_scaled_rows_of_bt", lambda: gemm_cases.transposed_b(128, 128, 128, scaled=True), "128,128,64,2,2"),
     ("nt_f32_operands", lambda: gemm_cases.transposed_b(64, 96, 64, dtype="f32"), "64,64,32,2,2,3"),
     ("nt_eight_waves_256", lambda: gemm_cases.transposed_b(256, 256, 128), "256,256,64,2,4"),
+    ("tn_direct_both_operands", lambda: gemm_cases.transposed_a(128, 256, 192), "128,128,64,2,2"),
+    ("tn_ragged_staged", lambda: gemm_cases.transposed_a(70, 100, 88, batch=2), "128,128,64,2,2"),
+    ("tt_both_transposed", lambda: gemm_cases.transposed_a(128, 128, 128, both=True), "128,128,64,2,2"),
+    ("tn_f32_operands", lambda: gemm_cases.transposed_a(64, 96, 64, dtype="f32"), "64,64,32,2,2,3"),
+    ("tn_eight_waves_256", lambda: gemm_cases.transposed_a(256, 256, 128), "256,256,64,2,4"),
     ("one_wave_32x32_f32_direct", lambda: gemm_cases.plain(64, 96, 128, dtype="f32"), "32,32,32,1,1,4"),
     ("two_waves_64x32_linear_layer", lambda: gemm_cases.linear_layer(48, 40, 72), "64,32,32,2,1,4"),
 ]
@@ -92,7 +97,7 @@ def test_fused_gemm_on_cpu(name, build, tile):
     g, inputs, outs = build()
     k, got = run_emulated(g, inputs, tile, env=("HELIUM_HIP_GEMM_EPIPIPE",) if "prefetched" in name else ())
     assert sorted(got) == sorted(outs), k.description
-    f32_cases = ("f32_operands", "f32_linear_layer", "one_wave_32x32_f32_direct", "two_waves_64x32_linear_layer", "nt_f32_operands")
+    f32_cases = ("f32_operands", "f32_linear_layer", "one_wave_32x32_f32_direct", "two_waves_64x32_linear_layer", "nt_f32_operands", "tn_f32_operands")
     rounding = "f16" if name == "f16_operands" else None if name in f32_cases else "bf16"
     want = oracle.outputs(g.nodes, inputs, round_mainloop_to=rounding)
     if rounding is None:

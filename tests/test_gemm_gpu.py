@@ -145,3 +145,17 @@ def test_b_operand_stored_transposed(gpu, m, n, k, batch, scaled):
 def test_b_operand_stored_transposed_f32(gpu):
     g, inputs, outs = gemm_cases.transposed_b(192, 200, 136, dtype="f32")
     check(g, inputs, outs, mma=None, rel=1e-4, eps=1e-5)
+
+
+@pytest.mark.parametrize("m,n,k,batch,both", [(256, 256, 128, 1, False), (512, 768, 320, 1, False), (100, 100, 100, 2, False),
+                                              (257, 263, 129, 1, True), (1024, 1024, 1024, 1, True), (4096, 4096, 512, 1, False)])
+def test_a_operand_stored_transposed(gpu, m, n, k, batch, both):
+    """C = At^T * B with At stored [k][m]: the A tile is staged and read like a [k][n] B tile (chunks along m,
+    transposing LDS reads); with `both`, B is stored [n][k] as well (the TT product)."""
+    g, inputs, outs = gemm_cases.transposed_a(m, n, k, batch=batch, both=both)
+    check(g, inputs, outs)
+
+
+def test_a_operand_stored_transposed_f32(gpu):
+    g, inputs, outs = gemm_cases.transposed_a(192, 200, 136, dtype="f32")
+    check(g, inputs, outs, mma=None, rel=1e-4, eps=1e-5)
