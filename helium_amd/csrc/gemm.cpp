@@ -87,7 +87,8 @@ const char* kGemmBody = R"HIP(
 #if NSTAGES * STAGE_BYTES < NWAVES * 32 * EP * 4
 #error "the epilogue strip does not fit in the operand stages"
 #endif
-#define KT ((GK + BK - 1) / BK)
+#define KT_ALL ((GK + BK - 1) / BK)
+#define KT_PER_SPLIT ((KT_ALL + SPLIT_K - 1) / SPLIT_K)
 
 __device__ __forceinline__ u32 a_off(u32 m, u32 kc) { return m * (BK * ESZ) + ((kc ^ ((m >> A_SWZ_SHIFT) & (A_CHUNKS - 1))) << 4); }
 // B rows keep their memory order; the chunk index is XORed with 4 * (k % 4) for the transposing 16-bit reads
@@ -117,7 +118,7 @@ struct WavePos {
     const void* img;  /* CONV_A: the image the A operand is gathered from */
     const void* bsrc; /* B_ROW_GATHER: the tensor B's rows are picked from */
 };
-#if CONV_A
+#if CONV_A || CONV_B
 // Where the taps that fall outside the image (or the matrix) are read from by the direct global->LDS loads.
 __device__ __attribute__((aligned(16))) const u32 conv_zeros[4] = {0u, 0u, 0u, 0u};
 #endif
@@ -312,7 +313,13 @@ __device__ __forceinline__ void direct_issue(unsigned char* __restrict__ st, con
 #else
         const u32 krow = blk * (64 / B_CHUNKS) + lane / B_CHUNKS, pc = lane % B_CHUNKS;
         const u32 nc = pc ^ B_SWZ(krow);
-#if B_ROW_GATHER
+#if CONV_B
+        // `gb` carries the tile's first k (an output pixel index) as an element offset from null; the lane's chunk is
+        // 8 (4) channels of tap n of that pixel, or zeros when the tap is outside the image
+        size_t bat;
+        const bool binside = conv_tap((u32)(gb - (const mul_t*)nullptr) + krow, w.n0 + nc * EPC, bat);
+        const mul_t* gp = binside ? (const mul_t*)w.bsrc + bat : (const mul_t*)conv_zeros;
+#elif B_ROW_GATHER
         // `gb` carries the tile's first k as an element offset from null; row k of B starts at b_row_addr(k)
         const mul_t* gp = (const mul_t*)w.bsrc + b_row_addr((u32)(gb - (const mul_t*)nullptr) + krow) + w.n0 + nc * EPC;
 #else
@@ -347,12 +354,19 @@ void fused_matmul(KERNEL_PARAMS) {
     const u32 wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
     u32 tile_m, tile_n;
     TILE_ORDER
-    const u32 bz = blockIdx.y;
+#if SPLIT_K > 1
+    // blockIdx.y is the k-range index, not a batch index: this workgroup multiplies k-tiles [kt0, kt0 + KT)
+    const u32 bz = 0, split = blockIdx.y, kt0 = split * KT_PER_SPLIT;
+    const u32 KT = kt0 >= KT_ALL ? 0u : (KT_ALL - kt0 < KT_PER_SPLIT ? KT_ALL - kt0 : KT_PER_SPLIT);
+#else
+    const u32 bz = blockIdx.y, kt0 = 0;
+    constexpr u32 KT = KT_ALL;
+#endif
     const u32 m0 = tile_m * BM, n0 = tile_n * BN;
     // Optional rotation of the k loop per workgroup (tuning knob, off by default: workgroups that share an A or B
     // panel read the same k range at the same time, which is what lets them share it through L2).
-    const u32 k_shift = (STAGGER_EXPR) % KT;
-    auto k_tile = [&](u32 kt) { u32 x = kt + k_shift; return x >= KT ? x - KT : x; };
+    const u32 k_shift = KT ? (STAGGER_EXPR) % KT : 0u;
+    auto k_tile = [&](u32 kt) { u32 x = kt + k_shift; return kt0 + (x >= KT ? x - KT : x); };
 
     f32x16 acc[MB][NB];
 #pragma unroll
@@ -476,7 +490,7 @@ void fused_matmul(KERNEL_PARAMS) {
 #if B_NK
     const mul_t* const gb0 = (const mul_t*)DIRECT_B_PTR + ((size_t)bz * GN + n0) * GK;
 #define B_TILE_AT(k) (gb0 + (k))
-#elif B_ROW_GATHER
+#elif B_ROW_GATHER || CONV_B
     const mul_t* const gb0 = (const mul_t*)nullptr;  // direct_issue reads the k offset back from it
 #define B_TILE_AT(k) (gb0 + (k))
 #else
@@ -733,7 +747,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     Tile t;
     bool small = false;
     const bool raw_a0 = pr.conv_a.on || (is_raw_copy(pr.op_a, pr.root_a, pr.mma_dtype) && (pr.a_km ? pr.M : pr.K) % epc == 0);
-    const bool raw_b0 = pr.b_rows.on ? pr.N % epc == 0 : is_raw_copy(pr.op_b, pr.root_b, pr.mma_dtype) && (pr.b_nk ? pr.K : pr.N) % epc == 0;
+    const bool raw_b0 = pr.conv_b.on ? true : pr.b_rows.on ? pr.N % epc == 0 : is_raw_copy(pr.op_b, pr.root_b, pr.mma_dtype) && (pr.b_nk ? pr.K : pr.N) % epc == 0;
     const bool want_direct = !getenv("HELIUM_HIP_GEMM_NO_DIRECT");
     const int esz = 16 / epc;  // bytes per multiplicand
     if (const char* env = getenv("HELIUM_HIP_GEMM_TILE")) {
@@ -752,6 +766,12 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
             t.bn = 64;
             t.wm = 4;
             t.wn = 2;
+        } else if (!f32 && pr.M <= 64 && pr.M > 32 && pr.N >= 128) {
+            // few output rows (a filter gradient with 64 output channels): tiles as low as M
+            t.bm = 64;
+            t.bn = 128;
+            t.wm = t.wn = 2;
+            small = true;
         } else
         // Smaller problems take smaller tiles so that every CU gets work.
         if (pr.M <= 128 || pr.N <= 128 || ((pr.M + 255) / 256) * ((pr.N + 255) / 256) * pr.batch < 128) {
@@ -777,7 +797,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     const bool direct_a = want_direct && raw_a && (pr.conv_a.on ? pr.conv_a.C % epc == 0 : pr.M % t.bm == 0 && pr.K % t.bk == 0) &&
                           (!pr.a_km || 64 % (t.bm / epc) == 0) && (t.bm * t.bk * esz / 1024) % (threads / 64) == 0 &&
                           !getenv("HELIUM_HIP_GEMM_NO_DIRECT_A");
-    const bool direct_b = want_direct && raw_b && pr.N % t.bn == 0 && pr.K % t.bk == 0 && (t.bk * t.bn * esz / 1024) % (threads / 64) == 0 &&
+    const bool direct_b = want_direct && raw_b && (pr.conv_b.on || (pr.N % t.bn == 0 && pr.K % t.bk == 0)) && (t.bk * t.bn * esz / 1024) % (threads / 64) == 0 &&
                           (pr.b_nk || 64 % (t.bn / epc) == 0) && !getenv("HELIUM_HIP_GEMM_NO_DIRECT_B");
     if (!(direct_a && direct_b)) t.stages = 2;  // register staging is double-buffered only
     else if (!getenv("HELIUM_HIP_GEMM_TILE") && small) {
@@ -807,7 +827,8 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
       << "\n#define DIRECT_A " << (direct_a ? 1 : 0) << "\n#define DIRECT_B " << (direct_b ? 1 : 0)
       << "\n#define A_KM " << (pr.a_km ? 1 : 0) << "\n#define B_NK " << (pr.b_nk ? 1 : 0) << "\n#define CONV_A " << (pr.conv_a.on ? 1 : 0) << "\n#define CONV_IMG p" << (pr.conv_a.on ? pr.map_a[0] : 0)
       << "\n#define CONV_IMG_OR_NULL " << (pr.conv_a.on ? "p" + std::to_string(pr.map_a[0]) : std::string("nullptr"))
-      << "\n#define B_ROW_GATHER " << (pr.b_rows.on ? 1 : 0) << "\n#define B_SRC_OR_NULL " << (pr.b_rows.on ? "p" + std::to_string(pr.map_b[0]) : std::string("nullptr")) << "\n#define DIRECT_LOADS (DIRECT_A || DIRECT_B)\n#define STAGED (!DIRECT_A || !DIRECT_B)"
+      << "\n#define B_ROW_GATHER " << (pr.b_rows.on ? 1 : 0) << "\n#define CONV_B " << (pr.conv_b.on ? 1 : 0) << "\n#define SPLIT_K " << pr.split_k
+      << "\n#define B_SRC_OR_NULL " << (pr.b_rows.on || pr.conv_b.on ? "p" + std::to_string(pr.map_b[0]) : std::string("nullptr")) << "\n#define DIRECT_LOADS (DIRECT_A || DIRECT_B)\n#define STAGED (!DIRECT_A || !DIRECT_B)"
       << "\n#define DIRECT_A_PTR p" << (direct_a ? pr.map_a[0] : 0)
       << "\n#define DIRECT_B_PTR p" << (direct_b ? pr.map_b[0] : 0) << "\n#define STAGE_SCHED_BARRIER "
       << ((getenv("HELIUM_HIP_GEMM_PIN") ? atoi(getenv("HELIUM_HIP_GEMM_PIN")) != 0 : true) ? "__builtin_amdgcn_sched_barrier(0);" : "") << "\n#define A_SWZ_SHIFT " << (getenv("HELIUM_HIP_GEMM_ASWZ") ? atoi(getenv("HELIUM_HIP_GEMM_ASWZ")) : (t.bk == 64 ? 1 : 2)) << "\n";
@@ -818,6 +839,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         std::ostringstream ps;
         for (size_t a = 0; a < pr.args.size(); a++)
             ps << (a ? ", " : "") << (pr.args[a].is_output ? "" : "const ") << tp::c_type(pr.args[a].dtype) << "* __restrict__ p" << a;
+        if (pr.split_k > 1) ps << ", float* __restrict__ splitk_ws";
         s << "#define KERNEL_PARAMS " << ps.str() << "\n";
     }
     // operand fetchers
@@ -857,16 +879,12 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         else s << guard << "operand_" << W << "_eval(" << pass << "b, row, col + j, R[j / " << nv << "], v + j);\nelse {\n#pragma unroll\nfor (int k = 0; k < " << nv << "; k++) v[j + k] = 0.0f; }\n}\n";
         s << "return pack_chunk(v);\n}\n";
     };
-    if (pr.conv_a.on) {
-        // The gather of an implicit-GEMM convolution in place of A's loads: one 16-byte chunk is EPC consecutive
-        // channels of one filter tap when the channel count allows, EPC separate taps otherwise (a 3-channel image).
-        const auto& cv = pr.conv_a;
-        const tp::Arg& img = pr.op_a.args[0];
-        s << "#define FETCH_A_ARGS p" << pr.map_a[0] << ", \n#define RAW_A 1\n#define SPLIT_A 1\n";
+    auto emit_conv_tap = [&](const GemmProblem::ConvGather& cv) {
+        // (row, col) = (pixel (n, p, q), tap (r, s, c)) -> element offset in the gathered NHWC tensor; false when the
+        // tap lies outside it (or outside the matrix)
         s << "__device__ __forceinline__ bool conv_tap(u32 row, u32 col, size_t& at) {\n"
           << "const u32 n = row / " << cv.P * cv.Q << "u, pq = row % " << cv.P * cv.Q << "u, p = pq / " << cv.Q << "u, q = pq % " << cv.Q << "u;\n"
-          << "const u32 rs = col / " << cv.C << "u, c = col % " << cv.C << "u, r = rs / " << cv.S << "u, sx = rs % " << cv.S << "u;\n"
-          ;
+          << "const u32 rs = col / " << cv.C << "u, c = col % " << cv.C << "u, r = rs / " << cv.S << "u, sx = rs % " << cv.S << "u;\n";
         if (!cv.bwd)
             s << "const int ih = (int)(p * " << cv.sh << "u + r * " << cv.dh << "u) - " << cv.ph << ", iw = (int)(q * " << cv.sw << "u + sx * " << cv.dw << "u) - " << cv.pw << ";\n"
               << "const bool hit = true;\n";
@@ -875,7 +893,15 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
               << "const bool hit = th >= 0 && tw >= 0 && th % " << cv.sh << " == 0 && tw % " << cv.sw << " == 0;\n"
               << "const int ih = th / " << cv.sh << ", iw = tw / " << cv.sw << ";\n";
         s << "at = (((size_t)n * " << cv.H << "u + (u32)ih) * " << cv.W << "u + (u32)iw) * " << cv.C << "u + c;\n"
-          << "return row < GM && col < GK && hit && ih >= 0 && ih < " << cv.H << " && iw >= 0 && iw < " << cv.W << ";\n}\n";
+          << "return row < " << cv.N * cv.P * cv.Q << "u && col < " << cv.R * cv.S * cv.C << "u && hit && ih >= 0 && ih < " << cv.H << " && iw >= 0 && iw < " << cv.W << ";\n}\n";
+    };
+    if (pr.conv_a.on) {
+        // The gather of an implicit-GEMM convolution in place of A's loads: one 16-byte chunk is EPC consecutive
+        // channels of one filter tap when the channel count allows, EPC separate taps otherwise (a 3-channel image).
+        const auto& cv = pr.conv_a;
+        const tp::Arg& img = pr.op_a.args[0];
+        s << "#define FETCH_A_ARGS p" << pr.map_a[0] << ", \n#define RAW_A 1\n#define SPLIT_A 1\n";
+        emit_conv_tap(cv);
         s << "__device__ __forceinline__ u32x4 fetch_a(const " << tp::c_type(img.dtype) << "* __restrict__ q0, u32 b, u32 row, u32 col) {\n(void)b;\n";
         if (cv.C % epc == 0) {
             s << "u32x4 v = {0u, 0u, 0u, 0u};\nsize_t at;\nif (conv_tap(row, col, at)) v = *(const u32x4*)(q0 + at);\nreturn v;\n}\n";
@@ -888,7 +914,12 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     } else {
         emit_fetch("a", pr.op_a, pr.root_a, pr.map_a, raw_a, nva, "GM", "GK", pr.M % t.bm == 0 && pr.K % t.bk == 0);
     }
-    if (pr.b_rows.on) {
+    if (pr.conv_b.on) {
+        emit_conv_tap(pr.conv_b);
+        s << "#define FETCH_B_ARGS p" << pr.map_b[0] << ", \n#define RAW_B 1\n#define SPLIT_B 1\n";
+        s << "__device__ __forceinline__ u32x4 fetch_b(const " << tp::c_type(pr.op_b.args[0].dtype) << "* __restrict__ q0, u32 b, u32 row, u32 col) {\n(void)b;\n"
+          << "u32x4 v = {0u, 0u, 0u, 0u};\nsize_t at;\nif (conv_tap(row, col, at)) v = *(const u32x4*)(q0 + at);\nreturn v;\n}\n";
+    } else if (pr.b_rows.on) {
         const auto& br = pr.b_rows;
         s << "__device__ __forceinline__ size_t b_row_addr(u32 k) { return (size_t)(k % " << br.group << "u) * " << br.o_stride << "ull + (size_t)(k / "
           << br.group << "u) * " << br.rs_stride << "ull; }\n";
@@ -942,6 +973,10 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         // body: runs once per (row, NVE columns) of the strip
         for (size_t oi = 0; oi < pr.epi.outs.size(); oi++)
             if (pr.epi.outs[oi].reduce && pr.epi.outs[oi].fold_n && !pr.epi.outs[oi].fold_m) body << "float rr" << oi << " = 0.0f;\n";
+        if (pr.split_k > 1) {
+            // the partial tile of this k range, as f32, for the second launch to add up
+            body << "if (ok) {\nfloat* dst = splitk_ws + ((size_t)split * GM + m) * GN + nn;\n#pragma unroll\nfor (int k = 0; k < NVE; k++) if (nn + k < GN) dst[k] = acc_v[k];\n}\n";
+        } else {
         body << "if (ok) {\nconst u32 n0 = nn; (void)n0;\nfloat (&acc)[NVE] = acc_v;\n";
         tp::EmitCtx cx;
         cx.nv = nve;
@@ -973,6 +1008,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
             const int width = std::min(lanes_per_row, 64);
             body << "{ float r = wave_reduce<0, " << width << ">(rr" << oi << ");\nif ((lane % " << width
                  << ") == 0 && m < GM && nn < GN) atomicAdd(a" << o.arg << " + (size_t)bz * GM + m, r); }\n";
+        }
         }
     }
     for (size_t oi = 0; oi < pr.epi.outs.size(); oi++) {
@@ -1090,22 +1126,35 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     splice("EPILOGUE_BODY", body.str());
     splice("EPILOGUE_FINISH", finish.str());
     s << body_text;
+    if (pr.split_k > 1) {
+        // second launch of a split-k product: the output element is the sum of its partials, rounded once
+        HE_REQUIRE(pr.batch == 1 && pr.epi.outs.size() == 1 && !pr.epi.outs[0].reduce && pr.epi.exprs.size() == 1, HE_ERR_UNSUPPORTED,
+                   "split-k needs an unbatched product with a plain epilogue");
+        const tp::Out& o = pr.epi.outs[0];
+        s << "extern \"C\" __global__ __launch_bounds__(256) void fused_matmul_finalize(const float* __restrict__ ws, " << tp::c_type(o.dtype)
+          << "* __restrict__ out) {\nconst size_t total = (size_t)GM * GN;\nfor (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {\n"
+          << "float acc = 0.0f;\n#pragma unroll 4\nfor (u32 sp = 0; sp < " << pr.split_k << "u; sp++) acc += ws[(size_t)sp * total + i];\n"
+          << "float one[1] = {acc};\nst_vec<1>(out + i, one);\n}\n}\n";
+    }
     source_ = s.str();
 
     const int64_t tiles = ((pr.M + t.bm - 1) / t.bm) * ((pr.N + t.bn - 1) / t.bn);
     HE_REQUIRE(tiles < (1ll << 31) && pr.batch < 65536, HE_ERR_INVALID, "GEMM grid too large");
     grid_[0] = (uint32_t)tiles;
-    grid_[1] = (uint32_t)pr.batch;
+    grid_[1] = (uint32_t)(pr.split_k > 1 ? pr.split_k : pr.batch);
     threads_ = (uint32_t)threads;
     for (auto& o : pr.epi.outs)
         if (o.reduce) fills_.push_back({pr.map_e[o.arg], 0u});
     describe_ = strfmt("gemm [%lld,%lld,%lld]x[%lld] tile=%dx%dx%d stages=%d waves=%dx%d threads=%d grid=%ux%u rawA=%d rawB=%d NVA=%d NVB=%d NVE=%d "
-                       "direct=%d%d mma=%s epilogue_exprs=%zu outs=%zu",
+                       "direct=%d%d mma=%s epilogue_exprs=%zu outs=%zu split_k=%d",
                        (long long)pr.batch, (long long)pr.M, (long long)pr.K, (long long)pr.N, t.bm, t.bn, t.bk, t.stages, t.wm, t.wn, threads,
                        grid_[0], grid_[1], (int)raw_a, (int)raw_b, nva, nvb, nve, (int)direct_a, (int)direct_b, dtype_name(pr.mma_dtype), pr.epi.exprs.size(),
-                       pr.epi.outs.size());
+                       pr.epi.outs.size(), pr.split_k);
     kernel_.reset(new JitKernel(source_, "fused_matmul", {"-ffp-contract=fast", "-munsafe-fp-atomics"}));
+    if (pr.split_k > 1) finalize_.reset(new JitKernel(source_, "fused_matmul_finalize", {"-ffp-contract=fast", "-munsafe-fp-atomics"}));
 }
+
+GemmKernel::~GemmKernel() { scratch_.release(); }
 
 void GemmKernel::execute(void* const* ptrs, hipStream_t stream) {
     const size_t nargs = prob_.args.size();
@@ -1119,10 +1168,23 @@ void GemmKernel::execute(void* const* ptrs, hipStream_t stream) {
         fills.push_back({ptrs[f.first], {(uint32_t)(storage_bytes(a.dtype, (size_t)a.numel) / 4), f.second}});
     }
     if (!fills.empty()) fill_buffers(fills, stream);
-    std::vector<void*> holders(ptrs, ptrs + nargs), argv(nargs);
-    for (size_t i = 0; i < nargs; i++) argv[i] = &holders[i];
+    std::vector<void*> holders(ptrs, ptrs + nargs);
+    float* ws = nullptr;
+    if (prob_.split_k > 1) {
+        ws = scratch_.get((uint64_t)prob_.split_k * prob_.M * prob_.N, 0, stream).floats;
+        holders.push_back(ws);
+    }
+    std::vector<void*> argv(holders.size());
+    for (size_t i = 0; i < holders.size(); i++) argv[i] = &holders[i];
     const uint32_t block[3] = {threads_, 1, 1};
     kernel_->launch(grid_, block, 0, stream, argv.data());
+    if (finalize_) {
+        void* out = ptrs[prob_.map_e[prob_.epi.outs[0].arg]];
+        void* fargv[] = {&ws, &out};
+        const uint64_t total = (uint64_t)prob_.M * prob_.N;
+        const uint32_t fgrid[3] = {(uint32_t)std::min<uint64_t>((total + 255) / 256, 2048), 1, 1}, fblock[3] = {256, 1, 1};
+        finalize_->launch(fgrid, fblock, 0, stream, fargv);
+    }
 }
 
 }  // namespace he

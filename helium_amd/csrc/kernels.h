@@ -85,6 +85,13 @@ struct GemmProblem {
         bool on = false, bwd = false;
         int64_t N = 0, H = 0, W = 0, C = 0, R = 0, S = 0, P = 0, Q = 0, sh = 1, sw = 1, dh = 1, dw = 1, ph = 0, pw = 0;
     } conv_a;
+    // ConvBackwardFilter: B[k = output pixel (n, p, q)][n = tap (r, s, c)] is gathered from the image with the same
+    // map as a forward convolution's A operand, transposed in role.
+    ConvGather conv_b;
+    // The k range is dealt to `split_k` workgroups per output tile (blockIdx.y); each writes its f32 partial tile to
+    // scratch and a second launch adds them up. For products with few output tiles and a long k (a filter gradient:
+    // 64 x 576 outputs, k = 200704). Needs batch == 1 and a plain epilogue (one full-size output, no reduction).
+    int split_k = 1;
     // B rows that are not consecutive in memory: row k = rs * group + o lives at element o * o_stride + rs * rs_stride
     // (the filter [o][r][s][c] seen as the [(r, s, o)][c] matrix of ConvBackwardData). Columns stay contiguous.
     struct RowGather {
@@ -112,14 +119,16 @@ public:
     const std::string& describe() const override { return describe_; }
     void execute(void* const* ptrs, hipStream_t stream) override;
     const GemmProblem& problem() const { return prob_; }
+    ~GemmKernel() override;
 
 private:
     GemmProblem prob_;
     std::string source_, describe_;
-    std::unique_ptr<JitKernel> kernel_;
+    std::unique_ptr<JitKernel> kernel_, finalize_;  // finalize_: adds up the partial tiles of a split-k product
     uint32_t grid_[3] = {1, 1, 1};
     uint32_t threads_ = 256;
     std::vector<std::pair<int, uint32_t>> fills_;
+    ReduceScratch scratch_;
 };
 
 }  // namespace he

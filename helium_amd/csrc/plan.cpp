@@ -133,8 +133,9 @@ Instr make_instr_for_op(const std::shared_ptr<const ir::OpGraph>& g, NodeId node
         // The reference hands convolutions to cuDNN (cuda.rs:55-58, cudnn_graph.rs:193-204); here the forward
         // convolution is the fused GEMM with an implicit im2col gather as its A operand.
         case ir::OpKind::Conv:
-        case ir::OpKind::ConvBackwardData: return Instr(InstrKind::Gemm, sg);
-        default: fail(HE_ERR_UNSUPPORTED, "ConvBackwardFilter has no instruction in this backend");
+        case ir::OpKind::ConvBackwardData:
+        case ir::OpKind::ConvBackwardFilter: return Instr(InstrKind::Gemm, sg);
+        default: fail(HE_ERR_INVALID, "unknown op kind");
     }
 }
 
@@ -608,9 +609,81 @@ GemmProblem conv_backward_data_problem(const ir::OpSubgraph& sg, NodeId node) {
 }
 }  // namespace
 
+namespace {
+// Op::ConvBackwardFilter as a GEMM: rows = output channels o, columns = filter taps (r, s, c), k = output pixels
+// (n, p, q). A is the flow read as [k][m] (its own memory order: m contiguous); B[k][(r, s, c)] is gathered from the
+// image with the forward convolution's map. The product has few output tiles and a very long k, so the k range is
+// split over many workgroups whose partial tiles a second launch adds up.
+GemmProblem conv_backward_filter_problem(const ir::OpSubgraph& sg, NodeId node) {
+    const ir::OpGraph& g = *sg.graph();
+    HE_REQUIRE(sg.nodes().size() == 1, HE_ERR_UNSUPPORTED, "a convolution instruction holds the op alone");
+    const ir::Op& op = g.get(node).op;
+    const ir::Descriptor &flow = g.get(op.inputs[0]).desc, &image = g.get(op.inputs[1]).desc, &out = g.get(node).desc;
+    HE_REQUIRE(flow.shape.size() == 4 && image.shape.size() == 4, HE_ERR_INVALID, "conv backward takes rank-4 tensors");
+    HE_REQUIRE(dtype_class(flow.dtype) == DataClass::Float && image.dtype == flow.dtype, HE_ERR_UNSUPPORTED,
+               "conv backward takes a float flow and an image of the same type");
+    HE_REQUIRE(flow.shape[3] == op.conv.out_channels && image.shape[3] == op.conv.in_channels && flow.shape[0] == image.shape[0],
+               HE_ERR_INVALID, "conv backward filter: flow / image shapes do not match the parameters");
+    GemmProblem pr;
+    auto& cv = pr.conv_b;
+    cv.on = true;
+    cv.N = image.shape[0]; cv.H = image.shape[1]; cv.W = image.shape[2]; cv.C = image.shape[3];
+    cv.R = op.conv.kernel[0]; cv.S = op.conv.kernel[1];
+    cv.P = flow.shape[1]; cv.Q = flow.shape[2];
+    cv.sh = op.conv.stride[0]; cv.sw = op.conv.stride[1];
+    cv.dh = op.conv.dilation[0]; cv.dw = op.conv.dilation[1];
+    int64_t pad[2];
+    op.conv.padding(pad);
+    cv.ph = pad[0]; cv.pw = pad[1];
+    pr.batch = 1;
+    pr.M = op.conv.out_channels;
+    pr.N = cv.R * cv.S * cv.C;
+    pr.K = cv.N * cv.P * cv.Q;
+    HE_REQUIRE(pr.K > 0 && pr.K < (1ll << 31) && ir::num_elements(image.shape) < (1ll << 32), HE_ERR_UNSUPPORTED, "conv too large for 32-bit tile indices");
+    pr.mma_dtype = flow.dtype == HE_F32 ? HE_F32 : flow.dtype == HE_F16 ? HE_F16 : HE_BF16;
+    const int64_t epc = pr.mma_dtype == HE_F32 ? 4 : 8;
+    HE_REQUIRE(cv.C % epc == 0, HE_ERR_UNSUPPORTED, "conv backward filter needs an input-channel count that fills 16-byte chunks");
+    auto operand = [&](tp::Program& p, const ir::Descriptor& d, NodeId n, int64_t rows, int64_t cols) {
+        p.dims = {1, rows, cols};
+        p.args.push_back({d.dtype, ir::num_elements(d.shape), false, n});
+        tp::Expr e;
+        e.kind = tp::Expr::Load;
+        e.cls = tp::Cls::F;
+        e.access.arg = 0;
+        e.access.dtype = d.dtype;
+        e.access.stride = ir::packed_strides(p.dims);
+        p.exprs.push_back(e);
+    };
+    operand(pr.op_a, flow, op.inputs[0], pr.K, pr.M);   // [k][m] as stored
+    pr.a_km = true;
+    operand(pr.op_b, image, op.inputs[1], pr.K, pr.N);  // stand-in: only the argument is used
+    pr.root_a = pr.root_b = 0;
+    // about two workgroups per CU, each with at least four 64-wide k-tiles (128x128 output tiles)
+    const int64_t tiles = ((pr.M + 127) / 128) * ((pr.N + 127) / 128), k_tiles = (pr.K + 63) / 64;
+    pr.split_k = (int)std::max<int64_t>(1, std::min<int64_t>({(512 + tiles - 1) / tiles, k_tiles / 4, 1024}));
+    pr.epi.dims = {1, pr.M, pr.N};
+    pr.epi.fast_math = true;
+    tp::Expr acc;
+    acc.kind = tp::Expr::Acc;
+    acc.cls = tp::Cls::F;
+    pr.epi.exprs.push_back(acc);
+    pr.epi.acc_expr = 0;
+    tp::Out o;
+    o.expr = 0;
+    o.arg = 0;
+    o.dtype = out.dtype;
+    pr.epi.outs.push_back(o);
+    pr.epi.args.push_back({out.dtype, ir::num_elements(out.shape), true, node});
+    validate_gemm_epilogue(pr.epi);
+    assemble_gemm_args(pr);
+    return pr;
+}
+}  // namespace
+
 GemmProblem gemm_problem_from_ir(const ir::OpSubgraph& sg) {
     const ir::OpGraph& g = *sg.graph();
     for (NodeId n : sg.nodes()) {
+        if (g.get(n).op.kind == ir::OpKind::ConvBackwardFilter) return conv_backward_filter_problem(sg, n);
         if (g.get(n).op.kind == ir::OpKind::Conv) return conv_problem(sg, n);
         if (g.get(n).op.kind == ir::OpKind::ConvBackwardData) return conv_backward_data_problem(sg, n);
     }

@@ -60,6 +60,9 @@ def infer(node, desc):
         return [image[0], out[0], out[1], node["params"]["out_channels"]], t0
     if op == "conv_bwd_data":  # op.rs:143-158
         return [s0[0], node["input_size"][0], node["input_size"][1], node["params"]["in_channels"]], t0
+    if op == "conv_bwd_filter":  # op.rs:159-173
+        p = node["params"]
+        return [p["out_channels"], p["kernel_size"][0], p["kernel_size"][1], p["in_channels"]], t0
     raise ValueError(op)
 
 
@@ -289,6 +292,8 @@ def _eval_op(n, desc, val):
         return conv(val[ins[0]], val[ins[1]], n["params"], desc[ins[0]][1])
     if op == "conv_bwd_data":
         return conv_backward_data(val[ins[0]], val[ins[1]], n["params"], n["input_size"])
+    if op == "conv_bwd_filter":
+        return conv_backward_filter(val[ins[0]], val[ins[1]], n["params"])
     raise ValueError(op)
 
 
@@ -315,6 +320,30 @@ def conv_backward_data(flow, filt, params, input_size):
                 continue
             contrib = np.einsum("nhwo,oc->nhwc", dy[:, vh][:, :, vw], f[:, r, s, :])
             out[np.ix_(np.arange(n), ih[vh], iw[vw], np.arange(c))] += contrib
+    return out.astype(np.float32)
+
+
+def conv_backward_filter(flow, image, params):
+    """Gradient of `conv` with respect to its filter (cuDNN's CONVOLUTION_BACKWARD_FILTER for the descriptor of
+    cudnn_graph.rs:217-228,384-396): filter tap (o, r, s, c) collects flow[n,p,q,o] * image[n, p*sh + r*dh - ph,
+    q*sw + s*dw - pw, c] over every output pixel whose tap lies inside the image. Evaluated in float64."""
+    n, oh, ow, o = flow.shape
+    _, h, w, c = image.shape
+    kr, ks = params["kernel_size"]
+    sh, sw = params.get("stride", (1, 1))
+    dh, dw = params.get("dilation", (1, 1))
+    ph, pw = conv_padding(params)
+    dy = flow.astype(np.float64)
+    x = image.astype(np.float64)
+    out = np.zeros((o, kr, ks, c), dtype=np.float64)
+    for r in range(kr):
+        for s in range(ks):
+            ih = np.arange(oh) * sh + r * dh - ph
+            iw = np.arange(ow) * sw + s * dw - pw
+            vh, vw = (ih >= 0) & (ih < h), (iw >= 0) & (iw < w)
+            if not vh.any() or not vw.any():
+                continue
+            out[:, r, s, :] = np.einsum("nhwo,nhwc->oc", dy[:, vh][:, :, vw], x[:, ih[vh]][:, :, iw[vw]])
     return out.astype(np.float32)
 
 

@@ -287,3 +287,40 @@ def test_convolution_backward_data_runs_as_an_implicit_gemm(gpu, image, oc, kern
     lhs, rhs = (y * dys).sum(), (xs * dx).sum()
     scale = np.sqrt((y * y).sum() * (dys * dys).sum())
     assert abs(lhs - rhs) <= (1e-5 if dtype == "f32" else 5e-3) * scale, (lhs, rhs, scale)
+
+
+@pytest.mark.parametrize("image,oc,kernel,stride,dtype", [
+    ((8, 28, 28, 64), 64, (3, 3), (1, 1), "bf16"),
+    ((4, 30, 30, 64), 128, (3, 3), (2, 2), "bf16"),
+    ((4, 30, 30, 64), 128, (1, 1), (2, 2), "bf16"),
+    ((2, 17, 19, 16), 24, (3, 3), (1, 1), "f32"),
+])
+def test_convolution_backward_filter_runs_as_a_split_k_gemm(gpu, image, oc, kernel, stride, dtype):
+    """Op::ConvBackwardFilter through execute_graph against the oracle, and the identity that ties it to the
+    forward op on the device results: <conv(x, w), dy> = <w, conv_backward_filter(dy, x)>."""
+    rng = np.random.default_rng(13)
+    params = {"in_channels": image[3], "out_channels": oc, "kernel_size": list(kernel), "stride": list(stride)}
+    out_hw = oracle_ir.conv_output_size(params, image[1:3], kernel)
+    flow_shape, fshape = [image[0], out_hw[0], out_hw[1], oc], [oc, kernel[0], kernel[1], image[3]]
+    g = ha.ir.OpGraph()
+    x = g.new_input(list(image), dtype); dy = g.new_input(flow_shape, dtype); w = g.new_input(fshape, dtype)
+    y_out = g.new_output(g.conv(x, w, params))
+    dw_out = g.new_output(g.conv_backward_filter(dy, x, params))
+    host = {x: nm.to_storage(rng.uniform(-1, 1, image).astype(np.float32), dtype),
+            dy: nm.to_storage((rng.uniform(-1, 1, flow_shape) * 0.1).astype(np.float32), dtype),
+            w: nm.to_storage((rng.uniform(-1, 1, fshape) * 0.2).astype(np.float32), dtype)}
+    got, steps = run_graph(g, host)
+    assert sorted(k for instrs, _ in steps for k, _ in instrs) == ["gemm", "gemm"], steps
+    want = oracle_ir.plan_outputs(g.nodes, host, steps)
+    tol = 1e-4 if dtype == "f32" else 1e-2
+    for o in (y_out, dw_out):
+        a = nm.from_storage(got[o], dtype, [got[o].size]).astype(np.float64)
+        b = nm.from_storage(want[o].reshape(-1), dtype, [want[o].size]).astype(np.float64)
+        assert (np.abs(a - b) <= tol * np.maximum(np.abs(b), 1.0)).all(), (o, float(np.abs(a - b).max()))
+    y = nm.from_storage(got[y_out], dtype, flow_shape).astype(np.float64)
+    dw = nm.from_storage(got[dw_out], dtype, fshape).astype(np.float64)
+    ws = nm.from_storage(host[w], dtype, fshape).astype(np.float64)
+    dys = nm.from_storage(host[dy], dtype, flow_shape).astype(np.float64)
+    lhs, rhs = (y * dys).sum(), (ws * dw).sum()
+    scale = np.sqrt((y * y).sum() * (dys * dys).sum())
+    assert abs(lhs - rhs) <= (1e-5 if dtype == "f32" else 5e-3) * scale, (lhs, rhs, scale)

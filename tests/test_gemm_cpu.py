@@ -161,12 +161,20 @@ def run_ir_kernel_on_cpu(g, nodes, inputs):
     k = ha.backend.matmul_kernel(g, nodes)
     gx, gy = map(int, re.search(r"grid=(\d+)x(\d+)", k.description).groups())
     threads = int(re.search(r"threads=(\d+)", k.description).group(1))
+    split = int(re.search(r"split_k=(\d+)", k.description).group(1))
+    m, n = (int(v) for v in re.search(r"gemm \[\d+,(\d+),\d+\]x\[(\d+)\]", k.description).groups())
     bufs = []
     for a in k.args:
         dt = nm.NP_STORAGE[a["dtype"]]
         bufs.append((np.zeros(a["numel"], dtype=dt), 2) if a["is_output"] else (inputs[a["node"]], 0))
-    res = run_kernel(k.source, "fused_matmul", gx, threads, bufs, grid_y=gy)
     outs = [a for a in k.args if a["is_output"]]
+    if split > 1:
+        # a split-k product: partial tiles go to scratch, a second launch adds them up into the one output
+        res = run_kernel(k.source, "fused_matmul", gx, threads, bufs + [(np.full(split * m * n, np.nan, dtype=np.float32), 2)], grid_y=gy)
+        (out,) = outs
+        res = run_kernel(k.source, "fused_matmul_finalize", 2, 256, [(res[-1], 0), (np.zeros(out["numel"], dtype=nm.NP_STORAGE[out["dtype"]]), 1)])
+    else:
+        res = run_kernel(k.source, "fused_matmul", gx, threads, bufs, grid_y=gy)
     return k, {a["node"]: nm.from_storage(r, a["dtype"], [r.size]).astype(np.float64) for a, r in zip(outs, res)}
 
 
@@ -292,3 +300,42 @@ def test_conv_backward_data_on_cpu(name, image, oc, kernel, dtype, stride, dilat
     want = nm.from_storage(want.reshape(-1), dtype, [want.size]).astype(np.float64)
     tol = 1e-4 if dtype == "f32" else 2e-2
     assert np.abs(got[dx] - want).max() <= tol * max(1.0, np.abs(want).max()), (k.description, np.abs(got[dx] - want).max())
+
+
+BWD_FILTER_CASES = [
+    # name, image NHWC, out channels, kernel, dtype, stride, dilation, mode, tile
+    ("3x3_same_bf16", (2, 9, 10, 16), 24, (3, 3), "bf16", (1, 1), (1, 1), "same", "128,128,64,2,2"),
+    ("3x3_stride2_bf16", (2, 12, 12, 8), 32, (3, 3), "bf16", (2, 2), (1, 1), "same", "64,64,64,2,2"),
+    ("1x1_stride2_shortcut", (2, 8, 8, 32), 64, (1, 1), "bf16", (2, 2), (1, 1), "same", "128,128,64,2,2"),
+    ("direct_loads_both_operands", (4, 16, 16, 16), 128, (3, 3), "bf16", (1, 1), (1, 1), "same", "128,128,64,2,2"),
+    ("valid_and_dilated_f32", (2, 9, 9, 4), 8, (3, 3), "f32", (1, 1), (2, 1), "valid", "64,64,32,2,2"),
+]
+
+
+@pytest.mark.parametrize("name,image,oc,kernel,dtype,stride,dilation,mode,tile", BWD_FILTER_CASES, ids=[c[0] for c in BWD_FILTER_CASES])
+def test_conv_backward_filter_on_cpu(name, image, oc, kernel, dtype, stride, dilation, mode, tile):
+    """Op::ConvBackwardFilter as a split-k implicit GEMM: the flow read as a [k][m] A operand, the image gathered
+    as B, partial tiles added by the second launch."""
+    from oracle import helium_ir as oracle_ir
+
+    rng = np.random.default_rng(11)
+    params = {"in_channels": image[3], "out_channels": oc, "kernel_size": list(kernel), "stride": list(stride),
+              "dilation": list(dilation), "padding_mode": mode}
+    out_hw = oracle_ir.conv_output_size(params, image[1:3], kernel)
+    flow_shape = [image[0], out_hw[0], out_hw[1], oc]
+    g = ha.ir.OpGraph()
+    dy = g.new_input(flow_shape, dtype); x = g.new_input(list(image), dtype)
+    dw = g.conv_backward_filter(dy, x, params)
+    g.new_output(dw)
+    assert g.descriptor(dw) == ([oc, kernel[0], kernel[1], image[3]], dtype)
+    inputs = {dy: nm.to_storage((rng.uniform(-1, 1, flow_shape) * 0.5).astype(np.float32), dtype),
+              x: nm.to_storage(rng.uniform(-1, 1, image).astype(np.float32), dtype)}
+    os.environ["HELIUM_HIP_GEMM_TILE"] = tile
+    try:
+        k, got = run_ir_kernel_on_cpu(g, [dw], inputs)
+    finally:
+        del os.environ["HELIUM_HIP_GEMM_TILE"]
+    want = oracle_ir.kernel_outputs(g.nodes, inputs, [dw])[dw]
+    want = nm.from_storage(want.reshape(-1), dtype, [want.size]).astype(np.float64)
+    tol = 1e-4 if dtype == "f32" else 2e-2
+    assert np.abs(got[dw] - want).max() <= tol * max(1.0, np.abs(want).max()), (k.description, np.abs(got[dw] - want).max())
