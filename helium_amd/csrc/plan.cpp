@@ -77,8 +77,9 @@ void set_fold_swap_into_reduce(bool on) { g_fold_swap_into_reduce.store(on); }
 bool fold_swap_into_reduce() { return g_fold_swap_into_reduce.load(); }
 
 bool Instr::can_fuse_with(const Instr& next) const {
+    // (a large SwapDims is a Permute instruction: it joins a following Matmul as a transposed operand the same way)
     const bool gemm_and_pointwise = (kind_ == InstrKind::Gemm && next.kind_ == InstrKind::Pointwise) ||
-                                    (kind_ == InstrKind::Pointwise && next.kind_ == InstrKind::Gemm);
+                                    ((kind_ == InstrKind::Pointwise || kind_ == InstrKind::Permute) && next.kind_ == InstrKind::Gemm);
     if (gemm_and_pointwise && fuse_matmul_epilogue()) {
         // Beyond the reference, whose matmul instruction never fuses: pointwise and reduce ops that follow a Matmul
         // join it when they can run on the accumulators as the fused GEMM's epilogue; so do the ops that only prepare
@@ -720,8 +721,25 @@ GemmProblem gemm_problem_from_ir(const ir::OpSubgraph& sg) {
         case ir::Precision::MulF16AccumF16: pr.mma_dtype = HE_F16; break;
         default: pr.mma_dtype = HE_BF16; break;
     }
-    auto operand = [&](tp::Program& p, const ir::Descriptor& d, NodeId node, int64_t rows, int64_t cols) {
-        p.dims = {batch, rows, cols};
+    // An operand is a subgraph input, or (beyond the reference, whose matmul takes materialised operands only) a
+    // SwapDims of the two matrix dims of one: `x.transpose().matmul(dy)`, `dy.matmul(w.transpose())` of a linear
+    // layer's backward pass. The transposed tensor is then never written: the kernel reads the source as it lies.
+    size_t operand_swaps = 0;
+    auto operand = [&](tp::Program& p, NodeId node, int64_t rows, int64_t cols) -> bool {
+        bool swapped = false;
+        if (!sg.is_input(node)) {
+            const ir::Node& sn = g.get(node);
+            const int64_t rank = (int64_t)sn.desc.shape.size();
+            const bool last_two = sn.kind == ir::Node::Intermediate && sn.op.kind == ir::OpKind::SwapDims &&
+                                  std::min(sn.op.axis_a, sn.op.axis_b) == rank - 2 && std::max(sn.op.axis_a, sn.op.axis_b) == rank - 1;
+            HE_REQUIRE(last_two && sg.contains(node) && sg.is_input(sn.op.inputs[0]) && g.outbound(node).size() == 1, HE_ERR_UNSUPPORTED,
+                       "ops that feed a Matmul operand are fused through the fusion IR only (a transposition of the matrix dims aside)");
+            swapped = true;
+            operand_swaps++;
+            node = sn.op.inputs[0];
+        }
+        const ir::Descriptor& d = g.get(node).desc;
+        p.dims = swapped ? ir::Shape{batch, cols, rows} : ir::Shape{batch, rows, cols};
         p.args.push_back({d.dtype, ir::num_elements(d.shape), false, node});
         tp::Expr e;
         e.kind = tp::Expr::Load;
@@ -730,13 +748,12 @@ GemmProblem gemm_problem_from_ir(const ir::OpSubgraph& sg) {
         e.access.dtype = d.dtype;
         e.access.stride = ir::packed_strides(p.dims);
         p.exprs.push_back(e);
+        return swapped;
     };
-    operand(pr.op_a, da, op.inputs[0], pr.M, pr.K);
-    operand(pr.op_b, db, op.inputs[1], pr.K, pr.N);
+    pr.a_km = operand(pr.op_a, op.inputs[0], pr.M, pr.K);
+    pr.b_nk = operand(pr.op_b, op.inputs[1], pr.K, pr.N);
     pr.root_a = pr.root_b = 0;
-    HE_REQUIRE(sg.is_input(op.inputs[0]) && sg.is_input(op.inputs[1]), HE_ERR_UNSUPPORTED,
-               "ops that feed a Matmul operand are fused through the fusion IR only");
-    if (sg.nodes().size() == 1) {
+    if (sg.nodes().size() == 1 + operand_swaps) {
         pr.epi.dims = {batch, pr.M, pr.N};
         pr.epi.fast_math = true;
         tp::Expr acc;

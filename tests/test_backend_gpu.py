@@ -324,3 +324,17 @@ def test_convolution_backward_filter_runs_as_a_split_k_gemm(gpu, image, oc, kern
     lhs, rhs = (y * dys).sum(), (ws * dw).sum()
     scale = np.sqrt((y * y).sum() * (dys * dys).sum())
     assert abs(lhs - rhs) <= (1e-5 if dtype == "f32" else 5e-3) * scale, (lhs, rhs, scale)
+
+
+@pytest.mark.parametrize("dtype,precision", [("f32", "f32_f32"), ("bf16", "bf16_f32")])
+def test_linear_layer_backward_products(gpu, dtype, precision):
+    """dW = x^T dy and dX = dy w^T through execute_graph: two GEMM instructions that read the untransposed
+    operands, no permute and no pointwise transposition in the plan."""
+    g, n = plans.linear_backward_graph(512, 384, 640, dtype, precision)
+    rng = np.random.default_rng(15)
+    host = {n["x"]: nm.to_storage(rng.uniform(-1, 1, (512, 384)).astype(np.float32), dtype),
+            n["w"]: nm.to_storage(rng.uniform(-1, 1, (384, 640)).astype(np.float32), dtype),
+            n["dy"]: nm.to_storage(rng.uniform(-1, 1, (512, 640)).astype(np.float32), dtype)}
+    got, steps = run_graph(g, host)
+    assert sorted(k for instrs, _ in steps for k, _ in instrs) == ["gemm", "gemm"], steps
+    check_against_oracle(g, host, got, steps, matmul_rel=1e-4 if dtype == "f32" else 1e-2)

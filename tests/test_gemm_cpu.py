@@ -339,3 +339,26 @@ def test_conv_backward_filter_on_cpu(name, image, oc, kernel, dtype, stride, dil
     want = nm.from_storage(want.reshape(-1), dtype, [want.size]).astype(np.float64)
     tol = 1e-4 if dtype == "f32" else 2e-2
     assert np.abs(got[dw] - want).max() <= tol * max(1.0, np.abs(want).max()), (k.description, np.abs(got[dw] - want).max())
+
+
+@pytest.mark.parametrize("dtype,precision,tol", [("f32", "f32_f32", 1e-4), ("bf16", "bf16_f32", 2e-2)])
+def test_ir_matmul_with_transposed_operands_on_cpu(dtype, precision, tol):
+    """x^T dy and dy w^T of a linear layer's backward pass: each SwapDims joins its Matmul and the kernel reads
+    the untransposed tensor (A as [k][m], B as [n][k])."""
+    import test_plan_cpu as plans
+    from oracle import helium_ir as oracle_ir
+
+    g, n = plans.linear_backward_graph(64, 96, 80, dtype, precision)
+    rng = np.random.default_rng(14)
+    host = {n["x"]: nm.to_storage(rng.uniform(-1, 1, (64, 96)).astype(np.float32), dtype),
+            n["w"]: nm.to_storage(rng.uniform(-1, 1, (96, 80)).astype(np.float32), dtype),
+            n["dy"]: nm.to_storage(rng.uniform(-1, 1, (64, 80)).astype(np.float32), dtype)}
+    val, _ = oracle_ir.evaluate(g.nodes, host)
+    for nodes, out in (([n["xt"], n["dw"]], n["dw"]), ([n["wt"], n["dx"]], n["dx"])):
+        os.environ["HELIUM_HIP_GEMM_TILE"] = "64,64,32,2,2" if dtype == "f32" else "64,64,64,2,2"
+        try:
+            k, got = run_ir_kernel_on_cpu(g, nodes, host)
+        finally:
+            del os.environ["HELIUM_HIP_GEMM_TILE"]
+        want = val[out].reshape(-1).astype(np.float64)
+        assert np.abs(got[out] - want).max() <= tol * max(1.0, np.abs(want).max()), (k.description, np.abs(got[out] - want).max())

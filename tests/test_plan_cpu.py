@@ -230,3 +230,30 @@ def test_batch_norm_reference_plan_has_the_permute(reference_grouping):
     assert [k for k, _ in steps[0][0]] == ["permute"]
     assert sorted(k for k, _ in steps[1][0]) == ["pointwise", "pointwise"]  # the two statistics read xt separately
     assert oracle_plan.generate_plan(g.nodes) == steps
+
+
+def linear_backward_graph(rows=64, inner=96, cols=80, dtype="f32", precision="f32_f32"):
+    """The two products of a linear layer's backward pass as the front end records them:
+    dW = x^T dy and dX = dy w^T (transpositions as SwapDims of the matrix dims)."""
+    g = ha.ir.OpGraph()
+    x = g.new_input([rows, inner], dtype); w = g.new_input([inner, cols], dtype); dy = g.new_input([rows, cols], dtype)
+    xt = g.swap_dims(x, 0, 1)
+    dw = g.matmul(xt, dy, precision)
+    wt = g.swap_dims(w, 0, 1)
+    dx = g.matmul(dy, wt, precision)
+    names = {"x": x, "w": w, "dy": dy, "xt": xt, "wt": wt, "dw": dw, "dx": dx, "dw_out": g.new_output(dw), "dx_out": g.new_output(dx)}
+    return g, names
+
+
+def test_transposed_matmul_operands_join_the_gemm_instruction():
+    g, n = linear_backward_graph()
+    instrs = [i for step, _ in Plan(g).steps for i in step]
+    assert sorted(instrs) == sorted([("gemm", [n["xt"], n["dw"]]), ("gemm", [n["wt"], n["dx"]])]), instrs
+
+
+def test_transposed_matmul_operands_reference_grouping(reference_grouping):
+    g, n = linear_backward_graph()
+    steps = Plan(g).steps
+    assert oracle_plan.generate_plan(g.nodes) == steps
+    kinds = sorted(k for step, _ in steps for k, _ in step)
+    assert kinds == ["gemm", "gemm", "pointwise", "pointwise"], steps
