@@ -680,6 +680,13 @@ GemmProblem gemm_problem_from_fusion(const fir::OpGraph& g) {
     return pr;
 }
 
+int choose_split_k(int64_t M, int64_t N, int64_t K, int64_t batch) {
+    if (getenv("HELIUM_HIP_GEMM_NO_SPLIT_K") || batch != 1) return 1;
+    const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128), k_tiles = (K + 63) / 64;
+    if (tiles >= 128) return 1;
+    return (int)std::max<int64_t>(1, std::min<int64_t>({(384 + tiles - 1) / tiles, k_tiles / 8, 1024}));
+}
+
 bool operand_b_prefers_nk(const tp::Program& op_b) {
     const tp::Expr* big = nullptr;
     for (auto& e : op_b.exprs) {
@@ -779,7 +786,8 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
             t.wm = t.wn = 2;
             small = true;
             // still fewer workgroups than half the CUs: 64x64 tiles (one MFMA block per wave) spread the work
-            if (pr.M > 64 && pr.N > 64 && ((pr.M + 127) / 128) * ((pr.N + 127) / 128) * pr.batch < 128) t.bm = t.bn = 64;
+            // (a split k range multiplies the workgroups instead and keeps the tile's arithmetic intensity)
+            if (pr.M > 64 && pr.N > 64 && ((pr.M + 127) / 128) * ((pr.N + 127) / 128) * pr.batch * pr.split_k < 128) t.bm = t.bn = 64;
         }
     }
     HE_REQUIRE(t.bm % (t.wm * 32) == 0 && t.bn % (t.wn * 32) == 0 && (t.bk == 64 || t.bk == 32) && (!f32 || t.bk == 32), HE_ERR_INVALID, "bad GEMM tile");

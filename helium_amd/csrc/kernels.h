@@ -108,6 +108,9 @@ void assemble_gemm_args(GemmProblem& pr);
 // True when the B operand program (over [batch,K,N]) reads its largest source with unit stride along k and a
 // larger one along n: lowering it over [batch,N,K] instead makes its accesses vectors.
 bool operand_b_prefers_nk(const tp::Program& op_b);
+// How many workgroups should share one output tile's k range: 1 unless 128x128 tiles leave most CUs idle and k is
+// long enough to give every share at least eight 64-wide k-tiles. Only products with a plain epilogue may split.
+int choose_split_k(int64_t M, int64_t N, int64_t K, int64_t batch);
 // Throws HE_ERR_UNSUPPORTED for an epilogue program the GEMM kernel cannot run.
 void validate_gemm_epilogue(const tp::Program& epi);
 

@@ -501,6 +501,7 @@ GemmProblem conv_problem(const ir::OpSubgraph& sg, NodeId conv) {
     pr.M = cv.N * cv.P * cv.Q;
     pr.N = op.conv.out_channels;
     pr.K = cv.R * cv.S * cv.C;
+    pr.split_k = choose_split_k(pr.M, pr.N, pr.K, 1);
     HE_REQUIRE(pr.M > 0 && pr.M < (1ll << 31) && ir::num_elements(image.shape) < (1ll << 32), HE_ERR_UNSUPPORTED, "conv too large for 32-bit tile indices");
     pr.mma_dtype = image.dtype == HE_F32 ? HE_F32 : image.dtype == HE_F16 ? HE_F16 : HE_BF16;
     auto operand = [&](tp::Program& p, const ir::Descriptor& d, NodeId node, int64_t rows, int64_t cols) {
@@ -569,6 +570,7 @@ GemmProblem conv_backward_data_problem(const ir::OpSubgraph& sg, NodeId node) {
     pr.M = cv.N * cv.P * cv.Q;
     pr.N = in_channels;
     pr.K = cv.R * cv.S * cv.C;
+    pr.split_k = choose_split_k(pr.M, pr.N, pr.K, 1);
     HE_REQUIRE(pr.M > 0 && pr.M < (1ll << 31) && ir::num_elements(flow.shape) < (1ll << 32), HE_ERR_UNSUPPORTED, "conv too large for 32-bit tile indices");
     pr.mma_dtype = flow.dtype == HE_F32 ? HE_F32 : flow.dtype == HE_F16 ? HE_F16 : HE_BF16;
     HE_REQUIRE(in_channels % (pr.mma_dtype == HE_F32 ? 4 : 8) == 0, HE_ERR_UNSUPPORTED,
