@@ -257,3 +257,60 @@ def test_transposed_matmul_operands_reference_grouping(reference_grouping):
     assert oracle_plan.generate_plan(g.nodes) == steps
     kinds = sorted(k for step, _ in steps for k, _ in step)
     assert kinds == ["gemm", "gemm", "pointwise", "pointwise"], steps
+
+
+def conv_graph(kind, image=(2, 8, 8, 16), oc=32, kernel=(3, 3), dtype="bf16", filter_shape=None):
+    g = ha.ir.OpGraph()
+    params = {"in_channels": image[3], "out_channels": oc, "kernel_size": list(kernel)}
+    fshape = filter_shape or [oc, kernel[0], kernel[1], image[3]]
+    flow_shape = [image[0], image[1], image[2], oc]
+    if kind == "conv":
+        x = g.new_input(list(image), dtype); w = g.new_input(fshape, dtype)
+        out = g.conv(x, w, params)
+    elif kind == "data":
+        dy = g.new_input(flow_shape, dtype); w = g.new_input(fshape, dtype)
+        out = g.conv_backward_data(dy, w, params, image[1:3])
+    else:
+        dy = g.new_input(flow_shape, dtype); x = g.new_input(list(image), dtype)
+        out = g.conv_backward_filter(dy, x, params)
+    g.new_output(out)
+    return g, out
+
+
+@pytest.mark.parametrize("kind,shape", [("conv", [2, 8, 8, 32]), ("data", [2, 8, 8, 16]), ("filter", [32, 3, 3, 16])])
+def test_convolution_ops_are_gemm_instructions(kind, shape):
+    """Descriptors as op.rs:123-173 infers them, and one Gemm instruction per convolution op (the reference hands
+    them to cuDNN, cuda.rs:55-58)."""
+    g, out = conv_graph(kind)
+    assert g.descriptor(out) == (shape, "bf16")
+    assert [k for step, _ in Plan(g).steps for k, _ in step] == ["gemm"]
+
+
+def test_convolution_output_size_follows_the_reference_formula():
+    """compute_output_size (conv.rs:51-73): Same keeps the size, Valid subtracts kernel/2, Full adds kernel/2,
+    then the stride divides (rounding down)."""
+    for mode, stride, want in [("same", 1, 9), ("same", 2, 4), ("valid", 1, 8), ("valid", 2, 4), ("full", 1, 10), ("full", 3, 3)]:
+        g = ha.ir.OpGraph()
+        x = g.new_input([1, 9, 9, 8], "f32"); w = g.new_input([4, 3, 3, 8], "f32")
+        y = g.conv(x, w, {"in_channels": 8, "out_channels": 4, "kernel_size": [3, 3], "stride": [stride, stride], "padding_mode": mode})
+        assert g.descriptor(y)[0] == [1, want, want, 4], (mode, stride)
+
+
+def test_unsupported_convolutions_fail_with_a_message():
+    """What the implicit-GEMM instructions cannot run is refused when the kernel is made, not computed wrongly:
+    a filter whose shape contradicts the parameters, a filter type that differs from the image's, and backward
+    ops over channel counts that do not fill 16-byte chunks."""
+    g, out = conv_graph("conv", filter_shape=[32, 5, 3, 16])
+    with pytest.raises(ha.HeliumError, match="do not match"):
+        ha.backend.matmul_kernel(g, [out])
+    g = ha.ir.OpGraph()
+    x = g.new_input([1, 8, 8, 16], "bf16"); w = g.new_input([8, 3, 3, 16], "f32")
+    out = g.conv(x, w, {"in_channels": 16, "out_channels": 8, "kernel_size": [3, 3]})
+    with pytest.raises(ha.HeliumError, match="same type"):
+        ha.backend.matmul_kernel(g, [out])
+    g, out = conv_graph("data", image=(1, 8, 8, 3))
+    with pytest.raises(ha.HeliumError, match="16-byte chunks"):
+        ha.backend.matmul_kernel(g, [out])
+    g, out = conv_graph("filter", image=(1, 8, 8, 3))
+    with pytest.raises(ha.HeliumError, match="16-byte chunks"):
+        ha.backend.matmul_kernel(g, [out])
