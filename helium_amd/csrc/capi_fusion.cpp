@@ -198,11 +198,10 @@ int he_fusion_plan_execute(he_fusion_plan_t plan, const uint64_t* producer_nodes
             (void)c;
             fail(HE_ERR_UNSUPPORTED, "two Consumers of one value");
         }
-        hipEvent_t done;
-        HE_HIP(hipEventCreateWithFlags(&done, hipEventDisableTiming));
-        HE_HIP(hipEventRecord(done, s));
+        exec::EventRef done = pool.take_event();
+        HE_HIP(hipEventRecord(done->e, s));
         temporaries.clear();  // blocks return to the scope; the pool frees them for others when `done` has passed
-        pool.end_scope_after(scope, done);
+        pool.end_scope_after(scope, std::move(done));
     });
 }
 

@@ -28,35 +28,47 @@ size_t DevicePool::size_class(size_t bytes) {
     return (bytes + g - 1) / g * g;
 }
 
-void DevicePool::end_scope_after(uint64_t scope, hipEvent_t done) {
+SharedEvent::~SharedEvent() {
+    if (e) DevicePool::global().recycle(e);
+}
+
+void DevicePool::end_scope_after(uint64_t scope, EventRef done) {
     std::lock_guard<std::mutex> lk(mu_);
-    pending_.push_back({scope, done});
+    pending_.push_back({scope, std::move(done)});
+}
+
+void DevicePool::recycle(hipEvent_t event) {
+    std::lock_guard<std::mutex> lk(mu_);
+    spare_events_.push_back(event);
 }
 
 void DevicePool::poll() {
-    std::lock_guard<std::mutex> lk(mu_);
     // Oldest first, and no further than the first execution that is still running: a host that runs many
     // executions ahead of the device would otherwise query every one of them on every allocation. Executions of
     // one thread finish in order; another thread's younger ones wait for the next poll at worst.
-    while (!pending_.empty() && hipEventQuery(pending_.front().second) == hipSuccess) {
-        end_scope_locked(pending_.front().first);
-        spare_events_.push_back(pending_.front().second);
-        pending_.pop_front();
+    std::vector<EventRef> passed;  // let go of outside the lock: the last holder's release takes it again
+    {
+        std::lock_guard<std::mutex> lk(mu_);
+        while (!pending_.empty() && hipEventQuery(pending_.front().second->e) == hipSuccess) {
+            end_scope_locked(pending_.front().first);
+            passed.push_back(std::move(pending_.front().second));
+            pending_.pop_front();
+        }
     }
 }
 
-hipEvent_t DevicePool::take_event() {
+EventRef DevicePool::take_event() {
+    auto ev = std::make_shared<SharedEvent>();
     {
         std::lock_guard<std::mutex> lk(mu_);
         if (!spare_events_.empty()) {
-            hipEvent_t e = spare_events_.back();
+            ev->e = spare_events_.back();
             spare_events_.pop_back();
-            return e;
+            return ev;
         }
     }
-    hipEvent_t e;
-    HE_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
-    return e;
+    HE_HIP(hipEventCreateWithFlags(&ev->e, hipEventDisableTiming));
+    return ev;
 }
 
 uint64_t DevicePool::begin_scope(uint64_t thread) {
@@ -174,10 +186,7 @@ void DevicePool::stats(uint64_t* driver_bytes, uint64_t* driver_allocs, uint64_t
 // Tensors
 // ---------------------------------------------------------------------------------------------------------
 Tensor::~Tensor() {
-    if (ready) {
-        if (uploaded) (void)hipEventSynchronize(ready);  // the copy that fills the block may still be queued
-        (void)hipEventDestroy(ready);
-    }
+    if (ready && uploaded) (void)hipEventSynchronize(ready->e);  // the copy that fills the block may still be queued
     DevicePool::global().release(ptr, bytes, scope, used);
 }
 
@@ -188,7 +197,6 @@ TensorRef allocate_tensor(int dtype, size_t len, uint64_t scope) {
     t->bytes = storage_bytes(dtype, len);
     t->scope = scope;
     t->ptr = DevicePool::global().allocate(t->bytes, scope);
-    HE_HIP(hipEventCreateWithFlags(&t->ready, hipEventDisableTiming));
     return t;
 }
 
@@ -200,7 +208,7 @@ struct Staging {
 };
 struct Streams {
     std::vector<hipStream_t> s;
-    hipEvent_t exec_end = nullptr;  // end of this thread's latest execution (recorded on s[0] after it joined the others)
+    EventRef exec_end;  // end of this thread's latest execution (recorded on s[0] after it joined the others)
     bool has_run = false;
     hipStream_t h2d = nullptr, d2h = nullptr;
     std::vector<Staging> staging;  // pinned upload buffers, reused once their copy has finished
@@ -255,13 +263,14 @@ TensorRef create_tensor_with_data(const void* data, int dtype, size_t len) {
         HE_HIP(hipEventRecord(b.done, st.h2d));
     }
     t->uploaded = true;
-    HE_HIP(hipEventRecord(t->ready, st.h2d));
+    t->ready = DevicePool::global().take_event();
+    HE_HIP(hipEventRecord(t->ready->e, st.h2d));
     return t;
 }
 
 void download_tensor(const TensorRef& t, void* dst) {
     Streams& st = thread_streams();
-    HE_HIP(hipStreamWaitEvent(st.d2h, t->ready, 0));
+    if (t->ready) HE_HIP(hipStreamWaitEvent(st.d2h, t->ready->e, 0));
     if (t->bytes) HE_HIP(hipMemcpyAsync(dst, t->ptr, t->bytes, hipMemcpyDeviceToHost, st.d2h));
     HE_HIP(hipStreamSynchronize(st.d2h));
 }
@@ -371,7 +380,7 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
             // a stream's first work of this execution comes after the end of the thread's previous execution
             // (stream 0 carried that end itself)
             if (used_streams.insert(i % width).second && i % width != 0 && st.has_run)
-                HE_HIP(hipStreamWaitEvent(stream, st.exec_end, 0));
+                HE_HIP(hipStreamWaitEvent(stream, st.exec_end->e, 0));
             for (NodeId out : instr.outputs()) {
                 const ir::Descriptor& d = graph->get(out).desc;
                 tensors[out] = allocate_tensor(d.dtype, (size_t)ir::num_elements(d.shape), scope);
@@ -383,11 +392,11 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
                 if (inputs.count(in) && !synced.count(it->second.get())) {
                     Tensor& t = *it->second;
                     // a producer seen finished once stays finished: no wait is queued for it again
-                    if (!t.ready_seen.load(std::memory_order_acquire)) {
-                        if (hipEventQuery(t.ready) == hipSuccess) {
+                    if (t.ready && !t.ready_seen.load(std::memory_order_acquire)) {
+                        if (hipEventQuery(t.ready->e) == hipSuccess) {
                             t.ready_seen.store(true, std::memory_order_release);
                         } else {
-                            HE_HIP(hipStreamWaitEvent(stream, t.ready, 0));
+                            HE_HIP(hipStreamWaitEvent(stream, t.ready->e, 0));
                             local.event_waits++;
                         }
                     }
@@ -398,8 +407,6 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
             instr.execute([&](NodeId n) -> void* { return tensors.at(n)->ptr; }, stream);
             ht.lap(4);
             local.instrs++;
-            for (NodeId out : instr.outputs())
-                if (alive.count(out)) HE_HIP(hipEventRecord(tensors.at(out)->ready, stream));
         }
         // every stream of the next steps is ordered after this step's streams, so one wait per tensor is enough
         synced.insert(waited.begin(), waited.end());
@@ -409,13 +416,14 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
     // Drop of the executor (cuda.rs:232-260): when everything queued above has run, the scope's freed blocks
     // become available to everyone. Stream 0 joins the last step and carries the event the pool polls.
     join({0});
-    hipEvent_t done = pool.take_event();
-    HE_HIP(hipEventRecord(done, st.s[0]));
-    // The same event orders this thread's next execution after this one. The pool may hand it to another execution
-    // once it has completed; waiting for that one instead would be a needless wait, never a wrong one.
+    EventRef done = pool.take_event();
+    HE_HIP(hipEventRecord(done->e, st.s[0]));
+    // The same event orders this thread's next execution after this one, and it is the ready event of every tensor
+    // that outlives the plan (enumerate_output_tensors, cuda.rs:142-153, records one per tensor).
+    for (NodeId out : alive) tensors.at(out)->ready = done;
     st.exec_end = done;
     st.has_run = true;
-    pool.end_scope_after(scope, done);
+    pool.end_scope_after(scope, std::move(done));
     {
         // join events of the previous execution on this thread: recorded and waited on long ago
         static thread_local std::vector<hipEvent_t> garbage;

@@ -15,6 +15,15 @@ namespace he::exec {
 
 using ir::NodeId;
 
+// A device event with shared ownership: an execution records one at its end and hands it to every tensor it
+// returns, to the pool (which ends the execution's scope once it has passed) and to the thread's next execution.
+// When the last holder lets go the event returns to the pool's spare list.
+struct SharedEvent {
+    hipEvent_t e = nullptr;
+    ~SharedEvent();
+};
+using EventRef = std::shared_ptr<SharedEvent>;
+
 // Pooling device allocator (helium/src/cuda/allocator/device.rs): memory is never returned to the driver; a block
 // freed inside an execution scope is reusable by that scope at once and by everyone else when the scope has ended
 // on the device (device.rs:60-89, block.rs:216-244).
@@ -26,8 +35,8 @@ public:
     uint64_t begin_scope(uint64_t thread = 0);
     void end_scope(uint64_t scope);  // called once the scope's device work has finished
     // Ends the scope once `done` (recorded after all of its device work) has completed; polled from begin_scope and
-    // from allocate, so no host callback sits in any stream. The pool takes the event over.
-    void end_scope_after(uint64_t scope, hipEvent_t done);
+    // from allocate, so no host callback sits in any stream.
+    void end_scope_after(uint64_t scope, EventRef done);
     void poll();
     void* allocate(size_t bytes, uint64_t scope);
     // `owner`: the scope the block was allocated in (0: none); `used`: every scope whose device work touches it.
@@ -36,7 +45,8 @@ public:
     void release(void* ptr, size_t bytes, uint64_t owner, const std::vector<uint64_t>& used);
     void note_use(struct Tensor& t, uint64_t scope);
     void note_uses(const std::map<ir::NodeId, std::shared_ptr<struct Tensor>>& tensors, uint64_t scope);
-    hipEvent_t take_event();  // an event nobody waits on any more, or a new one
+    EventRef take_event();          // an event nobody holds any more, or a new one
+    void recycle(hipEvent_t event);  // called when an event's last holder lets go
     void stats(uint64_t* driver_bytes, uint64_t* driver_allocs, uint64_t* reuses);
 
 private:
@@ -51,7 +61,7 @@ private:
         std::vector<uint64_t> waiting;
     };
     std::vector<Deferred> deferred_;
-    std::deque<std::pair<uint64_t, hipEvent_t>> pending_;  // scopes whose device work may still be running, oldest first
+    std::deque<std::pair<uint64_t, EventRef>> pending_;  // scopes whose device work may still be running, oldest first
     std::vector<hipEvent_t> spare_events_;
     void end_scope_locked(uint64_t scope);
     uint64_t next_scope_ = 1, driver_bytes_ = 0, driver_allocs_ = 0, reuses_ = 0;
@@ -66,7 +76,10 @@ struct Tensor {
     std::vector<uint64_t> used;  // execution scopes that read or wrote the tensor (guarded by the pool's mutex)
     bool uploaded = false;       // filled by an asynchronous host-to-device copy
     std::atomic<bool> ready_seen{false};  // `ready` has been observed complete (it is recorded once per tensor)
-    hipEvent_t ready = nullptr;
+    // Recorded after the work that fills the tensor: the upload's own event, or the one event its execution records
+    // at its end (a record costs the device about as much as a small kernel, so an execution records one, not one
+    // per output). Null while the producing execution is still being queued.
+    EventRef ready;
     ~Tensor();
 };
 using TensorRef = std::shared_ptr<Tensor>;
