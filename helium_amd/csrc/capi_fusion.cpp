@@ -83,21 +83,31 @@ FusionKernel& kernel_of(he_fusion_plan_s& plan, FusionId id) {
 
 extern "C" {
 
+namespace {
+void fusion_search(he_fgraph_t graph, int objective, bool subdivided, he_fusion_plan_t* plan) {
+    HE_REQUIRE(graph && plan && objective >= 0 && objective <= 2, HE_ERR_INVALID, "bad argument");
+    auto p = std::make_unique<he_fusion_plan_s>();
+    p->g = std::make_shared<fir::OpGraph>(graph->g);
+    const auto params = fsearch::CostParams::mi355x();
+    fsearch::SearchResult r = subdivided ? fsearch::minimize_cost_with_subdivision(p->g, (fsearch::Objective)objective, params)
+                                         : fsearch::minimize_cost(p->g, (fsearch::Objective)objective, params);
+    r.graph.assert_invariants(false);
+    p->fg = r.graph;
+    p->cost = r.cost;
+    p->states = r.states_visited;
+    for (FusionId id : p->fg.topo_sort())
+        if (!p->fg.fusions().at(id).is_input_output(*p->g)) p->order.push_back(id);
+    p->text = p->fg.describe();
+    *plan = p.release();
+}
+}  // namespace
+
 int he_fusion_search(he_fgraph_t graph, int objective, he_fusion_plan_t* plan) {
-    return he::guard([&] {
-        HE_REQUIRE(graph && plan && objective >= 0 && objective <= 2, HE_ERR_INVALID, "bad argument");
-        auto p = std::make_unique<he_fusion_plan_s>();
-        p->g = std::make_shared<fir::OpGraph>(graph->g);
-        fsearch::SearchResult r = fsearch::minimize_cost(p->g, (fsearch::Objective)objective, fsearch::CostParams::mi355x());
-        r.graph.assert_invariants(false);
-        p->fg = r.graph;
-        p->cost = r.cost;
-        p->states = r.states_visited;
-        for (FusionId id : p->fg.topo_sort())
-            if (!p->fg.fusions().at(id).is_input_output(*p->g)) p->order.push_back(id);
-        p->text = p->fg.describe();
-        *plan = p.release();
-    });
+    return he::guard([&] { fusion_search(graph, objective, false, plan); });
+}
+
+int he_fusion_search_subdivided(he_fgraph_t graph, int objective, he_fusion_plan_t* plan) {
+    return he::guard([&] { fusion_search(graph, objective, true, plan); });
 }
 
 int he_fusion_plan_num_fusions(he_fusion_plan_t plan, int* count) {

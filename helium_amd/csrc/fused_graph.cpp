@@ -85,10 +85,10 @@ std::string Action::describe() const {
 // ---------------------------------------------------------------------------------------------------------
 // FusedGraph
 // ---------------------------------------------------------------------------------------------------------
-FusedGraph FusedGraph::identity(std::shared_ptr<const fir::OpGraph> g) {
+FusedGraph FusedGraph::identity(std::shared_ptr<const fir::OpGraph> g, FusionId first_id) {
     FusedGraph fg;
     fg.g_ = g;
-    FusionId next = 0;
+    FusionId next = first_id;
     for (OpNode n : g->nodes()) {
         Fusion f;
         if (g->get(n).is_anchor()) {
@@ -692,8 +692,9 @@ double analytical_cost(const FusedGraph& fg) {
 // ---------------------------------------------------------------------------------------------------------
 // Search
 // ---------------------------------------------------------------------------------------------------------
-SearchResult minimize_cost(std::shared_ptr<const fir::OpGraph> g, Objective objective, const CostParams& p, size_t max_states) {
-    FusedGraph initial = FusedGraph::identity(g);
+SearchResult minimize_cost(std::shared_ptr<const fir::OpGraph> g, Objective objective, const CostParams& p, size_t max_states,
+                           FusionId first_id) {
+    FusedGraph initial = FusedGraph::identity(g, first_id);
     initial.produce_maximal_fusions();
     auto cost_of = [&](const FusedGraph& fg) { return objective == Objective::Analytical ? analytical_cost(fg) : naive_cost(fg, p); };
     if (objective == Objective::Maximal) return {initial, naive_cost(initial, p), 1};
@@ -737,6 +738,120 @@ SearchResult minimize_cost(std::shared_ptr<const fir::OpGraph> g, Objective obje
     }
     best.clean();
     return {best, best_cost, total_states};
+}
+
+SearchResult minimize_cost_with_subdivision(std::shared_ptr<const fir::OpGraph> g, Objective objective, const CostParams& p,
+                                            size_t max_states) {
+    const auto subdivisions = subdivide(*g);
+    std::vector<FusedGraph> fused;
+    size_t states = 0;
+    FusionId first_id = 0;
+    for (auto& sub : subdivisions) {
+        std::vector<OpNode> nodes;
+        for (auto& entry : sub) nodes.push_back(entry.first);
+        auto part = std::make_shared<fir::OpGraph>(g->subgraph(nodes));
+        SearchResult r = minimize_cost(part, objective, p, max_states, first_id);
+        first_id += part->nodes().size();
+        states += r.states_visited;
+        fused.push_back(std::move(r.graph));
+    }
+    FusedGraph merged = FusedGraph::merge_from_subdivisions(subdivisions, fused, g);
+    const double cost = objective == Objective::Analytical ? analytical_cost(merged) : naive_cost(merged, p);
+    return {merged, cost, states};
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Merging separately fused subdivisions
+// ---------------------------------------------------------------------------------------------------------
+FusedGraph FusedGraph::merge_from_subdivisions(const std::vector<std::set<std::pair<OpNode, NodePortion>>>& subdivisions,
+                                               const std::vector<FusedGraph>& fused, std::shared_ptr<const fir::OpGraph> original) {
+    HE_REQUIRE(subdivisions.size() == fused.size(), HE_ERR_INVALID, "%zu subdivisions but %zu fused graphs", subdivisions.size(), fused.size());
+    for (auto& fg : fused) fg.assert_invariants(false);
+    std::map<FusionId, Fusion> fusions;
+    std::map<OpNode, FusionId> merged;  // anchor -> the fusion that stands for it
+    std::set<FusionId> collapsed;       // an anchor's fusion in a later subdivision, folded into the one above
+
+    // first pass: the two portions of every anchor (fused_graph.rs:925-966)
+    for (size_t i = 0; i < subdivisions.size(); i++)
+        for (auto& [node, portion] : subdivisions[i]) {
+            if (portion == NodePortion::Full) continue;
+            auto nf = fused[i].node_fusions_.find(node);
+            HE_REQUIRE(nf != fused[i].node_fusions_.end() && !nf->second.empty(), HE_ERR_INTERNAL,
+                       "anchor %llu is in no fusion of its subdivision (nothing reads it there)", (unsigned long long)node);
+            const FusionId from_id = nf->second[0];
+            const Fusion& from = fused[i].fusions_.at(from_id);
+            HE_REQUIRE(from.core, HE_ERR_INTERNAL, "anchor %llu sits in an Aux fusion", (unsigned long long)node);
+            auto seen = merged.find(node);
+            if (seen == merged.end()) {
+                HE_REQUIRE(!fusions.count(from_id), HE_ERR_INVALID, "fusion id %llu appears in two subdivisions", (unsigned long long)from_id);
+                fusions[from_id] = from;
+                merged[node] = from_id;
+                continue;
+            }
+            Fusion& into = fusions.at(seen->second);
+            if (portion == NodePortion::Epilogue) {
+                into.epilogue = from.epilogue;
+                into.dependents.insert(from.dependents.begin(), from.dependents.end());
+                // the epilogue's own reads from outside come along (the reference takes the dependents only, which
+                // leaves an epilogue node that reads another kernel's value without a provider)
+                for (auto& d : from.dependencies)
+                    if (!has(original->inbound(node), d.first)) into.dependencies[d.first] = d.second;
+            } else {
+                into.mainloop = from.mainloop;
+                for (auto& d : from.dependencies) into.dependencies[d.first] = d.second;
+            }
+            if (seen->second != from_id) collapsed.insert(from_id);
+        }
+
+    // second pass: everything else but the stand-in Producers and Consumers of the subgraphs (:968-994)
+    for (auto& fg : fused)
+        for (auto& [id, f] : fg.fusions_) {
+            if (!f.core && f.fused.size() == 1 && is_input_output(fg.g_->get(f.fused[0]))) {
+                const OpNode n = f.fused[0];
+                if (!original->has(n) || !is_input_output(original->get(n))) continue;
+                bool placed = false;
+                for (auto& kv : fusions) placed = placed || kv.second.contains(n);
+                if (placed) continue;
+            }
+            if (!collapsed.count(id) && !fusions.count(id)) fusions[id] = f;
+        }
+
+    // edges (:996-1031): a provider that did not survive is replaced by the first fusion that computes the value;
+    // readers that did not survive are dropped
+    auto first_with = [&](OpNode n) {
+        auto it = fusions.begin();
+        while (it != fusions.end() && !it->second.contains(n)) ++it;
+        HE_REQUIRE(it != fusions.end(), HE_ERR_INTERNAL, "no fusion computes node %llu after the merge", (unsigned long long)n);
+        return it->first;
+    };
+    for (auto& [id, f] : fusions) {
+        // An anchor's operand that the other subdivision fused into the mainloop is computed here now: the read the
+        // first subdivision recorded for it is gone (the reference keeps it, and the fusion then waits for itself).
+        for (auto it = f.dependencies.begin(); it != f.dependencies.end();)
+            it = f.contains(it->first) ? f.dependencies.erase(it) : std::next(it);
+        for (auto& [node, provider] : f.dependencies)
+            if (!fusions.count(provider)) provider = first_with(node);
+        for (auto it = f.dependents.begin(); it != f.dependents.end();)
+            it = fusions.count(it->second) ? std::next(it) : f.dependents.erase(it);
+    }
+    // Every read is listed by its provider. The reference adds this entry only where it replaced the provider, so an
+    // unfused producer of an anchor whose fusion was folded into an earlier one keeps pointing at the folded id and the
+    // reference's own invariant check then aborts; listing every read covers that case too.
+    for (auto& [id, f] : fusions)
+        for (auto& [node, provider] : f.dependencies) fusions.at(provider).dependents.insert({node, id});
+
+    FusedGraph out;
+    out.g_ = original;
+    out.fusions_ = std::move(fusions);
+    for (OpNode n : original->nodes()) {
+        auto& list = out.node_fusions_[n];
+        for (auto& kv : out.fusions_)
+            if (kv.second.contains(n)) list.push_back(kv.first);
+    }
+    // a node that nothing reads is in no fusion of its subdivision (clean) and so in none here; the reference insists on
+    // every node being placed and aborts on such a graph
+    out.assert_invariants(false);
+    return out;
 }
 
 // ---------------------------------------------------------------------------------------------------------

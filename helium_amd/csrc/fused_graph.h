@@ -14,6 +14,7 @@ namespace he::fsearch {
 
 using fir::OpNode;
 using FusionId = uint64_t;
+enum class NodePortion : int { Mainloop = 0, Epilogue = 1, Full = 2 };  // subdivision.rs:9-14
 
 // fused_graph.rs:1082-1235
 struct Fusion {
@@ -46,7 +47,9 @@ struct Action {
 
 class FusedGraph {
 public:
-    static FusedGraph identity(std::shared_ptr<const fir::OpGraph> g);  // fused_graph.rs:62-111
+    // fused_graph.rs:62-111. Fusion ids count up from `first_id` (the reference draws them from one process-wide
+    // counter, which is what lets graphs of several subdivisions be merged).
+    static FusedGraph identity(std::shared_ptr<const fir::OpGraph> g, FusionId first_id = 0);
     void produce_maximal_fusions();                                      // :113-223
     void clean();                                                        // :237-282
     std::vector<Action> enumerate_possible_actions() const;              // :285-358
@@ -56,6 +59,12 @@ public:
     void assert_invariants(bool every_node_placed = true) const;
     uint64_t state_hash() const;  // order-independent over the fusions (:51-55)
     std::string describe() const; // the printed form (:1060-1068, :1152-1183)
+
+    // fused_graph.rs:910-1058: one graph over `original` from the separately fused subdivisions (fusion ids must
+    // not repeat between them). An anchor's fusion takes its epilogue from the subdivision that holds its epilogue
+    // portion and its mainloop from the one that holds its mainloop portion.
+    static FusedGraph merge_from_subdivisions(const std::vector<std::set<std::pair<OpNode, NodePortion>>>& subdivisions,
+                                              const std::vector<FusedGraph>& fused, std::shared_ptr<const fir::OpGraph> original);
 
     const std::map<FusionId, Fusion>& fusions() const { return fusions_; }
     const fir::OpGraph& opgraph() const { return *g_; }
@@ -97,10 +106,14 @@ struct SearchResult {
     size_t states_visited;
 };
 enum class Objective : int { Maximal = 0, Naive = 1, Analytical = 2 };
-SearchResult minimize_cost(std::shared_ptr<const fir::OpGraph> g, Objective objective, const CostParams& p, size_t max_states = 200000);
+SearchResult minimize_cost(std::shared_ptr<const fir::OpGraph> g, Objective objective, const CostParams& p, size_t max_states = 200000,
+                           FusionId first_id = 0);
+// cost_model.rs:241-259: subdivide, search every subdivision's subgraph on its own, merge. The search is exponential
+// in the graph's size; the subdivisions are what keeps large graphs searchable.
+SearchResult minimize_cost_with_subdivision(std::shared_ptr<const fir::OpGraph> g, Objective objective, const CostParams& p,
+                                            size_t max_states = 200000);
 
 // subdivision.rs:24-113
-enum class NodePortion : int { Mainloop = 0, Epilogue = 1, Full = 2 };
 std::vector<std::set<std::pair<OpNode, NodePortion>>> subdivide(const fir::OpGraph& g);
 
 }  // namespace he::fsearch

@@ -1,5 +1,7 @@
 #include "fusion_ir.h"
 
+#include <set>
+
 namespace he::fir {
 
 std::vector<OpNode> Op::inputs() const {
@@ -70,6 +72,38 @@ OpNode OpGraph::insert_with_id(OpNode id, const Op& op) {
     out_[id];
     if (id >= next_) next_ = id + 1;
     return id;
+}
+
+OpGraph OpGraph::subgraph(const std::vector<OpNode>& nodes) const {
+    std::set<OpNode> keep(nodes.begin(), nodes.end());
+    OpGraph out;
+    for (OpNode n : keep)
+        for (OpNode dep : inbound(n)) {
+            if (keep.count(dep) || out.has(dep)) continue;
+            Op producer;
+            producer.kind = OpKind::Producer;
+            producer.shape = shape(dep);
+            // what a kernel boundary stores: the declared type of a Producer, f32 for a reduction, bf16 otherwise
+            const Op& src = get(dep);
+            producer.dtype = src.kind == OpKind::Producer ? src.dtype : src.kind == OpKind::Reduction ? HE_F32 : HE_BF16;
+            out.insert_with_id(dep, producer);
+        }
+    for (OpNode n : keep) out.insert_with_id(n, get(n));  // ids grow along every edge, so this order is topological
+    OpNode fresh = next_;
+    for (OpNode n : keep)
+        for (OpNode user : outbound(n)) {
+            if (keep.count(user)) continue;
+            Op consumer;
+            consumer.kind = OpKind::Consumer;
+            consumer.a = n;
+            consumer.dtype = get(n).kind == OpKind::Reduction ? HE_F32 : HE_BF16;
+            // The reference files the Consumer under the reader's id even when that id is taken (a reader of two of
+            // the nodes, or one that feeds the set again), which loses the earlier entry; an id beyond the graph's
+            // keeps both.
+            out.insert_with_id(out.has(user) ? fresh++ : user, consumer);
+            break;
+        }
+    return out;
 }
 
 const Op& OpGraph::get(OpNode n) const {

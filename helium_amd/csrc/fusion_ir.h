@@ -52,6 +52,10 @@ public:
     const std::vector<OpNode>& outbound(OpNode n) const;
     OpNode anchor() const;  // the Matmul node, or ~0 when there is none
     static Shape3 shape_given_inputs(const Op& op, const OpGraph& g);  // opgraph.rs:386-426
+    // opgraph.rs:96-178: the given nodes with their ids kept; every value they read from outside becomes a
+    // Producer under that value's id, and every node read from outside gets one Consumer, under the id of its first
+    // outside reader.
+    OpGraph subgraph(const std::vector<OpNode>& nodes) const;
 
 private:
     std::map<OpNode, Op> nodes_;

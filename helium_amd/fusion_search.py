@@ -10,6 +10,7 @@ ROLES = ["mainloop", "epilogue", "anchor", "aux"]
 PORTIONS = ["mainloop", "epilogue", "full"]
 
 _ffi._sig("he_fusion_search", C.c_void_p, C.c_int, C.POINTER(C.c_void_p))
+_ffi._sig("he_fusion_search_subdivided", C.c_void_p, C.c_int, C.POINTER(C.c_void_p))
 _ffi._sig("he_fusion_plan_num_fusions", C.c_void_p, C.POINTER(C.c_int))
 _ffi._sig("he_fusion_plan_fusion_info", C.c_void_p, C.c_int, C.POINTER(C.c_int32), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64),
           C.POINTER(C.c_int32), C.c_int, C.POINTER(C.c_int))
@@ -27,10 +28,13 @@ class FusionPlan:
     """minimize_cost_function / produce_maximal_fusions for `graph`. `fusions` lists the kernels in execution
     order: {"core": bool, "anchor": id, "mainloop": [...], "epilogue": [...], "aux": [...]}."""
 
-    def __init__(self, graph, objective=MAXIMAL):
+    def __init__(self, graph, objective=MAXIMAL, subdivided=False):
+        """subdivided: minimize_cost_function_with_subdivision (cost_model.rs:241-259) — every subdivision is
+        searched on its own and the results are merged (fused_graph.rs:910-1058)."""
         self.graph = graph
         self.handle = C.c_void_p()
-        check(lib.he_fusion_search(graph.handle, objective, C.byref(self.handle)))
+        search = lib.he_fusion_search_subdivided if subdivided else lib.he_fusion_search
+        check(search(graph.handle, objective, C.byref(self.handle)))
         n = C.c_int()
         check(lib.he_fusion_plan_num_fusions(self.handle, C.byref(n)))
         self.fusions = []

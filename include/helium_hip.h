@@ -313,6 +313,10 @@ enum { HE_FUSION_ROLE_MAINLOOP = 0, HE_FUSION_ROLE_EPILOGUE = 1, HE_FUSION_ROLE_
 /* objective HE_FUSE_MAXIMAL: produce_maximal_fusions only (fused_graph.rs:113-223); otherwise minimize_cost_function
  * (cost_model.rs:256-343) with the naive model on MI355X rates or the analytical model. */
 int he_fusion_search(he_fgraph_t graph, int objective, he_fusion_plan_t* plan);
+/* minimize_cost_function_with_subdivision (cost_model.rs:241-259): subdivide, search each subdivision's subgraph
+ * (OpGraph::subgraph, opgraph.rs:96-178) on its own, then FusedGraph::merge_from_subdivisions
+ * (fused_graph.rs:910-1058). The plan is used like he_fusion_search's. */
+int he_fusion_search_subdivided(he_fgraph_t graph, int objective, he_fusion_plan_t* plan);
 int he_fusion_plan_num_fusions(he_fusion_plan_t plan, int* count);   /* kernels, in execution order */
 int he_fusion_plan_fusion_info(he_fusion_plan_t plan, int index, int32_t* is_core, uint64_t* anchor, uint64_t* nodes,
                                int32_t* roles, int capacity, int* count);

@@ -155,3 +155,112 @@ def test_random_graphs_keep_the_invariants(seed):
         if seed < 6:
             p.precompile()
     assert costs[fs.MIN_NAIVE_COST] <= costs[fs.MAXIMAL] * (1 + 1e-12)
+
+
+# ---------------------------------------------------------------------------------------------------------
+# Subdivided search: minimize_cost_function_with_subdivision (cost_model.rs:241-259) and
+# FusedGraph::merge_from_subdivisions (fused_graph.rs:910-1058). The reference's one test of the merge
+# (fused_graph.rs:1414-1445) prints the result and asserts only the invariants; the expectations below are worked out by
+# hand: subdivisions meet only at anchors and graph inputs, so merging the separately found optima must give what the
+# search over the whole graph gives wherever that search is exhaustive.
+# ---------------------------------------------------------------------------------------------------------
+def members(plan):
+    return sorted((-1 if f["anchor"] is None else f["anchor"], tuple(sorted(f["mainloop"])), tuple(sorted(f["epilogue"])), tuple(sorted(f["aux"]))) for f in plan.fusions)
+
+
+def test_merge_on_the_graph_of_the_reference_test():
+    """fused_graph.rs:1416-1433: input -> mm1(input, input) -> relu -> add(relu, input) -> Consumer."""
+    g = ha.fusion.OpGraph()
+    inp = g.producer([1, 256, 256])
+    mm1 = g.matmul(inp, inp); relu1 = g.unary(mm1, "relu"); add1 = g.binary(relu1, inp, "add")
+    g.consumer(add1)
+    assert sorted(map(sorted, fs.subdivide(g))) == sorted(map(sorted, [{(mm1, "epilogue"), (relu1, "full"), (add1, "full")},
+                                                                      {(mm1, "mainloop")}]))
+    p = fs.FusionPlan(g, fs.MIN_NAIVE_COST, subdivided=True)
+    assert p.fusions == [{"core": True, "anchor": mm1, "mainloop": [], "epilogue": [relu1, add1], "aux": []}]
+    whole = fs.FusionPlan(g, fs.MIN_NAIVE_COST)
+    assert p.cost() == pytest.approx(whole.cost(), rel=1e-12)
+    p.precompile()
+
+
+def test_merge_joins_the_two_portions_of_an_anchor_found_in_different_subdivisions():
+    """The example of subdivision.rs:120-171 with readers: mm2's mainloop portion is met first (with mm1's epilogue), its
+    epilogue later, with a value (`other`) that only the epilogue reads."""
+    g = ha.fusion.OpGraph()
+    inp = g.producer([1, 256, 256]); other = g.producer([1, 256, 256])
+    mm1 = g.matmul(inp, inp); relu1 = g.unary(mm1, "relu"); add1 = g.binary(relu1, inp, "add")
+    mm2 = g.matmul(mm1, inp); relu2 = g.unary(mm2, "relu"); add2 = g.binary(relu2, other, "add")
+    g.consumer(add1); g.consumer(add2)
+    p = fs.FusionPlan(g, fs.MIN_NAIVE_COST, subdivided=True)
+    assert members(p) == [(mm1, (), (relu1, add1), ()), (mm2, (), (relu2, add2), ())]
+    whole = fs.FusionPlan(g, fs.MIN_NAIVE_COST)
+    assert members(whole) == members(p)
+    assert p.cost() == pytest.approx(whole.cost(), rel=1e-12)
+    p.precompile()
+
+
+def test_merge_keeps_an_unfused_producer_of_a_folded_anchor_connected():
+    """A reduction cannot join a mainloop, so the anchor's mainloop subdivision holds a kernel of its own that feeds the
+    anchor; the anchor's fusion of that subdivision is folded into the one found with its epilogue, and the reduction's
+    kernel must then list the surviving fusion as its reader (the reference's edge update leaves the folded id there,
+    which its own invariant check rejects)."""
+    g = ha.fusion.OpGraph()
+    a = g.producer([1, 128, 128]); w = g.producer([1, 128, 128]); b = g.producer([1, 128, 128])
+    nb = g.unary(b, "neg")   # the lowest op id: its subdivision comes first and reaches the Matmul from the epilogue side
+    r = g.reduction(g.unary(a, "exp"), "rows")
+    x = g.binary(a, g.broadcast(r, 2, 128), "mul")
+    mm = g.matmul(x, w)
+    y = g.binary(mm, nb, "add")
+    g.consumer(y)
+    subs = fs.subdivide(g)
+    assert (mm, "epilogue") in subs[0] and (mm, "mainloop") in subs[1] and (r, "full") in subs[1]
+    p = fs.FusionPlan(g, fs.MIN_NAIVE_COST, subdivided=True)
+    whole = fs.FusionPlan(g, fs.MIN_NAIVE_COST)
+    assert members(p) == members(whole)
+    assert p.cost() == pytest.approx(whole.cost(), rel=1e-12)
+    core = [f for f in p.fusions if f["core"]]
+    assert len(core) == 1 and len(p.fusions) == 2 and p.fusions[-1] is core[0]   # the reduction's kernel runs first
+    assert sorted(core[0]["mainloop"]) == sorted([x, x - 1]) and sorted(core[0]["epilogue"]) == sorted([nb, y])
+    p.precompile()
+
+
+def test_readme_graph_gives_the_same_fusion_when_searched_by_subdivision():
+    from helium_amd import configs
+
+    g, outs = configs.c4_graph(256)
+    for node in outs.values():
+        g.consumer(node, "f32")
+    p = fs.FusionPlan(g, fs.MIN_NAIVE_COST, subdivided=True)
+    whole = fs.FusionPlan(g, fs.MIN_NAIVE_COST)
+    assert members(p) == members(whole) and len(p.fusions) == 1
+    assert p.cost() == pytest.approx(whole.cost(), rel=1e-12)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_graphs_searched_by_subdivision(seed):
+    """Every op lands in a kernel, kernels run after what they read, every kernel lowers, and the merged optimum never
+    costs more than the maximal fusions of the whole graph."""
+    g = random_fusion_graph(seed)
+    if not any(n["op"] == "consumer" for n in g.nodes):
+        pytest.skip("nothing is read")
+    by_id = {n["id"]: n for n in g.nodes}
+    p = fs.FusionPlan(g, fs.MIN_NAIVE_COST, subdivided=True)
+    done = set(n["id"] for n in g.nodes if n["op"] == "producer")
+    for f in p.fusions:
+        inside = set(f["mainloop"] + f["epilogue"] + f["aux"] + ([f["anchor"]] if f["core"] else []))
+        for n in inside:
+            for k in ("a", "b", "x", "lhs", "rhs"):
+                if k in by_id[n] and by_id[n][k] not in inside:
+                    assert by_id[n][k] in done, (f, n)
+        done |= inside
+    live = set()
+    stack = [n["id"] for n in g.nodes if n["op"] == "consumer"]
+    while stack:
+        n = stack.pop()
+        if n in live:
+            continue
+        live.add(n)
+        stack += [by_id[n][k] for k in ("a", "b", "x", "lhs", "rhs") if k in by_id[n]]
+    assert {n for n in live if by_id[n]["op"] not in ("producer", "consumer")} <= done
+    assert p.cost() <= fs.FusionPlan(g, fs.MAXIMAL).cost() * (1 + 1e-12)
+    p.precompile()

@@ -62,10 +62,11 @@ def boundary_values(g, plan):
     return mat
 
 
-@pytest.mark.parametrize("objective", [fs.MAXIMAL, fs.MIN_NAIVE_COST, fs.MIN_ANALYTICAL_COST])
-def test_two_layer_graph_through_the_search(gpu, objective):
+@pytest.mark.parametrize("objective,subdivided", [(fs.MAXIMAL, False), (fs.MIN_NAIVE_COST, False), (fs.MIN_ANALYTICAL_COST, False),
+                                                  (fs.MIN_NAIVE_COST, True), (fs.MIN_ANALYTICAL_COST, True)])
+def test_two_layer_graph_through_the_search(gpu, objective, subdivided):
     g, inputs, outs = two_layer_graph()
-    plan = fs.FusionPlan(g, objective)
+    plan = fs.FusionPlan(g, objective, subdivided=subdivided)
     print(plan.text, flush=True)
     got = run_plan(g, inputs, plan)
     val, _ = oracle.evaluate(g.nodes, inputs, round_mainloop_to="bf16", materialize=boundary_values(g, plan))
@@ -91,3 +92,28 @@ def test_readme_graph_found_by_the_search_matches_the_hand_fed_fusion(gpu):
     for c, node in leaf_of.items():
         a, b = got[c].astype(np.float64), want[node].reshape(-1).astype(np.float64)
         assert np.abs(a - b).max() <= 1e-3 * np.abs(b).max(), (node, float(np.abs(a - b).max()))
+
+
+def test_merged_plan_with_a_kernel_feeding_a_mainloop(gpu):
+    """Searched by subdivision: a row reduction (a kernel of its own) feeds a broadcast that is fused into the Matmul's
+    mainloop, and the Matmul's epilogue reads a value of the other subdivision."""
+    n = 128
+    g = ha.fusion.OpGraph()
+    a = g.producer([1, n, n]); w = g.producer([1, n, n]); b = g.producer([1, n, n])
+    nb = g.unary(b, "neg")
+    r = g.reduction(g.unary(a, "tanh"), "rows")
+    x = g.binary(a, g.broadcast(r, 2, n), "mul")
+    y = g.binary(g.matmul(x, w), nb, "add")
+    out = g.consumer(y, "bf16")
+    rng = np.random.default_rng(3)
+    inputs = {a: configs.bf16_rne((rng.standard_normal((1, n, n)) * 0.3).astype(np.float32)),
+              w: configs.bf16_rne((rng.standard_normal((1, n, n)) * 0.1).astype(np.float32)),
+              b: configs.bf16_rne(rng.standard_normal((1, n, n)).astype(np.float32))}
+    plan = fs.FusionPlan(g, fs.MIN_NAIVE_COST, subdivided=True)
+    print(plan.text, flush=True)
+    assert len(plan.fusions) == 2
+    got = run_plan(g, inputs, plan)
+    val, _ = oracle.evaluate(g.nodes, inputs, round_mainloop_to="bf16", materialize=boundary_values(g, plan))
+    t = nm.bf16_bits_to_f32(got[out]).astype(np.float64)
+    want = val[out].reshape(-1).astype(np.float64)
+    assert (np.abs(t - want) <= 2e-2 * np.maximum(np.abs(want), 0.25)).all(), float(np.abs(t - want).max())
