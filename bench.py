@@ -197,7 +197,7 @@ class LinearLayerWorkload:
         self.work = 2.0 * 256 * 512 * 512
 
     def describe(self):
-        return "C1: f32 X[256,512] W[512,512] + b, relu, column sums via execute_graph (2 kernels)"
+        return "C1: f32 X[256,512] W[512,512] + b, relu, column sums via execute_graph (1 kernel)"
 
     def setup(self):
         from helium_amd import configs
@@ -387,6 +387,237 @@ class ConvWorkload:
         self.tensors, self.last = {}, None
 
 
+class ConvBatchNormWorkload(ConvWorkload):
+    """The first half of a residual block of BASELINE config 5b (resnet-train/src/model.rs): 3x3 convolution ->
+    BatchNorm2d in Train mode -> relu, one graph through execute_graph. The convolution's kernel also folds its output
+    per channel (the batch norm's statistics); two pointwise kernels finish the batch norm. Work = the convolution's
+    FLOP."""
+
+    name = "C5b-conv-bn"
+
+    def describe(self):
+        return "C5b-conv-bn: bf16 [64,56,56,64] conv 3x3 -> 64 channels -> BatchNorm2d train -> relu via execute_graph"
+
+    def setup(self):
+        import helium_amd as ha
+        from helium_amd import configs, frontend
+        from helium_amd.backend import Plan, Tensor
+
+        g = ha.ir.OpGraph()
+        rec = frontend.Recorder(g)
+        c, oc = self.image[3], self.out_channels
+        fshape = [oc, self.kernel[0], self.kernel[1], c]
+        x = g.new_input(list(self.image), "bf16")
+        w = g.new_input(fshape, "bf16")
+        self.params = {"in_channels": c, "out_channels": oc, "kernel_size": list(self.kernel)}
+        conv = g.conv(x, w, self.params)
+        bn = [g.new_input([oc], "f32") for _ in range(4)]
+        y, new_mean, new_var = frontend.batch_norm_train(rec, conv, *bn)
+        self.outs = {"conv": g.new_output(conv), "y": g.new_output(y), "mean": g.new_output(new_mean), "var": g.new_output(new_var)}
+        rng = np.random.default_rng(58)
+        self.host = {x: configs.bf16_rne(rng.standard_normal(self.image, dtype=np.float32)),
+                     w: configs.bf16_rne(rng.standard_normal(fshape, dtype=np.float32) * 0.05),
+                     bn[0]: np.zeros(oc, np.float32), bn[1]: np.ones(oc, np.float32),
+                     bn[2]: rng.uniform(0.5, 1.5, oc).astype(np.float32), bn[3]: rng.standard_normal(oc).astype(np.float32),
+                     **rec.scalars}
+        self.x, self.w, self.bn, self.graph = x, w, bn, g
+        by_id = {n["id"]: n for n in g.nodes}
+        self.tensors = {i: Tensor.from_numpy(a, by_id[i]["dtype"], int(np.prod(by_id[i]["shape"]))) for i, a in self.host.items()}
+        self.last = None
+        log(f"[bench] {self.describe()} :: plan: " + Plan(g).text.replace("\n", " ; "))
+
+    def check(self):
+        """The convolution's first two images against the oracle; statistics and y against the f64 closed form of the
+        batch norm applied to the convolution output the device stored."""
+        from oracle import helium_ir as oracle
+        from oracle import numerics as nm
+
+        oc = self.out_channels
+        img = nm.bf16_bits_to_f32(self.host[self.x]).reshape(self.image)[:2]
+        flt = nm.bf16_bits_to_f32(self.host[self.w]).reshape(oc, *self.kernel, self.image[3])
+        want = oracle.conv(img, flt, self.params, "bf16").astype(np.float64)
+        conv = nm.bf16_bits_to_f32(self.last[self.outs["conv"]].to_numpy()).reshape(-1, oc)
+        got = conv.reshape(self.image[0], -1)[:2].reshape(want.shape).astype(np.float64)
+        if not (np.abs(got - want) <= 1e-2 * np.maximum(np.abs(want), 1.0)).all():
+            raise SystemExit("[bench] PARITY FAILURE in C5b-conv-bn: convolution differs from the oracle")
+        mean = conv.mean(axis=0, dtype=np.float64)
+        var = (conv.astype(np.float64) ** 2).mean(axis=0) - mean ** 2
+        got_mean = self.last[self.outs["mean"]].to_numpy().astype(np.float64)
+        got_var = self.last[self.outs["var"]].to_numpy().astype(np.float64)
+        if not np.allclose(got_mean, 0.1 * mean, rtol=1e-3, atol=1e-4) or not np.allclose(got_var, 0.9 + 0.1 * var, rtol=1e-3, atol=1e-4):
+            raise SystemExit("[bench] PARITY FAILURE in C5b-conv-bn: running statistics differ from the closed form")
+        rows = np.random.default_rng(3).integers(0, conv.shape[0], 4096)
+        scale, bias = self.host[self.bn[2]].astype(np.float64), self.host[self.bn[3]].astype(np.float64)
+        want_y = np.maximum((conv[rows] - mean) / np.sqrt(var + 1e-3) * scale + bias, 0.0)
+        y = nm.bf16_bits_to_f32(self.last[self.outs["y"]].to_numpy()).reshape(-1, oc)[rows].astype(np.float64)
+        if not np.allclose(y, want_y, rtol=2e-2, atol=2e-2):
+            raise SystemExit("[bench] PARITY FAILURE in C5b-conv-bn: y differs from the closed form")
+        return "conv (2 images) within 1e-2 of the oracle; statistics within 1e-3, y (4096 pixels) within 2e-2 of the f64 closed form"
+
+
+class ConvBackwardDataWorkload(ConvWorkload):
+    """The gradient of the same layer with respect to its input (Op::ConvBackwardData): an implicit GEMM whose rows are
+    the image pixels, A the flow gathered through the filter taps, B the filter's [o][r][s][:] rows."""
+
+    name = "C5b-conv-bwd-data"
+
+    def describe(self):
+        return "C5b-conv-bwd-data: bf16 flow [64,56,56,64] x filter [64,3,3,64] -> image gradient via execute_graph (implicit GEMM 200704 x 64 x 576)"
+
+    def setup(self):
+        import helium_amd as ha
+        from helium_amd import configs
+        from helium_amd.backend import Plan, Tensor
+
+        g = ha.ir.OpGraph()
+        n, h, w_, c = self.image
+        fshape = [self.out_channels, self.kernel[0], self.kernel[1], c]
+        dy = g.new_input([n, h, w_, self.out_channels], "bf16")
+        w = g.new_input(fshape, "bf16")
+        self.params = {"in_channels": c, "out_channels": self.out_channels, "kernel_size": list(self.kernel)}
+        self.out = g.new_output(g.conv_backward_data(dy, w, self.params, [h, w_]))
+        rng = np.random.default_rng(54)
+        self.host = {dy: configs.bf16_rne(rng.standard_normal((n, h, w_, self.out_channels), dtype=np.float32)),
+                     w: configs.bf16_rne(rng.standard_normal(fshape, dtype=np.float32) * 0.05)}
+        self.dy, self.w, self.graph = dy, w, g
+        self.tensors = {i: Tensor.from_numpy(a, "bf16", a.size) for i, a in self.host.items()}
+        self.last = None
+        log(f"[bench] {self.describe()} :: plan: " + Plan(g).text.replace("\n", " ; "))
+
+    def check(self):
+        from oracle import helium_ir as oracle
+        from oracle import numerics as nm
+
+        n, h, w_, c = self.image
+        flow = nm.bf16_bits_to_f32(self.host[self.dy]).reshape(n, h, w_, self.out_channels)[:2]
+        flt = nm.bf16_bits_to_f32(self.host[self.w]).reshape(self.out_channels, *self.kernel, c)
+        want = oracle.conv_backward_data(flow, flt, self.params, (h, w_)).astype(np.float64)
+        got = nm.bf16_bits_to_f32(self.last[self.out].to_numpy()).reshape(n, -1)[:2].reshape(want.shape).astype(np.float64)
+        if not (np.abs(got - want) <= 1e-2 * np.maximum(np.abs(want), 1.0)).all():
+            raise SystemExit("[bench] PARITY FAILURE in C5b-conv-bwd-data: output differs from the oracle")
+        return "first two images within 1e-2 of the oracle's float64 adjoint"
+
+
+class ConvBackwardFilterWorkload(ConvWorkload):
+    """The gradient of the same layer with respect to its filter (Op::ConvBackwardFilter): rows = output channels,
+    k = the 200704 output pixels, split over many workgroups per tile whose partial tiles a second launch adds."""
+
+    name = "C5b-conv-bwd-filter"
+
+    def describe(self):
+        return "C5b-conv-bwd-filter: bf16 flow [64,56,56,64] x image [64,56,56,64] -> filter gradient via execute_graph (implicit GEMM 64 x 576 x 200704, split-k)"
+
+    def setup(self):
+        import helium_amd as ha
+        from helium_amd import configs
+        from helium_amd.backend import Plan, Tensor
+
+        g = ha.ir.OpGraph()
+        n, h, w_, c = self.image
+        dy = g.new_input([n, h, w_, self.out_channels], "bf16")
+        x = g.new_input(list(self.image), "bf16")
+        self.params = {"in_channels": c, "out_channels": self.out_channels, "kernel_size": list(self.kernel)}
+        self.out = g.new_output(g.conv_backward_filter(dy, x, self.params))
+        rng = np.random.default_rng(55)
+        self.host = {dy: configs.bf16_rne(rng.standard_normal((n, h, w_, self.out_channels), dtype=np.float32) * 0.05),
+                     x: configs.bf16_rne(rng.standard_normal(self.image, dtype=np.float32))}
+        self.dy, self.x, self.graph = dy, x, g
+        self.tensors = {i: Tensor.from_numpy(a, "bf16", a.size) for i, a in self.host.items()}
+        self.last = None
+        log(f"[bench] {self.describe()} :: plan: " + Plan(g).text.replace("\n", " ; "))
+
+    def check(self):
+        """32 filter taps, each as one float64 dot product over all output pixels (zero padding by slicing)."""
+        from oracle import numerics as nm
+
+        n, h, w_, c = self.image
+        flow = nm.bf16_bits_to_f32(self.host[self.dy]).reshape(n, h, w_, self.out_channels)
+        img = nm.bf16_bits_to_f32(self.host[self.x]).reshape(self.image)
+        got = nm.bf16_bits_to_f32(self.last[self.out].to_numpy()).reshape(self.out_channels, *self.kernel, c).astype(np.float64)
+        rng = np.random.default_rng(56)
+        for _ in range(32):
+            o, r, s_, ch = (int(rng.integers(self.out_channels)), int(rng.integers(self.kernel[0])),
+                            int(rng.integers(self.kernel[1])), int(rng.integers(c)))
+            dr, ds = r - self.kernel[0] // 2, s_ - self.kernel[1] // 2   # image pixel = output pixel + (dr, ds)
+            p0, p1 = max(0, -dr), min(h, h - dr)
+            q0, q1 = max(0, -ds), min(w_, w_ - ds)
+            want = float(np.sum(flow[:, p0:p1, q0:q1, o].astype(np.float64) * img[:, p0 + dr:p1 + dr, q0 + ds:q1 + ds, ch].astype(np.float64)))
+            scale = max(abs(want), 5.0)   # a sum of 200704 products of magnitude 0.05: the bf16 result carries 2^-9 relative
+            if abs(got[o, r, s_, ch] - want) > 1e-2 * scale:
+                raise SystemExit(f"[bench] PARITY FAILURE in C5b-conv-bwd-filter: tap {(o, r, s_, ch)} is {got[o, r, s_, ch]}, want {want}")
+        return "32 sampled taps within 1e-2 of float64 dot products over all 200704 output pixels"
+
+
+class SgdWorkload:
+    """The optimizer step of BASELINE config 5b for one parameter tensor (helium/src/optimizer/sgd.rs:42-66): momentum
+    average and weight update of a bf16 [512,3,3,512] filter (the largest of the network) with its f32 average, one
+    pointwise kernel through execute_graph. Bytes: weights and gradient read as bf16, average read and written as f32,
+    weights written as bf16."""
+
+    bound = "hbm"
+    unit = "GB/s"
+    dtype = "bf16 storage, f32 math"
+    name = "C5b-sgd"
+    wall_timed = True
+    shape = (512, 3, 3, 512)
+
+    def __init__(self):
+        n = int(np.prod(self.shape))
+        self.work = n * (2 + 2 + 4 + 4 + 2)
+
+    def describe(self):
+        return "C5b-sgd: SGD momentum step of a bf16 [512,3,3,512] filter (f32 average) via execute_graph"
+
+    def setup(self):
+        import helium_amd as ha
+        from helium_amd import configs, frontend
+        from helium_amd.backend import Plan, Tensor
+
+        g = ha.ir.OpGraph()
+        rec = frontend.Recorder(g)
+        w = g.new_input(list(self.shape), "bf16")
+        grad = g.new_input(list(self.shape), "bf16")
+        avg = g.new_input(list(self.shape), "f32")
+        new_w, new_avg = frontend.sgd_momentum_step(rec, w, grad, avg, momentum=0.9, learning_rate=0.1)
+        self.out_w, self.out_avg = g.new_output(new_w), g.new_output(new_avg)
+        rng = np.random.default_rng(57)
+        self.host = {w: configs.bf16_rne(rng.standard_normal(self.shape, dtype=np.float32) * 0.05),
+                     grad: configs.bf16_rne(rng.standard_normal(self.shape, dtype=np.float32) * 0.01),
+                     avg: (rng.standard_normal(self.shape, dtype=np.float32) * 0.01), **rec.scalars}
+        self.w, self.grad, self.avg, self.graph = w, grad, avg, g
+        by_id = {n["id"]: n for n in g.nodes}
+        self.tensors = {i: Tensor.from_numpy(a, by_id[i]["dtype"], int(np.prod(by_id[i]["shape"]))) for i, a in self.host.items()}
+        self.last = None
+        log(f"[bench] {self.describe()} :: plan: " + Plan(g).text.replace("\n", " ; "))
+
+    def step(self, stream, i):
+        from helium_amd.backend import execute_graph
+
+        self.last = execute_graph(self.graph, self.tensors)
+
+    def check(self):
+        from oracle import numerics as nm
+
+        w = nm.bf16_bits_to_f32(self.host[self.w]).astype(np.float64).reshape(-1)
+        gr = nm.bf16_bits_to_f32(self.host[self.grad]).astype(np.float64).reshape(-1)
+        av = self.host[self.avg].astype(np.float64).reshape(-1)
+        want_avg = 0.1 * gr + 0.9 * av
+        got_avg = self.last[self.out_avg].to_numpy().astype(np.float64)
+        got_w = nm.bf16_bits_to_f32(self.last[self.out_w].to_numpy()).astype(np.float64)
+        if not np.allclose(got_avg, want_avg, rtol=1e-5, atol=1e-7):
+            raise SystemExit("[bench] PARITY FAILURE in C5b-sgd: momentum average differs from the closed form")
+        want_w = w - 0.1 * want_avg
+        if not (np.abs(got_w - want_w) <= 2.0 ** -8 * np.maximum(np.abs(want_w), 1e-4)).all():
+            raise SystemExit("[bench] PARITY FAILURE in C5b-sgd: weights differ from the closed form")
+        return "average within 1e-5 (f32), weights within one bf16 rounding of the f64 closed form"
+
+    def cpu_baseline(self, budget_s=5.0):
+        return None
+
+    def free(self):
+        self.tensors, self.last = {}, None
+
+
 class FusedGemmWorkload:
     """BASELINE configs 4 / 5a: 4096^3 bf16 GEMM with fused mainloop / epilogue. Work = 2*M*N*K FLOP."""
 
@@ -528,6 +759,10 @@ def make_workloads():
     w["C3"] = AuxChainWorkload()
     w["C5b-bn"] = BatchNormWorkload()
     w["C5b-conv"] = ConvWorkload()
+    w["C5b-conv-bn"] = ConvBatchNormWorkload()
+    w["C5b-conv-bwd-data"] = ConvBackwardDataWorkload()
+    w["C5b-conv-bwd-filter"] = ConvBackwardFilterWorkload()
+    w["C5b-sgd"] = SgdWorkload()
     for name in ("C4", "C5a", "C4m", "GEMM"):
         w[name] = FusedGemmWorkload(name)
     return w

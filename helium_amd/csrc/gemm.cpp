@@ -735,7 +735,7 @@ void validate_gemm_epilogue(const tp::Program& epi) {
     HE_REQUIRE(!epi.outs.empty(), HE_ERR_UNSUPPORTED, "GEMM fusion without an output");
     for (auto& o : epi.outs) {
         HE_REQUIRE(epi.exprs[o.expr].cls == tp::Cls::F, HE_ERR_UNSUPPORTED, "GEMM epilogues store float values");
-        if (o.reduce) HE_REQUIRE(o.rop == tp::ROp::Sum, HE_ERR_UNSUPPORTED, "GEMM epilogues reduce with Sum only");
+        if (o.reduce) HE_REQUIRE((o.rop == tp::ROp::Sum || o.rop == tp::ROp::Mean) && o.dtype == HE_F32, HE_ERR_UNSUPPORTED, "GEMM epilogues reduce with Sum or Mean, into f32");
         else HE_REQUIRE(o.dtype == HE_F32 || o.dtype == HE_BF16 || o.dtype == HE_F16, HE_ERR_UNSUPPORTED, "GEMM epilogues store float tensors");
     }
 }
@@ -797,6 +797,47 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     HE_REQUIRE(t.stages >= 2 && t.stages <= 5 && t.stages * (t.bm + t.bn) * t.bk * (16 / epc) <= 160 * 1024, HE_ERR_INVALID,
                "GEMM tile exceeds LDS");
     const int wtn = t.bn / t.wn;
+    // Reductions of the epilogue never meet in memory: every wave parks its partial result in a workspace (plain
+    // stores) and a second small launch folds the partials of each output element in a fixed order. Float atomics on
+    // the outputs were the alternative: the 2048 waves of a 4096^2 product adding into one scalar cost 12 us of its
+    // launch, and the per-channel sums of a convolution (784 workgroups, 64 columns = two cache lines) 680 us, since
+    // atomics on one line are served one after another.
+    struct RedOut {
+        size_t out;         // index into epi.outs
+        uint64_t off;       // first float of this output's partials
+        int64_t elems;      // output elements
+        int64_t parts;      // partials per element
+        int64_t inner;      // partials of one element lie `inner` floats apart (GN for column sums, else 1)
+    };
+    std::vector<RedOut> reds;
+    const int64_t tiles_m = (pr.M + t.bm - 1) / t.bm, tiles_n = (pr.N + t.bn - 1) / t.bn;
+    uint64_t red_floats = 0;
+    for (size_t oi = 0; oi < pr.epi.outs.size(); oi++) {
+        const tp::Out& o = pr.epi.outs[oi];
+        if (!o.reduce) continue;
+        HE_REQUIRE(pr.split_k == 1, HE_ERR_UNSUPPORTED, "a split k range has no epilogue reductions");
+        RedOut r{oi, red_floats, 0, 0, 1};
+        if (o.fold_m && !o.fold_n) {
+            r.elems = pr.batch * pr.N;
+            r.parts = tiles_m * t.wm;
+            r.inner = pr.N;
+        } else if (o.fold_m && o.fold_n) {
+            HE_REQUIRE(o.b_div >= 1 && pr.batch % o.b_div == 0, HE_ERR_INVALID, "bad batch fold of a reduction");
+            r.elems = pr.batch / o.b_div;
+            r.parts = o.b_div * tiles_m * tiles_n * t.wm * t.wn;
+        } else {
+            r.elems = pr.batch * pr.M;
+            r.parts = tiles_n * t.wn;
+        }
+        HE_REQUIRE(r.elems < (1ll << 31) && r.parts < (1ll << 31), HE_ERR_UNSUPPORTED, "reduction too large");
+        red_floats += (uint64_t)r.elems * r.parts;
+        reds.push_back(r);
+    }
+    auto red_of = [&](size_t oi) -> const RedOut& {
+        for (auto& r : reds)
+            if (r.out == oi) return r;
+        fail(HE_ERR_INTERNAL, "output is not a reduction");
+    };
 
     const bool raw_a = raw_a0, raw_b = raw_b0;
     const int nva = std::min(epc, tp::pick_nv(pr.op_a, 16)), nvb = std::min(epc, tp::pick_nv(pr.op_b, 16));
@@ -848,6 +889,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         for (size_t a = 0; a < pr.args.size(); a++)
             ps << (a ? ", " : "") << (pr.args[a].is_output ? "" : "const ") << tp::c_type(pr.args[a].dtype) << "* __restrict__ p" << a;
         if (pr.split_k > 1) ps << ", float* __restrict__ splitk_ws";
+        if (!reds.empty()) ps << ", float* __restrict__ red_ws";
         s << "#define KERNEL_PARAMS " << ps.str() << "\n";
     }
     // operand fetchers
@@ -970,7 +1012,6 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     for (size_t oi = 0; oi < pr.epi.outs.size(); oi++) {
         const tp::Out& o = pr.epi.outs[oi];
         if (!o.reduce) continue;
-        HE_REQUIRE(o.rop == tp::ROp::Sum, HE_ERR_UNSUPPORTED, "GEMM epilogues reduce with Sum only");
         if (o.fold_m && !o.fold_n)
             setup << "float rc" << oi << "[" << colsets << "][NVE];\n#pragma unroll\nfor (int c = 0; c < " << colsets
                   << "; c++)\n#pragma unroll\nfor (int k = 0; k < NVE; k++) rc" << oi << "[c][k] = 0.0f;\n";
@@ -1009,13 +1050,15 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
             }
         }
         body << "}\n";
-        // per-row sums: combine the lanes that share the row, one atomic per row segment
+        // per-row sums: combine the lanes that share the row; every wave that holds a piece of the row parks its
+        // partial (zero where its columns lie beyond the matrix)
         for (size_t oi = 0; oi < pr.epi.outs.size(); oi++) {
             const tp::Out& o = pr.epi.outs[oi];
             if (!(o.reduce && o.fold_n && !o.fold_m)) continue;
             const int width = std::min(lanes_per_row, 64);
-            body << "{ float r = wave_reduce<0, " << width << ">(rr" << oi << ");\nif ((lane % " << width
-                 << ") == 0 && m < GM && nn < GN) atomicAdd(a" << o.arg << " + (size_t)bz * GM + m, r); }\n";
+            const RedOut& ro = red_of(oi);
+            body << "{ float r = wave_reduce<0, " << width << ">(rr" << oi << ");\nif ((lane % " << width << ") == 0 && m < GM) red_ws[" << ro.off
+                 << "ull + ((size_t)bz * GM + m) * " << ro.parts << "u + tile_n * WAVES_N + wave_n] = r; }\n";
         }
         }
     }
@@ -1028,10 +1071,14 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
                    << oi << "[c][k];\n";
             for (int off = lanes_per_row; off < 64; off *= 2) finish << "r += __shfl_xor(r, " << off << ", 64);\n";
             finish << "const u32 col = ((c * 64 + lane) * NVE) % WTN + k;\nconst u32 nn = n0 + wave_n * WTN + col;\n";
-            finish << "if (lane < " << std::min(lanes_per_row, 64) << " && nn < GN) atomicAdd(a" << o.arg << " + (size_t)bz * GN + nn, r);\n}\n}\n";
+            const RedOut& ro = red_of(oi);
+            finish << "if (lane < " << std::min(lanes_per_row, 64) << " && nn < GN) red_ws[" << ro.off << "ull + ((size_t)bz * " << ro.parts
+                   << "u + tile_m * WAVES_M + wave_m) * GN + nn] = r;\n}\n}\n";
         } else if (o.fold_m && o.fold_n) {
-            finish << "{ float r = wave_reduce<0, 64>(rs" << oi << ");\nif (lane == 0) atomicAdd(a" << o.arg << " + (size_t)(bz / " << o.b_div
-                   << "u), r); }\n";
+            const RedOut& ro = red_of(oi);
+            const int64_t per_b = ro.parts / o.b_div;  // partials per batch index: tiles x waves
+            finish << "{ float r = wave_reduce<0, 64>(rs" << oi << ");\nif (lane == 0) red_ws[" << ro.off << "ull + (size_t)(bz / " << o.b_div << "u) * "
+                   << ro.parts << "u + (size_t)(bz % " << o.b_div << "u) * " << per_b << "u + (tile_m * " << tiles_n << "u + tile_n) * (WAVES_M * WAVES_N) + wave] = r; }\n";
         }
     }
     // splice the generated pieces into the body
@@ -1144,6 +1191,33 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
           << "float acc = 0.0f;\n#pragma unroll 4\nfor (u32 sp = 0; sp < " << pr.split_k << "u; sp++) acc += ws[(size_t)sp * total + i];\n"
           << "float one[1] = {acc};\nst_vec<1>(out + i, one);\n}\n}\n";
     }
+    if (!reds.empty()) {
+        // Second launch: one workgroup folds EB output elements, PG = 256 / EB threads share the partials of each
+        // (thread q takes partials q, q + PG, ...), then one thread adds the PG sums in order: the same order every run.
+        s << "template <int EB, bool CONTIG>\n__device__ __forceinline__ void fold_partials(const float* __restrict__ ws, float* __restrict__ out, u32 n, u32 parts, "
+             "u32 inner, float scale, u32 blk, float* part) {\n"
+             "constexpr int PG = 256 / EB;\nconst u32 tid = threadIdx.x;\n"
+             "const u32 e = CONTIG ? tid / PG : tid % EB, pg = CONTIG ? tid % PG : tid / EB;\nconst u32 j = blk * EB + e;\nfloat acc = 0.0f;\n"
+             "if (j < n) {\nconst float* src = ws + (size_t)(j / inner) * parts * inner + (j % inner);\n#pragma unroll 8\n"
+             "for (u32 p = pg; p < parts; p += PG) acc += src[(size_t)p * inner];\n}\n"
+             "part[e * PG + pg] = acc;\n__syncthreads();\n"
+             "if (pg == 0 && j < n) {\nfloat r = 0.0f;\nfor (int q = 0; q < PG; q++) r += part[e * PG + q];\nout[j] = r * scale;\n}\n}\n";
+        s << "extern \"C\" __global__ __launch_bounds__(256) void fused_matmul_reduce(const float* __restrict__ ws";
+        for (size_t i = 0; i < reds.size(); i++) s << ", float* __restrict__ o" << i;
+        s << ") {\n__shared__ float part[256];\nu32 blk = blockIdx.x;\n";
+        for (size_t i = 0; i < reds.size(); i++) {
+            const RedOut& r = reds[i];
+            const tp::Out& o = pr.epi.outs[r.out];
+            const int eb = r.elems < 16 ? 1 : r.parts >= 512 ? 4 : 16;
+            const uint32_t blocks = (uint32_t)((r.elems + eb - 1) / eb);
+            char scale[64];
+            snprintf(scale, sizeof scale, "%.9ef", o.rop == tp::ROp::Mean ? (float)o.mean_scale : 1.0f);
+            s << "if (blk < " << blocks << "u) { fold_partials<" << eb << ", " << (r.inner == 1 ? "true" : "false") << ">(ws + " << r.off << "ull, o" << i << ", "
+              << r.elems << "u, " << r.parts << "u, " << r.inner << "u, " << scale << ", blk, part); return; }\nblk -= " << blocks << "u;\n";
+            reduce_grid_ += blocks;
+        }
+        s << "}\n";
+    }
     source_ = s.str();
 
     const int64_t tiles = ((pr.M + t.bm - 1) / t.bm) * ((pr.N + t.bn - 1) / t.bn);
@@ -1151,15 +1225,18 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     grid_[0] = (uint32_t)tiles;
     grid_[1] = (uint32_t)(pr.split_k > 1 ? pr.split_k : pr.batch);
     threads_ = (uint32_t)threads;
-    for (auto& o : pr.epi.outs)
-        if (o.reduce) fills_.push_back({pr.map_e[o.arg], 0u});
+    for (auto& r : reds) reduce_outs_.push_back(pr.map_e[pr.epi.outs[r.out].arg]);
+    reduce_floats_ = red_floats;
+    std::string reduce_args;
+    for (int a : reduce_outs_) reduce_args += (reduce_args.empty() ? "" : ",") + std::to_string(a);
     describe_ = strfmt("gemm [%lld,%lld,%lld]x[%lld] tile=%dx%dx%d stages=%d waves=%dx%d threads=%d grid=%ux%u rawA=%d rawB=%d NVA=%d NVB=%d NVE=%d "
-                       "direct=%d%d mma=%s epilogue_exprs=%zu outs=%zu split_k=%d",
+                       "direct=%d%d mma=%s epilogue_exprs=%zu outs=%zu split_k=%d reduce_ws=%llu reduce_grid=%u reduce_args=[%s]",
                        (long long)pr.batch, (long long)pr.M, (long long)pr.K, (long long)pr.N, t.bm, t.bn, t.bk, t.stages, t.wm, t.wn, threads,
                        grid_[0], grid_[1], (int)raw_a, (int)raw_b, nva, nvb, nve, (int)direct_a, (int)direct_b, dtype_name(pr.mma_dtype), pr.epi.exprs.size(),
-                       pr.epi.outs.size(), pr.split_k);
+                       pr.epi.outs.size(), pr.split_k, (unsigned long long)reduce_floats_, reduce_grid_, reduce_args.c_str());
     kernel_.reset(new JitKernel(source_, "fused_matmul", {"-ffp-contract=fast", "-munsafe-fp-atomics"}));
     if (pr.split_k > 1) finalize_.reset(new JitKernel(source_, "fused_matmul_finalize", {"-ffp-contract=fast", "-munsafe-fp-atomics"}));
+    if (reduce_grid_) reduce_.reset(new JitKernel(source_, "fused_matmul_reduce", {"-ffp-contract=fast"}));
 }
 
 GemmKernel::~GemmKernel() { scratch_.release(); }
@@ -1170,16 +1247,13 @@ void GemmKernel::execute(void* const* ptrs, hipStream_t stream) {
         HE_REQUIRE(ptrs[i] != nullptr, HE_ERR_INVALID, "kernel argument %zu is null", i);
         HE_REQUIRE(((uintptr_t)ptrs[i] & 15) == 0, HE_ERR_INVALID, "kernel argument %zu is not 16-byte aligned", i);
     }
-    std::vector<std::pair<void*, std::pair<uint32_t, uint32_t>>> fills;
-    for (auto& f : fills_) {
-        const tp::Arg& a = prob_.args[f.first];
-        fills.push_back({ptrs[f.first], {(uint32_t)(storage_bytes(a.dtype, (size_t)a.numel) / 4), f.second}});
-    }
-    if (!fills.empty()) fill_buffers(fills, stream);
     std::vector<void*> holders(ptrs, ptrs + nargs);
     float* ws = nullptr;
     if (prob_.split_k > 1) {
         ws = scratch_.get((uint64_t)prob_.split_k * prob_.M * prob_.N, 0, stream).floats;
+        holders.push_back(ws);
+    } else if (reduce_floats_) {
+        ws = scratch_.get(reduce_floats_, 0, stream).floats;
         holders.push_back(ws);
     }
     std::vector<void*> argv(holders.size());
@@ -1192,6 +1266,14 @@ void GemmKernel::execute(void* const* ptrs, hipStream_t stream) {
         const uint64_t total = (uint64_t)prob_.M * prob_.N;
         const uint32_t fgrid[3] = {(uint32_t)std::min<uint64_t>((total + 255) / 256, 2048), 1, 1}, fblock[3] = {256, 1, 1};
         finalize_->launch(fgrid, fblock, 0, stream, fargv);
+    }
+    if (reduce_) {
+        std::vector<void*> rh{ws};
+        for (int a : reduce_outs_) rh.push_back(ptrs[a]);
+        std::vector<void*> rargv(rh.size());
+        for (size_t i = 0; i < rh.size(); i++) rargv[i] = &rh[i];
+        const uint32_t rgrid[3] = {reduce_grid_, 1, 1}, rblock[3] = {256, 1, 1};
+        reduce_->launch(rgrid, rblock, 0, stream, rargv.data());
     }
 }
 

@@ -127,10 +127,13 @@ public:
 private:
     GemmProblem prob_;
     std::string source_, describe_;
-    std::unique_ptr<JitKernel> kernel_, finalize_;  // finalize_: adds up the partial tiles of a split-k product
+    // finalize_: adds up the partial tiles of a split-k product; reduce_: folds the partials of the epilogue's reductions
+    std::unique_ptr<JitKernel> kernel_, finalize_, reduce_;
     uint32_t grid_[3] = {1, 1, 1};
     uint32_t threads_ = 256;
-    std::vector<std::pair<int, uint32_t>> fills_;
+    uint32_t reduce_grid_ = 0;
+    uint64_t reduce_floats_ = 0;
+    std::vector<int> reduce_outs_;  // kernel arguments the reduce launch writes, in its parameter order
     ReduceScratch scratch_;
 };
 

@@ -138,7 +138,10 @@ class PointwiseLowering {
 public:
     // With `anchor` set the subgraph is a Matmul plus the ops that follow it: the program is the epilogue, iterates
     // over the Matmul's output and reads the anchor's value as the accumulator.
-    explicit PointwiseLowering(const ir::OpSubgraph& sg, ir::NodeId anchor = ir::kNoNode) : sg_(sg), g_(*sg.graph()), anchor_(anchor) {}
+    // `row_dims` > 1: the anchor's leading `row_dims` dims together are the rows of the product (the n, p, q of a
+    // convolution's NHWC output) and are merged into one dim once the program is built.
+    explicit PointwiseLowering(const ir::OpSubgraph& sg, ir::NodeId anchor = ir::kNoNode, size_t row_dims = 1)
+        : sg_(sg), g_(*sg.graph()), anchor_(anchor), row_dims_(row_dims) {}
 
     Program run() {
         HE_REQUIRE(!sg_.leafs().empty(), HE_ERR_INVALID, "pointwise subgraph has no output");
@@ -170,23 +173,43 @@ public:
                 HE_REQUIRE(ir::num_elements(rs) == numel, HE_ERR_UNSUPPORTED,
                            "reduction input has a different element count than the other outputs");
                 Shape rdims = rs.empty() ? Shape{1} : rs;
-                HE_REQUIRE(rdims == p_.dims, HE_ERR_UNSUPPORTED, "all reductions of a kernel must share one input shape");
                 const size_t rank = rdims.size();
                 const size_t depth = n.op.depth;
                 HE_REQUIRE(depth >= 1 && depth <= rank, HE_ERR_INVALID, "bad reduce depth");
                 o.reduce = true;
                 o.rop = (ROp)n.op.sub_op;
-                o.fold_n = true;
-                o.fold_m = depth >= 2;
-                o.b_div = 1;
-                for (size_t k = rank - depth; k + 2 < rank; k++) o.b_div *= rdims[k];
                 int64_t group = 1;
                 for (size_t k = rank - depth; k < rank; k++) group *= rdims[k];
                 o.mean_scale = 1.0 / (double)group;
-                out_depth_.resize(p_.outs.size() + 1, 0);
-                out_depth_[p_.outs.size()] = depth;
                 o.dtype = HE_F32;
-                o.expr = eval(n.op.inputs[0], ident);
+                // In an epilogue the Reduce's index space may be the product's with its dims permuted (SwapDims + Reduce:
+                // column sums, BatchNorm2d statistics of a convolution's output) even where the two shapes are equal
+                // (a square product), so the plain reading is only tried first there.
+                bool plain = rdims == p_.dims && (row_dims_ <= 1 || depth == 1 || depth == rank);
+                if (plain) {
+                    o.fold_n = true;
+                    o.fold_m = depth >= 2;
+                    o.b_div = 1;
+                    for (size_t k = rank - depth; k + 2 < rank; k++) o.b_div *= rdims[k];
+                    if (row_dims_ > 1) o.b_div = 1;  // all of the rows fold, or none
+                    out_depth_.resize(p_.outs.size() + 1, 0);
+                    out_depth_[p_.outs.size()] = depth;
+                    const size_t exprs = p_.exprs.size(), memo = memo_.size();
+                    const int acc = p_.acc_expr;
+                    try {
+                        o.expr = eval(n.op.inputs[0], ident);
+                    } catch (const Error&) {
+                        if (anchor_ == ir::kNoNode) throw;
+                        p_.exprs.resize(exprs);
+                        memo_.resize(memo);
+                        p_.acc_expr = acc;
+                        plain = false;
+                    }
+                }
+                if (!plain) {
+                    HE_REQUIRE(anchor_ != ir::kNoNode, HE_ERR_UNSUPPORTED, "all reductions of a kernel must share one input shape");
+                    lower_permuted_reduction(n, rdims, depth, o);
+                }
                 HE_REQUIRE(p_.exprs[o.expr].cls == Cls::F, HE_ERR_UNSUPPORTED, "reductions take float operands");
                 p_.args.push_back({HE_F32, ir::num_elements(n.desc.shape), true, leaf});
             } else {
@@ -198,12 +221,92 @@ public:
             }
             p_.outs.push_back(o);
         }
-        if (anchor_ != ir::kNoNode) drop_unused_inputs();
-        else fold_leading_dims_as_columns();
+        if (anchor_ != ir::kNoNode) {
+            drop_unused_inputs();
+            merge_row_dims();
+        } else {
+            fold_leading_dims_as_columns();
+        }
         return std::move(p_);
     }
 
 private:
+    bool reads_anchor(ir::NodeId node) const {
+        if (node == anchor_) return true;
+        if (sg_.is_input(node) || !sg_.contains(node)) return false;
+        for (ir::NodeId in : g_.get(node).op.inputs)
+            if (reads_anchor(in)) return true;
+        return false;
+    }
+
+    // Reduce leaf of an epilogue whose input shape `rdims` is a permutation of the iteration dims. Extents may repeat
+    // (a square product), so every matching permutation is tried: the right one is the one under which the path back
+    // to the anchor arrives with the identity mapping.
+    void lower_permuted_reduction(const ir::Node& n, const Shape& rdims, size_t depth, Out& o) {
+        const size_t R = p_.dims.size();
+        HE_REQUIRE(rdims.size() == R && reads_anchor(n.op.inputs[0]), HE_ERR_UNSUPPORTED,
+                   "reduction input is not a permutation of the Matmul result");
+        const Shape rst = ir::packed_strides(rdims);
+        std::vector<size_t> perm(R);  // perm[j]: the iteration dim that the Reduce's dim j walks
+        for (size_t j = 0; j < R; j++) perm[j] = j;
+        bool done = false;
+        do {
+            bool fits = true;
+            for (size_t j = 0; j < R; j++) fits = fits && rdims[j] == p_.dims[perm[j]];
+            if (!fits) continue;
+            Mapping mp;
+            mp.w.assign(R, 0);
+            for (size_t j = 0; j < R; j++) mp.w[perm[j]] = rst[j];
+            const size_t exprs = p_.exprs.size(), memo = memo_.size();
+            const int acc = p_.acc_expr;
+            try {
+                o.expr = eval(n.op.inputs[0], mp);
+                done = true;
+            } catch (const Error&) {
+                p_.exprs.resize(exprs);
+                memo_.resize(memo);
+                p_.acc_expr = acc;
+            }
+        } while (!done && std::next_permutation(perm.begin(), perm.end()));
+        HE_REQUIRE(done, HE_ERR_UNSUPPORTED, "the reduction reads the Matmul result through more than a permutation of its dims");
+        HE_REQUIRE(p_.exprs[o.expr].cls == Cls::F, HE_ERR_UNSUPPORTED, "reductions take float operands");
+        // which of [batch.., rows, cols] the folded dims are
+        const size_t rows_first = row_dims_ > 1 ? 0 : R - 2, cols = R - 1;
+        size_t rows_folded = 0, rows_total = R >= 2 ? cols - rows_first : 0;
+        bool cols_folded = false;
+        for (size_t j = R - depth; j < R; j++) {
+            const size_t d = perm[j];
+            if (d == cols) cols_folded = true;
+            else if (R >= 2 && d >= rows_first) rows_folded++;
+            else fail(HE_ERR_UNSUPPORTED, "a reduction over the batch dim of a product is not fused");
+        }
+        HE_REQUIRE(rows_folded == 0 || rows_folded == rows_total, HE_ERR_UNSUPPORTED, "the reduction folds part of the product's rows");
+        o.fold_n = cols_folded;
+        o.fold_m = rows_folded != 0;
+        o.b_div = 1;
+        // the kept dims keep their order, so that the output is indexed like the product with the folded dims dropped
+        size_t last = 0;
+        for (size_t j = 0; j + depth < R; j++) {
+            HE_REQUIRE(j == 0 || perm[j] > last, HE_ERR_UNSUPPORTED, "the reduction's kept dims are permuted");
+            last = perm[j];
+        }
+    }
+
+    // A convolution's epilogue is lowered over [n, p, q, channels]; the product's rows are (n, p, q) together.
+    void merge_row_dims() {
+        while (row_dims_ > 1) {
+            for (auto& e : p_.exprs)
+                if (e.kind == Expr::Load)
+                    HE_REQUIRE(e.access.chain.empty() && e.access.stride[0] == e.access.stride[1] * p_.dims[1], HE_ERR_UNSUPPORTED,
+                               "an epilogue operand does not walk the product's rows as one dim");
+            p_.dims[1] *= p_.dims[0];
+            p_.dims.erase(p_.dims.begin());
+            for (auto& e : p_.exprs)
+                if (e.kind == Expr::Load) e.access.stride.erase(e.access.stride.begin());
+            row_dims_--;
+        }
+    }
+
     // helium-ir's Reduce folds trailing dims only, so a reduction over leading dims reaches the kernel as
     // SwapDims + Reduce (BatchNorm2d statistics over N, H, W of an NHWC tensor, helium/src/modules/batch_norm.rs:38-46;
     // column sums). Iterated in the Reduce's own index space, the innermost coordinate then strides through memory.
@@ -417,6 +520,7 @@ private:
     const ir::OpSubgraph& sg_;
     const ir::OpGraph& g_;
     ir::NodeId anchor_;
+    size_t row_dims_ = 1;
     Program p_;
     std::map<ir::NodeId, int> input_arg_;
     std::vector<Memo> memo_;
@@ -703,7 +807,9 @@ bool pointwise_supports(const ir::OpSubgraph& sg) {
 }
 
 Program lower_pointwise(const ir::OpSubgraph& sg) { return PointwiseLowering(sg).run(); }
-Program lower_ir_epilogue(const ir::OpSubgraph& sg, ir::NodeId anchor) { return PointwiseLowering(sg, anchor).run(); }
+Program lower_ir_epilogue(const ir::OpSubgraph& sg, ir::NodeId anchor, size_t row_dims) {
+    return PointwiseLowering(sg, anchor, row_dims).run();
+}
 Program lower_aux(const fir::OpGraph& g) {
     HE_REQUIRE(g.anchor() == fir::kNoOpNode, HE_ERR_INVALID, "an auxiliary fusion holds no Matmul");
     return FusionLowering(g, fir::kNoOpNode).run();

@@ -335,6 +335,27 @@ std::shared_ptr<const Plan> generate_plan(const std::shared_ptr<const ir::OpGrap
         }
     }
 
+    // Beyond the reference, with the epilogue option on: the greedy pass visits a product before the pointwise group
+    // that reduces it has formed (a SwapDims alone is no epilogue; SwapDims + Reduce is a column reduction), so
+    // products are offered their finished pointwise dependents once more.
+    if (fuse_matmul_epilogue()) {
+        for (bool changed = true; changed;) {
+            changed = false;
+            for (auto& kv : ig.instrs) {
+                if (kv.second->kind() != InstrKind::Gemm) continue;
+                const uint64_t cur = kv.first;
+                std::vector<uint64_t> nexts(ig.dependents.at(cur).begin(), ig.dependents.at(cur).end());
+                for (uint64_t nxt : nexts)
+                    if (ig.instrs.at(nxt)->kind() == InstrKind::Pointwise && ig.can_fuse(cur, nxt)) {
+                        ig.fuse(cur, nxt);
+                        changed = true;
+                        break;
+                    }
+                if (changed) break;  // the map changed under the loop
+            }
+        }
+    }
+
     // generate_plan_from_graph (:275-321): Kahn levels
     auto plan = std::make_shared<Plan>();
     {
@@ -478,8 +499,8 @@ namespace {
 // filter [out_channels, kh, kw, in_channels] is B with k contiguous; A is gathered from the NHWC image on the fly.
 GemmProblem conv_problem(const ir::OpSubgraph& sg, NodeId conv) {
     const ir::OpGraph& g = *sg.graph();
-    HE_REQUIRE(sg.nodes().size() == 1, HE_ERR_UNSUPPORTED, "a convolution instruction holds the Conv alone");
     const ir::Op& op = g.get(conv).op;
+    HE_REQUIRE(sg.is_input(op.inputs[0]) && sg.is_input(op.inputs[1]), HE_ERR_UNSUPPORTED, "a convolution reads materialised operands");
     const ir::Descriptor &image = g.get(op.inputs[0]).desc, &filter = g.get(op.inputs[1]).desc, &out = g.get(conv).desc;
     HE_REQUIRE(dtype_class(image.dtype) == DataClass::Float && filter.dtype == image.dtype, HE_ERR_UNSUPPORTED,
                "conv takes a float image and a filter of the same type");
@@ -519,6 +540,16 @@ GemmProblem conv_problem(const ir::OpSubgraph& sg, NodeId conv) {
     operand(pr.op_b, filter, op.inputs[1], pr.N, pr.K);  // [n][k]: k contiguous
     pr.b_nk = true;
     pr.root_a = pr.root_b = 0;
+    if (sg.nodes().size() > 1) {
+        // Conv + the pointwise / reduce ops after it (beyond the reference, whose convolution instruction never
+        // fuses): the epilogue runs on the accumulators, over [n, p, q, channels] with (n, p, q) as the rows. The
+        // partial tiles of a split k range could not run it, so the k range stays whole.
+        pr.split_k = 1;
+        pr.epi = tp::lower_ir_epilogue(sg, conv, 3);
+        validate_gemm_epilogue(pr.epi);
+        assemble_gemm_args(pr);
+        return pr;
+    }
     pr.epi.dims = {1, pr.M, pr.N};
     pr.epi.fast_math = true;
     tp::Expr acc;

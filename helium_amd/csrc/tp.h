@@ -96,7 +96,9 @@ struct Program {
 Program lower_pointwise(const ir::OpSubgraph& sg);
 // A Matmul node (`anchor`) and the pointwise / reduce ops downstream of it -> the GEMM epilogue program over the
 // Matmul's output shape. Throws HE_ERR_UNSUPPORTED when the ops cannot run on the accumulator in place.
-Program lower_ir_epilogue(const ir::OpSubgraph& sg, ir::NodeId anchor);
+// `row_dims`: how many leading dims of the anchor's output form the rows of the product (3 for a convolution's
+// [n, p, q, channels]); they end up merged into one dim.
+Program lower_ir_epilogue(const ir::OpSubgraph& sg, ir::NodeId anchor, size_t row_dims = 1);
 // supports_subgraph of helium/src/cuda/instr/pointwise.rs:121-186.
 bool pointwise_supports(const ir::OpSubgraph& sg);
 

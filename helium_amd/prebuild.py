@@ -35,6 +35,36 @@ def prebuild_kernels(verbose=True):
         g.new_output(v)
     Plan(g).precompile()
     n += 2
+    # one residual-block convolution and its two gradients, and the optimizer step of the largest filter
+    conv = {"in_channels": 64, "out_channels": 64, "kernel_size": [3, 3]}
+    for which in ("forward", "data", "filter"):
+        g = ir.OpGraph()
+        a = g.new_input([64, 56, 56, 64], "bf16")
+        if which == "forward":
+            out = g.conv(a, g.new_input([64, 3, 3, 64], "bf16"), conv)
+        elif which == "data":
+            out = g.conv_backward_data(a, g.new_input([64, 3, 3, 64], "bf16"), conv, [56, 56])
+        else:
+            out = g.conv_backward_filter(a, g.new_input([64, 56, 56, 64], "bf16"), conv)
+        g.new_output(out)
+        Plan(g).precompile()
+        n += 1
+    g = ir.OpGraph()
+    rec = frontend.Recorder(g)
+    out = g.conv(g.new_input([64, 56, 56, 64], "bf16"), g.new_input([64, 3, 3, 64], "bf16"), conv)
+    g.new_output(out)
+    for v in frontend.batch_norm_train(rec, out, *[g.new_input([64], "f32") for _ in range(4)]):
+        g.new_output(v)
+    Plan(g).precompile()
+    n += 1
+    g = ir.OpGraph()
+    rec = frontend.Recorder(g)
+    shape = [512, 3, 3, 512]
+    new_w, new_avg = frontend.sgd_momentum_step(rec, g.new_input(shape, "bf16"), g.new_input(shape, "bf16"), g.new_input(shape, "f32"))
+    g.new_output(new_w)
+    g.new_output(new_avg)
+    Plan(g).precompile()
+    n += 1
     if verbose:
         print(f"prebuilt {n + 1} kernels in {time.time() - t0:.1f}s")
     return n + 1

@@ -219,6 +219,25 @@ def generate_plan(nodes, gemm_epilogue=None):
                 work.add(new)
                 break
 
+    if gemm_epilogue is not None:
+        # the backend's second look: every product is offered its finished pointwise dependents again (a SwapDims
+        # alone is no epilogue, SwapDims + Reduce is a column reduction), until nothing merges
+        changed = True
+        while changed:
+            changed = False
+            for cur in sorted(ig.instrs):
+                if ig.instrs[cur].kind != "gemm":
+                    continue
+                for nxt in sorted(ig.dependents[cur]):
+                    if (ig.instrs[nxt].kind == "pointwise" and ig.instrs[cur].can_fuse_with(ig.instrs[nxt], gemm_epilogue)
+                            and not ig.exist_multiple_paths(cur, nxt)):
+                        a, b = ig.remove(cur), ig.remove(nxt)
+                        ig.insert(a.merged(b), slot=nxt)
+                        changed = True
+                        break
+                if changed:
+                    break
+
     total = len(ig.instrs)
     indeg, stack = {}, []
     for s in sorted(ig.instrs):

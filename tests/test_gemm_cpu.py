@@ -14,6 +14,28 @@ import gemm_cases
 from cpu_emul import run_kernel
 
 
+def launch_gemm(k, bufs):
+    """Runs a fused-GEMM kernel object on the CPU as its host side launches it: `fused_matmul`, then, when the
+    epilogue reduces, `fused_matmul_reduce` over the partial results the first launch parked in the workspace (which
+    starts as NaN here, so a partial that no wave wrote shows). bufs: one (array, mode) per kernel argument.
+    Returns the arrays of the output arguments, in argument order."""
+    gx, gy = map(int, re.search(r"grid=(\d+)x(\d+)", k.description).groups())
+    threads = int(re.search(r"threads=(\d+)", k.description).group(1))
+    ws_floats, reduce_grid = map(int, re.search(r"reduce_ws=(\d+) reduce_grid=(\d+)", k.description).groups())
+    if not reduce_grid:
+        return run_kernel(k.source, "fused_matmul", gx, threads, bufs, grid_y=gy)
+    res = run_kernel(k.source, "fused_matmul", gx, threads, bufs + [(np.full(ws_floats, np.nan, dtype=np.float32), 2)], grid_y=gy)
+    ws, res = res[-1], res[:-1]
+    out_args = [i for i, a in enumerate(k.args) if a["is_output"]]
+    # the reduce launch takes the reduction outputs in the order the description lists their kernel arguments
+    listed = re.search(r"reduce_args=\[([\d,]*)\]", k.description).group(1)
+    reduced = [out_args.index(int(i)) for i in listed.split(",")]
+    folded = run_kernel(k.source, "fused_matmul_reduce", reduce_grid, 256, [(ws, 0)] + [(res[j], 1) for j in reduced])
+    for j, r in zip(reduced, folded):
+        res[j] = r
+    return res
+
+
 def run_emulated(g, inputs, tile, env=()):
     os.environ["HELIUM_HIP_GEMM_TILE"] = tile
     for name in env:
@@ -24,13 +46,11 @@ def run_emulated(g, inputs, tile, env=()):
         del os.environ["HELIUM_HIP_GEMM_TILE"]
         for name in env:
             del os.environ[name]
-    gx, gy = map(int, re.search(r"grid=(\d+)x(\d+)", k.description).groups())
-    threads = int(re.search(r"threads=(\d+)", k.description).group(1))
     bufs = []
     for a in k.args:
         dt = nm.NP_STORAGE[a["dtype"]]
         bufs.append((np.zeros(a["numel"], dtype=dt), 2) if a["is_output"] else (inputs[a["node"]], 0))
-    res = run_kernel(k.source, "fused_matmul", gx, threads, bufs, grid_y=gy)
+    res = launch_gemm(k, bufs)
     outs = [a for a in k.args if a["is_output"]]
     return k, {a["node"]: (r, a["dtype"]) for a, r in zip(outs, res)}
 
@@ -174,7 +194,7 @@ def run_ir_kernel_on_cpu(g, nodes, inputs):
         (out,) = outs
         res = run_kernel(k.source, "fused_matmul_finalize", 2, 256, [(res[-1], 0), (np.zeros(out["numel"], dtype=nm.NP_STORAGE[out["dtype"]]), 1)])
     else:
-        res = run_kernel(k.source, "fused_matmul", gx, threads, bufs, grid_y=gy)
+        res = launch_gemm(k, bufs)
     return k, {a["node"]: nm.from_storage(r, a["dtype"], [r.size]).astype(np.float64) for a, r in zip(outs, res)}
 
 
@@ -362,3 +382,67 @@ def test_ir_matmul_with_transposed_operands_on_cpu(dtype, precision, tol):
             del os.environ["HELIUM_HIP_GEMM_TILE"]
         want = val[out].reshape(-1).astype(np.float64)
         assert np.abs(got[out] - want).max() <= tol * max(1.0, np.abs(want).max()), (k.description, np.abs(got[out] - want).max())
+
+
+# ---- reductions over leading dims of the product (SwapDims + Reduce) in the epilogue ------------------------------
+@pytest.mark.parametrize("m,n,k", [(40, 72, 24), (48, 48, 16)])
+def test_ir_matmul_with_column_sums_on_cpu(m, n, k):
+    """Config 1 whole: relu(X W + b) and its column sums, which helium-ir writes as SwapDims + Reduce, in one fused
+    GEMM. The square case has a Reduce input of the product's own shape: only the path back to the Matmul tells which
+    dim is folded."""
+    from helium_amd import configs
+    from oracle import helium_ir as oracle_ir
+
+    g, names = configs.c1_ir_graph(m, k, n)
+    host = configs.c1_inputs(names, m, k, n, batched=False)
+    ops = [nd["id"] for nd in g.nodes if nd["node"] == "op"]
+    kern, got = run_ir_kernel_on_cpu(g, ops, host)
+    val, _ = oracle_ir.evaluate(g.nodes, host)
+    outs = {nd["from"] for nd in g.nodes if nd["node"] == "output"}
+    assert set(got) == outs and len(outs) == 2
+    for node in outs:
+        want = val[node].reshape(-1)
+        assert got[node].shape == want.shape
+        assert np.abs(got[node] - want).max() <= 1e-4 * max(1.0, np.abs(want).max()), (node, kern.description)
+
+
+def test_ir_conv_with_batch_norm_statistics_on_cpu():
+    """A convolution with the per-channel mean of its output and of its square (BatchNorm2d's statistics: SwapDims of
+    batch and channel dims, Reduce over the three trailing dims) as one implicit GEMM; batch = channels, so the
+    Reduce's input has the output's own shape."""
+    from helium_amd import frontend
+    from oracle import helium_ir as oracle_ir
+
+    rng = np.random.default_rng(21)
+    g = ha.ir.OpGraph()
+    rec = frontend.Recorder(g)
+    x = g.new_input([8, 6, 5, 16], "bf16"); w = g.new_input([8, 3, 3, 16], "bf16")
+    y = g.conv(x, w, {"in_channels": 16, "out_channels": 8, "kernel_size": [3, 3]})
+    yt = g.swap_dims(y, 0, 3)
+    mean = g.reduce(yt, "mean", 3)
+    mean_sq = g.reduce(rec.pow_scalar(yt, 2.0), "mean", 3)
+    for v in (y, mean, mean_sq):
+        g.new_output(v)
+    host = {x: nm.to_storage(rng.standard_normal((8, 6, 5, 16)).astype(np.float32), "bf16"),
+            w: nm.to_storage((rng.standard_normal((8, 3, 3, 16)) * 0.2).astype(np.float32), "bf16"), **rec.scalars}
+    ops = [nd["id"] for nd in g.nodes if nd["node"] == "op"]
+    kern, got = run_ir_kernel_on_cpu(g, ops, host)
+    val, desc = oracle_ir.evaluate(g.nodes, host)
+    want_y = val[y].reshape(-1)
+    assert np.abs(got[y] - want_y).max() <= 1e-2 * max(1.0, np.abs(want_y).max()), kern.description
+    for node in (mean, mean_sq):
+        want = val[node].reshape(-1)
+        assert got[node].shape == want.shape
+        assert np.abs(got[node] - want).max() <= 2e-3 * max(1.0, np.abs(want).max()), (node, got[node], want)
+
+
+def test_epilogue_refuses_what_it_cannot_reduce():
+    """Part of the rows (one image dim of a convolution), or a reduction that keeps its dims in another order, stays a
+    kernel of its own."""
+    g = ha.ir.OpGraph()
+    x = g.new_input([4, 6, 5, 16], "bf16"); w = g.new_input([8, 3, 3, 16], "bf16")
+    y = g.conv(x, w, {"in_channels": 16, "out_channels": 8, "kernel_size": [3, 3]})
+    r = g.reduce(g.swap_dims(y, 2, 3), "sum", 1)   # folds q only
+    g.new_output(y); g.new_output(r)
+    with pytest.raises(ha.HeliumError):
+        ha.backend.matmul_kernel(g, [nd["id"] for nd in g.nodes if nd["node"] == "op"])

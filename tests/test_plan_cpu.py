@@ -163,13 +163,18 @@ def test_random_graphs_match_the_restatement(reference_grouping, seed):
 
 def test_matmul_takes_the_ops_that_can_run_on_its_accumulators():
     # default grouping of this backend. Worked out by hand: the matmul (slot 1) takes the add, the bias broadcast
-    # (slot 2) then joins as an epilogue operand, the relu follows; the swap cannot run in place on accumulators and
-    # starts the second kernel, which takes the reduction.
+    # (slot 2) then joins as an epilogue operand, the relu follows; the swap alone cannot run on accumulators and
+    # starts a second instruction, which takes the reduction; swap + reduce together are a column reduction of the
+    # product, so the second look at the product's dependents merges the two instructions.
     g, _ = linear_layer()
-    want = [([("gemm", [3, 4, 5, 6])], []), ([("pointwise", [7, 8])], [0, 1, 2]), ([], [])]
+    want = [([("gemm", [3, 4, 5, 6, 7, 8])], []), ([], [0, 1, 2])]
     assert Plan(g).steps == want
-    in_place = lambda instr: not any(instr.g.nodes[n]["op"] == "swap_dims" for n in instr.nodes)  # noqa: E731
-    assert oracle_plan.generate_plan(g.nodes, gemm_epilogue=in_place) == want
+
+    def runs_on_accumulators(instr):
+        ops = [instr.g.nodes[n]["op"] for n in instr.nodes]
+        return ops.count("swap_dims") == ops.count("reduce")   # a transposition only together with its reduction
+
+    assert oracle_plan.generate_plan(g.nodes, gemm_epilogue=runs_on_accumulators) == want
 
 
 def test_ops_feeding_a_matmul_operand_stay_outside_it():
@@ -230,6 +235,28 @@ def test_batch_norm_reference_plan_has_the_permute(reference_grouping):
     assert [k for k, _ in steps[0][0]] == ["permute"]
     assert sorted(k for k, _ in steps[1][0]) == ["pointwise", "pointwise"]  # the two statistics read xt separately
     assert oracle_plan.generate_plan(g.nodes) == steps
+
+
+def test_batch_norm_statistics_join_the_convolution_that_feeds_them():
+    """conv -> BatchNorm2d (a resnet block's first half): the per-channel means of y and y^2 are column reductions of the
+    implicit GEMM, so the convolution's instruction takes the SwapDims, the square and both reductions; the rest of
+    the batch norm needs the finished statistics and stays outside."""
+    from helium_amd import frontend
+
+    g = ha.ir.OpGraph()
+    rec = frontend.Recorder(g)
+    x = g.new_input([64, 56, 56, 64], "bf16"); w = g.new_input([64, 3, 3, 64], "bf16")
+    conv = g.conv(x, w, {"in_channels": 64, "out_channels": 64, "kernel_size": [3, 3]})
+    outs = frontend.batch_norm_train(rec, conv, *[g.new_input([64], "f32") for _ in range(4)])
+    for v in outs:
+        g.new_output(v)
+    steps = Plan(g).steps
+    kind, members = steps[0][0][0]
+    by_id = {n["id"]: n for n in g.nodes}
+    assert kind == "gemm" and len(steps[0][0]) == 1
+    assert sorted(by_id[m]["op"] for m in members) == ["binary", "broadcast", "conv", "reduce", "reduce", "swap_dims"]
+    assert all(k == "pointwise" for instrs, _ in steps[1:] for k, _ in instrs)
+    check_invariants(g, steps)
 
 
 def linear_backward_graph(rows=64, inner=96, cols=80, dtype="f32", precision="f32_f32"):
