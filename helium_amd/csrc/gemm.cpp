@@ -344,8 +344,9 @@ __device__ __forceinline__ void direct_tile(const unsigned char* __restrict__ rd
 #endif
 
 #ifndef KERNEL_ATTRS
-/* NWAVES / 4 waves per SIMD: with four waves each one owns the full 512-register budget */
-#define KERNEL_ATTRS __attribute__((amdgpu_waves_per_eu(NWAVES / 4, NWAVES / 4)))
+/* NWAVES / 4 waves per SIMD and workgroup: with four waves each one owns the full 512-register budget; WGS_PER_CU
+   workgroups are meant to share a CU */
+#define KERNEL_ATTRS __attribute__((amdgpu_waves_per_eu(NWAVES / 4 * WGS_PER_CU, NWAVES / 4 * WGS_PER_CU)))
 #endif
 extern "C" __global__ __launch_bounds__(NTHREADS) KERNEL_ATTRS
 void fused_matmul(KERNEL_PARAMS) {
@@ -797,8 +798,9 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     HE_REQUIRE(t.stages >= 2 && t.stages <= 5 && t.stages * (t.bm + t.bn) * t.bk * (16 / epc) <= 160 * 1024, HE_ERR_INVALID,
                "GEMM tile exceeds LDS");
     const int wtn = t.bn / t.wn;
-    // Reductions of the epilogue never meet in memory: every wave parks its partial result in a workspace (plain
-    // stores) and a second small launch folds the partials of each output element in a fixed order. Float atomics on
+    // Reductions of the epilogue never meet in memory: every workgroup (for row sums: every wave) parks its partial
+    // result in a workspace (plain stores) and a second small launch folds the partials of each output element in a
+    // fixed order. Float atomics on
     // the outputs were the alternative: the 2048 waves of a 4096^2 product adding into one scalar cost 12 us of its
     // launch, and the per-channel sums of a convolution (784 workgroups, 64 columns = two cache lines) 680 us, since
     // atomics on one line are served one after another.
@@ -819,12 +821,12 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         RedOut r{oi, red_floats, 0, 0, 1};
         if (o.fold_m && !o.fold_n) {
             r.elems = pr.batch * pr.N;
-            r.parts = tiles_m * t.wm;
+            r.parts = tiles_m;
             r.inner = pr.N;
         } else if (o.fold_m && o.fold_n) {
             HE_REQUIRE(o.b_div >= 1 && pr.batch % o.b_div == 0, HE_ERR_INVALID, "bad batch fold of a reduction");
             r.elems = pr.batch / o.b_div;
-            r.parts = o.b_div * tiles_m * tiles_n * t.wm * t.wn;
+            r.parts = o.b_div * tiles_m * tiles_n;
         } else {
             r.elems = pr.batch * pr.M;
             r.parts = tiles_n * t.wn;
@@ -867,8 +869,19 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
       << pr.K << "," << pr.N << "], tile " << t.bm << "x" << t.bn << "x" << t.bk << "\n";
     s << tp::emit_prelude(pr.epi) << kGemmPrelude;
     s << "#define GM " << pr.M << "u\n#define GN " << pr.N << "u\n#define GK " << pr.K << "u\n";
+    // Two workgroups share a CU when the LDS ring of one takes at most half of it: the second one's mainloop then runs
+    // under the first one's epilogue, and a launch of a few workgroups per CU ends in a shorter tail. For that the
+    // waves of both must fit the register file, so the allocation is held to the budget of twice the waves.
+    std::string wgs_per_cu_attr;
+    {
+        const int lds_bytes = t.stages * (t.bm + t.bn) * t.bk * esz;
+        const int acc_regs = t.bm * t.bn / threads;
+        int wgs = getenv("HELIUM_HIP_GEMM_WGS_PER_CU") ? atoi(getenv("HELIUM_HIP_GEMM_WGS_PER_CU")) : (lds_bytes * 2 <= 160 * 1024 && acc_regs <= 32 ? 2 : 1);
+        if (threads < 256) wgs = 1;
+        wgs_per_cu_attr = "\n#define WGS_PER_CU " + std::to_string(std::max(1, wgs));
+    }
     s << "#define BM " << t.bm << "\n#define BN " << t.bn << "\n#define BK " << t.bk << "\n#define WAVES_M " << t.wm
-      << "\n#define WAVES_N " << t.wn << "\n#define NSTAGES " << t.stages << "\n#define NVE " << nve << "\n#define MMA_BF16 " << (pr.mma_dtype == HE_BF16 ? 1 : 0) << "\n#define MMA_F32 " << (f32 ? 1 : 0)
+      << "\n#define WAVES_N " << t.wn << wgs_per_cu_attr << "\n#define NSTAGES " << t.stages << "\n#define NVE " << nve << "\n#define MMA_BF16 " << (pr.mma_dtype == HE_BF16 ? 1 : 0) << "\n#define MMA_F32 " << (f32 ? 1 : 0)
       << "\n#define STAGGER_EXPR " << (getenv("HELIUM_HIP_GEMM_STAGGER") ? getenv("HELIUM_HIP_GEMM_STAGGER") : "0u")
       << "\n#define ISSUE_FRONT " << (issue_front ? 1 : 0)
       << "\n#define GEMM_SKIP " << (getenv("HELIUM_HIP_GEMM_SKIP") ? atoi(getenv("HELIUM_HIP_GEMM_SKIP")) : 0)
@@ -981,10 +994,13 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
 
     // epilogue pieces
     std::ostringstream setup, body, finish, prefetch;
-    // Optional (HELIUM_HIP_GEMM_EPIPIPE=1): full-size tensors the epilogue reads are requested one step ahead of the
-    // step that uses them. Measured no faster than the compiler's own placement on the 40-op epilogue, so off.
+    // Full-size tensors the epilogue reads are requested one step ahead of the step that uses them, so that a wave
+    // computes one step while the next one's operands travel (the 40-op epilogue: 163 -> 158 us; every CU is in its
+    // epilogue at the same time, so the memory system idles whenever the waves compute). HELIUM_HIP_GEMM_EPIPIPE=0
+    // leaves the placement to the compiler.
     const std::string raw_members = tp::emit_raw_members(pr.epi, nve, true);
-    const bool pipelined = !raw_members.empty() && getenv("HELIUM_HIP_GEMM_EPIPIPE");
+    const char* epipipe = getenv("HELIUM_HIP_GEMM_EPIPIPE");
+    const bool pipelined = !raw_members.empty() && (!epipipe || atoi(epipipe) != 0);
     if (pipelined) {
         tp::EmitCtx lx;
         lx.nv = nve;
@@ -1026,29 +1042,48 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
             // the partial tile of this k range, as f32, for the second launch to add up
             body << "if (ok) {\nfloat* dst = splitk_ws + ((size_t)split * GM + m) * GN + nn;\n#pragma unroll\nfor (int k = 0; k < NVE; k++) if (nn + k < GN) dst[k] = acc_v[k];\n}\n";
         } else {
-        body << "if (ok) {\nconst u32 n0 = nn; (void)n0;\nfloat (&acc)[NVE] = acc_v;\n";
-        tp::EmitCtx cx;
-        cx.nv = nve;
-        if (pipelined) {
-            cx.phase = 2;
-            cx.defer_row_varying_only = true;
-            body << "const RawE& R = Rb[(i * EPI_STEPS + step) & 1]; (void)R;\n";
+        // `x.pow_scalar(2.0)` reaches the kernel as Pow with a broadcast 1-element operand (the square in BatchNorm2d's
+        // statistics). The exponents are read once per workgroup; when all of them are 2 the copy of the body that
+        // squares runs, and the general routine stays out of the common case's instruction stream.
+        std::vector<int> exps;
+        for (size_t i = 0; i < pr.epi.exprs.size(); i++)
+            if (tp::is_uniform_pow(pr.epi, (int)i)) exps.push_back(pr.epi.exprs[pr.epi.exprs[i].b].access.arg);
+        std::sort(exps.begin(), exps.end());
+        exps.erase(std::unique(exps.begin(), exps.end()), exps.end());
+        if (!exps.empty()) {
+            setup << "bool all_squares = true;\n";
+            for (int a : exps) setup << "all_squares = all_squares && ld_one(a" << a << ") == 2.0f;\n";
         }
-        // the emitter names the first of the NV columns `n0`; the tile origin of the same name is shadowed here
-        body << tp::emit_exprs(pr.epi, cx);
-        for (size_t oi = 0; oi < pr.epi.outs.size(); oi++) {
-            const tp::Out& o = pr.epi.outs[oi];
-            const std::string v = "e" + std::to_string(o.expr);
-            if (!o.reduce) {
-                body << "st_vec<NVE>(a" << o.arg << " + ((size_t)bz * GM + m) * GN + nn, " << v << ");\n";
-            } else if (o.fold_m && !o.fold_n) {
-                body << "#pragma unroll\nfor (int k = 0; k < NVE; k++) rc" << oi << "[step % " << colsets << "][k] += " << v << "[k];\n";
-            } else if (o.fold_m && o.fold_n) {
-                body << "#pragma unroll\nfor (int k = 0; k < NVE; k++) rs" << oi << " += " << v << "[k];\n";
-            } else {
-                body << "#pragma unroll\nfor (int k = 0; k < NVE; k++) rr" << oi << " += " << v << "[k];\n";
+        auto element_body = [&](bool squares) {
+            std::ostringstream b;
+            tp::EmitCtx cx;
+            cx.nv = nve;
+            cx.uniform_pow_is_square = squares;
+            if (pipelined) {
+                cx.phase = 2;
+                cx.defer_row_varying_only = true;
+                b << "const RawE& R = Rb[(i * EPI_STEPS + step) & 1]; (void)R;\n";
             }
-        }
+            // the emitter names the first of the NV columns `n0`; the tile origin of the same name is shadowed here
+            b << tp::emit_exprs(pr.epi, cx);
+            for (size_t oi = 0; oi < pr.epi.outs.size(); oi++) {
+                const tp::Out& o = pr.epi.outs[oi];
+                const std::string v = "e" + std::to_string(o.expr);
+                if (!o.reduce) {
+                    b << "st_vec<NVE>(a" << o.arg << " + ((size_t)bz * GM + m) * GN + nn, " << v << ");\n";
+                } else if (o.fold_m && !o.fold_n) {
+                    b << "#pragma unroll\nfor (int k = 0; k < NVE; k++) rc" << oi << "[step % " << colsets << "][k] += " << v << "[k];\n";
+                } else if (o.fold_m && o.fold_n) {
+                    b << "#pragma unroll\nfor (int k = 0; k < NVE; k++) rs" << oi << " += " << v << "[k];\n";
+                } else {
+                    b << "#pragma unroll\nfor (int k = 0; k < NVE; k++) rr" << oi << " += " << v << "[k];\n";
+                }
+            }
+            return b.str();
+        };
+        body << "if (ok) {\nconst u32 n0 = nn; (void)n0;\nfloat (&acc)[NVE] = acc_v;\n";
+        if (exps.empty()) body << element_body(false);
+        else body << "if (all_squares) {\n" << element_body(true) << "} else {\n" << element_body(false) << "}\n";
         body << "}\n";
         // per-row sums: combine the lanes that share the row; every wave that holds a piece of the row parks its
         // partial (zero where its columns lie beyond the matrix)
@@ -1062,23 +1097,54 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         }
         }
     }
-    for (size_t oi = 0; oi < pr.epi.outs.size(); oi++) {
-        const tp::Out& o = pr.epi.outs[oi];
-        if (!o.reduce) continue;
-        if (o.fold_m && !o.fold_n) {
-            // lanes that hold the same columns differ by multiples of lanes_per_row
-            finish << "#pragma unroll\nfor (int c = 0; c < " << colsets << "; c++) {\n#pragma unroll\nfor (int k = 0; k < NVE; k++) {\nfloat r = rc"
-                   << oi << "[c][k];\n";
-            for (int off = lanes_per_row; off < 64; off *= 2) finish << "r += __shfl_xor(r, " << off << ", 64);\n";
-            finish << "const u32 col = ((c * 64 + lane) * NVE) % WTN + k;\nconst u32 nn = n0 + wave_n * WTN + col;\n";
-            const RedOut& ro = red_of(oi);
-            finish << "if (lane < " << std::min(lanes_per_row, 64) << " && nn < GN) red_ws[" << ro.off << "ull + ((size_t)bz * " << ro.parts
-                   << "u + tile_m * WAVES_M + wave_m) * GN + nn] = r;\n}\n}\n";
-        } else if (o.fold_m && o.fold_n) {
-            const RedOut& ro = red_of(oi);
-            const int64_t per_b = ro.parts / o.b_div;  // partials per batch index: tiles x waves
-            finish << "{ float r = wave_reduce<0, 64>(rs" << oi << ");\nif (lane == 0) red_ws[" << ro.off << "ull + (size_t)(bz / " << o.b_div << "u) * "
-                   << ro.parts << "u + (size_t)(bz % " << o.b_div << "u) * " << per_b << "u + (tile_m * " << tiles_n << "u + tile_n) * (WAVES_M * WAVES_N) + wave] = r; }\n";
+    {
+        // Column and scalar sums: the waves of the workgroup meet in LDS (free once every wave has left its strip), so
+        // the workgroup parks one partial per column, or one in all, instead of one per wave.
+        int ncol = 0, nsc = 0;
+        for (auto& o : pr.epi.outs) {
+            if (o.reduce && o.fold_m && !o.fold_n) ncol++;
+            if (o.reduce && o.fold_m && o.fold_n) nsc++;
+        }
+        if (ncol + nsc) {
+            HE_REQUIRE((size_t)(ncol * t.wm * t.bn + nsc * t.wm * t.wn) * 4 <= (size_t)t.stages * (t.bm + t.bn) * t.bk * esz, HE_ERR_INTERNAL,
+                       "reduction exchange exceeds the tile's LDS");
+            finish << "__syncthreads();\nfloat* red = (float*)lds;\n";
+            int ci = 0, si = 0;
+            for (size_t oi = 0; oi < pr.epi.outs.size(); oi++) {
+                const tp::Out& o = pr.epi.outs[oi];
+                if (!o.reduce || !o.fold_m) continue;
+                if (!o.fold_n) {
+                    // lanes that hold the same columns differ by multiples of lanes_per_row
+                    finish << "#pragma unroll\nfor (int c = 0; c < " << colsets << "; c++) {\n#pragma unroll\nfor (int k = 0; k < NVE; k++) {\nfloat r = rc"
+                           << oi << "[c][k];\n";
+                    for (int off = lanes_per_row; off < 64; off *= 2) finish << "r += __shfl_xor(r, " << off << ", 64);\n";
+                    finish << "const u32 col = ((c * 64 + lane) * NVE) % WTN + k;\n";
+                    finish << "if (lane < " << std::min(lanes_per_row, 64) << ") red[" << ci * t.wm * t.bn << " + wave_m * BN + wave_n * WTN + col] = r;\n}\n}\n";
+                    ci++;
+                } else {
+                    finish << "{ float r = wave_reduce<0, 64>(rs" << oi << ");\nif (lane == 0) red[" << ncol * t.wm * t.bn + si * t.wm * t.wn << " + wave] = r; }\n";
+                    si++;
+                }
+            }
+            finish << "__syncthreads();\n";
+            ci = si = 0;
+            for (size_t oi = 0; oi < pr.epi.outs.size(); oi++) {
+                const tp::Out& o = pr.epi.outs[oi];
+                if (!o.reduce || !o.fold_m) continue;
+                const RedOut& ro = red_of(oi);
+                if (!o.fold_n) {
+                    finish << "for (u32 c = tid; c < BN; c += NTHREADS) {\nfloat r = 0.0f;\n#pragma unroll\nfor (int w = 0; w < WAVES_M; w++) r += red["
+                           << ci * t.wm * t.bn << " + w * BN + c];\nif (n0 + c < GN) red_ws[" << ro.off << "ull + ((size_t)bz * " << ro.parts
+                           << "u + tile_m) * GN + n0 + c] = r;\n}\n";
+                    ci++;
+                } else {
+                    const int64_t per_b = ro.parts / o.b_div;  // partials per batch index: one per tile
+                    finish << "if (tid == 0) {\nfloat r = 0.0f;\n#pragma unroll\nfor (int w = 0; w < WAVES_M * WAVES_N; w++) r += red["
+                           << ncol * t.wm * t.bn + si * t.wm * t.wn << " + w];\nred_ws[" << ro.off << "ull + (size_t)(bz / " << o.b_div << "u) * " << ro.parts
+                           << "u + (size_t)(bz % " << o.b_div << "u) * " << per_b << "u + tile_m * " << tiles_n << "u + tile_n] = r;\n}\n";
+                    si++;
+                }
+            }
         }
     }
     // splice the generated pieces into the body
@@ -1208,7 +1274,10 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         for (size_t i = 0; i < reds.size(); i++) {
             const RedOut& r = reds[i];
             const tp::Out& o = pr.epi.outs[r.out];
-            const int eb = r.elems < 16 ? 1 : r.parts >= 512 ? 4 : 16;
+            // elements per workgroup: 16 where there are many elements with few partials each, fewer (more threads per
+            // element, more workgroups) where a few elements have thousands of partials
+            int eb = 16;
+            while (eb > 1 && (r.elems < eb || (r.elems / eb < 64 && r.parts > 256 / eb))) eb /= 2;
             const uint32_t blocks = (uint32_t)((r.elems + eb - 1) / eb);
             char scale[64];
             snprintf(scale, sizeof scale, "%.9ef", o.rop == tp::ROp::Mean ? (float)o.mean_scale : 1.0f);

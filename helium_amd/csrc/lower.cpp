@@ -226,6 +226,7 @@ public:
             merge_row_dims();
         } else {
             fold_leading_dims_as_columns();
+            merge_row_like_dims();
         }
         return std::move(p_);
     }
@@ -289,6 +290,29 @@ private:
         for (size_t j = 0; j + depth < R; j++) {
             HE_REQUIRE(j == 0 || perm[j] > last, HE_ERR_UNSUPPORTED, "the reduction's kept dims are permuted");
             last = perm[j];
+        }
+    }
+
+    // A kernel without reductions treats every dim but the last as rows: neighbours that every operand walks as one dim
+    // (packed tensors; vectors broadcast along all of them) are merged, so that an NHWC activation normalised per
+    // channel is [n*h*w, c] — long columns of rows for a block to walk — instead of [n, h][w][c] with w rows per block.
+    void merge_row_like_dims() {
+        for (auto& o : p_.outs)
+            if (o.reduce) return;
+        for (auto& e : p_.exprs)
+            if (e.kind == Expr::Load && (!e.access.chain.empty() || e.access.stride.size() != p_.dims.size())) return;
+        for (size_t i = 0; i + 2 < p_.dims.size();) {
+            bool ok = true;
+            for (auto& e : p_.exprs)
+                if (e.kind == Expr::Load && e.access.stride[i] != e.access.stride[i + 1] * p_.dims[i + 1]) ok = false;
+            if (!ok) {
+                i++;
+                continue;
+            }
+            p_.dims[i + 1] *= p_.dims[i];
+            p_.dims.erase(p_.dims.begin() + i);
+            for (auto& e : p_.exprs)
+                if (e.kind == Expr::Load) e.access.stride.erase(e.access.stride.begin() + i);
         }
     }
 
