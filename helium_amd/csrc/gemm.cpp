@@ -994,13 +994,12 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
 
     // epilogue pieces
     std::ostringstream setup, body, finish, prefetch;
-    // Full-size tensors the epilogue reads are requested one step ahead of the step that uses them, so that a wave
-    // computes one step while the next one's operands travel (the 40-op epilogue: 163 -> 158 us; every CU is in its
-    // epilogue at the same time, so the memory system idles whenever the waves compute). HELIUM_HIP_GEMM_EPIPIPE=0
-    // leaves the placement to the compiler.
+    // Optional (HELIUM_HIP_GEMM_EPIPIPE=1): full-size tensors the epilogue reads are requested one step ahead of the
+    // step that uses them. Measured within run-to-run noise of the compiler's own placement on the 40-op epilogue
+    // (162.5 vs 162.6 us over three alternating runs each), so off.
     const std::string raw_members = tp::emit_raw_members(pr.epi, nve, true);
     const char* epipipe = getenv("HELIUM_HIP_GEMM_EPIPIPE");
-    const bool pipelined = !raw_members.empty() && (!epipipe || atoi(epipipe) != 0);
+    const bool pipelined = !raw_members.empty() && epipipe && atoi(epipipe) != 0;
     if (pipelined) {
         tp::EmitCtx lx;
         lx.nv = nve;

@@ -335,8 +335,10 @@ int he_fgraph_subdivide(he_fgraph_t graph, uint64_t* nodes, int32_t* portions, i
 
 /* Backend options. HE_OPT_FUSE_MATMUL_EPILOGUE (default 1): pointwise / reduce ops that follow a Matmul join its
  * instruction and run as the fused GEMM's epilogue (the MatmulGenerator path, matmul.rs:88-130), and a SwapDims of the
- * two matrix dims that feeds only a Matmul joins it as a transposed operand; 0 restores the
- * grouping of helium/src/cuda/instr/cudnn_graph.rs:319-321, where a matmul instruction never fuses.
+ * two matrix dims that feeds only a Matmul joins it as a transposed operand; the same holds for a Conv, and a
+ * SwapDims + Reduce that folds all rows of the product (column sums, BatchNorm2d statistics of a convolution's output)
+ * joins as a column reduction of the epilogue; 0 restores the grouping of
+ * helium/src/cuda/instr/cudnn_graph.rs:319-321, where a matmul or convolution instruction never fuses.
  * HE_OPT_FOLD_SWAP_INTO_REDUCE (default 1): a SwapDims above the 1M-element threshold of cuda.rs:38-41 whose values
  * all end in Reduce ops (BatchNorm2d statistics, column sums) stays in the pointwise instruction, which then folds the
  * leading dims of the untransposed tensor in one pass; 0 makes it a permute instruction as the reference does. */

@@ -39,7 +39,7 @@ def launch_gemm(k, bufs):
 def run_emulated(g, inputs, tile, env=()):
     os.environ["HELIUM_HIP_GEMM_TILE"] = tile
     for name in env:
-        os.environ[name] = "0" if name == "HELIUM_HIP_GEMM_EPIPIPE" else "1"
+        os.environ[name] = "1"
     try:
         k = ha.TileKernel.fused(g)
     finally:
@@ -75,7 +75,7 @@ def readme_fusion(size, mainloop, full):
 
 CASES = [
     ("readme_epilogue_with_prefetched_aux_tensors", lambda: readme_fusion(128, False, False), "128,128,64,2,2"),
-    ("readme_epilogue_unpipelined", lambda: readme_fusion(128, False, False), "128,128,64,2,2"),
+    ("readme_epilogue", lambda: readme_fusion(128, False, False), "128,128,64,2,2"),
     ("readme_epilogue_ragged_with_mainloop", lambda: readme_fusion(72, True, True), "128,128,64,2,2"),
     ("plain_2x2_tiles", lambda: gemm_cases.plain(160, 136, 72), "128,128,64,2,2"),
     ("ragged_scalar_paths", lambda: gemm_cases.plain(97, 131, 67), "128,128,64,2,2"),
@@ -116,7 +116,7 @@ CASES = [
 @pytest.mark.parametrize("name,build,tile", CASES, ids=[c[0] for c in CASES])
 def test_fused_gemm_on_cpu(name, build, tile):
     g, inputs, outs = build()
-    k, got = run_emulated(g, inputs, tile, env=("HELIUM_HIP_GEMM_EPIPIPE",) if "unpipelined" in name else ())
+    k, got = run_emulated(g, inputs, tile, env=("HELIUM_HIP_GEMM_EPIPIPE",) if "prefetched" in name else ())
     assert sorted(got) == sorted(outs), k.description
     f32_cases = ("f32_operands", "f32_linear_layer", "one_wave_32x32_f32_direct", "two_waves_64x32_linear_layer", "nt_f32_operands", "tn_f32_operands")
     rounding = "f16" if name == "f16_operands" else None if name in f32_cases else "bf16"
