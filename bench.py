@@ -802,8 +802,11 @@ def roofline(wl, ms):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    # The device's clock settles only after some milliseconds of load: right after an idle phase it runs fast for a
+    # few launches, dips for some tens, then recovers (the 4096^3 GEMM: 115 us, then 128-147 us, then 115 us again
+    # from about the 100th launch on). 200 warm-up launches put the timed ones into the settled state.
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--workload", default=None, help="headline workload (default: the best-covered BASELINE config)")
     ap.add_argument("--only", action="store_true", help="measure the headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
