@@ -36,9 +36,19 @@ class Tensor:
 
     def __init__(self, handle):
         self.handle = handle
-        dt, ln, nb, ptr = C.c_int32(), C.c_uint64(), C.c_uint64(), C.c_void_p()
-        check(lib.he_tensor_info(handle, C.byref(dt), C.byref(ln), C.byref(nb), C.byref(ptr)))
-        self.dtype, self.len, self.nbytes, self.ptr = _ffi.DTYPE_NAMES[dt.value], ln.value, nb.value, ptr
+        self._info = None  # (dtype, len, nbytes, ptr), asked for on first use: a result that is only passed on costs no call
+
+    def _get(self, i):
+        if self._info is None:
+            dt, ln, nb, ptr = C.c_int32(), C.c_uint64(), C.c_uint64(), C.c_void_p()
+            check(lib.he_tensor_info(self.handle, C.byref(dt), C.byref(ln), C.byref(nb), C.byref(ptr)))
+            self._info = (_ffi.DTYPE_NAMES[dt.value], ln.value, nb.value, ptr)
+        return self._info[i]
+
+    dtype = property(lambda self: self._get(0))
+    len = property(lambda self: self._get(1))
+    nbytes = property(lambda self: self._get(2))
+    ptr = property(lambda self: self._get(3))
 
     @classmethod
     def from_numpy(cls, storage, dtype, length=None):
@@ -107,14 +117,27 @@ def execute_graph(graph, inputs):
     """BackendExt::execute_graph. `inputs`: {input node id: Tensor}. Returns {output node id: Tensor}."""
     init()
     n = len(inputs)
-    nodes = _ffi.arr(C.c_uint32, list(inputs.keys()))
-    handles = (C.c_void_p * max(n, 1))(*[t.handle for t in inputs.values()])
-    cap = max(1, sum(1 for x in graph.nodes if x["node"] == "output"))
-    out_nodes = (C.c_uint32 * cap)()
-    out_handles = (C.c_void_p * cap)()
+    # array types are cached per size: building a ctypes array type costs more than filling an array
+    in_nodes_t, in_handles_t = _array_types(max(n, 1))
+    nodes = in_nodes_t(*inputs.keys())
+    handles = in_handles_t(*[t.handle for t in inputs.values()])
+    cap = max(1, graph.num_outputs)
+    out_nodes_t, out_handles_t = _array_types(cap)
+    out_nodes = out_nodes_t()
+    out_handles = out_handles_t()
     count = C.c_int()
     check(lib.he_execute_graph(graph.handle, nodes, handles, n, out_nodes, out_handles, cap, C.byref(count)))
     return {out_nodes[i]: Tensor(C.c_void_p(out_handles[i])) for i in range(count.value)}
+
+
+_ARRAY_TYPES = {}
+
+
+def _array_types(n):
+    t = _ARRAY_TYPES.get(n)
+    if t is None:
+        t = _ARRAY_TYPES[n] = (C.c_uint32 * n, C.c_void_p * n)
+    return t
 
 
 def stats():

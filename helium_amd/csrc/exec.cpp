@@ -364,6 +364,19 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
                 }
         }
     };
+    // An execution whose steps hold one instruction each runs on stream 0 alone: its last launch can carry the
+    // execution's event itself.
+    const plan::Instr* closing = nullptr;
+    {
+        bool one_stream = true;
+        for (auto& step : plan->steps) {
+            one_stream = one_stream && step.instrs.size() <= 1;
+            if (!step.instrs.empty()) closing = step.instrs.back().get();
+        }
+        if (!one_stream || getenv("HELIUM_HIP_NO_LAUNCH_EVENTS")) closing = nullptr;
+    }
+    EventRef done = pool.take_event();
+    bool done_recorded = false;
     for (auto& step : plan->steps) {
         for (NodeId r : step.tensors_to_release) tensors.erase(r);
         if (step.instrs.empty()) continue;
@@ -404,7 +417,15 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
                 }
             }
             ht.lap(3);
-            instr.execute([&](NodeId n) -> void* { return tensors.at(n)->ptr; }, stream);
+            if (&instr == closing) set_pending_stop_event(done->e);
+            try {
+                instr.execute([&](NodeId n) -> void* { return tensors.at(n)->ptr; }, stream);
+            } catch (...) {
+                (void)take_pending_stop_event();
+                throw;
+            }
+            // taken by the instruction's last launch, or still pending (a launch too large for that entry point)
+            if (&instr == closing) done_recorded = take_pending_stop_event() == nullptr;
             ht.lap(4);
             local.instrs++;
         }
@@ -416,8 +437,7 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
     // Drop of the executor (cuda.rs:232-260): when everything queued above has run, the scope's freed blocks
     // become available to everyone. Stream 0 joins the last step and carries the event the pool polls.
     join({0});
-    EventRef done = pool.take_event();
-    HE_HIP(hipEventRecord(done->e, st.s[0]));
+    if (!done_recorded) HE_HIP(hipEventRecord(done->e, st.s[0]));
     // The same event orders this thread's next execution after this one, and it is the ready event of every tensor
     // that outlives the plan (enumerate_output_tensors, cuda.rs:142-153, records one per tensor).
     for (NodeId out : alive) tensors.at(out)->ready = done;

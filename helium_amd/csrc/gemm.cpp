@@ -1327,13 +1327,13 @@ void GemmKernel::execute(void* const* ptrs, hipStream_t stream) {
     std::vector<void*> argv(holders.size());
     for (size_t i = 0; i < holders.size(); i++) argv[i] = &holders[i];
     const uint32_t block[3] = {threads_, 1, 1};
-    kernel_->launch(grid_, block, 0, stream, argv.data());
+    kernel_->launch(grid_, block, 0, stream, argv.data(), !finalize_ && !reduce_);
     if (finalize_) {
         void* out = ptrs[prob_.map_e[prob_.epi.outs[0].arg]];
         void* fargv[] = {&ws, &out};
         const uint64_t total = (uint64_t)prob_.M * prob_.N;
         const uint32_t fgrid[3] = {(uint32_t)std::min<uint64_t>((total + 255) / 256, 2048), 1, 1}, fblock[3] = {256, 1, 1};
-        finalize_->launch(fgrid, fblock, 0, stream, fargv);
+        finalize_->launch(fgrid, fblock, 0, stream, fargv, !reduce_);
     }
     if (reduce_) {
         std::vector<void*> rh{ws};
@@ -1341,7 +1341,7 @@ void GemmKernel::execute(void* const* ptrs, hipStream_t stream) {
         std::vector<void*> rargv(rh.size());
         for (size_t i = 0; i < rh.size(); i++) rargv[i] = &rh[i];
         const uint32_t rgrid[3] = {reduce_grid_, 1, 1}, rblock[3] = {256, 1, 1};
-        reduce_->launch(rgrid, rblock, 0, stream, rargv.data());
+        reduce_->launch(rgrid, rblock, 0, stream, rargv.data(), true);
     }
 }
 

@@ -336,7 +336,7 @@ void Permute::execute(const void* in, void* out, hipStream_t stream) {
                "permute operands must be aligned to %d bytes", (int)amask + 1);
     const uint32_t grid[3] = {plan_.grid, 1, 1}, block[3] = {(uint32_t)plan_.threads, 1, 1};
     void* args[] = {(void*)&in, (void*)&out};
-    kernel_->launch(grid, block, 0, stream, args);
+    kernel_->launch(grid, block, 0, stream, args, true);
 }
 
 }  // namespace he

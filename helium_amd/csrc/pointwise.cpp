@@ -96,12 +96,12 @@ void TileKernel::execute(void* const* ptrs, hipStream_t stream) {
     std::vector<void*> argv(holders.size());
     for (size_t i = 0; i < holders.size(); i++) argv[i] = &holders[i];
     const uint32_t grid[3] = {launch_.grid, 1, 1}, block[3] = {launch_.threads, 1, 1};
-    kernel_->launch(grid, block, 0, stream, argv.data());
+    kernel_->launch(grid, block, 0, stream, argv.data(), !finalize_);
     if (finalize_) {
         // same arguments, then the float scratch
         argv.resize(nargs + 1);
         const uint32_t fgrid[3] = {launch_.finalize_grid, 1, 1};
-        finalize_->launch(fgrid, block, 0, stream, argv.data());
+        finalize_->launch(fgrid, block, 0, stream, argv.data(), true);
     }
 }
 

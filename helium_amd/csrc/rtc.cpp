@@ -1,5 +1,7 @@
 #include "rtc.h"
 
+#include <hip/hip_ext.h>
+
 #include <dlfcn.h>
 #include <hip/hiprtc.h>
 #include <sys/stat.h>
@@ -178,10 +180,30 @@ void JitKernel::ensure_loaded() {
     func_ = f;
 }
 
+namespace {
+thread_local hipEvent_t t_pending_stop = nullptr;
+}
+void set_pending_stop_event(hipEvent_t event) { t_pending_stop = event; }
+hipEvent_t take_pending_stop_event() {
+    hipEvent_t e = t_pending_stop;
+    t_pending_stop = nullptr;
+    return e;
+}
+
 void JitKernel::launch(const uint32_t grid[3], const uint32_t block[3], uint32_t lds_bytes, hipStream_t stream,
-                       void** args) {
+                       void** args, bool closes_instruction) {
     ensure_loaded();
     HE_REQUIRE(grid[0] && grid[1] && grid[2], HE_ERR_INVALID, "kernel %s: empty grid", entry_.c_str());
+    if (closes_instruction && t_pending_stop) {
+        // this entry point takes the global work size, in 32 bits per dim
+        const uint64_t gx = (uint64_t)grid[0] * block[0], gy = (uint64_t)grid[1] * block[1], gz = (uint64_t)grid[2] * block[2];
+        if (gx < (1ull << 32) && gy < (1ull << 32) && gz < (1ull << 32)) {
+            hipEvent_t stop = take_pending_stop_event();
+            HE_HIP(hipExtModuleLaunchKernel(func_, (uint32_t)gx, (uint32_t)gy, (uint32_t)gz, block[0], block[1], block[2], lds_bytes, stream,
+                                            args, nullptr, nullptr, stop, 0));
+            return;
+        }
+    }
     HE_HIP(hipModuleLaunchKernel(func_, grid[0], grid[1], grid[2], block[0], block[1], block[2], lds_bytes,
                                  stream, args, nullptr));
 }

@@ -20,6 +20,12 @@ std::vector<std::string> default_kernel_options();
 
 // A compiled kernel: code object + entry name. The module is loaded lazily on first launch (so that
 // generation and compilation work on a machine without a GPU) and kept for the life of the object.
+// An event the next instruction-closing launch of this thread should signal on completion. The executor sets it ahead
+// of the last instruction of an execution that used one stream only; whoever set it takes it back afterwards and
+// records it the ordinary way if no launch took it.
+void set_pending_stop_event(hipEvent_t event);
+hipEvent_t take_pending_stop_event();
+
 class JitKernel {
 public:
     JitKernel(std::string source, std::string entry, std::vector<std::string> options = {});
@@ -29,8 +35,11 @@ public:
 
     const std::string& source() const { return source_; }
     const std::string& entry() const { return entry_; }
+    // `closes_instruction`: this is the last launch an instruction makes. If the calling thread has an event pending
+    // (set_pending_stop_event), the launch carries it as its completion event, which saves the separate record (a
+    // record occupies the device for about as long as a small kernel does).
     void launch(const uint32_t grid[3], const uint32_t block[3], uint32_t lds_bytes, hipStream_t stream,
-                void** args);
+                void** args, bool closes_instruction = false);
     // Number of scratch bytes per lane the compiler reported (0 == no spills); -1 before the module is loaded.
     int private_bytes();
     int vgprs();

@@ -64,6 +64,7 @@ class OpGraph:
         self.handle = C.c_void_p()
         check(lib.he_graph_create(C.byref(self.handle)))
         self.nodes = []  # plain-data record of the graph: dicts with id / kind / op fields
+        self.num_outputs = 0
 
     def __del__(self):
         try:
@@ -85,6 +86,7 @@ class OpGraph:
         node = C.c_uint32()
         check(lib.he_graph_new_output(self.handle, from_node, C.byref(node)))
         self.nodes.append({"id": node.value, "node": "output", "from": from_node})
+        self.num_outputs += 1
         return node.value
 
     def _op(self, kind, inputs, record, **f):
