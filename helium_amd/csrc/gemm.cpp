@@ -117,6 +117,13 @@ struct WavePos {
     u32 m0, n0;       /* first row / column of the workgroup's tile (gathers need absolute coordinates) */
     const void* img;  /* CONV_A: the image the A operand is gathered from */
     const void* bsrc; /* B_ROW_GATHER: the tensor B's rows are picked from */
+#if CONV_A_FAST
+    /* CONV_A with direct loads: the rows a lane fetches are the same in every k-tile, so their pixel coordinates are
+       worked out once. Per direct-load instruction of the wave: image offset of the pixel's image, the pixel's
+       coordinate terms that do not depend on the tap, and whether the row exists at all. */
+    u32 cbase[A_DPW_MAX];
+    int ch0[A_DPW_MAX], cw0[A_DPW_MAX];
+#endif
 };
 #if CONV_A || CONV_B
 // Where the taps that fall outside the image (or the matrix) are read from by the direct global->LDS loads.
@@ -294,7 +301,14 @@ __device__ __forceinline__ void direct_issue(unsigned char* __restrict__ st, con
 #endif
         const u32 row = blk * (64 / A_CHUNKS) + lane / A_CHUNKS, pc = lane % A_CHUNKS;
         const u32 kc = pc ^ ((row >> A_SWZ_SHIFT) & (A_CHUNKS - 1));
-#if CONV_A
+#if CONV_A_FAST
+        // `ga` carries the tile's first k as an element offset from null. The channel count is a multiple of the
+        // k-tile, so the whole tile lies in one filter tap: the tap is worked out once per wave (scalar), and the
+        // lane adds it to the pixel terms it keeps from before the k-loop.
+        size_t at;
+        const bool inside = conv_tap_fast((u32)(ga - (const mul_t*)nullptr), kc * EPC, w.cbase[i], w.ch0[i], w.cw0[i], at);
+        const mul_t* gp = inside ? (const mul_t*)w.img + at : (const mul_t*)conv_zeros;
+#elif CONV_A
         // `ga` carries the tile's first k as an element offset from null: every lane computes the address of its
         // own chunk of 8 (4) channels of one filter tap, or points at zeros when the tap is outside the image
         size_t at;
@@ -473,7 +487,13 @@ void fused_matmul(KERNEL_PARAMS) {
         }
 #endif
     };
+#if CONV_A_FAST
+    WavePos wpos = {lane, wave, wave_m, wave_n, m0, n0, (const void*)CONV_IMG_OR_NULL, (const void*)B_SRC_OR_NULL, {}, {}, {}};
+#pragma unroll
+    for (int i = 0; i < A_DPW_MAX; i++) conv_row_terms(m0 + (wave * A_DPW_MAX + i) * (64 / A_CHUNKS) + lane / A_CHUNKS, wpos.cbase[i], wpos.ch0[i], wpos.cw0[i]);
+#else
     const WavePos wpos = {lane, wave, wave_m, wave_n, m0, n0, (const void*)CONV_IMG_OR_NULL, (const void*)B_SRC_OR_NULL};
+#endif
 
 /* s_waitcnt immediate: vmcnt lives in bits [3:0] and [15:14] */
 #define WAITCNT_VM(n) ((((n) & 15) | (((n) >> 4) << 14)))
@@ -683,8 +703,12 @@ GemmProblem gemm_problem_from_fusion(const fir::OpGraph& g) {
 
 int choose_split_k(int64_t M, int64_t N, int64_t K, int64_t batch) {
     if (getenv("HELIUM_HIP_GEMM_NO_SPLIT_K") || batch != 1) return 1;
+    if (const char* env = getenv("HELIUM_HIP_GEMM_SPLIT_K")) return std::max(1, atoi(env));
     const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128), k_tiles = (K + 63) / 64;
     if (tiles >= 128) return 1;
+    // 64x64 tiles fill the chip before a split k range has to: the partial tiles of a split cost a second pass over
+    // the output (a 3136 x 512 x 4608 convolution: 51 us with 128x128 tiles and four k ranges, 34 us with 64x64 tiles)
+    if (((M + 63) / 64) * ((N + 63) / 64) >= 192) return 1;
     return (int)std::max<int64_t>(1, std::min<int64_t>({(384 + tiles - 1) / tiles, k_tiles / 8, 1024}));
 }
 
@@ -850,10 +874,18 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
                           !getenv("HELIUM_HIP_GEMM_NO_DIRECT_A");
     const bool direct_b = want_direct && raw_b && (pr.conv_b.on || (pr.N % t.bn == 0 && pr.K % t.bk == 0)) && (t.bk * t.bn * esz / 1024) % (threads / 64) == 0 &&
                           (pr.b_nk || 64 % (t.bn / epc) == 0) && !getenv("HELIUM_HIP_GEMM_NO_DIRECT_B");
+    // A convolution's gather with direct loads, a channel count that is a multiple of the k-tile (every tile then lies in
+    // one filter tap) and a wave that issues a whole number of loads: the per-lane address arithmetic of a load
+    // shrinks from a full (pixel, tap) decomposition to a few adds.
+    const bool conv_a_fast = pr.conv_a.on && direct_a && pr.conv_a.C % t.bk == 0 && (t.bm * t.bk * esz / 1024) % (threads / 64) == 0 &&
+                             !getenv("HELIUM_HIP_GEMM_NO_CONV_FAST");
     if (!(direct_a && direct_b)) t.stages = 2;  // register staging is double-buffered only
     else if (!getenv("HELIUM_HIP_GEMM_TILE") && small) {
         // A grid that leaves CUs idle is bound by the latency of its k-loop: keep as many tiles in flight as LDS holds.
-        while (t.stages < 4 && (t.stages + 1) * (t.bm + t.bn) * t.bk * esz <= 128 * 1024) t.stages++;
+        // With more than one workgroup per CU (a split k range) the LDS is better spent on a second and third
+        // workgroup, whose loads hide each other's waits (filter gradient of a 64-channel layer: 66 -> 56 us).
+        const int64_t workgroups = ((pr.M + t.bm - 1) / t.bm) * ((pr.N + t.bn - 1) / t.bn) * pr.batch * pr.split_k;
+        while (workgroups <= 256 && t.stages < 4 && (t.stages + 1) * (t.bm + t.bn) * t.bk * esz <= 128 * 1024) t.stages++;
     }
     // All direct loads of the next tile are issued at the start of a tile's MFMAs (the round trip needs the whole
     // tile to hide); HELIUM_HIP_GEMM_ISSUE=0 spreads them over the k-steps instead.
@@ -887,6 +919,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
       << "\n#define GEMM_SKIP " << (getenv("HELIUM_HIP_GEMM_SKIP") ? atoi(getenv("HELIUM_HIP_GEMM_SKIP")) : 0)
       << "\n#define GEMM_TIMING " << (getenv("HELIUM_HIP_GEMM_TIMING") ? 1 : 0) << "\n#define GEMM_TIMING_PTR p" << (pr.args.size() - 1)
       << "\n#define DIRECT_A " << (direct_a ? 1 : 0) << "\n#define DIRECT_B " << (direct_b ? 1 : 0)
+      << "\n#define CONV_A_FAST " << (conv_a_fast ? 1 : 0) << "\n#define A_DPW_MAX " << std::max(1, t.bm * t.bk * esz / 1024 / (threads / 64))
       << "\n#define A_KM " << (pr.a_km ? 1 : 0) << "\n#define B_NK " << (pr.b_nk ? 1 : 0) << "\n#define CONV_A " << (pr.conv_a.on ? 1 : 0) << "\n#define CONV_IMG p" << (pr.conv_a.on ? pr.map_a[0] : 0)
       << "\n#define CONV_IMG_OR_NULL " << (pr.conv_a.on ? "p" + std::to_string(pr.map_a[0]) : std::string("nullptr"))
       << "\n#define B_ROW_GATHER " << (pr.b_rows.on ? 1 : 0) << "\n#define CONV_B " << (pr.conv_b.on ? 1 : 0) << "\n#define SPLIT_K " << pr.split_k
@@ -958,6 +991,28 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         s << "at = (((size_t)n * " << cv.H << "u + (u32)ih) * " << cv.W << "u + (u32)iw) * " << cv.C << "u + c;\n"
           << "return row < " << cv.N * cv.P * cv.Q << "u && col < " << cv.R * cv.S * cv.C << "u && hit && ih >= 0 && ih < " << cv.H << " && iw >= 0 && iw < " << cv.W << ";\n}\n";
     };
+    if (conv_a_fast) {
+        const auto& cv = pr.conv_a;
+        // row -> (image offset, tap-independent coordinate terms); a row beyond the matrix gets coordinates that no tap
+        // brings inside the image
+        s << "__device__ __forceinline__ void conv_row_terms(u32 row, u32& base, int& h0, int& w0) {\n"
+          << "const u32 n = row / " << cv.P * cv.Q << "u, pq = row % " << cv.P * cv.Q << "u, p = pq / " << cv.Q << "u, q = pq % " << cv.Q << "u;\n"
+          << "base = n * " << cv.H * cv.W * cv.C << "u;\n";
+        if (!cv.bwd) s << "h0 = (int)(p * " << cv.sh << "u) - " << cv.ph << "; w0 = (int)(q * " << cv.sw << "u) - " << cv.pw << ";\n";
+        else s << "h0 = (int)p + " << cv.ph << "; w0 = (int)q + " << cv.pw << ";\n";
+        s << "if (row >= " << cv.N * cv.P * cv.Q << "u) { base = 0u; h0 = -(1 << 24); w0 = -(1 << 24); }\n}\n";
+        // k0: first k of the tile (uniform), kc: the lane's channel offset inside the tile
+        s << "__device__ __forceinline__ bool conv_tap_fast(u32 k0, u32 kc, u32 base, int h0, int w0, size_t& at) {\n"
+          << "const u32 rs = k0 / " << cv.C << "u, c = k0 % " << cv.C << "u + kc, r = rs / " << cv.S << "u, sx = rs % " << cv.S << "u;\n";
+        if (!cv.bwd)
+            s << "const int ih = h0 + (int)(r * " << cv.dh << "u), iw = w0 + (int)(sx * " << cv.dw << "u);\nconst bool hit = true;\n";
+        else
+            s << "const int th = h0 - (int)(r * " << cv.dh << "u), tw = w0 - (int)(sx * " << cv.dw << "u);\n"
+              << "const bool hit = th >= 0 && tw >= 0 && th % " << cv.sh << " == 0 && tw % " << cv.sw << " == 0;\n"
+              << "const int ih = th / " << cv.sh << ", iw = tw / " << cv.sw << ";\n";
+        s << "at = (size_t)base + (size_t)(((u32)ih * " << cv.W << "u + (u32)iw) * " << cv.C << "u + c);\n"
+          << "return k0 < " << cv.R * cv.S * cv.C << "u && hit && ih >= 0 && ih < " << cv.H << " && iw >= 0 && iw < " << cv.W << ";\n}\n";
+    }
     if (pr.conv_a.on) {
         // The gather of an implicit-GEMM convolution in place of A's loads: one 16-byte chunk is EPC consecutive
         // channels of one filter tap when the channel count allows, EPC separate taps otherwise (a 3-channel image).
@@ -1251,10 +1306,13 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         HE_REQUIRE(pr.batch == 1 && pr.epi.outs.size() == 1 && !pr.epi.outs[0].reduce && pr.epi.exprs.size() == 1, HE_ERR_UNSUPPORTED,
                    "split-k needs an unbatched product with a plain epilogue");
         const tp::Out& o = pr.epi.outs[0];
+        // 32 consecutive output elements per workgroup, 8 threads per element (thread q adds partials q, q + 8, ...),
+        // then one thread per element adds the 8 sums in order
         s << "extern \"C\" __global__ __launch_bounds__(256) void fused_matmul_finalize(const float* __restrict__ ws, " << tp::c_type(o.dtype)
-          << "* __restrict__ out) {\nconst size_t total = (size_t)GM * GN;\nfor (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {\n"
-          << "float acc = 0.0f;\n#pragma unroll 4\nfor (u32 sp = 0; sp < " << pr.split_k << "u; sp++) acc += ws[(size_t)sp * total + i];\n"
-          << "float one[1] = {acc};\nst_vec<1>(out + i, one);\n}\n}\n";
+          << "* __restrict__ out) {\n__shared__ float part[256];\nconst size_t total = (size_t)GM * GN;\nconst u32 e = threadIdx.x % 32u, pg = threadIdx.x / 32u;\n"
+          << "const size_t i = (size_t)blockIdx.x * 32 + e;\nfloat acc = 0.0f;\nif (i < total) {\n#pragma unroll 4\nfor (u32 sp = pg; sp < " << pr.split_k
+          << "u; sp += 8u) acc += ws[(size_t)sp * total + i];\n}\npart[pg * 32u + e] = acc;\n__syncthreads();\n"
+          << "if (pg == 0 && i < total) {\nfloat r = 0.0f;\n#pragma unroll\nfor (int q = 0; q < 8; q++) r += part[q * 32 + e];\nfloat one[1] = {r};\nst_vec<1>(out + i, one);\n}\n}\n";
     }
     if (!reds.empty()) {
         // Second launch: one workgroup folds EB output elements, PG = 256 / EB threads share the partials of each
@@ -1332,7 +1390,7 @@ void GemmKernel::execute(void* const* ptrs, hipStream_t stream) {
         void* out = ptrs[prob_.map_e[prob_.epi.outs[0].arg]];
         void* fargv[] = {&ws, &out};
         const uint64_t total = (uint64_t)prob_.M * prob_.N;
-        const uint32_t fgrid[3] = {(uint32_t)std::min<uint64_t>((total + 255) / 256, 2048), 1, 1}, fblock[3] = {256, 1, 1};
+        const uint32_t fgrid[3] = {(uint32_t)((total + 31) / 32), 1, 1}, fblock[3] = {256, 1, 1};
         finalize_->launch(fgrid, fblock, 0, stream, fargv, !reduce_);
     }
     if (reduce_) {

@@ -193,7 +193,7 @@ def run_ir_kernel_on_cpu(g, nodes, inputs):
         # a split-k product: partial tiles go to scratch, a second launch adds them up into the one output
         res = run_kernel(k.source, "fused_matmul", gx, threads, bufs + [(np.full(split * m * n, np.nan, dtype=np.float32), 2)], grid_y=gy)
         (out,) = outs
-        res = run_kernel(k.source, "fused_matmul_finalize", 2, 256, [(res[-1], 0), (np.zeros(out["numel"], dtype=nm.NP_STORAGE[out["dtype"]]), 1)])
+        res = run_kernel(k.source, "fused_matmul_finalize", (m * n + 31) // 32, 256, [(res[-1], 0), (np.zeros(out["numel"], dtype=nm.NP_STORAGE[out["dtype"]]), 1)])
     else:
         res = launch_gemm(k, bufs)
     return k, {a["node"]: nm.from_storage(r, a["dtype"], [r.size]).astype(np.float64) for a, r in zip(outs, res)}
@@ -264,6 +264,10 @@ CONV_CASES = [
     ("three_channel_image_7x7", (1, 10, 9, 3), 16, (7, 7), "bf16", (2, 2), (1, 1), "same", "128,128,64,2,2"),
     ("valid_and_dilated_f32", (1, 9, 9, 4), 8, (3, 3), "f32", (1, 1), (2, 1), "valid", "64,64,32,2,2"),
     ("full_padding_f16", (1, 6, 7, 8), 8, (3, 2), "f16", (1, 1), (1, 1), "full", "128,128,64,2,2"),
+    # 64 channels = one k-tile per filter tap: the gather keeps the pixel terms of its rows across the k-loop
+    ("hoisted_pixel_terms_ragged_rows", (2, 7, 9, 64), 32, (3, 3), "bf16", (1, 1), (1, 1), "same", "128,128,64,2,2"),
+    ("hoisted_pixel_terms_stride2_eight_waves", (1, 12, 10, 128), 64, (3, 3), "bf16", (2, 2), (1, 1), "same", "256,64,64,4,2"),
+    ("hoisted_pixel_terms_f32_dilated", (1, 9, 8, 32), 16, (3, 3), "f32", (1, 1), (2, 2), "valid", "64,64,32,2,2"),
 ]
 
 
@@ -281,6 +285,7 @@ def test_conv_on_cpu(name, image, oc, kernel, dtype, stride, dilation, mode, til
     want = nm.from_storage(want.reshape(-1), dtype, [want.size]).astype(np.float64)
     tol = 1e-4 if dtype == "f32" else 2e-2
     assert np.abs(got[y] - want).max() <= tol * max(1.0, np.abs(want).max()), (k.description, np.abs(got[y] - want).max())
+    assert ("#define CONV_A_FAST 1" in k.source) == name.startswith("hoisted"), name
 
 
 BWD_DATA_CASES = [
@@ -290,6 +295,7 @@ BWD_DATA_CASES = [
     ("1x1_stride2_shortcut", (2, 8, 8, 32), 64, (1, 1), "bf16", (2, 2), (1, 1), "same", "128,128,64,2,2"),
     ("direct_loads_both_operands", (1, 16, 16, 128), 64, (3, 3), "bf16", (1, 1), (1, 1), "same", "128,128,64,2,2"),
     ("valid_and_dilated_f32", (1, 9, 9, 4), 8, (3, 3), "f32", (1, 1), (2, 1), "valid", "64,64,32,2,2"),
+    ("hoisted_pixel_terms_stride2", (2, 10, 9, 16), 64, (3, 3), "bf16", (2, 2), (1, 1), "same", "128,128,64,2,2"),
 ]
 
 
