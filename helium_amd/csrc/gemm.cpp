@@ -1024,7 +1024,23 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         if (cv.C % epc == 0) {
             s << "u32x4 v = {0u, 0u, 0u, 0u};\nsize_t at;\nif (conv_tap(row, col, at)) v = *(const u32x4*)(q0 + at);\nreturn v;\n}\n";
         } else {
-            s << "float v[" << epc << "];\n#pragma unroll\nfor (int j = 0; j < " << epc << "; j++) {\nsize_t at;\nv[j] = conv_tap(row, col + j, at) ? ld_one(q0 + at) : 0.0f;\n}\n"
+            // EPC consecutive columns of one row: the pixel is decomposed once, and the tap walks on by one channel per
+            // element (a 3-channel image: 8 elements span 3 taps) instead of being decomposed 8 times
+            s << "float v[" << epc << "];\n"
+              << "const u32 n = row / " << cv.P * cv.Q << "u, pq = row % " << cv.P * cv.Q << "u, p = pq / " << cv.Q << "u, q = pq % " << cv.Q << "u;\n"
+              << "u32 rs = col / " << cv.C << "u, c = col % " << cv.C << "u, r = rs / " << cv.S << "u, sx = rs % " << cv.S << "u;\n"
+              << "const bool row_ok = row < " << cv.N * cv.P * cv.Q << "u;\n"
+              << "#pragma unroll\nfor (int j = 0; j < " << epc << "; j++) {\n";
+            if (!cv.bwd)
+                s << "const int ih = (int)(p * " << cv.sh << "u + r * " << cv.dh << "u) - " << cv.ph << ", iw = (int)(q * " << cv.sw << "u + sx * " << cv.dw << "u) - " << cv.pw << ";\n"
+                  << "const bool hit = true;\n";
+            else
+                s << "const int th = (int)p + " << cv.ph << " - (int)(r * " << cv.dh << "u), tw = (int)q + " << cv.pw << " - (int)(sx * " << cv.dw << "u);\n"
+                  << "const bool hit = th >= 0 && tw >= 0 && th % " << cv.sh << " == 0 && tw % " << cv.sw << " == 0;\n"
+                  << "const int ih = th / " << cv.sh << ", iw = tw / " << cv.sw << ";\n";
+            s << "const bool inside = row_ok && r < " << cv.R << "u && hit && ih >= 0 && ih < " << cv.H << " && iw >= 0 && iw < " << cv.W << ";\n"
+              << "v[j] = inside ? ld_one(q0 + (((size_t)n * " << cv.H << "u + (u32)ih) * " << cv.W << "u + (u32)iw) * " << cv.C << "u + c) : 0.0f;\n"
+              << "if (++c == " << cv.C << "u) { c = 0u; if (++sx == " << cv.S << "u) { sx = 0u; ++r; } }\n}\n"
               << "return pack_chunk(v);\n}\n";
         }
     } else if (pr.a_km) {

@@ -296,6 +296,7 @@ BWD_DATA_CASES = [
     ("direct_loads_both_operands", (1, 16, 16, 128), 64, (3, 3), "bf16", (1, 1), (1, 1), "same", "128,128,64,2,2"),
     ("valid_and_dilated_f32", (1, 9, 9, 4), 8, (3, 3), "f32", (1, 1), (2, 1), "valid", "64,64,32,2,2"),
     ("hoisted_pixel_terms_stride2", (2, 10, 9, 16), 64, (3, 3), "bf16", (2, 2), (1, 1), "same", "128,128,64,2,2"),
+    ("flow_gathered_element_by_element", (1, 9, 8, 16), 12, (3, 3), "bf16", (2, 1), (1, 1), "same", "64,64,64,2,2"),
 ]
 
 
