@@ -618,6 +618,103 @@ class SgdWorkload:
         self.tensors, self.last = {}, None
 
 
+class BasicBlockWorkload:
+    """One residual block of BASELINE config 5b's network, forward in Train mode (BasicBlock::forward,
+    resnet-train/src/model.rs:155-165): bn -> relu -> conv 3x3 -> bn -> relu -> conv 3x3 -> + shortcut on a bf16 NHWC
+    activation of [64,56,56,64], one graph through execute_graph. Work = the two convolutions' FLOP."""
+
+    bound = "mfma"
+    unit = "TFLOP/s"
+    dtype = "bf16 storage, bf16 x bf16 -> f32 products, f32 math"
+    name = "C5b-block"
+    wall_timed = True
+    shape = (64, 56, 56, 64)
+
+    def __init__(self):
+        n, h, w, c = self.shape
+        self.work = 2 * 2.0 * n * h * w * c * 9 * c
+
+    def describe(self):
+        return "C5b-block: bf16 [64,56,56,64] residual block forward (bn, relu, conv 3x3, bn, relu, conv 3x3, + shortcut) via execute_graph"
+
+    @staticmethod
+    def build(shape, seed):
+        import helium_amd as ha
+        from helium_amd import configs, frontend
+
+        g = ha.ir.OpGraph()
+        rec = frontend.Recorder(g)
+        c = shape[3]
+        x = g.new_input(list(shape), "bf16")
+        bn1 = [g.new_input([c], "f32") for _ in range(4)]
+        bn2 = [g.new_input([c], "f32") for _ in range(4)]
+        k1, b1 = g.new_input([c, 3, 3, c], "bf16"), g.new_input([c], "bf16")
+        k2, b2 = g.new_input([c, 3, 3, c], "bf16"), g.new_input([c], "bf16")
+        out, stats = frontend.basic_block_forward(rec, x, bn1, k1, b1, bn2, k2, b2)
+        outs = [g.new_output(out)] + [g.new_output(s) for s in stats]
+        rng = np.random.default_rng(seed)
+        host = {x: configs.bf16_rne(rng.standard_normal(shape, dtype=np.float32) * 1.2 + 0.2)}
+        for bn in (bn1, bn2):
+            host[bn[0]] = np.zeros(c, np.float32)
+            host[bn[1]] = np.ones(c, np.float32)
+            host[bn[2]] = rng.uniform(0.5, 1.5, c).astype(np.float32)
+            host[bn[3]] = rng.standard_normal(c).astype(np.float32) * 0.5
+        for k, b in ((k1, b1), (k2, b2)):
+            host[k] = configs.bf16_rne(rng.standard_normal((c, 3, 3, c), dtype=np.float32) * 0.06)   # Kaiming: sqrt(2 / (9 c))
+            host[b] = configs.bf16_rne(rng.standard_normal(c, dtype=np.float32) * 0.1)
+        host.update(rec.scalars)
+        return g, host, outs
+
+    def setup(self):
+        from helium_amd.backend import Plan, Tensor
+
+        self.graph, self.host, self.outs = self.build(self.shape, 59)
+        by_id = {n["id"]: n for n in self.graph.nodes}
+        self.tensors = {i: Tensor.from_numpy(a, by_id[i]["dtype"], int(np.prod(by_id[i]["shape"]))) for i, a in self.host.items()}
+        self.last = None
+        log(f"[bench] {self.describe()} :: plan: " + Plan(self.graph).text.replace("\n", " ; "))
+
+    def step(self, stream, i):
+        from helium_amd.backend import execute_graph
+
+        self.last = execute_graph(self.graph, self.tensors)
+
+    def check(self):
+        """The same graph at [4,12,12,64] against the oracle (kernel by kernel, as the plan groups it), and the full-size
+        run's running statistics of the first batch norm against the float64 closed form."""
+        from helium_amd.backend import Plan, Tensor, execute_graph
+        from oracle import helium_ir as oracle
+        from oracle import numerics as nm
+
+        g, host, outs = self.build((4, 12, 12, 64), 60)
+        by_id = {n["id"]: n for n in g.nodes}
+        got = execute_graph(g, {i: Tensor.from_numpy(a, by_id[i]["dtype"], int(np.prod(by_id[i]["shape"]))) for i, a in host.items()})
+        want = oracle.plan_outputs(g.nodes, host, Plan(g).steps)
+        _, desc = oracle.evaluate(g.nodes, host)
+        for o in outs:
+            dt = desc[o][1]
+            a = nm.from_storage(got[o].to_numpy(), dt, [got[o].len]).astype(np.float64)
+            b = nm.from_storage(want[o].reshape(-1), dt, [want[o].size]).astype(np.float64)
+            tol = 4e-2 if dt == "bf16" else 2e-3
+            if not np.allclose(a, b, rtol=tol, atol=tol):
+                raise SystemExit(f"[bench] PARITY FAILURE in C5b-block: output {o} differs from the oracle by {np.abs(a - b).max()}")
+        c = self.shape[3]
+        x = nm.bf16_bits_to_f32(self.host[next(iter(self.host))]).reshape(-1, c)
+        mean = x.mean(axis=0, dtype=np.float64)
+        var = (x.astype(np.float64) ** 2).mean(axis=0) - mean ** 2
+        got_mean = self.last[self.outs[1]].to_numpy().astype(np.float64)
+        got_var = self.last[self.outs[2]].to_numpy().astype(np.float64)
+        if not np.allclose(got_mean, 0.1 * mean, rtol=1e-3, atol=1e-4) or not np.allclose(got_var, 0.9 + 0.1 * var, rtol=1e-3, atol=1e-4):
+            raise SystemExit("[bench] PARITY FAILURE in C5b-block: running statistics differ from the closed form")
+        return "all outputs of the same graph at [4,12,12,64] within 4e-2 (bf16) / 2e-3 (f32) of the oracle; first batch norm's statistics at full size within 1e-3"
+
+    def cpu_baseline(self, budget_s=5.0):
+        return None
+
+    def free(self):
+        self.tensors, self.last = {}, None
+
+
 class FusedGemmWorkload:
     """BASELINE configs 4 / 5a: 4096^3 bf16 GEMM with fused mainloop / epilogue. Work = 2*M*N*K FLOP."""
 
@@ -763,6 +860,7 @@ def make_workloads():
     w["C5b-conv-bwd-data"] = ConvBackwardDataWorkload()
     w["C5b-conv-bwd-filter"] = ConvBackwardFilterWorkload()
     w["C5b-sgd"] = SgdWorkload()
+    w["C5b-block"] = BasicBlockWorkload()
     for name in ("C4", "C5a", "C4m", "GEMM"):
         w[name] = FusedGemmWorkload(name)
     return w

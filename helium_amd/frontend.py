@@ -97,3 +97,27 @@ def sgd_momentum_step(rec, weights, gradient, average, momentum=0.9, learning_ra
     updated = g.binary(rec.mul_scalar(gradient, 1.0 - momentum), rec.mul_scalar(average, momentum), "add")
     new_weights = sub(g, weights, rec.mul_scalar(updated, learning_rate))
     return new_weights, g.change_data_type(updated, "f32")
+
+
+def conv2d(g, x, kernel, bias, params):
+    """Conv2d::forward (helium/src/modules/conv.rs:62-68): the convolution, plus the bias broadcast over the pixels."""
+    y = g.conv(x, kernel, params)
+    if bias is not None:
+        shape, _ = g.descriptor(y)
+        y = g.binary(y, broadcast_to(g, bias, [shape[3]], shape), "add")
+    return y
+
+
+def basic_block_forward(rec, x, bn1, kernel1, bias1, bn2, kernel2, bias2):
+    """BasicBlock::forward in Train mode (resnet-train/src/model.rs:155-165): bn1 -> relu -> conv1 -> bn2 -> relu ->
+    conv2 -> + shortcut, 3x3 convolutions that keep the channel count. `bn1` / `bn2`: (running mean, running variance,
+    scale, bias). Returns (output, [new running mean 1, new running variance 1, new running mean 2, ...])."""
+    g = rec.g
+    shape, _ = g.descriptor(x)
+    c = shape[3]
+    params = {"in_channels": c, "out_channels": c, "kernel_size": [3, 3]}
+    h, m1, v1 = batch_norm_train(rec, x, *bn1, relu=True)
+    h = conv2d(g, h, kernel1, bias1, params)
+    h, m2, v2 = batch_norm_train(rec, h, *bn2, relu=True)
+    h = conv2d(g, h, kernel2, bias2, params)
+    return g.binary(h, x, "add"), [m1, v1, m2, v2]

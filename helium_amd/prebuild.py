@@ -59,6 +59,15 @@ def prebuild_kernels(verbose=True):
     n += 1
     g = ir.OpGraph()
     rec = frontend.Recorder(g)
+    block = [[g.new_input([64], "f32") for _ in range(4)], g.new_input([64, 3, 3, 64], "bf16"), g.new_input([64], "bf16")]
+    block += [[g.new_input([64], "f32") for _ in range(4)], g.new_input([64, 3, 3, 64], "bf16"), g.new_input([64], "bf16")]
+    out, stats = frontend.basic_block_forward(rec, g.new_input([64, 56, 56, 64], "bf16"), *block)
+    for v in [out] + stats:
+        g.new_output(v)
+    Plan(g).precompile()
+    n += 1
+    g = ir.OpGraph()
+    rec = frontend.Recorder(g)
     shape = [512, 3, 3, 512]
     new_w, new_avg = frontend.sgd_momentum_step(rec, g.new_input(shape, "bf16"), g.new_input(shape, "bf16"), g.new_input(shape, "f32"))
     g.new_output(new_w)

@@ -224,6 +224,45 @@ def test_batch_norm_train_step(gpu, fold):
         assert np.allclose(a, b, rtol=tol, atol=tol), (o, np.abs(a - b).max())
 
 
+def test_residual_block_forward(gpu):
+    """BasicBlock::forward in Train mode (resnet-train/src/model.rs:155-165) through execute_graph: the first convolution's
+    instruction takes its bias and the second batch norm's statistics, the second one its bias and the shortcut add."""
+    from helium_amd import frontend
+
+    shape = [4, 12, 10, 64]
+    c = shape[3]
+    rng = np.random.default_rng(41)
+    g = ha.ir.OpGraph()
+    rec = frontend.Recorder(g)
+    x = g.new_input(shape, "bf16")
+    bn1 = [g.new_input([c], "f32") for _ in range(4)]
+    bn2 = [g.new_input([c], "f32") for _ in range(4)]
+    k1, b1 = g.new_input([c, 3, 3, c], "bf16"), g.new_input([c], "bf16")
+    k2, b2 = g.new_input([c, 3, 3, c], "bf16"), g.new_input([c], "bf16")
+    out, stats = frontend.basic_block_forward(rec, x, bn1, k1, b1, bn2, k2, b2)
+    outs = [g.new_output(out)] + [g.new_output(v) for v in stats]
+    host = {x: nm.to_storage((rng.standard_normal(shape) * 1.2 + 0.2).astype(np.float32), "bf16")}
+    for bn in (bn1, bn2):
+        host.update({bn[0]: rng.standard_normal(c).astype(np.float32), bn[1]: rng.uniform(0.5, 2.0, c).astype(np.float32),
+                     bn[2]: rng.uniform(0.5, 1.5, c).astype(np.float32), bn[3]: (rng.standard_normal(c) * 0.5).astype(np.float32)})
+    for k, b in ((k1, b1), (k2, b2)):
+        host[k] = nm.to_storage((rng.standard_normal((c, 3, 3, c)) * 0.06).astype(np.float32), "bf16")
+        host[b] = nm.to_storage((rng.standard_normal(c) * 0.1).astype(np.float32), "bf16")
+    host.update(rec.scalars)
+    got, steps = run_graph(g, host)
+    gemms = [members for instrs, _ in steps for kind, members in instrs if kind == "gemm"]
+    by_id = {n["id"]: n for n in g.nodes}
+    assert len(gemms) == 2 and sorted(by_id[m]["op"] for m in gemms[0]).count("reduce") == 2, steps
+    assert [by_id[m]["op"] for m in gemms[1]].count("binary") == 2, steps   # bias and shortcut
+    want = oracle_ir.plan_outputs(g.nodes, host, steps)
+    _, desc = oracle_ir.evaluate(g.nodes, host)
+    for o in outs:
+        a = nm.from_storage(got[o], desc[o][1], [got[o].size]).astype(np.float64)
+        b = nm.from_storage(want[o].reshape(-1), desc[o][1], [want[o].size]).astype(np.float64)
+        tol = 4e-2 if desc[o][1] == "bf16" else 2e-3
+        assert np.allclose(a, b, rtol=tol, atol=tol), (o, np.abs(a - b).max())
+
+
 @pytest.mark.parametrize("image,oc", [((8, 28, 28, 64), 64), ((4, 30, 26, 32), 128), ((64, 14, 14, 64), 64)])
 def test_convolution_takes_the_batch_norm_statistics_of_its_output(gpu, image, oc):
     """conv -> BatchNorm2d(train) -> relu through execute_graph: the convolution's kernel also folds its output per
