@@ -23,7 +23,7 @@ def build(verbose=True, jobs=8):
     hipcc = os.path.join(ROCM, "bin", "hipcc")
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
-    flags = ["-O2", "-g0", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-Wno-unused-parameter",
+    flags = ["-O2", "-g0", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-Wno-unused-parameter", "-Wno-c++20-extensions",
              "-D__HIP_PLATFORM_AMD__", f"-I{ROCM}/include"]
     procs = []
     objs = []
