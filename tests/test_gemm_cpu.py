@@ -268,6 +268,10 @@ CONV_CASES = [
     ("hoisted_pixel_terms_ragged_rows", (2, 7, 9, 64), 32, (3, 3), "bf16", (1, 1), (1, 1), "same", "128,128,64,2,2"),
     ("hoisted_pixel_terms_stride2_eight_waves", (1, 12, 10, 128), 64, (3, 3), "bf16", (2, 2), (1, 1), "same", "256,64,64,4,2"),
     ("hoisted_pixel_terms_f32_dilated", (1, 9, 8, 32), 16, (3, 3), "f32", (1, 1), (2, 2), "valid", "64,64,32,2,2"),
+    # channel counts that are no multiple of a chunk: gathered element by element
+    ("odd_channels_five_3x3", (2, 7, 6, 5), 16, (3, 3), "bf16", (1, 1), (1, 1), "same", "64,64,64,2,2"),
+    ("odd_channels_three_f32_full", (1, 6, 5, 3), 8, (3, 3), "f32", (1, 1), (2, 1), "full", "64,64,32,2,2"),
+    ("odd_channels_three_5x5_stride3", (1, 11, 13, 3), 8, (5, 5), "f16", (3, 3), (1, 1), "same", "64,64,64,2,2"),
 ]
 
 
