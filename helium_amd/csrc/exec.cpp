@@ -16,18 +16,6 @@ DevicePool& DevicePool::global() {
     return *pool;
 }
 
-size_t DevicePool::size_class(size_t bytes) {
-    // 256-byte granules up to 1 MiB, then 2 MiB granules: few distinct sizes, so freed blocks get reused
-    if (bytes == 0) bytes = 1;
-    if (bytes <= (1u << 20)) {
-        size_t c = 256;
-        while (c < bytes) c *= 2;
-        return c;
-    }
-    const size_t g = 2u << 20;
-    return (bytes + g - 1) / g * g;
-}
-
 SharedEvent::~SharedEvent() {
     if (e) DevicePool::global().recycle(e);
 }
@@ -50,7 +38,7 @@ void DevicePool::poll() {
     {
         std::lock_guard<std::mutex> lk(mu_);
         while (!pending_.empty() && hipEventQuery(pending_.front().second->e) == hipSuccess) {
-            end_scope_locked(pending_.front().first);
+            if (blocks_.stream_is_live(pending_.front().first)) blocks_.end_stream(pending_.front().first);
             passed.push_back(std::move(pending_.front().second));
             pending_.pop_front();
         }
@@ -74,105 +62,86 @@ EventRef DevicePool::take_event() {
 uint64_t DevicePool::begin_scope(uint64_t thread) {
     poll();
     std::lock_guard<std::mutex> lk(mu_);
-    uint64_t s = next_scope_++;
-    free_scoped_[s];
-    scope_thread_[s] = thread;
+    uint64_t parent = 0;
+    if (thread) {
+        auto it = thread_last_scope_.find(thread);
+        if (it != thread_last_scope_.end() && blocks_.stream_is_live(it->second)) parent = it->second;
+    }
+    const uint64_t s = blocks_.begin_stream(parent);
+    if (thread) thread_last_scope_[thread] = s;
     return s;
 }
 
 void DevicePool::end_scope(uint64_t scope) {
     std::lock_guard<std::mutex> lk(mu_);
-    end_scope_locked(scope);
+    if (blocks_.stream_is_live(scope)) blocks_.end_stream(scope);
 }
 
-void DevicePool::end_scope_locked(uint64_t scope) {
-    auto it = free_scoped_.find(scope);
-    if (it == free_scoped_.end()) return;
-    for (auto& kv : it->second) free_global_.insert(kv);
-    free_scoped_.erase(it);
-    scope_thread_.erase(scope);
-    for (size_t i = 0; i < deferred_.size();) {
-        auto& w = deferred_[i].waiting;
-        w.erase(std::remove(w.begin(), w.end(), scope), w.end());
-        if (w.empty()) {
-            free_global_.insert({deferred_[i].cls, deferred_[i].ptr});
-            deferred_[i] = deferred_.back();
-            deferred_.pop_back();
-        } else {
-            i++;
+size_t DevicePool::live_scopes() {
+    std::lock_guard<std::mutex> lk(mu_);
+    return blocks_.num_streams();
+}
+
+void DevicePool::note_locked(Tensor& t, uint64_t scope) {
+    size_t kept = 0;
+    bool present = false;
+    for (uint64_t s : t.used)
+        if (blocks_.stream_is_live(s)) {
+            t.used[kept++] = s;
+            present = present || s == scope;
         }
-    }
+    t.used.resize(kept);
+    if (!present) t.used.push_back(scope);
 }
 
 void DevicePool::note_use(Tensor& t, uint64_t scope) {
     std::lock_guard<std::mutex> lk(mu_);
-    if (std::find(t.used.begin(), t.used.end(), scope) == t.used.end()) t.used.push_back(scope);
+    note_locked(t, scope);
 }
 
 void DevicePool::note_uses(const std::map<ir::NodeId, TensorRef>& tensors, uint64_t scope) {
     std::lock_guard<std::mutex> lk(mu_);
-    for (auto& kv : tensors) {
-        Tensor& t = *kv.second;
-        if (std::find(t.used.begin(), t.used.end(), scope) == t.used.end()) t.used.push_back(scope);
-    }
+    for (auto& kv : tensors) note_locked(*kv.second, scope);
 }
 
-void* DevicePool::allocate(size_t bytes, uint64_t scope) {
-    const size_t cls = size_class(bytes);
-    {
+Allocation DevicePool::allocate(size_t bytes, uint64_t scope) {
+    // sizes are rounded up to the alignment so that small requests do not fragment the pages (device.rs:104-108)
+    const uint64_t size = std::max<uint64_t>((bytes + kAlign - 1) / kAlign * kAlign, kAlign);
+    Allocation a;
+    for (int attempt = 0; attempt < 2; attempt++) {
+        if (attempt == 1) poll();  // blocks of executions that have finished since become available
         std::lock_guard<std::mutex> lk(mu_);
-        auto take = [&](std::multimap<size_t, void*>& m) -> void* {
-            auto it = m.find(cls);
-            if (it == m.end()) return nullptr;
-            void* p = it->second;
-            m.erase(it);
+        if (blocks_.allocate(size, kAlign, scope, &a.block)) {
+            a.ptr = page_base_[a.block.page] + a.block.start;
             reuses_++;
-            return p;
-        };
-        auto sc = free_scoped_.find(scope);
-        if (sc != free_scoped_.end())
-            if (void* p = take(sc->second)) return p;
-        // blocks freed by this thread's earlier executions that are still queued: this one runs after them
-        auto mine = scope_thread_.find(scope);
-        if (mine != scope_thread_.end() && mine->second != 0)
-            for (auto& other : scope_thread_)
-                if (other.second == mine->second && other.first != scope)
-                    if (void* p = take(free_scoped_[other.first])) return p;
-        if (void* p = take(free_global_)) return p;
-    }
-    poll();  // blocks of executions that have finished since become available
-    {
-        std::lock_guard<std::mutex> lk(mu_);
-        auto it = free_global_.find(cls);
-        if (it != free_global_.end()) {
-            void* p = it->second;
-            free_global_.erase(it);
-            reuses_++;
-            return p;
+            return a;
         }
-        driver_bytes_ += cls;
-        driver_allocs_++;
     }
-    void* p = nullptr;
-    HE_HIP(hipMalloc(&p, cls));
-    return p;
+    // a new page: at least 1 GiB, a power of two (device.rs:144-154)
+    uint64_t page = kMinPage;
+    while (page < size) page *= 2;
+    void* base = nullptr;
+    HE_HIP(hipMalloc(&base, page));
+    std::lock_guard<std::mutex> lk(mu_);
+    const alloc::PageId id = blocks_.add_page(page);
+    if (page_base_.size() <= id) page_base_.resize(id + 1);
+    page_base_[id] = (char*)base;
+    driver_bytes_ += page;
+    driver_allocs_++;
+    HE_REQUIRE(blocks_.allocate(size, kAlign, scope, &a.block), HE_ERR_INTERNAL, "a new page does not hold the allocation");
+    a.ptr = page_base_[a.block.page] + a.block.start;
+    return a;
 }
 
-void DevicePool::release(void* ptr, size_t bytes, uint64_t owner, const std::vector<uint64_t>& used) {
-    if (!ptr) return;
+void DevicePool::release(const Allocation& a, uint64_t owner, const std::vector<uint64_t>& used) {
+    if (!a.ptr) return;
     std::lock_guard<std::mutex> lk(mu_);
-    const size_t cls = size_class(bytes);
-    std::vector<uint64_t> live;
+    alloc::Block b = a.block;
+    b.in_use.clear();
+    if (owner && blocks_.stream_is_live(owner)) b.in_use.insert(owner);
     for (uint64_t s : used)
-        if (s != owner && free_scoped_.count(s)) live.push_back(s);
-    auto own = free_scoped_.find(owner);
-    if (live.empty()) {
-        if (own != free_scoped_.end()) own->second.insert({cls, ptr});
-        else free_global_.insert({cls, ptr});
-        return;
-    }
-    if (own != free_scoped_.end()) live.push_back(owner);
-    deferred_.push_back({ptr, cls, std::move(live)});
+        if (blocks_.stream_is_live(s)) b.in_use.insert(s);
+    blocks_.deallocate(std::move(b));
 }
 
 void DevicePool::stats(uint64_t* driver_bytes, uint64_t* driver_allocs, uint64_t* reuses) {
@@ -187,7 +156,10 @@ void DevicePool::stats(uint64_t* driver_bytes, uint64_t* driver_allocs, uint64_t
 // ---------------------------------------------------------------------------------------------------------
 Tensor::~Tensor() {
     if (ready && uploaded) (void)hipEventSynchronize(ready->e);  // the copy that fills the block may still be queued
-    DevicePool::global().release(ptr, bytes, scope, used);
+    Allocation a;
+    a.ptr = ptr;
+    a.block = block;
+    DevicePool::global().release(a, scope, used);
 }
 
 TensorRef allocate_tensor(int dtype, size_t len, uint64_t scope) {
@@ -196,7 +168,9 @@ TensorRef allocate_tensor(int dtype, size_t len, uint64_t scope) {
     t->len = len;
     t->bytes = storage_bytes(dtype, len);
     t->scope = scope;
-    t->ptr = DevicePool::global().allocate(t->bytes, scope);
+    Allocation a = DevicePool::global().allocate(t->bytes, scope);
+    t->ptr = a.ptr;
+    t->block = std::move(a.block);
     return t;
 }
 
@@ -297,6 +271,13 @@ struct HostTimer {
         if (on()) t = std::chrono::steady_clock::now();
     }
 };
+// Join events of an execution are destroyed one execution later on the same thread: by then they were recorded and
+// waited on long ago.
+void retire_join_events(const std::vector<hipEvent_t>& events) {
+    static thread_local std::vector<hipEvent_t> garbage;
+    for (hipEvent_t e : garbage) (void)hipEventDestroy(e);
+    garbage = events;
+}
 thread_local double g_host_acc[8] = {0};
 thread_local int g_host_calls = 0;
 }  // namespace
@@ -335,10 +316,10 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
     const std::set<NodeId>& alive = prepared.alive;
     DevicePool& pool = DevicePool::global();
     Streams& st = thread_streams();
+    for (NodeId in : graph->inputs())
+        HE_REQUIRE(inputs.count(in), HE_ERR_INVALID, "missing storage for input node %u", in);
     const uint64_t scope = pool.begin_scope((uint64_t)(uintptr_t)&st);
     std::map<NodeId, TensorRef> tensors = inputs;
-    for (NodeId in : graph->inputs())
-        HE_REQUIRE(tensors.count(in), HE_ERR_INVALID, "missing storage for input node %u", in);
     pool.note_uses(tensors, scope);
     ht.lap(2);
     ExecStats local;
@@ -377,6 +358,10 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
     }
     EventRef done = pool.take_event();
     bool done_recorded = false;
+    // Whatever happens below, the scope must end, and only after the work already queued: a failing instruction leaves
+    // earlier launches running on up to four streams. On failure stream 0 is ordered after every stream this execution
+    // used, the end event is recorded there as usual, and the error goes on to the caller.
+    try {
     for (auto& step : plan->steps) {
         for (NodeId r : step.tensors_to_release) tensors.erase(r);
         if (step.instrs.empty()) continue;
@@ -433,6 +418,21 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
         synced.insert(waited.begin(), waited.end());
         prev_streams = cur;
     }
+    } catch (...) {
+        try {
+            prev_streams.assign(used_streams.begin(), used_streams.end());
+            join({0});
+            HE_HIP(hipEventRecord(done->e, st.s[0]));
+            st.exec_end = done;
+            st.has_run = true;
+            pool.end_scope_after(scope, done);
+        } catch (...) {
+            (void)hipDeviceSynchronize();
+            pool.end_scope(scope);
+        }
+        retire_join_events(events);
+        throw;
+    }
     ht.lap(3);
     // Drop of the executor (cuda.rs:232-260): when everything queued above has run, the scope's freed blocks
     // become available to everyone. Stream 0 joins the last step and carries the event the pool polls.
@@ -444,12 +444,7 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
     st.exec_end = done;
     st.has_run = true;
     pool.end_scope_after(scope, std::move(done));
-    {
-        // join events of the previous execution on this thread: recorded and waited on long ago
-        static thread_local std::vector<hipEvent_t> garbage;
-        for (hipEvent_t e : garbage) (void)hipEventDestroy(e);
-        garbage = events;
-    }
+    retire_join_events(events);
     local.streams_used = (int)used_streams.size();
     if (stats) *stats = local;
 

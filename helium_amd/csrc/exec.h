@@ -9,6 +9,7 @@
 #include <mutex>
 #include <vector>
 
+#include "alloc.h"
 #include "plan.h"
 
 namespace he::exec {
@@ -24,56 +25,62 @@ struct SharedEvent {
 };
 using EventRef = std::shared_ptr<SharedEvent>;
 
-// Pooling device allocator (helium/src/cuda/allocator/device.rs): memory is never returned to the driver; a block
-// freed inside an execution scope is reusable by that scope at once and by everyone else when the scope has ended
-// on the device (device.rs:60-89, block.rs:216-244).
+// A piece of device memory handed out by the pool: its address and the block of the page it was cut from.
+struct Allocation {
+    void* ptr = nullptr;
+    alloc::Block block;
+};
+
+// Pooling device allocator (helium/src/cuda/allocator/device.rs): pages of at least 1 GiB (a power of two) come from
+// the driver and are never returned; inside them a best-fit block allocator with coalescing hands out 256-byte
+// aligned blocks. An execution is a logical allocation stream ("scope"): a block freed inside a scope is reusable by
+// that scope and by later scopes of the same host thread at once (their device work is ordered after it), and by
+// everyone else when the scope has ended on the device (device.rs:60-89, block.rs:216-244).
 class DevicePool {
 public:
+    static constexpr uint64_t kAlign = 256;             // alignment of every block (device.rs:33)
+    static constexpr uint64_t kMinPage = 1ull << 30;    // device.rs:35
     static DevicePool& global();
-    // `thread`: a token of the calling host thread. The executions of one thread are ordered on the device (each
-    // waits for the end of the one before), so a later one may take the blocks an earlier one has freed at once.
+    // `thread`: a token of the calling host thread (0: none). The executions of one thread are ordered on the device
+    // (each waits for the end of the one before), so the thread's previous scope is the new scope's parent.
     uint64_t begin_scope(uint64_t thread = 0);
     void end_scope(uint64_t scope);  // called once the scope's device work has finished
     // Ends the scope once `done` (recorded after all of its device work) has completed; polled from begin_scope and
     // from allocate, so no host callback sits in any stream.
     void end_scope_after(uint64_t scope, EventRef done);
     void poll();
-    void* allocate(size_t bytes, uint64_t scope);
-    // `owner`: the scope the block was allocated in (0: none); `used`: every scope whose device work touches it.
-    // The block goes to the owner's free list while only the owner can still touch it, to the global list when no
-    // live scope can, and otherwise waits until the last such scope has ended on the device.
-    void release(void* ptr, size_t bytes, uint64_t owner, const std::vector<uint64_t>& used);
+    Allocation allocate(size_t bytes, uint64_t scope);
+    // `owner`: the scope the block was allocated in (0: none); `used`: every scope whose device work touches it. The
+    // block is free again for whoever comes after all of those that are still live.
+    void release(const Allocation& a, uint64_t owner, const std::vector<uint64_t>& used);
     void note_use(struct Tensor& t, uint64_t scope);
     void note_uses(const std::map<ir::NodeId, std::shared_ptr<struct Tensor>>& tensors, uint64_t scope);
     EventRef take_event();          // an event nobody holds any more, or a new one
     void recycle(hipEvent_t event);  // called when an event's last holder lets go
     void stats(uint64_t* driver_bytes, uint64_t* driver_allocs, uint64_t* reuses);
+    size_t live_scopes();
 
 private:
-    static size_t size_class(size_t bytes);
     std::mutex mu_;
-    std::multimap<size_t, void*> free_global_;
-    std::map<uint64_t, std::multimap<size_t, void*>> free_scoped_;  // one entry per live scope
-    std::map<uint64_t, uint64_t> scope_thread_;                     // live scope -> thread token
-    struct Deferred {
-        void* ptr;
-        size_t cls;
-        std::vector<uint64_t> waiting;
-    };
-    std::vector<Deferred> deferred_;
+    alloc::BlockAllocator blocks_;
+    std::vector<char*> page_base_;                   // by page id
+    std::map<uint64_t, uint64_t> thread_last_scope_;  // thread token -> its latest scope
     std::deque<std::pair<uint64_t, EventRef>> pending_;  // scopes whose device work may still be running, oldest first
     std::vector<hipEvent_t> spare_events_;
-    void end_scope_locked(uint64_t scope);
-    uint64_t next_scope_ = 1, driver_bytes_ = 0, driver_allocs_ = 0, reuses_ = 0;
+    void note_locked(struct Tensor& t, uint64_t scope);
+    uint64_t driver_bytes_ = 0, driver_allocs_ = 0, reuses_ = 0;
 };
 
 // TensorStorage (helium/src/cuda/tensor_storage.rs:31-42): device buffer + ready event; shared by reference count.
 struct Tensor {
     void* ptr = nullptr;
+    alloc::Block block;  // where `ptr` lies in the pool's pages
     size_t bytes = 0, len = 0;
     int dtype = HE_F32;
     uint64_t scope = 0;
-    std::vector<uint64_t> used;  // execution scopes that read or wrote the tensor (guarded by the pool's mutex)
+    // Live execution scopes that read or wrote the tensor (guarded by the pool's mutex); scopes that have ended on
+    // the device are dropped whenever another one is noted, so a long-lived tensor's list stays short.
+    std::vector<uint64_t> used;
     bool uploaded = false;       // filled by an asynchronous host-to-device copy
     std::atomic<bool> ready_seen{false};  // `ready` has been observed complete (it is recorded once per tensor)
     // Recorded after the work that fills the tensor: the upload's own event, or the one event its execution records

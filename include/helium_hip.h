@@ -350,6 +350,39 @@ int he_backend_set_option(int option, int64_t value);
  * [7] driver allocations, [8] pooled reuses. */
 int he_backend_stats(uint64_t stats[9]);
 
+/* ---- device memory pool ------------------------------------------------------------------------------------------
+ * helium/src/cuda/allocator/block.rs (BlockAllocator: best-fit free blocks, coalescing, logical allocation streams)
+ * and allocator/device.rs (DeviceAllocator: pages from the driver, never returned). The block allocator is pure host
+ * logic over address ranges and needs no device. */
+typedef struct he_block_allocator_s* he_block_allocator_t;
+typedef struct he_block {
+    uint32_t page;
+    uint64_t start, size;
+    uint64_t streams[8]; /* streams whose device work may still touch the block (Block::in_use_by_streams) */
+    int32_t num_streams;
+} he_block;
+int he_block_allocator_create(he_block_allocator_t* allocator);            /* BlockAllocator::new, block.rs:17-19 */
+int he_block_allocator_destroy(he_block_allocator_t allocator);
+int he_block_allocator_add_page(he_block_allocator_t allocator, uint64_t size, uint32_t* page); /* add_page :22-34 */
+/* allocate (block.rs:37-118); stream 0 = None. *found = 0 when no free block fits (the Rust None). */
+int he_block_allocator_allocate(he_block_allocator_t allocator, uint64_t size, uint64_t align, uint64_t stream,
+                                he_block* block, int* found);
+int he_block_allocator_deallocate(he_block_allocator_t allocator, const he_block* block);       /* :124-127 */
+int he_block_allocator_begin_stream(he_block_allocator_t allocator, uint64_t parent, uint64_t* stream); /* :216-231 */
+int he_block_allocator_end_stream(he_block_allocator_t allocator, uint64_t stream);                    /* :233-244 */
+/* [0] free blocks, [1] free bytes, [2] largest free block, [3] live streams; also checks the allocator's indices
+ * against each other and fails with HE_ERR_INTERNAL if they disagree. */
+int he_block_allocator_stats(he_block_allocator_t allocator, uint64_t stats[4]);
+
+/* DeviceAllocator (allocator/device.rs): begin_stream / end_stream (:78-89), allocate_in_stream (:66-73; scope 0 =
+ * allocate, :57-59) and the drop of a DeviceMemory (:181-185). `thread` is any non-zero token of the calling host
+ * thread whose scopes run one after the other on the device (0: none); he_pool_end_scope is for a caller that knows
+ * the scope's device work has finished. */
+int he_pool_begin_scope(uint64_t thread, uint64_t* scope);
+int he_pool_end_scope(uint64_t scope);
+int he_pool_allocate(size_t bytes, uint64_t scope, void** ptr, he_block* block);
+int he_pool_release(void* ptr, const he_block* block, uint64_t scope);
+
 #ifdef __cplusplus
 }
 #endif

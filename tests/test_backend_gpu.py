@@ -86,24 +86,80 @@ def test_large_swap_chain_runs_as_one_permute_and_is_bit_exact(gpu):
     assert np.array_equal(out.reshape(64, 256, 56, 56), np.transpose(x, (0, 3, 1, 2)))
 
 
+def live_nodes(nodes):
+    """The nodes OpGraph::optimize keeps (helium-ir/src/opgraph.rs:165-191): those an Output node reaches."""
+    by_id = {n["id"]: n for n in nodes}
+    stack = [n["id"] for n in nodes if n["node"] == "output"]
+    seen = set()
+    while stack:
+        i = stack.pop()
+        if i in seen:
+            continue
+        seen.add(i)
+        n = by_id[i]
+        stack += [n["from"]] if n["node"] == "output" else list(n.get("inputs", []))
+    return [n for n in nodes if n["id"] in seen]
+
+
+@pytest.mark.parametrize("grouping", ["reference", "default"])
 @pytest.mark.parametrize("seed", range(24))
-def test_random_graphs_execute(gpu, seed):
+def test_random_graphs_execute(gpu, seed, grouping):
+    """Random graphs of 8x8, 1024x1024 and 1100x1100 tensors through plan generation and the executor: steps with several
+    instructions on several streams, scoped block reuse, and (from 1,000,000 elements) SwapDims chains that run as
+    permute instructions in the middle of a graph. With the reference's grouping rules the plan the library runs must
+    be the one the CPU restatement of plan_generation.rs derives, and that plan - not the library's - tells the oracle
+    where values are rounded to their storage type."""
+    from helium_amd.backend import OPT_FOLD_SWAP_INTO_REDUCE, OPT_FUSE_MATMUL_EPILOGUE, set_option
+    from oracle import plan as oracle_plan
+
     g = plans.random_graph(seed)
-    if g.nodes[0]["shape"][0] != 8:
-        pytest.skip("large-extent variants are plan-only cases")
-    if not any(n["node"] == "output" for n in g.nodes):
+    n = g.nodes[0]["shape"][0]
+    if not any(nd["node"] == "output" for nd in g.nodes):
         pytest.skip("graph without outputs")
-    host = seeded_inputs(g, seed)
-    got, steps = run_graph(g, host)
+    nodes = live_nodes(g.nodes)
+    g.optimize()
+    # large extents: small operands keep a first product well inside f32 (a product of exp'ed values then overflows to
+    # infinity on both sides alike)
+    rng = np.random.default_rng(seed)
+    scale = 1.0 if n == 8 else 1.0 / 32
+    host = {nd["id"]: (rng.uniform(-1, 1, nd["shape"]) * scale).astype(np.float32) for nd in nodes if nd["node"] == "input"}
+    reference = grouping == "reference"
+    set_option(OPT_FUSE_MATMUL_EPILOGUE, 0 if reference else 1)
+    set_option(OPT_FOLD_SWAP_INTO_REDUCE, 0 if reference else 1)
+    try:
+        got, steps = run_graph(g, host)
+    finally:
+        set_option(OPT_FUSE_MATMUL_EPILOGUE, 1)
+        set_option(OPT_FOLD_SWAP_INTO_REDUCE, 1)
+    if reference:
+        want_steps = oracle_plan.generate_plan(nodes)
+        assert steps == want_steps
+        steps = want_steps
+        if n * n > 1_000_000 and any(nd.get("op") == "swap_dims" for nd in nodes):
+            assert any(k == "permute" for instrs, _ in steps for k, _ in instrs)
     # chains of exp/tanh over matmuls amplify 1-ulp differences; the bound here is on the whole graph
-    want = oracle_ir.plan_outputs(g.nodes, host, steps)
-    _, desc = oracle_ir.evaluate(g.nodes, host)
+    want = oracle_ir.plan_outputs(nodes, host, steps)
+    _, desc = oracle_ir.evaluate(nodes, host)
+    assert sorted(got) == sorted(want)
     for o in want:
         a = nm.from_storage(got[o], desc[o][1], [got[o].size]).astype(np.float64)
         b = nm.from_storage(want[o].reshape(-1), desc[o][1], [want[o].size]).astype(np.float64)
         fin = np.isfinite(b)
-        assert np.array_equal(np.isfinite(a), fin)
+        assert np.array_equal(np.isfinite(a), fin), (o, steps)
         assert np.allclose(a[fin], b[fin], rtol=2e-2 if desc[o][1] == "bf16" else 1e-3, atol=1e-5), (o, steps)
+
+
+def test_random_graphs_cover_concurrent_steps_and_permute_instructions():
+    """What the random cases above are there for: plans with several instructions in one step and plans with a permute
+    instruction are among them (the plans are generated without a device)."""
+    multi = permute = 0
+    for seed in range(24):
+        g = plans.random_graph(seed)
+        g.optimize()
+        kinds = [[k for k, _ in instrs] for instrs, _ in Plan(g).steps]
+        multi += any(len(k) > 1 for k in kinds)
+        permute += any("permute" in k for k in kinds)
+    assert multi >= 12 and permute >= 8, (multi, permute)
 
 
 @pytest.mark.parametrize("fuse", [1, 0], ids=["matmul_takes_its_epilogue", "reference_grouping"])
