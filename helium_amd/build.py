@@ -15,7 +15,8 @@ ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
 
 def sources():
-    return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".cpp"))
+    """Host C++ (.cpp) and the one file with device data (.hip, compiled for gfx950)."""
+    return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".cpp", ".hip")))
 
 
 def build(verbose=True, jobs=8):
@@ -30,14 +31,18 @@ def build(verbose=True, jobs=8):
     for src in sources():
         obj = os.path.join(objdir, os.path.basename(src)[:-4] + ".o")
         objs.append(obj)
-        cmd = [hipcc, "-x", "c++", *flags, "-c", src, "-o", obj]
+        if src.endswith(".hip"):
+            cmd = [hipcc, "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                   *[f for f in flags if f != "-D__HIP_PLATFORM_AMD__"], "-c", src, "-o", obj]
+        else:
+            cmd = [hipcc, "-x", "c++", *flags, "-c", src, "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd)))
         if len(procs) >= jobs:
             _wait(procs)
     _wait(procs)
-    link = [hipcc, "-shared", "-o", LIB, *objs, f"-L{ROCM}/lib", "-lamdhip64", "-lhiprtc", "-lpthread", "-ldl",
+    link = [hipcc, "--offload-arch=gfx950", "-shared", "-o", LIB, *objs, f"-L{ROCM}/lib", "-lamdhip64", "-lhiprtc", "-lpthread", "-ldl",
             f"-Wl,-rpath,{ROCM}/lib", "-Wl,--no-undefined"]
     if verbose:
         print(" ".join(link), flush=True)

@@ -109,6 +109,7 @@ int he_pointwise_create(he_tile_kernel_t* kernel, he_graph_t graph, const uint32
         he::ir::OpSubgraph sg(graph->g, std::vector<he::ir::NodeId>(nodes, nodes + num_nodes));
         auto k = std::make_unique<he_tile_kernel_s>();
         k->k.reset(new he::TileKernel(he::tp::lower_pointwise(sg), "pointwise_kernel"));
+        if (he::device_initialised()) k->k->load();  // so that later launches need not
         *kernel = k.release();
     });
 }
@@ -117,6 +118,7 @@ int he_aux_kernel_create(he_tile_kernel_t* kernel, he_fgraph_t graph) {
         HE_REQUIRE(kernel && graph, HE_ERR_INVALID, "bad argument");
         auto k = std::make_unique<he_tile_kernel_s>();
         k->k.reset(new he::TileKernel(he::tp::lower_aux(graph->g), "fused_auxiliary"));
+        if (he::device_initialised()) k->k->load();  // so that later launches need not
         *kernel = k.release();
     });
 }
@@ -128,6 +130,7 @@ int he_fused_kernel_create(he_tile_kernel_t* kernel, he_fgraph_t graph) {
             k->k.reset(new he::TileKernel(he::tp::lower_aux(graph->g), "fused_auxiliary"));
         else
             k->k.reset(new he::GemmKernel(he::gemm_problem_from_fusion(graph->g)));
+        if (he::device_initialised()) k->k->load();  // so that later launches need not
         *kernel = k.release();
     });
 }

@@ -95,6 +95,9 @@ inline size_t storage_bytes(int dt, size_t len) {
 
 const char* dtype_name(int dt);
 
+// he_init has run in this process: code objects can be loaded.
+bool device_initialised();
+
 uint64_t fnv1a(const void* data, size_t n, uint64_t seed = 1469598103934665603ull);
 
 }  // namespace he

@@ -1,5 +1,6 @@
 // Device shim: the HIP equivalents of the driver-API wrappers in helium/src/cuda/context.rs
 // (streams, events, modules, launches, memory), exported through the C ABI.
+#include <atomic>
 #include <cstring>
 #include <mutex>
 
@@ -57,6 +58,12 @@ struct he_module_s {
 
 static hipStream_t raw(he_stream_t s) { return s ? s->s : nullptr; }
 
+static std::atomic<bool> g_initialised{false};
+namespace he {
+void noalloc_init_device(int device);  // noalloc.hip
+bool device_initialised() { return g_initialised.load(std::memory_order_acquire); }
+}  // namespace he
+
 extern "C" {
 
 const char* he_last_error(void) { return he::last_error(); }
@@ -71,6 +78,8 @@ int he_init(int device) {
         HE_REQUIRE(device >= 0 && device < n, HE_ERR_INVALID, "device %d out of range (%d devices)", device, n);
         HE_HIP(hipSetDevice(device));
         HE_HIP(hipFree(nullptr));  // forces creation of the primary context
+        he::noalloc_init_device(device);
+        g_initialised.store(true, std::memory_order_release);
     });
 }
 

@@ -1383,21 +1383,45 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
 
 GemmKernel::~GemmKernel() { scratch_.release(); }
 
+size_t GemmKernel::scratch_bytes_needed() const {
+    if (prob_.split_k > 1) return (size_t)prob_.split_k * prob_.M * prob_.N * 4;
+    return (size_t)reduce_floats_ * 4;
+}
+
+void GemmKernel::load() {
+    kernel_->load();
+    if (finalize_) finalize_->load();
+    if (reduce_) reduce_->load();
+}
+
+bool GemmKernel::loaded() const {
+    return kernel_->loaded() && (!finalize_ || finalize_->loaded()) && (!reduce_ || reduce_->loaded());
+}
+
 void GemmKernel::execute(void* const* ptrs, hipStream_t stream) {
+    float* ws = nullptr;
+    if (const size_t need = scratch_bytes_needed()) ws = scratch_.get(need / 4, 0, stream).floats;
+    run(ptrs, stream, ws);
+}
+
+void GemmKernel::execute_in_scratch(void* const* ptrs, hipStream_t stream, void* scratch, size_t scratch_bytes) {
+    HE_REQUIRE(loaded(), HE_ERR_INVALID, "the kernel's code objects are not loaded on this device yet");
+    const size_t need = scratch_bytes_needed();
+    HE_REQUIRE(need <= scratch_bytes, HE_ERR_INVALID,
+               "the kernel needs %zu bytes of scratch for its partial results, the buffer holds %zu", need, scratch_bytes);
+    HE_REQUIRE(!need || (scratch && ((uintptr_t)scratch & 255) == 0), HE_ERR_INVALID, "scratch buffer missing or not 256-byte aligned");
+    // every partial the second launch reads is written by the first: nothing has to be cleared
+    run(ptrs, stream, need ? (float*)scratch : nullptr);
+}
+
+void GemmKernel::run(void* const* ptrs, hipStream_t stream, float* ws) {
     const size_t nargs = prob_.args.size();
     for (size_t i = 0; i < nargs; i++) {
         HE_REQUIRE(ptrs[i] != nullptr, HE_ERR_INVALID, "kernel argument %zu is null", i);
         HE_REQUIRE(((uintptr_t)ptrs[i] & 15) == 0, HE_ERR_INVALID, "kernel argument %zu is not 16-byte aligned", i);
     }
     std::vector<void*> holders(ptrs, ptrs + nargs);
-    float* ws = nullptr;
-    if (prob_.split_k > 1) {
-        ws = scratch_.get((uint64_t)prob_.split_k * prob_.M * prob_.N, 0, stream).floats;
-        holders.push_back(ws);
-    } else if (reduce_floats_) {
-        ws = scratch_.get(reduce_floats_, 0, stream).floats;
-        holders.push_back(ws);
-    }
+    if (ws) holders.push_back(ws);
     std::vector<void*> argv(holders.size());
     for (size_t i = 0; i < holders.size(); i++) argv[i] = &holders[i];
     const uint32_t block[3] = {threads_, 1, 1};

@@ -22,7 +22,20 @@ public:
     virtual const std::string& describe() const = 0;
     // `ptrs[i]` is the device address of argument i.
     virtual void execute(void* const* ptrs, hipStream_t stream) = 0;
+    // The same launches with the kernels' scratch (partial results, arrival counters) taken from `scratch`, a device
+    // buffer of `scratch_bytes` bytes that the caller owns, instead of a buffer the kernel object allocates on its
+    // first launch on a stream. Allocates no device memory; fails with HE_ERR_INVALID when the buffer is too small
+    // or a code object is not loaded yet. Whatever must start at zero is cleared by a fill kernel ahead of the launch.
+    virtual void execute_in_scratch(void* const* ptrs, hipStream_t stream, void* scratch, size_t scratch_bytes) = 0;
+    virtual size_t scratch_bytes_needed() const = 0;
+    // Loads every code object of the kernel onto the current device.
+    virtual void load() = 0;
+    virtual bool loaded() const = 0;
 };
+
+// Loads the fill kernel's code object (fill_buffers otherwise loads it on its first use).
+void load_fill_kernel();
+bool fill_kernel_loaded();
 
 // Device scratch of a kernel whose reductions span several blocks: per-block partials (floats) followed by arrival
 // counters (u32). One buffer per stream the kernel has run on, because launches on one stream run in order and
@@ -53,9 +66,14 @@ public:
     const std::string& source() const override { return launch_.source; }
     const std::string& describe() const override { return launch_.describe; }
     void execute(void* const* ptrs, hipStream_t stream) override;
+    void execute_in_scratch(void* const* ptrs, hipStream_t stream, void* scratch, size_t scratch_bytes) override;
+    size_t scratch_bytes_needed() const override;
+    void load() override;
+    bool loaded() const override;
     ~TileKernel() override;
 
 private:
+    void run(void* const* ptrs, hipStream_t stream, ReduceScratch::Buf ws);
     tp::Program prog_;
     tp::PointwiseLaunch launch_;
     std::unique_ptr<JitKernel> kernel_, finalize_;
@@ -121,10 +139,15 @@ public:
     const std::string& source() const override { return source_; }
     const std::string& describe() const override { return describe_; }
     void execute(void* const* ptrs, hipStream_t stream) override;
+    void execute_in_scratch(void* const* ptrs, hipStream_t stream, void* scratch, size_t scratch_bytes) override;
+    size_t scratch_bytes_needed() const override;
+    void load() override;
+    bool loaded() const override;
     const GemmProblem& problem() const { return prob_; }
     ~GemmKernel() override;
 
 private:
+    void run(void* const* ptrs, hipStream_t stream, float* ws);
     GemmProblem prob_;
     std::string source_, describe_;
     // finalize_: adds up the partial tiles of a split-k product; reduce_: folds the partials of the epilogue's reductions

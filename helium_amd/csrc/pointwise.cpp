@@ -25,6 +25,9 @@ JitKernel& fill_kernel() {
 }
 }  // namespace
 
+void load_fill_kernel() { fill_kernel().load(); }
+bool fill_kernel_loaded() { return fill_kernel().loaded(); }
+
 void fill_buffers(const std::vector<std::pair<void*, std::pair<uint32_t, uint32_t>>>& fills, hipStream_t stream) {
     for (size_t base = 0; base < fills.size(); base += 8) {
         FillArgs a{};
@@ -43,8 +46,12 @@ void fill_buffers(const std::vector<std::pair<void*, std::pair<uint32_t, uint32_
     }
 }
 
+namespace {
+uint64_t aligned_float_bytes(uint64_t n_floats) { return (n_floats * 4 + 255) & ~255ull; }
+}  // namespace
+
 ReduceScratch::Buf ReduceScratch::get(uint64_t n_floats, uint64_t n_counters, hipStream_t stream) {
-    const uint64_t float_bytes = (n_floats * 4 + 255) & ~255ull;
+    const uint64_t float_bytes = aligned_float_bytes(n_floats);
     std::lock_guard<std::mutex> lk(mu_);
     auto it = per_stream_.find(stream);
     if (it == per_stream_.end()) {
@@ -72,6 +79,44 @@ TileKernel::TileKernel(tp::Program prog, const std::string& entry) : prog_(std::
 }
 
 void TileKernel::execute(void* const* ptrs, hipStream_t stream) {
+    ReduceScratch::Buf ws{nullptr, nullptr};
+    if (launch_.grid && launch_.ws_floats) ws = scratch_.get(launch_.ws_floats, launch_.ws_counters, stream);
+    run(ptrs, stream, ws);
+}
+
+size_t TileKernel::scratch_bytes_needed() const {
+    if (!launch_.grid || !launch_.ws_floats) return 0;
+    return (size_t)(aligned_float_bytes(launch_.ws_floats) + launch_.ws_counters * 4);
+}
+
+void TileKernel::load() {
+    if (kernel_) kernel_->load();
+    if (finalize_) finalize_->load();
+    if (!launch_.fills.empty() || launch_.ws_counters) load_fill_kernel();
+}
+
+bool TileKernel::loaded() const {
+    return (!kernel_ || kernel_->loaded()) && (!finalize_ || finalize_->loaded()) &&
+           ((launch_.fills.empty() && !launch_.ws_counters) || fill_kernel_loaded());
+}
+
+void TileKernel::execute_in_scratch(void* const* ptrs, hipStream_t stream, void* scratch, size_t scratch_bytes) {
+    HE_REQUIRE(loaded(), HE_ERR_INVALID, "the kernel's code objects are not loaded on this device yet");
+    const size_t need = scratch_bytes_needed();
+    HE_REQUIRE(need <= scratch_bytes, HE_ERR_INVALID,
+               "the kernel needs %zu bytes of scratch for its partial results, the buffer holds %zu", need, scratch_bytes);
+    ReduceScratch::Buf ws{nullptr, nullptr};
+    if (need) {
+        HE_REQUIRE(scratch && ((uintptr_t)scratch & 255) == 0, HE_ERR_INVALID, "scratch buffer missing or not 256-byte aligned");
+        ws.floats = (float*)scratch;
+        ws.counters = (uint32_t*)((char*)scratch + aligned_float_bytes(launch_.ws_floats));
+        // the buffer is shared with whatever ran before: arrival counters must start at zero
+        if (launch_.ws_counters) fill_buffers({{ws.counters, {(uint32_t)launch_.ws_counters, 0u}}}, stream);
+    }
+    run(ptrs, stream, ws);
+}
+
+void TileKernel::run(void* const* ptrs, hipStream_t stream, ReduceScratch::Buf ws) {
     const size_t nargs = prog_.args.size();
     for (size_t i = 0; i < nargs; i++)
         HE_REQUIRE(ptrs[i] != nullptr || prog_.args[i].numel == 0, HE_ERR_INVALID, "kernel argument %zu is null", i);
@@ -89,7 +134,6 @@ void TileKernel::execute(void* const* ptrs, hipStream_t stream) {
         HE_REQUIRE(((uintptr_t)ptrs[i] & 15) == 0, HE_ERR_INVALID, "kernel argument %zu is not 16-byte aligned", i);
     std::vector<void*> holders(ptrs, ptrs + nargs);
     if (launch_.ws_floats) {
-        ReduceScratch::Buf ws = scratch_.get(launch_.ws_floats, launch_.ws_counters, stream);
         holders.push_back(ws.floats);
         holders.push_back(ws.counters);
     }

@@ -43,6 +43,9 @@ public:
     // Number of scratch bytes per lane the compiler reported (0 == no spills); -1 before the module is loaded.
     int private_bytes();
     int vgprs();
+    // Loads the code object onto the current device (allocates device memory for the code); launch does it on demand.
+    void load() { ensure_loaded(); }
+    bool loaded() const { return func_ != nullptr; }
 
 private:
     void ensure_loaded();

@@ -14,6 +14,7 @@ _ffi._sig("he_tile_kernel_num_args", C.c_void_p, C.POINTER(C.c_int))
 _ffi._sig("he_tile_kernel_arg_info", C.c_void_p, C.c_int, C.POINTER(C.c_uint64), C.POINTER(C.c_int32),
           C.POINTER(C.c_int32), C.POINTER(C.c_int64))
 _ffi._sig("he_tile_kernel_execute", C.c_void_p, C.POINTER(C.c_void_p), C.c_int, C.c_void_p)
+_ffi._sig("he_tile_kernel_execute_noalloc", C.c_void_p, C.POINTER(C.c_void_p), C.c_int, C.c_void_p)
 _ffi._sig("he_tile_kernel_source", C.c_void_p, restype=C.c_char_p)
 _ffi._sig("he_tile_kernel_describe", C.c_void_p, restype=C.c_char_p)
 _ffi._sig("he_tile_kernel_destroy", C.c_void_p)
@@ -74,6 +75,12 @@ class TileKernel:
         ptrs = [(b.ptr if hasattr(b, "ptr") else C.c_void_p(b)) for b in buffers]
         argv = (C.c_void_p * len(ptrs))(*ptrs)
         check(lib.he_tile_kernel_execute(self.handle, argv, len(ptrs), _h(stream)))
+
+    def execute_noalloc(self, buffers, stream=None):
+        """The same launches with the kernels' scratch in the library's own device array: no allocation happens."""
+        ptrs = [(b.ptr if hasattr(b, "ptr") else C.c_void_p(b)) for b in buffers]
+        argv = (C.c_void_p * len(ptrs))(*ptrs)
+        check(lib.he_tile_kernel_execute_noalloc(self.handle, argv, len(ptrs), _h(stream)))
 
     def __del__(self):
         try:

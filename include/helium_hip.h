@@ -214,6 +214,15 @@ int he_tile_kernel_arg_info(he_tile_kernel_t kernel, int index, uint64_t* node, 
                             int64_t* numel);
 /* PointwiseGraph::execute (pointwise.rs:57-86): fills reduction / bitset outputs, then one launch. */
 int he_tile_kernel_execute(he_tile_kernel_t kernel, void* const* arg_ptrs, int num_args, he_stream_t stream);
+/* The same launches without any allocation. No counterpart in the reference; for callers that cannot allocate:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid it. The kernels' scratch (per-workgroup
+ * partial results and arrival counters of reductions, partial tiles of a split product) lies in a device array of
+ * HE_NOALLOC_SCRATCH_BYTES that is part of the library and is resolved per device by he_init; a kernel that needs more
+ * is refused with HE_ERR_INVALID. The call makes no hipMalloc / hipFree and loads no code object: the kernel must
+ * have been created after he_init (creation then loads its code) or have run once through he_tile_kernel_execute.
+ * All calls on a device share the one array: calls that overlap on a device (other streams, other threads) race. */
+#define HE_NOALLOC_SCRATCH_BYTES (8u << 20)
+int he_tile_kernel_execute_noalloc(he_tile_kernel_t kernel, void* const* arg_ptrs, int num_args, he_stream_t stream);
 const char* he_tile_kernel_source(he_tile_kernel_t kernel);
 const char* he_tile_kernel_describe(he_tile_kernel_t kernel);
 int he_tile_kernel_destroy(he_tile_kernel_t kernel);
