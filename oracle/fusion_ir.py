@@ -5,8 +5,9 @@ x ** c for PowConstant, where(rhs > 0, lhs, 0) for Drelu, keepdim sums over dim 
 Rows / Columns / Item / Batch, transpose(1, 2), matmul, implicit broadcast) and the shape rules of
 opgraph.rs:386-426. All arithmetic is f32 (the build's stated precision); the reference's prototype kernels compute
 in bf16 intrinsics (kernel_generator.rs:363-414), so bit-level agreement with them is "parity unpinned" — what is
-pinned: the closed forms in tests/test_fusion_oracle.py (each op against numpy, the autodiff identities, the C4
-graph's hand-derived formulas of README.md:41-79) and torch_synthesizer's definitions above.
+pinned (tests/test_oracle_cpu.py): each unary / binary op against Python's `math` (`math.erf` for Gelu, Drelu as
+torch_synthesizer.rs:76-78 writes it), the four reduction depths and the shape rules against loops, and the README
+graph (README.md:33-79, with and without its mainloop ops) against its closed forms written directly in float64.
 
 The graph is plain data: the list of dicts recorded by helium_amd.fusion.OpGraph.nodes.
 """

@@ -4,11 +4,16 @@ Follows helium-ir/src/opgraph/op.rs (inference), helium/src/cuda/instr/pointwise
 op is computed in f32 whatever the storage type; same-class casts are transparent inside a kernel; stores round
 to the storage type) and helium/src/raw_tensor.rs (front-end lowerings, in `lower_*` helpers used by the tests).
 
-Pinned by tests/golden/tensor_ops.json (helium/tests/tensor_ops.rs: add/mul/div/recip/scalar ops, op chain = 0.4,
-reduce sum/mean/max/min incl. 200k elements, broadcast, reshape, swaps, relu, constant, max/min, matmul small
-cases, conv_simple) and by closed forms in tests/test_oracle.py. Transcendentals (`expf`, `tanhf`, `powf`, ...) are evaluated
-in float64 and rounded once to float32; the reference uses CUDA libdevice for them, whose last-bit behaviour is
-"parity unpinned" beyond the exact-answer cases.
+Pinned by tests/test_oracle_cpu.py: `conv` against the reference's conv_simple vector and a seven-loop brute force
+over the three padding modes, strides and dilations (with the output-size rule of conv.rs:51-73 checked against a
+hand-made table); `conv_backward_data` / `conv_backward_filter` against scatter loops and the adjoint identities;
+Compare / Select / casts / Reduce / Broadcast / SwapDims / Constant through the gradient graphs of
+helium/tests/autodiff.rs and helium/tests/loss.rs with the values those tests assert (tests/golden/autodiff.json); the
+matmul cases of tensor_ops.rs:172-318 (tests/golden/tensor_ops.json); unary and binary functions against Python's
+`math`. tests/test_pointwise_cpu.py adds the pointwise known answers of tensor_ops.rs (add/mul/div/recip/scalar ops,
+the op chain = 0.4, reductions incl. 200k elements, broadcast, reshape, relu, constant, max/min). Transcendentals
+(`expf`, `tanhf`, `powf`, ...) are evaluated in float64 and rounded once to float32; the reference uses CUDA libdevice
+for them, whose last-bit behaviour is "parity unpinned" beyond the exact-answer cases.
 
 The graph is plain data: a list of dicts as recorded by helium_amd.ir.OpGraph.nodes
   {"id", "node": "input", "shape", "dtype"} | {"id", "node": "output", "from"} |
