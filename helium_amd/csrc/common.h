@@ -100,4 +100,18 @@ bool device_initialised();
 
 uint64_t fnv1a(const void* data, size_t n, uint64_t seed = 1469598103934665603ull);
 
+// Overrides of the kernel generators' choices (HELIUM_HIP_GEMM_TILE, HELIUM_HIP_POINTWISE_RPT, ...). They exist for
+// tuning and measurement and are dead unless the process starts with HELIUM_HIP_TUNING set: then every generator reads
+// them through get(), and key() - all of them, sorted, as text - is part of every kernel-cache key and of the plan
+// cache's, so a changed override never meets a kernel built under another. HELIUM_HIP_TUNING=measure also admits the
+// switches that take a component out of a kernel (its results are then wrong on purpose).
+namespace tuning {
+bool enabled();
+bool measuring();
+const char* get(const char* name);  // nullptr when tuning is off or the variable is unset
+int get_int(const char* name, int dflt);
+std::string key();                  // empty when tuning is off
+uint32_t hash();                    // 0 when tuning is off
+}  // namespace tuning
+
 }  // namespace he

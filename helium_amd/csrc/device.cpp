@@ -1,5 +1,6 @@
 // Device shim: the HIP equivalents of the driver-API wrappers in helium/src/cuda/context.rs
 // (streams, events, modules, launches, memory), exported through the C ABI.
+#include <algorithm>
 #include <atomic>
 #include <cstring>
 #include <mutex>
@@ -59,6 +60,51 @@ struct he_module_s {
 static hipStream_t raw(he_stream_t s) { return s ? s->s : nullptr; }
 
 static std::atomic<bool> g_initialised{false};
+
+extern char** environ;
+
+namespace he::tuning {
+namespace {
+int mode() {
+    static const int m = [] {
+        const char* v = getenv("HELIUM_HIP_TUNING");
+        if (!v || !*v || !strcmp(v, "0")) return 0;
+        return !strcmp(v, "measure") ? 2 : 1;
+    }();
+    return m;
+}
+// what a generated kernel or plan never depends on
+bool is_override(const char* entry) {
+    if (strncmp(entry, "HELIUM_HIP_", 11) != 0) return false;
+    for (const char* other : {"HELIUM_HIP_TUNING=", "HELIUM_HIP_CACHE_DIR=", "HELIUM_HIP_DUMP_DIR=", "HELIUM_HIP_DUMP_FAILED=",
+                              "HELIUM_HIP_EXEC_TIMING=", "HELIUM_HIP_NO_LAUNCH_EVENTS="})
+        if (strncmp(entry, other, strlen(other)) == 0) return false;
+    return true;
+}
+}  // namespace
+bool enabled() { return mode() != 0; }
+bool measuring() { return mode() == 2; }
+const char* get(const char* name) { return enabled() ? getenv(name) : nullptr; }
+int get_int(const char* name, int dflt) {
+    const char* v = get(name);
+    return v ? atoi(v) : dflt;
+}
+std::string key() {
+    if (!enabled()) return std::string();
+    std::vector<std::string> all;
+    for (char** e = environ; e && *e; e++)
+        if (is_override(*e)) all.push_back(*e);
+    std::sort(all.begin(), all.end());
+    std::string k = measuring() ? "measure;" : "tuning;";
+    for (auto& v : all) k += v + ";";
+    return k;
+}
+uint32_t hash() {
+    if (!enabled()) return 0;
+    const std::string k = key();
+    return (uint32_t)fnv1a(k.data(), k.size()) | 1u;
+}
+}  // namespace he::tuning
 namespace he {
 void noalloc_init_device(int device);  // noalloc.hip
 bool device_initialised() { return g_initialised.load(std::memory_order_acquire); }

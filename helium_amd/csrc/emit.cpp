@@ -491,14 +491,14 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
     // Threads along a row. With a column reduction a block should be tall rather than wide: its TY row groups are
     // combined in LDS, so every block leaves one partial per column it spans, not one per column per row group.
     int tx_cap = any_col ? 64 : threads;
-    if (const char* env = getenv("HELIUM_HIP_POINTWISE_TX")) tx_cap = std::max(1, atoi(env));
+    if (const char* env = tuning::get("HELIUM_HIP_POINTWISE_TX")) tx_cap = std::max(1, atoi(env));
     int TX = (int)std::min<int64_t>(tx_cap, pow2_ceil((N + NV - 1) / NV));
     int TY = threads / TX;
     const int64_t gx = (N + (int64_t)TX * NV - 1) / ((int64_t)TX * NV);
     const int64_t gy1 = (M + TY - 1) / TY;
     int64_t blocks1 = gx * gy1 * B;
     int RPT = 1;
-    if (const char* env = getenv("HELIUM_HIP_POINTWISE_RPT")) {
+    if (const char* env = tuning::get("HELIUM_HIP_POINTWISE_RPT")) {
         RPT = std::max(1, atoi(env));
     } else {
         // Blocks that end in a column or scalar reduction pay for it once per block (LDS exchange, partials) and are
@@ -560,7 +560,7 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
     // 50 us with two launches; a [256,512] f32 column sum inside a graph 29 us -> 26 us with tickets).
     const uint64_t CS = 32;  // counter stride in u32
     bool tickets = B * M * N <= (int64_t)1 << 21;
-    if (const char* env = getenv("HELIUM_HIP_REDUCE")) tickets = std::string(env) == "ticket";
+    if (const char* env = tuning::get("HELIUM_HIP_REDUCE")) tickets = std::string(env) == "ticket";
     std::vector<WsUse> ws(p.outs.size());
     bool any_finalize = false;
     for (size_t oi = 0; oi < p.outs.size(); oi++) {
@@ -687,7 +687,7 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
         const bool ragged = M % TRv != 0 || N % ((int64_t)TX * NV) != 0;
         // UNROLL rows are in flight at a time: all RPT at once would keep every row's operands in registers
         int unroll = std::min(RPT, 2);
-        if (const char* env = getenv("HELIUM_HIP_POINTWISE_UNROLL")) unroll = std::max(1, std::min(RPT, atoi(env)));
+        if (const char* env = tuning::get("HELIUM_HIP_POINTWISE_UNROLL")) unroll = std::max(1, std::min(RPT, atoi(env)));
         while (RPT % unroll) unroll--;
         const std::string head = "#pragma unroll 1\nfor (u32 i0 = 0; i0 < RPT; i0 += " + std::to_string(unroll) + ") {\n#pragma unroll\nfor (u32 iu = 0; iu < " +
                                  std::to_string(unroll) + "; iu++) {\nconst u32 i = i0 + iu;\nconst u32 m = tile_y * TR + i * TY + ty;\n";

@@ -1,15 +1,18 @@
 // Fused GEMM generator for gfx950: bf16/f16 MFMA (v_mfma_f32_32x32x16) with f32 accumulators.
 //
-//   * Operand tiles are staged global -> registers -> LDS. Mainloop op chains (e.g. Relu, Mul by a tensor) run in
-//     f32 on the staged registers and are rounded to the multiplicand type before they reach LDS, so every
-//     element is computed once per workgroup and the MFMA loop reads finished operands.
+//   * Raw operands travel by direct global -> LDS loads (global_load_lds_dwordx4) into a ring of LDS stages; an
+//     operand with mainloop ops (e.g. Relu, Mul by a tensor) is staged global -> registers -> LDS instead: its source
+//     vectors are requested ahead of a k-tile's MFMAs, evaluated in f32 after them and rounded to the multiplicand
+//     type on the way to LDS, so every element is computed once per workgroup and the MFMA loop reads finished
+//     operands.
 //   * A tiles sit in LDS as [m][k] (k contiguous, 16-byte chunks XOR-swizzled by m), read with one 128-bit LDS
 //     load per MFMA operand. B tiles sit as [k][n] exactly as they are in memory and are read with the
 //     transposing LDS load of gfx950 (ds_read_b64_tr_b16), which hands every lane the 4 consecutive k it needs.
 //   * The epilogue program runs on the f32 accumulators: each wave passes its accumulators through a private LDS
 //     strip to get row-major vectors of NV consecutive columns, so auxiliary tensors are read and outputs written
-//     with coalesced 16-byte accesses; column / row / scalar reductions are folded per lane, combined with wave
-//     shuffles and finished with one atomic per wave and output element.
+//     with coalesced 16-byte accesses. Column / row / scalar reductions are folded per lane, combined with wave
+//     shuffles and through LDS per workgroup, parked as one partial per workgroup in a workspace, and folded in a
+//     fixed order by a second small launch (no atomics: results are the same from run to run).
 #include <cmath>
 #include <cstring>
 #include <sstream>
@@ -532,14 +535,6 @@ void fused_matmul(KERNEL_PARAMS) {
     stage_load(0);
     stage_store(0, 0);
 #endif
-#if GEMM_TIMING
-    unsigned long long t_load = 0, t_compute = 0, t_wait = 0, t_barrier = 0, t0, t1;
-#define TICK(var) t1 = __builtin_readcyclecounter(); var += t1 - t0; t0 = t1;
-    t0 = __builtin_readcyclecounter();
-    const unsigned long long wall0 = __builtin_amdgcn_s_memrealtime();
-#else
-#define TICK(var)
-#endif
     Frags frags;
     init_frags(frags);
     for (u32 kt = 0; kt < KT; kt++) {
@@ -552,7 +547,6 @@ void fused_matmul(KERNEL_PARAMS) {
         else if (younger == 1) __builtin_amdgcn_s_waitcnt(0x0070 | WAITCNT_VM(A_DPW + B_DPW));
         else __builtin_amdgcn_s_waitcnt(0x0070);
 #endif
-        TICK(t_wait)
         // every wave's share of tile kt is in LDS (direct loads waited for above, staged stores made before the
         // barrier) and nobody still reads the stage that this iteration refills
 #if DIRECT_LOADS
@@ -562,7 +556,6 @@ void fused_matmul(KERNEL_PARAMS) {
 #else
         __syncthreads();
 #endif
-        TICK(t_barrier)
         const u32 next = kt + NSTAGES - 1;
         const bool more = next < KT;
 #if STAGED
@@ -582,19 +575,9 @@ void fused_matmul(KERNEL_PARAMS) {
         if (more) stage_store(next, next % NSTAGES);
 #endif
         __builtin_amdgcn_sched_barrier(0);
-        TICK(t_compute)
     }
     finish_tiles(acc, frags);
     __syncthreads();
-#if GEMM_TIMING
-    if (blockIdx.x == 0 && tid == 64) {
-        unsigned long long* dbg = (unsigned long long*)GEMM_TIMING_PTR;
-        dbg[0] = t_load; dbg[1] = t_compute; dbg[2] = t_wait; dbg[3] = t_barrier;
-        dbg[4] = __builtin_amdgcn_s_memrealtime() - wall0;  // 100 MHz ticks
-    }
-    __syncthreads();
-    if (blockIdx.x == 0) return;
-#endif
 
     // ---- epilogue: accumulators -> wave-private LDS strip -> row-major NV-wide vectors -----------------------
     float* strip = (float*)lds + wave * (32 * EP);
@@ -676,13 +659,13 @@ GemmProblem gemm_problem_from_fusion(const fir::OpGraph& g) {
     pr.N = sc[2];
     pr.K = sa[2];
     pr.op_a = tp::lower_operand(g, mm.a, &pr.root_a);
-    if (operand_b_prefers_nk(pr.op_a) && !getenv("HELIUM_HIP_GEMM_NO_KM")) {
+    if (operand_b_prefers_nk(pr.op_a) && !tuning::get("HELIUM_HIP_GEMM_NO_KM")) {
         // the same test on A's [batch, M, K] program asks whether A's source is contiguous along m
         pr.op_a = tp::lower_operand(g, mm.a, &pr.root_a, true);
         pr.a_km = true;
     }
     pr.op_b = tp::lower_operand(g, mm.b, &pr.root_b);
-    if (operand_b_prefers_nk(pr.op_b) && !getenv("HELIUM_HIP_GEMM_NO_NK")) {
+    if (operand_b_prefers_nk(pr.op_b) && !tuning::get("HELIUM_HIP_GEMM_NO_NK")) {
         pr.op_b = tp::lower_operand(g, mm.b, &pr.root_b, true);
         pr.b_nk = true;
     }
@@ -702,8 +685,8 @@ GemmProblem gemm_problem_from_fusion(const fir::OpGraph& g) {
 }
 
 int choose_split_k(int64_t M, int64_t N, int64_t K, int64_t batch) {
-    if (getenv("HELIUM_HIP_GEMM_NO_SPLIT_K") || batch != 1) return 1;
-    if (const char* env = getenv("HELIUM_HIP_GEMM_SPLIT_K")) return std::max(1, atoi(env));
+    if (tuning::get("HELIUM_HIP_GEMM_NO_SPLIT_K") || batch != 1) return 1;
+    if (const char* env = tuning::get("HELIUM_HIP_GEMM_SPLIT_K")) return std::max(1, atoi(env));
     const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128), k_tiles = (K + 63) / 64;
     if (tiles >= 128) return 1;
     // 64x64 tiles fill the chip before a split k range has to: the partial tiles of a split cost a second pass over
@@ -780,9 +763,9 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     bool small = false;
     const bool raw_a0 = pr.conv_a.on || (is_raw_copy(pr.op_a, pr.root_a, pr.mma_dtype) && (pr.a_km ? pr.M : pr.K) % epc == 0);
     const bool raw_b0 = pr.conv_b.on ? true : pr.b_rows.on ? pr.N % epc == 0 : is_raw_copy(pr.op_b, pr.root_b, pr.mma_dtype) && (pr.b_nk ? pr.K : pr.N) % epc == 0;
-    const bool want_direct = !getenv("HELIUM_HIP_GEMM_NO_DIRECT");
+    const bool want_direct = !tuning::get("HELIUM_HIP_GEMM_NO_DIRECT");
     const int esz = 16 / epc;  // bytes per multiplicand
-    if (const char* env = getenv("HELIUM_HIP_GEMM_TILE")) {
+    if (const char* env = tuning::get("HELIUM_HIP_GEMM_TILE")) {
         int v[6] = {256, 256, 64, 2, 4, 2};
         int n = sscanf(env, "%d,%d,%d,%d,%d,%d", &v[0], &v[1], &v[2], &v[3], &v[4], &v[5]);
         HE_REQUIRE(n >= 5, HE_ERR_INVALID, "HELIUM_HIP_GEMM_TILE wants bm,bn,bk,wm,wn[,stages]");
@@ -871,16 +854,16 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     // Each operand qualifies on its own; the other one then goes through registers.
     const bool direct_a = want_direct && raw_a && (pr.conv_a.on ? pr.conv_a.C % epc == 0 : pr.M % t.bm == 0 && pr.K % t.bk == 0) &&
                           (!pr.a_km || 64 % (t.bm / epc) == 0) && (t.bm * t.bk * esz / 1024) % (threads / 64) == 0 &&
-                          !getenv("HELIUM_HIP_GEMM_NO_DIRECT_A");
+                          !tuning::get("HELIUM_HIP_GEMM_NO_DIRECT_A");
     const bool direct_b = want_direct && raw_b && (pr.conv_b.on || (pr.N % t.bn == 0 && pr.K % t.bk == 0)) && (t.bk * t.bn * esz / 1024) % (threads / 64) == 0 &&
-                          (pr.b_nk || 64 % (t.bn / epc) == 0) && !getenv("HELIUM_HIP_GEMM_NO_DIRECT_B");
+                          (pr.b_nk || 64 % (t.bn / epc) == 0) && !tuning::get("HELIUM_HIP_GEMM_NO_DIRECT_B");
     // A convolution's gather with direct loads, a channel count that is a multiple of the k-tile (every tile then lies in
     // one filter tap) and a wave that issues a whole number of loads: the per-lane address arithmetic of a load
     // shrinks from a full (pixel, tap) decomposition to a few adds.
     const bool conv_a_fast = pr.conv_a.on && direct_a && pr.conv_a.C % t.bk == 0 && (t.bm * t.bk * esz / 1024) % (threads / 64) == 0 &&
-                             !getenv("HELIUM_HIP_GEMM_NO_CONV_FAST");
+                             !tuning::get("HELIUM_HIP_GEMM_NO_CONV_FAST");
     if (!(direct_a && direct_b)) t.stages = 2;  // register staging is double-buffered only
-    else if (!getenv("HELIUM_HIP_GEMM_TILE") && small) {
+    else if (!tuning::get("HELIUM_HIP_GEMM_TILE") && small) {
         // A grid that leaves CUs idle is bound by the latency of its k-loop: keep as many tiles in flight as LDS holds.
         // With more than one workgroup per CU (a split k range) the LDS is better spent on a second and third
         // workgroup, whose loads hide each other's waits (filter gradient of a 64-channel layer: 66 -> 56 us).
@@ -889,7 +872,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     }
     // All direct loads of the next tile are issued at the start of a tile's MFMAs (the round trip needs the whole
     // tile to hide); HELIUM_HIP_GEMM_ISSUE=0 spreads them over the k-steps instead.
-    const bool issue_front = getenv("HELIUM_HIP_GEMM_ISSUE") ? atoi(getenv("HELIUM_HIP_GEMM_ISSUE")) != 0 : true;
+    const bool issue_front = tuning::get("HELIUM_HIP_GEMM_ISSUE") ? atoi(tuning::get("HELIUM_HIP_GEMM_ISSUE")) != 0 : true;
     int nve = tp::pick_nv(pr.epi, 32);
     while (nve > 1 && ((32 * wtn) % (64 * nve) != 0)) nve /= 2;
     nve = std::min(nve, 8);
@@ -908,16 +891,17 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     {
         const int lds_bytes = t.stages * (t.bm + t.bn) * t.bk * esz;
         const int acc_regs = t.bm * t.bn / threads;
-        int wgs = getenv("HELIUM_HIP_GEMM_WGS_PER_CU") ? atoi(getenv("HELIUM_HIP_GEMM_WGS_PER_CU")) : (lds_bytes * 2 <= 160 * 1024 && acc_regs <= 32 ? 2 : 1);
+        int wgs = tuning::get("HELIUM_HIP_GEMM_WGS_PER_CU") ? atoi(tuning::get("HELIUM_HIP_GEMM_WGS_PER_CU")) : (lds_bytes * 2 <= 160 * 1024 && acc_regs <= 32 ? 2 : 1);
         if (threads < 256) wgs = 1;
         wgs_per_cu_attr = "\n#define WGS_PER_CU " + std::to_string(std::max(1, wgs));
     }
     s << "#define BM " << t.bm << "\n#define BN " << t.bn << "\n#define BK " << t.bk << "\n#define WAVES_M " << t.wm
       << "\n#define WAVES_N " << t.wn << wgs_per_cu_attr << "\n#define NSTAGES " << t.stages << "\n#define NVE " << nve << "\n#define MMA_BF16 " << (pr.mma_dtype == HE_BF16 ? 1 : 0) << "\n#define MMA_F32 " << (f32 ? 1 : 0)
-      << "\n#define STAGGER_EXPR " << (getenv("HELIUM_HIP_GEMM_STAGGER") ? getenv("HELIUM_HIP_GEMM_STAGGER") : "0u")
+      << "\n#define STAGGER_EXPR " << (tuning::measuring() && tuning::get("HELIUM_HIP_GEMM_STAGGER") ? tuning::get("HELIUM_HIP_GEMM_STAGGER") : "0u")
       << "\n#define ISSUE_FRONT " << (issue_front ? 1 : 0)
-      << "\n#define GEMM_SKIP " << (getenv("HELIUM_HIP_GEMM_SKIP") ? atoi(getenv("HELIUM_HIP_GEMM_SKIP")) : 0)
-      << "\n#define GEMM_TIMING " << (getenv("HELIUM_HIP_GEMM_TIMING") ? 1 : 0) << "\n#define GEMM_TIMING_PTR p" << (pr.args.size() - 1)
+      // measurement only (HELIUM_HIP_TUNING=measure): bit 0 drops the direct loads, bit 1 the fragment reads, bit 2 the
+      // MFMAs - the kernel's results are then wrong, its timing tells what the rest costs
+      << "\n#define GEMM_SKIP " << (tuning::measuring() ? tuning::get_int("HELIUM_HIP_GEMM_SKIP", 0) : 0)
       << "\n#define DIRECT_A " << (direct_a ? 1 : 0) << "\n#define DIRECT_B " << (direct_b ? 1 : 0)
       << "\n#define CONV_A_FAST " << (conv_a_fast ? 1 : 0) << "\n#define A_DPW_MAX " << std::max(1, t.bm * t.bk * esz / 1024 / (threads / 64))
       << "\n#define A_KM " << (pr.a_km ? 1 : 0) << "\n#define B_NK " << (pr.b_nk ? 1 : 0) << "\n#define CONV_A " << (pr.conv_a.on ? 1 : 0) << "\n#define CONV_IMG p" << (pr.conv_a.on ? pr.map_a[0] : 0)
@@ -926,7 +910,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
       << "\n#define B_SRC_OR_NULL " << (pr.b_rows.on || pr.conv_b.on ? "p" + std::to_string(pr.map_b[0]) : std::string("nullptr")) << "\n#define DIRECT_LOADS (DIRECT_A || DIRECT_B)\n#define STAGED (!DIRECT_A || !DIRECT_B)"
       << "\n#define DIRECT_A_PTR p" << (direct_a ? pr.map_a[0] : 0)
       << "\n#define DIRECT_B_PTR p" << (direct_b ? pr.map_b[0] : 0) << "\n#define STAGE_SCHED_BARRIER "
-      << ((getenv("HELIUM_HIP_GEMM_PIN") ? atoi(getenv("HELIUM_HIP_GEMM_PIN")) != 0 : true) ? "__builtin_amdgcn_sched_barrier(0);" : "") << "\n#define A_SWZ_SHIFT " << (getenv("HELIUM_HIP_GEMM_ASWZ") ? atoi(getenv("HELIUM_HIP_GEMM_ASWZ")) : (t.bk == 64 ? 1 : 2)) << "\n";
+      << ((tuning::get("HELIUM_HIP_GEMM_PIN") ? atoi(tuning::get("HELIUM_HIP_GEMM_PIN")) != 0 : true) ? "__builtin_amdgcn_sched_barrier(0);" : "") << "\n#define A_SWZ_SHIFT " << (tuning::get("HELIUM_HIP_GEMM_ASWZ") ? atoi(tuning::get("HELIUM_HIP_GEMM_ASWZ")) : (t.bk == 64 ? 1 : 2)) << "\n";
 
     s << kGemmHelpers;
     // kernel parameters
@@ -1069,7 +1053,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     // step that uses them. Measured within run-to-run noise of the compiler's own placement on the 40-op epilogue
     // (162.5 vs 162.6 us over three alternating runs each), so off.
     const std::string raw_members = tp::emit_raw_members(pr.epi, nve, true);
-    const char* epipipe = getenv("HELIUM_HIP_GEMM_EPIPIPE");
+    const char* epipipe = tuning::get("HELIUM_HIP_GEMM_EPIPIPE");
     const bool pipelined = !raw_members.empty() && epipipe && atoi(epipipe) != 0;
     if (pipelined) {
         tp::EmitCtx lx;
@@ -1230,16 +1214,16 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         // column, so the tiles resident on one XCD form a compact block sharing few A and B panels.
         const int64_t tm = (pr.M + t.bm - 1) / t.bm, tn = (pr.N + t.bn - 1) / t.bn;
         std::ostringstream o;
-        const bool xcd = (tm * tn) % 8 == 0 && !getenv("HELIUM_HIP_GEMM_NO_XCD");
+        const bool xcd = (tm * tn) % 8 == 0 && !tuning::get("HELIUM_HIP_GEMM_NO_XCD");
         o << "{ u32 b = blockIdx.x;\n";
         if (xcd) o << "b = (b % 8u) * " << (tm * tn / 8) << "u + b / 8u;\n";
-        const int G = getenv("HELIUM_HIP_GEMM_GROUP") ? atoi(getenv("HELIUM_HIP_GEMM_GROUP")) : 4;
+        const int G = tuning::get("HELIUM_HIP_GEMM_GROUP") ? atoi(tuning::get("HELIUM_HIP_GEMM_GROUP")) : 4;
         o << "const u32 gsize = " << G * tn << "u, group = b / gsize, first = group * " << G << "u;\n";
         o << "const u32 rows = (" << tm << "u - first) < " << G << "u ? (" << tm << "u - first) : " << G << "u;\n";
         o << "tile_m = first + (b % gsize) % rows; tile_n = (b % gsize) / rows; }\n";
         splice("TILE_ORDER", o.str());
         std::ostringstream h;
-        if (getenv("HELIUM_HIP_GEMM_SCHED")) {
+        if (tuning::get("HELIUM_HIP_GEMM_SCHED")) {
             // ask the scheduler to alternate LDS reads with MFMAs instead of batching either
             h << "_Pragma(\"unroll\") for (int q = 0; q < MB + 2 * NB; q++) { __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); "
                  "__builtin_amdgcn_sched_group_barrier(0x008, 1, 0); }\n";
@@ -1249,7 +1233,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         std::ostringstream plan;
         // The instruction-order plan is written for tiles whose operands both arrive by direct loads; with an operand
         // staged through registers the compiler's own order, fenced off from the staging code, measured 1.9x faster.
-        const int mode = getenv("HELIUM_HIP_GEMM_PLAN") ? atoi(getenv("HELIUM_HIP_GEMM_PLAN")) : (direct_a && direct_b) ? 3 : 0;
+        const int mode = tuning::get("HELIUM_HIP_GEMM_PLAN") ? atoi(tuning::get("HELIUM_HIP_GEMM_PLAN")) : (direct_a && direct_b) ? 3 : 0;
         const int mb = t.bm / t.wm / 32, nb = t.bn / t.wn / 32, kk_steps = t.bk / (2 * epc);
         const int nr = f32 ? mb + 4 * nb : mb + 2 * nb, nm = f32 ? 4 * mb * nb : mb * nb;
         if (mode == 1) {

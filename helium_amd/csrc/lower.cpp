@@ -130,7 +130,7 @@ uint32_t f32_bits(float f) {
 // ---------------------------------------------------------------------------------------------------------
 // Element count from which a reduction over leading dims is reordered into a column reduction.
 int64_t fold_columns_threshold() {
-    if (const char* env = getenv("HELIUM_HIP_FOLD_COLUMNS_MIN")) return atoll(env);
+    if (const char* env = tuning::get("HELIUM_HIP_FOLD_COLUMNS_MIN")) return atoll(env);
     return 1 << 20;
 }
 

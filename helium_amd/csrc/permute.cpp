@@ -30,7 +30,7 @@ static int pow2_ceil(int64_t x) {
     return p;
 }
 static int env_int(const char* name, int dflt) {
-    const char* v = getenv(name);
+    const char* v = tuning::get(name);
     return v ? atoi(v) : dflt;
 }
 

@@ -72,7 +72,10 @@ bool feeds_only_reductions(const ir::OpGraph& g, NodeId node, int budget = 64) {
 }  // namespace
 void set_fuse_matmul_epilogue(bool on) { g_fuse_matmul_epilogue.store(on); }
 bool fuse_matmul_epilogue() { return g_fuse_matmul_epilogue.load(); }
-unsigned option_mask() { return (fuse_matmul_epilogue() ? 1u : 0u) | (g_fold_swap_into_reduce.load() ? 2u : 0u); }
+unsigned option_mask() {
+    // the hash of the tuning overrides (0 unless tuning is on) rides along: plans keep their kernels
+    return (fuse_matmul_epilogue() ? 1u : 0u) | (g_fold_swap_into_reduce.load() ? 2u : 0u) | (tuning::hash() << 2);
+}
 void set_fold_swap_into_reduce(bool on) { g_fold_swap_into_reduce.store(on); }
 bool fold_swap_into_reduce() { return g_fold_swap_into_reduce.load(); }
 
@@ -173,12 +176,12 @@ void Instr::precompile() const {
     if (kernel_ || permute_) return;
     switch (kind_) {
         case InstrKind::Pointwise:
-            kernel_ = g_tile_kernels.get_or_insert("pw:" + sg_.cache_key(), [&] {
+            kernel_ = g_tile_kernels.get_or_insert(tuning::key() + "pw:" + sg_.cache_key(), [&] {
                 return std::shared_ptr<KernelBase>(new TileKernel(tp::lower_pointwise(sg_), "pointwise_kernel"));
             });
             break;
         case InstrKind::Gemm:
-            kernel_ = g_tile_kernels.get_or_insert("mm:" + sg_.cache_key(), [&] {
+            kernel_ = g_tile_kernels.get_or_insert(tuning::key() + "mm:" + sg_.cache_key(), [&] {
                 return std::shared_ptr<KernelBase>(new GemmKernel(gemm_problem_from_ir(sg_)));
             });
             break;
@@ -188,7 +191,7 @@ void Instr::precompile() const {
             const ir::Descriptor& d = sg_.graph()->get(sg_.inputs()[0]).desc;
             std::vector<int> perm = perm_from_swaps((int)d.shape.size(), swaps);
             std::ostringstream key;
-            key << d.dtype << ':';
+            key << tuning::key() << d.dtype << ':';
             for (int64_t e : d.shape) key << e << ',';
             key << ':';
             for (int p : perm) key << p << ',';
@@ -695,7 +698,7 @@ GemmProblem conv_backward_filter_problem(const ir::OpSubgraph& sg, NodeId node) 
     // about two workgroups per CU, each with at least four 64-wide k-tiles (128x128 output tiles)
     const int64_t tiles = ((pr.M + 127) / 128) * ((pr.N + 127) / 128), k_tiles = (pr.K + 63) / 64;
     pr.split_k = (int)std::max<int64_t>(1, std::min<int64_t>({(512 + tiles - 1) / tiles, k_tiles / 4, 1024}));
-    if (const char* env = getenv("HELIUM_HIP_GEMM_SPLIT_K")) pr.split_k = std::max(1, atoi(env));
+    if (const char* env = tuning::get("HELIUM_HIP_GEMM_SPLIT_K")) pr.split_k = std::max(1, atoi(env));
     pr.epi.dims = {1, pr.M, pr.N};
     pr.epi.fast_math = true;
     tp::Expr acc;

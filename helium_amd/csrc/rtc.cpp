@@ -9,6 +9,7 @@
 
 #include <atomic>
 #include <cstdlib>
+#include <cstring>
 #include <fstream>
 #include <mutex>
 #include <unordered_map>
@@ -42,13 +43,70 @@ std::string cache_dir() {
     return dir;
 }
 
+// What a cached code object depends on besides the source and the options: the compiler that made it.
+const std::string& toolchain_tag() {
+    static const std::string tag = [] {
+        int major = 0, minor = 0;
+        if (hiprtcVersion(&major, &minor) != HIPRTC_SUCCESS) major = minor = -1;
+        return strfmt("hiprtc %d.%d|hip %d|%s", major, minor, (int)HIP_VERSION, he_version());
+    }();
+    return tag;
+}
+
 std::string key_of(const std::string& source, const std::vector<std::string>& opts) {
     std::string k = source;
     for (auto& o : opts) {
         k.push_back('\0');
         k += o;
     }
+    k.push_back('\0');
+    k += toolchain_tag();
     return k;
+}
+
+// A cache file is a header followed by the code object. A file that is short, was written by another format version,
+// fails its checksum or does not hold an ELF image is ignored (and overwritten by the compile that follows).
+struct CacheHeader {
+    char magic[8];       // "HEKCACHE"
+    uint32_t format;     // kCacheFormat
+    uint32_t reserved;
+    uint64_t payload_bytes;
+    uint64_t payload_hash;  // fnv1a
+};
+constexpr uint32_t kCacheFormat = 2;
+
+bool read_cache_file(const std::string& path, std::vector<char>* blob) {
+    std::ifstream f(path, std::ios::binary);
+    if (!f) return false;
+    CacheHeader h;
+    if (!f.read((char*)&h, sizeof h)) return false;
+    if (memcmp(h.magic, "HEKCACHE", 8) != 0 || h.format != kCacheFormat || h.payload_bytes < 64 || h.payload_bytes > (1ull << 31)) return false;
+    blob->resize(h.payload_bytes);
+    if (!f.read(blob->data(), (std::streamsize)h.payload_bytes)) return false;
+    if (f.peek() != std::ifstream::traits_type::eof()) return false;
+    if (memcmp(blob->data(), "\x7f" "ELF", 4) != 0) return false;
+    return fnv1a(blob->data(), blob->size()) == h.payload_hash;
+}
+
+void write_cache_file(const std::string& path, const std::vector<char>& blob) {
+    // written under a private name and renamed: a reader never sees half a file
+    const std::string tmp = path + strfmt(".tmp%d", (int)getpid());
+    {
+        std::ofstream f(tmp, std::ios::binary);
+        CacheHeader h{};
+        memcpy(h.magic, "HEKCACHE", 8);
+        h.format = kCacheFormat;
+        h.payload_bytes = blob.size();
+        h.payload_hash = fnv1a(blob.data(), blob.size());
+        f.write((const char*)&h, sizeof h);
+        f.write(blob.data(), (std::streamsize)blob.size());
+        if (!f) {
+            f.close();
+            unlink(tmp.c_str());
+            return;
+        }
+    }
+    if (rename(tmp.c_str(), path.c_str()) != 0) unlink(tmp.c_str());
 }
 
 }  // namespace
@@ -70,11 +128,11 @@ void rtc_stats(uint64_t stats[3]) {
 }
 
 std::shared_ptr<const std::vector<char>> rtc_compile(const std::string& source, const std::string& name,
-                                                     const std::vector<std::string>& extra_options) {
+                                                     const std::vector<std::string>& extra_options, bool bypass_caches) {
     std::vector<std::string> opts = default_kernel_options();
     for (auto& o : extra_options) opts.push_back(o);
     std::string key = key_of(source, opts);
-    {
+    if (!bypass_caches) {
         std::lock_guard<std::mutex> lk(g_mu);
         auto it = g_cache.find(key);
         if (it != g_cache.end()) {
@@ -89,17 +147,14 @@ std::shared_ptr<const std::vector<char>> rtc_compile(const std::string& source, 
     if (!dir.empty()) {
         uint64_t h1 = fnv1a(key.data(), key.size());
         uint64_t h2 = fnv1a(key.data(), key.size(), 0x9e3779b97f4a7c15ull);
-        path = strfmt("%s/%016llx%016llx.hsaco", dir.c_str(), (unsigned long long)h1, (unsigned long long)h2);
-        std::ifstream f(path, std::ios::binary);
-        if (f) {
-            std::vector<char> blob((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
-            if (blob.size() > 64) {
-                g_disk_hits++;
-                auto sp = std::make_shared<const std::vector<char>>(std::move(blob));
-                std::lock_guard<std::mutex> lk(g_mu);
-                g_cache[key] = sp;
-                return sp;
-            }
+        path = strfmt("%s/%016llx%016llx.hekc", dir.c_str(), (unsigned long long)h1, (unsigned long long)h2);
+        std::vector<char> blob;
+        if (!bypass_caches && read_cache_file(path, &blob)) {
+            g_disk_hits++;
+            auto sp = std::make_shared<const std::vector<char>>(std::move(blob));
+            std::lock_guard<std::mutex> lk(g_mu);
+            g_cache[key] = sp;
+            return sp;
         }
     }
 
@@ -140,14 +195,7 @@ std::shared_ptr<const std::vector<char>> rtc_compile(const std::string& source, 
     HE_REQUIRE(r == HIPRTC_SUCCESS, HE_ERR_RTC, "hiprtcGetCode: %s", hiprtcGetErrorString(r));
     g_compiles++;
 
-    if (!path.empty()) {
-        std::string tmp = path + strfmt(".tmp%d", (int)getpid());
-        {
-            std::ofstream f(tmp, std::ios::binary);
-            f.write(blob.data(), (std::streamsize)blob.size());
-        }
-        rename(tmp.c_str(), path.c_str());
-    }
+    if (!path.empty()) write_cache_file(path, blob);
     auto sp = std::make_shared<const std::vector<char>>(std::move(blob));
     std::lock_guard<std::mutex> lk(g_mu);
     g_cache[key] = sp;
@@ -155,8 +203,8 @@ std::shared_ptr<const std::vector<char>> rtc_compile(const std::string& source, 
 }
 
 JitKernel::JitKernel(std::string source, std::string entry, std::vector<std::string> options)
-    : source_(std::move(source)), entry_(std::move(entry)) {
-    code_ = rtc_compile(source_, entry_, options);
+    : source_(std::move(source)), entry_(std::move(entry)), options_(std::move(options)) {
+    code_ = rtc_compile(source_, entry_, options_);
 }
 
 JitKernel::~JitKernel() {
@@ -169,7 +217,13 @@ void JitKernel::ensure_loaded() {
     std::lock_guard<std::mutex> lk(mu);
     if (func_) return;
     hipModule_t m;
-    HE_HIP(hipModuleLoadData(&m, code_->data()));
+    if (hipModuleLoadData(&m, code_->data()) != hipSuccess) {
+        // a code object this device does not take (a cache directory carried over from another machine): compile
+        // afresh, past the caches, and load that
+        (void)hipGetLastError();
+        code_ = rtc_compile(source_, entry_, options_, true);
+        HE_HIP(hipModuleLoadData(&m, code_->data()));
+    }
     hipFunction_t f;
     hipError_t e = hipModuleGetFunction(&f, m, entry_.c_str());
     if (e != hipSuccess) {

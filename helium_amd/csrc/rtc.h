@@ -9,10 +9,11 @@
 
 namespace he {
 
-// Compiles HIP source for gfx950. Cached by (source, options): in memory, and as a code-object file under the
-// cache directory (HELIUM_HIP_CACHE_DIR, default <library dir>/_kcache) when that directory is usable.
+// Compiles HIP source for gfx950. Cached by (source, options, hiprtc / HIP / library version): in memory, and as a
+// checksummed code-object file under the cache directory (HELIUM_HIP_CACHE_DIR, default <library dir>/_kcache) when
+// that directory is usable. `bypass_caches` compiles regardless and replaces both entries.
 std::shared_ptr<const std::vector<char>> rtc_compile(const std::string& source, const std::string& name,
-                                                     const std::vector<std::string>& extra_options);
+                                                     const std::vector<std::string>& extra_options, bool bypass_caches = false);
 void rtc_stats(uint64_t stats[3]);
 
 // Flags every generated kernel is compiled with.
@@ -50,6 +51,7 @@ public:
 private:
     void ensure_loaded();
     std::string source_, entry_;
+    std::vector<std::string> options_;
     std::shared_ptr<const std::vector<char>> code_;
     hipModule_t module_ = nullptr;
     hipFunction_t func_ = nullptr;
