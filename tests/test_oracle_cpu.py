@@ -320,3 +320,35 @@ def test_c4_graph_against_its_closed_forms(mainloop):
     assert np.allclose(val[57], dpre_c, rtol=1e-4, atol=1e-8)
     assert got[outs["loss"]].dtype == np.float32 and got[outs["dpre_c"]].dtype == np.uint16
     assert got[outs["db8"]].shape == (1, 1, size)
+
+
+@pytest.mark.parametrize("mainloop", [False, True], ids=["epilogue", "mainloop_and_epilogue"])
+@pytest.mark.parametrize("size", [40, 200])
+def test_c_restatement_of_the_c4_fusion_against_closed_forms_and_the_numpy_oracle(size, mainloop):
+    """oracle/c4_cpu.c (what bench.py times as the CPU baseline) against the same closed forms in float64 and against
+    the graph walker; sizes that are no multiple of its row and column blocks."""
+    from oracle import c4_cpu
+
+    g, _ = configs.c4_graph(size, mainloop=mainloop)
+    inputs = configs.c4_inputs(g, size)
+    f = {k: nm.from_storage(v, "f32" if v.dtype == np.float32 else "bf16", v.shape).astype(np.float64) for k, v in inputs.items()}
+    a = f[22] if mainloop else f[1]
+    if mainloop:
+        a = nm.bf16_bits_to_f32(nm.f32_to_bf16_bits((np.maximum(a, 0.0) * f[9]).astype(np.float32))).astype(np.float64)
+    pre_z = a @ f[2] + f[13] + f[6]
+    z, c = np.maximum(pre_z, 0.0), np.tanh(f[24] + f[26] + f[8])
+    d = (1.0 - z) * f[9] + z * c - f[11]
+    inv = float(np.float32(0.00024414063))
+    dh = d * 2.0 * inv
+    near = np.abs(pre_z) < 1e-5  # may fall on either side of Drelu's test
+    want = {39: (d * d * inv).sum(), 58: (z * dh * (1.0 - c * c)).sum(axis=1).reshape(-1),
+            87: np.where((pre_z > 0) & ~near, dh * c - dh * f[9], 0.0).sum(axis=1).reshape(-1)}
+    got = c4_cpu.c4(inputs, size, mainloop=mainloop)
+    slack = np.abs(np.where(near, dh * c - dh * f[9], 0.0)).sum(axis=1).reshape(-1)
+    assert np.allclose(got[39][0], want[39], rtol=2e-5)
+    assert np.allclose(got[58], want[58], rtol=1e-3, atol=1e-6 * np.abs(want[58]).max())
+    assert np.all(np.abs(got[87] - want[87]) <= 1e-3 * np.abs(want[87]) + 1e-6 * np.abs(want[87]).max() + slack)
+    walker = oracle_fir.outputs(g.nodes, inputs, round_mainloop_to="bf16" if mainloop else None)
+    for k in (39, 58, 87):
+        w = walker[k].reshape(-1).astype(np.float64)
+        assert np.max(np.abs(got[k] - w)) <= 1e-5 * np.abs(w).max()
