@@ -100,3 +100,27 @@ def all_reductions(m, n, k, batch=2, seed=2):
     outs = [g.consumer(g.reduction(v, d), "f32") for d in ("rows", "columns", "item", "batch")]
     outs.append(g.consumer(v, "f32"))
     return g, inputs, outs
+
+
+MATMUL_DTYPES = ("f32", "bf16", "f16")
+# helium-kernel-generator/tests/matmul.rs:171-181: the precisions of matmul_no_fusion (the four F8 mode pairs share one
+# entry here: the modes change nothing on hardware whose F8 products run as bf16)
+MATMUL_PRECISIONS = ("f32_f32", "tf32_f32", "bf16_f32", "f16_f32", "f16_f16", "f8_f32")
+
+
+def ir_matmul(m, n, k, dtype_a, dtype_b, precision, out_dtype, seed=7):
+    """matmul_no_fusion of helium-kernel-generator/tests/matmul.rs:24-70: Input a, Input b, Matmul(precision),
+    ChangeDataType(output type), Output, handed to the MatmulGenerator boundary as the subgraph {matmul, cast}.
+    Operands are uniform in [0, 1) like the reference's `rand::random::<f32>()`. Returns (graph, kernel, inputs by
+    node, the cast's node id)."""
+    from helium_amd import backend, ir
+    from oracle import numerics as nm
+
+    g = ir.OpGraph()
+    a, b = g.new_input([m, k], dtype_a), g.new_input([k, n], dtype_b)
+    mm = g.matmul(a, b, precision)
+    out = g.change_data_type(mm, out_dtype)
+    g.new_output(out)
+    rng = np.random.default_rng(seed)
+    host = {a: nm.to_storage(rng.random((m, k), dtype=np.float32), dtype_a), b: nm.to_storage(rng.random((k, n), dtype=np.float32), dtype_b)}
+    return g, backend.matmul_kernel(g, [mm, out]), host, out
