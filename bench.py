@@ -24,7 +24,7 @@ BF16_PEAK_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
 F32_PEAK_TFLOPS = 157.3      # MI355X dense fp32 matrix, published
 # Bytes that left the XCD L2s per launch of each workload's dominant kernel: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE,
 # each scaled by what the same counter reads for the COPY workload (profiles/<kernel>_<workload>.txt).
-TRAFFIC_BYTES = {"COPY": 268435456, "C2a": 205509374, "C2b": 67196580, "C2c": 17587916, "C3": 269743029, "C4": 370218917, "C5a": 302134023, "GEMM": 234914277, "C5b-bn": 313174768, "C5b-conv": 52383120}
+TRAFFIC_BYTES = {"COPY": 268435456, "C2a": 205509374, "C2b": 67196580, "C2c": 17587916, "C3": 269743029, "C4": 370218917, "C5a-fused": 302134023, "GEMM": 234914277, "C5b-bn": 313174768, "C5b-conv": 52383120}
 HEADLINE = "C4"              # the workload `value` is quoted on
 ROTATE_BYTES = 768 << 20     # rotate operand sets so repeated steps cannot live in the 256 MB Infinity Cache
 
@@ -869,6 +869,95 @@ class FusedGemmWorkload:
         self.sets = []
 
 
+class PlannedGemmWorkload(FusedGemmWorkload):
+    """The same graphs, run the way the fusion search plans them under the MI355X cost model (he_fusion_search with
+    HE_FUSE_MIN_MI355X_COST, then he_fusion_plan_execute): a mainloop chain that 16 tile columns would each repeat is
+    split off into a kernel of its own and the product reads its finished operand."""
+
+    def __init__(self, name, size=4096):
+        super().__init__(name, size)
+        self.graph_name = name
+
+    def describe(self):
+        return super().describe() + " as planned by the fusion search (MI355X cost model)"
+
+    def setup(self):
+        import helium_amd as ha
+        from helium_amd import configs, fusion_search as fs
+
+        n = self.size
+        if self.name == "C4m":
+            self.graph, outs = configs.c4_graph(n, mainloop=True, full_size_outputs=True)
+            self.inputs = configs.c4_inputs(self.graph, n)
+            for node in ("loss", "db8", "db6"):  # bare reductions of the README listing: the search keeps what a Consumer reads
+                self.graph.consumer(outs[node], "f32")
+        else:
+            self.graph, names = configs.c5a_graph(n)
+            self.inputs = configs.c5a_inputs(names, n)
+        self.plan = fs.FusionPlan(self.graph, fs.MIN_MI355X_COST)
+        self.plan.precompile()
+        itemsize = {"bf16": 2, "f16": 2, "f32": 4}
+        used = {nd[k] for nd in self.graph.nodes for k in ("a", "b", "x", "lhs", "rhs") if k in nd}
+        self.leaves = [nd for nd in self.graph.nodes if nd["id"] not in used]
+        per_set = sum(v.nbytes for v in self.inputs.values())
+        nsets = max(2, min(6, ROTATE_BYTES // per_set + 1))
+        self.sets = []
+        for _ in range(nsets):
+            prod = {k: ha.DeviceBuffer.from_numpy(v) for k, v in self.inputs.items()}
+            cons = {nd["id"]: ha.DeviceBuffer(max(16, int(np.prod(nd["shape"])) * itemsize[nd["dtype"]])) for nd in self.leaves}
+            self.sets.append((prod, cons))
+        kinds = " + ".join(("core(mainloop %d, epilogue %d)" % (len(f["mainloop"]), len(f["epilogue"]))) if f["core"] else "aux(%d ops)" % len(f["aux"])
+                           for f in self.plan.fusions)
+        log(f"[bench] {self.describe()} :: plan = {kinds}; predicted {self.plan.cost(fs.MIN_MI355X_COST) * 1e6:.1f} us :: {nsets} operand sets")
+        log("[bench] chosen plan:\n" + self.plan.text)
+
+    def step(self, stream, i):
+        prod, cons = self.sets[i % len(self.sets)]
+        self.plan.execute(prod, cons, stream=stream)
+
+    def check(self):
+        from oracle import fusion_ir as oracle
+        from oracle import numerics as nm
+
+        # values that cross from one kernel to the next are stored as bf16 (f32 for reductions)
+        crossing = {}
+        by_id = {nd["id"]: nd for nd in self.graph.nodes}
+        for f in self.plan.fusions[:-1]:
+            members = set(f["mainloop"] + f["epilogue"] + f["aux"])
+            for nd in self.graph.nodes:
+                for k in ("a", "b", "x", "lhs", "rhs"):
+                    if k in nd and nd[k] in members and nd["id"] not in members and nd["op"] != "consumer":
+                        crossing[nd[k]] = "f32" if by_id[nd[k]]["op"] == "reduction" else "bf16"
+        want = oracle.outputs(self.graph.nodes, self.inputs, round_mainloop_to="bf16", materialize=crossing)
+        worst = 0.0
+        for nd in self.leaves:
+            buf = self.sets[0][1][nd["id"]]
+            numel = int(np.prod(nd["shape"]))
+            w = want[nd["id"]].reshape(-1)
+            if nd["dtype"] == "bf16":
+                got, w = nm.bf16_bits_to_f32(buf.to_numpy(np.uint16)[:numel]), nm.bf16_bits_to_f32(w)
+                d = np.abs(got.astype(np.float64) - w)
+                ok = (d <= 1e-3) | (d <= 1e-2 * np.maximum(np.abs(got), np.abs(w)))
+                if not ok.all():
+                    raise SystemExit(f"[bench] PARITY FAILURE in {self.name} output {nd['id']}: {int((~ok).sum())} elements off")
+            else:
+                got = buf.to_numpy(np.float32)[:numel].astype(np.float64)
+                err = float(np.max(np.abs(got - w)) / max(float(np.abs(w).max()), 1e-30))
+                worst = max(worst, err)
+                if not err <= 1e-3:
+                    raise SystemExit(f"[bench] PARITY FAILURE in {self.name} reduction {nd['id']}: {err} of the largest element")
+        return f"full-size outputs within 1e-2 relative, reductions within 1e-3 (worst {worst:.1e}) of the f64-accumulated oracle"
+
+    def cpu_baseline(self, budget_s=25.0):
+        return None
+
+    def free(self):
+        for prod, cons in self.sets:
+            for b in list(prod.values()) + list(cons.values()):
+                b.free()
+        self.sets = []
+
+
 def make_workloads():
     from helium_amd import configs
 
@@ -888,6 +977,11 @@ def make_workloads():
     w["C5b-block"] = BasicBlockWorkload()
     for name in ("C4", "C5a", "C4m", "GEMM"):
         w[name] = FusedGemmWorkload(name)
+    # C5a and C4m as one kernel each (every mainloop op fused) stay measurable next to the planned form
+    w["C5a-fused"], w["C4m-fused"] = w.pop("C5a"), w.pop("C4m")
+    w["C5a-fused"].traffic_key, w["C4m-fused"].traffic_key = "C5a-fused", "C4m-fused"
+    w["C5a"], w["C4m"] = PlannedGemmWorkload("C5a"), PlannedGemmWorkload("C4m")
+    w["C5a"].traffic_key, w["C4m"].traffic_key = "C5a-planned", "C4m-planned"
     return w
 
 
@@ -925,7 +1019,7 @@ def roofline(wl, ms):
         achieved = wl.work / (ms * 1e-3) / 1e12
         peak, unit = getattr(wl, "peak", BF16_PEAK_TFLOPS), "TFLOP/s"
     return {"bound": wl.bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
-            "frac": round(achieved / peak, 4), "traffic": TRAFFIC_BYTES.get(wl.name)}
+            "frac": round(achieved / peak, 4), "traffic": TRAFFIC_BYTES.get(getattr(wl, "traffic_key", wl.name))}
 
 
 def main():

@@ -57,9 +57,24 @@ FusionKernel& kernel_of(he_fusion_plan_s& plan, FusionId id) {
         sub.insert_with_id(dep, p);
         fk.bindings.push_back({provider, dep});
     }
+    // members go in after what they read (ids need not follow the dataflow: the README numbers its mainloop ops
+    // above their anchor)
     std::vector<OpNode> members = f.nodes();
     std::sort(members.begin(), members.end());
-    for (OpNode n : members) sub.insert_with_id(n, g.get(n));
+    std::set<OpNode> placed;
+    while (placed.size() < members.size()) {
+        bool progressed = false;
+        for (OpNode n : members) {
+            if (placed.count(n)) continue;
+            bool ready = true;
+            for (OpNode in : g.get(n).inputs()) ready = ready && (sub.has(in) || !f.contains(in));
+            if (!ready) continue;
+            sub.insert_with_id(n, g.get(n));
+            placed.insert(n);
+            progressed = true;
+        }
+        HE_REQUIRE(progressed, HE_ERR_INTERNAL, "fusion %llu has a cycle", (unsigned long long)id);
+    }
     // one consumer per distinct value this fusion provides
     std::set<OpNode> provided;
     for (auto& d : f.dependents) provided.insert(d.first);
@@ -85,7 +100,7 @@ extern "C" {
 
 namespace {
 void fusion_search(he_fgraph_t graph, int objective, bool subdivided, he_fusion_plan_t* plan) {
-    HE_REQUIRE(graph && plan && objective >= 0 && objective <= 2, HE_ERR_INVALID, "bad argument");
+    HE_REQUIRE(graph && plan && objective >= 0 && objective <= 3, HE_ERR_INVALID, "bad argument");
     auto p = std::make_unique<he_fusion_plan_s>();
     p->g = std::make_shared<fir::OpGraph>(graph->g);
     const auto params = fsearch::CostParams::mi355x();
@@ -141,8 +156,18 @@ int he_fusion_plan_cost(he_fusion_plan_t plan, int objective, int reference_cons
     return he::guard([&] {
         HE_REQUIRE(plan && cost, HE_ERR_INVALID, "bad argument");
         const fsearch::CostParams p = reference_constants ? fsearch::CostParams::reference() : fsearch::CostParams::mi355x();
-        *cost = objective == 2 ? fsearch::analytical_cost(plan->fg) : fsearch::naive_cost(plan->fg, p);
+        *cost = objective == 3 ? fsearch::mi355x_cost(plan->fg) : objective == 2 ? fsearch::analytical_cost(plan->fg) : fsearch::naive_cost(plan->fg, p);
         if (states_visited) *states_visited = plan->states;
+    });
+}
+
+int he_fusion_plan_cost_terms(he_fusion_plan_t plan, double* terms, int capacity, int* count) {
+    return he::guard([&] {
+        HE_REQUIRE(plan && terms && count && capacity >= fsearch::CostTerms::kCount, HE_ERR_INVALID, "bad argument");
+        double v[fsearch::CostTerms::kCount];
+        fsearch::mi355x_cost_terms(plan->fg).to_array(v);
+        for (int i = 0; i < fsearch::CostTerms::kCount; i++) terms[i] = v[i];
+        *count = fsearch::CostTerms::kCount;
     });
 }
 

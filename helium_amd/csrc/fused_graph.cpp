@@ -1,5 +1,7 @@
 #include "fused_graph.h"
 
+#include <cmath>
+
 #include <algorithm>
 #include <functional>
 #include <sstream>
@@ -690,13 +692,135 @@ double analytical_cost(const FusedGraph& fg) {
 }
 
 // ---------------------------------------------------------------------------------------------------------
+// MI355X model
+// ---------------------------------------------------------------------------------------------------------
+namespace {
+// Vector instructions an op costs per element in the generated kernels (fast intrinsics; transcendental instructions
+// issue at a quarter of the plain rate).
+double op_weight(const fir::Op& op) {
+    if (op.kind == OpKind::UnaryPointwise) {
+        switch ((fir::UnaryOp)op.sub_op) {
+            case fir::UnaryOp::Neg:
+            case fir::UnaryOp::Relu:
+            case fir::UnaryOp::AddConstant:
+            case fir::UnaryOp::MulConstant: return 1;
+            case fir::UnaryOp::PowConstant: return op.constant == 2.0f ? 1 : 12;
+            case fir::UnaryOp::Exp: return 5;
+            case fir::UnaryOp::Gelu: return 14;
+            case fir::UnaryOp::Ln: return 5;
+            case fir::UnaryOp::Sqrt: return 4;
+            case fir::UnaryOp::Tanh: return 10;
+        }
+    } else if (op.kind == OpKind::BinaryPointwise) {
+        switch ((fir::BinaryOp)op.sub_op) {
+            case fir::BinaryOp::Add:
+            case fir::BinaryOp::Sub:
+            case fir::BinaryOp::Mul: return 1;
+            case fir::BinaryOp::Div: return 6;
+            case fir::BinaryOp::Pow: return 12;
+            case fir::BinaryOp::Drelu: return 2;
+        }
+    } else if (op.kind == OpKind::Reduction) {
+        return 2;
+    }
+    return 0;
+}
+double storage_bytes(const fir::OpGraph& g, OpNode n) {
+    const fir::Op& op = g.get(n);
+    int dt = HE_BF16;  // values between kernels travel as bf16, reductions as f32
+    if (op.kind == OpKind::Producer) dt = op.dtype;
+    else if (op.kind == OpKind::Reduction) dt = HE_F32;
+    else
+        for (OpNode c : g.outbound(n))
+            if (g.get(c).kind == OpKind::Consumer) dt = g.get(c).dtype;
+    return (double)elements(g, n) * (double)(dtype_bits(dt) / 8);
+}
+}  // namespace
+
+void CostTerms::to_array(double (&out)[kCount]) const {
+    const double v[kCount] = {launches, mma_flops, mainloop_l2_bytes, mainloop_ops, hbm_bytes, epilogue_ops, aux_ops};
+    for (int i = 0; i < kCount; i++) out[i] = v[i];
+}
+
+CostTerms mi355x_cost_terms(const FusedGraph& fg) {
+    const fir::OpGraph& g = fg.opgraph();
+    CostTerms t;
+    for (auto& [id, f] : fg.fusions()) {
+        if (f.is_input_output(g)) continue;
+        t.launches += 1;
+        bool reduces = false;
+        std::set<OpNode> written;
+        for (auto& d : f.dependents) written.insert(d.first);
+        for (OpNode n : written) t.hbm_bytes += storage_bytes(g, n);
+        if (!f.core) {
+            for (OpNode n : f.fused) {
+                t.aux_ops += op_weight(g.get(n)) * (double)elements(g, g.get(n).kind == OpKind::Reduction ? g.get(n).a : n);
+                reduces = reduces || g.get(n).kind == OpKind::Reduction;
+            }
+            for (auto& [dep, provider] : f.dependencies) t.hbm_bytes += storage_bytes(g, dep);
+            if (reduces) t.launches += 1;
+            continue;
+        }
+        const fir::Op& mm = g.get(f.anchor);
+        const fir::Shape3 &sa = g.shape(mm.a), &sb = g.shape(mm.b);
+        const double batch = sa[0], M = sa[1], K = sa[2], N = sb[2];
+        t.mma_flops += 2.0 * batch * M * N * K;
+        // an operand's chain is computed again by every 256-wide tile column (A) or tile row (B) of the product
+        const double rep_a = std::ceil(N / 256.0), rep_b = std::ceil(M / 256.0);
+        const std::vector<OpNode> side_a = ancestors_in_fusion(f, g, mm.a), side_b = ancestors_in_fusion(f, g, mm.b);
+        std::set<OpNode> operand_deps_a, operand_deps_b;
+        auto side = [&](const std::vector<OpNode>& nodes, OpNode operand, double rep, std::set<OpNode>& deps) {
+            double bytes = 0;
+            for (OpNode n : nodes) {
+                if (f.contains(n) && n != f.anchor) t.mainloop_ops += op_weight(g.get(n)) * (double)elements(g, n) * rep;
+                for (OpNode prev : g.inbound(n))
+                    if (f.dependencies.count(prev) && deps.insert(prev).second) bytes += storage_bytes(g, prev) * rep;
+            }
+            if (f.dependencies.count(operand) && deps.insert(operand).second) bytes += storage_bytes(g, operand) * rep;
+            // the plain operand's own stream is part of the product's rate
+            bytes -= (double)elements(g, operand) * 2.0 * rep;
+            if (bytes > 0) t.mainloop_l2_bytes += bytes;
+        };
+        side(side_a, mm.a, rep_a, operand_deps_a);
+        side(side_b, mm.b, rep_b, operand_deps_b);
+        for (OpNode n : f.epilogue) {
+            t.epilogue_ops += op_weight(g.get(n)) * (double)elements(g, g.get(n).kind == OpKind::Reduction ? g.get(n).a : n);
+            reduces = reduces || g.get(n).kind == OpKind::Reduction;
+        }
+        for (auto& [dep, provider] : f.dependencies)
+            if (!operand_deps_a.count(dep) && !operand_deps_b.count(dep)) t.hbm_bytes += storage_bytes(g, dep);
+        if (reduces) t.launches += 1;
+    }
+    return t;
+}
+
+Mi355xCoefficients Mi355xCoefficients::fitted() {
+    // seconds per: launch, matrix-core FLOP, L2->CU byte of extra operands, weighted mainloop op, HBM byte, weighted
+    // epilogue op, weighted op of an anchor-less kernel. Non-negative least squares over the 30 measured plans listed in
+    // profiles/cost_model_fit.txt (helium_amd/cost_fit.py): mean relative error 5%, worst 12%. The launch term carries
+    // the host's time per kernel of he_fusion_plan_execute; the extra-operand bytes and the mainloop ops of the measured
+    // plans grow together, and the fit puts all of their weight on the ops.
+    return {1.467e-05, 6.998e-16, 0.0, 1.022e-13, 6.747e-14, 8.514e-15, 3.356e-14};
+}
+
+double mi355x_cost(const FusedGraph& fg, const Mi355xCoefficients& k) {
+    double v[CostTerms::kCount];
+    mi355x_cost_terms(fg).to_array(v);
+    double c = 0;
+    for (int i = 0; i < CostTerms::kCount; i++) c += k.c[i] * v[i];
+    return c;
+}
+
+// ---------------------------------------------------------------------------------------------------------
 // Search
 // ---------------------------------------------------------------------------------------------------------
 SearchResult minimize_cost(std::shared_ptr<const fir::OpGraph> g, Objective objective, const CostParams& p, size_t max_states,
                            FusionId first_id) {
     FusedGraph initial = FusedGraph::identity(g, first_id);
     initial.produce_maximal_fusions();
-    auto cost_of = [&](const FusedGraph& fg) { return objective == Objective::Analytical ? analytical_cost(fg) : naive_cost(fg, p); };
+    auto cost_of = [&](const FusedGraph& fg) {
+        return objective == Objective::Analytical ? analytical_cost(fg) : objective == Objective::Mi355x ? mi355x_cost(fg) : naive_cost(fg, p);
+    };
     if (objective == Objective::Maximal) return {initial, naive_cost(initial, p), 1};
 
     bool have_best = false, best_updated = false;
@@ -756,7 +880,7 @@ SearchResult minimize_cost_with_subdivision(std::shared_ptr<const fir::OpGraph> 
         fused.push_back(std::move(r.graph));
     }
     FusedGraph merged = FusedGraph::merge_from_subdivisions(subdivisions, fused, g);
-    const double cost = objective == Objective::Analytical ? analytical_cost(merged) : naive_cost(merged, p);
+    const double cost = objective == Objective::Analytical ? analytical_cost(merged) : objective == Objective::Mi355x ? mi355x_cost(merged) : naive_cost(merged, p);
     return {merged, cost, states};
 }
 

@@ -98,6 +98,31 @@ struct CostParams {
 double naive_cost(const FusedGraph& fg, const CostParams& p);  // cost_model.rs:9-89
 double analytical_cost(const FusedGraph& fg);                   // cost_model.rs:91-231 (coefficients as published there)
 
+// A cost model of the same purpose as the analytical one, for this backend's kernels on MI355X: the time of a plan
+// is a sum over its kernels, linear in seven terms whose coefficients are fitted to measured kernels
+// (helium_amd/cost_fit.py measures and fits; profiles/cost_model_fit.txt holds the data). The terms say what the
+// hardware bounds: matrix-core work, the bytes a kernel moves to and from HBM, the vector work of epilogue / anchor-less
+// kernels, and - what makes a mainloop fusion lose on this chip - the operand traffic from L2 to the CUs, which every
+// tile column (for A) or tile row (for B) of a product repeats: a fused `relu(A0) * T` makes 16 workgroups per tile row
+// stream T next to A0, 1.5x the plain k-loop's bytes on a loop that is bound by exactly that stream.
+struct CostTerms {
+    double launches = 0;           // kernels, plus one fold launch per kernel that ends in reductions
+    double mma_flops = 0;          // 2 b M N K of every anchor
+    double mainloop_l2_bytes = 0;  // operand bytes streamed to the CUs beyond the two plain operands
+    double mainloop_ops = 0;       // weighted vector ops on operand elements, times the tiles that repeat them
+    double hbm_bytes = 0;          // tensors read from and written to memory by epilogues and anchor-less kernels
+    double epilogue_ops = 0;       // weighted vector ops on accumulator elements
+    double aux_ops = 0;            // weighted vector ops of anchor-less kernels
+    static constexpr int kCount = 7;
+    void to_array(double (&out)[kCount]) const;
+};
+struct Mi355xCoefficients {
+    double c[CostTerms::kCount];
+    static Mi355xCoefficients fitted();
+};
+CostTerms mi355x_cost_terms(const FusedGraph& fg);
+double mi355x_cost(const FusedGraph& fg, const Mi355xCoefficients& k = Mi355xCoefficients::fitted());
+
 // cost_model.rs:256-343: maximal fusions, then depth-7 searches from the best state until none improves.
 // `max_states` bounds the states visited per search (the reference has no bound).
 struct SearchResult {
@@ -105,7 +130,7 @@ struct SearchResult {
     double cost;
     size_t states_visited;
 };
-enum class Objective : int { Maximal = 0, Naive = 1, Analytical = 2 };
+enum class Objective : int { Maximal = 0, Naive = 1, Analytical = 2, Mi355x = 3 };
 SearchResult minimize_cost(std::shared_ptr<const fir::OpGraph> g, Objective objective, const CostParams& p, size_t max_states = 200000,
                            FusionId first_id = 0);
 // cost_model.rs:241-259: subdivide, search every subdivision's subgraph on its own, merge. The search is exponential

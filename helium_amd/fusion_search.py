@@ -5,7 +5,8 @@ import ctypes as C
 from . import _ffi
 from ._ffi import check, lib
 
-MAXIMAL, MIN_NAIVE_COST, MIN_ANALYTICAL_COST = 0, 1, 2
+MAXIMAL, MIN_NAIVE_COST, MIN_ANALYTICAL_COST, MIN_MI355X_COST = 0, 1, 2, 3
+COST_TERMS = ["launches", "mma_flops", "mainloop_l2_bytes", "mainloop_ops", "hbm_bytes", "epilogue_ops", "aux_ops"]
 ROLES = ["mainloop", "epilogue", "anchor", "aux"]
 PORTIONS = ["mainloop", "epilogue", "full"]
 
@@ -16,6 +17,7 @@ _ffi._sig("he_fusion_plan_fusion_info", C.c_void_p, C.c_int, C.POINTER(C.c_int32
           C.POINTER(C.c_int32), C.c_int, C.POINTER(C.c_int))
 _ffi._sig("he_fusion_plan_describe", C.c_void_p, restype=C.c_char_p)
 _ffi._sig("he_fusion_plan_cost", C.c_void_p, C.c_int, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_uint64))
+_ffi._sig("he_fusion_plan_cost_terms", C.c_void_p, C.POINTER(C.c_double), C.c_int, C.POINTER(C.c_int))
 _ffi._sig("he_fusion_plan_precompile", C.c_void_p)
 _ffi._sig("he_fusion_plan_execute", C.c_void_p, C.POINTER(C.c_uint64), C.POINTER(C.c_void_p), C.c_int, C.POINTER(C.c_uint64),
           C.POINTER(C.c_void_p), C.c_int, C.c_void_p)
@@ -54,6 +56,12 @@ class FusionPlan:
         c, states = C.c_double(), C.c_uint64()
         check(lib.he_fusion_plan_cost(self.handle, objective, int(reference_constants), C.byref(c), C.byref(states)))
         return c.value
+
+    def cost_terms(self):
+        """The terms of the MI355X cost model for this plan, by name (the model is their weighted sum)."""
+        v, n = (C.c_double * 16)(), C.c_int()
+        check(lib.he_fusion_plan_cost_terms(self.handle, v, 16, C.byref(n)))
+        return dict(zip(COST_TERMS, v[: n.value]))
 
     def precompile(self):
         check(lib.he_fusion_plan_precompile(self.handle))

@@ -317,7 +317,10 @@ int he_execute_graph(he_graph_t graph, const uint32_t* input_nodes, const he_ten
  * and Aux fusions; each becomes one kernel (he_fused_kernel_create's generators) and he_fusion_plan_execute runs
  * them in dependency order with pooled temporaries. */
 typedef struct he_fusion_plan_s* he_fusion_plan_t;
-enum { HE_FUSE_MAXIMAL = 0, HE_FUSE_MIN_NAIVE_COST = 1, HE_FUSE_MIN_ANALYTICAL_COST = 2 };
+/* HE_FUSE_MIN_ANALYTICAL_COST is analytical_cost_function with the coefficients its authors fitted on their hardware
+ * (cost_model.rs:200-207); HE_FUSE_MIN_MI355X_COST is the model of the same purpose fitted to this backend's kernels on
+ * MI355X (terms: launches, matrix-core FLOP, L2->CU bytes of operands a mainloop fusion adds, HBM bytes, vector ops). */
+enum { HE_FUSE_MAXIMAL = 0, HE_FUSE_MIN_NAIVE_COST = 1, HE_FUSE_MIN_ANALYTICAL_COST = 2, HE_FUSE_MIN_MI355X_COST = 3 };
 enum { HE_FUSION_ROLE_MAINLOOP = 0, HE_FUSION_ROLE_EPILOGUE = 1, HE_FUSION_ROLE_ANCHOR = 2, HE_FUSION_ROLE_AUX = 3 };
 /* objective HE_FUSE_MAXIMAL: produce_maximal_fusions only (fused_graph.rs:113-223); otherwise minimize_cost_function
  * (cost_model.rs:256-343) with the naive model on MI355X rates or the analytical model. */
@@ -330,8 +333,14 @@ int he_fusion_plan_num_fusions(he_fusion_plan_t plan, int* count);   /* kernels,
 int he_fusion_plan_fusion_info(he_fusion_plan_t plan, int index, int32_t* is_core, uint64_t* anchor, uint64_t* nodes,
                                int32_t* roles, int capacity, int* count);
 const char* he_fusion_plan_describe(he_fusion_plan_t plan);           /* FusedGraph::print (fused_graph.rs:1060-1068) */
-/* objective 1: naive model (reference_constants != 0: the constants of cost_model.rs:10-12), 2: analytical model */
+/* objective 1: naive model (reference_constants != 0: the constants of cost_model.rs:10-12), 2: analytical model, 3: the
+ * MI355X model (seconds) */
 int he_fusion_plan_cost(he_fusion_plan_t plan, int objective, int reference_constants, double* cost, uint64_t* states_visited);
+/* The MI355X model's terms for the plan, in the order: launches, matrix-core FLOP, L2->CU bytes of extra mainloop
+ * operands, weighted mainloop ops, HBM bytes, weighted epilogue ops, weighted ops of anchor-less kernels. The model is
+ * linear in them, which is what its fit uses. No counterpart in the reference (its coefficients are constants in
+ * cost_model.rs:200-207 with no code that derived them). */
+int he_fusion_plan_cost_terms(he_fusion_plan_t plan, double* terms, int capacity, int* count);
 int he_fusion_plan_precompile(he_fusion_plan_t plan);
 /* Producers and Consumers of the whole graph are bound by node id; values between kernels are bf16 (f32 for
  * reductions) in pooled device memory. */

@@ -264,3 +264,60 @@ def test_random_graphs_searched_by_subdivision(seed):
     assert {n for n in live if by_id[n]["op"] not in ("producer", "consumer")} <= done
     assert p.cost() <= fs.FusionPlan(g, fs.MAXIMAL).cost() * (1 + 1e-12)
     p.precompile()
+
+
+# ---- the MI355X cost model (no counterpart in the reference beyond its fitted constants, cost_model.rs:200-207) ------
+# Times measured on an MI355X with `python -m helium_amd.cost_fit` (profiles/cost_model_fit.txt), microseconds.
+MEASURED_US = {
+    ("C5a", "core[m2,e3]"): 164.7, ("C5a", "aux[2]+core[m0,e3]"): 133.3, ("C5a", "aux[1]+aux[2]+core[m0,e2]"): 148.1,
+    ("C4m", "core[m2,e39]"): 199.3, ("C4m", "aux[2]+core[m0,e39]"): 171.4,
+    ("C4", "core[m0,e39]"): 146.8, ("C4", "aux[5]+aux[1]+aux[6]+core[m0,e27]"): 195.7,
+    ("relu(A) gemm", "core[m1,e0]"): 138.6, ("relu(A) gemm", "aux[1]+core[m0,e0]"): 126.9,
+    ("gemm + bias + relu", "core[m0,e3]"): 116.4, ("gemm + bias + relu", "aux[1]+core[m0,e2]"): 128.8,
+}
+
+
+def _kinds(plan):
+    return "+".join(("core[m%d,e%d]" % (len(f["mainloop"]), len(f["epilogue"]))) if f["core"] else "aux[%d]" % len(f["aux"])
+                    for f in plan.fusions)
+
+
+def test_mi355x_model_ranks_the_measured_plans_the_way_the_gpu_did():
+    from helium_amd import cost_fit
+
+    graphs = cost_fit.graphs()
+    for name in sorted({k[0] for k in MEASURED_US}):
+        plans = {}
+        for objective in (fs.MAXIMAL, fs.MIN_NAIVE_COST, fs.MIN_ANALYTICAL_COST, fs.MIN_MI355X_COST):
+            p = fs.FusionPlan(graphs[name], objective)
+            plans[_kinds(p)] = p
+        known = [(MEASURED_US[(name, k)], plans[k].cost(fs.MIN_MI355X_COST) * 1e6, k) for k in plans if (name, k) in MEASURED_US]
+        assert len(known) >= 2, (name, list(plans))
+        # same order, and each prediction within 15% of its measurement
+        assert [k for _, _, k in sorted(known)] == [k for _, _, k in sorted(known, key=lambda r: r[1])], (name, known)
+        for measured, predicted, k in known:
+            assert abs(predicted - measured) <= 0.15 * measured, (name, k, measured, predicted)
+        # and what the search returns under this model is the fastest of the measured plans
+        best = _kinds(fs.FusionPlan(graphs[name], fs.MIN_MI355X_COST))
+        assert MEASURED_US[(name, best)] == min(m for m, _, _ in known), (name, best, known)
+
+
+def test_mi355x_model_materialises_a_mainloop_chain_that_many_tile_columns_would_repeat():
+    """Config 5a: relu(A0) * T feeds a 4096-wide product, so 16 workgroups per tile row would each stream T and
+    recompute the chain; the model prices that above one pass over A0 and T, and the search splits the chain off. With
+    a single tile column nothing is repeated and the chain stays in the mainloop."""
+    from helium_amd import configs
+
+    g, names = configs.c5a_graph(4096)
+    p = fs.FusionPlan(g, fs.MIN_MI355X_COST)
+    assert _kinds(p) == "aux[2]+core[m0,e3]"
+    terms = p.cost_terms()
+    assert terms["launches"] == 2 and terms["mainloop_ops"] == 0 and terms["mma_flops"] == 2.0 * 4096 ** 3
+    fused = fs.FusionPlan(g, fs.MIN_NAIVE_COST)
+    assert _kinds(fused) == "core[m2,e3]" and fused.cost(fs.MIN_MI355X_COST) > p.cost(fs.MIN_MI355X_COST)
+    assert fused.cost_terms()["mainloop_l2_bytes"] == 16 * 4096 * 4096 * 2   # T, once per tile column
+
+    narrow = ha.fusion.OpGraph()
+    a0, t, b = narrow.producer([1, 4096, 4096]), narrow.producer([1, 4096, 4096]), narrow.producer([1, 4096, 256])
+    narrow.consumer(narrow.matmul(narrow.binary(narrow.unary(a0, "relu"), t, "mul"), b))
+    assert _kinds(fs.FusionPlan(narrow, fs.MIN_MI355X_COST)) == "core[m2,e0]"
