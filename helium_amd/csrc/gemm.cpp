@@ -855,7 +855,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     const bool direct_a = want_direct && raw_a && (pr.conv_a.on ? pr.conv_a.C % epc == 0 : pr.M % t.bm == 0 && pr.K % t.bk == 0) &&
                           (!pr.a_km || 64 % (t.bm / epc) == 0) && (t.bm * t.bk * esz / 1024) % (threads / 64) == 0 &&
                           !tuning::get("HELIUM_HIP_GEMM_NO_DIRECT_A");
-    const bool direct_b = want_direct && raw_b && (pr.conv_b.on || (pr.N % t.bn == 0 && pr.K % t.bk == 0)) && (t.bk * t.bn * esz / 1024) % (threads / 64) == 0 &&
+    const bool direct_b = want_direct && raw_b && (pr.conv_b.on ? pr.conv_b.C % epc == 0 : pr.N % t.bn == 0 && pr.K % t.bk == 0) && (t.bk * t.bn * esz / 1024) % (threads / 64) == 0 &&
                           (pr.b_nk || 64 % (t.bn / epc) == 0) && !tuning::get("HELIUM_HIP_GEMM_NO_DIRECT_B");
     // A convolution's gather with direct loads, a channel count that is a multiple of the k-tile (every tile then lies in
     // one filter tap) and a wave that issues a whole number of loads: the per-lane address arithmetic of a load
@@ -997,19 +997,10 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         s << "at = (size_t)base + (size_t)(((u32)ih * " << cv.W << "u + (u32)iw) * " << cv.C << "u + c);\n"
           << "return k0 < " << cv.R * cv.S * cv.C << "u && hit && ih >= 0 && ih < " << cv.H << " && iw >= 0 && iw < " << cv.W << ";\n}\n";
     }
-    if (pr.conv_a.on) {
-        // The gather of an implicit-GEMM convolution in place of A's loads: one 16-byte chunk is EPC consecutive
-        // channels of one filter tap when the channel count allows, EPC separate taps otherwise (a 3-channel image).
-        const auto& cv = pr.conv_a;
-        const tp::Arg& img = pr.op_a.args[0];
-        s << "#define FETCH_A_ARGS p" << pr.map_a[0] << ", \n#define RAW_A 1\n#define SPLIT_A 1\n";
-        emit_conv_tap(cv);
-        s << "__device__ __forceinline__ u32x4 fetch_a(const " << tp::c_type(img.dtype) << "* __restrict__ q0, u32 b, u32 row, u32 col) {\n(void)b;\n";
-        if (cv.C % epc == 0) {
-            s << "u32x4 v = {0u, 0u, 0u, 0u};\nsize_t at;\nif (conv_tap(row, col, at)) v = *(const u32x4*)(q0 + at);\nreturn v;\n}\n";
-        } else {
-            // EPC consecutive columns of one row: the pixel is decomposed once, and the tap walks on by one channel per
-            // element (a 3-channel image: 8 elements span 3 taps) instead of being decomposed 8 times
+    // Body of a gather that fetches EPC consecutive taps (columns) of one pixel (row) element by element, for images whose
+    // channel count does not fill 16-byte chunks (a 3-channel image: 8 elements span 3 taps): the pixel is decomposed
+    // once, and the tap walks on by one channel per element instead of being decomposed 8 times.
+    auto emit_elementwise_gather = [&](const GemmProblem::ConvGather& cv) {
             s << "float v[" << epc << "];\n"
               << "const u32 n = row / " << cv.P * cv.Q << "u, pq = row % " << cv.P * cv.Q << "u, p = pq / " << cv.Q << "u, q = pq % " << cv.Q << "u;\n"
               << "u32 rs = col / " << cv.C << "u, c = col % " << cv.C << "u, r = rs / " << cv.S << "u, sx = rs % " << cv.S << "u;\n"
@@ -1026,6 +1017,19 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
               << "v[j] = inside ? ld_one(q0 + (((size_t)n * " << cv.H << "u + (u32)ih) * " << cv.W << "u + (u32)iw) * " << cv.C << "u + c) : 0.0f;\n"
               << "if (++c == " << cv.C << "u) { c = 0u; if (++sx == " << cv.S << "u) { sx = 0u; ++r; } }\n}\n"
               << "return pack_chunk(v);\n}\n";
+    };
+    if (pr.conv_a.on) {
+        // The gather of an implicit-GEMM convolution in place of A's loads: one 16-byte chunk is EPC consecutive
+        // channels of one filter tap when the channel count allows, EPC separate taps otherwise.
+        const auto& cv = pr.conv_a;
+        const tp::Arg& img = pr.op_a.args[0];
+        s << "#define FETCH_A_ARGS p" << pr.map_a[0] << ", \n#define RAW_A 1\n#define SPLIT_A 1\n";
+        emit_conv_tap(cv);
+        s << "__device__ __forceinline__ u32x4 fetch_a(const " << tp::c_type(img.dtype) << "* __restrict__ q0, u32 b, u32 row, u32 col) {\n(void)b;\n";
+        if (cv.C % epc == 0) {
+            s << "u32x4 v = {0u, 0u, 0u, 0u};\nsize_t at;\nif (conv_tap(row, col, at)) v = *(const u32x4*)(q0 + at);\nreturn v;\n}\n";
+        } else {
+            emit_elementwise_gather(cv);
         }
     } else if (pr.a_km) {
         emit_fetch("a", pr.op_a, pr.root_a, pr.map_a, raw_a, nva, "GK", "GM", pr.M % t.bm == 0 && pr.K % t.bk == 0);
@@ -1035,8 +1039,9 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     if (pr.conv_b.on) {
         emit_conv_tap(pr.conv_b);
         s << "#define FETCH_B_ARGS p" << pr.map_b[0] << ", \n#define RAW_B 1\n#define SPLIT_B 1\n";
-        s << "__device__ __forceinline__ u32x4 fetch_b(const " << tp::c_type(pr.op_b.args[0].dtype) << "* __restrict__ q0, u32 b, u32 row, u32 col) {\n(void)b;\n"
-          << "u32x4 v = {0u, 0u, 0u, 0u};\nsize_t at;\nif (conv_tap(row, col, at)) v = *(const u32x4*)(q0 + at);\nreturn v;\n}\n";
+        s << "__device__ __forceinline__ u32x4 fetch_b(const " << tp::c_type(pr.op_b.args[0].dtype) << "* __restrict__ q0, u32 b, u32 row, u32 col) {\n(void)b;\n";
+        if (pr.conv_b.C % epc == 0) s << "u32x4 v = {0u, 0u, 0u, 0u};\nsize_t at;\nif (conv_tap(row, col, at)) v = *(const u32x4*)(q0 + at);\nreturn v;\n}\n";
+        else emit_elementwise_gather(pr.conv_b);  // the filter gradient of a 3-channel image: B[pixel][(r, s, c)]
     } else if (pr.b_rows.on) {
         const auto& br = pr.b_rows;
         s << "__device__ __forceinline__ size_t b_row_addr(u32 k) { return (size_t)(k % " << br.group << "u) * " << br.o_stride << "ull + (size_t)(k / "

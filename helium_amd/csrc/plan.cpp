@@ -678,8 +678,6 @@ GemmProblem conv_backward_filter_problem(const ir::OpSubgraph& sg, NodeId node) 
     pr.K = cv.N * cv.P * cv.Q;
     HE_REQUIRE(pr.K > 0 && pr.K < (1ll << 31) && ir::num_elements(image.shape) < (1ll << 32), HE_ERR_UNSUPPORTED, "conv too large for 32-bit tile indices");
     pr.mma_dtype = flow.dtype == HE_F32 ? HE_F32 : flow.dtype == HE_F16 ? HE_F16 : HE_BF16;
-    const int64_t epc = pr.mma_dtype == HE_F32 ? 4 : 8;
-    HE_REQUIRE(cv.C % epc == 0, HE_ERR_UNSUPPORTED, "conv backward filter needs an input-channel count that fills 16-byte chunks");
     auto operand = [&](tp::Program& p, const ir::Descriptor& d, NodeId n, int64_t rows, int64_t cols) {
         p.dims = {1, rows, cols};
         p.args.push_back({d.dtype, ir::num_elements(d.shape), false, n});

@@ -341,6 +341,10 @@ BWD_FILTER_CASES = [
     ("1x1_stride2_shortcut", (2, 8, 8, 32), 64, (1, 1), "bf16", (2, 2), (1, 1), "same", "128,128,64,2,2"),
     ("direct_loads_both_operands", (4, 16, 16, 16), 128, (3, 3), "bf16", (1, 1), (1, 1), "same", "128,128,64,2,2"),
     ("valid_and_dilated_f32", (2, 9, 9, 4), 8, (3, 3), "f32", (1, 1), (2, 1), "valid", "64,64,32,2,2"),
+    # channel counts that do not fill a 16-byte chunk: the image operand is gathered element by element
+    ("three_channel_stem_7x7_stride2", (2, 16, 16, 3), 32, (7, 7), "bf16", (2, 2), (1, 1), "same", "64,128,64,2,2"),
+    ("five_channels_3x3_f16", (1, 7, 9, 5), 8, (3, 3), "f16", (1, 1), (1, 1), "same", "64,64,64,2,2"),
+    ("three_channels_f32_full", (1, 6, 5, 3), 8, (3, 3), "f32", (1, 1), (1, 2), "full", "64,64,32,2,2"),
 ]
 
 
