@@ -869,6 +869,73 @@ class FusedGemmWorkload:
         self.sets = []
 
 
+class TrainStepWorkload:
+    """BASELINE config 5b: one whole training step of the resnet-train example (resnet-train/src/train.rs:383-396 on the
+    model of model.rs) through execute_graph: forward in Train mode, cross-entropy, backward, SGD with momentum 0.9.
+    Every step feeds the previous step's parameters, gradient averages and running statistics back in. The work figure
+    is the matrix-core FLOP of the step's convolutions (forward, data and filter gradients; the data gradient of the
+    3-channel image is never asked for); images/s is reported next to it."""
+
+    bound = "mfma"
+    unit = "TFLOP/s"
+    dtype = "bf16 activations and flows, f32 parameters and accumulation"
+    wall_timed = True
+
+    def __init__(self, name, batch, image):
+        self.name, self.batch, self.image = name, batch, image
+        self.work = 0
+
+    def describe(self):
+        return (f"{self.name}: resnet-train training step (forward, cross-entropy, backward, SGD momentum), batch {self.batch}, "
+                f"{self.image}x{self.image}x3 bf16 images, 1000 classes, via execute_graph")
+
+    def setup(self):
+        from helium_amd import resnet
+        from helium_amd.backend import Tensor, stats
+
+        self.rec = resnet.record_training_step(self.batch, self.image)
+        G = self.rec["graph"]
+        self.g = G.g
+        by_id = {n["id"]: n for n in self.g.nodes}
+        flop = 0
+        for n in self.g.nodes:
+            if n.get("op") in ("conv", "conv_bwd_data", "conv_bwd_filter"):
+                p = n["params"]
+                if n["op"] == "conv_bwd_data" and p["in_channels"] == 3:
+                    continue  # the image has no gradient: pruned
+                pixels = by_id[n["inputs"][0]]["shape"] if n["op"] != "conv" else n["shape"]
+                flop += 2 * int(np.prod(pixels[:3])) * p["out_channels"] * p["kernel_size"][0] * p["kernel_size"][1] * p["in_channels"]
+        self.work = flop
+        self.tensors = {i: Tensor.from_numpy(a, by_id[i]["dtype"], int(np.prod(by_id[i]["shape"]))) for i, a in G.feeds.items()}
+        self.outs = None
+        self._stats = stats
+        log(f"[bench] {self.describe()} :: {len(self.g.nodes)} graph nodes, {self.work / 1e9:.1f} GFLOP of convolutions per step")
+
+    def step(self, stream, i):
+        from helium_amd.backend import execute_graph
+
+        outs = execute_graph(self.g, self.tensors)
+        for src, dst in self.rec["carried"]:
+            self.tensors[src] = outs[dst]
+        self.outs = outs
+
+    def check(self):
+        st = self._stats()
+        loss = float(self.outs[self.rec["loss"]].to_numpy()[0])
+        probs = self.outs[self.rec["probs"]].to_numpy().reshape(self.batch, -1).astype(np.float64)
+        if not (abs(loss - np.log(1000.0)) < 0.35 and np.allclose(probs.sum(axis=1), 1.0, atol=1e-3)):
+            raise SystemExit(f"[bench] PARITY FAILURE in {self.name}: first-step loss {loss}, probabilities sum to {probs.sum(axis=1)[:4]}")
+        self.instrs = st["instrs"]
+        return (f"first step: loss {loss:.4f} (ln 1000 = 6.9078), probabilities sum to 1 per image; {st['instrs']} instructions in {st['steps']} plan "
+                f"steps; the same graph at [8,64,64,3] agrees with the oracle output by output (tests/test_resnet_step_gpu.py)")
+
+    def cpu_baseline(self, budget_s=5.0):
+        return None
+
+    def free(self):
+        self.tensors, self.outs = {}, None
+
+
 class PlannedGemmWorkload(FusedGemmWorkload):
     """The same graphs, run the way the fusion search plans them under the MI355X cost model (he_fusion_search with
     HE_FUSE_MIN_MI355X_COST, then he_fusion_plan_execute): a mainloop chain that 16 tile columns would each repeat is
@@ -975,6 +1042,8 @@ def make_workloads():
     w["C5b-conv-bwd-filter"] = ConvBackwardFilterWorkload()
     w["C5b-sgd"] = SgdWorkload()
     w["C5b-block"] = BasicBlockWorkload()
+    w["C5b"] = TrainStepWorkload("C5b", 128, 224)          # BASELINE's batch and image size
+    w["C5b-ref"] = TrainStepWorkload("C5b-ref", 64, 256)   # the reference's own (train.rs:33,286-287)
     for name in ("C4", "C5a", "C4m", "GEMM"):
         w[name] = FusedGemmWorkload(name)
     # C5a and C4m as one kernel each (every mainloop op fused) stay measurable next to the planned form
@@ -1065,6 +1134,9 @@ def main():
         rl = roofline(wl, ms)
         kernels[name] = {"workload": wl.describe(), "ms": round(ms, 5), "wall_ms": round(wall, 5), "parity": parity,
                          "roofline": rl}
+        if isinstance(wl, TrainStepWorkload):
+            kernels[name]["images_per_s"] = round(wl.batch / (ms * 1e-3), 1)
+            log(f"[bench] {name}: {kernels[name]['images_per_s']} images/s")
         log(f"[bench] {name}: {ms * 1e3:.1f} us/step -> {rl['achieved']} {rl['unit']} ({rl['frac'] * 100:.1f}% of peak)")
         if name == headline:
             cpu = None if args.no_cpu else wl.cpu_baseline()

@@ -1,0 +1,136 @@
+"""The whole training step of the reference's resnet-train example (resnet-train/src/train.rs:383-396 on the model of
+model.rs:22-84,155-249) through execute_graph: forward in Train mode, cross-entropy, the backward pass the reference's
+gradient rules record (helium/src/tensor.rs), Sgd::step with momentum - about 4800 helium-ir nodes, 720 instructions.
+
+Parity is taken twice. With f32 images every output has to agree with the oracle, run under the same plan, to 1e-3 of
+the tensor's largest element. With the reference's bf16 images (train.rs:68-87) the same holds for everything the
+forward pass produces; the gradients below the last layer are not a function the arithmetic pins down there: batch
+norm takes its variance as E[x^2] - E[x]^2 from bf16 means (batch_norm.rs:44-49), and the oracle itself moves by 30-60%
+of a gradient's largest element when only the places where values are rounded to bf16 change (one kernel per op versus
+the plan's kernels). So there the test asks for no more than that: the GPU stays as close to the oracle as the oracle
+stays to itself. The gradient of a convolution's bias is the sum of a flow that a following batch norm has centred: zero
+but for rounding, in any arithmetic - those are checked to be small, not equal."""
+import numpy as np
+import pytest
+
+from helium_amd import resnet
+from helium_amd.backend import Plan, Tensor, execute_graph
+from oracle import helium_ir as oracle_ir
+from oracle import numerics as nm
+
+pytestmark = pytest.mark.gpu
+
+BATCH, IMAGE, WIDTH, CLASSES = 8, 64, 8, 16
+
+
+def _run(dtype):
+    r = resnet.record_training_step(BATCH, IMAGE, width=WIDTH, num_classes=CLASSES, dtype=dtype)
+    G = r["graph"]
+    by_id = {n["id"]: n for n in G.g.nodes}
+    tensors = {i: Tensor.from_numpy(a, by_id[i]["dtype"], int(np.prod(by_id[i]["shape"]))) for i, a in G.feeds.items()}
+    got = {o: t.to_numpy() for o, t in execute_graph(G.g, tensors).items()}
+    # the executor plans the pruned graph: the oracle follows the plan of the same
+    G.g.optimize()
+    steps = Plan(G.g).steps
+    return r, got, steps
+
+
+def _names(r):
+    """{output node: (module index, kind)} with kind in kernel / bias / scale / shift / mean / variance, each as the new
+    weights ('.w') or the new gradient average ('.avg')."""
+    names, k, model = {}, 0, r["model"]
+    for mi, m in enumerate(model.modules()):
+        kinds = ("kernel", "bias") if isinstance(m, resnet.Conv2d) else ("scale", "shift")
+        for kind in kinds:
+            names[r["carried"][k][1]] = (mi, kind + ".w")
+            names[r["carried"][k + 1][1]] = (mi, kind + ".avg")
+            k += 2
+    for bi, _ in enumerate(model.batch_norms()):
+        names[r["carried"][k][1]] = (bi, "mean")
+        names[r["carried"][k + 1][1]] = (bi, "variance")
+        k += 2
+    names[r["loss"]], names[r["probs"]] = (0, "loss"), (0, "probs")
+    return names
+
+
+def _f64(storage, dtype):
+    return nm.from_storage(np.asarray(storage).reshape(-1), dtype, [np.asarray(storage).size]).astype(np.float64)
+
+
+def _rel(a, b):
+    return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
+
+
+def test_training_step_in_f32_matches_the_oracle_everywhere(gpu):
+    r, got, steps = _run("f32")
+    G = r["graph"]
+    want = oracle_ir.plan_outputs(G.g.nodes, G.feeds, steps)
+    _, desc = oracle_ir.evaluate(G.g.nodes, G.feeds)
+    names = _names(r)
+    assert sorted(got) == sorted(want) == sorted(names)
+    last_conv = len(r["model"].modules()) - 1
+    kernel_scale = {}
+    for o, (mi, kind) in names.items():
+        if kind == "kernel.avg":
+            kernel_scale[mi] = np.abs(_f64(want[o], desc[o][1])).max()
+    for o, (mi, kind) in sorted(names.items()):
+        g_, w_ = _f64(got[o], desc[o][1]), _f64(want[o], desc[o][1])
+        assert np.isfinite(g_).all()
+        if kind == "bias.avg" and mi != last_conv:
+            # a batch norm follows: the true gradient is zero
+            assert max(np.abs(g_).max(), np.abs(w_).max()) <= 1e-5 * kernel_scale[mi], (mi, kind)
+        elif kind == "bias.w" and mi != last_conv:
+            assert np.abs(g_ - w_).max() <= 1e-5 * kernel_scale[mi], (mi, kind)
+        else:
+            assert _rel(g_, w_) <= 1e-3, (mi, kind, _rel(g_, w_))
+
+
+def test_training_step_in_bf16_matches_the_oracle_as_far_as_the_arithmetic_pins_it(gpu):
+    r, got, steps = _run("bf16")
+    G = r["graph"]
+    want = oracle_ir.plan_outputs(G.g.nodes, G.feeds, steps)
+    other, desc = oracle_ir.evaluate(G.g.nodes, G.feeds, materialize=True)   # the same graph, one kernel per op
+    names = _names(r)
+    last_bn = len(r["model"].batch_norms()) - 1
+    modules = r["model"].modules()
+    for o, (mi, kind) in sorted(names.items()):
+        dt = desc[o][1]
+        g_, w_ = _f64(got[o], dt), _f64(want[o], dt)
+        assert np.isfinite(g_).all()
+        if kind in ("loss",):
+            assert _rel(g_, w_) <= 1e-2
+        elif kind == "probs":
+            assert np.abs(g_ - w_).max() <= 2e-2 and np.allclose(g_.reshape(BATCH, CLASSES).sum(axis=1), 1.0, atol=1e-3)
+        elif kind in ("mean", "variance"):
+            assert _rel(g_, w_) <= (2e-2 if mi <= last_bn else 0), (mi, kind, _rel(g_, w_))
+        elif kind.endswith(".avg") and not (kind == "bias.avg" and mi != len(modules) - 1):
+            spread = _rel(_f64(nm.to_storage(other[o], dt), dt), w_)
+            assert _rel(g_, w_) <= max(2.0 * spread, 5e-2), (mi, kind, _rel(g_, w_), spread)
+    # the last layer's gradients sit above every batch norm's backward pass: they are pinned
+    for o, (mi, kind) in names.items():
+        if mi == len(modules) - 1 and kind in ("kernel.avg", "bias.avg"):
+            assert _rel(_f64(got[o], "f32"), _f64(want[o], "f32")) <= 0.1, (kind,)
+
+
+def test_training_step_at_the_reference_size_has_the_invariants_of_a_first_step(gpu):
+    """Batch 64 of 256 x 256 images (train.rs:33,286-287), 1000 classes, random He-initialised weights: the loss is
+    ln(1000) within a few percent, every row of the probabilities sums to one, the running statistics have moved a
+    tenth of the way from (0, 1) towards the batch statistics, and every new parameter is finite."""
+    batch = 64
+    r = resnet.record_training_step(batch, 256)
+    G = r["graph"]
+    by_id = {n["id"]: n for n in G.g.nodes}
+    tensors = {i: Tensor.from_numpy(a, by_id[i]["dtype"], int(np.prod(by_id[i]["shape"]))) for i, a in G.feeds.items()}
+    outs = execute_graph(G.g, tensors)
+    loss = float(outs[r["loss"]].to_numpy()[0])
+    assert abs(loss - np.log(1000.0)) < 0.35, loss
+    probs = outs[r["probs"]].to_numpy().reshape(batch, 1000).astype(np.float64)
+    assert np.allclose(probs.sum(axis=1), 1.0, atol=1e-3) and (probs >= 0).all()
+    names = _names(r)
+    for o, (mi, kind) in names.items():
+        v = _f64(outs[o].to_numpy(), outs[o].dtype)
+        assert np.isfinite(v).all(), (mi, kind)
+        if kind == "variance":
+            assert (v > 0.85).all() and (v < 2.0).all(), (mi, v.min(), v.max())   # 0.9 * 1 + 0.1 * batch variance
+        if kind == "mean":
+            assert np.abs(v).max() < 1.0, (mi,)
