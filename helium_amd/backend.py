@@ -25,6 +25,7 @@ _ffi._sig("he_backend_stats", C.POINTER(C.c_uint64))
 _ffi._sig("he_backend_set_option", C.c_int, C.c_int64)
 OPT_FUSE_MATMUL_EPILOGUE = 0
 OPT_FOLD_SWAP_INTO_REDUCE = 1
+OPT_REMATERIALIZE = 2
 
 
 def set_option(option, value):

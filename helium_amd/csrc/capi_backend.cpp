@@ -59,7 +59,8 @@ int he_plan_generate(he_graph_t graph, he_plan_t* plan) {
     return he::guard([&] {
         HE_REQUIRE(graph && plan, HE_ERR_INVALID, "bad argument");
         // a snapshot of the graph: later edits do not disturb the plan's subgraphs
-        auto snapshot = std::make_shared<he::ir::OpGraph>(*graph->g);
+        std::shared_ptr<const he::ir::OpGraph> snapshot = std::make_shared<he::ir::OpGraph>(*graph->g);
+        snapshot = he::plan::graph_for_execution(snapshot);
         auto p = std::make_unique<he_plan_s>();
         p->graph = snapshot;
         p->plan = he::plan::generate_plan(snapshot);
@@ -77,7 +78,14 @@ int he_plan_precompile(he_plan_t plan) {
         std::vector<std::future<void>> jobs;
         for (auto& step : plan->plan->steps)
             for (auto& instr : step.instrs)
-                if (!instr->compiled()) jobs.push_back(std::async(std::launch::async, [instr] { instr->precompile(); }));
+                if (!instr->compiled())
+                    jobs.push_back(std::async(std::launch::async, [instr] {
+                        try {
+                            instr->precompile();
+                        } catch (const he::Error& e) {
+                            he::fail(e.code, std::string(e.what()) + " (instruction " + instr->describe() + ")");
+                        }
+                    }));
         for (auto& j : jobs) j.get();
     });
 }
@@ -129,6 +137,7 @@ int he_backend_set_option(int option, int64_t value) {
         switch (option) {
             case HE_OPT_FUSE_MATMUL_EPILOGUE: he::plan::set_fuse_matmul_epilogue(value != 0); break;
             case HE_OPT_FOLD_SWAP_INTO_REDUCE: he::plan::set_fold_swap_into_reduce(value != 0); break;
+            case HE_OPT_REMATERIALIZE: he::plan::set_rematerialize(value != 0); break;
             default: he::fail(HE_ERR_INVALID, "unknown backend option");
         }
     });

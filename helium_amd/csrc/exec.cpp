@@ -286,8 +286,12 @@ std::shared_ptr<const Prepared> prepare(const ir::OpGraph& graph_in) {
     auto pr = std::make_shared<Prepared>();
     auto graph = std::make_shared<ir::OpGraph>(graph_in);
     graph->optimize();
-    pr->graph = graph;
-    pr->plan = plan::generate_cached_plan(graph);
+    pr->graph = plan::graph_for_execution(graph);
+    if (pr->graph->has_origins()) {
+        for (NodeId in : pr->graph->inputs()) pr->input_of[pr->graph->origin(in)] = in;
+        for (NodeId out : pr->graph->outputs()) pr->caller_output[out] = pr->graph->origin(out);
+    }
+    pr->plan = plan::generate_cached_plan(pr->graph);
     // begin_execute (cuda.rs:98-139): compile every kernel of the plan up front, in parallel (cuda.rs:262-270)
     std::vector<std::future<void>> jobs;
     for (auto& step : pr->plan->steps)
@@ -308,9 +312,17 @@ std::map<NodeId, TensorRef> execute_graph(const ir::OpGraph& graph_in, const std
     return execute_prepared(*prepare(graph_in), inputs, stats);
 }
 
-std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std::map<NodeId, TensorRef>& inputs,
+std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std::map<NodeId, TensorRef>& caller_inputs,
                                              ExecStats* stats) {
     HostTimer ht;
+    // the ids of a rewritten graph differ from the caller's: inputs are renamed on the way in, outputs on the way out
+    std::map<NodeId, TensorRef> renamed;
+    if (!prepared.input_of.empty())
+        for (auto& kv : caller_inputs) {
+            auto it = prepared.input_of.find(kv.first);
+            if (it != prepared.input_of.end()) renamed[it->second] = kv.second;
+        }
+    const std::map<NodeId, TensorRef>& inputs = prepared.input_of.empty() ? caller_inputs : renamed;
     const std::shared_ptr<const ir::OpGraph>& graph = prepared.graph;
     const std::shared_ptr<const plan::Plan>& plan = prepared.plan;
     const std::set<NodeId>& alive = prepared.alive;
@@ -453,7 +465,7 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
         NodeId from = graph->inbound(out)[0];
         auto it = tensors.find(from);
         HE_REQUIRE(it != tensors.end(), HE_ERR_INTERNAL, "output node %u has no storage", out);
-        result[out] = it->second;
+        result[prepared.caller_output.empty() ? out : prepared.caller_output.at(out)] = it->second;
     }
     ht.lap(5);
     if (HostTimer::on()) {

@@ -105,6 +105,9 @@ struct Prepared {
     std::shared_ptr<const ir::OpGraph> graph;
     std::shared_ptr<const plan::Plan> plan;
     std::set<NodeId> alive;  // enumerate_output_tensors (cuda.rs:142-153)
+    // When the graph that runs is a rewritten form of the caller's (plan::graph_for_execution): its Input node for each
+    // of the caller's, and the caller's Output node for each of its own. Empty when the ids are the caller's.
+    std::map<NodeId, NodeId> input_of, caller_output;
 };
 std::shared_ptr<const Prepared> prepare(const ir::OpGraph& graph);
 std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std::map<NodeId, TensorRef>& inputs,

@@ -1,5 +1,6 @@
 #include "ir.h"
 
+#include <functional>
 #include <sstream>
 
 namespace he::ir {
@@ -322,6 +323,109 @@ std::string OpSubgraph::cache_key() const {
     s << "|L";
     for (NodeId n : leafs_) s << n << ',';
     return s.str();
+}
+
+}  // namespace he::ir
+
+namespace he::ir {
+
+std::shared_ptr<OpGraph> rematerialized(const OpGraph& g) {
+    const size_t cap = g.capacity();
+    // What a node's value depends on once the cheap ops in between are looked through: the tensors that exist in memory
+    // anyway (`anchors`: inputs, products, reductions, permutes - listed only when they are not small next to the node),
+    // and how many ops a recomputation takes.
+    struct Info {
+        bool cheap = false;          // an op that may be duplicated
+        bool remat = false;          // ... and is, once per use
+        int cost = 0;
+        std::vector<NodeId> anchors; // sorted, at most kMaxAnchors + 1 entries
+    };
+    constexpr int kMaxCost = 24, kMaxCopies = 32;
+    constexpr int64_t kMinElements = 1 << 16;
+    constexpr size_t kMaxAnchors = 1;
+    std::vector<Info> info(cap);
+    bool any = false;
+    for (NodeId id : g.nodes()) {
+        const Node& n = g.get(id);
+        Info& I = info[id];
+        if (n.kind != Node::Intermediate) continue;
+        switch (n.op.kind) {
+            case OpKind::UnaryPointwise:
+            case OpKind::BinaryPointwise:
+            case OpKind::ChangeDataType:
+            case OpKind::Broadcast:
+            case OpKind::Reshape:
+            case OpKind::Compare:
+            case OpKind::Select:
+            case OpKind::Constant: I.cheap = true; break;
+            default: break;
+        }
+        if (!I.cheap) continue;
+        const int64_t numel = num_elements(n.desc.shape);
+        I.cost = 1;
+        for (NodeId in : n.op.inputs) {
+            const Info& J = info[in];
+            if (J.cheap) {
+                I.cost += J.cost;
+                for (NodeId a : J.anchors) I.anchors.push_back(a);
+            } else if (num_elements(g.get(in).desc.shape) * 8 >= numel) {
+                I.anchors.push_back(in);
+            }
+        }
+        std::sort(I.anchors.begin(), I.anchors.end());
+        I.anchors.erase(std::unique(I.anchors.begin(), I.anchors.end()), I.anchors.end());
+        // a tensor that is small next to this node may still have been an anchor of an input: keep what is not small
+        std::vector<NodeId> kept;
+        for (NodeId a : I.anchors)
+            if (num_elements(g.get(a).desc.shape) * 8 >= numel) kept.push_back(a);
+        I.anchors = kept;
+        if (I.anchors.size() > kMaxAnchors + 1) I.anchors.resize(kMaxAnchors + 1);
+        I.cost = std::min(I.cost, kMaxCost + 1);
+        // (a node with one consumer is copied as well when that consumer is: its copies' inputs must not meet in one
+        // shared node, which would then have several consumers and travel through memory after all)
+        I.remat = numel >= kMinElements && I.anchors.size() <= kMaxAnchors && I.cost <= kMaxCost;
+        any = any || (I.remat && g.outbound(id).size() > 1);
+    }
+    if (!any) return nullptr;
+
+    auto out = std::make_shared<OpGraph>();
+    std::vector<NodeId> placed(cap, kNoNode);  // node of `g` -> its one node in `out` (nodes that are not duplicated)
+    std::vector<int> copies(cap, 0);
+    auto note_origin = [&](NodeId fresh, NodeId old) {
+        if (out->origin_.size() <= fresh) out->origin_.resize(fresh + 1, kNoNode);
+        out->origin_[fresh] = old;
+    };
+    // emits `id` for one consumer: duplicated nodes anew (with their duplicated inputs), every other node once
+    std::function<NodeId(NodeId)> emit = [&](NodeId id) -> NodeId {
+        const Node& n = g.get(id);
+        const bool dup = info[id].remat && copies[id] < kMaxCopies;
+        if (!dup && placed[id] != kNoNode) return placed[id];
+        NodeId fresh;
+        if (n.kind == Node::Input) {
+            fresh = out->new_input(n.desc);
+        } else {
+            Op op = n.op;
+            for (NodeId& in : op.inputs) in = emit(in);
+            fresh = out->new_op(std::move(op));
+        }
+        note_origin(fresh, id);
+        if (dup) copies[id]++;
+        else placed[id] = fresh;
+        return fresh;
+    };
+    // inputs first, in their own order: their ids then only shift by a constant count
+    for (NodeId id : g.inputs()) emit(id);
+    for (NodeId id : g.nodes()) {
+        const Node& n = g.get(id);
+        if (n.kind == Node::Output) {
+            NodeId fresh = out->new_output(emit(g.inbound(id)[0]));
+            note_origin(fresh, id);
+        } else if (n.kind == Node::Intermediate && !info[id].remat) {
+            emit(id);
+        }
+    }
+    out->optimize();
+    return out;
 }
 
 }  // namespace he::ir

@@ -108,12 +108,28 @@ public:
     static Descriptor infer(const Op& op, const OpGraph& g);
     static Shape broadcast_output_shape(const Op& op, const Shape& in);
 
+    // For a graph that `rematerialized` built: the node of the graph it was built from that a node stands for (several
+    // nodes may stand for the same one); the node itself in any other graph.
+    NodeId origin(NodeId id) const { return id < origin_.size() ? origin_[id] : id; }
+    bool has_origins() const { return !origin_.empty(); }
+
 private:
     NodeId push(Node n);
     std::vector<Node> nodes_;
     std::vector<NodeId> inputs_, outputs_;
     std::vector<std::vector<NodeId>> in_, out_;
+    std::vector<NodeId> origin_;
+    friend std::shared_ptr<OpGraph> rematerialized(const OpGraph& g);
 };
+
+// A copy of `g` in which values that are cheap to compute again are computed once per use instead of once: every
+// pointwise / shape op whose value depends on at most one tensor of its own size (the rest being broadcasts of small
+// tensors) is duplicated for each of its consumers, so that plan generation can fuse every copy into the kernel that
+// uses it and the value never travels through memory. A batch norm's forward pass is the case in point: as recorded
+// (batch_norm.rs:53-71) it leaves eight full-size intermediates for the backward pass to read - the broadcast scale,
+// the broadcast reciprocal of the deviation, x minus the mean, ... - each a few instructions away from x and four
+// per-channel vectors. Node ids are new (in dataflow order); `origin` maps them back. Returns null when nothing changes.
+std::shared_ptr<OpGraph> rematerialized(const OpGraph& g);
 
 // Subset of an OpGraph (opgraph/subgraph.rs): nodes sorted by id; `inputs` = outside producers feeding it,
 // `roots` = members with an outside input, `leafs` = members with an outside consumer.

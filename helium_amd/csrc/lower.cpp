@@ -5,6 +5,9 @@
 
 #include "tp.h"
 
+namespace he::plan {
+bool rematerialize();
+}
 namespace he::tp {
 
 namespace {
@@ -814,6 +817,11 @@ bool pointwise_supports(const ir::OpSubgraph& sg) {
                 break;
             case ir::OpKind::Reduce: {
                 if (!sg.is_leaf(node)) return false;
+                // (not in the reference's text, which asks for a leaf only: a reduction with one consumer inside and
+                // one outside is a leaf, but the inside one cannot read a value that only exists when every thread
+                // has finished - that merge is refused as well)
+                for (ir::NodeId c : g.outbound(node))
+                    if (sg.contains(c)) return false;
                 const Shape& s = g.get(op.inputs[0]).desc.shape;
                 if (!have_red) {
                     have_red = true;
@@ -824,7 +832,13 @@ bool pointwise_supports(const ir::OpSubgraph& sg) {
                 }
                 break;
             }
-            default: return false;  // includes Constant, exactly as the reference's `_ => return false`
+            case ir::OpKind::Constant:
+                // The reference's `_ => return false` includes Constant: a constant is always a kernel of its own that
+                // fills a tensor (the zeros and ones of a relu's gradient mask, each as large as the activation). With
+                // rematerialisation on it is an immediate of the kernel that uses it.
+                if (!plan::rematerialize()) return false;
+                continue;
+            default: return false;
         }
     }
     return true;

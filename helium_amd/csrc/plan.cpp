@@ -46,6 +46,7 @@ bool enumerate_swaps(const ir::OpSubgraph& sg, std::vector<std::pair<int, int>>*
 namespace {
 std::atomic<bool> g_fuse_matmul_epilogue{true};
 std::atomic<bool> g_fold_swap_into_reduce{true};
+std::atomic<bool> g_rematerialize{true};
 
 // True when every value computed from `node` inside the graph ends in a Reduce, through pointwise ops only: nothing
 // then needs the transposed tensor in memory.
@@ -74,9 +75,11 @@ void set_fuse_matmul_epilogue(bool on) { g_fuse_matmul_epilogue.store(on); }
 bool fuse_matmul_epilogue() { return g_fuse_matmul_epilogue.load(); }
 unsigned option_mask() {
     // the hash of the tuning overrides (0 unless tuning is on) rides along: plans keep their kernels
-    return (fuse_matmul_epilogue() ? 1u : 0u) | (g_fold_swap_into_reduce.load() ? 2u : 0u) | (tuning::hash() << 2);
+    return (fuse_matmul_epilogue() ? 1u : 0u) | (g_fold_swap_into_reduce.load() ? 2u : 0u) | (g_rematerialize.load() ? 4u : 0u) | (tuning::hash() << 3);
 }
 void set_fold_swap_into_reduce(bool on) { g_fold_swap_into_reduce.store(on); }
+void set_rematerialize(bool on) { g_rematerialize.store(on); }
+bool rematerialize() { return g_rematerialize.load(); }
 bool fold_swap_into_reduce() { return g_fold_swap_into_reduce.load(); }
 
 bool Instr::can_fuse_with(const Instr& next) const {
@@ -216,7 +219,8 @@ void Instr::execute(const std::function<void*(NodeId)>& storage, hipStream_t str
 std::string Instr::describe() const {
     std::ostringstream s;
     s << (kind_ == InstrKind::Gemm ? "gemm" : kind_ == InstrKind::Pointwise ? "pointwise" : "permute") << "{";
-    for (size_t i = 0; i < sg_.nodes().size(); i++) s << (i ? "," : "") << sg_.nodes()[i];
+    // (a rematerialised graph's nodes are named by the nodes they stand for)
+    for (size_t i = 0; i < sg_.nodes().size(); i++) s << (i ? "," : "") << sg_.graph()->origin(sg_.nodes()[i]);
     s << "}";
     return s.str();
 }
@@ -442,14 +446,38 @@ std::shared_ptr<const Plan> generate_plan(const std::shared_ptr<const ir::OpGrap
 
 std::string Plan::describe() const {
     std::ostringstream s;
+    const ir::OpGraph* g = nullptr;
+    for (auto& st : steps)
+        for (auto& instr : st.instrs) g = instr->subgraph().graph().get();
     for (size_t i = 0; i < steps.size(); i++) {
         s << "step " << i << ":";
         for (auto& instr : steps[i].instrs) s << " " << instr->describe();
         s << " | release";
-        for (NodeId t : steps[i].tensors_to_release) s << " " << t;
+        for (NodeId t : steps[i].tensors_to_release) s << " " << (g ? g->origin(t) : t);
         s << "\n";
     }
     return s.str();
+}
+
+int64_t plan_traffic_bytes(const Plan& plan) {
+    int64_t bytes = 0;
+    for (auto& st : plan.steps)
+        for (auto& instr : st.instrs) {
+            const ir::OpGraph& g = *instr->subgraph().graph();
+            for (NodeId n : instr->inputs()) bytes += (int64_t)storage_bytes(g.get(n).desc.dtype, (size_t)ir::num_elements(g.get(n).desc.shape));
+            for (NodeId n : instr->outputs()) bytes += (int64_t)storage_bytes(g.get(n).desc.dtype, (size_t)ir::num_elements(g.get(n).desc.shape));
+        }
+    return bytes;
+}
+
+std::shared_ptr<const ir::OpGraph> graph_for_execution(const std::shared_ptr<const ir::OpGraph>& g) {
+    if (!rematerialize()) return g;
+    std::shared_ptr<const ir::OpGraph> other = ir::rematerialized(*g);
+    if (!other) return g;
+    // Copies that the fusion rules keep out of their consumers' kernels would each be written out: the rewritten graph is
+    // taken only when its plan moves fewer bytes.
+    const int64_t before = plan_traffic_bytes(*generate_cached_plan(g)), after = plan_traffic_bytes(*generate_cached_plan(other));
+    return after < before ? other : g;
 }
 
 // ---------------------------------------------------------------------------------------------------------

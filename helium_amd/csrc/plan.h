@@ -75,6 +75,16 @@ unsigned option_mask();  // the options above as bits: what a generated plan dep
 void set_fold_swap_into_reduce(bool on);
 bool fold_swap_into_reduce();
 
+// Whether values that are cheap to compute again are computed per use instead of travelling through memory
+// (ir::rematerialized; on by default, off plans the graph as recorded, like the reference).
+void set_rematerialize(bool on);
+bool rematerialize();
+// Bytes the plan's kernels read and write: the sizes of every instruction's inputs and outputs.
+int64_t plan_traffic_bytes(const Plan& plan);
+// The graph the backend plans and runs for `g` (already pruned): `g` itself, or its rematerialised form when that
+// form's plan moves fewer bytes. Input and Output nodes of the result map back through OpGraph::origin.
+std::shared_ptr<const ir::OpGraph> graph_for_execution(const std::shared_ptr<const ir::OpGraph>& g);
+
 // generate_plan (plan_generation.rs:22-26).
 std::shared_ptr<const Plan> generate_plan(const std::shared_ptr<const ir::OpGraph>& g);
 // generate_cached_plan (:16-19): LRU of 256 plans keyed by the graph's structure.

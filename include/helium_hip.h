@@ -359,8 +359,14 @@ int he_fgraph_subdivide(he_fgraph_t graph, uint64_t* nodes, int32_t* portions, i
  * helium/src/cuda/instr/cudnn_graph.rs:319-321, where a matmul or convolution instruction never fuses.
  * HE_OPT_FOLD_SWAP_INTO_REDUCE (default 1): a SwapDims above the 1M-element threshold of cuda.rs:38-41 whose values
  * all end in Reduce ops (BatchNorm2d statistics, column sums) stays in the pointwise instruction, which then folds the
- * leading dims of the untransposed tensor in one pass; 0 makes it a permute instruction as the reference does. */
-enum { HE_OPT_FUSE_MATMUL_EPILOGUE = 0, HE_OPT_FOLD_SWAP_INTO_REDUCE = 1 };
+ * leading dims of the untransposed tensor in one pass; 0 makes it a permute instruction as the reference does.
+ * HE_OPT_REMATERIALIZE (default 1): pointwise / shape ops whose value depends on at most one tensor of their own size
+ * (the rest being broadcasts of small tensors) are planned once per consumer, so that every copy fuses into the kernel
+ * that uses it and the value never travels through memory - a batch norm's forward pass as the reference records it
+ * (modules/batch_norm.rs:53-71) otherwise leaves eight full-size intermediates for the backward pass. The rewritten
+ * graph is used only when its plan moves fewer bytes; he_plan_describe names copies by the nodes they stand for. 0 plans
+ * the graph as recorded, like plan_generation.rs. */
+enum { HE_OPT_FUSE_MATMUL_EPILOGUE = 0, HE_OPT_FOLD_SWAP_INTO_REDUCE = 1, HE_OPT_REMATERIALIZE = 2 };
 int he_backend_set_option(int option, int64_t value);
 
 /* Counters of the last he_execute_graph on this thread: [0] steps run, [1] instructions, [2] streams used,

@@ -361,15 +361,34 @@ def kernel_outputs(nodes, inputs, leaf_ids):
 def plan_outputs(nodes, inputs, plan_steps):
     """Storage-domain value of every Output node when the graph runs as the kernels of `plan_steps`
     ([(instrs, released)], instrs = [(kind, [node ids])]): a value is rounded to its storage dtype exactly where it
-    leaves the kernel that computes it. Returns {output node id: storage array}."""
+    leaves the kernel that computes it, and is kept in f32 inside a kernel. The kernels are evaluated one by one, in
+    plan order, each on its own members: a node may be a member of several instructions (a value the plan computes
+    again in every kernel that uses it instead of passing it through memory), and every kernel then works on its own,
+    unrounded copy. Returns {output node id: storage array}."""
+    by_id = {n["id"]: n for n in nodes}
     consumers = {}
     for n in nodes:
         for p in (n.get("inputs") or ([n["from"]] if n["node"] == "output" else [])):
             consumers.setdefault(p, []).append(n["id"])
-    boundary = set()
+    desc, stored = {}, {}
+    for n in nodes:  # descriptors of everything; values of the inputs
+        i = n["id"]
+        if n["node"] == "input":
+            desc[i] = (list(n["shape"]), n["dtype"])
+            stored[i] = nm.from_storage(inputs[i], n["dtype"], n["shape"])
+        elif n["node"] == "output":
+            desc[i] = desc[n["from"]]
+        else:
+            desc[i] = infer(n, desc)
     for instrs, _ in plan_steps:
         for _, members in instrs:
             inside = set(members)
-            boundary |= {m for m in members if any(c not in inside for c in consumers.get(m, []))}
-    val, desc = evaluate(nodes, inputs, materialize=boundary)
-    return {n["id"]: nm.to_storage(val[n["id"]], desc[n["id"]][1]) for n in nodes if n["node"] == "output"}
+            local = dict(stored)  # what memory holds, overlaid by this kernel's own values
+            for m in sorted(inside):
+                local[m] = _eval_op(by_id[m], desc, local)
+                assert list(local[m].shape) == list(desc[m][0]), (by_id[m], local[m].shape)
+            for m in inside:
+                if any(c not in inside for c in consumers.get(m, [])):
+                    shape, dtype = desc[m]
+                    stored[m] = nm.from_storage(nm.to_storage(local[m], dtype), dtype, shape)
+    return {n["id"]: nm.to_storage(stored[n["from"]], desc[n["id"]][1]) for n in nodes if n["node"] == "output"}

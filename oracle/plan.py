@@ -103,6 +103,10 @@ def supports_subgraph(instr):
         elif op == "reduce":
             if node not in instr.outputs:
                 return False
+            # (not in the reference's text, which asks for a leaf only: a reduction that another member reads cannot
+            # be computed by that member's threads, so such a merge is refused as well)
+            if any(o in instr.nodes for o in g.outbound[node]):
+                return False
             key = (list(g.desc[n["inputs"][0]][0]), n["depth"])
             if reduction_shape is None:
                 reduction_shape = key

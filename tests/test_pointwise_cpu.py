@@ -29,10 +29,17 @@ def test_generated_kernel_on_cpu_matches_oracle(case, monkeypatch):
     for name, value in case.env.items():
         monkeypatch.setenv(name, value)
     # what the reference's fusion rule admits (pointwise.rs:121-186); the generator itself accepts more
-    admitted = ha.kernels.pointwise_supports(case.g, case.nodes)
+    from helium_amd.backend import OPT_REMATERIALIZE, set_option
+
     has_constant = any(n.get("op") == "constant" for n in case.g.nodes if n["id"] in case.nodes)
-    # a Constant is an instruction of its own that the rule never merges (pointwise.rs:181)
-    assert admitted == (case.admitted_by_fusion_rule and not has_constant), case.name
+    set_option(OPT_REMATERIALIZE, 0)
+    try:
+        # a Constant is an instruction of its own that the reference's rule never merges (pointwise.rs:181)
+        assert ha.kernels.pointwise_supports(case.g, case.nodes) == (case.admitted_by_fusion_rule and not has_constant), case.name
+    finally:
+        set_option(OPT_REMATERIALIZE, 1)
+    # ... and an immediate of the kernel that uses it when values may be computed where they are used
+    assert ha.kernels.pointwise_supports(case.g, case.nodes) == case.admitted_by_fusion_rule, case.name
     kernel = ha.TileKernel.pointwise(case.g, case.nodes)
     assert [a["node"] for a in kernel.args if a["is_output"]] == sorted(case.leaves)
     want = oracle_ir.kernel_outputs(case.g.nodes, case.inputs, case.leaves)
