@@ -370,6 +370,12 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
     }
     EventRef done = pool.take_event();
     bool done_recorded = false;
+    struct InstrTime {
+        double us;
+        int64_t bytes;
+        const plan::Instr* instr;
+    };
+    std::vector<InstrTime> instr_times;
     // Whatever happens below, the scope must end, and only after the work already queued: a failing instruction leaves
     // earlier launches running on up to four streams. On failure stream 0 is ordered after every stream this execution
     // used, the end event is recorded there as usual, and the error goes on to the caller.
@@ -415,11 +421,28 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
             }
             ht.lap(3);
             if (&instr == closing) set_pending_stop_event(done->e);
+            // HELIUM_HIP_INSTR_TIMING=<n>: every instruction is timed on its own (the device is drained before and after
+            // it), and the n slowest of the execution are listed with the bytes they read and write. A debugging aid:
+            // the execution is serialised while it is on.
+            static const int instr_timing = getenv("HELIUM_HIP_INSTR_TIMING") ? atoi(getenv("HELIUM_HIP_INSTR_TIMING")) : 0;
+            std::chrono::steady_clock::time_point t_instr;
+            if (instr_timing) {
+                HE_HIP(hipDeviceSynchronize());
+                t_instr = std::chrono::steady_clock::now();
+            }
             try {
                 instr.execute([&](NodeId n) -> void* { return tensors.at(n)->ptr; }, stream);
             } catch (...) {
                 (void)take_pending_stop_event();
                 throw;
+            }
+            if (instr_timing) {
+                HE_HIP(hipDeviceSynchronize());
+                const double us = std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t_instr).count();
+                int64_t bytes = 0;
+                for (NodeId n : instr.inputs()) bytes += (int64_t)tensors.at(n)->bytes;
+                for (NodeId n : instr.outputs()) bytes += (int64_t)tensors.at(n)->bytes;
+                instr_times.push_back({us, bytes, &instr});
             }
             // taken by the instruction's last launch, or still pending (a launch too large for that entry point)
             if (&instr == closing) done_recorded = take_pending_stop_event() == nullptr;
@@ -460,6 +483,21 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
     local.streams_used = (int)used_streams.size();
     if (stats) *stats = local;
 
+    if (!instr_times.empty()) {
+        static std::atomic<int> reports{0};
+        if (reports.fetch_add(1) == 1) {  // the second execution: kernels are compiled and loaded by then
+            std::sort(instr_times.begin(), instr_times.end(), [](const InstrTime& a, const InstrTime& b) { return a.us > b.us; });
+            double total = 0;
+            for (auto& t : instr_times) total += t.us;
+            fprintf(stderr, "[instr timing] %zu instructions, %.1f us in all; slowest:\n", instr_times.size(), total);
+            const int top = atoi(getenv("HELIUM_HIP_INSTR_TIMING"));
+            for (int i = 0; i < top && i < (int)instr_times.size(); i++) {
+                const std::string d = instr_times[i].instr->describe();
+                fprintf(stderr, "  %8.1f us %8.1f MB %6.2f TB/s  %s\n", instr_times[i].us, instr_times[i].bytes / 1e6,
+                        instr_times[i].bytes / instr_times[i].us / 1e6, d.substr(0, 200).c_str());
+            }
+        }
+    }
     std::map<NodeId, TensorRef> result;
     for (NodeId out : graph->outputs()) {
         NodeId from = graph->inbound(out)[0];

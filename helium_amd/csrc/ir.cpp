@@ -1,7 +1,9 @@
 #include "ir.h"
 
 #include <functional>
+#include <set>
 #include <sstream>
+#include <unordered_map>
 
 namespace he::ir {
 
@@ -329,14 +331,48 @@ std::string OpSubgraph::cache_key() const {
 
 namespace he::ir {
 
-std::shared_ptr<OpGraph> rematerialized(const OpGraph& g) {
+std::shared_ptr<OpGraph> rematerialized(const OpGraph& g, const std::set<NodeId>& keep_single) {
     const size_t cap = g.capacity();
-    // What a node's value depends on once the cheap ops in between are looked through: the tensors that exist in memory
-    // anyway (`anchors`: inputs, products, reductions, permutes - listed only when they are not small next to the node),
-    // and how many ops a recomputation takes.
+    // 1. Ops that compute the same thing are one op. The reference's tape records a forward op again when the backward
+    //    pass needs its value (tensor/tape.rs:93-158 recomputes from the last checkpoint), so every batch norm's
+    //    normalisation chain is in the graph twice.
+    std::vector<NodeId> canon(cap, kNoNode);
+    {
+        std::unordered_map<uint64_t, std::vector<NodeId>> seen;
+        for (NodeId id : g.nodes()) {
+            const Node& n = g.get(id);
+            canon[id] = id;
+            if (n.kind != Node::Intermediate) continue;
+            Op op = n.op;
+            for (NodeId& in : op.inputs) in = canon[in];
+            auto& bucket = seen[op.hash()];
+            for (NodeId other : bucket) {
+                Op theirs = g.get(other).op;
+                for (NodeId& in : theirs.inputs) in = canon[in];
+                if (theirs == op && g.get(other).desc == n.desc) {
+                    canon[id] = other;
+                    break;
+                }
+            }
+            if (canon[id] == id) bucket.push_back(id);
+        }
+    }
+    std::vector<std::vector<NodeId>> users(cap);  // consumers of a canonical node, themselves canonical
+    bool merged_any = false;
+    for (NodeId id : g.nodes()) {
+        if (canon[id] != id) {
+            merged_any = true;
+            continue;
+        }
+        for (NodeId in : g.inbound(id)) users[canon[in]].push_back(id);
+    }
+
+    // 2. What a node's value depends on once the cheap ops in between are looked through: the tensors that exist in
+    //    memory anyway (`anchors`: inputs, products, reductions, permutes - listed only when they are not small next to
+    //    the node), and how many ops a recomputation takes.
     struct Info {
         bool cheap = false;          // an op that may be duplicated
-        bool remat = false;          // ... and is, once per use
+        bool remat = false;          // ... and is, once per use by a kernel that can take it in
         int cost = 0;
         std::vector<NodeId> anchors; // sorted, at most kMaxAnchors + 1 entries
     };
@@ -346,6 +382,7 @@ std::shared_ptr<OpGraph> rematerialized(const OpGraph& g) {
     std::vector<Info> info(cap);
     bool any = false;
     for (NodeId id : g.nodes()) {
+        if (canon[id] != id) continue;
         const Node& n = g.get(id);
         Info& I = info[id];
         if (n.kind != Node::Intermediate) continue;
@@ -363,7 +400,8 @@ std::shared_ptr<OpGraph> rematerialized(const OpGraph& g) {
         if (!I.cheap) continue;
         const int64_t numel = num_elements(n.desc.shape);
         I.cost = 1;
-        for (NodeId in : n.op.inputs) {
+        for (NodeId raw : n.op.inputs) {
+            const NodeId in = canon[raw];
             const Info& J = info[in];
             if (J.cheap) {
                 I.cost += J.cost;
@@ -383,29 +421,43 @@ std::shared_ptr<OpGraph> rematerialized(const OpGraph& g) {
         I.cost = std::min(I.cost, kMaxCost + 1);
         // (a node with one consumer is copied as well when that consumer is: its copies' inputs must not meet in one
         // shared node, which would then have several consumers and travel through memory after all)
-        I.remat = numel >= kMinElements && I.anchors.size() <= kMaxAnchors && I.cost <= kMaxCost;
-        any = any || (I.remat && g.outbound(id).size() > 1);
+        I.remat = numel >= kMinElements && I.anchors.size() <= kMaxAnchors && I.cost <= kMaxCost && !keep_single.count(id);
+        any = any || (I.remat && users[id].size() > 1);
     }
-    if (!any) return nullptr;
+    if (!any && !merged_any) return nullptr;
 
     auto out = std::make_shared<OpGraph>();
-    std::vector<NodeId> placed(cap, kNoNode);  // node of `g` -> its one node in `out` (nodes that are not duplicated)
+    std::vector<NodeId> placed(cap, kNoNode);  // node of `g` -> its one node in `out` (what is not duplicated)
     std::vector<int> copies(cap, 0);
     auto note_origin = [&](NodeId fresh, NodeId old) {
         if (out->origin_.size() <= fresh) out->origin_.resize(fresh + 1, kNoNode);
         out->origin_[fresh] = old;
     };
-    // emits `id` for one consumer: duplicated nodes anew (with their duplicated inputs), every other node once
-    std::function<NodeId(NodeId)> emit = [&](NodeId id) -> NodeId {
+    // A kernel that cannot take a producer in (a product reads operands from memory, so does a permute, and an Output is
+    // memory) reads the one shared copy; every other consumer gets a copy of its own.
+    auto takes_producers_in = [&](const Node& consumer) {
+        if (consumer.kind != Node::Intermediate) return false;
+        switch (consumer.op.kind) {
+            case OpKind::Matmul:
+            case OpKind::Conv:
+            case OpKind::ConvBackwardData:
+            case OpKind::ConvBackwardFilter: return false;
+            case OpKind::SwapDims: return num_elements(consumer.desc.shape) <= 1000000;
+            default: return true;
+        }
+    };
+    std::function<NodeId(NodeId, bool)> emit = [&](NodeId raw, bool for_fusing_consumer) -> NodeId {
+        const NodeId id = canon[raw];
         const Node& n = g.get(id);
-        const bool dup = info[id].remat && copies[id] < kMaxCopies;
+        const bool dup = info[id].remat && for_fusing_consumer && copies[id] < kMaxCopies;
         if (!dup && placed[id] != kNoNode) return placed[id];
         NodeId fresh;
         if (n.kind == Node::Input) {
             fresh = out->new_input(n.desc);
         } else {
             Op op = n.op;
-            for (NodeId& in : op.inputs) in = emit(in);
+            const bool fusing = takes_producers_in(n);
+            for (NodeId& in : op.inputs) in = emit(in, fusing);
             fresh = out->new_op(std::move(op));
         }
         note_origin(fresh, id);
@@ -413,15 +465,15 @@ std::shared_ptr<OpGraph> rematerialized(const OpGraph& g) {
         else placed[id] = fresh;
         return fresh;
     };
-    // inputs first, in their own order: their ids then only shift by a constant count
-    for (NodeId id : g.inputs()) emit(id);
+    // inputs first, in their own order
+    for (NodeId id : g.inputs()) emit(id, false);
     for (NodeId id : g.nodes()) {
         const Node& n = g.get(id);
         if (n.kind == Node::Output) {
-            NodeId fresh = out->new_output(emit(g.inbound(id)[0]));
+            NodeId fresh = out->new_output(emit(g.inbound(id)[0], false));
             note_origin(fresh, id);
-        } else if (n.kind == Node::Intermediate && !info[id].remat) {
-            emit(id);
+        } else if (n.kind == Node::Intermediate && canon[id] == id && !info[id].remat) {
+            emit(id, false);
         }
     }
     out->optimize();

@@ -5,6 +5,7 @@
 #include <algorithm>
 #include <cstdint>
 #include <memory>
+#include <set>
 #include <string>
 #include <vector>
 
@@ -119,7 +120,7 @@ private:
     std::vector<NodeId> inputs_, outputs_;
     std::vector<std::vector<NodeId>> in_, out_;
     std::vector<NodeId> origin_;
-    friend std::shared_ptr<OpGraph> rematerialized(const OpGraph& g);
+    friend std::shared_ptr<OpGraph> rematerialized(const OpGraph& g, const std::set<NodeId>& keep_single);
 };
 
 // A copy of `g` in which values that are cheap to compute again are computed once per use instead of once: every
@@ -128,8 +129,11 @@ private:
 // uses it and the value never travels through memory. A batch norm's forward pass is the case in point: as recorded
 // (batch_norm.rs:53-71) it leaves eight full-size intermediates for the backward pass to read - the broadcast scale,
 // the broadcast reciprocal of the deviation, x minus the mean, ... - each a few instructions away from x and four
-// per-channel vectors. Node ids are new (in dataflow order); `origin` maps them back. Returns null when nothing changes.
-std::shared_ptr<OpGraph> rematerialized(const OpGraph& g);
+// per-channel vectors. Ops that compute the same thing are merged first (the reference's tape records a forward op again
+// when the backward pass needs its value). A consumer that reads its operands from memory whatever happens (a product, a
+// large permute, an Output) shares one copy. `keep_single`: nodes of `g` that are not to be duplicated. Node ids are new
+// (in dataflow order); `origin` maps them back to `g`. Returns null when nothing changes.
+std::shared_ptr<OpGraph> rematerialized(const OpGraph& g, const std::set<NodeId>& keep_single = {});
 
 // Subset of an OpGraph (opgraph/subgraph.rs): nodes sorted by id; `inputs` = outside producers feeding it,
 // `roots` = members with an outside input, `leafs` = members with an outside consumer.

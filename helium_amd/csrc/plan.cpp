@@ -474,8 +474,25 @@ std::shared_ptr<const ir::OpGraph> graph_for_execution(const std::shared_ptr<con
     if (!rematerialize()) return g;
     std::shared_ptr<const ir::OpGraph> other = ir::rematerialized(*g);
     if (!other) return g;
-    // Copies that the fusion rules keep out of their consumers' kernels would each be written out: the rewritten graph is
-    // taken only when its plan moves fewer bytes.
+    // Copies that the fusion rules keep out of their consumers' kernels are written out, each on its own: where one
+    // kernel ends up with several copies of a value among its outputs, that value goes back to being computed once, and
+    // the graph is planned again.
+    std::set<ir::NodeId> keep_single;
+    for (int round = 0; round < 3; round++) {
+        const size_t known = keep_single.size();
+        if (getenv("HELIUM_HIP_PLAN_DEBUG")) fprintf(stderr, "[plan] round %d: %zu -> %zu nodes, %zu kept single\n", round, g->num_nodes(), other->num_nodes(), known);
+        const auto plan = generate_plan(other);
+        for (auto& st : plan->steps)
+            for (auto& instr : st.instrs) {
+                std::set<ir::NodeId> origins;
+                for (ir::NodeId leaf : instr->outputs())
+                    if (!origins.insert(other->origin(leaf)).second) keep_single.insert(other->origin(leaf));
+            }
+        if (keep_single.size() == known) break;
+        other = ir::rematerialized(*g, keep_single);
+        if (!other) return g;
+    }
+    // ... and the rewritten graph is taken only when its plan moves fewer bytes.
     const int64_t before = plan_traffic_bytes(*generate_cached_plan(g)), after = plan_traffic_bytes(*generate_cached_plan(other));
     return after < before ? other : g;
 }

@@ -366,11 +366,32 @@ def plan_outputs(nodes, inputs, plan_steps):
     again in every kernel that uses it instead of passing it through memory), and every kernel then works on its own,
     unrounded copy. Returns {output node id: storage array}."""
     by_id = {n["id"]: n for n in nodes}
+    # ops that compute the same thing may be one op of the plan (it then names the first of them): every id is read
+    # through `canon`
+    canon, seen = {}, {}
+    for n in nodes:
+        i = n["id"]
+        canon[i] = i
+        if n["node"] != "op":
+            continue
+        key = (tuple(canon[p] for p in n["inputs"]), repr(sorted((k, repr(v)) for k, v in n.items() if k not in ("id", "inputs"))))
+        canon[i] = seen.setdefault(key, i)
+
+    class _Through(dict):
+        def __getitem__(self, k):
+            return dict.__getitem__(self, canon[k])
+
+        def __contains__(self, k):
+            return dict.__contains__(self, canon[k])
+
+        def __setitem__(self, k, v):
+            dict.__setitem__(self, canon[k], v)
+
     consumers = {}
     for n in nodes:
         for p in (n.get("inputs") or ([n["from"]] if n["node"] == "output" else [])):
-            consumers.setdefault(p, []).append(n["id"])
-    desc, stored = {}, {}
+            consumers.setdefault(canon[p], []).append(canon[n["id"]])
+    desc, stored = {}, _Through()
     for n in nodes:  # descriptors of everything; values of the inputs
         i = n["id"]
         if n["node"] == "input":
@@ -383,12 +404,14 @@ def plan_outputs(nodes, inputs, plan_steps):
     for instrs, _ in plan_steps:
         for _, members in instrs:
             inside = set(members)
-            local = dict(stored)  # what memory holds, overlaid by this kernel's own values
+            local = _Through(stored)  # what memory holds, overlaid by this kernel's own values
             for m in sorted(inside):
                 local[m] = _eval_op(by_id[m], desc, local)
                 assert list(local[m].shape) == list(desc[m][0]), (by_id[m], local[m].shape)
+            inside_canon = {canon[m] for m in inside}
             for m in inside:
-                if any(c not in inside for c in consumers.get(m, [])):
+                if any(c not in inside_canon for c in consumers.get(canon[m], [])):
                     shape, dtype = desc[m]
                     stored[m] = nm.from_storage(nm.to_storage(local[m], dtype), dtype, shape)
     return {n["id"]: nm.to_storage(stored[n["from"]], desc[n["id"]][1]) for n in nodes if n["node"] == "output"}
+
