@@ -776,11 +776,31 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         // narrow as N, so that no matrix-core work is spent on columns that do not exist; eight waves of 64x32
         // (measured on [200704 x 576] x [576 x 64]: 71 us with 128x128 tiles, 44 us with 256x64).
         const bool skinny = !f32 && pr.N <= 64 && pr.N > 32 && pr.M >= 256 * 256;
-        if (skinny) {
+        // Half as wide again (a convolution into 32 channels, the data gradient of one out of 32): four waves of 64x32.
+        // Measured at batch 128 on the 112x112x32 layer of the resnet-train model: data gradient of the 3x3 stride-2
+        // layer 469 -> 131 us, of the 1x1 shortcut 121 -> 34 us. When the operand is gathered element by element (a
+        // 3-channel image) the gather is what takes the time, and twice the threads per row of pixels gather faster
+        // than the unused half of a 256x64 tile costs (7x7 stem: 885 us with 128x128 tiles, 408 with 256x32, 276 with 256x64).
+        const bool narrow = !f32 && pr.N <= 32 && pr.N > 16 && pr.M >= 256 * 256;
+        const bool gathered_by_element = pr.conv_a.on && pr.conv_a.C % epc != 0;
+        if (skinny || (narrow && gathered_by_element)) {
             t.bm = 256;
             t.bn = 64;
             t.wm = 4;
             t.wn = 2;
+        } else if (narrow) {
+            t.bm = 256;
+            t.bn = 32;
+            t.wm = 4;
+            t.wn = 1;
+        } else if (!f32 && pr.M <= 32 && pr.M > 16 && pr.N >= 128) {
+            // few output rows (a filter gradient with 32 output channels): four waves side by side
+            // (the 7x7x3 stem's: 1095 us with 128x128 tiles, 668 us)
+            t.bm = 32;
+            t.bn = 128;
+            t.wm = 1;
+            t.wn = 4;
+            small = true;
         } else if (!f32 && pr.M <= 64 && pr.M > 32 && pr.N >= 128) {
             // few output rows (a filter gradient with 64 output channels): tiles as low as M
             t.bm = 64;

@@ -272,6 +272,9 @@ CONV_CASES = [
     ("odd_channels_five_3x3", (2, 7, 6, 5), 16, (3, 3), "bf16", (1, 1), (1, 1), "same", "64,64,64,2,2"),
     ("odd_channels_three_f32_full", (1, 6, 5, 3), 8, (3, 3), "f32", (1, 1), (2, 1), "full", "64,64,32,2,2"),
     ("odd_channels_three_5x5_stride3", (1, 11, 13, 3), 8, (5, 5), "f16", (3, 3), (1, 1), "same", "64,64,64,2,2"),
+    # the tiles of products with 32 columns: four waves of 64x32 (direct loads), 256x64 for the element-wise gather
+    ("thirty_two_channels_out_narrow_tile", (2, 12, 12, 32), 32, (3, 3), "bf16", (2, 2), (1, 1), "same", "256,32,64,4,1"),
+    ("three_channel_stem_wide_gather_tile", (2, 16, 16, 3), 32, (7, 7), "bf16", (2, 2), (1, 1), "same", "256,64,64,4,2"),
 ]
 
 
@@ -298,6 +301,8 @@ BWD_DATA_CASES = [
     ("3x3_stride2_bf16", (1, 12, 12, 8), 32, (3, 3), "bf16", (2, 2), (1, 1), "same", "64,64,64,2,2"),
     ("1x1_stride2_shortcut", (2, 8, 8, 32), 64, (1, 1), "bf16", (2, 2), (1, 1), "same", "128,128,64,2,2"),
     ("direct_loads_both_operands", (1, 16, 16, 128), 64, (3, 3), "bf16", (1, 1), (1, 1), "same", "128,128,64,2,2"),
+    ("thirty_two_channels_in_narrow_tile_stride2", (2, 12, 12, 32), 64, (3, 3), "bf16", (2, 2), (1, 1), "same", "256,32,64,4,1"),
+    ("thirty_two_channels_in_narrow_tile_1x1", (2, 12, 12, 32), 64, (1, 1), "bf16", (2, 2), (1, 1), "same", "256,32,64,4,1"),
     ("valid_and_dilated_f32", (1, 9, 9, 4), 8, (3, 3), "f32", (1, 1), (2, 1), "valid", "64,64,32,2,2"),
     ("hoisted_pixel_terms_stride2", (2, 10, 9, 16), 64, (3, 3), "bf16", (2, 2), (1, 1), "same", "128,128,64,2,2"),
     ("flow_gathered_element_by_element", (1, 9, 8, 16), 12, (3, 3), "bf16", (2, 1), (1, 1), "same", "64,64,64,2,2"),
@@ -343,6 +348,8 @@ BWD_FILTER_CASES = [
     ("valid_and_dilated_f32", (2, 9, 9, 4), 8, (3, 3), "f32", (1, 1), (2, 1), "valid", "64,64,32,2,2"),
     # channel counts that do not fill a 16-byte chunk: the image operand is gathered element by element
     ("three_channel_stem_7x7_stride2", (2, 16, 16, 3), 32, (7, 7), "bf16", (2, 2), (1, 1), "same", "64,128,64,2,2"),
+    ("three_channel_stem_thirty_two_rows_tile", (2, 16, 16, 3), 32, (7, 7), "bf16", (2, 2), (1, 1), "same", "32,128,64,1,4"),
+    ("thirty_two_rows_tile_direct_loads", (2, 12, 12, 16), 32, (3, 3), "bf16", (1, 1), (1, 1), "same", "32,128,64,1,4"),
     ("five_channels_3x3_f16", (1, 7, 9, 5), 8, (3, 3), "f16", (1, 1), (1, 1), "same", "64,64,64,2,2"),
     ("three_channels_f32_full", (1, 6, 5, 3), 8, (3, 3), "f32", (1, 1), (1, 2), "full", "64,64,32,2,2"),
 ]
