@@ -74,6 +74,25 @@ def prebuild_kernels(verbose=True):
     g.new_output(new_avg)
     Plan(g).precompile()
     n += 1
+    # C5a and C4m the way the fusion search plans them
+    from . import fusion_search as fs
+
+    g, outs = configs.c4_graph(4096, mainloop=True, full_size_outputs=True)
+    for node in ("loss", "db8", "db6"):
+        g.consumer(outs[node], "f32")
+    for g in (g, configs.c5a_graph(4096)[0]):
+        fs.FusionPlan(g, fs.MIN_MI355X_COST).precompile()
+        n += 1
+    # the whole training step at the benchmark's two sizes and at the size the parity tests run it
+    from . import resnet
+
+    for kwargs in (dict(batch=128, image_size=224), dict(batch=64, image_size=256),
+                   dict(batch=8, image_size=64, width=8, num_classes=16, dtype="f32"),
+                   dict(batch=8, image_size=64, width=8, num_classes=16, dtype="bf16")):
+        g = resnet.record_training_step(**kwargs)["graph"].g
+        g.optimize()
+        Plan(g).precompile()
+        n += 1
     if verbose:
         print(f"prebuilt {n + 1} kernels in {time.time() - t0:.1f}s")
     return n + 1
