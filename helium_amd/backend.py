@@ -17,6 +17,7 @@ _ffi._sig("he_tensor_free", C.c_void_p)
 _ffi._sig("he_plan_generate", C.c_void_p, C.POINTER(C.c_void_p))
 _ffi._sig("he_plan_num_steps", C.c_void_p, C.POINTER(C.c_int))
 _ffi._sig("he_plan_describe", C.c_void_p, restype=C.c_char_p)
+_ffi._sig("he_plan_graph", C.c_void_p, C.POINTER(C.c_void_p))
 _ffi._sig("he_plan_destroy", C.c_void_p)
 _ffi._sig("he_plan_precompile", C.c_void_p)
 _ffi._sig("he_execute_graph", C.c_void_p, C.POINTER(C.c_uint32), C.POINTER(C.c_void_p), C.c_int, C.POINTER(C.c_uint32),
@@ -26,6 +27,7 @@ _ffi._sig("he_backend_set_option", C.c_int, C.c_int64)
 OPT_FUSE_MATMUL_EPILOGUE = 0
 OPT_FOLD_SWAP_INTO_REDUCE = 1
 OPT_REMATERIALIZE = 2
+OPT_CANCEL_TRANSPOSES = 3
 
 
 def set_option(option, value):
@@ -100,6 +102,15 @@ class Plan:
                 instrs.append((kind, [int(x) for x in nodes.rstrip("}").split(",") if x]))
             released = [int(x) for x in rel.replace("release", "").split()]
             self.steps.append((instrs, released))
+
+    def graph(self):
+        """The graph the instructions are made of (he_plan_graph): the planned graph as the backend's rewrites left
+        it, as an ir.OpGraph whose node dicts carry "origin"."""
+        from . import ir
+
+        handle = C.c_void_p()
+        check(lib.he_plan_graph(self.handle, C.byref(handle)))
+        return ir.OpGraph.from_handle(handle)
 
     def precompile(self):
         """Compiles the kernels of all instructions (in parallel) into the kernel caches; needs no device."""

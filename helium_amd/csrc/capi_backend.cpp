@@ -68,6 +68,14 @@ int he_plan_generate(he_graph_t graph, he_plan_t* plan) {
         *plan = p.release();
     });
 }
+int he_plan_graph(he_plan_t plan, he_graph_t* graph) {
+    return he::guard([&] {
+        HE_REQUIRE(plan && graph, HE_ERR_INVALID, "bad argument");
+        auto g = std::make_unique<he_graph_s>();
+        g->g = std::make_shared<he::ir::OpGraph>(*plan->graph);
+        *graph = g.release();
+    });
+}
 int he_plan_num_steps(he_plan_t plan, int* steps) {
     return he::guard([&] { *steps = (int)plan->plan->steps.size(); });
 }
@@ -138,6 +146,7 @@ int he_backend_set_option(int option, int64_t value) {
             case HE_OPT_FUSE_MATMUL_EPILOGUE: he::plan::set_fuse_matmul_epilogue(value != 0); break;
             case HE_OPT_FOLD_SWAP_INTO_REDUCE: he::plan::set_fold_swap_into_reduce(value != 0); break;
             case HE_OPT_REMATERIALIZE: he::plan::set_rematerialize(value != 0); break;
+            case HE_OPT_CANCEL_TRANSPOSES: he::plan::set_cancel_transposes(value != 0); break;
             default: he::fail(HE_ERR_INVALID, "unknown backend option");
         }
     });

@@ -97,6 +97,56 @@ int he_graph_node_info(he_graph_t graph, uint32_t node, int32_t* kind, int32_t* 
     });
 }
 
+int he_graph_node_op(he_graph_t graph, uint32_t node, he_op_desc* op, int64_t* axes_out, int64_t* shape_out, uint32_t* origin) {
+    return he::guard([&] {
+        HE_REQUIRE(graph && op && axes_out && shape_out && origin, HE_ERR_INVALID, "bad argument");
+        const he::ir::Node& n = graph->g->get(node);
+        *origin = graph->g->origin(node);
+        *op = he_op_desc{};
+        op->kind = -1;
+        if (n.kind == he::ir::Node::Output) {
+            op->inputs[0] = graph->g->inbound(node)[0];
+            op->num_inputs = 1;
+        }
+        if (n.kind != he::ir::Node::Intermediate) return;
+        const he::ir::Op& o = n.op;
+        HE_REQUIRE(o.broadcast_axes.size() <= 16 && o.shape.size() <= 16, HE_ERR_INVALID, "rank too large");
+        op->kind = (int)o.kind;
+        op->num_inputs = (int)o.inputs.size();
+        for (size_t i = 0; i < o.inputs.size(); i++) op->inputs[i] = o.inputs[i];
+        op->sub_op = o.sub_op;
+        op->precision = (int)o.precision;
+        op->target_type = o.target_type;
+        op->depth = o.depth;
+        op->new_dim_count = o.new_dim_count;
+        op->num_broadcast_axes = (int)o.broadcast_axes.size();
+        for (size_t i = 0; i < o.broadcast_axes.size(); i++) {
+            axes_out[2 * i] = o.broadcast_axes[i].axis;
+            axes_out[2 * i + 1] = o.broadcast_axes[i].new_size;
+        }
+        op->broadcast_axes = axes_out;
+        op->shape_rank = (int)o.shape.size();
+        for (size_t i = 0; i < o.shape.size(); i++) shape_out[i] = o.shape[i];
+        op->shape = shape_out;
+        op->axis_a = o.axis_a;
+        op->axis_b = o.axis_b;
+        op->const_bits = o.const_bits;
+        op->const_dtype = o.const_dtype;
+        op->conv_in_channels = o.conv.in_channels;
+        op->conv_out_channels = o.conv.out_channels;
+        for (int i = 0; i < 2; i++) {
+            op->conv_kernel[i] = o.conv.kernel[i];
+            op->conv_stride[i] = o.conv.stride[i];
+            op->conv_dilation[i] = o.conv.dilation[i];
+            op->conv_input_size[i] = o.conv.input_size[i];
+        }
+        op->conv_padding_mode = o.conv.padding_mode;
+    });
+}
+int he_graph_capacity(he_graph_t graph, uint32_t* capacity) {
+    return he::guard([&] { *capacity = (uint32_t)graph->g->capacity(); });
+}
+
 int he_pointwise_supports(he_graph_t graph, const uint32_t* nodes, int num_nodes, int* supported) {
     return he::guard([&] {
         he::ir::OpSubgraph sg(graph->g, std::vector<he::ir::NodeId>(nodes, nodes + num_nodes));

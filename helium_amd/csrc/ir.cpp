@@ -1,6 +1,7 @@
 #include "ir.h"
 
 #include <functional>
+#include <map>
 #include <set>
 #include <sstream>
 #include <unordered_map>
@@ -479,5 +480,280 @@ std::shared_ptr<OpGraph> rematerialized(const OpGraph& g, const std::set<NodeId>
     out->optimize();
     return out;
 }
+
+// ---------------------------------------------------------------------------------------------------------
+// Transpositions that cancel
+// ---------------------------------------------------------------------------------------------------------
+namespace {
+using Perm = std::vector<int>;  // transposed.shape[i] = source.shape[perm[i]]
+
+bool is_identity(const Perm& p) {
+    for (size_t i = 0; i < p.size(); i++)
+        if (p[i] != (int)i) return false;
+    return true;
+}
+// transposing by `first`, then by `second`
+Perm compose(const Perm& first, const Perm& second) {
+    Perm out(second.size());
+    for (size_t i = 0; i < second.size(); i++) out[i] = first[second[i]];
+    return out;
+}
+Perm swap_perm(size_t rank, int64_t a, int64_t b) {
+    Perm p(rank);
+    for (size_t i = 0; i < rank; i++) p[i] = (int)i;
+    std::swap(p[a], p[b]);
+    return p;
+}
+// swaps (applied in order) that turn the identity into `p`
+std::vector<std::pair<int, int>> swaps_for(const Perm& p) {
+    std::vector<std::pair<int, int>> out;
+    Perm cur(p.size());
+    for (size_t i = 0; i < p.size(); i++) cur[i] = (int)i;
+    for (size_t i = 0; i < p.size(); i++) {
+        if (cur[i] == p[i]) continue;
+        size_t j = i + 1;
+        while (cur[j] != p[i]) j++;
+        out.push_back({(int)i, (int)j});
+        std::swap(cur[i], cur[j]);
+    }
+    return out;
+}
+}  // namespace
+
+std::shared_ptr<OpGraph> transposes_cancelled(const OpGraph& g) {
+    const size_t cap = g.capacity();
+    constexpr int kStop = 1000;  // a transposition that would have to stay, somewhere further up
+    // What is left of a transposition by `p` of `node`'s value once it has been moved towards the producers: 0 when it
+    // disappears (it meets its inverse, a broadcast, or a constant on every path), the number of transpositions
+    // that remain otherwise.
+    std::map<std::pair<NodeId, Perm>, int> left_memo;
+    std::function<int(NodeId, const Perm&)> left = [&](NodeId node, const Perm& p) -> int {
+        if (is_identity(p)) return 0;
+        auto key = std::make_pair(node, p);
+        auto it = left_memo.find(key);
+        if (it != left_memo.end()) return it->second;
+        left_memo[key] = kStop;  // (no cycles in a graph; the entry is overwritten below)
+        const Node& n = g.get(node);
+        int cost = kStop;
+        if (n.kind == Node::Intermediate && n.desc.shape.size() == p.size()) {
+            switch (n.op.kind) {
+                case OpKind::SwapDims: cost = left(n.op.inputs[0], compose(swap_perm(p.size(), n.op.axis_a, n.op.axis_b), p)); break;
+                case OpKind::UnaryPointwise:
+                case OpKind::ChangeDataType:
+                case OpKind::BinaryPointwise:
+                case OpKind::Compare:
+                case OpKind::Select: {
+                    cost = 0;
+                    for (NodeId in : n.op.inputs) {
+                        if (g.get(in).desc.shape != g.get(n.op.inputs[0]).desc.shape) cost = kStop;
+                        cost = std::min(kStop, cost + left(in, p));
+                    }
+                    break;
+                }
+                case OpKind::Constant: cost = 0; break;
+                case OpKind::Broadcast: {
+                    // the listed axes must be extents of 1 in the source, and the source small next to the result
+                    Shape padded = g.get(n.op.inputs[0]).desc.shape;
+                    while ((int64_t)padded.size() < n.op.new_dim_count) padded.insert(padded.begin(), 1);
+                    bool plain = padded.size() == p.size() && num_elements(padded) * 8 <= num_elements(n.desc.shape);
+                    for (auto& a : n.op.broadcast_axes) plain = plain && padded[a.axis] == 1;
+                    if (plain) cost = 0;
+                    break;
+                }
+                default: break;
+            }
+        }
+        left_memo[key] = cost;
+        return cost;
+    };
+
+    auto out = std::make_shared<OpGraph>();
+    std::vector<NodeId> placed(cap, kNoNode);
+    auto note_origin = [&](NodeId fresh, NodeId old) {
+        if (out->origin_.size() <= fresh) out->origin_.resize(fresh + 1, kNoNode);
+        out->origin_[fresh] = old;
+    };
+    auto swapped = [&](NodeId fresh, const Perm& p, NodeId origin) {
+        for (auto [a, b] : swaps_for(p)) {
+            Op op;
+            op.kind = OpKind::SwapDims;
+            op.inputs = {fresh};
+            op.axis_a = a;
+            op.axis_b = b;
+            fresh = out->new_op(std::move(op));
+            note_origin(fresh, origin);
+        }
+        return fresh;
+    };
+    bool changed = false;
+    // `node`'s value transposed by `p`, as a node of `out`. `recorded`: a SwapDims of `g` that SwapDims nodes made here
+    // stand for (an origin has to be a node that only moves data: whoever evaluates the plan on `g` reads such nodes
+    // through, and would otherwise recompute a value that the plan keeps in memory).
+    std::map<std::pair<NodeId, Perm>, NodeId> built;
+    std::function<NodeId(NodeId, const Perm&, NodeId)> build = [&](NodeId node, const Perm& p, NodeId recorded) -> NodeId {
+        if (is_identity(p)) return placed[node];
+        auto key = std::make_pair(node, p);
+        auto it = built.find(key);
+        if (it != built.end()) return it->second;
+        const Node& n = g.get(node);
+        NodeId fresh = kNoNode;
+        if (left(node, p) != 0) {
+            fresh = swapped(placed[node], p, recorded);
+        } else {
+            switch (n.op.kind) {
+                case OpKind::SwapDims: fresh = build(n.op.inputs[0], compose(swap_perm(p.size(), n.op.axis_a, n.op.axis_b), p), recorded); break;
+                case OpKind::Constant: {
+                    Op op = n.op;
+                    for (size_t i = 0; i < p.size(); i++) op.shape[i] = n.op.shape[p[i]];
+                    fresh = out->new_op(std::move(op));
+                    note_origin(fresh, node);
+                    break;
+                }
+                case OpKind::Broadcast: {
+                    const Shape& src = g.get(n.op.inputs[0]).desc.shape;
+                    Shape padded = src;
+                    while (padded.size() < p.size()) padded.insert(padded.begin(), 1);
+                    Shape moved(p.size());
+                    for (size_t i = 0; i < p.size(); i++) moved[i] = padded[p[i]];
+                    // extents of 1 do not count: when the others keep their order the source is only given a new shape
+                    std::vector<int64_t> before, after;
+                    for (size_t i = 0; i < p.size(); i++) {
+                        if (padded[i] != 1) before.push_back((int64_t)i);
+                        if (moved[i] != 1) after.push_back(p[i]);
+                    }
+                    NodeId source = placed[n.op.inputs[0]];
+                    if (before == after) {
+                        if (moved != src) {
+                            Op r;
+                            r.kind = OpKind::Reshape;
+                            r.inputs = {source};
+                            r.shape = moved;
+                            source = out->new_op(std::move(r));
+                            note_origin(source, node);
+                        }
+                    } else {
+                        if (padded != src) {
+                            Op r;
+                            r.kind = OpKind::Reshape;
+                            r.inputs = {source};
+                            r.shape = padded;
+                            source = out->new_op(std::move(r));
+                            note_origin(source, node);
+                        }
+                        source = swapped(source, p, node);
+                    }
+                    Op op = n.op;
+                    op.inputs = {source};
+                    op.new_dim_count = (int64_t)p.size();
+                    for (auto& a : op.broadcast_axes)
+                        for (size_t i = 0; i < p.size(); i++)
+                            if (p[i] == a.axis) {
+                                a.axis = (int64_t)i;
+                                break;
+                            }
+                    std::sort(op.broadcast_axes.begin(), op.broadcast_axes.end(), [](const BroadcastAxis& x, const BroadcastAxis& y) { return x.axis < y.axis; });
+                    fresh = out->new_op(std::move(op));
+                    note_origin(fresh, node);
+                    break;
+                }
+                default: {  // pointwise: the same op on transposed operands
+                    Op op = n.op;
+                    for (NodeId& in : op.inputs) in = build(in, p, recorded);
+                    fresh = out->new_op(std::move(op));
+                    note_origin(fresh, node);
+                    break;
+                }
+            }
+        }
+        built[key] = fresh;
+        return fresh;
+    };
+
+    for (NodeId id : g.inputs()) {
+        placed[id] = out->new_input(g.get(id).desc);
+        note_origin(placed[id], id);
+    }
+    for (NodeId id : g.nodes()) {
+        const Node& n = g.get(id);
+        if (n.kind == Node::Input) continue;
+        if (n.kind == Node::Output) {
+            placed[id] = out->new_output(placed[g.inbound(id)[0]]);
+            note_origin(placed[id], id);
+            continue;
+        }
+        const size_t rank = n.op.inputs.empty() ? 0 : g.get(n.op.inputs[0]).desc.shape.size();
+        if (n.op.kind == OpKind::SwapDims) {
+            const Perm p = swap_perm(rank, n.op.axis_a, n.op.axis_b);
+            if (left(n.op.inputs[0], p) == 0) {
+                placed[id] = build(n.op.inputs[0], p, id);
+                changed = true;
+                continue;
+            }
+        }
+        if (n.op.kind == OpKind::Reduce && g.get(n.op.inputs[0]).kind == Node::Intermediate && g.get(n.op.inputs[0]).op.kind == OpKind::SwapDims) {
+            // The reduced dims may come in any order. Of all transpositions that put the kept dims first, in their
+            // order, the one with the fewest swaps is taken: a chain of swaps (the gradient of a broadcast is recorded as
+            // one, tensor.rs) becomes the single swap that the pointwise kernel folds into its walk over the tensor.
+            NodeId base = n.op.inputs[0];
+            Perm p(rank);
+            for (size_t i = 0; i < rank; i++) p[i] = (int)i;
+            size_t chain = 0;
+            while (g.get(base).kind == Node::Intermediate && g.get(base).op.kind == OpKind::SwapDims) {
+                const Op& s = g.get(base).op;
+                p = compose(swap_perm(rank, s.axis_a, s.axis_b), p);
+                base = s.inputs[0];
+                chain++;
+            }
+            const size_t kept = rank - n.op.depth;
+            Perm q(rank, -1);
+            std::vector<bool> used(rank, false);
+            for (size_t i = 0; i < kept; i++) {
+                q[i] = p[i];
+                used[p[i]] = true;
+            }
+            for (size_t j = kept; j < rank; j++)  // a reduced dim that can stay where it is
+                if (!used[j]) {
+                    q[j] = (int)j;
+                    used[j] = true;
+                }
+            for (size_t j = kept; j < rank; j++) {
+                if (q[j] >= 0) continue;
+                // dim j is kept, at position i: dim i coming here closes a cycle of two
+                size_t i = 0;
+                while (q[i] != (int)j) i++;
+                size_t pick = !used[i] ? i : rank;
+                for (size_t d = 0; d < rank && pick == rank; d++)
+                    if (!used[d]) pick = d;
+                q[j] = (int)pick;
+                used[pick] = true;
+            }
+            if (swaps_for(q).size() < chain) {
+                Op op = n.op;
+                op.inputs = {build(base, q, n.op.inputs[0])};
+                const NodeId fresh = out->new_op(std::move(op));
+                if (out->get(fresh).desc == n.desc) {
+                    placed[id] = fresh;
+                    note_origin(fresh, id);
+                    changed = true;
+                    continue;
+                }
+                // (a reduction that did not keep its shape is left in place, unused, and pruned below)
+            }
+        }
+        Op op = n.op;
+        for (NodeId& in : op.inputs) in = placed[in];
+        placed[id] = out->new_op(std::move(op));
+        note_origin(placed[id], id);
+    }
+    if (!changed) return nullptr;
+    out->optimize();
+    return out;
+}
+
+void OpGraph::rebase_origins(const OpGraph& through) {
+    for (NodeId& o : origin_)
+        if (o != kNoNode) o = through.origin(o);
+}
+
 
 }  // namespace he::ir

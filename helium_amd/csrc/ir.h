@@ -113,6 +113,8 @@ public:
     // nodes may stand for the same one); the node itself in any other graph.
     NodeId origin(NodeId id) const { return id < origin_.size() ? origin_[id] : id; }
     bool has_origins() const { return !origin_.empty(); }
+    // When the graph this one was built from was itself built from another: origins then name that one's nodes.
+    void rebase_origins(const OpGraph& through);
 
 private:
     NodeId push(Node n);
@@ -121,6 +123,7 @@ private:
     std::vector<std::vector<NodeId>> in_, out_;
     std::vector<NodeId> origin_;
     friend std::shared_ptr<OpGraph> rematerialized(const OpGraph& g, const std::set<NodeId>& keep_single);
+    friend std::shared_ptr<OpGraph> transposes_cancelled(const OpGraph& g);
 };
 
 // A copy of `g` in which values that are cheap to compute again are computed once per use instead of once: every
@@ -134,6 +137,17 @@ private:
 // large permute, an Output) shares one copy. `keep_single`: nodes of `g` that are not to be duplicated. Node ids are new
 // (in dataflow order); `origin` maps them back to `g`. Returns null when nothing changes.
 std::shared_ptr<OpGraph> rematerialized(const OpGraph& g, const std::set<NodeId>& keep_single = {});
+
+// A copy of `g` without the transpositions that undo each other. The reference's front end writes a reduction over
+// leading dims as SwapDims + Reduce and its gradient rules answer a SwapDims with a SwapDims (tensor.rs), so a recorded
+// backward pass computes whole chains of pointwise ops on the transposed tensor and transposes the result back (batch
+// norm: the statistics over N, H, W of an NHWC activation). Here a SwapDims is moved towards the producers of its
+// operand - through pointwise ops (the same op on transposed operands), into broadcasts (whose axes are renamed) and
+// constants - and is dropped when on every path it meets the SwapDims it undoes; the ops in between are then computed
+// in the layout of the tensors in memory. A chain of SwapDims in front of a Reduce is replaced by the shortest chain that
+// reduces the same dims (their order does not matter to a Sum / Mean / Min / Max beyond rounding). Node ids are new;
+// `origin` names the node of `g` whose value, possibly transposed, a node computes. Returns null when nothing changes.
+std::shared_ptr<OpGraph> transposes_cancelled(const OpGraph& g);
 
 // Subset of an OpGraph (opgraph/subgraph.rs): nodes sorted by id; `inputs` = outside producers feeding it,
 // `roots` = members with an outside input, `leafs` = members with an outside consumer.

@@ -149,8 +149,14 @@ public:
     Program run() {
         HE_REQUIRE(!sg_.leafs().empty(), HE_ERR_INVALID, "pointwise subgraph has no output");
         // Iteration space: the (pre-reduction) shape of the first leaf, as compute_output_shape picks it
-        // (jit.rs:350-362).
+        // (jit.rs:350-362) - of the first Reduce leaf when there is one: the reductions of a kernel share one input
+        // shape and have to walk it dim by dim, the other outputs only need their element.
         ir::NodeId first = sg_.leafs()[0];
+        for (ir::NodeId leaf : sg_.leafs())
+            if (g_.get(leaf).op.kind == ir::OpKind::Reduce) {
+                first = leaf;
+                break;
+            }
         const ir::Node& fn = g_.get(first);
         p_.dims = fn.op.kind == ir::OpKind::Reduce ? g_.get(fn.op.inputs[0]).desc.shape : fn.desc.shape;
         if (anchor_ != ir::kNoNode) {

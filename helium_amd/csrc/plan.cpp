@@ -47,6 +47,7 @@ namespace {
 std::atomic<bool> g_fuse_matmul_epilogue{true};
 std::atomic<bool> g_fold_swap_into_reduce{true};
 std::atomic<bool> g_rematerialize{true};
+std::atomic<bool> g_cancel_transposes{true};
 
 // True when every value computed from `node` inside the graph ends in a Reduce, through pointwise ops only: nothing
 // then needs the transposed tensor in memory.
@@ -75,11 +76,13 @@ void set_fuse_matmul_epilogue(bool on) { g_fuse_matmul_epilogue.store(on); }
 bool fuse_matmul_epilogue() { return g_fuse_matmul_epilogue.load(); }
 unsigned option_mask() {
     // the hash of the tuning overrides (0 unless tuning is on) rides along: plans keep their kernels
-    return (fuse_matmul_epilogue() ? 1u : 0u) | (g_fold_swap_into_reduce.load() ? 2u : 0u) | (g_rematerialize.load() ? 4u : 0u) | (tuning::hash() << 3);
+    return (fuse_matmul_epilogue() ? 1u : 0u) | (g_fold_swap_into_reduce.load() ? 2u : 0u) | (g_rematerialize.load() ? 4u : 0u) | (g_cancel_transposes.load() ? 8u : 0u) | (tuning::hash() << 4);
 }
 void set_fold_swap_into_reduce(bool on) { g_fold_swap_into_reduce.store(on); }
 void set_rematerialize(bool on) { g_rematerialize.store(on); }
 bool rematerialize() { return g_rematerialize.load(); }
+void set_cancel_transposes(bool on) { g_cancel_transposes.store(on); }
+bool cancel_transposes() { return g_cancel_transposes.load(); }
 bool fold_swap_into_reduce() { return g_fold_swap_into_reduce.load(); }
 
 bool Instr::can_fuse_with(const Instr& next) const {
@@ -471,30 +474,53 @@ int64_t plan_traffic_bytes(const Plan& plan) {
 }
 
 std::shared_ptr<const ir::OpGraph> graph_for_execution(const std::shared_ptr<const ir::OpGraph>& g) {
-    if (!rematerialize()) return g;
-    std::shared_ptr<const ir::OpGraph> other = ir::rematerialized(*g);
-    if (!other) return g;
-    // Copies that the fusion rules keep out of their consumers' kernels are written out, each on its own: where one
-    // kernel ends up with several copies of a value among its outputs, that value goes back to being computed once, and
-    // the graph is planned again.
-    std::set<ir::NodeId> keep_single;
-    for (int round = 0; round < 3; round++) {
-        const size_t known = keep_single.size();
-        if (getenv("HELIUM_HIP_PLAN_DEBUG")) fprintf(stderr, "[plan] round %d: %zu -> %zu nodes, %zu kept single\n", round, g->num_nodes(), other->num_nodes(), known);
-        const auto plan = generate_plan(other);
-        for (auto& st : plan->steps)
-            for (auto& instr : st.instrs) {
-                std::set<ir::NodeId> origins;
-                for (ir::NodeId leaf : instr->outputs())
-                    if (!origins.insert(other->origin(leaf)).second) keep_single.insert(other->origin(leaf));
-            }
-        if (keep_single.size() == known) break;
-        other = ir::rematerialized(*g, keep_single);
-        if (!other) return g;
+    const bool debug = getenv("HELIUM_HIP_PLAN_DEBUG") != nullptr;
+    // 1. transpositions that undo each other go
+    std::shared_ptr<const ir::OpGraph> base = g;
+    if (cancel_transposes())
+        if (auto untransposed = ir::transposes_cancelled(*g)) {
+            if (debug) fprintf(stderr, "[plan] transpositions cancelled: %zu -> %zu nodes\n", g->num_nodes(), untransposed->num_nodes());
+            base = untransposed;
+        }
+    // 2. cheap values are computed where they are used
+    std::shared_ptr<ir::OpGraph> other = rematerialize() ? ir::rematerialized(*base) : nullptr;
+    if (other) {
+        // Copies that the fusion rules keep out of their consumers' kernels are written out, each on its own: where one
+        // kernel ends up with several copies of a value among its outputs, that value goes back to being computed once,
+        // and the graph is planned again.
+        std::set<ir::NodeId> keep_single;
+        for (int round = 0; round < 3 && other; round++) {
+            const size_t known = keep_single.size();
+            if (debug) fprintf(stderr, "[plan] round %d: %zu -> %zu nodes, %zu kept single\n", round, base->num_nodes(), other->num_nodes(), known);
+            const auto plan = generate_plan(other);
+            for (auto& st : plan->steps)
+                for (auto& instr : st.instrs) {
+                    std::set<ir::NodeId> origins;
+                    for (ir::NodeId leaf : instr->outputs())
+                        if (!origins.insert(other->origin(leaf)).second) keep_single.insert(other->origin(leaf));
+                }
+            if (keep_single.size() == known) break;
+            other = ir::rematerialized(*base, keep_single);
+        }
     }
-    // ... and the rewritten graph is taken only when its plan moves fewer bytes.
-    const int64_t before = plan_traffic_bytes(*generate_cached_plan(g)), after = plan_traffic_bytes(*generate_cached_plan(other));
-    return after < before ? other : g;
+    std::shared_ptr<const ir::OpGraph> chosen = base;
+    if (other) {
+        if (base != g) other->rebase_origins(*base);
+        chosen = other;
+    }
+    if (chosen == g) return g;
+    // ... and a rewritten graph is taken only when its plan moves fewer bytes.
+    const int64_t before = plan_traffic_bytes(*generate_cached_plan(g));
+    int64_t after = plan_traffic_bytes(*generate_cached_plan(chosen));
+    if (chosen != base && base != g) {
+        const int64_t without_copies = plan_traffic_bytes(*generate_cached_plan(base));
+        if (without_copies <= after) {
+            chosen = base;
+            after = without_copies;
+        }
+    }
+    if (debug) fprintf(stderr, "[plan] bytes moved by the plan: %lld as recorded, %lld rewritten\n", (long long)before, (long long)after);
+    return after < before ? chosen : g;
 }
 
 // ---------------------------------------------------------------------------------------------------------

@@ -79,10 +79,13 @@ bool fold_swap_into_reduce();
 // (ir::rematerialized; on by default, off plans the graph as recorded, like the reference).
 void set_rematerialize(bool on);
 bool rematerialize();
+// Whether transpositions that undo each other are taken out of the graph first (ir::transposes_cancelled; on by default).
+void set_cancel_transposes(bool on);
+bool cancel_transposes();
 // Bytes the plan's kernels read and write: the sizes of every instruction's inputs and outputs.
 int64_t plan_traffic_bytes(const Plan& plan);
-// The graph the backend plans and runs for `g` (already pruned): `g` itself, or its rematerialised form when that
-// form's plan moves fewer bytes. Input and Output nodes of the result map back through OpGraph::origin.
+// The graph the backend plans and runs for `g` (already pruned): `g` itself, or the form the two rewrites above give it
+// when that form's plan moves fewer bytes. Input and Output nodes of the result map back through OpGraph::origin.
 std::shared_ptr<const ir::OpGraph> graph_for_execution(const std::shared_ptr<const ir::OpGraph>& g);
 
 // generate_plan (plan_generation.rs:22-26).

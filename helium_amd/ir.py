@@ -41,6 +41,9 @@ _ffi._sig("he_graph_optimize", C.c_void_p)
 _ffi._sig("he_graph_num_nodes", C.c_void_p, C.POINTER(C.c_uint32))
 _ffi._sig("he_graph_node_info", C.c_void_p, C.c_uint32, C.POINTER(C.c_int32), C.POINTER(C.c_int32),
           C.POINTER(C.c_int32), C.POINTER(C.c_int64))
+_ffi._sig("he_graph_node_op", C.c_void_p, C.c_uint32, C.POINTER(OpDesc), C.POINTER(C.c_int64), C.POINTER(C.c_int64),
+          C.POINTER(C.c_uint32))
+_ffi._sig("he_graph_capacity", C.c_void_p, C.POINTER(C.c_uint32))
 
 
 def scalar_bits(value, dtype):
@@ -59,6 +62,21 @@ def scalar_bits(value, dtype):
     raise ValueError(dtype)
 
 
+def scalar_from_bits(bits, dtype):
+    """Inverse of scalar_bits."""
+    if dtype == "f32":
+        return struct.unpack("<f", struct.pack("<I", bits))[0]
+    if dtype == "bf16":
+        return struct.unpack("<f", struct.pack("<I", (bits & 0xFFFF) << 16))[0]
+    if dtype == "f16":
+        return float(np.array(bits & 0xFFFF, dtype=np.uint16).view(np.float16))
+    if dtype == "u32":
+        return int(bits)
+    if dtype == "bool":
+        return bool(bits)
+    raise ValueError(dtype)
+
+
 class OpGraph:
     def __init__(self):
         self.handle = C.c_void_p()
@@ -73,6 +91,57 @@ class OpGraph:
                 self.handle = C.c_void_p()
         except Exception:
             pass
+
+    @classmethod
+    def from_handle(cls, handle):
+        """Takes over a graph handle the library made (he_plan_graph) and reads its nodes back; every node dict also
+        carries "origin", the node of the planned graph it stands for."""
+        self = cls.__new__(cls)
+        self.handle, self.nodes, self.num_outputs = handle, [], 0
+        cap = C.c_uint32()
+        check(lib.he_graph_capacity(handle, C.byref(cap)))
+        d, axes, shape, origin = OpDesc(), (C.c_int64 * 32)(), (C.c_int64 * 16)(), C.c_uint32()
+        kind, dtype, rank, dims = C.c_int32(), C.c_int32(), C.c_int32(), (C.c_int64 * 16)()
+        for i in range(cap.value):
+            if lib.he_graph_node_info(handle, i, C.byref(kind), C.byref(dtype), C.byref(rank), dims) != 0 or kind.value == 3:
+                continue  # pruned
+            check(lib.he_graph_node_op(handle, i, C.byref(d), axes, shape, C.byref(origin)))
+            desc = {"shape": list(dims[: rank.value]), "dtype": _ffi.DTYPE_NAMES[dtype.value]}
+            if kind.value == 0:
+                n = {"id": i, "node": "input", **desc}
+            elif kind.value == 2:
+                n = {"id": i, "node": "output", "from": d.inputs[0]}
+                self.num_outputs += 1
+            else:
+                op = KINDS[d.kind]
+                n = {"id": i, "node": "op", "op": op, "inputs": list(d.inputs[: d.num_inputs]), **desc}
+                if op == "matmul":
+                    n["precision"] = PRECISION[d.precision]
+                elif op in ("unary", "binary", "reduce", "compare"):
+                    n["fn"] = {"unary": UNARY, "binary": BINARY, "reduce": REDUCE, "compare": COMPARE}[op][d.sub_op]
+                    if op == "reduce":
+                        n["depth"] = d.depth
+                elif op == "change_dtype":
+                    n["target"] = _ffi.DTYPE_NAMES[d.target_type]
+                elif op == "broadcast":
+                    n["new_dim_count"] = d.new_dim_count
+                    n["axes"] = [[axes[2 * k], axes[2 * k + 1]] for k in range(d.num_broadcast_axes)]
+                elif op == "reshape":
+                    n["new_shape"] = list(shape[: d.shape_rank])
+                elif op == "swap_dims":
+                    n["axis_a"], n["axis_b"] = d.axis_a, d.axis_b
+                elif op == "constant":
+                    n["const_dtype"] = _ffi.DTYPE_NAMES[d.const_dtype]
+                    n["value"] = scalar_from_bits(d.const_bits, n["const_dtype"])
+                elif op in ("conv", "conv_bwd_data", "conv_bwd_filter"):
+                    n["params"] = {"in_channels": d.conv_in_channels, "out_channels": d.conv_out_channels,
+                                   "kernel_size": list(d.conv_kernel), "stride": list(d.conv_stride),
+                                   "dilation": list(d.conv_dilation), "padding_mode": PADDING[d.conv_padding_mode]}
+                    if op == "conv_bwd_data":
+                        n["input_size"] = list(d.conv_input_size)
+            n["origin"] = origin.value
+            self.nodes.append(n)
+        return self
 
     # -- node creation -----------------------------------------------------------------------------------
     def new_input(self, shape, dtype):

@@ -198,6 +198,12 @@ int he_graph_optimize(he_graph_t graph);                                      /*
 int he_graph_num_nodes(he_graph_t graph, uint32_t* count);
 /* Descriptor of a node (opgraph.rs:240-246). shape_out must hold 16 entries. kind: 0 input, 1 intermediate, 2 output. */
 int he_graph_node_info(he_graph_t graph, uint32_t node, int32_t* kind, int32_t* dtype, int32_t* rank, int64_t* shape_out);
+/* Reads a node back: the counterpart of he_graph_new_op. `op->kind` is -1 for an Input or Output node (an Output's
+ * source is inputs[0]); `op->broadcast_axes` and `op->shape` point into axes_out (32 entries) and shape_out (16).
+ * `origin`: for a graph that he_plan_graph returned, the node of the planned graph this node stands for; the node itself
+ * otherwise. he_graph_capacity: one more than the largest node id ever given out (ids of pruned nodes stay unused). */
+int he_graph_node_op(he_graph_t graph, uint32_t node, he_op_desc* op, int64_t* axes_out, int64_t* shape_out, uint32_t* origin);
+int he_graph_capacity(he_graph_t graph, uint32_t* capacity);
 
 /* ==================================================================================================
  * 4. Pointwise / reduction instruction — helium/src/cuda/instr/pointwise.rs + pointwise/jit.rs (kernels K2, K3).
@@ -296,6 +302,10 @@ int he_tensor_free(he_tensor_t tensor);
 
 /* generate_plan (plan_generation.rs:22-26) for the graph as it stands; the graph must outlive the plan. */
 int he_plan_generate(he_graph_t graph, he_plan_t* plan);
+/* The graph the plan's instructions are made of, as a new graph the caller destroys: the planned graph itself, or the
+ * form the backend's rewrites gave it (HE_OPT_CANCEL_TRANSPOSES, HE_OPT_REMATERIALIZE). Instructions and
+ * he_plan_describe name nodes of the planned graph (he_graph_node_op's `origin`). */
+int he_plan_graph(he_plan_t plan, he_graph_t* graph);
 int he_plan_num_steps(he_plan_t plan, int* steps);
 /* One line per step: "step i: kind{node,node,...} ... | release node ...". */
 const char* he_plan_describe(he_plan_t plan);
@@ -365,8 +375,14 @@ int he_fgraph_subdivide(he_fgraph_t graph, uint64_t* nodes, int32_t* portions, i
  * that uses it and the value never travels through memory - a batch norm's forward pass as the reference records it
  * (modules/batch_norm.rs:53-71) otherwise leaves eight full-size intermediates for the backward pass. The rewritten
  * graph is used only when its plan moves fewer bytes; he_plan_describe names copies by the nodes they stand for. 0 plans
- * the graph as recorded, like plan_generation.rs. */
-enum { HE_OPT_FUSE_MATMUL_EPILOGUE = 0, HE_OPT_FOLD_SWAP_INTO_REDUCE = 1, HE_OPT_REMATERIALIZE = 2 };
+ * the graph as recorded, like plan_generation.rs.
+ * HE_OPT_CANCEL_TRANSPOSES (default 1): a SwapDims is moved towards the producers of its operand (through pointwise ops,
+ * into broadcasts and constants) and dropped where on every path it meets the SwapDims it undoes, so the pointwise ops
+ * between the two run in the layout the tensors have in memory; the chain of SwapDims in front of a Reduce becomes the
+ * shortest chain that reduces the same dims. The backward pass of a reduction over leading dims (tensor.rs answers a
+ * SwapDims with a SwapDims) otherwise transposes a full-size tensor twice. Applied before HE_OPT_REMATERIALIZE, under
+ * the same condition (fewer bytes moved by the plan); 0 keeps every SwapDims as recorded. */
+enum { HE_OPT_FUSE_MATMUL_EPILOGUE = 0, HE_OPT_FOLD_SWAP_INTO_REDUCE = 1, HE_OPT_REMATERIALIZE = 2, HE_OPT_CANCEL_TRANSPOSES = 3 };
 int he_backend_set_option(int option, int64_t value);
 
 /* Counters of the last he_execute_graph on this thread: [0] steps run, [1] instructions, [2] streams used,

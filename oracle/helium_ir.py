@@ -364,7 +364,10 @@ def plan_outputs(nodes, inputs, plan_steps):
     leaves the kernel that computes it, and is kept in f32 inside a kernel. The kernels are evaluated one by one, in
     plan order, each on its own members: a node may be a member of several instructions (a value the plan computes
     again in every kernel that uses it instead of passing it through memory), and every kernel then works on its own,
-    unrounded copy. Returns {output node id: storage array}."""
+    unrounded copy. A member may also stand for its value in another layout (a plan that cancels transpositions computes a
+    pointwise op on the untransposed operands and leaves the SwapDims out): element by element that is the same
+    arithmetic, so the op is evaluated as recorded and the SwapDims, a member of no kernel, is read through.
+    Returns {output node id: storage array}."""
     by_id = {n["id"]: n for n in nodes}
     # ops that compute the same thing may be one op of the plan (it then names the first of them): every id is read
     # through `canon`
@@ -379,7 +382,14 @@ def plan_outputs(nodes, inputs, plan_steps):
 
     class _Through(dict):
         def __getitem__(self, k):
-            return dict.__getitem__(self, canon[k])
+            k = canon[k]
+            if not dict.__contains__(self, k) and by_id[k].get("op") in ("swap_dims", "reshape", "broadcast"):
+                # A plan may have taken a transposition out (the ops behind it then run on the untransposed tensor and
+                # the plan names them, not the SwapDims) or folded a shape op into a neighbour: such ops only move
+                # values, so they are read through, from whatever holds their operand.
+                # (not kept: a later kernel may compute the operand afresh, and must then see its own copy)
+                return _eval_op(by_id[k], desc, self)
+            return dict.__getitem__(self, k)
 
         def __contains__(self, k):
             return dict.__contains__(self, canon[k])

@@ -109,7 +109,8 @@ def test_random_graphs_execute(gpu, seed, grouping):
     permute instructions in the middle of a graph. With the reference's grouping rules the plan the library runs must
     be the one the CPU restatement of plan_generation.rs derives, and that plan - not the library's - tells the oracle
     where values are rounded to their storage type."""
-    from helium_amd.backend import OPT_FOLD_SWAP_INTO_REDUCE, OPT_FUSE_MATMUL_EPILOGUE, OPT_REMATERIALIZE, set_option
+    from helium_amd.backend import (OPT_CANCEL_TRANSPOSES, OPT_FOLD_SWAP_INTO_REDUCE, OPT_FUSE_MATMUL_EPILOGUE, OPT_REMATERIALIZE,
+                                    set_option)
     from oracle import plan as oracle_plan
 
     g = plans.random_graph(seed)
@@ -127,12 +128,14 @@ def test_random_graphs_execute(gpu, seed, grouping):
     set_option(OPT_FUSE_MATMUL_EPILOGUE, 0 if reference else 1)
     set_option(OPT_FOLD_SWAP_INTO_REDUCE, 0 if reference else 1)
     set_option(OPT_REMATERIALIZE, 0 if reference else 1)
+    set_option(OPT_CANCEL_TRANSPOSES, 0 if reference else 1)
     try:
         got, steps = run_graph(g, host)
     finally:
         set_option(OPT_FUSE_MATMUL_EPILOGUE, 1)
         set_option(OPT_FOLD_SWAP_INTO_REDUCE, 1)
         set_option(OPT_REMATERIALIZE, 1)
+        set_option(OPT_CANCEL_TRANSPOSES, 1)
     if reference:
         want_steps = oracle_plan.generate_plan(nodes)
         assert steps == want_steps

@@ -8,7 +8,8 @@ import numpy as np
 import pytest
 
 import helium_amd as ha
-from helium_amd.backend import OPT_FOLD_SWAP_INTO_REDUCE, OPT_FUSE_MATMUL_EPILOGUE, OPT_REMATERIALIZE, Plan, set_option, stats
+from helium_amd.backend import (OPT_CANCEL_TRANSPOSES, OPT_FOLD_SWAP_INTO_REDUCE, OPT_FUSE_MATMUL_EPILOGUE, OPT_REMATERIALIZE, Plan,
+                                set_option, stats)
 from oracle import plan as oracle_plan
 
 
@@ -16,14 +17,16 @@ from oracle import plan as oracle_plan
 def reference_grouping():
     """The reference's rules: a matmul instruction never fuses (cudnn_graph.rs:319-321), a SwapDims of more
     than 1M elements is always a permute instruction (cuda.rs:38-41), and the graph is planned as recorded (no value
-    is computed twice; a Constant is a kernel of its own, pointwise.rs:181)."""
+    is computed twice, every SwapDims stays; a Constant is a kernel of its own, pointwise.rs:181)."""
     set_option(OPT_FUSE_MATMUL_EPILOGUE, 0)
     set_option(OPT_FOLD_SWAP_INTO_REDUCE, 0)
     set_option(OPT_REMATERIALIZE, 0)
+    set_option(OPT_CANCEL_TRANSPOSES, 0)
     yield
     set_option(OPT_FUSE_MATMUL_EPILOGUE, 1)
     set_option(OPT_FOLD_SWAP_INTO_REDUCE, 1)
     set_option(OPT_REMATERIALIZE, 1)
+    set_option(OPT_CANCEL_TRANSPOSES, 1)
 
 
 def linear_layer():
