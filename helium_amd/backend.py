@@ -18,6 +18,7 @@ _ffi._sig("he_plan_generate", C.c_void_p, C.POINTER(C.c_void_p))
 _ffi._sig("he_plan_num_steps", C.c_void_p, C.POINTER(C.c_int))
 _ffi._sig("he_plan_describe", C.c_void_p, restype=C.c_char_p)
 _ffi._sig("he_plan_graph", C.c_void_p, C.POINTER(C.c_void_p))
+_ffi._sig("he_plan_describe_planned", C.c_void_p, restype=C.c_char_p)
 _ffi._sig("he_plan_destroy", C.c_void_p)
 _ffi._sig("he_plan_precompile", C.c_void_p)
 _ffi._sig("he_execute_graph", C.c_void_p, C.POINTER(C.c_uint32), C.POINTER(C.c_void_p), C.c_int, C.POINTER(C.c_uint32),
@@ -93,15 +94,24 @@ class Plan:
         self.handle = C.c_void_p()
         check(lib.he_plan_generate(graph.handle, C.byref(self.handle)))
         self.text = lib.he_plan_describe(self.handle).decode()
-        self.steps = []
-        for line in self.text.strip().split("\n"):
+        self.steps = self._parse(self.text)
+
+    def planned_steps(self):
+        """`steps` with the node ids of `graph()` instead of the planned graph's."""
+        return self._parse(lib.he_plan_describe_planned(self.handle).decode())
+
+    @staticmethod
+    def _parse(text):
+        steps = []
+        for line in text.strip().split("\n"):
             body, rel = line.split("|")
             instrs = []
             for tok in body.split(":", 1)[1].split():
                 kind, nodes = tok.split("{")
                 instrs.append((kind, [int(x) for x in nodes.rstrip("}").split(",") if x]))
             released = [int(x) for x in rel.replace("release", "").split()]
-            self.steps.append((instrs, released))
+            steps.append((instrs, released))
+        return steps
 
     def graph(self):
         """The graph the instructions are made of (he_plan_graph): the planned graph as the backend's rewrites left

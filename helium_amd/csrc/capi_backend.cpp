@@ -10,7 +10,7 @@ struct he_tensor_s {
 struct he_plan_s {
     std::shared_ptr<const he::plan::Plan> plan;
     std::shared_ptr<const he::ir::OpGraph> graph;
-    std::string text;
+    std::string text, text_planned;
 };
 
 static thread_local he::exec::ExecStats g_last_stats;
@@ -65,6 +65,7 @@ int he_plan_generate(he_graph_t graph, he_plan_t* plan) {
         p->graph = snapshot;
         p->plan = he::plan::generate_plan(snapshot);
         p->text = p->plan->describe();
+        p->text_planned = p->plan->describe(false);
         *plan = p.release();
     });
 }
@@ -80,6 +81,7 @@ int he_plan_num_steps(he_plan_t plan, int* steps) {
     return he::guard([&] { *steps = (int)plan->plan->steps.size(); });
 }
 const char* he_plan_describe(he_plan_t plan) { return plan ? plan->text.c_str() : ""; }
+const char* he_plan_describe_planned(he_plan_t plan) { return plan ? plan->text_planned.c_str() : ""; }
 int he_plan_precompile(he_plan_t plan) {
     return he::guard([&] {
         HE_REQUIRE(plan, HE_ERR_INVALID, "bad argument");

@@ -374,10 +374,11 @@ std::shared_ptr<OpGraph> rematerialized(const OpGraph& g, const std::set<NodeId>
     struct Info {
         bool cheap = false;          // an op that may be duplicated
         bool remat = false;          // ... and is, once per use by a kernel that can take it in
+        bool remat_for_reduction = false;  // ... or at least once per use by a kernel that only reduces it
         int cost = 0;
         std::vector<NodeId> anchors; // sorted, at most kMaxAnchors + 1 entries
     };
-    constexpr int kMaxCost = 24, kMaxCopies = 32;
+    constexpr int kMaxCost = 64, kMaxCopies = 32;
     constexpr int64_t kMinElements = 1 << 16;
     constexpr size_t kMaxAnchors = 1;
     std::vector<Info> info(cap);
@@ -418,14 +419,35 @@ std::shared_ptr<OpGraph> rematerialized(const OpGraph& g, const std::set<NodeId>
         for (NodeId a : I.anchors)
             if (num_elements(g.get(a).desc.shape) * 8 >= numel) kept.push_back(a);
         I.anchors = kept;
-        if (I.anchors.size() > kMaxAnchors + 1) I.anchors.resize(kMaxAnchors + 1);
+        if (I.anchors.size() > kMaxAnchors + 2) I.anchors.resize(kMaxAnchors + 2);
         I.cost = std::min(I.cost, kMaxCost + 1);
         // (a node with one consumer is copied as well when that consumer is: its copies' inputs must not meet in one
         // shared node, which would then have several consumers and travel through memory after all)
         I.remat = numel >= kMinElements && I.anchors.size() <= kMaxAnchors && I.cost <= kMaxCost && !keep_single.count(id);
-        any = any || (I.remat && users[id].size() > 1);
+        // A value that only reductions read (through transpositions and pointwise ops) may depend on one tensor more:
+        // written out and read back it moves as many bytes as its two operands do, and the reductions of one backward
+        // pass (a batch norm's four) then share one pass over those operands instead of reading a tensor each.
+        I.remat_for_reduction = numel >= kMinElements && I.anchors.size() <= kMaxAnchors + 1 && I.cost <= kMaxCost && !keep_single.count(id);
+        any = any || (I.remat && users[id].size() > 1) || (I.remat_for_reduction && !I.remat);
     }
     if (!any && !merged_any) return nullptr;
+    // nodes whose value ends in reductions only (a SwapDims and pointwise ops may lie in between)
+    std::vector<char> reduced_only(cap, 0);
+    {
+        std::vector<NodeId> order = g.nodes();
+        for (auto it = order.rbegin(); it != order.rend(); ++it) {
+            const NodeId id = *it;
+            if (canon[id] != id || g.get(id).kind != Node::Intermediate) continue;
+            if (g.get(id).op.kind == OpKind::Reduce) {
+                reduced_only[id] = 1;
+                continue;
+            }
+            if (!info[id].cheap && g.get(id).op.kind != OpKind::SwapDims) continue;
+            bool all = !users[id].empty();
+            for (NodeId u : users[id]) all = all && reduced_only[u];
+            reduced_only[id] = all;
+        }
+    }
 
     auto out = std::make_shared<OpGraph>();
     std::vector<NodeId> placed(cap, kNoNode);  // node of `g` -> its one node in `out` (what is not duplicated)
@@ -447,34 +469,43 @@ std::shared_ptr<OpGraph> rematerialized(const OpGraph& g, const std::set<NodeId>
             default: return true;
         }
     };
-    std::function<NodeId(NodeId, bool)> emit = [&](NodeId raw, bool for_fusing_consumer) -> NodeId {
+    // for_fusing_consumer: 0 a consumer that reads from memory, 1 one that can compute the value itself, 2 one that does
+    // and ends in reductions only
+    std::function<NodeId(NodeId, int)> emit = [&](NodeId raw, int for_fusing_consumer) -> NodeId {
         const NodeId id = canon[raw];
         const Node& n = g.get(id);
-        const bool dup = info[id].remat && for_fusing_consumer && copies[id] < kMaxCopies;
+        const bool dup = (info[id].remat || (for_fusing_consumer == 2 && info[id].remat_for_reduction)) && for_fusing_consumer && copies[id] < kMaxCopies;
         if (!dup && placed[id] != kNoNode) return placed[id];
         NodeId fresh;
         if (n.kind == Node::Input) {
             fresh = out->new_input(n.desc);
         } else {
             Op op = n.op;
-            const bool fusing = takes_producers_in(n);
+            // (a large SwapDims is a permute, which reads from memory, unless only reductions read it: then it is part
+            // of their kernel)
+            const int fusing = reduced_only[id] && (info[id].cheap || n.op.kind == OpKind::SwapDims) ? 2 : takes_producers_in(n) ? 1 : 0;
             for (NodeId& in : op.inputs) in = emit(in, fusing);
             fresh = out->new_op(std::move(op));
         }
         note_origin(fresh, id);
-        if (dup) copies[id]++;
-        else placed[id] = fresh;
+        if (dup) {
+            copies[id]++;
+            if (out->for_consumer_.size() <= fresh) out->for_consumer_.resize(fresh + 1, 0);
+            out->for_consumer_[fresh] = 1;
+        } else {
+            placed[id] = fresh;
+        }
         return fresh;
     };
     // inputs first, in their own order
-    for (NodeId id : g.inputs()) emit(id, false);
+    for (NodeId id : g.inputs()) emit(id, 0);
     for (NodeId id : g.nodes()) {
         const Node& n = g.get(id);
         if (n.kind == Node::Output) {
-            NodeId fresh = out->new_output(emit(g.inbound(id)[0], false));
+            NodeId fresh = out->new_output(emit(g.inbound(id)[0], 0));
             note_origin(fresh, id);
         } else if (n.kind == Node::Intermediate && canon[id] == id && !info[id].remat) {
-            emit(id, false);
+            emit(id, 0);
         }
     }
     out->optimize();
@@ -621,6 +652,8 @@ std::shared_ptr<OpGraph> transposes_cancelled(const OpGraph& g) {
                         if (padded[i] != 1) before.push_back((int64_t)i);
                         if (moved[i] != 1) after.push_back(p[i]);
                     }
+                    // (the nodes that bring the small source into shape stand for no node of `g`: the broadcast as recorded
+                    // reads the recorded source)
                     NodeId source = placed[n.op.inputs[0]];
                     if (before == after) {
                         if (moved != src) {
@@ -629,7 +662,7 @@ std::shared_ptr<OpGraph> transposes_cancelled(const OpGraph& g) {
                             r.inputs = {source};
                             r.shape = moved;
                             source = out->new_op(std::move(r));
-                            note_origin(source, node);
+                            note_origin(source, kNoNode);
                         }
                     } else {
                         if (padded != src) {
@@ -638,9 +671,9 @@ std::shared_ptr<OpGraph> transposes_cancelled(const OpGraph& g) {
                             r.inputs = {source};
                             r.shape = padded;
                             source = out->new_op(std::move(r));
-                            note_origin(source, node);
+                            note_origin(source, kNoNode);
                         }
-                        source = swapped(source, p, node);
+                        source = swapped(source, p, kNoNode);
                     }
                     Op op = n.op;
                     op.inputs = {source};

@@ -110,11 +110,14 @@ public:
     static Shape broadcast_output_shape(const Op& op, const Shape& in);
 
     // For a graph that `rematerialized` built: the node of the graph it was built from that a node stands for (several
-    // nodes may stand for the same one); the node itself in any other graph.
+    // nodes may stand for the same one; kNoNode for a helper node that stands for none); the node itself in any other graph.
     NodeId origin(NodeId id) const { return id < origin_.size() ? origin_[id] : id; }
     bool has_origins() const { return !origin_.empty(); }
     // When the graph this one was built from was itself built from another: origins then name that one's nodes.
     void rebase_origins(const OpGraph& through);
+    // For a graph that `rematerialized` built: whether the node is a copy made for one consumer, to be computed in that
+    // consumer's kernel. A kernel that would write such a copy to memory has the wrong one.
+    bool made_for_consumer(NodeId id) const { return id < for_consumer_.size() && for_consumer_[id]; }
 
 private:
     NodeId push(Node n);
@@ -122,6 +125,7 @@ private:
     std::vector<NodeId> inputs_, outputs_;
     std::vector<std::vector<NodeId>> in_, out_;
     std::vector<NodeId> origin_;
+    std::vector<uint8_t> for_consumer_;
     friend std::shared_ptr<OpGraph> rematerialized(const OpGraph& g, const std::set<NodeId>& keep_single);
     friend std::shared_ptr<OpGraph> transposes_cancelled(const OpGraph& g);
 };

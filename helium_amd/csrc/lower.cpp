@@ -7,6 +7,7 @@
 
 namespace he::plan {
 bool rematerialize();
+bool feeds_only_reductions(const ir::OpGraph& g, ir::NodeId node, int budget);
 }
 namespace he::tp {
 
@@ -819,7 +820,9 @@ bool pointwise_supports(const ir::OpSubgraph& sg) {
             case ir::OpKind::Broadcast: x += 1; break;
             case ir::OpKind::SwapDims:
                 x += 1;
-                if (x > 1) return false;
+                // (the generator here walks any number of broadcasts and transpositions as strides; the count is the
+                // reference's, kept when graphs are planned as recorded)
+                if (x > 1 && !plan::rematerialize()) return false;
                 break;
             case ir::OpKind::Reduce: {
                 if (!sg.is_leaf(node)) return false;
@@ -846,6 +849,28 @@ bool pointwise_supports(const ir::OpSubgraph& sg) {
                 continue;
             default: return false;
         }
+    }
+    // A kernel iterates over one shape: that of its first output, or the input shape of its reductions. Outputs of
+    // another shape (the transposed tensor next to the untransposed one) are then written element by element in an
+    // order that shares nothing with what the others read, which a large tensor cannot afford: they stay in a kernel
+    // of their own. (The reference's rule compares element counts only.)
+    // A transposition inside a large kernel is there for reductions over leading dims, which walk the untransposed
+    // tensor in memory order when every output of the kernel is such a reduction; any other output next to them (the
+    // transposed tensor itself, or a tensor of the same extents in another order - a batch as large as the channel
+    // count makes the two shapes equal) would be written element by element.
+    if (plan::rematerialize() && output_size >= fold_columns_threshold()) {
+        const Shape* shape = nullptr;
+        bool transposes = false, only_reductions = true;
+        for (ir::NodeId node : sg.nodes()) transposes = transposes || g.get(node).op.kind == ir::OpKind::SwapDims;
+        for (ir::NodeId node : sg.leafs()) {
+            const ir::Op& op = g.get(node).op;
+            // (an output on its way to reductions that have not joined yet is let through: instructions fuse in pairs)
+            only_reductions = only_reductions && (op.kind == ir::OpKind::Reduce || plan::feeds_only_reductions(g, node, 64));
+            const Shape& mine = g.get(op.kind == ir::OpKind::Reduce ? op.inputs[0] : node).desc.shape;
+            if (shape && *shape != mine) return false;
+            shape = &mine;
+        }
+        if (transposes && !only_reductions && sg.nodes().size() > 1) return false;
     }
     return true;
 }

@@ -49,9 +49,10 @@ std::atomic<bool> g_fold_swap_into_reduce{true};
 std::atomic<bool> g_rematerialize{true};
 std::atomic<bool> g_cancel_transposes{true};
 
+}  // namespace
 // True when every value computed from `node` inside the graph ends in a Reduce, through pointwise ops only: nothing
 // then needs the transposed tensor in memory.
-bool feeds_only_reductions(const ir::OpGraph& g, NodeId node, int budget = 64) {
+bool feeds_only_reductions(const ir::OpGraph& g, NodeId node, int budget) {
     const auto& users = g.outbound(node);
     if (users.empty() || budget <= 0) return false;
     for (NodeId u : users) {
@@ -71,7 +72,6 @@ bool feeds_only_reductions(const ir::OpGraph& g, NodeId node, int budget = 64) {
     }
     return true;
 }
-}  // namespace
 void set_fuse_matmul_epilogue(bool on) { g_fuse_matmul_epilogue.store(on); }
 bool fuse_matmul_epilogue() { return g_fuse_matmul_epilogue.load(); }
 unsigned option_mask() {
@@ -94,7 +94,13 @@ bool Instr::can_fuse_with(const Instr& next) const {
         // join it when they can run on the accumulators as the fused GEMM's epilogue; so do the ops that only prepare
         // epilogue operands (a bias broadcast), whichever of the two the greedy pass visits first.
         try {
-            (void)gemm_problem_from_ir(sg_.merge_with(next.sg_));
+            const ir::OpSubgraph merged = sg_.merge_with(next.sg_);
+            // A value that was copied so that its consumer computes it is not to become an output of the product (the
+            // greedy pass visits the copy next to its producer first): it waits for its consumer, and the product is
+            // offered the finished group again.
+            for (NodeId leaf : merged.leafs())
+                if (merged.graph()->made_for_consumer(leaf)) return false;
+            (void)gemm_problem_from_ir(merged);
             return true;
         } catch (const Error&) {
             return false;
@@ -219,11 +225,17 @@ void Instr::execute(const std::function<void*(NodeId)>& storage, hipStream_t str
     kernel_->execute(ptrs.data(), stream);
 }
 
-std::string Instr::describe() const {
+std::string Instr::describe(bool origins) const {
     std::ostringstream s;
     s << (kind_ == InstrKind::Gemm ? "gemm" : kind_ == InstrKind::Pointwise ? "pointwise" : "permute") << "{";
     // (a rematerialised graph's nodes are named by the nodes they stand for)
-    for (size_t i = 0; i < sg_.nodes().size(); i++) s << (i ? "," : "") << sg_.graph()->origin(sg_.nodes()[i]);
+    bool first = true;
+    for (NodeId node : sg_.nodes()) {
+        const NodeId name = origins ? sg_.graph()->origin(node) : node;
+        if (name == ir::kNoNode) continue;  // a node a rewrite added that stands for none of the planned graph's
+        s << (first ? "" : ",") << name;
+        first = false;
+    }
     s << "}";
     return s.str();
 }
@@ -328,7 +340,8 @@ std::shared_ptr<const Plan> generate_plan(const std::shared_ptr<const ir::OpGrap
         if (g->get(n).kind == ir::Node::Intermediate) ig.insert(std::make_shared<Instr>(make_instr_for_op(g, n)));
 
     // do_fusions (:243-256)
-    {
+    auto do_fusions = [&] {
+        bool fused = false;
         std::set<uint64_t> work;
         for (auto& kv : ig.instrs) work.insert(kv.first);
         while (!work.empty()) {
@@ -340,9 +353,16 @@ std::shared_ptr<const Plan> generate_plan(const std::shared_ptr<const ir::OpGrap
                     uint64_t merged = ig.fuse(cur, nxt);
                     work.erase(nxt);
                     work.insert(merged);
+                    fused = true;
                     break;
                 }
         }
+        return fused;
+    };
+    // The reference makes one pass: an instruction whose dependents all refuse it is not looked at again. Here a
+    // dependent may become acceptable later (a transposition joins its reduction, and only then the ops before it
+    // can follow), so when the graph is not planned as recorded the pass is repeated until nothing fuses.
+    while (do_fusions() && rematerialize()) {
     }
 
     // Beyond the reference, with the epilogue option on: the greedy pass visits a product before the pointwise group
@@ -447,16 +467,17 @@ std::shared_ptr<const Plan> generate_plan(const std::shared_ptr<const ir::OpGrap
     return plan;
 }
 
-std::string Plan::describe() const {
+std::string Plan::describe(bool origins) const {
     std::ostringstream s;
     const ir::OpGraph* g = nullptr;
     for (auto& st : steps)
         for (auto& instr : st.instrs) g = instr->subgraph().graph().get();
     for (size_t i = 0; i < steps.size(); i++) {
         s << "step " << i << ":";
-        for (auto& instr : steps[i].instrs) s << " " << instr->describe();
+        for (auto& instr : steps[i].instrs) s << " " << instr->describe(origins);
         s << " | release";
-        for (NodeId t : steps[i].tensors_to_release) s << " " << (g ? g->origin(t) : t);
+        for (NodeId t : steps[i].tensors_to_release)
+            if (!(g && origins) || g->origin(t) != ir::kNoNode) s << " " << (g && origins ? g->origin(t) : t);
         s << "\n";
     }
     return s.str();
@@ -503,24 +524,19 @@ std::shared_ptr<const ir::OpGraph> graph_for_execution(const std::shared_ptr<con
             other = ir::rematerialized(*base, keep_single);
         }
     }
-    std::shared_ptr<const ir::OpGraph> chosen = base;
-    if (other) {
-        if (base != g) other->rebase_origins(*base);
-        chosen = other;
+    // A rewritten graph is taken only when its plan moves fewer bytes - or as many, where transpositions went: the
+    // kernels then walk their tensors in memory order.
+    if (base != g && plan_traffic_bytes(*generate_cached_plan(base)) > plan_traffic_bytes(*generate_cached_plan(g))) {
+        base = g;
+        other = rematerialize() ? ir::rematerialized(*g) : nullptr;  // (without the rounds above: the rare case)
     }
-    if (chosen == g) return g;
-    // ... and a rewritten graph is taken only when its plan moves fewer bytes.
-    const int64_t before = plan_traffic_bytes(*generate_cached_plan(g));
-    int64_t after = plan_traffic_bytes(*generate_cached_plan(chosen));
-    if (chosen != base && base != g) {
-        const int64_t without_copies = plan_traffic_bytes(*generate_cached_plan(base));
-        if (without_copies <= after) {
-            chosen = base;
-            after = without_copies;
-        }
-    }
-    if (debug) fprintf(stderr, "[plan] bytes moved by the plan: %lld as recorded, %lld rewritten\n", (long long)before, (long long)after);
-    return after < before ? chosen : g;
+    if (debug) fprintf(stderr, "[plan] bytes moved by the plan: %lld as recorded, %lld without the transpositions\n",
+                       (long long)plan_traffic_bytes(*generate_cached_plan(g)), (long long)plan_traffic_bytes(*generate_cached_plan(base)));
+    if (!other) return base;
+    if (base != g) other->rebase_origins(*base);
+    const int64_t before = plan_traffic_bytes(*generate_cached_plan(base)), after = plan_traffic_bytes(*generate_cached_plan(other));
+    if (debug) fprintf(stderr, "[plan] ... %lld with cheap values computed where they are used\n", (long long)after);
+    return after < before ? std::shared_ptr<const ir::OpGraph>(other) : base;
 }
 
 // ---------------------------------------------------------------------------------------------------------

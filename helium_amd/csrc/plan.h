@@ -40,7 +40,7 @@ public:
     }
     // execute (instr.rs:27-42): `storage(node)` returns the device address of a tensor.
     void execute(const std::function<void*(NodeId)>& storage, hipStream_t stream) const;
-    std::string describe() const;
+    std::string describe(bool origins = true) const;  // origins: name nodes by OpGraph::origin
 
 private:
     InstrKind kind_;
@@ -62,7 +62,7 @@ struct Step {
 };
 struct Plan {
     std::vector<Step> steps;
-    std::string describe() const;  // one line per step: instruction kinds, node sets, releases
+    std::string describe(bool origins = true) const;  // one line per step: instruction kinds, node sets, releases
 };
 
 // Whether pointwise / reduce ops downstream of a Matmul may join its instruction (on by default). Off gives the
@@ -82,6 +82,8 @@ bool rematerialize();
 // Whether transpositions that undo each other are taken out of the graph first (ir::transposes_cancelled; on by default).
 void set_cancel_transposes(bool on);
 bool cancel_transposes();
+// True when every value computed from `node` ends in a Reduce, through pointwise ops only.
+bool feeds_only_reductions(const ir::OpGraph& g, ir::NodeId node, int budget = 64);
 // Bytes the plan's kernels read and write: the sizes of every instruction's inputs and outputs.
 int64_t plan_traffic_bytes(const Plan& plan);
 // The graph the backend plans and runs for `g` (already pruned): `g` itself, or the form the two rewrites above give it

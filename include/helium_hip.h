@@ -309,6 +309,8 @@ int he_plan_graph(he_plan_t plan, he_graph_t* graph);
 int he_plan_num_steps(he_plan_t plan, int* steps);
 /* One line per step: "step i: kind{node,node,...} ... | release node ...". */
 const char* he_plan_describe(he_plan_t plan);
+/* The same text with the node ids of the graph he_plan_graph returns. */
+const char* he_plan_describe_planned(he_plan_t plan);
 /* Compiles the kernels of every instruction of the plan, in parallel, into the kernel caches: what begin_execute does
  * on first sight of a plan (cuda.rs:98-139, parallel_compile_kernels :262-270). Needs no device. */
 int he_plan_precompile(he_plan_t plan);

@@ -397,10 +397,32 @@ def plan_outputs(nodes, inputs, plan_steps):
         def __setitem__(self, k, v):
             dict.__setitem__(self, canon[k], v)
 
-    consumers = {}
+    # What a kernel writes to memory: the members that another kernel (or an Output) reads without computing them
+    # itself. A shape op that no kernel holds is read through, so the need passes on to its operand.
+    computed = {canon[m] for instrs, _ in plan_steps for _, members in instrs for m in members}
+    needed = set()
+
+    def need(i, inside):
+        i = canon[i]
+        if i in inside or by_id[i]["node"] == "input":
+            return
+        if i in computed:
+            needed.add(i)
+        else:
+            assert by_id[i].get("op") in ("swap_dims", "reshape", "broadcast"), ("no kernel computes", by_id[i])
+            for j in by_id[i]["inputs"]:
+                need(j, inside)
+
+    for instrs, _ in plan_steps:
+        for _, members in instrs:
+            inside = {canon[m] for m in members}
+            for m in members:
+                for j in by_id[m]["inputs"]:
+                    need(j, inside)
     for n in nodes:
-        for p in (n.get("inputs") or ([n["from"]] if n["node"] == "output" else [])):
-            consumers.setdefault(canon[p], []).append(canon[n["id"]])
+        if n["node"] == "output":
+            need(n["from"], set())
+
     desc, stored = {}, _Through()
     for n in nodes:  # descriptors of everything; values of the inputs
         i = n["id"]
@@ -418,9 +440,8 @@ def plan_outputs(nodes, inputs, plan_steps):
             for m in sorted(inside):
                 local[m] = _eval_op(by_id[m], desc, local)
                 assert list(local[m].shape) == list(desc[m][0]), (by_id[m], local[m].shape)
-            inside_canon = {canon[m] for m in inside}
             for m in inside:
-                if any(c not in inside_canon for c in consumers.get(canon[m], [])):
+                if canon[m] in needed:
                     shape, dtype = desc[m]
                     stored[m] = nm.from_storage(nm.to_storage(local[m], dtype), dtype, shape)
     return {n["id"]: nm.to_storage(stored[n["from"]], desc[n["id"]][1]) for n in nodes if n["node"] == "output"}

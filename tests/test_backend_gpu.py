@@ -169,15 +169,20 @@ def test_random_graphs_cover_concurrent_steps_and_permute_instructions():
 
 @pytest.mark.parametrize("fuse", [1, 0], ids=["matmul_takes_its_epilogue", "reference_grouping"])
 def test_config1_linear_layer(gpu, fuse):
-    from helium_amd.backend import OPT_FUSE_MATMUL_EPILOGUE, set_option
+    from helium_amd.backend import (OPT_CANCEL_TRANSPOSES, OPT_FOLD_SWAP_INTO_REDUCE, OPT_FUSE_MATMUL_EPILOGUE, OPT_REMATERIALIZE,
+                                    set_option)
 
     g, names = configs.c1_ir_graph()
     host = configs.c1_inputs(names, batched=False)
-    set_option(OPT_FUSE_MATMUL_EPILOGUE, fuse)
+    options = (OPT_FUSE_MATMUL_EPILOGUE, OPT_FOLD_SWAP_INTO_REDUCE, OPT_REMATERIALIZE, OPT_CANCEL_TRANSPOSES)
+    for option in options:
+        set_option(option, fuse)
     try:
         got, steps = run_graph(g, host)
     finally:
-        set_option(OPT_FUSE_MATMUL_EPILOGUE, 1)
+        for option in options:
+            set_option(option, 1)
+    # (the reference's rule keeps the column sums' SwapDims out of the kernel that broadcasts the bias, pointwise.rs:150-160)
     assert [k for instrs, _ in steps for k, _ in instrs] == (["gemm"] if fuse else ["gemm", "pointwise", "pointwise"])
     val, _ = oracle_ir.evaluate(g.nodes, host)
     y = got[names["y"]].reshape(256, 512).astype(np.float64)

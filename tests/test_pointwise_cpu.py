@@ -38,8 +38,9 @@ def test_generated_kernel_on_cpu_matches_oracle(case, monkeypatch):
         assert ha.kernels.pointwise_supports(case.g, case.nodes) == (case.admitted_by_fusion_rule and not has_constant), case.name
     finally:
         set_option(OPT_REMATERIALIZE, 1)
-    # ... and an immediate of the kernel that uses it when values may be computed where they are used
-    assert ha.kernels.pointwise_supports(case.g, case.nodes) == case.admitted_by_fusion_rule, case.name
+    # ... and an immediate of the kernel that uses it when values may be computed where they are used; the count of
+    # broadcasts and transpositions (pointwise.rs:150-160) is then not applied either: the generator walks them all
+    assert ha.kernels.pointwise_supports(case.g, case.nodes), case.name
     kernel = ha.TileKernel.pointwise(case.g, case.nodes)
     assert [a["node"] for a in kernel.args if a["is_output"]] == sorted(case.leaves)
     want = oracle_ir.kernel_outputs(case.g.nodes, case.inputs, case.leaves)
