@@ -29,6 +29,7 @@ OPT_FUSE_MATMUL_EPILOGUE = 0
 OPT_FOLD_SWAP_INTO_REDUCE = 1
 OPT_REMATERIALIZE = 2
 OPT_CANCEL_TRANSPOSES = 3
+OPT_HOIST_BROADCASTS = 4
 
 
 def set_option(option, value):

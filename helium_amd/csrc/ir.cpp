@@ -783,6 +783,108 @@ std::shared_ptr<OpGraph> transposes_cancelled(const OpGraph& g) {
     return out;
 }
 
+std::shared_ptr<OpGraph> broadcasts_hoisted(const OpGraph& g) {
+    const size_t cap = g.capacity();
+    auto out = std::make_shared<OpGraph>();
+    std::vector<NodeId> placed(cap, kNoNode);
+    auto note_origin = [&](NodeId fresh, NodeId old) {
+        if (out->origin_.size() <= fresh) out->origin_.resize(fresh + 1, kNoNode);
+        out->origin_[fresh] = old;
+    };
+    // a Broadcast of `out` that only repeats its source: the source's extents at the listed axes are 1
+    auto plain_broadcast = [&](NodeId id, Shape* padded) {
+        const Node& n = out->get(id);
+        if (n.kind != Node::Intermediate || n.op.kind != OpKind::Broadcast) return false;
+        *padded = out->get(n.op.inputs[0]).desc.shape;
+        while ((int64_t)padded->size() < n.op.new_dim_count) padded->insert(padded->begin(), 1);
+        for (auto& a : n.op.broadcast_axes)
+            if ((*padded)[a.axis] != 1) return false;
+        return num_elements(*padded) < num_elements(n.desc.shape);
+    };
+    bool changed = false;
+    for (NodeId id : g.inputs()) {
+        placed[id] = out->new_input(g.get(id).desc);
+        note_origin(placed[id], id);
+    }
+    for (NodeId id : g.nodes()) {
+        const Node& n = g.get(id);
+        if (n.kind == Node::Input) continue;
+        if (n.kind == Node::Output) {
+            placed[id] = out->new_output(placed[g.inbound(id)[0]]);
+            note_origin(placed[id], id);
+            continue;
+        }
+        Op op = n.op;
+        for (NodeId& in : op.inputs) in = placed[in];
+        bool pointwise = false;
+        switch (op.kind) {
+            case OpKind::UnaryPointwise:
+            case OpKind::BinaryPointwise:
+            case OpKind::ChangeDataType:
+            case OpKind::Compare:
+            case OpKind::Select: pointwise = true; break;
+            default: break;
+        }
+        // every operand the same broadcast of a small tensor, or a constant: the op is applied before the broadcast
+        const Op* pattern = nullptr;
+        Shape small;
+        bool hoist = pointwise;
+        for (size_t i = 0; i < op.inputs.size() && hoist; i++) {
+            const Node& in = out->get(op.inputs[i]);
+            if (in.kind == Node::Intermediate && in.op.kind == OpKind::Constant) continue;
+            Shape padded;
+            if (!plain_broadcast(op.inputs[i], &padded)) {
+                hoist = false;
+            } else if (!pattern) {
+                pattern = &in.op;
+                small = padded;
+            } else {
+                hoist = padded == small && in.op.new_dim_count == pattern->new_dim_count && in.op.broadcast_axes == pattern->broadcast_axes;
+            }
+        }
+        if (hoist && pattern) {
+            const Op broadcast = *pattern;  // (a copy: new nodes move the node table)
+            Op inner = op;
+            for (NodeId& in : inner.inputs) {
+                const Node src = out->get(in);
+                // (the constants and reshapes made here stand for no node of `g`)
+                if (src.op.kind == OpKind::Constant) {
+                    Op c = src.op;
+                    c.shape = small;
+                    in = out->new_op(std::move(c));
+                    note_origin(in, kNoNode);
+                } else {
+                    in = src.op.inputs[0];
+                    if (out->get(in).desc.shape != small) {
+                        Op r;
+                        r.kind = OpKind::Reshape;
+                        r.inputs = {in};
+                        r.shape = small;
+                        in = out->new_op(std::move(r));
+                        note_origin(in, kNoNode);
+                    }
+                }
+            }
+            const NodeId computed = out->new_op(std::move(inner));
+            note_origin(computed, id);
+            Op again = broadcast;
+            again.inputs = {computed};
+            placed[id] = out->new_op(std::move(again));
+            // (the broadcast stands for no node of `g`: whoever evaluates the plan on `g` reads `id` from memory there)
+            note_origin(placed[id], kNoNode);
+            if (out->get(placed[id]).desc == n.desc) {
+                changed = true;
+                continue;
+            }
+        }
+        placed[id] = out->new_op(std::move(op));
+        note_origin(placed[id], id);
+    }
+    if (!changed) return nullptr;
+    out->optimize();
+    return out;
+}
+
 void OpGraph::rebase_origins(const OpGraph& through) {
     for (NodeId& o : origin_)
         if (o != kNoNode) o = through.origin(o);

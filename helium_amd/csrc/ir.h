@@ -128,6 +128,7 @@ private:
     std::vector<uint8_t> for_consumer_;
     friend std::shared_ptr<OpGraph> rematerialized(const OpGraph& g, const std::set<NodeId>& keep_single);
     friend std::shared_ptr<OpGraph> transposes_cancelled(const OpGraph& g);
+    friend std::shared_ptr<OpGraph> broadcasts_hoisted(const OpGraph& g);
 };
 
 // A copy of `g` in which values that are cheap to compute again are computed once per use instead of once: every
@@ -152,6 +153,12 @@ std::shared_ptr<OpGraph> rematerialized(const OpGraph& g, const std::set<NodeId>
 // reduces the same dims (their order does not matter to a Sum / Mean / Min / Max beyond rounding). Node ids are new;
 // `origin` names the node of `g` whose value, possibly transposed, a node computes. Returns null when nothing changes.
 std::shared_ptr<OpGraph> transposes_cancelled(const OpGraph& g);
+
+// A copy of `g` in which a pointwise op whose operands all are the same broadcast of small tensors (or constants) is
+// applied to the small tensors, and its result broadcast: the front end writes `(variance.broadcast_to(x.shape) +
+// 1e-3).sqrt()` (batch_norm.rs:56), a square root per element of x where one per channel does. Element by element the
+// values are the same. Node ids are new; `origin` as above. Returns null when nothing changes.
+std::shared_ptr<OpGraph> broadcasts_hoisted(const OpGraph& g);
 
 // Subset of an OpGraph (opgraph/subgraph.rs): nodes sorted by id; `inputs` = outside producers feeding it,
 // `roots` = members with an outside input, `leafs` = members with an outside consumer.

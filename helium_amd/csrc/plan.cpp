@@ -48,6 +48,7 @@ std::atomic<bool> g_fuse_matmul_epilogue{true};
 std::atomic<bool> g_fold_swap_into_reduce{true};
 std::atomic<bool> g_rematerialize{true};
 std::atomic<bool> g_cancel_transposes{true};
+std::atomic<bool> g_hoist_broadcasts{true};
 
 }  // namespace
 // True when every value computed from `node` inside the graph ends in a Reduce, through pointwise ops only: nothing
@@ -76,13 +77,15 @@ void set_fuse_matmul_epilogue(bool on) { g_fuse_matmul_epilogue.store(on); }
 bool fuse_matmul_epilogue() { return g_fuse_matmul_epilogue.load(); }
 unsigned option_mask() {
     // the hash of the tuning overrides (0 unless tuning is on) rides along: plans keep their kernels
-    return (fuse_matmul_epilogue() ? 1u : 0u) | (g_fold_swap_into_reduce.load() ? 2u : 0u) | (g_rematerialize.load() ? 4u : 0u) | (g_cancel_transposes.load() ? 8u : 0u) | (tuning::hash() << 4);
+    return (fuse_matmul_epilogue() ? 1u : 0u) | (g_fold_swap_into_reduce.load() ? 2u : 0u) | (g_rematerialize.load() ? 4u : 0u) | (g_cancel_transposes.load() ? 8u : 0u) | (g_hoist_broadcasts.load() ? 16u : 0u) | (tuning::hash() << 5);
 }
 void set_fold_swap_into_reduce(bool on) { g_fold_swap_into_reduce.store(on); }
 void set_rematerialize(bool on) { g_rematerialize.store(on); }
 bool rematerialize() { return g_rematerialize.load(); }
 void set_cancel_transposes(bool on) { g_cancel_transposes.store(on); }
 bool cancel_transposes() { return g_cancel_transposes.load(); }
+void set_hoist_broadcasts(bool on) { g_hoist_broadcasts.store(on); }
+bool hoist_broadcasts() { return g_hoist_broadcasts.load(); }
 bool fold_swap_into_reduce() { return g_fold_swap_into_reduce.load(); }
 
 bool Instr::can_fuse_with(const Instr& next) const {
@@ -502,6 +505,13 @@ std::shared_ptr<const ir::OpGraph> graph_for_execution(const std::shared_ptr<con
         if (auto untransposed = ir::transposes_cancelled(*g)) {
             if (debug) fprintf(stderr, "[plan] transpositions cancelled: %zu -> %zu nodes\n", g->num_nodes(), untransposed->num_nodes());
             base = untransposed;
+        }
+    // ... and pointwise ops on broadcasts alone are applied before the broadcast
+    if (hoist_broadcasts())
+        if (auto hoisted = ir::broadcasts_hoisted(*base)) {
+            if (debug) fprintf(stderr, "[plan] broadcasts hoisted: %zu -> %zu nodes\n", base->num_nodes(), hoisted->num_nodes());
+            if (base != g) hoisted->rebase_origins(*base);
+            base = hoisted;
         }
     // 2. cheap values are computed where they are used
     std::shared_ptr<ir::OpGraph> other = rematerialize() ? ir::rematerialized(*base) : nullptr;

@@ -82,6 +82,9 @@ bool rematerialize();
 // Whether transpositions that undo each other are taken out of the graph first (ir::transposes_cancelled; on by default).
 void set_cancel_transposes(bool on);
 bool cancel_transposes();
+// Whether pointwise ops whose operands are all one broadcast are applied before it (ir::broadcasts_hoisted; on by default).
+void set_hoist_broadcasts(bool on);
+bool hoist_broadcasts();
 // True when every value computed from `node` ends in a Reduce, through pointwise ops only.
 bool feeds_only_reductions(const ir::OpGraph& g, ir::NodeId node, int budget = 64);
 // Bytes the plan's kernels read and write: the sizes of every instruction's inputs and outputs.

@@ -383,8 +383,13 @@ int he_fgraph_subdivide(he_fgraph_t graph, uint64_t* nodes, int32_t* portions, i
  * between the two run in the layout the tensors have in memory; the chain of SwapDims in front of a Reduce becomes the
  * shortest chain that reduces the same dims. The backward pass of a reduction over leading dims (tensor.rs answers a
  * SwapDims with a SwapDims) otherwise transposes a full-size tensor twice. Applied before HE_OPT_REMATERIALIZE, under
- * the same condition (fewer bytes moved by the plan); 0 keeps every SwapDims as recorded. */
-enum { HE_OPT_FUSE_MATMUL_EPILOGUE = 0, HE_OPT_FOLD_SWAP_INTO_REDUCE = 1, HE_OPT_REMATERIALIZE = 2, HE_OPT_CANCEL_TRANSPOSES = 3 };
+ * the same condition (no more bytes moved by the plan); 0 keeps every SwapDims as recorded.
+ * HE_OPT_HOIST_BROADCASTS (default 1): a pointwise op whose operands all are the same Broadcast of small tensors (or
+ * Constants) is applied to the small tensors and its result broadcast - `(variance.broadcast_to(x.shape) + 1e-3).sqrt()`
+ * (modules/batch_norm.rs:56) costs one square root per channel instead of one per element. 0 keeps the ops where they
+ * were recorded. */
+enum { HE_OPT_FUSE_MATMUL_EPILOGUE = 0, HE_OPT_FOLD_SWAP_INTO_REDUCE = 1, HE_OPT_REMATERIALIZE = 2, HE_OPT_CANCEL_TRANSPOSES = 3,
+       HE_OPT_HOIST_BROADCASTS = 4 };
 int he_backend_set_option(int option, int64_t value);
 
 /* Counters of the last he_execute_graph on this thread: [0] steps run, [1] instructions, [2] streams used,

@@ -389,6 +389,9 @@ def plan_outputs(nodes, inputs, plan_steps):
                 # values, so they are read through, from whatever holds their operand.
                 # (not kept: a later kernel may compute the operand afresh, and must then see its own copy)
                 return _eval_op(by_id[k], desc, self)
+            if not dict.__contains__(self, k) and k in unnamed:
+                shape, dtype = desc[k]
+                return nm.from_storage(nm.to_storage(_eval_op(by_id[k], desc, stored), dtype), dtype, shape)
             return dict.__getitem__(self, k)
 
         def __contains__(self, k):
@@ -400,7 +403,7 @@ def plan_outputs(nodes, inputs, plan_steps):
     # What a kernel writes to memory: the members that another kernel (or an Output) reads without computing them
     # itself. A shape op that no kernel holds is read through, so the need passes on to its operand.
     computed = {canon[m] for instrs, _ in plan_steps for _, members in instrs for m in members}
-    needed = set()
+    needed, unnamed = set(), set()
 
     def need(i, inside):
         i = canon[i]
@@ -409,9 +412,13 @@ def plan_outputs(nodes, inputs, plan_steps):
         if i in computed:
             needed.add(i)
         else:
-            assert by_id[i].get("op") in ("swap_dims", "reshape", "broadcast"), ("no kernel computes", by_id[i])
+            # A shape op that no kernel holds is read through. So is, rounded to its storage type, any other op that no
+            # kernel names: a rewrite of the plan's may have merged it with an op that computes the same values from
+            # other nodes (the op applied before a broadcast instead of after it) and names only that one.
+            if by_id[i].get("op") not in ("swap_dims", "reshape", "broadcast"):
+                unnamed.add(i)
             for j in by_id[i]["inputs"]:
-                need(j, inside)
+                need(j, set())
 
     for instrs, _ in plan_steps:
         for _, members in instrs:

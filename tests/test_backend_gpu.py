@@ -109,7 +109,8 @@ def test_random_graphs_execute(gpu, seed, grouping):
     permute instructions in the middle of a graph. With the reference's grouping rules the plan the library runs must
     be the one the CPU restatement of plan_generation.rs derives, and that plan - not the library's - tells the oracle
     where values are rounded to their storage type."""
-    from helium_amd.backend import (OPT_CANCEL_TRANSPOSES, OPT_FOLD_SWAP_INTO_REDUCE, OPT_FUSE_MATMUL_EPILOGUE, OPT_REMATERIALIZE,
+    from helium_amd.backend import (OPT_CANCEL_TRANSPOSES, OPT_FOLD_SWAP_INTO_REDUCE, OPT_FUSE_MATMUL_EPILOGUE, OPT_HOIST_BROADCASTS,
+                                OPT_REMATERIALIZE,
                                     set_option)
     from oracle import plan as oracle_plan
 
@@ -129,6 +130,7 @@ def test_random_graphs_execute(gpu, seed, grouping):
     set_option(OPT_FOLD_SWAP_INTO_REDUCE, 0 if reference else 1)
     set_option(OPT_REMATERIALIZE, 0 if reference else 1)
     set_option(OPT_CANCEL_TRANSPOSES, 0 if reference else 1)
+    set_option(OPT_HOIST_BROADCASTS, 0 if reference else 1)
     try:
         got, steps = run_graph(g, host)
     finally:
@@ -136,6 +138,8 @@ def test_random_graphs_execute(gpu, seed, grouping):
         set_option(OPT_FOLD_SWAP_INTO_REDUCE, 1)
         set_option(OPT_REMATERIALIZE, 1)
         set_option(OPT_CANCEL_TRANSPOSES, 1)
+        set_option(OPT_HOIST_BROADCASTS, 1)
+    set_option(OPT_HOIST_BROADCASTS, 1)
     if reference:
         want_steps = oracle_plan.generate_plan(nodes)
         assert steps == want_steps
@@ -169,12 +173,13 @@ def test_random_graphs_cover_concurrent_steps_and_permute_instructions():
 
 @pytest.mark.parametrize("fuse", [1, 0], ids=["matmul_takes_its_epilogue", "reference_grouping"])
 def test_config1_linear_layer(gpu, fuse):
-    from helium_amd.backend import (OPT_CANCEL_TRANSPOSES, OPT_FOLD_SWAP_INTO_REDUCE, OPT_FUSE_MATMUL_EPILOGUE, OPT_REMATERIALIZE,
+    from helium_amd.backend import (OPT_CANCEL_TRANSPOSES, OPT_FOLD_SWAP_INTO_REDUCE, OPT_FUSE_MATMUL_EPILOGUE, OPT_HOIST_BROADCASTS,
+                                OPT_REMATERIALIZE,
                                     set_option)
 
     g, names = configs.c1_ir_graph()
     host = configs.c1_inputs(names, batched=False)
-    options = (OPT_FUSE_MATMUL_EPILOGUE, OPT_FOLD_SWAP_INTO_REDUCE, OPT_REMATERIALIZE, OPT_CANCEL_TRANSPOSES)
+    options = (OPT_FUSE_MATMUL_EPILOGUE, OPT_FOLD_SWAP_INTO_REDUCE, OPT_REMATERIALIZE, OPT_CANCEL_TRANSPOSES, OPT_HOIST_BROADCASTS)
     for option in options:
         set_option(option, fuse)
     try:

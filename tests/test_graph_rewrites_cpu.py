@@ -1,4 +1,4 @@
-"""The two rewrites a graph goes through before it is planned (ir.cpp: transposes_cancelled, rematerialized), checked on
+"""The rewrites a graph goes through before it is planned (ir.cpp: transposes_cancelled, broadcasts_hoisted, rematerialized), checked on
 the CPU: the graph a plan is made of is read back through the C ABI (he_plan_graph, he_graph_node_op) and evaluated by
 the oracle next to the graph as recorded. Both must give the same outputs - exactly where only data moves, to rounding
 where a reduction walks its operand in another order - and the transpositions that undo each other must be gone.
@@ -11,17 +11,19 @@ import pytest
 
 from helium_amd import autodiff as ad
 from helium_amd import ir, resnet
-from helium_amd.backend import OPT_CANCEL_TRANSPOSES, OPT_REMATERIALIZE, Plan, set_option
+from helium_amd.backend import OPT_CANCEL_TRANSPOSES, OPT_HOIST_BROADCASTS, OPT_REMATERIALIZE, Plan, set_option
 from oracle import helium_ir as oracle_ir
 from oracle import numerics as nm
 
 
-@pytest.fixture(params=["transposes only", "both rewrites"])
+@pytest.fixture(params=["transposes only", "all rewrites"])
 def rewrites(request):
     set_option(OPT_REMATERIALIZE, 0 if request.param == "transposes only" else 1)
+    set_option(OPT_HOIST_BROADCASTS, 0 if request.param == "transposes only" else 1)
     set_option(OPT_CANCEL_TRANSPOSES, 1)
     yield request.param
     set_option(OPT_REMATERIALIZE, 1)
+    set_option(OPT_HOIST_BROADCASTS, 1)
 
 
 def _feeds(g, seed=3):
@@ -117,6 +119,28 @@ def test_the_chain_of_swaps_in_front_of_a_reduction_becomes_the_shortest_one(rew
     assert len(swaps) == 2, swaps
     for o in want:
         np.testing.assert_allclose(got[o], want[o], rtol=1e-6, atol=1e-6)
+
+
+def test_pointwise_ops_on_broadcasts_alone_are_applied_before_the_broadcast():
+    """batch_norm.rs:56 as recorded: (variance.broadcast_to(x.shape) + 1e-3).sqrt() and the division by it."""
+    g = ir.OpGraph()
+    x = g.new_input([6, 5, 5, 8], "bf16")
+    var = g.new_input([8], "bf16")
+    mean = g.new_input([8], "bf16")
+    axes = [(0, 6), (1, 5), (2, 5)]
+    deviation = g.unary(g.binary(g.broadcast(var, 4, axes), g.constant(1e-3, "bf16", [6, 5, 5, 8]), "add"), "sqrt")
+    centred = g.binary(x, g.unary(g.broadcast(mean, 4, axes), "neg"), "add")
+    g.new_output(g.binary(centred, g.unary(deviation, "recip"), "mul"))
+    # a broadcast along other axes next to it: nothing to hoist for the op that reads both
+    other = g.broadcast(g.new_input([6, 1, 1, 1], "bf16"), 4, [(1, 5), (2, 5), (3, 8)])
+    g.new_output(g.binary(other, g.broadcast(var, 4, axes), "mul"))
+    want, got, nodes, _ = _both(g, _feeds(g))
+    full = [n for n in nodes if n.get("op") in ("unary", "binary") and int(np.prod(n["shape"])) == 6 * 5 * 5 * 8]
+    assert sorted((n["op"], n["fn"]) for n in full) == [("binary", "add"), ("binary", "mul"), ("binary", "mul")], full
+    small = [n for n in nodes if n.get("op") in ("unary", "binary") and int(np.prod(n["shape"])) == 8]
+    assert sorted(n["fn"] for n in small) == ["add", "neg", "recip", "sqrt"]
+    for o in want:
+        np.testing.assert_array_equal(want[o], got[o])
 
 
 def _batch_norm_backward_graph(dtype):

@@ -8,7 +8,8 @@ import numpy as np
 import pytest
 
 import helium_amd as ha
-from helium_amd.backend import (OPT_CANCEL_TRANSPOSES, OPT_FOLD_SWAP_INTO_REDUCE, OPT_FUSE_MATMUL_EPILOGUE, OPT_REMATERIALIZE, Plan,
+from helium_amd.backend import (OPT_CANCEL_TRANSPOSES, OPT_FOLD_SWAP_INTO_REDUCE, OPT_FUSE_MATMUL_EPILOGUE, OPT_HOIST_BROADCASTS,
+                                OPT_REMATERIALIZE, Plan,
                                 set_option, stats)
 from oracle import plan as oracle_plan
 
@@ -22,11 +23,13 @@ def reference_grouping():
     set_option(OPT_FOLD_SWAP_INTO_REDUCE, 0)
     set_option(OPT_REMATERIALIZE, 0)
     set_option(OPT_CANCEL_TRANSPOSES, 0)
+    set_option(OPT_HOIST_BROADCASTS, 0)
     yield
     set_option(OPT_FUSE_MATMUL_EPILOGUE, 1)
     set_option(OPT_FOLD_SWAP_INTO_REDUCE, 1)
     set_option(OPT_REMATERIALIZE, 1)
     set_option(OPT_CANCEL_TRANSPOSES, 1)
+    set_option(OPT_HOIST_BROADCASTS, 1)
 
 
 def linear_layer():
@@ -256,13 +259,15 @@ def test_batch_norm_statistics_join_the_convolution_that_feeds_them():
     outs = frontend.batch_norm_train(rec, conv, *[g.new_input([64], "f32") for _ in range(4)])
     for v in outs:
         g.new_output(v)
-    steps = Plan(g).steps
+    plan = Plan(g)
+    steps = plan.steps
     kind, members = steps[0][0][0]
     by_id = {n["id"]: n for n in g.nodes}
     assert kind == "gemm" and len(steps[0][0]) == 1
     assert sorted(by_id[m]["op"] for m in members) == ["binary", "broadcast", "conv", "reduce", "reduce", "swap_dims"]
     assert all(k == "pointwise" for instrs, _ in steps[1:] for k, _ in instrs)
-    check_invariants(g, steps)
+    # (the invariants hold on the graph the plan is made of: the backend's rewrites add and drop ops)
+    check_invariants(plan.graph(), plan.planned_steps())
 
 
 def linear_backward_graph(rows=64, inner=96, cols=80, dtype="f32", precision="f32_f32"):
