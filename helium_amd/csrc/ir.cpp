@@ -378,7 +378,7 @@ std::shared_ptr<OpGraph> rematerialized(const OpGraph& g, const std::set<NodeId>
         int cost = 0;
         std::vector<NodeId> anchors; // sorted, at most kMaxAnchors + 1 entries
     };
-    constexpr int kMaxCost = 64, kMaxCopies = 32;
+    constexpr int kMaxCost = 64, kMaxCopies = 1024;
     constexpr int64_t kMinElements = 1 << 16;
     constexpr size_t kMaxAnchors = 1;
     std::vector<Info> info(cap);
@@ -405,7 +405,8 @@ std::shared_ptr<OpGraph> rematerialized(const OpGraph& g, const std::set<NodeId>
         for (NodeId raw : n.op.inputs) {
             const NodeId in = canon[raw];
             const Info& J = info[in];
-            if (J.cheap) {
+            // (a cheap op that is not copied exists once, in memory like a product: its consumers start from it)
+            if (J.cheap && (J.remat || num_elements(g.get(in).desc.shape) < kMinElements)) {
                 I.cost += J.cost;
                 for (NodeId a : J.anchors) I.anchors.push_back(a);
             } else if (num_elements(g.get(in).desc.shape) * 8 >= numel) {

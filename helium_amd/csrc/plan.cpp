@@ -342,6 +342,22 @@ std::shared_ptr<const Plan> generate_plan(const std::shared_ptr<const ir::OpGrap
     for (NodeId n : g->nodes())
         if (g->get(n).kind == ir::Node::Intermediate) ig.insert(std::make_shared<Instr>(make_instr_for_op(g, n)));
 
+    // A value that was copied so that its consumer computes it joins that consumer before anything else: the greedy
+    // pass below walks from producers to consumers and would put the copy into its producer's kernel, to be written
+    // out from there. Last copies first, so that a chain of copies ends up in the kernel at its end.
+    if (g->has_origins()) {
+        std::vector<uint64_t> ids;
+        for (auto& kv : ig.instrs) ids.push_back(kv.first);
+        for (auto it = ids.rbegin(); it != ids.rend(); ++it) {
+            auto found = ig.instrs.find(*it);
+            if (found == ig.instrs.end()) continue;
+            const auto& nodes = found->second->subgraph().nodes();
+            if (nodes.size() != 1 || !g->made_for_consumer(nodes[0])) continue;
+            const auto& next = ig.dependents.at(*it);
+            if (next.size() == 1 && ig.can_fuse(*it, *next.begin())) ig.fuse(*it, *next.begin());
+        }
+    }
+
     // do_fusions (:243-256)
     auto do_fusions = [&] {
         bool fused = false;
@@ -520,10 +536,17 @@ std::shared_ptr<const ir::OpGraph> graph_for_execution(const std::shared_ptr<con
         // kernel ends up with several copies of a value among its outputs, that value goes back to being computed once,
         // and the graph is planned again.
         std::set<ir::NodeId> keep_single;
+        std::shared_ptr<ir::OpGraph> best;
+        int64_t best_bytes = 0;
         for (int round = 0; round < 3 && other; round++) {
             const size_t known = keep_single.size();
-            if (debug) fprintf(stderr, "[plan] round %d: %zu -> %zu nodes, %zu kept single\n", round, base->num_nodes(), other->num_nodes(), known);
             const auto plan = generate_plan(other);
+            const int64_t bytes = plan_traffic_bytes(*plan);
+            if (debug) fprintf(stderr, "[plan] round %d: %zu -> %zu nodes, %zu kept single, %lld bytes\n", round, base->num_nodes(), other->num_nodes(), known, (long long)bytes);
+            if (!best || bytes < best_bytes) {
+                best = other;
+                best_bytes = bytes;
+            }
             for (auto& st : plan->steps)
                 for (auto& instr : st.instrs) {
                     std::set<ir::NodeId> origins;
@@ -533,6 +556,7 @@ std::shared_ptr<const ir::OpGraph> graph_for_execution(const std::shared_ptr<con
             if (keep_single.size() == known) break;
             other = ir::rematerialized(*base, keep_single);
         }
+        other = best;  // (a round that takes copies back usually moves fewer bytes, not always)
     }
     // A rewritten graph is taken only when its plan moves fewer bytes - or as many, where transpositions went: the
     // kernels then walk their tensors in memory order.
