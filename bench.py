@@ -24,7 +24,7 @@ BF16_PEAK_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
 F32_PEAK_TFLOPS = 157.3      # MI355X dense fp32 matrix, published
 # Bytes that left the XCD L2s per launch of each workload's dominant kernel: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE,
 # each scaled by what the same counter reads for the COPY workload (profiles/<kernel>_<workload>.txt).
-TRAFFIC_BYTES = {"COPY": 268435456, "C2a": 205509374, "C2b": 67196580, "C2c": 17587916, "C3": 269743029, "C4": 370218917, "C5a-fused": 302134023, "GEMM": 234914277, "C5b-bn": 313174768, "C5b-conv": 52383120}
+TRAFFIC_BYTES = {"COPY": 268435456, "C2a": 205509374, "C2b": 67196580, "C2c": 12867962, "C3": 269743029, "C4": 370218917, "C5a-fused": 302134023, "C5a-planned": 335673461, "GEMM": 234914277, "C5b-bn": 313174768, "C5b-conv": 52383120}
 HEADLINE = "C4"              # the workload `value` is quoted on
 ROTATE_BYTES = 768 << 20     # rotate operand sets so repeated steps cannot live in the 256 MB Infinity Cache
 
