@@ -89,7 +89,7 @@ def c3_chain(rows=4096, cols=4096, bias_axis=2, seed=31, make_inputs=True):
     return g, inputs, {"batch": out_batch, "columns": out_cols, "r": r}
 
 
-def c4_graph(size=4096, mainloop=False, full_size_outputs=False):
+def c4_graph(size=4096, mainloop=False, full_size_outputs=False, bias_rows=False):
     """Config 4: the reference README's fusion (README.md:33-79), node ids as printed there.
 
     Core = Matmul{a: n1, b: n2} is node 12; n13, n24, n26 are the other GEMM results of the LSTM-cell-like graph
@@ -97,13 +97,16 @@ def c4_graph(size=4096, mainloop=False, full_size_outputs=False):
     broadcast along axis 1. 39 epilogue ops follow the anchor; the leaves are the three reductions n39 (Batch),
     n58 and n87 (Columns). With mainloop=True the anchor's A operand is n25 = Relu(n22) * n9 (README.md:36-38).
     With full_size_outputs=True n57 and n86 (the gradients the backward GEMMs would read) are also stored, as bf16.
+    With bias_rows=True the biases are [1,size,1] columns broadcast along axis 2, as the headline configuration words
+    them, and their gradients n58 / n87 are sums over each row.
     """
     g = fusion.OpGraph()
     full = [1, size, size]
     P = lambda i, shape=full, dt="bf16": g.producer(shape, dt, node_id=i)  # noqa: E731
     n1 = P(22) if mainloop else P(1)
     n2 = P(2)
-    n6, n8 = P(6, [1, 1, size], "f32"), P(8, [1, 1, size], "f32")
+    bias_shape, bias_axis, bias_sum = ([1, size, 1], 2, "rows") if bias_rows else ([1, 1, size], 1, "columns")
+    n6, n8 = P(6, bias_shape, "f32"), P(8, bias_shape, "f32")
     n9, n11, n13, n24, n26 = P(9), P(11), P(13), P(24), P(26)
     a_operand = n1
     if mainloop:
@@ -113,8 +116,8 @@ def c4_graph(size=4096, mainloop=False, full_size_outputs=False):
     U = lambda i, x, fn, c=0.0: g.unary(x, fn, c, node_id=i)  # noqa: E731
     B = lambda i, lhs, rhs, fn: g.binary(lhs, rhs, fn, node_id=i)  # noqa: E731
     inv = np.float32(0.00024414063)
-    B(14, 12, n13, "add"); g.broadcast(n6, 1, size, node_id=15); B(16, 14, 15, "add"); U(17, 16, "relu")
-    B(27, n24, n26, "add"); g.broadcast(n8, 1, size, node_id=28); B(29, 27, 28, "add"); U(30, 29, "tanh")
+    B(14, 12, n13, "add"); g.broadcast(n6, bias_axis, size, node_id=15); B(16, 14, 15, "add"); U(17, 16, "relu")
+    B(27, n24, n26, "add"); g.broadcast(n8, bias_axis, size, node_id=28); B(29, 27, 28, "add"); U(30, 29, "tanh")
     U(31, 17, "neg"); U(32, 31, "add_constant", 1.0); B(33, 32, n9, "mul"); B(34, 17, 30, "mul"); B(35, 33, 34, "add")
     B(36, 35, n11, "sub"); U(37, 36, "pow_constant", 2.0); U(38, 37, "mul_constant", inv)
     g.reduction(38, "batch", node_id=39)
@@ -125,9 +128,9 @@ def c4_graph(size=4096, mainloop=False, full_size_outputs=False):
     B(48, 36, 47, "pow"); B(49, 48, 46, "mul"); B(50, 49, 45, "mul")
     B(52, 50, 30, "mul"); B(53, 17, 50, "mul"); U(54, 30, "pow_constant", 2.0); U(55, 54, "neg")
     U(56, 55, "add_constant", 1.0); B(57, 53, 56, "mul")
-    g.reduction(57, "columns", node_id=58)
+    g.reduction(57, bias_sum, node_id=58)
     B(81, 50, n9, "mul"); U(84, 81, "neg"); B(85, 52, 84, "add"); B(86, 85, 16, "drelu")
-    g.reduction(86, "columns", node_id=87)
+    g.reduction(86, bias_sum, node_id=87)
     outs = {"loss": 39, "db8": 58, "db6": 87}
     if full_size_outputs:
         outs["dpre_c"] = g.consumer(57, "bf16", node_id=90)

@@ -880,7 +880,9 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     // A convolution's gather with direct loads, a channel count that is a multiple of the k-tile (every tile then lies in
     // one filter tap) and a wave that issues a whole number of loads: the per-lane address arithmetic of a load
     // shrinks from a full (pixel, tap) decomposition to a few adds.
+    // (the image offset a lane carries across the k-loop is 32 bits wide: larger images take the general gather)
     const bool conv_a_fast = pr.conv_a.on && direct_a && pr.conv_a.C % t.bk == 0 && (t.bm * t.bk * esz / 1024) % (threads / 64) == 0 &&
+                             (int64_t)pr.conv_a.N * pr.conv_a.H * pr.conv_a.W * pr.conv_a.C < (int64_t(1) << 32) &&
                              !tuning::get("HELIUM_HIP_GEMM_NO_CONV_FAST");
     if (!(direct_a && direct_b)) t.stages = 2;  // register staging is double-buffered only
     else if (!tuning::get("HELIUM_HIP_GEMM_TILE") && small) {

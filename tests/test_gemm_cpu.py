@@ -66,10 +66,10 @@ def compare(got, want, rel=1e-2, eps=1e-3):
         assert ok.all(), (node, np.abs(g - w).max())
 
 
-def readme_fusion(size, mainloop, full):
+def readme_fusion(size, mainloop, full, bias_rows=False):
     from helium_amd import configs
 
-    g, outs = configs.c4_graph(size, mainloop=mainloop, full_size_outputs=full)
+    g, outs = configs.c4_graph(size, mainloop=mainloop, full_size_outputs=full, bias_rows=bias_rows)
     return g, configs.c4_inputs(g, size), sorted(outs.values())
 
 
@@ -77,6 +77,7 @@ CASES = [
     ("readme_epilogue_with_prefetched_aux_tensors", lambda: readme_fusion(128, False, False), "128,128,64,2,2"),
     ("readme_epilogue", lambda: readme_fusion(128, False, False), "128,128,64,2,2"),
     ("readme_epilogue_ragged_with_mainloop", lambda: readme_fusion(72, True, True), "128,128,64,2,2"),
+    ("readme_epilogue_with_biases_along_the_rows", lambda: readme_fusion(136, False, False, bias_rows=True), "128,128,64,2,2"),
     ("plain_2x2_tiles", lambda: gemm_cases.plain(160, 136, 72), "128,128,64,2,2"),
     ("ragged_scalar_paths", lambda: gemm_cases.plain(97, 131, 67), "128,128,64,2,2"),
     ("mainloop_bias_relu_colsum", lambda: gemm_cases.bias_relu_colsum(130, 136, 80, mainloop=True), "128,128,64,2,2"),

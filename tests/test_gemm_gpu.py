@@ -124,6 +124,16 @@ def test_c4_readme_fusion(gpu, size, mainloop, full):
     check_reductions_and_full(g, configs.c4_inputs(g, size))
 
 
+@pytest.mark.parametrize("size", [384, 4096])
+def test_c4_with_biases_along_the_rows(gpu, size):
+    """The headline configuration words its biases [1,4096,1]: broadcast along the columns, their gradients sums over
+    each row (the README's own listing has them [1,1,4096])."""
+    from helium_amd import configs
+
+    g, outs = configs.c4_graph(size, bias_rows=True)
+    check_reductions_and_full(g, configs.c4_inputs(g, size))
+
+
 @pytest.mark.parametrize("size", [512, 4096])
 def test_c5a_mainloop_and_epilogue(gpu, size):
     from helium_amd import configs
