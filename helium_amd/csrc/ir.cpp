@@ -826,50 +826,63 @@ std::shared_ptr<OpGraph> broadcasts_hoisted(const OpGraph& g) {
             case OpKind::Select: pointwise = true; break;
             default: break;
         }
-        // every operand the same broadcast of a small tensor, or a constant: the op is applied before the broadcast
-        const Op* pattern = nullptr;
-        Shape small;
-        bool hoist = pointwise;
+        // Every operand a broadcast of a small tensor (or a constant): the op is applied to the small tensors, brought
+        // to the smallest shape that holds them all ([C] and [1] meet in [C]), and its result is broadcast.
+        const Shape& full = n.desc.shape;
+        Shape small(full.size(), 1);
+        std::vector<Shape> padded(op.inputs.size());
+        bool hoist = pointwise, any_broadcast = false;
         for (size_t i = 0; i < op.inputs.size() && hoist; i++) {
             const Node& in = out->get(op.inputs[i]);
             if (in.kind == Node::Intermediate && in.op.kind == OpKind::Constant) continue;
-            Shape padded;
-            if (!plain_broadcast(op.inputs[i], &padded)) {
+            if (!plain_broadcast(op.inputs[i], &padded[i]) || padded[i].size() != full.size()) {
                 hoist = false;
-            } else if (!pattern) {
-                pattern = &in.op;
-                small = padded;
-            } else {
-                hoist = padded == small && in.op.new_dim_count == pattern->new_dim_count && in.op.broadcast_axes == pattern->broadcast_axes;
+                break;
             }
+            any_broadcast = true;
+            for (size_t d = 0; d < full.size(); d++) small[d] = std::max(small[d], padded[i][d]);
         }
-        if (hoist && pattern) {
-            const Op broadcast = *pattern;  // (a copy: new nodes move the node table)
+        if (hoist && any_broadcast && num_elements(small) * 8 <= num_elements(full)) {
             Op inner = op;
-            for (NodeId& in : inner.inputs) {
-                const Node src = out->get(in);
-                // (the constants and reshapes made here stand for no node of `g`)
+            for (size_t i = 0; i < inner.inputs.size(); i++) {
+                NodeId& in = inner.inputs[i];
+                const Node src = out->get(in);  // (a copy: new nodes move the node table)
+                // (the constants, reshapes and small broadcasts made here stand for no node of `g`)
                 if (src.op.kind == OpKind::Constant) {
                     Op c = src.op;
                     c.shape = small;
                     in = out->new_op(std::move(c));
                     note_origin(in, kNoNode);
-                } else {
-                    in = src.op.inputs[0];
-                    if (out->get(in).desc.shape != small) {
-                        Op r;
-                        r.kind = OpKind::Reshape;
-                        r.inputs = {in};
-                        r.shape = small;
-                        in = out->new_op(std::move(r));
-                        note_origin(in, kNoNode);
-                    }
+                    continue;
+                }
+                in = src.op.inputs[0];
+                if (out->get(in).desc.shape != padded[i]) {
+                    Op r;
+                    r.kind = OpKind::Reshape;
+                    r.inputs = {in};
+                    r.shape = padded[i];
+                    in = out->new_op(std::move(r));
+                    note_origin(in, kNoNode);
+                }
+                if (padded[i] != small) {
+                    Op b;
+                    b.kind = OpKind::Broadcast;
+                    b.inputs = {in};
+                    b.new_dim_count = (int64_t)small.size();
+                    for (size_t d = 0; d < small.size(); d++)
+                        if (padded[i][d] == 1 && small[d] != 1) b.broadcast_axes.push_back({(int64_t)d, small[d]});
+                    in = out->new_op(std::move(b));
+                    note_origin(in, kNoNode);
                 }
             }
             const NodeId computed = out->new_op(std::move(inner));
             note_origin(computed, id);
-            Op again = broadcast;
+            Op again;
+            again.kind = OpKind::Broadcast;
             again.inputs = {computed};
+            again.new_dim_count = (int64_t)full.size();
+            for (size_t d = 0; d < full.size(); d++)
+                if (small[d] == 1 && full[d] != 1) again.broadcast_axes.push_back({(int64_t)d, full[d]});
             placed[id] = out->new_op(std::move(again));
             // (the broadcast stands for no node of `g`: whoever evaluates the plan on `g` reads `id` from memory there)
             note_origin(placed[id], kNoNode);

@@ -384,6 +384,57 @@ std::shared_ptr<const Plan> generate_plan(const std::shared_ptr<const ir::OpGrap
     while (do_fusions() && rematerialize()) {
     }
 
+    // Beyond the reference: kernels that only reduce, over the same index space, and read a tensor in common share one
+    // pass over it. The greedy pass merges along producer -> consumer edges only, and the sums of one backward pass (a
+    // batch norm's sum of dy and sum of dy * xhat) are siblings: each would read both tensors again. Two such kernels
+    // merge when neither depends on the other; four reductions per kernel at most (each keeps its own accumulators).
+    if (rematerialize()) {
+        auto only_reduces = [&](const Instr& instr, ir::Shape* shape, uint32_t* depth, size_t* count) {
+            if (instr.kind() != InstrKind::Pointwise) return false;
+            *count = 0;
+            for (NodeId leaf : instr.subgraph().leafs()) {
+                const ir::Node& n = g->get(leaf);
+                if (n.op.kind != ir::OpKind::Reduce) return false;
+                *shape = g->get(n.op.inputs[0]).desc.shape;
+                *depth = n.op.depth;
+                ++*count;
+            }
+            return *count > 0;
+        };
+        auto reaches = [&](uint64_t from, uint64_t to) {
+            std::vector<uint64_t> stack{from};
+            std::set<uint64_t> visited{from};
+            while (!stack.empty()) {
+                const uint64_t cur = stack.back();
+                stack.pop_back();
+                if (cur == to) return true;
+                for (uint64_t n : ig.dependents.at(cur))
+                    if (visited.insert(n).second) stack.push_back(n);
+            }
+            return false;
+        };
+        for (bool changed = true; changed;) {
+            changed = false;
+            for (auto& [tensor, readers] : ig.consumers) {
+                if (readers.size() < 2 || ir::num_elements(g->get(tensor).desc.shape) < (1 << 16)) continue;
+                const std::vector<uint64_t> ids(readers.begin(), readers.end());
+                for (size_t i = 0; i < ids.size() && !changed; i++)
+                    for (size_t j = i + 1; j < ids.size() && !changed; j++) {
+                        ir::Shape sa, sb;
+                        uint32_t da = 0, db = 0;
+                        size_t na = 0, nb = 0;
+                        if (!only_reduces(*ig.instrs.at(ids[i]), &sa, &da, &na) || !only_reduces(*ig.instrs.at(ids[j]), &sb, &db, &nb)) continue;
+                        if (sa != sb || da != db || na + nb > 4) continue;
+                        if (reaches(ids[i], ids[j]) || reaches(ids[j], ids[i])) continue;
+                        if (!ig.instrs.at(ids[i])->can_fuse_with(*ig.instrs.at(ids[j]))) continue;
+                        ig.fuse(ids[i], ids[j]);
+                        changed = true;
+                    }
+                if (changed) break;  // the maps changed under the loops
+            }
+        }
+    }
+
     // Beyond the reference, with the epilogue option on: the greedy pass visits a product before the pointwise group
     // that reduces it has formed (a SwapDims alone is no epilogue; SwapDims + Reduce is a column reduction), so
     // products are offered their finished pointwise dependents once more.
@@ -515,19 +566,31 @@ int64_t plan_traffic_bytes(const Plan& plan) {
 
 std::shared_ptr<const ir::OpGraph> graph_for_execution(const std::shared_ptr<const ir::OpGraph>& g) {
     const bool debug = getenv("HELIUM_HIP_PLAN_DEBUG") != nullptr;
-    // 1. transpositions that undo each other go
+    // 1. transpositions that undo each other go - when the plan then moves no more bytes (the kernels walk their tensors
+    //    in memory order instead)
     std::shared_ptr<const ir::OpGraph> base = g;
+    const int64_t recorded = plan_traffic_bytes(*generate_cached_plan(g));
+    int64_t base_bytes = recorded;
     if (cancel_transposes())
         if (auto untransposed = ir::transposes_cancelled(*g)) {
-            if (debug) fprintf(stderr, "[plan] transpositions cancelled: %zu -> %zu nodes\n", g->num_nodes(), untransposed->num_nodes());
-            base = untransposed;
+            const int64_t bytes = plan_traffic_bytes(*generate_cached_plan(untransposed));
+            if (debug) fprintf(stderr, "[plan] transpositions cancelled: %zu -> %zu nodes, %lld -> %lld bytes\n", g->num_nodes(), untransposed->num_nodes(), (long long)recorded, (long long)bytes);
+            if (bytes <= base_bytes) {
+                base = untransposed;
+                base_bytes = bytes;
+            }
         }
-    // ... and pointwise ops on broadcasts alone are applied before the broadcast
+    // ... and pointwise ops on broadcasts alone are applied before the broadcast: less arithmetic for about the same
+    // bytes (the small results are tensors of their own)
     if (hoist_broadcasts())
         if (auto hoisted = ir::broadcasts_hoisted(*base)) {
-            if (debug) fprintf(stderr, "[plan] broadcasts hoisted: %zu -> %zu nodes\n", base->num_nodes(), hoisted->num_nodes());
             if (base != g) hoisted->rebase_origins(*base);
-            base = hoisted;
+            const int64_t bytes = plan_traffic_bytes(*generate_cached_plan(hoisted));
+            if (debug) fprintf(stderr, "[plan] broadcasts hoisted: %zu -> %zu nodes, %lld -> %lld bytes\n", base->num_nodes(), hoisted->num_nodes(), (long long)base_bytes, (long long)bytes);
+            if (bytes <= base_bytes + base_bytes / 20 + (64 << 10)) {
+                base = hoisted;
+                base_bytes = bytes;
+            }
         }
     // 2. cheap values are computed where they are used
     std::shared_ptr<ir::OpGraph> other = rematerialize() ? ir::rematerialized(*base) : nullptr;
@@ -558,19 +621,11 @@ std::shared_ptr<const ir::OpGraph> graph_for_execution(const std::shared_ptr<con
         }
         other = best;  // (a round that takes copies back usually moves fewer bytes, not always)
     }
-    // A rewritten graph is taken only when its plan moves fewer bytes - or as many, where transpositions went: the
-    // kernels then walk their tensors in memory order.
-    if (base != g && plan_traffic_bytes(*generate_cached_plan(base)) > plan_traffic_bytes(*generate_cached_plan(g))) {
-        base = g;
-        other = rematerialize() ? ir::rematerialized(*g) : nullptr;  // (without the rounds above: the rare case)
-    }
-    if (debug) fprintf(stderr, "[plan] bytes moved by the plan: %lld as recorded, %lld without the transpositions\n",
-                       (long long)plan_traffic_bytes(*generate_cached_plan(g)), (long long)plan_traffic_bytes(*generate_cached_plan(base)));
     if (!other) return base;
     if (base != g) other->rebase_origins(*base);
-    const int64_t before = plan_traffic_bytes(*generate_cached_plan(base)), after = plan_traffic_bytes(*generate_cached_plan(other));
-    if (debug) fprintf(stderr, "[plan] ... %lld with cheap values computed where they are used\n", (long long)after);
-    return after < before ? std::shared_ptr<const ir::OpGraph>(other) : base;
+    const int64_t after = plan_traffic_bytes(*generate_cached_plan(other));
+    if (debug) fprintf(stderr, "[plan] ... %lld bytes with cheap values computed where they are used\n", (long long)after);
+    return after < base_bytes ? std::shared_ptr<const ir::OpGraph>(other) : base;
 }
 
 // ---------------------------------------------------------------------------------------------------------
