@@ -331,10 +331,31 @@ bool is_uniform_pow(const Program& p, int id) {
            std::all_of(rhs.access.stride.begin(), rhs.access.stride.end(), [](int64_t w) { return w == 0; });
 }
 
+std::vector<char> row_invariant_exprs(const Program& p) {
+    const int n = (int)p.dims.size();
+    std::vector<char> inv(p.exprs.size(), 0);
+    if (n < 2) return inv;
+    for (size_t i = 0; i < p.exprs.size(); i++) {
+        const Expr& e = p.exprs[i];
+        switch (e.kind) {
+            case Expr::Load: inv[i] = e.access.chain.empty() && (p.dims[n - 2] <= 1 || e.access.stride[n - 2] == 0); break;
+            case Expr::Acc: inv[i] = 0; break;
+            case Expr::Const: inv[i] = 1; break;
+            case Expr::Unary:
+            case Expr::Cast: inv[i] = inv[e.a]; break;
+            case Expr::Binary:
+            case Expr::Compare: inv[i] = inv[e.a] && inv[e.b]; break;
+            case Expr::Select: inv[i] = inv[e.a] && inv[e.b] && inv[e.c]; break;
+        }
+    }
+    return inv;
+}
+
 std::string emit_exprs(const Program& p, const EmitCtx& cx) {
     const int n = (int)p.dims.size();
     const int NV = cx.nv;
     std::ostringstream s;
+    const std::vector<char> invariant = cx.row_part ? row_invariant_exprs(p) : std::vector<char>();
     auto coord_sum = [&](const std::vector<int64_t>& stride) {
         // Linear index of the first of the NV columns.
         std::ostringstream o;
@@ -350,6 +371,8 @@ std::string emit_exprs(const Program& p, const EmitCtx& cx) {
         const Expr& e = p.exprs[i];
         const std::string v = "e" + std::to_string(i);
         const char* T = cls_type(e.cls);
+        if (cx.row_part == 1 && !invariant[i]) continue;
+        if (cx.row_part == 2 && invariant[i]) continue;
         if (cx.phase != 0) {
             const bool deferred = is_deferred_load(p, e, NV, cx.defer_row_varying_only);
             if (cx.phase == 1) {
@@ -376,7 +399,8 @@ std::string emit_exprs(const Program& p, const EmitCtx& cx) {
                 const Access& a = e.access;
                 const int64_t sn = p.dims[n - 1] > 1 ? a.stride[n - 1] : 0;
                 const std::string ptr = "a" + std::to_string(a.arg);
-                s << T << " " << v << "[" << NV << "];\n{ const size_t o = " << coord_sum(a.stride) << ";\n";
+                if (cx.row_part == 1) s << T << " " << v << "[" << NV << "] = {};\nif (col_ok) { const size_t o = " << coord_sum(a.stride) << ";\n";
+                else s << T << " " << v << "[" << NV << "];\n{ const size_t o = " << coord_sum(a.stride) << ";\n";
                 if (!a.chain.empty()) {
                     s << "#pragma unroll\nfor (int k = 0; k < " << NV << "; k++) { u32 lin = (u32)(o + (size_t)k * " << sn
                       << "ull);\n";
@@ -627,6 +651,21 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
     // The rows of a block whose tile lies wholly inside the tensor carry no bounds test: a load under a per-row
     // predicate cannot be issued ahead of the previous row's work, and a streaming kernel then waits out one memory
     // round trip per row.
+    // What is the same in every row a thread walks (per-channel operands of an NHWC activation seen as [rows, channels],
+    // and what is computed from them alone) is loaded and computed once, ahead of the rows: under the rows' predicate
+    // the compiler may not move those loads itself.
+    bool hoist_rows = false;
+    {
+        const std::vector<char> inv = row_invariant_exprs(p);
+        for (size_t i = 0; i < p.exprs.size(); i++) hoist_rows = hoist_rows || (inv[i] && p.exprs[i].kind == Expr::Load);
+        hoist_rows = hoist_rows && RPT > 1;
+        if (hoist_rows) {
+            EmitCtx cx;
+            cx.nv = NV;
+            cx.row_part = 1;
+            s << emit_exprs(p, cx);
+        }
+    }
     std::ostringstream& main_stream = s;
     auto row_body = [&](bool squares) {
     std::ostringstream s;
@@ -637,6 +676,7 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
     EmitCtx cx;
     cx.nv = NV;
     cx.uniform_pow_is_square = squares;
+    cx.row_part = hoist_rows ? 2 : 0;
     s << emit_exprs(p, cx);
     // outputs
     Shape pst = ir::packed_strides(p.dims);

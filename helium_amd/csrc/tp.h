@@ -146,7 +146,13 @@ struct EmitCtx {
     bool defer_row_varying_only = false;  // phases 1/2: loads whose address ignores the row stay in phase 2
     // Pow whose exponent is a launch-uniform operand: written as x * x (the caller has tested the exponents)
     bool uniform_pow_is_square = false;
+    // 0: every expression. 1: only those whose value is the same in every row a thread walks (operands that are
+    // broadcast along the rows, and what is computed from them alone); their loads are issued only `if (col_ok)`.
+    // 2: the others, which read the former from the enclosing scope.
+    int row_part = 0;
 };
+// Per expression: whether its value ignores the row coordinate `m`.
+std::vector<char> row_invariant_exprs(const Program& p);
 // Whether expression `id` is a Pow whose exponent is a float operand read at one address by the whole launch.
 bool is_uniform_pow(const Program& p, int id);
 // Members of the struct phase 1 fills: one native vector per deferred Load of the program.
