@@ -793,6 +793,15 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
             t.bn = 32;
             t.wm = 4;
             t.wn = 1;
+        } else if (!f32 && pr.M <= 32 && pr.M > 16 && pr.N >= 128 && pr.conv_b.on && pr.conv_b.C % epc != 0) {
+            // ... and a B operand gathered element by element (the filter gradient of the 7x7 stem on a 3-channel
+            // image): the gather is bound by the loads it keeps in flight, so small workgroups, six of which share a
+            // CU's LDS, and as many k ranges as fill the chip once (plan.cpp); 664 -> 439 us at batch 128
+            t.bm = 32;
+            t.bn = 64;
+            t.wm = 1;
+            t.wn = 2;
+            small = true;
         } else if (!f32 && pr.M <= 32 && pr.M > 16 && pr.N >= 128) {
             // few output rows (a filter gradient with 32 output channels): four waves side by side
             // (the 7x7x3 stem's: 1095 us with 128x128 tiles, 668 us)
@@ -802,14 +811,21 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
             t.wn = 4;
             small = true;
         } else if (!f32 && pr.M <= 64 && pr.M > 32 && pr.N >= 128) {
-            // few output rows (a filter gradient with 64 output channels): tiles as low as M
+            // few output rows (a filter gradient with 64 output channels): tiles as low as M, and twice as wide when the
+            // k range is split (eight waves share the 64 rows of the flow: 107 -> 99 us on the 56x56x64 layer)
             t.bm = 64;
             t.bn = 128;
             t.wm = t.wn = 2;
+            if (pr.split_k > 1 && pr.N >= 256) {
+                t.bn = 256;
+                t.wn = 4;
+            }
             small = true;
         } else
         // Smaller problems take smaller tiles so that every CU gets work.
-        if (pr.M <= 128 || pr.N <= 128 || ((pr.M + 255) / 256) * ((pr.N + 255) / 256) * pr.batch < 128) {
+        // (a split k range multiplies the workgroups: the filter gradients of 256 and 512 channels keep the large tile,
+        // 81 -> 70 us and 93 -> 78 us)
+        if (pr.M <= 128 || pr.N <= 128 || ((pr.M + 255) / 256) * ((pr.N + 255) / 256) * pr.batch * pr.split_k < 128) {
             t.bm = t.bn = 128;
             t.wm = t.wn = 2;
             small = true;

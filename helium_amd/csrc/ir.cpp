@@ -1,5 +1,6 @@
 #include "ir.h"
 
+#include <cstring>
 #include <functional>
 #include <map>
 #include <set>
@@ -825,6 +826,57 @@ std::shared_ptr<OpGraph> broadcasts_hoisted(const OpGraph& g) {
             case OpKind::Compare:
             case OpKind::Select: pointwise = true; break;
             default: break;
+        }
+        // A reduction of a broadcast along reduced dims only: the repeated terms need not be walked. Sum: the small
+        // tensor's sum times the number of repeats; Mean, Max, Min: the small tensor's.
+        if (op.kind == OpKind::Reduce) {
+            Shape padded;
+            const Shape full_in = out->get(op.inputs[0]).desc.shape;
+            if (plain_broadcast(op.inputs[0], &padded) && padded.size() == full_in.size() && op.depth <= padded.size()) {
+                const Op broadcast = out->get(op.inputs[0]).op;
+                bool inside = true;
+                double repeats = 1;
+                for (auto& a : broadcast.broadcast_axes) {
+                    inside = inside && (size_t)a.axis >= padded.size() - op.depth;
+                    repeats *= (double)full_in[a.axis];
+                }
+                if (inside && repeats > 1) {
+                    NodeId small_in = broadcast.inputs[0];
+                    if (out->get(small_in).desc.shape != padded) {
+                        Op r;
+                        r.kind = OpKind::Reshape;
+                        r.inputs = {small_in};
+                        r.shape = padded;
+                        small_in = out->new_op(std::move(r));
+                        note_origin(small_in, kNoNode);
+                    }
+                    Op red = op;
+                    red.inputs = {small_in};
+                    NodeId result = out->new_op(std::move(red));
+                    if (out->get(result).desc == n.desc) {
+                        if ((ReduceOp)op.sub_op == ReduceOp::Sum) {
+                            note_origin(result, kNoNode);
+                            Op c;
+                            c.kind = OpKind::Constant;
+                            c.shape = n.desc.shape;
+                            c.const_dtype = HE_F32;
+                            const float f = (float)repeats;
+                            memcpy(&c.const_bits, &f, 4);
+                            const NodeId factor = out->new_op(std::move(c));
+                            note_origin(factor, kNoNode);
+                            Op mul;
+                            mul.kind = OpKind::BinaryPointwise;
+                            mul.sub_op = (int)BinaryOp::Mul;
+                            mul.inputs = {result, factor};
+                            result = out->new_op(std::move(mul));
+                        }
+                        placed[id] = result;
+                        note_origin(result, id);
+                        changed = true;
+                        continue;
+                    }
+                }
+            }
         }
         // Every operand a broadcast of a small tensor (or a constant): the op is applied to the small tensors, brought
         // to the smallest shape that holds them all ([C] and [1] meet in [C]), and its result is broadcast.

@@ -872,6 +872,11 @@ GemmProblem conv_backward_filter_problem(const ir::OpSubgraph& sg, NodeId node) 
     // about two workgroups per CU, each with at least four 64-wide k-tiles (128x128 output tiles)
     const int64_t tiles = ((pr.M + 127) / 128) * ((pr.N + 127) / 128), k_tiles = (pr.K + 63) / 64;
     pr.split_k = (int)std::max<int64_t>(1, std::min<int64_t>({(512 + tiles - 1) / tiles, k_tiles / 4, 1024}));
+    // (an image whose channels do not fill 16-byte chunks is gathered element by element, by 32x64 tiles of two waves: six
+    // workgroups per CU, one round of them over the chip)
+    const int64_t chunk = image.dtype == HE_F32 ? 4 : 8;
+    if (image.dtype != HE_F32 && cv.C % chunk != 0 && pr.M <= 32 && pr.M > 16 && pr.N >= 128)
+        pr.split_k = (int)std::max<int64_t>(1, std::min<int64_t>({1536 / ((pr.N + 63) / 64), k_tiles / 4, 1024}));
     if (const char* env = tuning::get("HELIUM_HIP_GEMM_SPLIT_K")) pr.split_k = std::max(1, atoi(env));
     pr.epi.dims = {1, pr.M, pr.N};
     pr.epi.fast_math = true;

@@ -350,6 +350,7 @@ BWD_FILTER_CASES = [
     # channel counts that do not fill a 16-byte chunk: the image operand is gathered element by element
     ("three_channel_stem_7x7_stride2", (2, 16, 16, 3), 32, (7, 7), "bf16", (2, 2), (1, 1), "same", "64,128,64,2,2"),
     ("three_channel_stem_thirty_two_rows_tile", (2, 16, 16, 3), 32, (7, 7), "bf16", (2, 2), (1, 1), "same", "32,128,64,1,4"),
+    ("three_channel_stem_two_wave_tile", (2, 16, 16, 3), 32, (7, 7), "bf16", (2, 2), (1, 1), "same", "32,64,64,1,2"),
     ("thirty_two_rows_tile_direct_loads", (2, 12, 12, 16), 32, (3, 3), "bf16", (1, 1), (1, 1), "same", "32,128,64,1,4"),
     ("five_channels_3x3_f16", (1, 7, 9, 5), 8, (3, 3), "f16", (1, 1), (1, 1), "same", "64,64,64,2,2"),
     ("three_channels_f32_full", (1, 6, 5, 3), 8, (3, 3), "f32", (1, 1), (1, 2), "full", "64,64,32,2,2"),

@@ -144,6 +144,23 @@ def test_pointwise_ops_on_broadcasts_alone_are_applied_before_the_broadcast():
         np.testing.assert_array_equal(want[o], got[o])
 
 
+def test_a_reduction_of_a_broadcast_along_reduced_dims_walks_the_small_tensor():
+    g = ir.OpGraph()
+    x = g.new_input([10, 16, 1, 1], "bf16")
+    full = g.broadcast(x, 4, [(2, 7), (3, 7)])
+    g.new_output(g.reduce(full, "sum", 3))
+    g.new_output(g.reduce(full, "mean", 3))
+    g.new_output(g.reduce(full, "max", 2))
+    # a broadcast along a kept dim is left alone
+    g.new_output(g.reduce(g.broadcast(g.new_input([1, 16, 7, 7], "bf16"), 4, [(0, 10)]), "sum", 3))
+    want, got, nodes, _ = _both(g, _feeds(g))
+    by_id = {n["id"]: n for n in nodes}
+    sizes = sorted(int(np.prod(by_id[n["inputs"][0]]["shape"])) for n in nodes if n.get("op") == "reduce")
+    assert sizes == [160, 160, 160, 10 * 16 * 49], sizes
+    for o in want:
+        np.testing.assert_allclose(got[o], want[o], rtol=1e-6)
+
+
 def _batch_norm_backward_graph(dtype):
     G = ad.Graph()
     rng = np.random.default_rng(5)
