@@ -878,6 +878,25 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         red_floats += (uint64_t)r.elems * r.parts;
         reds.push_back(r);
     }
+    // Reductions of a small product fold inside the kernel: the last workgroup of a tile column adds that column's
+    // partials (one per tile row), the last workgroup of all the scalar's. That saves the second launch where launches
+    // are what a graph's time consists of (a 256 x 512 x 512 linear layer with bias, relu and column sums: 15.8 -> 13.7 us
+    // per graph). A large product is better off with the second launch: its workgroups all end together, the tickets and
+    // the loads of the partials are three dependent round trips at the very end of the kernel, and a 4096^3 product with
+    // the README's epilogue took 155 us this way against 141. Row sums keep the second launch as well.
+    bool fold_in_kernel = !reds.empty() && pr.split_k == 1 && tiles_m * tiles_n * pr.batch <= 64 && !tuning::get("HELIUM_HIP_GEMM_NO_TICKET_FOLD");
+    for (auto& r : reds) {
+        const tp::Out& o = pr.epi.outs[r.out];
+        fold_in_kernel = fold_in_kernel && o.fold_m && (!o.fold_n || r.parts <= 4096);
+    }
+    // arrival counters: one per (batch index, tile column), then one per scalar output element group
+    uint64_t ticket_cols = 0, ticket_all = 0;
+    if (fold_in_kernel) {
+        ticket_cols = (uint64_t)pr.batch * tiles_n;
+        for (auto& r : reds)
+            if (pr.epi.outs[r.out].fold_n) ticket_all = std::max<uint64_t>(ticket_all, (uint64_t)r.elems);
+    }
+    reduce_counters_ = ticket_cols + ticket_all;
     auto red_of = [&](size_t oi) -> const RedOut& {
         for (auto& r : reds)
             if (r.out == oi) return r;
@@ -958,6 +977,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
             ps << (a ? ", " : "") << (pr.args[a].is_output ? "" : "const ") << tp::c_type(pr.args[a].dtype) << "* __restrict__ p" << a;
         if (pr.split_k > 1) ps << ", float* __restrict__ splitk_ws";
         if (!reds.empty()) ps << ", float* __restrict__ red_ws";
+        if (fold_in_kernel) ps << ", u32* __restrict__ red_cnt";
         s << "#define KERNEL_PARAMS " << ps.str() << "\n";
     }
     // operand fetchers
@@ -1231,15 +1251,52 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
                 const RedOut& ro = red_of(oi);
                 if (!o.fold_n) {
                     finish << "for (u32 c = tid; c < BN; c += NTHREADS) {\nfloat r = 0.0f;\n#pragma unroll\nfor (int w = 0; w < WAVES_M; w++) r += red["
-                           << ci * t.wm * t.bn << " + w * BN + c];\nif (n0 + c < GN) red_ws[" << ro.off << "ull + ((size_t)bz * " << ro.parts
-                           << "u + tile_m) * GN + n0 + c] = r;\n}\n";
+                           << ci * t.wm * t.bn << " + w * BN + c];\nif (n0 + c < GN) " << (fold_in_kernel ? "HE_WS_STORE(red_ws + " : "red_ws[") << ro.off
+                           << "ull + ((size_t)bz * " << ro.parts << "u + tile_m) * GN + n0 + c" << (fold_in_kernel ? ", r);" : "] = r;") << "\n}\n";
                     ci++;
                 } else {
                     const int64_t per_b = ro.parts / o.b_div;  // partials per batch index: one per tile
                     finish << "if (tid == 0) {\nfloat r = 0.0f;\n#pragma unroll\nfor (int w = 0; w < WAVES_M * WAVES_N; w++) r += red["
-                           << ncol * t.wm * t.bn + si * t.wm * t.wn << " + w];\nred_ws[" << ro.off << "ull + (size_t)(bz / " << o.b_div << "u) * " << ro.parts
-                           << "u + (size_t)(bz % " << o.b_div << "u) * " << per_b << "u + tile_m * " << tiles_n << "u + tile_n] = r;\n}\n";
+                           << ncol * t.wm * t.bn + si * t.wm * t.wn << " + w];\n" << (fold_in_kernel ? "HE_WS_STORE(red_ws + " : "red_ws[") << ro.off
+                           << "ull + (size_t)(bz / " << o.b_div << "u) * " << ro.parts << "u + (size_t)(bz % " << o.b_div << "u) * " << per_b << "u + tile_m * "
+                           << tiles_n << "u + tile_n" << (fold_in_kernel ? ", r);" : "] = r;") << "\n}\n";
                     si++;
+                }
+            }
+            if (fold_in_kernel) {
+                // every partial of this workgroup has left the CU before its tickets are taken; whoever takes the last
+                // ticket of a counter finds all partials in memory, adds them in tile order, and leaves the counter at
+                // zero for the next launch
+                finish << "HE_WS_DRAIN();\n__syncthreads();\n__shared__ u32 red_last[2];\nif (tid == 0) {\n"
+                       << "u32* c0 = red_cnt + (size_t)bz * " << tiles_n << "u + tile_n;\nconst bool l0 = HE_WS_TICKET(c0) == " << tiles_m - 1 << "u;\nif (l0) HE_WS_STORE(c0, 0u);\nred_last[0] = l0;\n";
+                if (nsc) {
+                    // (scalar outputs of one kernel share b_div: one counter per element group)
+                    uint32_t b_div = 1;
+                    for (auto& o : pr.epi.outs)
+                        if (o.reduce && o.fold_m && o.fold_n) b_div = (uint32_t)o.b_div;
+                    finish << "u32* c1 = red_cnt + " << ticket_cols << "ull + bz / " << b_div << "u;\nconst bool l1 = HE_WS_TICKET(c1) == "
+                           << (uint64_t)b_div * tiles_m * tiles_n - 1 << "u;\nif (l1) HE_WS_STORE(c1, 0u);\nred_last[1] = l1;\n";
+                } else {
+                    finish << "red_last[1] = 0u;\n";
+                }
+                finish << "}\n__syncthreads();\n";
+                for (size_t oi = 0; oi < pr.epi.outs.size(); oi++) {
+                    const tp::Out& o = pr.epi.outs[oi];
+                    if (!o.reduce || !o.fold_m) continue;
+                    const RedOut& ro = red_of(oi);
+                    char scale[64];
+                    snprintf(scale, sizeof scale, "%.9ef", o.rop == tp::ROp::Mean ? (float)o.mean_scale : 1.0f);
+                    if (!o.fold_n) {
+                        finish << "if (red_last[0]) {\nfor (u32 c = tid; c < BN; c += NTHREADS) {\nif (n0 + c < GN) {\nfloat r = 0.0f;\n#pragma unroll 8\nfor (u32 p = 0; p < "
+                               << ro.parts << "u; p++) r += HE_WS_LOAD(red_ws + " << ro.off << "ull + ((size_t)bz * " << ro.parts << "u + p) * GN + n0 + c);\na"
+                               << o.arg << "[(size_t)bz * GN + n0 + c] = r * " << scale << ";\n}\n}\n}\n";
+                    } else {
+                        // one thread per partial (at most 4096), then the waves' sums in order
+                        finish << "if (red_last[1]) {\nfloat r = 0.0f;\nfor (u32 p = tid; p < " << ro.parts << "u; p += NTHREADS) r += HE_WS_LOAD(red_ws + " << ro.off
+                               << "ull + (size_t)(bz / " << o.b_div << "u) * " << ro.parts << "u + p);\nr = wave_reduce<0, 64>(r);\n__syncthreads();\nif (lane == 0) red[wave] = r;\n__syncthreads();\n"
+                               << "if (tid == 0) {\nfloat total = 0.0f;\nfor (int w = 0; w < WAVES_M * WAVES_N; w++) total += red[w];\na" << o.arg << "[bz / " << o.b_div
+                               << "u] = total * " << scale << ";\n}\n}\n";
+                    }
                 }
             }
         }
@@ -1357,7 +1414,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
           << "u; sp += 8u) acc += ws[(size_t)sp * total + i];\n}\npart[pg * 32u + e] = acc;\n__syncthreads();\n"
           << "if (pg == 0 && i < total) {\nfloat r = 0.0f;\n#pragma unroll\nfor (int q = 0; q < 8; q++) r += part[q * 32 + e];\nfloat one[1] = {r};\nst_vec<1>(out + i, one);\n}\n}\n";
     }
-    if (!reds.empty()) {
+    if (!reds.empty() && !fold_in_kernel) {
         // Second launch: one workgroup folds EB output elements, PG = 256 / EB threads share the partials of each
         // (thread q takes partials q, q + PG, ...), then one thread adds the PG sums in order: the same order every run.
         s << "template <int EB, bool CONTIG>\n__device__ __forceinline__ void fold_partials(const float* __restrict__ ws, float* __restrict__ out, u32 n, u32 parts, "
@@ -1399,10 +1456,10 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     std::string reduce_args;
     for (int a : reduce_outs_) reduce_args += (reduce_args.empty() ? "" : ",") + std::to_string(a);
     describe_ = strfmt("gemm [%lld,%lld,%lld]x[%lld] tile=%dx%dx%d stages=%d waves=%dx%d threads=%d grid=%ux%u rawA=%d rawB=%d NVA=%d NVB=%d NVE=%d "
-                       "direct=%d%d mma=%s epilogue_exprs=%zu outs=%zu split_k=%d reduce_ws=%llu reduce_grid=%u reduce_args=[%s]",
+                       "direct=%d%d mma=%s epilogue_exprs=%zu outs=%zu split_k=%d reduce_ws=%llu reduce_grid=%u reduce_args=[%s] reduce_counters=%llu",
                        (long long)pr.batch, (long long)pr.M, (long long)pr.K, (long long)pr.N, t.bm, t.bn, t.bk, t.stages, t.wm, t.wn, threads,
                        grid_[0], grid_[1], (int)raw_a, (int)raw_b, nva, nvb, nve, (int)direct_a, (int)direct_b, dtype_name(pr.mma_dtype), pr.epi.exprs.size(),
-                       pr.epi.outs.size(), pr.split_k, (unsigned long long)reduce_floats_, reduce_grid_, reduce_args.c_str());
+                       pr.epi.outs.size(), pr.split_k, (unsigned long long)reduce_floats_, reduce_grid_, reduce_args.c_str(), (unsigned long long)reduce_counters_);
     kernel_.reset(new JitKernel(source_, "fused_matmul", {"-ffp-contract=fast", "-munsafe-fp-atomics"}));
     if (pr.split_k > 1) finalize_.reset(new JitKernel(source_, "fused_matmul_finalize", {"-ffp-contract=fast", "-munsafe-fp-atomics"}));
     if (reduce_grid_) reduce_.reset(new JitKernel(source_, "fused_matmul_reduce", {"-ffp-contract=fast"}));
@@ -1410,8 +1467,11 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
 
 GemmKernel::~GemmKernel() { scratch_.release(); }
 
+static uint64_t counters_offset(uint64_t n_floats) { return (n_floats * 4 + 255) & ~255ull; }  // as ReduceScratch lays them out
+
 size_t GemmKernel::scratch_bytes_needed() const {
     if (prob_.split_k > 1) return (size_t)prob_.split_k * prob_.M * prob_.N * 4;
+    if (reduce_counters_) return (size_t)(counters_offset(reduce_floats_) + reduce_counters_ * 4);
     return (size_t)reduce_floats_ * 4;
 }
 
@@ -1426,9 +1486,10 @@ bool GemmKernel::loaded() const {
 }
 
 void GemmKernel::execute(void* const* ptrs, hipStream_t stream) {
-    float* ws = nullptr;
-    if (const size_t need = scratch_bytes_needed()) ws = scratch_.get(need / 4, 0, stream).floats;
-    run(ptrs, stream, ws);
+    ReduceScratch::Buf ws{nullptr, nullptr};
+    if (reduce_counters_) ws = scratch_.get(reduce_floats_, reduce_counters_, stream);  // (counters start at zero and are left there)
+    else if (const size_t need = scratch_bytes_needed()) ws = scratch_.get(need / 4, 0, stream);
+    run(ptrs, stream, ws.floats, reduce_counters_ ? ws.counters : nullptr);
 }
 
 void GemmKernel::execute_in_scratch(void* const* ptrs, hipStream_t stream, void* scratch, size_t scratch_bytes) {
@@ -1437,11 +1498,17 @@ void GemmKernel::execute_in_scratch(void* const* ptrs, hipStream_t stream, void*
     HE_REQUIRE(need <= scratch_bytes, HE_ERR_INVALID,
                "the kernel needs %zu bytes of scratch for its partial results, the buffer holds %zu", need, scratch_bytes);
     HE_REQUIRE(!need || (scratch && ((uintptr_t)scratch & 255) == 0), HE_ERR_INVALID, "scratch buffer missing or not 256-byte aligned");
-    // every partial the second launch reads is written by the first: nothing has to be cleared
-    run(ptrs, stream, need ? (float*)scratch : nullptr);
+    // every partial that is read is written by the same call first: only arrival counters have to be cleared (the buffer
+    // is shared with whatever ran before)
+    uint32_t* counters = nullptr;
+    if (reduce_counters_) {
+        counters = (uint32_t*)((char*)scratch + counters_offset(reduce_floats_));
+        fill_buffers({{counters, {(uint32_t)reduce_counters_, 0u}}}, stream);
+    }
+    run(ptrs, stream, need ? (float*)scratch : nullptr, counters);
 }
 
-void GemmKernel::run(void* const* ptrs, hipStream_t stream, float* ws) {
+void GemmKernel::run(void* const* ptrs, hipStream_t stream, float* ws, uint32_t* counters) {
     const size_t nargs = prob_.args.size();
     for (size_t i = 0; i < nargs; i++) {
         HE_REQUIRE(ptrs[i] != nullptr, HE_ERR_INVALID, "kernel argument %zu is null", i);
@@ -1449,6 +1516,7 @@ void GemmKernel::run(void* const* ptrs, hipStream_t stream, float* ws) {
     }
     std::vector<void*> holders(ptrs, ptrs + nargs);
     if (ws) holders.push_back(ws);
+    if (counters) holders.push_back(counters);
     std::vector<void*> argv(holders.size());
     for (size_t i = 0; i < holders.size(); i++) argv[i] = &holders[i];
     const uint32_t block[3] = {threads_, 1, 1};

@@ -147,7 +147,7 @@ public:
     ~GemmKernel() override;
 
 private:
-    void run(void* const* ptrs, hipStream_t stream, float* ws);
+    void run(void* const* ptrs, hipStream_t stream, float* ws, uint32_t* counters);
     GemmProblem prob_;
     std::string source_, describe_;
     // finalize_: adds up the partial tiles of a split-k product; reduce_: folds the partials of the epilogue's reductions
@@ -156,6 +156,7 @@ private:
     uint32_t threads_ = 256;
     uint32_t reduce_grid_ = 0;
     uint64_t reduce_floats_ = 0;
+    uint64_t reduce_counters_ = 0;  // arrival counters of reductions that fold inside the kernel (no reduce_ launch then)
     std::vector<int> reduce_outs_;  // kernel arguments the reduce launch writes, in its parameter order
     ReduceScratch scratch_;
 };

@@ -22,6 +22,15 @@ def launch_gemm(k, bufs):
     gx, gy = map(int, re.search(r"grid=(\d+)x(\d+)", k.description).groups())
     threads = int(re.search(r"threads=(\d+)", k.description).group(1))
     ws_floats, reduce_grid = map(int, re.search(r"reduce_ws=(\d+) reduce_grid=(\d+)", k.description).groups())
+    counters = int(re.search(r"reduce_counters=(\d+)", k.description).group(1))
+    if counters:
+        # the reductions fold inside the kernel: the last workgroup to arrive at a counter adds the partials, and leaves
+        # the counter at zero for the next launch
+        assert not reduce_grid
+        res = run_kernel(k.source, "fused_matmul", gx, threads,
+                         bufs + [(np.full(ws_floats, np.nan, dtype=np.float32), 2), (np.zeros(counters, dtype=np.uint32), 2)], grid_y=gy)
+        assert not res[-1].any(), "arrival counters are not back at zero"
+        return res[:-2]
     if not reduce_grid:
         return run_kernel(k.source, "fused_matmul", gx, threads, bufs, grid_y=gy)
     res = run_kernel(k.source, "fused_matmul", gx, threads, bufs + [(np.full(ws_floats, np.nan, dtype=np.float32), 2)], grid_y=gy)
