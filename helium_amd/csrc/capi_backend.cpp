@@ -22,7 +22,7 @@ int he_matmul_kernel_create(he_tile_kernel_t* kernel, he_graph_t graph, const ui
         HE_REQUIRE(kernel && graph && nodes && num_nodes > 0, HE_ERR_INVALID, "bad argument");
         he::ir::OpSubgraph sg(graph->g, std::vector<he::ir::NodeId>(nodes, nodes + num_nodes));
         auto k = std::make_unique<he_tile_kernel_s>();
-        k->k.reset(new he::GemmKernel(he::plan::gemm_problem_from_ir(sg)));
+        k->k = he::plan::make_gemm_kernel(sg);
         if (he::device_initialised()) k->k->load();  // so that later launches need not
         *kernel = k.release();
     });

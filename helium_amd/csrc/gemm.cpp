@@ -834,6 +834,8 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
             if (pr.M > 64 && pr.N > 64 && ((pr.M + 127) / 128) * ((pr.N + 127) / 128) * pr.batch * pr.split_k < 128) t.bm = t.bn = 64;
         }
     }
+    HE_REQUIRE(!pr.out_rows.on || (pr.split_k == 1 && pr.batch == 1 && pr.epi.outs.size() == 1 && !pr.epi.outs[0].reduce), HE_ERR_INVALID,
+               "scattered output rows need a plain epilogue and a whole k range");
     HE_REQUIRE(t.bm % (t.wm * 32) == 0 && t.bn % (t.wn * 32) == 0 && (t.bk == 64 || t.bk == 32) && (!f32 || t.bk == 32), HE_ERR_INVALID, "bad GEMM tile");
     const int threads = t.wm * t.wn * 64;
     HE_REQUIRE(threads == 64 || threads == 128 || threads == 256 || threads == 512, HE_ERR_INVALID, "GEMM workgroups have 1, 2, 4 or 8 waves");
@@ -1102,6 +1104,11 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         else emit_elementwise_gather(pr.conv_b);  // the filter gradient of a 3-channel image: B[pixel][(r, s, c)]
     } else if (pr.b_rows.on) {
         const auto& br = pr.b_rows;
+        if (br.s_count > 0)
+            s << "__device__ __forceinline__ size_t b_row_addr(u32 k) { const u32 rs = k / " << br.group << "u; return (size_t)(k % " << br.group << "u) * "
+              << br.o_stride << "ull + " << br.base << "ull + (size_t)(rs / " << br.s_count << "u) * " << br.r_stride << "ull + (size_t)(rs % " << br.s_count
+              << "u) * " << br.s_stride << "ull; }\n";
+        else
         s << "__device__ __forceinline__ size_t b_row_addr(u32 k) { return (size_t)(k % " << br.group << "u) * " << br.o_stride << "ull + (size_t)(k / "
           << br.group << "u) * " << br.rs_stride << "ull; }\n";
         s << "#define FETCH_B_ARGS p" << pr.map_b[0] << ", \n#define RAW_B 1\n#define SPLIT_B 1\n";
@@ -1187,6 +1194,12 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
                 const tp::Out& o = pr.epi.outs[oi];
                 const std::string v = "e" + std::to_string(o.expr);
                 if (!o.reduce) {
+                    if (pr.out_rows.on) {
+                        const auto& orow = pr.out_rows;
+                        b << "{ const u32 on_ = m / " << orow.P * orow.Q << "u, opq = m % " << orow.P * orow.Q << "u, op_ = opq / " << orow.Q << "u, oq = opq % " << orow.Q
+                          << "u;\nst_vec<NVE>(a" << o.arg << " + (((size_t)on_ * " << orow.H << "u + op_ * " << orow.sh << "u + " << orow.a << "u) * " << orow.W << "u + oq * "
+                          << orow.sw << "u + " << orow.b << "u) * GN + nn, " << v << "); }\n";
+                    } else
                     b << "st_vec<NVE>(a" << o.arg << " + ((size_t)bz * GM + m) * GN + nn, " << v << ");\n";
                 } else if (o.fold_m && !o.fold_n) {
                     b << "#pragma unroll\nfor (int k = 0; k < NVE; k++) rc" << oi << "[step % " << colsets << "][k] += " << v << "[k];\n";
@@ -1536,6 +1549,53 @@ void GemmKernel::run(void* const* ptrs, hipStream_t stream, float* ws, uint32_t*
         const uint32_t rgrid[3] = {reduce_grid_, 1, 1}, rblock[3] = {256, 1, 1};
         reduce_->launch(rgrid, rblock, 0, stream, rargv.data(), true);
     }
+}
+
+CompositeKernel::CompositeKernel(std::vector<std::unique_ptr<KernelBase>> parts, bool zero_outputs_first)
+    : parts_(std::move(parts)), zero_first_(zero_outputs_first) {
+    HE_REQUIRE(!parts_.empty(), HE_ERR_INTERNAL, "a composite kernel needs a part");
+    for (auto& p : parts_) {
+        HE_REQUIRE(p->args().size() == parts_[0]->args().size(), HE_ERR_INTERNAL, "the parts of a composite kernel take different arguments");
+        // (sources and descriptions one after the other, each introduced by a line that names the part)
+        source_ += "// ---- part " + std::to_string(&p - &parts_[0]) + " of " + std::to_string(parts_.size()) + "\n" + p->source() + "\n";
+        describe_ += (describe_.empty() ? "" : "\n") + p->describe();
+    }
+    describe_ = "composite parts=" + std::to_string(parts_.size()) + " zero_first=" + (zero_first_ ? "1" : "0") + "\n" + describe_;
+}
+
+void CompositeKernel::zero_outputs(void* const* ptrs, hipStream_t stream) const {
+    std::vector<std::pair<void*, std::pair<uint32_t, uint32_t>>> fills;
+    const auto& a = args();
+    for (size_t i = 0; i < a.size(); i++)
+        if (a[i].is_output) fills.push_back({ptrs[i], {(uint32_t)(storage_bytes(a[i].dtype, (size_t)a[i].numel) / 4), 0u}});
+    if (!fills.empty()) fill_buffers(fills, stream);
+}
+
+void CompositeKernel::execute(void* const* ptrs, hipStream_t stream) {
+    if (zero_first_) zero_outputs(ptrs, stream);
+    for (auto& p : parts_) p->execute(ptrs, stream);
+}
+
+void CompositeKernel::execute_in_scratch(void* const* ptrs, hipStream_t stream, void* scratch, size_t scratch_bytes) {
+    if (zero_first_) zero_outputs(ptrs, stream);
+    for (auto& p : parts_) p->execute_in_scratch(ptrs, stream, scratch, scratch_bytes);  // (one after the other: they may share it)
+}
+
+size_t CompositeKernel::scratch_bytes_needed() const {
+    size_t need = 0;
+    for (auto& p : parts_) need = std::max(need, p->scratch_bytes_needed());
+    return need;
+}
+
+void CompositeKernel::load() {
+    for (auto& p : parts_) p->load();
+    if (zero_first_) load_fill_kernel();
+}
+
+bool CompositeKernel::loaded() const {
+    for (auto& p : parts_)
+        if (!p->loaded()) return false;
+    return !zero_first_ || fill_kernel_loaded();
 }
 
 }  // namespace he

@@ -112,10 +112,21 @@ struct GemmProblem {
     int split_k = 1;
     // B rows that are not consecutive in memory: row k = rs * group + o lives at element o * o_stride + rs * rs_stride
     // (the filter [o][r][s][c] seen as the [(r, s, o)][c] matrix of ConvBackwardData). Columns stay contiguous.
+    // With s_count > 0 only every few taps are used (one class of a strided data gradient): tap index rs = k / group
+    // stands for tap (rs / s_count, rs % s_count) of the classes's own grid and the row lives at
+    // o * o_stride + base + (rs / s_count) * r_stride + (rs % s_count) * s_stride.
     struct RowGather {
         bool on = false;
         int64_t group = 1, o_stride = 0, rs_stride = 0;
+        int64_t s_count = 0, r_stride = 0, s_stride = 0, base = 0;
     } b_rows;
+    // Output rows that are not consecutive in memory: row m = (n, p, q) over a P x Q grid is pixel (p * sh + a, q * sw + b)
+    // of an H x W image of N-element pixels (one class of a strided data gradient writes every sh-th row and sw-th
+    // column of the gradient). Needs a plain epilogue (one full-size output) and no split k range.
+    struct OutRows {
+        bool on = false;
+        int64_t P = 0, Q = 0, H = 0, W = 0, sh = 1, sw = 1, a = 0, b = 0;
+    } out_rows;
     int root_a = -1, root_b = -1;  // expression ids of the operand values in op_a / op_b
     std::vector<tp::Arg> args;     // the kernel's arguments: inputs in node order, then outputs in node order
     std::vector<int> map_a, map_b, map_e;  // program argument -> kernel argument
@@ -159,6 +170,28 @@ private:
     uint64_t reduce_counters_ = 0;  // arrival counters of reductions that fold inside the kernel (no reduce_ launch then)
     std::vector<int> reduce_outs_;  // kernel arguments the reduce launch writes, in its parameter order
     ReduceScratch scratch_;
+};
+
+// Several kernels with one argument list, launched one after the other on the same stream (the classes of a strided
+// data gradient). `zero_outputs_first`: the kernels do not write every element of the outputs; the rest is zero.
+class CompositeKernel : public KernelBase {
+public:
+    CompositeKernel(std::vector<std::unique_ptr<KernelBase>> parts, bool zero_outputs_first);
+    const std::vector<tp::Arg>& args() const override { return parts_[0]->args(); }
+    const std::string& source() const override { return source_; }
+    const std::string& describe() const override { return describe_; }
+    void execute(void* const* ptrs, hipStream_t stream) override;
+    void execute_in_scratch(void* const* ptrs, hipStream_t stream, void* scratch, size_t scratch_bytes) override;
+    size_t scratch_bytes_needed() const override;
+    void load() override;
+    bool loaded() const override;
+    const std::vector<std::unique_ptr<KernelBase>>& parts() const { return parts_; }
+
+private:
+    void zero_outputs(void* const* ptrs, hipStream_t stream) const;
+    std::vector<std::unique_ptr<KernelBase>> parts_;
+    bool zero_first_;
+    std::string source_, describe_;
 };
 
 }  // namespace he

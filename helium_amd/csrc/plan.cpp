@@ -43,6 +43,7 @@ bool enumerate_swaps(const ir::OpSubgraph& sg, std::vector<std::pair<int, int>>*
     return true;
 }
 
+std::unique_ptr<KernelBase> make_gemm_kernel(const ir::OpSubgraph& sg);
 namespace {
 std::atomic<bool> g_fuse_matmul_epilogue{true};
 std::atomic<bool> g_fold_swap_into_reduce{true};
@@ -197,7 +198,7 @@ void Instr::precompile() const {
             break;
         case InstrKind::Gemm:
             kernel_ = g_tile_kernels.get_or_insert(tuning::key() + "mm:" + sg_.cache_key(), [&] {
-                return std::shared_ptr<KernelBase>(new GemmKernel(gemm_problem_from_ir(sg_)));
+                return std::shared_ptr<KernelBase>(make_gemm_kernel(sg_));
             });
             break;
         case InstrKind::Permute: {
@@ -753,7 +754,13 @@ namespace {
 // k = (r, s, o). A is gathered from the flow (the gradient of the forward output): tap (r, s) of pixel (h, w) reads
 // flow[n][(h + ph - r*dh) / sh][(w + pw - s*dw) / sw][o] where that pixel exists; B's row (r, s, o) is the filter's
 // [o][r][s][:] row of input channels, picked out of the [out, kh, kw, in] tensor where it lies.
-GemmProblem conv_backward_data_problem(const ir::OpSubgraph& sg, NodeId node) {
+// `cls` < 0: the whole gradient as one product, every row testing every tap for divisibility by the stride. Otherwise
+// class cls = a * stride_w + b: the pixels (h, w) with h % stride_h == a and w % stride_w == b. Of the taps only
+// r = r0 + stride_h * r' (r0 = (a + pad) % stride_h) reach such a row, and with h = stride_h * i + a the flow row is
+// i + (a + pad - r0) / stride_h - r': a stride-1 data gradient over the class's own grid of pixels with every
+// stride-th tap of the filter, whose rows land on every stride-th pixel of the output. `empty` (if given) tells that
+// no tap reaches the class: those pixels of the gradient are zero.
+GemmProblem conv_backward_data_problem(const ir::OpSubgraph& sg, NodeId node, int cls = -1, bool* empty = nullptr) {
     const ir::OpGraph& g = *sg.graph();
     HE_REQUIRE(sg.nodes().size() == 1, HE_ERR_UNSUPPORTED, "a convolution instruction holds the op alone");
     const ir::Op& op = g.get(node).op;
@@ -777,18 +784,45 @@ GemmProblem conv_backward_data_problem(const ir::OpSubgraph& sg, NodeId node) {
     cv.ph = pad[0]; cv.pw = pad[1];
     const int64_t in_channels = op.conv.in_channels;
     pr.batch = 1;
+    int64_t r0 = 0, s0 = 0;
+    const int64_t full_r = cv.R, full_s = cv.S, image_h = cv.P, image_w = cv.Q, stride_h = cv.sh, stride_w = cv.sw;
+    if (cls >= 0) {
+        const int64_t a = cls / stride_w, b = cls % stride_w;
+        r0 = (a + cv.ph) % stride_h;
+        s0 = (b + cv.pw) % stride_w;
+        cv.R = r0 < full_r ? (full_r - r0 + stride_h - 1) / stride_h : 0;
+        cv.S = s0 < full_s ? (full_s - s0 + stride_w - 1) / stride_w : 0;
+        cv.P = a < image_h ? (image_h - a + stride_h - 1) / stride_h : 0;
+        cv.Q = b < image_w ? (image_w - b + stride_w - 1) / stride_w : 0;
+        cv.ph = (a + cv.ph - r0) / stride_h;
+        cv.pw = (b + cv.pw - s0) / stride_w;
+        cv.sh = cv.sw = 1;
+        pr.out_rows.on = true;
+        pr.out_rows.P = cv.P; pr.out_rows.Q = cv.Q;
+        pr.out_rows.H = image_h; pr.out_rows.W = image_w;
+        pr.out_rows.sh = stride_h; pr.out_rows.sw = stride_w;
+        pr.out_rows.a = a; pr.out_rows.b = b;
+        if (empty) *empty = cv.R == 0 || cv.S == 0 || cv.P == 0 || cv.Q == 0;
+        if (cv.R == 0 || cv.S == 0 || cv.P == 0 || cv.Q == 0) return pr;
+    }
     pr.M = cv.N * cv.P * cv.Q;
     pr.N = in_channels;
     pr.K = cv.R * cv.S * cv.C;
-    pr.split_k = choose_split_k(pr.M, pr.N, pr.K, 1);
+    pr.split_k = cls >= 0 ? 1 : choose_split_k(pr.M, pr.N, pr.K, 1);
     HE_REQUIRE(pr.M > 0 && pr.M < (1ll << 31) && ir::num_elements(flow.shape) < (1ll << 32), HE_ERR_UNSUPPORTED, "conv too large for 32-bit tile indices");
     pr.mma_dtype = flow.dtype == HE_F32 ? HE_F32 : flow.dtype == HE_F16 ? HE_F16 : HE_BF16;
     HE_REQUIRE(in_channels % (pr.mma_dtype == HE_F32 ? 4 : 8) == 0, HE_ERR_UNSUPPORTED,
                "conv backward data needs an input-channel count that fills 16-byte chunks");
     pr.b_rows.on = true;
     pr.b_rows.group = cv.C;                                 // k = (r*S + s) * out_channels + o
-    pr.b_rows.o_stride = cv.R * cv.S * in_channels;         // filter[o][..]
+    pr.b_rows.o_stride = full_r * full_s * in_channels;     // filter[o][..]
     pr.b_rows.rs_stride = in_channels;                      // filter[.][r][s][..]
+    if (cls >= 0) {                                         // filter[.][r0 + stride_h * r'][s0 + stride_w * s'][..]
+        pr.b_rows.s_count = cv.S;
+        pr.b_rows.base = (r0 * full_s + s0) * in_channels;
+        pr.b_rows.r_stride = stride_h * full_s * in_channels;
+        pr.b_rows.s_stride = stride_w * in_channels;
+    }
     auto operand = [&](tp::Program& p, const ir::Descriptor& d, NodeId n, int64_t rows, int64_t cols) {
         p.dims = {1, rows, cols};
         p.args.push_back({d.dtype, ir::num_elements(d.shape), false, n});
@@ -896,6 +930,37 @@ GemmProblem conv_backward_filter_problem(const ir::OpSubgraph& sg, NodeId node) 
     return pr;
 }
 }  // namespace
+
+std::vector<GemmProblem> strided_data_gradient_classes(const ir::OpSubgraph& sg, bool* any_empty) {
+    const ir::OpGraph& g = *sg.graph();
+    *any_empty = false;
+    if (sg.nodes().size() != 1 || tuning::get("HELIUM_HIP_GEMM_NO_STRIDE_CLASSES")) return {};
+    const ir::Op& op = g.get(sg.nodes()[0]).op;
+    if (op.kind != ir::OpKind::ConvBackwardData || (op.conv.stride[0] == 1 && op.conv.stride[1] == 1) || op.conv.dilation[0] != 1 ||
+        op.conv.dilation[1] != 1 || op.conv.stride[0] > 4 || op.conv.stride[1] > 4)
+        return {};
+    std::vector<GemmProblem> out;
+    for (int cls = 0; cls < (int)(op.conv.stride[0] * op.conv.stride[1]); cls++) {
+        bool empty = false;
+        GemmProblem pr = conv_backward_data_problem(sg, sg.nodes()[0], cls, &empty);
+        if (empty) *any_empty = true;
+        else out.push_back(std::move(pr));
+    }
+    return out;
+}
+
+std::unique_ptr<KernelBase> make_gemm_kernel(const ir::OpSubgraph& sg) {
+    // The data gradient of a strided convolution is one product per class of pixels (row and column modulo the
+    // stride): each multiplies only the taps that reach its pixels.
+    bool any_empty = false;
+    std::vector<GemmProblem> classes = strided_data_gradient_classes(sg, &any_empty);
+    if (!classes.empty()) {
+        std::vector<std::unique_ptr<KernelBase>> parts;
+        for (auto& pr : classes) parts.emplace_back(new GemmKernel(std::move(pr)));
+        return std::unique_ptr<KernelBase>(new CompositeKernel(std::move(parts), any_empty));
+    }
+    return std::unique_ptr<KernelBase>(new GemmKernel(gemm_problem_from_ir(sg)));
+}
 
 GemmProblem gemm_problem_from_ir(const ir::OpSubgraph& sg) {
     const ir::OpGraph& g = *sg.graph();

@@ -102,5 +102,11 @@ void plan_cache_stats(uint64_t* hits, uint64_t* misses);
 // GEMM problem of a Matmul-anchored helium-ir subgraph (MatmulGenerator::new,
 // helium-kernel-generator/src/generators/matmul.rs:88-130). Throws HE_ERR_UNSUPPORTED for an UnsupportedFusion.
 GemmProblem gemm_problem_from_ir(const ir::OpSubgraph& sg);
+// For a subgraph that is one ConvBackwardData with a stride: one product per class of output pixels (row and column
+// modulo the stride), each over the taps that reach the class; empty otherwise. `any_empty`: some class is reached by
+// no tap, so its pixels have to be zeroed.
+std::vector<GemmProblem> strided_data_gradient_classes(const ir::OpSubgraph& sg, bool* any_empty);
+// The kernel of a Gemm instruction: one fused GEMM, or the classes of a strided data gradient one after the other.
+std::unique_ptr<KernelBase> make_gemm_kernel(const ir::OpSubgraph& sg);
 
 }  // namespace he::plan

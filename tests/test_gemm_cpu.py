@@ -188,8 +188,32 @@ def test_ir_matmul_on_cpu(name, sa, sb, precision, dtype, tol):
     assert np.abs(got - want).max() <= tol, (k.description, np.abs(got - want).max())
 
 
+class _Part:
+    """One kernel of a composite kernel object (the classes of a strided data gradient), with its own source and
+    description and the composite's argument list."""
+
+    def __init__(self, source, description, args):
+        self.source, self.description, self.args = source, description, args
+
+
 def run_ir_kernel_on_cpu(g, nodes, inputs):
     k = ha.backend.matmul_kernel(g, nodes)
+    if k.description.startswith("composite"):
+        head, *lines = k.description.split("\n")
+        parts, zero_first = (int(v) for v in re.search(r"parts=(\d+) zero_first=(\d)", head).groups())
+        sources = re.split(r"// ---- part \d+ of \d+\n", k.source)[1:]
+        assert len(sources) == len(lines) == parts
+        outs = [a for a in k.args if a["is_output"]]
+        # what no part writes has to be zeroed first by the host; where every element is written the buffer starts as
+        # NaN here, so an element that no part wrote shows
+        current = {a["node"]: (np.zeros(a["numel"], dtype=nm.NP_STORAGE[a["dtype"]]) if zero_first
+                               else nm.to_storage(np.full(a["numel"], np.nan, dtype=np.float32), a["dtype"])) for a in outs}
+        for src, line in zip(sources, lines):
+            part = _Part(src, line, k.args)
+            bufs = [(current[a["node"]], 2) if a["is_output"] else (inputs[a["node"]], 0) for a in k.args]
+            for a, r in zip(outs, launch_gemm(part, bufs)):
+                current[a["node"]] = r
+        return k, {a["node"]: nm.from_storage(current[a["node"]], a["dtype"], [current[a["node"]].size]).astype(np.float64) for a in outs}
     gx, gy = map(int, re.search(r"grid=(\d+)x(\d+)", k.description).groups())
     threads = int(re.search(r"threads=(\d+)", k.description).group(1))
     split = int(re.search(r"split_k=(\d+)", k.description).group(1))
@@ -316,6 +340,11 @@ BWD_DATA_CASES = [
     ("valid_and_dilated_f32", (1, 9, 9, 4), 8, (3, 3), "f32", (1, 1), (2, 1), "valid", "64,64,32,2,2"),
     ("hoisted_pixel_terms_stride2", (2, 10, 9, 16), 64, (3, 3), "bf16", (2, 2), (1, 1), "same", "128,128,64,2,2"),
     ("flow_gathered_element_by_element", (1, 9, 8, 16), 12, (3, 3), "bf16", (2, 1), (1, 1), "same", "64,64,64,2,2"),
+    # one product per class of pixels (row and column modulo the stride): classes of 3x3, 3x2, 2x3 and 2x2 taps
+    ("5x5_stride2_classes", (2, 11, 12, 8), 16, (5, 5), "bf16", (2, 2), (1, 1), "same", "64,64,64,2,2"),
+    # ... of 1 to 4 taps per dim, one class that no tap reaches in valid mode; image extents that the stride does not divide
+    ("3x3_stride3_valid_classes", (1, 10, 11, 8), 16, (3, 3), "bf16", (3, 3), (1, 1), "valid", "64,64,64,2,2"),
+    ("7x7_stride2_full_f32", (1, 9, 10, 4), 8, (7, 7), "f32", (2, 2), (1, 1), "full", "64,64,32,2,2"),
 ]
 
 
@@ -343,6 +372,7 @@ def test_conv_backward_data_on_cpu(name, image, oc, kernel, dtype, stride, dilat
         k, got = run_ir_kernel_on_cpu(g, [dx], inputs)
     finally:
         del os.environ["HELIUM_HIP_GEMM_TILE"]
+    assert k.description.startswith("composite") == (tuple(stride) != (1, 1) and tuple(dilation) == (1, 1)), k.description
     want = oracle_ir.kernel_outputs(g.nodes, inputs, [dx])[dx]
     want = nm.from_storage(want.reshape(-1), dtype, [want.size]).astype(np.float64)
     tol = 1e-4 if dtype == "f32" else 2e-2
