@@ -30,6 +30,7 @@ OPT_FOLD_SWAP_INTO_REDUCE = 1
 OPT_REMATERIALIZE = 2
 OPT_CANCEL_TRANSPOSES = 3
 OPT_HOIST_BROADCASTS = 4
+OPT_STREAM_FAN_OUT = 5  # 0 one stream, 1 where it pays (default), 2 every step with several instructions
 
 
 def set_option(option, value):

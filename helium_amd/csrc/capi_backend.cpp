@@ -150,6 +150,7 @@ int he_backend_set_option(int option, int64_t value) {
             case HE_OPT_REMATERIALIZE: he::plan::set_rematerialize(value != 0); break;
             case HE_OPT_CANCEL_TRANSPOSES: he::plan::set_cancel_transposes(value != 0); break;
             case HE_OPT_HOIST_BROADCASTS: he::plan::set_hoist_broadcasts(value != 0); break;
+            case HE_OPT_STREAM_FAN_OUT: he::exec::set_stream_fan_out((int)value); break;
             default: he::fail(HE_ERR_INVALID, "unknown backend option");
         }
     });

@@ -77,7 +77,8 @@ int mode() {
 bool is_override(const char* entry) {
     if (strncmp(entry, "HELIUM_HIP_", 11) != 0) return false;
     for (const char* other : {"HELIUM_HIP_TUNING=", "HELIUM_HIP_CACHE_DIR=", "HELIUM_HIP_DUMP_DIR=", "HELIUM_HIP_DUMP_FAILED=",
-                              "HELIUM_HIP_EXEC_TIMING=", "HELIUM_HIP_NO_LAUNCH_EVENTS="})
+                              "HELIUM_HIP_EXEC_TIMING=", "HELIUM_HIP_NO_LAUNCH_EVENTS=", "HELIUM_HIP_STREAMS=",
+                              "HELIUM_HIP_INSTR_TIMING=", "HELIUM_HIP_PLAN_DEBUG="})
         if (strncmp(entry, other, strlen(other)) == 0) return false;
     return true;
 }

@@ -213,7 +213,9 @@ Streams& thread_streams() {
     // a small pool of non-blocking streams per host thread (helium/src/cuda/context.rs:112-125)
     static thread_local Streams st;
     if (st.s.empty()) {
-        const int n = 4;
+        // HELIUM_HIP_STREAMS=<1..4>: how many streams the independent instructions of a step fan out over
+        const char* env = getenv("HELIUM_HIP_STREAMS");
+        const int n = env ? std::max(1, std::min(4, atoi(env))) : 4;
         for (int i = 0; i < n; i++) {
             hipStream_t x;
             HE_HIP(hipStreamCreateWithFlags(&x, hipStreamNonBlocking));
@@ -280,7 +282,40 @@ void retire_join_events(const std::vector<hipEvent_t>& events) {
 }
 thread_local double g_host_acc[8] = {0};
 thread_local int g_host_calls = 0;
+std::atomic<int> g_fan_out{1};
+
+// Whether the independent instructions of a step are worth a stream each. Putting work on a second stream costs a
+// join before and after it: on this runtime a hipStreamWaitEvent takes the host 15-20 us for the first stream that
+// waits on an event and about 7 us for each further one, and the device a few microseconds per dependent queue. What
+// it can gain is the time of instructions too small to fill the chip, which then run beside each other (or under an
+// instruction that does fill it): an instruction that moves more than a few MiB already uses every CU or all of the
+// memory bandwidth, and two of those side by side finish when they would have finished one after the other.
+bool fan_out_pays(const plan::Step& step, const ir::OpGraph& g) {
+    if (step.instrs.size() < 2) return false;
+    constexpr double kLaunchUs = 4, kBytesPerUs = 2e6, kNarrowBytes = 4 << 20, kJoinUs = 20;
+    double narrow_sum = 0, narrow_max = 0;
+    bool wide = false;
+    for (auto& instr : step.instrs) {
+        double bytes = 0;
+        for (NodeId n : instr->inputs()) bytes += (double)storage_bytes(g.get(n).desc.dtype, (size_t)ir::num_elements(g.get(n).desc.shape));
+        for (NodeId n : instr->outputs()) bytes += (double)storage_bytes(g.get(n).desc.dtype, (size_t)ir::num_elements(g.get(n).desc.shape));
+        if (bytes > kNarrowBytes) {
+            wide = true;
+            continue;
+        }
+        const double us = kLaunchUs + bytes / kBytesPerUs;
+        narrow_sum += us;
+        narrow_max = std::max(narrow_max, us);
+    }
+    const double gain = wide ? narrow_sum : narrow_sum - narrow_max;
+    return gain > 2 * kJoinUs;
+}
 }  // namespace
+
+void set_stream_fan_out(int mode) {
+    HE_REQUIRE(mode >= 0 && mode <= 2, HE_ERR_INVALID, "stream fan-out is 0 (never), 1 (where it pays) or 2 (always)");
+    g_fan_out.store(mode);
+}
 
 std::shared_ptr<const Prepared> prepare(const ir::OpGraph& graph_in) {
     auto pr = std::make_shared<Prepared>();
@@ -303,6 +338,15 @@ std::shared_ptr<const Prepared> prepare(const ir::OpGraph& graph_in) {
         for (auto& instr : step.instrs)
             for (NodeId o : instr->outputs()) pr->alive.insert(o);
         for (NodeId r : step.tensors_to_release) pr->alive.erase(r);
+        pr->fan_out.push_back(fan_out_pays(step, *pr->graph));
+    }
+    if (getenv("HELIUM_HIP_PLAN_DEBUG")) {
+        size_t fanned = 0, multi = 0;
+        for (size_t k = 0; k < pr->plan->steps.size(); k++) {
+            fanned += pr->fan_out[k];
+            multi += pr->plan->steps[k].instrs.size() > 1;
+        }
+        fprintf(stderr, "[plan] %zu steps, %zu with several instructions, %zu of them fan out over streams\n", pr->plan->steps.size(), multi, fanned);
     }
     return pr;
 }
@@ -359,11 +403,18 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
     };
     // An execution whose steps hold one instruction each runs on stream 0 alone: its last launch can carry the
     // execution's event itself.
+    const int fan_mode = g_fan_out.load();
+    auto step_width = [&](size_t k) {
+        const plan::Step& step = plan->steps[k];
+        const bool fan = fan_mode == 2 || (fan_mode == 1 && prepared.fan_out[k]);
+        return fan ? std::min(step.instrs.size(), st.s.size()) : std::min<size_t>(step.instrs.size(), 1);
+    };
     const plan::Instr* closing = nullptr;
     {
         bool one_stream = true;
-        for (auto& step : plan->steps) {
-            one_stream = one_stream && step.instrs.size() <= 1;
+        for (size_t k = 0; k < plan->steps.size(); k++) {
+            auto& step = plan->steps[k];
+            one_stream = one_stream && step_width(k) <= 1;
             if (!step.instrs.empty()) closing = step.instrs.back().get();
         }
         if (!one_stream || getenv("HELIUM_HIP_NO_LAUNCH_EVENTS")) closing = nullptr;
@@ -380,16 +431,19 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
     // earlier launches running on up to four streams. On failure stream 0 is ordered after every stream this execution
     // used, the end event is recorded there as usual, and the error goes on to the caller.
     try {
-    for (auto& step : plan->steps) {
+    for (size_t step_no = 0; step_no < plan->steps.size(); step_no++) {
+        auto& step = plan->steps[step_no];
         for (NodeId r : step.tensors_to_release) tensors.erase(r);
         if (step.instrs.empty()) continue;
         local.steps++;
         std::vector<const Tensor*> waited;
-        // Instructions of one step are independent: they fan out over the stream pool.
-        const size_t width = std::min(step.instrs.size(), st.s.size());
+        // Instructions of one step are independent: they fan out over the stream pool where that pays.
+        const size_t width = step_width(step_no);
         std::vector<size_t> cur(width);
         for (size_t w = 0; w < width; w++) cur[w] = w;
+        ht.lap(3);
         join(cur);
+        ht.lap(6);
         for (size_t i = 0; i < step.instrs.size(); i++) {
             const plan::Instr& instr = *step.instrs[i];
             hipStream_t stream = st.s[i % width];
@@ -509,8 +563,8 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
     if (HostTimer::on()) {
         for (int i = 0; i < 8; i++) g_host_acc[i] += ht.acc[i];
         if (++g_host_calls % 100 == 0) {
-            fprintf(stderr, "[exec timing] per graph, us: copy+optimize %.1f, plan lookup %.1f, setup %.1f, alloc+waits %.1f, launches %.1f, finish %.1f\n",
-                    g_host_acc[0] / 100, g_host_acc[1] / 100, g_host_acc[2] / 100, g_host_acc[3] / 100, g_host_acc[4] / 100, g_host_acc[5] / 100);
+            fprintf(stderr, "[exec timing] per graph, us: copy+optimize %.1f, plan lookup %.1f, setup %.1f, alloc+waits %.1f, joins %.1f, launches %.1f, finish %.1f\n",
+                    g_host_acc[0] / 100, g_host_acc[1] / 100, g_host_acc[2] / 100, g_host_acc[3] / 100, g_host_acc[6] / 100, g_host_acc[4] / 100, g_host_acc[5] / 100);
             for (double& v : g_host_acc) v = 0;
         }
     }

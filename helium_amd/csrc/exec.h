@@ -108,7 +108,12 @@ struct Prepared {
     // When the graph that runs is a rewritten form of the caller's (plan::graph_for_execution): its Input node for each
     // of the caller's, and the caller's Output node for each of its own. Empty when the ids are the caller's.
     std::map<NodeId, NodeId> input_of, caller_output;
+    std::vector<uint8_t> fan_out;  // per step of the plan: whether its instructions are worth a stream each
 };
+// 0: every instruction runs on one stream; 1 (default): the instructions of a step fan out over the thread's streams
+// where the work that can overlap outweighs the joins; 2: every step with several instructions fans out, as
+// cuda.rs:190-221 does.
+void set_stream_fan_out(int mode);
 std::shared_ptr<const Prepared> prepare(const ir::OpGraph& graph);
 std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std::map<NodeId, TensorRef>& inputs,
                                              ExecStats* stats = nullptr);

@@ -387,9 +387,14 @@ int he_fgraph_subdivide(he_fgraph_t graph, uint64_t* nodes, int32_t* portions, i
  * HE_OPT_HOIST_BROADCASTS (default 1): a pointwise op whose operands all are the same Broadcast of small tensors (or
  * Constants) is applied to the small tensors and its result broadcast - `(variance.broadcast_to(x.shape) + 1e-3).sqrt()`
  * (modules/batch_norm.rs:56) costs one square root per channel instead of one per element. 0 keeps the ops where they
- * were recorded. */
+ * were recorded.
+ * HE_OPT_STREAM_FAN_OUT (default 1): how the independent instructions of a plan step are spread over the calling
+ * thread's streams. 2: every step with several instructions fans out and the next step waits for all of its streams
+ * (helium/src/cuda.rs:190-221). 1: only steps whose instructions are too small to fill the device and numerous enough to
+ * outweigh the joins (each costs the host 15-20 us here); all others run on the first stream in plan order. 0: one
+ * stream. Takes effect from the next he_execute_graph; results do not depend on it. */
 enum { HE_OPT_FUSE_MATMUL_EPILOGUE = 0, HE_OPT_FOLD_SWAP_INTO_REDUCE = 1, HE_OPT_REMATERIALIZE = 2, HE_OPT_CANCEL_TRANSPOSES = 3,
-       HE_OPT_HOIST_BROADCASTS = 4 };
+       HE_OPT_HOIST_BROADCASTS = 4, HE_OPT_STREAM_FAN_OUT = 5 };
 int he_backend_set_option(int option, int64_t value);
 
 /* Counters of the last he_execute_graph on this thread: [0] steps run, [1] instructions, [2] streams used,

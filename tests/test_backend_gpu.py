@@ -106,12 +106,12 @@ def live_nodes(nodes):
 def test_random_graphs_execute(gpu, seed, grouping):
     """Random graphs of 8x8, 1024x1024 and 1100x1100 tensors through plan generation and the executor: steps with several
     instructions on several streams, scoped block reuse, and (from 1,000,000 elements) SwapDims chains that run as
-    permute instructions in the middle of a graph. With the reference's grouping rules the plan the library runs must
+    permute instructions in the middle of a graph. With the reference's grouping rules (and its use of one stream per
+    instruction of a step) the plan the library runs must
     be the one the CPU restatement of plan_generation.rs derives, and that plan - not the library's - tells the oracle
     where values are rounded to their storage type."""
     from helium_amd.backend import (OPT_CANCEL_TRANSPOSES, OPT_FOLD_SWAP_INTO_REDUCE, OPT_FUSE_MATMUL_EPILOGUE, OPT_HOIST_BROADCASTS,
-                                OPT_REMATERIALIZE,
-                                    set_option)
+                                    OPT_REMATERIALIZE, OPT_STREAM_FAN_OUT, set_option)
     from oracle import plan as oracle_plan
 
     g = plans.random_graph(seed)
@@ -131,9 +131,15 @@ def test_random_graphs_execute(gpu, seed, grouping):
     set_option(OPT_REMATERIALIZE, 0 if reference else 1)
     set_option(OPT_CANCEL_TRANSPOSES, 0 if reference else 1)
     set_option(OPT_HOIST_BROADCASTS, 0 if reference else 1)
+    # the reference puts every instruction of a step on a stream of its own (cuda.rs:190-221); by default only steps
+    # where that pays do
+    set_option(OPT_STREAM_FAN_OUT, 2 if reference else 1)
     try:
         got, steps = run_graph(g, host)
+        if reference and any(len(instrs) > 1 for instrs, _ in steps):
+            assert stats()["streams_used"] > 1
     finally:
+        set_option(OPT_STREAM_FAN_OUT, 1)
         set_option(OPT_FUSE_MATMUL_EPILOGUE, 1)
         set_option(OPT_FOLD_SWAP_INTO_REDUCE, 1)
         set_option(OPT_REMATERIALIZE, 1)
@@ -174,8 +180,7 @@ def test_random_graphs_cover_concurrent_steps_and_permute_instructions():
 @pytest.mark.parametrize("fuse", [1, 0], ids=["matmul_takes_its_epilogue", "reference_grouping"])
 def test_config1_linear_layer(gpu, fuse):
     from helium_amd.backend import (OPT_CANCEL_TRANSPOSES, OPT_FOLD_SWAP_INTO_REDUCE, OPT_FUSE_MATMUL_EPILOGUE, OPT_HOIST_BROADCASTS,
-                                OPT_REMATERIALIZE,
-                                    set_option)
+                                    OPT_REMATERIALIZE, OPT_STREAM_FAN_OUT, set_option)
 
     g, names = configs.c1_ir_graph()
     host = configs.c1_inputs(names, batched=False)

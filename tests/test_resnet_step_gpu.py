@@ -23,12 +23,19 @@ pytestmark = pytest.mark.gpu
 BATCH, IMAGE, WIDTH, CLASSES = 8, 64, 8, 16
 
 
-def _run(dtype):
+def _run(dtype, fan_out=1):
+    from helium_amd.backend import OPT_STREAM_FAN_OUT, set_option, stats
+
     r = resnet.record_training_step(BATCH, IMAGE, width=WIDTH, num_classes=CLASSES, dtype=dtype)
     G = r["graph"]
     by_id = {n["id"]: n for n in G.g.nodes}
     tensors = {i: Tensor.from_numpy(a, by_id[i]["dtype"], int(np.prod(by_id[i]["shape"]))) for i, a in G.feeds.items()}
-    got = {o: t.to_numpy() for o, t in execute_graph(G.g, tensors).items()}
+    set_option(OPT_STREAM_FAN_OUT, fan_out)
+    try:
+        got = {o: t.to_numpy() for o, t in execute_graph(G.g, tensors).items()}
+        assert (stats()["streams_used"] > 1) == (fan_out == 2)
+    finally:
+        set_option(OPT_STREAM_FAN_OUT, 1)
     # the executor plans the pruned graph: the oracle follows the plan of the same
     G.g.optimize()
     steps = Plan(G.g).steps
@@ -61,8 +68,9 @@ def _rel(a, b):
     return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
 
 
-def test_training_step_in_f32_matches_the_oracle_everywhere(gpu):
-    r, got, steps = _run("f32")
+@pytest.mark.parametrize("fan_out", [1, 2], ids=["streams_where_they_pay", "a_stream_per_instruction_of_a_step"])
+def test_training_step_in_f32_matches_the_oracle_everywhere(gpu, fan_out):
+    r, got, steps = _run("f32", fan_out)
     G = r["graph"]
     want = oracle_ir.plan_outputs(G.g.nodes, G.feeds, steps)
     _, desc = oracle_ir.evaluate(G.g.nodes, G.feeds)
