@@ -1571,14 +1571,34 @@ void CompositeKernel::zero_outputs(void* const* ptrs, hipStream_t stream) const 
     if (!fills.empty()) fill_buffers(fills, stream);
 }
 
+// Only the last part's last launch closes the instruction: an event that is pending for it is held back until then.
+namespace {
+struct HeldStopEvent {
+    hipEvent_t e = take_pending_stop_event();
+    void give_back() {
+        if (e) set_pending_stop_event(e);
+        e = nullptr;
+    }
+    ~HeldStopEvent() { give_back(); }
+};
+}  // namespace
+
 void CompositeKernel::execute(void* const* ptrs, hipStream_t stream) {
+    HeldStopEvent held;
     if (zero_first_) zero_outputs(ptrs, stream);
-    for (auto& p : parts_) p->execute(ptrs, stream);
+    for (auto& p : parts_) {
+        if (&p == &parts_.back()) held.give_back();
+        p->execute(ptrs, stream);
+    }
 }
 
 void CompositeKernel::execute_in_scratch(void* const* ptrs, hipStream_t stream, void* scratch, size_t scratch_bytes) {
+    HeldStopEvent held;
     if (zero_first_) zero_outputs(ptrs, stream);
-    for (auto& p : parts_) p->execute_in_scratch(ptrs, stream, scratch, scratch_bytes);  // (one after the other: they may share it)
+    for (auto& p : parts_) {
+        if (&p == &parts_.back()) held.give_back();
+        p->execute_in_scratch(ptrs, stream, scratch, scratch_bytes);  // (one after the other: they may share it)
+    }
 }
 
 size_t CompositeKernel::scratch_bytes_needed() const {
@@ -1596,6 +1616,117 @@ bool CompositeKernel::loaded() const {
     for (auto& p : parts_)
         if (!p->loaded()) return false;
     return !zero_first_ || fill_kernel_loaded();
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Convolutions over a repacked few-channel image
+// ---------------------------------------------------------------------------------------------------------
+RepackedConvKernel::RepackedConvKernel(std::vector<tp::Arg> args, ConvRepack geometry, std::unique_ptr<KernelBase> inner)
+    : args_(std::move(args)), geo_(geometry), inner_(std::move(inner)) {
+    const ConvRepack& c = geo_;
+    HE_REQUIRE(inner_->args().size() == args_.size(), HE_ERR_INTERNAL, "the product over repacked operands takes other arguments");
+    HE_REQUIRE(c.C >= 1 && c.C <= 4 && c.image_arg >= 0 && c.filter_arg >= 0, HE_ERR_INTERNAL, "bad repacking geometry");
+    const uint64_t pixels = (uint64_t)c.N * c.Hp * c.Wp, taps = (uint64_t)c.O * c.R * c.Sp;
+    HE_REQUIRE(pixels + taps < (1ull << 31), HE_ERR_UNSUPPORTED, "image too large to repack");
+    image_bytes_ = (size_t)((pixels * 8 + 255) & ~255ull);
+    filter_bytes_ = (size_t)((taps * (c.filter_gradient ? 4 * c.elem_bytes : 8) + 255) & ~255ull);
+    std::ostringstream s;
+    s << "// repacks a " << c.C << "-channel 16-bit image [" << c.N << "," << c.H << "," << c.W << "," << c.C << "] as [" << c.N << "," << c.Hp << "," << c.Wp
+      << ",4] with the padding (" << c.ph << "," << c.pw << ") written out" << (c.filter_gradient ? "" : ", and the filter alike") << "\n"
+      << "typedef unsigned short u16;\ntypedef unsigned int u32;\ntypedef unsigned long long u64;\n"
+      << "#define PIXELS " << pixels << "u\n#define TAPS " << taps << "u\n";
+    // one thread per pixel of the copy: up to 4 two-byte loads, one 8-byte store
+    s << "static __device__ __forceinline__ u64 pixel_of(const u16* __restrict__ src) {\nu64 v = 0;\n";
+    for (int ch = 0; ch < c.C; ch++) s << "v |= (u64)src[" << ch << "] << " << 16 * ch << ";\n";
+    s << "return v;\n}\n";
+    s << "extern \"C\" __global__ __launch_bounds__(256) void repack_conv_operands(const u16* __restrict__ image, "
+      << (c.filter_gradient ? "" : "const u16* __restrict__ filter, ") << "u64* __restrict__ image_p" << (c.filter_gradient ? "" : ", u64* __restrict__ filter_p") << ") {\n"
+      << "u32 t = blockIdx.x * 256u + threadIdx.x;\n"
+      << "if (t < PIXELS) {\n"
+      << "u32 w = t % " << c.Wp << "u, rest = t / " << c.Wp << "u, h = rest % " << c.Hp << "u, n = rest / " << c.Hp << "u;\n"
+      << "int hs = (int)h - " << c.ph << ", ws = (int)w - " << c.pw << ";\n"
+      << "u64 v = 0;\n"
+      << "if (hs >= 0 && hs < " << c.H << " && ws >= 0 && ws < " << c.W << ") v = pixel_of(image + ((u64)(n * " << c.H << "u + (u32)hs) * " << c.W << "u + (u32)ws) * " << c.C << "u);\n"
+      << "image_p[t] = v;\nreturn;\n}\n";
+    if (!c.filter_gradient)
+        s << "t -= PIXELS;\nif (t < TAPS) {\n"
+          << "u32 sp = t % " << c.Sp << "u, row = t / " << c.Sp << "u;\n"  // row = o * R + r
+          << "u64 v = 0;\nif (sp < " << c.S << "u) v = pixel_of(filter + ((u64)row * " << c.S << "u + sp) * " << c.C << "u);\n"
+          << "filter_p[t] = v;\n}\n";
+    s << "}\n";
+    pack_grid_ = (uint32_t)((pixels + (c.filter_gradient ? 0 : taps) + 255) / 256);
+    if (c.filter_gradient) {
+        const uint64_t elems = (uint64_t)c.O * c.R * c.S * c.C;
+        const char* et = c.elem_bytes == 4 ? "u32" : "u16";
+        s << "extern \"C\" __global__ __launch_bounds__(256) void unpack_filter_gradient(const " << et << "* __restrict__ packed, " << et << "* __restrict__ out) {\n"
+          << "u32 t = blockIdx.x * 256u + threadIdx.x;\nif (t >= " << elems << "u) return;\n"
+          << "u32 ch = t % " << c.C << "u, rest = t / " << c.C << "u, sx = rest % " << c.S << "u, row = rest / " << c.S << "u;\n"
+          << "out[t] = packed[((u64)row * " << c.Sp << "u + sx) * 4u + ch];\n}\n";
+        unpack_grid_ = (uint32_t)((elems + 255) / 256);
+    }
+    pack_source_ = s.str();
+    source_ = "// ---- repack\n" + pack_source_ + "// ---- product\n" + inner_->source();
+    describe_ = strfmt("repacked image_arg=%d filter_arg=%d filter_gradient=%d image=[%lld,%lld,%lld,%lld] packed=[%lld,%lld,%lld,4] pad=[%lld,%lld] filter=[%lld,%lld,%lld->%lld] "
+                       "pack_grid=%u unpack_grid=%u image_bytes=%zu filter_bytes=%zu\n",
+                       c.image_arg, c.filter_arg, (int)c.filter_gradient, (long long)c.N, (long long)c.H, (long long)c.W, (long long)c.C, (long long)c.N,
+                       (long long)c.Hp, (long long)c.Wp, (long long)c.ph, (long long)c.pw, (long long)c.O, (long long)c.R, (long long)c.S, (long long)c.Sp, pack_grid_,
+                       unpack_grid_, image_bytes_, filter_bytes_) +
+                inner_->describe();
+    pack_.reset(new JitKernel(pack_source_, "repack_conv_operands"));
+    if (c.filter_gradient) unpack_.reset(new JitKernel(pack_source_, "unpack_filter_gradient"));
+}
+
+RepackedConvKernel::~RepackedConvKernel() { scratch_.release(); }
+
+size_t RepackedConvKernel::scratch_bytes_needed() const { return own_bytes() + inner_->scratch_bytes_needed(); }
+
+void RepackedConvKernel::load() {
+    pack_->load();
+    if (unpack_) unpack_->load();
+    inner_->load();
+}
+
+bool RepackedConvKernel::loaded() const { return pack_->loaded() && (!unpack_ || unpack_->loaded()) && inner_->loaded(); }
+
+void RepackedConvKernel::execute(void* const* ptrs, hipStream_t stream) {
+    run(ptrs, stream, (char*)scratch_.get(own_bytes() / 4, 0, stream).floats, nullptr, 0);
+}
+
+void RepackedConvKernel::execute_in_scratch(void* const* ptrs, hipStream_t stream, void* scratch, size_t scratch_bytes) {
+    HE_REQUIRE(loaded(), HE_ERR_INVALID, "the kernel's code objects are not loaded on this device yet");
+    HE_REQUIRE(scratch_bytes_needed() <= scratch_bytes, HE_ERR_INVALID,
+               "the kernel needs %zu bytes of scratch for its repacked operands and partial results, the buffer holds %zu", scratch_bytes_needed(), scratch_bytes);
+    HE_REQUIRE(scratch && ((uintptr_t)scratch & 255) == 0, HE_ERR_INVALID, "scratch buffer missing or not 256-byte aligned");
+    run(ptrs, stream, (char*)scratch, (char*)scratch + own_bytes(), scratch_bytes - own_bytes());
+}
+
+void RepackedConvKernel::run(void* const* ptrs, hipStream_t stream, char* own, void* inner_scratch, size_t inner_scratch_bytes) {
+    for (size_t i = 0; i < args_.size(); i++) HE_REQUIRE(ptrs[i] != nullptr, HE_ERR_INVALID, "kernel argument %zu is null", i);
+    void* image = ptrs[geo_.image_arg];
+    void* filter = ptrs[geo_.filter_arg];
+    void* image_p = own;
+    void* filter_p = own + image_bytes_;
+    const uint32_t block[3] = {256, 1, 1};
+    {
+        void* fwd[] = {&image, &filter, &image_p, &filter_p};
+        void* grad[] = {&image, &image_p};
+        const uint32_t grid[3] = {pack_grid_, 1, 1};
+        pack_->launch(grid, block, 0, stream, geo_.filter_gradient ? grad : fwd, false);
+    }
+    std::vector<void*> inner_ptrs(ptrs, ptrs + args_.size());
+    inner_ptrs[geo_.image_arg] = image_p;
+    inner_ptrs[geo_.filter_arg] = filter_p;
+    // (a forward convolution's last launch is the product's: it closes the instruction; a filter gradient's is the unpacking)
+    HeldStopEvent held;
+    if (!geo_.filter_gradient) held.give_back();
+    if (inner_scratch) inner_->execute_in_scratch(inner_ptrs.data(), stream, inner_scratch, inner_scratch_bytes);
+    else inner_->execute(inner_ptrs.data(), stream);
+    if (geo_.filter_gradient) {
+        held.give_back();
+        void* argv[] = {&filter_p, &filter};
+        const uint32_t grid[3] = {unpack_grid_, 1, 1};
+        unpack_->launch(grid, block, 0, stream, argv, true);
+    }
 }
 
 }  // namespace he

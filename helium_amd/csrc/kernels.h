@@ -194,4 +194,47 @@ private:
     std::string source_, describe_;
 };
 
+// A convolution (or its filter gradient) over a 16-bit image of 3 or 4 channels, run over a repacked copy of the
+// image. A chunk of 16 bytes is what one lane loads straight into LDS, and an image of 3 channels has no such chunk
+// that lies in one filter tap, so its gather would go element by element through registers. The copy has 4 channels
+// per pixel (the added ones zero) and the padding written out, which makes two neighbouring pixels one 8-channel
+// "pixel" of an image of half the width: with an even stride along w the convolution is an ordinary one over that
+// image, with ceil(S / 2) taps per filter row, no padding, and every chunk aligned. The filter is repacked the same
+// way ([O, R, 2 * ceil(S / 2), 4], zero where the source has nothing); a filter gradient comes out in that layout and
+// is unpacked. One launch repacks, the product runs, one launch unpacks (filter gradient only).
+struct ConvRepack {
+    bool filter_gradient = false;
+    int64_t N = 0, H = 0, W = 0, C = 0;     // the image as the caller holds it
+    int64_t Hp = 0, Wp = 0, ph = 0, pw = 0; // the copy: [N, Hp, Wp, 4]; pixel (h, w) of the image is pixel (h + ph, w + pw) of it
+    int64_t O = 0, R = 0, S = 0, Sp = 0;    // filter [O, R, S, C] and its packed row length Sp (pixels)
+    int image_arg = -1, filter_arg = -1;    // positions in the argument list (the filter gradient is the output)
+    int elem_bytes = 2;                     // of the filter gradient (2 or 4); images and filters are 16-bit
+};
+class RepackedConvKernel : public KernelBase {
+public:
+    // `args`: the instruction's arguments; `inner`: the product over the repacked operands, same argument positions.
+    RepackedConvKernel(std::vector<tp::Arg> args, ConvRepack geometry, std::unique_ptr<KernelBase> inner);
+    const std::vector<tp::Arg>& args() const override { return args_; }
+    const std::string& source() const override { return source_; }
+    const std::string& describe() const override { return describe_; }
+    void execute(void* const* ptrs, hipStream_t stream) override;
+    void execute_in_scratch(void* const* ptrs, hipStream_t stream, void* scratch, size_t scratch_bytes) override;
+    size_t scratch_bytes_needed() const override;
+    void load() override;
+    bool loaded() const override;
+    ~RepackedConvKernel() override;
+
+private:
+    size_t own_bytes() const { return image_bytes_ + filter_bytes_; }
+    void run(void* const* ptrs, hipStream_t stream, char* own, void* inner_scratch, size_t inner_scratch_bytes);
+    std::vector<tp::Arg> args_;
+    ConvRepack geo_;
+    std::unique_ptr<KernelBase> inner_;
+    std::string pack_source_, source_, describe_;
+    std::unique_ptr<JitKernel> pack_, unpack_;
+    size_t image_bytes_ = 0, filter_bytes_ = 0;  // of the packed copies (256-byte multiples)
+    uint32_t pack_grid_ = 0, unpack_grid_ = 0;
+    ReduceScratch scratch_;
+};
+
 }  // namespace he

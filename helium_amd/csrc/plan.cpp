@@ -857,6 +857,7 @@ GemmProblem conv_backward_data_problem(const ir::OpSubgraph& sg, NodeId node, in
 }  // namespace
 
 namespace {
+int filter_gradient_split_k(const GemmProblem& pr, bool element_gather);
 // Op::ConvBackwardFilter as a GEMM: rows = output channels o, columns = filter taps (r, s, c), k = output pixels
 // (n, p, q). A is the flow read as [k][m] (its own memory order: m contiguous); B[k][(r, s, c)] is gathered from the
 // image with the forward convolution's map. The product has few output tiles and a very long k, so the k range is
@@ -903,15 +904,7 @@ GemmProblem conv_backward_filter_problem(const ir::OpSubgraph& sg, NodeId node) 
     pr.a_km = true;
     operand(pr.op_b, image, op.inputs[1], pr.K, pr.N);  // stand-in: only the argument is used
     pr.root_a = pr.root_b = 0;
-    // about two workgroups per CU, each with at least four 64-wide k-tiles (128x128 output tiles)
-    const int64_t tiles = ((pr.M + 127) / 128) * ((pr.N + 127) / 128), k_tiles = (pr.K + 63) / 64;
-    pr.split_k = (int)std::max<int64_t>(1, std::min<int64_t>({(512 + tiles - 1) / tiles, k_tiles / 4, 1024}));
-    // (an image whose channels do not fill 16-byte chunks is gathered element by element, by 32x64 tiles of two waves: six
-    // workgroups per CU, one round of them over the chip)
-    const int64_t chunk = image.dtype == HE_F32 ? 4 : 8;
-    if (image.dtype != HE_F32 && cv.C % chunk != 0 && pr.M <= 32 && pr.M > 16 && pr.N >= 128)
-        pr.split_k = (int)std::max<int64_t>(1, std::min<int64_t>({1536 / ((pr.N + 63) / 64), k_tiles / 4, 1024}));
-    if (const char* env = tuning::get("HELIUM_HIP_GEMM_SPLIT_K")) pr.split_k = std::max(1, atoi(env));
+    pr.split_k = filter_gradient_split_k(pr, image.dtype != HE_F32 && cv.C % 8 != 0);
     pr.epi.dims = {1, pr.M, pr.N};
     pr.epi.fast_math = true;
     tp::Expr acc;
@@ -949,6 +942,72 @@ std::vector<GemmProblem> strided_data_gradient_classes(const ir::OpSubgraph& sg,
     return out;
 }
 
+namespace {
+int filter_gradient_split_k(const GemmProblem& pr, bool element_gather) {
+    // about two workgroups per CU, each with at least four 64-wide k-tiles (128x128 output tiles)
+    const int64_t tiles = ((pr.M + 127) / 128) * ((pr.N + 127) / 128), k_tiles = (pr.K + 63) / 64;
+    int split = (int)std::max<int64_t>(1, std::min<int64_t>({(512 + tiles - 1) / tiles, k_tiles / 4, 1024}));
+    // (an image whose channels do not fill 16-byte chunks is gathered element by element, by 32x64 tiles of two waves: six
+    // workgroups per CU, one round of them over the chip)
+    if (element_gather && pr.M <= 32 && pr.M > 16 && pr.N >= 128)
+        split = (int)std::max<int64_t>(1, std::min<int64_t>({1536 / ((pr.N + 63) / 64), k_tiles / 4, 1024}));
+    if (const char* env = tuning::get("HELIUM_HIP_GEMM_SPLIT_K")) split = std::max(1, atoi(env));
+    return split;
+}
+
+// A forward convolution or a filter gradient over a 16-bit image of 3 or 4 channels with an even stride along w and no
+// dilation along w: the same product over the image repacked to 4 channels with its padding written out, two pixels
+// making one 8-channel pixel of an image of half the width (kernels.h: ConvRepack). `packed` is that product: the image
+// argument stands for the copy [N, Hp, Wp / 2, 8], the filter argument (the output, for a filter gradient) for
+// [O, R, ceil(S / 2), 8].
+bool over_repacked_image(const GemmProblem& pr, GemmProblem* packed, ConvRepack* geo) {
+    const bool fwd = pr.conv_a.on && !pr.conv_a.bwd, grad = pr.conv_b.on;
+    if ((!fwd && !grad) || pr.mma_dtype == HE_F32 || tuning::get("HELIUM_HIP_GEMM_NO_REPACK")) return false;
+    const GemmProblem::ConvGather& cv = fwd ? pr.conv_a : pr.conv_b;
+    if (cv.C < 3 || cv.C > 4 || cv.dw != 1 || cv.sw % 2 != 0 || cv.S < 2) return false;
+    const int image_arg = fwd ? pr.map_a[0] : pr.map_b[0];
+    const int filter_arg = fwd ? pr.map_b[0] : pr.map_e[pr.epi.outs[0].arg];
+    // (an epilogue that reads the image or the filter itself would see the copies)
+    for (size_t i = 0; i < pr.epi.args.size(); i++)
+        if (!pr.epi.args[i].is_output && (pr.map_e[i] == image_arg || pr.map_e[i] == filter_arg)) return false;
+    ConvRepack g;
+    g.filter_gradient = grad;
+    g.N = cv.N; g.H = cv.H; g.W = cv.W; g.C = cv.C;
+    g.O = fwd ? pr.N : pr.M; g.R = cv.R; g.S = cv.S;
+    g.Sp = (cv.S + 1) / 2 * 2;
+    g.Hp = (cv.P - 1) * cv.sh + (cv.R - 1) * cv.dh + 1;
+    g.Wp = (cv.Q - 1) * cv.sw + g.Sp;
+    g.ph = cv.ph; g.pw = cv.pw;
+    g.image_arg = image_arg; g.filter_arg = filter_arg;
+    g.elem_bytes = grad ? dtype_bits(pr.args[filter_arg].dtype) / 8 : 2;
+    if (g.N * g.Hp * g.Wp * 4 >= (1ll << 31)) return false;
+    *packed = pr;
+    GemmProblem::ConvGather& pv = fwd ? packed->conv_a : packed->conv_b;
+    pv.H = g.Hp; pv.W = g.Wp / 2; pv.C = 8; pv.S = g.Sp / 2; pv.sw = cv.sw / 2; pv.ph = 0; pv.pw = 0;
+    const int64_t taps = pv.R * pv.S * pv.C;
+    auto resize = [](tp::Program& p, int64_t rows, int64_t cols, int64_t numel) {
+        p.dims = {1, rows, cols};
+        p.args[0].numel = numel;
+        p.exprs[0].access.stride = ir::packed_strides(p.dims);
+    };
+    if (fwd) {
+        packed->K = taps;
+        resize(packed->op_a, packed->M, packed->K, g.N * g.Hp * g.Wp * 4);
+        resize(packed->op_b, packed->N, packed->K, g.O * taps);
+        if (pr.split_k > 1) packed->split_k = choose_split_k(packed->M, packed->N, packed->K, 1);
+    } else {
+        packed->N = taps;
+        resize(packed->op_b, packed->K, packed->N, g.N * g.Hp * g.Wp * 4);
+        packed->epi.dims = {1, packed->M, packed->N};
+        packed->epi.args[0].numel = g.O * taps;
+        packed->split_k = filter_gradient_split_k(*packed, false);
+    }
+    assemble_gemm_args(*packed);
+    *geo = g;
+    return true;
+}
+}  // namespace
+
 std::unique_ptr<KernelBase> make_gemm_kernel(const ir::OpSubgraph& sg) {
     // The data gradient of a strided convolution is one product per class of pixels (row and column modulo the
     // stride): each multiplies only the taps that reach its pixels.
@@ -959,7 +1018,14 @@ std::unique_ptr<KernelBase> make_gemm_kernel(const ir::OpSubgraph& sg) {
         for (auto& pr : classes) parts.emplace_back(new GemmKernel(std::move(pr)));
         return std::unique_ptr<KernelBase>(new CompositeKernel(std::move(parts), any_empty));
     }
-    return std::unique_ptr<KernelBase>(new GemmKernel(gemm_problem_from_ir(sg)));
+    GemmProblem pr = gemm_problem_from_ir(sg);
+    ConvRepack geometry;
+    GemmProblem packed;
+    if (over_repacked_image(pr, &packed, &geometry)) {
+        std::vector<tp::Arg> args = pr.args;
+        return std::unique_ptr<KernelBase>(new RepackedConvKernel(std::move(args), geometry, std::unique_ptr<KernelBase>(new GemmKernel(std::move(packed)))));
+    }
+    return std::unique_ptr<KernelBase>(new GemmKernel(std::move(pr)));
 }
 
 GemmProblem gemm_problem_from_ir(const ir::OpSubgraph& sg) {

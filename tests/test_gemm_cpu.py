@@ -196,33 +196,21 @@ class _Part:
         self.source, self.description, self.args = source, description, args
 
 
-def run_ir_kernel_on_cpu(g, nodes, inputs):
-    k = ha.backend.matmul_kernel(g, nodes)
-    if k.description.startswith("composite"):
-        head, *lines = k.description.split("\n")
-        parts, zero_first = (int(v) for v in re.search(r"parts=(\d+) zero_first=(\d)", head).groups())
-        sources = re.split(r"// ---- part \d+ of \d+\n", k.source)[1:]
-        assert len(sources) == len(lines) == parts
-        outs = [a for a in k.args if a["is_output"]]
-        # what no part writes has to be zeroed first by the host; where every element is written the buffer starts as
-        # NaN here, so an element that no part wrote shows
-        current = {a["node"]: (np.zeros(a["numel"], dtype=nm.NP_STORAGE[a["dtype"]]) if zero_first
-                               else nm.to_storage(np.full(a["numel"], np.nan, dtype=np.float32), a["dtype"])) for a in outs}
-        for src, line in zip(sources, lines):
-            part = _Part(src, line, k.args)
-            bufs = [(current[a["node"]], 2) if a["is_output"] else (inputs[a["node"]], 0) for a in k.args]
-            for a, r in zip(outs, launch_gemm(part, bufs)):
-                current[a["node"]] = r
-        return k, {a["node"]: nm.from_storage(current[a["node"]], a["dtype"], [current[a["node"]].size]).astype(np.float64) for a in outs}
+def _run_one_product(k, inputs, current=None):
+    """One fused-GEMM kernel (anything with .source, .description and .args) on the CPU. inputs: {node: storage array};
+    current: {node: array} the outputs start from (zeros otherwise). Returns {node: storage array} of the outputs."""
     gx, gy = map(int, re.search(r"grid=(\d+)x(\d+)", k.description).groups())
     threads = int(re.search(r"threads=(\d+)", k.description).group(1))
     split = int(re.search(r"split_k=(\d+)", k.description).group(1))
     m, n = (int(v) for v in re.search(r"gemm \[\d+,(\d+),\d+\]x\[(\d+)\]", k.description).groups())
+    outs = [a for a in k.args if a["is_output"]]
     bufs = []
     for a in k.args:
-        dt = nm.NP_STORAGE[a["dtype"]]
-        bufs.append((np.zeros(a["numel"], dtype=dt), 2) if a["is_output"] else (inputs[a["node"]], 0))
-    outs = [a for a in k.args if a["is_output"]]
+        if a["is_output"]:
+            bufs.append((current[a["node"]] if current else np.zeros(a["numel"], dtype=nm.NP_STORAGE[a["dtype"]]), 2))
+        else:
+            assert inputs[a["node"]].size == a["numel"], (a, inputs[a["node"]].size)
+            bufs.append((inputs[a["node"]], 0))
     if split > 1:
         # a split-k product: partial tiles go to scratch, a second launch adds them up into the one output
         res = run_kernel(k.source, "fused_matmul", gx, threads, bufs + [(np.full(split * m * n, np.nan, dtype=np.float32), 2)], grid_y=gy)
@@ -230,7 +218,62 @@ def run_ir_kernel_on_cpu(g, nodes, inputs):
         res = run_kernel(k.source, "fused_matmul_finalize", (m * n + 31) // 32, 256, [(res[-1], 0), (np.zeros(out["numel"], dtype=nm.NP_STORAGE[out["dtype"]]), 1)])
     else:
         res = launch_gemm(k, bufs)
-    return k, {a["node"]: nm.from_storage(r, a["dtype"], [r.size]).astype(np.float64) for a, r in zip(outs, res)}
+    return {a["node"]: r for a, r in zip(outs, res)}
+
+
+def _run_repacked(k, inputs):
+    """A convolution over a repacked few-channel image: the repacking launch, the product over the copies, and for a
+    filter gradient the unpacking launch, each on the CPU with buffers of exactly the size the geometry gives."""
+    head, inner_desc = k.description.split("\n", 1)
+    f = {key: [int(v) for v in re.findall(r"-?\d+", val)] for key, val in re.findall(r"(\w+)=(\[[^\]]*\]|-?\d+)", head)}
+    image_arg, filter_arg, grad = f["image_arg"][0], f["filter_arg"][0], f["filter_gradient"][0]
+    n_, hp, wp, _ = f["packed"]
+    o_, r_, s_, sp = f["filter"]
+    pack_src, product_src = re.split(r"// ---- product\n", k.source.split("// ---- repack\n", 1)[1])
+    image = inputs[k.args[image_arg]["node"]]
+    image_p = np.zeros(n_ * hp * wp, dtype=np.uint64)
+    if grad:
+        (image_p,) = run_kernel(pack_src, "repack_conv_operands", f["pack_grid"][0], 256, [(image, 0), (image_p, 1)])
+    else:
+        filt = inputs[k.args[filter_arg]["node"]]
+        image_p, filter_p = run_kernel(pack_src, "repack_conv_operands", f["pack_grid"][0], 256,
+                                       [(image, 0), (filt, 0), (image_p, 1), (np.zeros(o_ * r_ * sp, dtype=np.uint64), 1)])
+    args = [dict(a) for a in k.args]
+    args[image_arg]["numel"] = image_p.size * 4
+    args[filter_arg]["numel"] = o_ * r_ * sp * 4
+    inner_inputs = dict(inputs)
+    inner_inputs[args[image_arg]["node"]] = image_p.view(np.uint16)
+    if not grad:
+        inner_inputs[args[filter_arg]["node"]] = filter_p.view(np.uint16)
+    res = _run_one_product(_Part(product_src, inner_desc, args), inner_inputs)
+    if grad:
+        a = k.args[filter_arg]
+        packed = res[a["node"]]
+        (res[a["node"]],) = run_kernel(pack_src, "unpack_filter_gradient", f["unpack_grid"][0], 256,
+                                       [(packed, 0), (np.zeros(a["numel"], dtype=packed.dtype), 1)])
+    return res
+
+
+def run_ir_kernel_on_cpu(g, nodes, inputs):
+    k = ha.backend.matmul_kernel(g, nodes)
+    outs = [a for a in k.args if a["is_output"]]
+    if k.description.startswith("composite"):
+        head, *lines = k.description.split("\n")
+        parts, zero_first = (int(v) for v in re.search(r"parts=(\d+) zero_first=(\d)", head).groups())
+        sources = re.split(r"// ---- part \d+ of \d+\n", k.source)[1:]
+        assert len(sources) == len(lines) == parts
+        # what no part writes has to be zeroed first by the host; where every element is written the buffer starts as
+        # NaN here, so an element that no part wrote shows
+        current = {a["node"]: (np.zeros(a["numel"], dtype=nm.NP_STORAGE[a["dtype"]]) if zero_first
+                               else nm.to_storage(np.full(a["numel"], np.nan, dtype=np.float32), a["dtype"])) for a in outs}
+        for src, line in zip(sources, lines):
+            current = _run_one_product(_Part(src, line, k.args), inputs, current)
+        res = current
+    elif k.description.startswith("repacked"):
+        res = _run_repacked(k, inputs)
+    else:
+        res = _run_one_product(k, inputs)
+    return k, {a["node"]: nm.from_storage(res[a["node"]], a["dtype"], [res[a["node"]].size]).astype(np.float64) for a in outs}
 
 
 def test_ir_matmul_with_epilogue_on_cpu():
@@ -308,8 +351,17 @@ CONV_CASES = [
     ("odd_channels_three_5x5_stride3", (1, 11, 13, 3), 8, (5, 5), "f16", (3, 3), (1, 1), "same", "64,64,64,2,2"),
     # the tiles of products with 32 columns: four waves of 64x32 (direct loads), 256x64 for the element-wise gather
     ("thirty_two_channels_out_narrow_tile", (2, 12, 12, 32), 32, (3, 3), "bf16", (2, 2), (1, 1), "same", "256,32,64,4,1"),
-    ("three_channel_stem_wide_gather_tile", (2, 16, 16, 3), 32, (7, 7), "bf16", (2, 2), (1, 1), "same", "256,64,64,4,2"),
+    ("three_channel_stem_wide_gather_tile", (2, 10, 10, 3), 32, (7, 7), "bf16", (1, 1), (1, 1), "same", "256,64,64,4,2"),
+    # 3 or 4 channels, 16-bit, even stride along w: the product runs over a 4-channel copy of the image with the padding
+    # written out, two pixels to a 16-byte chunk
+    ("repacked_three_channel_stem", (2, 16, 16, 3), 32, (7, 7), "bf16", (2, 2), (1, 1), "same", "256,64,64,4,2"),
+    ("repacked_four_channels_even_taps_valid", (1, 9, 14, 4), 16, (3, 4), "f16", (1, 2), (2, 1), "valid", "64,64,64,2,2"),
+    ("repacked_three_channels_stride_2x4_full", (2, 8, 11, 3), 8, (5, 3), "bf16", (2, 4), (1, 1), "full", "128,128,64,2,2"),
 ]
+
+
+def repacks(image, kernel, dtype, stride, dilation):
+    return dtype != "f32" and image[3] in (3, 4) and stride[1] % 2 == 0 and dilation[1] == 1 and kernel[1] >= 2
 
 
 @pytest.mark.parametrize("name,image,oc,kernel,dtype,stride,dilation,mode,tile", CONV_CASES, ids=[c[0] for c in CONV_CASES])
@@ -327,6 +379,7 @@ def test_conv_on_cpu(name, image, oc, kernel, dtype, stride, dilation, mode, til
     tol = 1e-4 if dtype == "f32" else 2e-2
     assert np.abs(got[y] - want).max() <= tol * max(1.0, np.abs(want).max()), (k.description, np.abs(got[y] - want).max())
     assert ("#define CONV_A_FAST 1" in k.source) == name.startswith("hoisted"), name
+    assert k.description.startswith("repacked") == repacks(image, kernel, dtype, stride, dilation), k.description
 
 
 BWD_DATA_CASES = [
@@ -388,8 +441,11 @@ BWD_FILTER_CASES = [
     ("valid_and_dilated_f32", (2, 9, 9, 4), 8, (3, 3), "f32", (1, 1), (2, 1), "valid", "64,64,32,2,2"),
     # channel counts that do not fill a 16-byte chunk: the image operand is gathered element by element
     ("three_channel_stem_7x7_stride2", (2, 16, 16, 3), 32, (7, 7), "bf16", (2, 2), (1, 1), "same", "64,128,64,2,2"),
-    ("three_channel_stem_thirty_two_rows_tile", (2, 16, 16, 3), 32, (7, 7), "bf16", (2, 2), (1, 1), "same", "32,128,64,1,4"),
-    ("three_channel_stem_two_wave_tile", (2, 16, 16, 3), 32, (7, 7), "bf16", (2, 2), (1, 1), "same", "32,64,64,1,2"),
+    ("three_channel_stem_thirty_two_rows_tile", (2, 10, 10, 3), 32, (7, 7), "bf16", (1, 1), (1, 1), "same", "32,128,64,1,4"),
+    ("three_channel_stem_two_wave_tile", (2, 10, 10, 3), 32, (7, 7), "bf16", (1, 1), (1, 1), "same", "32,64,64,1,2"),
+    # over a repacked copy of the image; the gradient comes out in the packed filter layout and is unpacked
+    ("repacked_four_channels_stride_1x2", (2, 9, 14, 4), 16, (3, 4), "f16", (1, 2), (2, 1), "valid", "64,64,64,2,2"),
+    ("repacked_three_channels_5x3_full", (2, 8, 11, 3), 8, (5, 3), "bf16", (2, 4), (1, 1), "full", "128,128,64,2,2"),
     ("thirty_two_rows_tile_direct_loads", (2, 12, 12, 16), 32, (3, 3), "bf16", (1, 1), (1, 1), "same", "32,128,64,1,4"),
     ("five_channels_3x3_f16", (1, 7, 9, 5), 8, (3, 3), "f16", (1, 1), (1, 1), "same", "64,64,64,2,2"),
     ("three_channels_f32_full", (1, 6, 5, 3), 8, (3, 3), "f32", (1, 1), (1, 2), "full", "64,64,32,2,2"),
@@ -423,6 +479,7 @@ def test_conv_backward_filter_on_cpu(name, image, oc, kernel, dtype, stride, dil
     want = nm.from_storage(want.reshape(-1), dtype, [want.size]).astype(np.float64)
     tol = 1e-4 if dtype == "f32" else 2e-2
     assert np.abs(got[dw] - want).max() <= tol * max(1.0, np.abs(want).max()), (k.description, np.abs(got[dw] - want).max())
+    assert k.description.startswith("repacked") == repacks(image, kernel, dtype, stride, dilation), k.description
 
 
 @pytest.mark.parametrize("dtype,precision,tol", [("f32", "f32_f32", 1e-4), ("bf16", "bf16_f32", 2e-2)])
