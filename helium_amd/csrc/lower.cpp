@@ -235,6 +235,7 @@ public:
             drop_unused_inputs();
             merge_row_dims();
         } else {
+            drop_unit_dims();
             fold_leading_dims_as_columns();
             merge_row_like_dims();
         }
@@ -323,6 +324,43 @@ private:
             p_.dims.erase(p_.dims.begin() + i);
             for (auto& e : p_.exprs)
                 if (e.kind == Expr::Load) e.access.stride.erase(e.access.stride.begin() + i);
+        }
+    }
+
+    // Dims of extent 1 leave the iteration space: the canonical view takes the last dim as the columns and the one
+    // before as the rows, and a reduction over [1000, 128, 1, 1] (the gradient of a bias that was broadcast from
+    // [1000, 1, 1]) would otherwise run with one element per workgroup. A reduction folds the trailing dims, so its
+    // depth counts the remaining ones; one that folded unit dims only is the identity.
+    void drop_unit_dims() {
+        const size_t R = p_.dims.size();
+        for (auto& e : p_.exprs)
+            if (e.kind == Expr::Load && e.access.stride.size() != R) return;
+        out_depth_.resize(p_.outs.size(), 0);
+        for (size_t i = 0; i < p_.outs.size(); i++) {
+            if (!p_.outs[i].reduce) continue;
+            size_t depth = 0;
+            for (size_t k = R - out_depth_[i]; k < R; k++) depth += p_.dims[k] != 1;
+            out_depth_[i] = depth;
+        }
+        for (size_t d = R; d-- > 0;) {
+            if (p_.dims[d] != 1 || p_.dims.size() == 1) continue;
+            p_.dims.erase(p_.dims.begin() + d);
+            for (auto& e : p_.exprs)
+                if (e.kind == Expr::Load) e.access.stride.erase(e.access.stride.begin() + d);
+        }
+        const size_t rank = p_.dims.size();
+        for (size_t i = 0; i < p_.outs.size(); i++) {
+            Out& o = p_.outs[i];
+            if (!o.reduce) continue;
+            const size_t depth = out_depth_[i];
+            if (depth == 0) {
+                o.reduce = false;
+                continue;
+            }
+            o.fold_n = true;
+            o.fold_m = depth >= 2;
+            o.b_div = 1;
+            for (size_t k = rank - depth; k + 2 < rank; k++) o.b_div *= p_.dims[k];
         }
     }
 
