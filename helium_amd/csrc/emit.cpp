@@ -169,12 +169,20 @@ __device__ __forceinline__ float tanh_2ulp(float x) {
 }
 // a / b as a * rcp(b): about 1 ulp, one quarter-rate instruction instead of the ten of an IEEE division
 __device__ __forceinline__ float fast_div(float a, float b) { return a * HE_FAST_RCP(b); }
-// powf whose exponent is one value for the whole launch (a broadcast 1-element operand, as `x.pow_scalar(2.0)`
-// reaches the kernel): the tests are the same in every lane, and squares skip the general routine.
-__device__ __forceinline__ float pow_uniform(float x, float y) {
+// powf, one copy per kernel: inlined at every use (a kernel of per-channel arithmetic has twenty, each in the interior
+// and the ragged form of the loop body) the routine makes a kernel of a few hundred elements spend its time fetching
+// code. Squares and first powers (`x.pow_scalar(2.0)`) skip the general routine when every lane of the wave has one.
+__device__ __attribute__((noinline)) float he_powf(float x, float y) {
     if (y == 2.0f) return x * x;
     if (y == 1.0f) return x;
     return powf(x, y);
+}
+// powf whose exponent is one value for the whole launch (a broadcast 1-element operand): the tests are the same in
+// every lane.
+__device__ __forceinline__ float pow_uniform(float x, float y) {
+    if (y == 2.0f) return x * x;
+    if (y == 1.0f) return x;
+    return he_powf(x, y);
 }
 __device__ __forceinline__ float fast_tanh(float x) {
     float t = __expf(2.0f * x);
@@ -213,7 +221,7 @@ static std::string unary_expr(const Expr& e, const std::string& x, bool fast) {
             // x*x for an exponent of exactly 2, as the reference's generator special-cases
             // (helium-playground/src/kernel_generator.rs:383-391); x**c otherwise (torch_synthesizer.rs:55).
             if (cf == 2.0f) return x + " * " + x;
-            return "powf(" + x + ", " + c + ")";
+            return "he_powf(" + x + ", " + c + ")";
     }
     fail(HE_ERR_INTERNAL, "bad unary op");
 }
@@ -224,7 +232,7 @@ static std::string binary_expr(const Expr& e, Cls cls, const std::string& a, con
         case BOp::Sub: return a + " - " + b;
         case BOp::Mul: return cls == Cls::B ? a + " && " + b : a + " * " + b;
         case BOp::Div: return fast ? "fast_div(" + a + ", " + b + ")" : a + " / " + b;
-        case BOp::Pow: return "powf(" + a + ", " + b + ")";
+        case BOp::Pow: return "he_powf(" + a + ", " + b + ")";
         case BOp::Min: return cls == Cls::F ? "fminf(" + a + ", " + b + ")" : "(" + a + " < " + b + " ? " + a + " : " + b + ")";
         case BOp::Max: return cls == Cls::F ? "fmaxf(" + a + ", " + b + ")" : "(" + a + " > " + b + " ? " + a + " : " + b + ")";
         case BOp::And: return cls == Cls::B ? a + " && " + b : a + " & " + b;
@@ -731,7 +739,14 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
         while (RPT % unroll) unroll--;
         const std::string head = "#pragma unroll 1\nfor (u32 i0 = 0; i0 < RPT; i0 += " + std::to_string(unroll) + ") {\n#pragma unroll\nfor (u32 iu = 0; iu < " +
                                  std::to_string(unroll) + "; iu++) {\nconst u32 i = i0 + iu;\nconst u32 m = tile_y * TR + i * TY + ty;\n";
+        // (a launch of a few workgroups runs its code once or twice: a second form of the body without the bounds tests
+        // costs more in instruction fetch than the tests do)
+        const bool few_blocks = grid <= 16;
         auto loops = [&](const std::string& body) {
+            if (ragged && few_blocks) {
+                s << head << "const bool ok = col_ok && m < DIM_M;\n" << body << "}\n}\n";
+                return;
+            }
             if (ragged) s << "if ((tile_y + 1) * TR <= DIM_M && (tile_x + 1) * (TX * NV) <= DIM_N) {\n";
             s << head << "const bool ok = true;\n" << body << "}\n}\n";
             if (ragged) s << "} else {\n" << head << "const bool ok = col_ok && m < DIM_M;\n" << body << "}\n}\n}\n";
