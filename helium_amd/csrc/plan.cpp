@@ -506,6 +506,42 @@ std::shared_ptr<const Plan> generate_plan(const std::shared_ptr<const ir::OpGrap
         plan->steps[i].instrs = kept;
     }
 
+    // Beyond the reference: small pointwise kernels of one step that walk the same index space run as one kernel. They
+    // are independent by construction (one step), each costs a launch of several microseconds for a few hundred
+    // elements (per-channel arithmetic of a batch norm's backward pass next to the optimizer's update of its scale and
+    // shift), and one launch computes all of them in the same time.
+    if (rematerialize()) {
+        auto small_space = [&](const Instr& instr, int64_t* numel) {
+            if (instr.kind() != InstrKind::Pointwise) return false;
+            *numel = -1;
+            for (NodeId leaf : instr.subgraph().leafs()) {
+                const ir::Node& n = g->get(leaf);
+                if (n.op.kind == ir::OpKind::Reduce) return false;
+                const int64_t e = ir::num_elements(n.desc.shape);
+                if (*numel >= 0 && e != *numel) return false;
+                *numel = e;
+            }
+            return *numel >= 0 && *numel <= (1 << 16);
+        };
+        for (Step& step : plan->steps) {
+            for (size_t i = 0; i < step.instrs.size(); i++) {
+                int64_t ni = 0;
+                if (!small_space(*step.instrs[i], &ni)) continue;
+                for (size_t j = i + 1; j < step.instrs.size();) {
+                    int64_t nj = 0;
+                    const Instr &a = *step.instrs[i], &b = *step.instrs[j];
+                    if (small_space(b, &nj) && nj == ni && a.outputs().size() + b.outputs().size() <= 24 &&
+                        a.subgraph().nodes().size() + b.subgraph().nodes().size() <= 160 && a.can_fuse_with(b)) {
+                        step.instrs[i] = std::make_shared<Instr>(a.fuse_with(b));
+                        step.instrs.erase(step.instrs.begin() + j);
+                    } else {
+                        j++;
+                    }
+                }
+            }
+        }
+    }
+
     // analyze_tensor_lifetimes (:360-416)
     {
         std::vector<std::vector<NodeId>> releases;
