@@ -811,15 +811,13 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
             t.wn = 4;
             small = true;
         } else if (!f32 && pr.M <= 64 && pr.M > 32 && pr.N >= 128) {
-            // few output rows (a filter gradient with 64 output channels): tiles as low as M, and twice as wide when the
-            // k range is split (eight waves share the 64 rows of the flow: 107 -> 99 us on the 56x56x64 layer)
+            // few output rows (a filter gradient with 64 output channels): tiles as low as M, of eight waves when the k
+            // range is split (the 56x56x64 layer: 107 us with four waves, 103-105 with eight on 64x128 or 64x256 at batch
+            // 128; at batch 64 48 us on 64x128 against 57 on 64x256)
             t.bm = 64;
             t.bn = 128;
             t.wm = t.wn = 2;
-            if (pr.split_k > 1 && pr.N >= 256) {
-                t.bn = 256;
-                t.wn = 4;
-            }
+            if (pr.split_k > 1 && pr.N >= 256) t.wn = 4;
             small = true;
         } else
         // Smaller problems take smaller tiles so that every CU gets work.
