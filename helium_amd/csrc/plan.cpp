@@ -982,7 +982,10 @@ namespace {
 int filter_gradient_split_k(const GemmProblem& pr, bool element_gather) {
     // about two workgroups per CU, each with at least four 64-wide k-tiles (128x128 output tiles)
     const int64_t tiles = ((pr.M + 127) / 128) * ((pr.N + 127) / 128), k_tiles = (pr.K + 63) / 64;
-    int split = (int)std::max<int64_t>(1, std::min<int64_t>({(512 + tiles - 1) / tiles, k_tiles / 4, 1024}));
+    // (many shares are rounded down: a few workgroups more than fit at once make a second round of the whole launch -
+    // the 56x56x64 layer 102 -> 87 us; few shares are rounded up: 3 instead of 4 leave a quarter of the chip idle)
+    const int64_t shares = 512 / tiles >= 32 ? 512 / tiles : (512 + tiles - 1) / tiles;
+    int split = (int)std::max<int64_t>(1, std::min<int64_t>({shares, k_tiles / 4, 1024}));
     // (an image whose channels do not fill 16-byte chunks is gathered element by element, by 32x64 tiles of two waves: six
     // workgroups per CU, one round of them over the chip)
     if (element_gather && pr.M <= 32 && pr.M > 16 && pr.N >= 128)
