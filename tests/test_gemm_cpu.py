@@ -344,6 +344,7 @@ CONV_CASES = [
     # 64 channels = one k-tile per filter tap: the gather keeps the pixel terms of its rows across the k-loop
     ("hoisted_pixel_terms_ragged_rows", (2, 7, 9, 64), 32, (3, 3), "bf16", (1, 1), (1, 1), "same", "128,128,64,2,2"),
     ("hoisted_pixel_terms_stride2_eight_waves", (1, 12, 10, 128), 64, (3, 3), "bf16", (2, 2), (1, 1), "same", "256,64,64,4,2"),
+    ("hoisted_pixel_terms_eight_waves_of_64x32", (2, 12, 11, 64), 128, (3, 3), "bf16", (1, 1), (1, 1), "same", "128,128,64,2,4"),
     ("hoisted_pixel_terms_f32_dilated", (1, 9, 8, 32), 16, (3, 3), "f32", (1, 1), (2, 2), "valid", "64,64,32,2,2"),
     # channel counts that are no multiple of a chunk: gathered element by element
     ("odd_channels_five_3x3", (2, 7, 6, 5), 16, (3, 3), "bf16", (1, 1), (1, 1), "same", "64,64,64,2,2"),
