@@ -823,13 +823,16 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         // Smaller problems take smaller tiles so that every CU gets work.
         // (a split k range multiplies the workgroups: the filter gradients of 256 and 512 channels keep the large tile,
         // 81 -> 70 us and 93 -> 78 us)
-        if (pr.M <= 128 || pr.N <= 128 || ((pr.M + 255) / 256) * ((pr.N + 255) / 256) * pr.batch * pr.split_k < 128) {
+        // (... of 512; with 256 output channels eight waves on the small tile do better: 46.8 -> 41.5 and 71.1 -> 67.1 us)
+        if (pr.M <= 128 || pr.N <= 128 || ((pr.M + 255) / 256) * ((pr.N + 255) / 256) * pr.batch * pr.split_k < 128 ||
+            (pr.conv_b.on && !f32 && pr.conv_b.C % epc == 0 && pr.M <= 256)) {
             t.bm = t.bn = 128;
             t.wm = t.wn = 2;
             // (a convolution's gather on direct loads: eight waves of 64x32 - twice as many waves issue the per-lane
             // addressed loads and cover each other's waits; at batch 128 the 28x28x128 layer 59.6 -> 42.5 us forward and
             // 60.1 -> 50.3 us data gradient, 14x14x256 54.8 -> 45.7 and 57.3 -> 47.3, 7x7x512 54.7 -> 51.0 and 62.2 -> 49.6)
-            if (!f32 && pr.conv_a.on && pr.conv_a.C % epc == 0) t.wn = 4;
+            // (the same for a filter gradient's gather: 128 output channels 82.4 -> 77.9 us, 54.5 -> 51.3 at stride 2)
+            if (!f32 && ((pr.conv_a.on && pr.conv_a.C % epc == 0) || (pr.conv_b.on && pr.conv_b.C % epc == 0))) t.wn = 4;
             small = true;
             // still fewer workgroups than half the CUs: 64x64 tiles (one MFMA block per wave) spread the work
             // (a split k range multiplies the workgroups instead and keeps the tile's arithmetic intensity)
