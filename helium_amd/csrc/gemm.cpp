@@ -1427,13 +1427,23 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         HE_REQUIRE(pr.batch == 1 && pr.epi.outs.size() == 1 && !pr.epi.outs[0].reduce && pr.epi.exprs.size() == 1, HE_ERR_UNSUPPORTED,
                    "split-k needs an unbatched product with a plain epilogue");
         const tp::Out& o = pr.epi.outs[0];
-        // 32 consecutive output elements per workgroup, 8 threads per element (thread q adds partials q, q + 8, ...),
-        // then one thread per element adds the 8 sums in order
-        s << "extern \"C\" __global__ __launch_bounds__(256) void fused_matmul_finalize(const float* __restrict__ ws, " << tp::c_type(o.dtype)
-          << "* __restrict__ out) {\n__shared__ float part[256];\nconst size_t total = (size_t)GM * GN;\nconst u32 e = threadIdx.x % 32u, pg = threadIdx.x / 32u;\n"
-          << "const size_t i = (size_t)blockIdx.x * 32 + e;\nfloat acc = 0.0f;\nif (i < total) {\n#pragma unroll 4\nfor (u32 sp = pg; sp < " << pr.split_k
-          << "u; sp += 8u) acc += ws[(size_t)sp * total + i];\n}\npart[pg * 32u + e] = acc;\n__syncthreads();\n"
-          << "if (pg == 0 && i < total) {\nfloat r = 0.0f;\n#pragma unroll\nfor (int q = 0; q < 8; q++) r += part[q * 32 + e];\nfloat one[1] = {r};\nst_vec<1>(out + i, one);\n}\n}\n";
+        // 32 consecutive output elements per workgroup. With 16 partial tiles or more and an element count that is a
+        // multiple of 4: 8 threads take 4 elements
+        // each (one 16-byte load per partial tile), 32 such groups share the partials (group q adds partials q, q + 32,
+        // ...), then one thread per element adds the 32 sums in order. Otherwise 8 threads per element, one element each.
+        if ((pr.M * pr.N) % 4 == 0 && pr.split_k >= 16)
+            s << "extern \"C\" __global__ __launch_bounds__(256) void fused_matmul_finalize(const float* __restrict__ ws, " << tp::c_type(o.dtype)
+              << "* __restrict__ out) {\n__shared__ float part[1024];\nconst size_t total = (size_t)GM * GN;\nconst u32 e4 = threadIdx.x % 8u, pg = threadIdx.x / 8u;\n"
+              << "const size_t i = (size_t)blockIdx.x * 32 + e4 * 4u;\nf32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};\nif (i < total) {\n#pragma unroll 4\nfor (u32 sp = pg; sp < " << pr.split_k
+              << "u; sp += 32u) acc += *(const f32x4*)(ws + (size_t)sp * total + i);\n}\n#pragma unroll\nfor (int k = 0; k < 4; k++) part[pg * 32u + e4 * 4u + k] = acc[k];\n__syncthreads();\n"
+              << "const size_t j = (size_t)blockIdx.x * 32 + threadIdx.x;\nif (threadIdx.x < 32u && j < total) {\nfloat r = 0.0f;\n#pragma unroll\nfor (int q = 0; q < 32; q++) r += part[q * 32 + threadIdx.x];\n"
+              << "float one[1] = {r};\nst_vec<1>(out + j, one);\n}\n}\n";
+        else
+            s << "extern \"C\" __global__ __launch_bounds__(256) void fused_matmul_finalize(const float* __restrict__ ws, " << tp::c_type(o.dtype)
+              << "* __restrict__ out) {\n__shared__ float part[256];\nconst size_t total = (size_t)GM * GN;\nconst u32 e = threadIdx.x % 32u, pg = threadIdx.x / 32u;\n"
+              << "const size_t i = (size_t)blockIdx.x * 32 + e;\nfloat acc = 0.0f;\nif (i < total) {\n#pragma unroll 4\nfor (u32 sp = pg; sp < " << pr.split_k
+              << "u; sp += 8u) acc += ws[(size_t)sp * total + i];\n}\npart[pg * 32u + e] = acc;\n__syncthreads();\n"
+              << "if (pg == 0 && i < total) {\nfloat r = 0.0f;\n#pragma unroll\nfor (int q = 0; q < 8; q++) r += part[q * 32 + e];\nfloat one[1] = {r};\nst_vec<1>(out + i, one);\n}\n}\n";
     }
     if (!reds.empty() && !fold_in_kernel) {
         // Second launch: one workgroup folds EB output elements, PG = 256 / EB threads share the partials of each
