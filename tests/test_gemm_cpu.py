@@ -483,6 +483,12 @@ def test_conv_backward_filter_on_cpu(name, image, oc, kernel, dtype, stride, dil
     assert k.description.startswith("repacked") == repacks(image, kernel, dtype, stride, dilation), k.description
 
 
+def test_conv_backward_filter_with_many_partial_tiles_on_cpu(monkeypatch):
+    """Sixteen shares of the k range: the launch that adds the partial tiles up takes them 16 bytes at a time."""
+    monkeypatch.setenv("HELIUM_HIP_GEMM_SPLIT_K", "16")
+    test_conv_backward_filter_on_cpu("sixteen_partial_tiles", (4, 16, 16, 16), 24, (3, 3), "bf16", (1, 1), (1, 1), "same", "64,64,64,2,2")
+
+
 @pytest.mark.parametrize("dtype,precision,tol", [("f32", "f32_f32", 1e-4), ("bf16", "bf16_f32", 2e-2)])
 def test_ir_matmul_with_transposed_operands_on_cpu(dtype, precision, tol):
     """x^T dy and dy w^T of a linear layer's backward pass: each SwapDims joins its Matmul and the kernel reads
