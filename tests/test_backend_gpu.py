@@ -231,6 +231,23 @@ def test_outputs_feed_the_next_graph_and_inputs_stay_intact(gpu):
     assert np.allclose(out, want, rtol=1e-5)
 
 
+def test_a_step_of_many_small_kernels_fans_out_over_streams(gpu):
+    """The executor's own rule (HE_OPT_STREAM_FAN_OUT = 1): sixteen independent kernels over 1 MB each in one step are
+    worth the joins and run on several streams; two are not and share one. (Kernels of 65,536 elements or fewer would be
+    merged into one launch instead.)"""
+    for count, fans in ((16, True), (2, False)):
+        g = ha.ir.OpGraph()
+        xs = [g.new_input([512, 512], "f32") for _ in range(count)]
+        # (two ops per branch that do not fuse across branches: each branch is an instruction of its own)
+        outs = [g.new_output(g.unary(g.unary(x, "exp"), "relu")) for x in xs]
+        rng = np.random.default_rng(count)
+        host = {x: rng.uniform(-1, 1, (512, 512)).astype(np.float32) for x in xs}
+        got, steps = run_graph(g, host)
+        assert max(len(instrs) for instrs, _ in steps) == count, steps
+        assert (stats()["streams_used"] > 1) == fans, stats()
+        check_against_oracle(g, host, got, steps)
+
+
 def test_four_threads_execute_concurrently(gpu):
     # helium/tests/stress_test.rs:16-17: any thread may call execute_graph
     g, names = configs.c1_ir_graph(64, 96, 80)
