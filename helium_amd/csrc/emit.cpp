@@ -306,8 +306,12 @@ int pick_nv(const Program& p, int max_bytes) {
             for (int d = 0; d + 1 < n; d++)
                 if (e.access.stride[d] % v) return false;
         }
-        for (auto& o : p.outs)
+        for (auto& o : p.outs) {
             if (!o.reduce && o.dtype == HE_BOOL) return false;
+            if (!o.reduce && !o.stride.empty() && o.stride[n - 1] == 1)
+                for (int d = 0; d + 1 < n; d++)
+                    if (o.stride[d] % v) return false;
+        }
         return true;
     };
     while (nv > 1 && !ok(nv)) nv /= 2;
@@ -692,7 +696,21 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
         const Out& o = p.outs[oi];
         const std::string v = "e" + std::to_string(o.expr);
         if (!o.reduce) {
-            s << "{ const size_t o = (size_t)b * " << (M * N) << "ull + (size_t)m * " << N << "ull + n0;\n";
+            if (o.stride.empty()) {
+                s << "{ const size_t o = (size_t)b * " << (M * N) << "ull + (size_t)m * " << N << "ull + n0;\n";
+            } else {
+                // stored by its own strides: vectors where its innermost coordinate is the iteration's
+                s << "{ const size_t o = (size_t)0";
+                for (int d = 0; d < n; d++) {
+                    if (o.stride[d] == 0 || p.dims[d] <= 1) continue;
+                    s << " + (size_t)" << (d == n - 1 ? std::string("n0") : d == n - 2 ? std::string("m") : "cB" + std::to_string(d)) << " * " << o.stride[d] << "ull";
+                }
+                s << ";\n";
+                if (!(p.dims[n - 1] <= 1 || o.stride[n - 1] == 1)) {
+                    s << "#pragma unroll\nfor (int k = 0; k < NV; k++) st_one(a" << o.arg << " + o + (size_t)k * " << o.stride[n - 1] << "ull, " << v << "[k]);\n}\n";
+                    continue;
+                }
+            }
             if (o.dtype == HE_BOOL) {
                 // bit k of word o/32; the buffer is cleared before the launch (jit.rs:293-301)
                 s << "#pragma unroll\nfor (int k = 0; k < NV; k++) { const size_t l = o + k; if (" << v

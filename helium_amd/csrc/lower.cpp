@@ -174,10 +174,29 @@ public:
         }
         Mapping ident;
         ident.w = ir::packed_strides(p_.dims);
-        for (ir::NodeId leaf : sg_.leafs()) {
+        // Arguments and outputs are in leaf order; the reductions are lowered first, so that a full-size output of another
+        // shape (the untransposed tensor next to reductions over its leading dims) can be walked the way they walk it.
+        const std::vector<ir::NodeId> leafs = sg_.leafs();
+        p_.outs.resize(leafs.size());
+        out_depth_.assign(leafs.size(), 0);
+        {
+            std::vector<Arg> out_args;
+            for (ir::NodeId leaf : leafs) {
+                const ir::Node& n = g_.get(leaf);
+                if (n.op.kind == ir::OpKind::Reduce) out_args.push_back({HE_F32, ir::num_elements(n.desc.shape), true, leaf});
+                else out_args.push_back({n.desc.dtype, numel, true, leaf});
+            }
+            for (size_t k = 0; k < leafs.size(); k++) p_.outs[k].arg = (int)(p_.args.size() + k);
+            p_.args.insert(p_.args.end(), out_args.begin(), out_args.end());
+        }
+        for (int pass = 0; pass < 2; pass++)
+        for (size_t leaf_no = 0; leaf_no < leafs.size(); leaf_no++) {
+            const ir::NodeId leaf = leafs[leaf_no];
             const ir::Node& n = g_.get(leaf);
+            if ((n.op.kind == ir::OpKind::Reduce) != (pass == 0)) continue;
             Out o;
-            o.arg = (int)p_.args.size();
+            o.arg = p_.outs[leaf_no].arg;
+            cur_out_ = leaf_no;
             if (n.op.kind == ir::OpKind::Reduce) {
                 const Shape& rs = g_.get(n.op.inputs[0]).desc.shape;
                 HE_REQUIRE(ir::num_elements(rs) == numel, HE_ERR_UNSUPPORTED,
@@ -202,8 +221,7 @@ public:
                     o.b_div = 1;
                     for (size_t k = rank - depth; k + 2 < rank; k++) o.b_div *= rdims[k];
                     if (row_dims_ > 1) o.b_div = 1;  // all of the rows fold, or none
-                    out_depth_.resize(p_.outs.size() + 1, 0);
-                    out_depth_[p_.outs.size()] = depth;
+                    out_depth_[leaf_no] = depth;
                     const size_t exprs = p_.exprs.size(), memo = memo_.size();
                     const int acc = p_.acc_expr;
                     try {
@@ -221,15 +239,23 @@ public:
                     lower_permuted_reduction(n, rdims, depth, o);
                 }
                 HE_REQUIRE(p_.exprs[o.expr].cls == Cls::F, HE_ERR_UNSUPPORTED, "reductions take float operands");
-                p_.args.push_back({HE_F32, ir::num_elements(n.desc.shape), true, leaf});
             } else {
                 HE_REQUIRE(ir::num_elements(n.desc.shape) == numel, HE_ERR_UNSUPPORTED,
                            "all outputs of a pointwise kernel must have the same element count");
                 o.dtype = n.desc.dtype;
-                o.expr = eval(leaf, ident);
-                p_.args.push_back({n.desc.dtype, numel, true, leaf});
+                // An output whose shape is that of the tensor the reductions' transposition takes is walked through that
+                // transposition too: it is then written in the order the reductions read. (Also where the transposed
+                // shape is the same - a batch as large as the channel count: the output is a tensor of the untransposed
+                // kind, and any one-to-one walk of it is correct.)
+                auto nat = natural_.find(n.desc.shape);
+                if (anchor_ == ir::kNoNode && n.desc.dtype != HE_BOOL && nat != natural_.end()) {
+                    o.stride = nat->second.w;
+                    o.expr = eval(leaf, nat->second);
+                } else {
+                    o.expr = eval(leaf, ident);
+                }
             }
-            p_.outs.push_back(o);
+            p_.outs[leaf_no] = o;
         }
         if (anchor_ != ir::kNoNode) {
             drop_unused_inputs();
@@ -312,6 +338,8 @@ private:
             if (o.reduce) return;
         for (auto& e : p_.exprs)
             if (e.kind == Expr::Load && (!e.access.chain.empty() || e.access.stride.size() != p_.dims.size())) return;
+        for (auto& o : p_.outs)
+            if (!o.stride.empty()) return;  // (only next to reductions, which returned above)
         for (size_t i = 0; i + 2 < p_.dims.size();) {
             bool ok = true;
             for (auto& e : p_.exprs)
@@ -335,6 +363,8 @@ private:
         const size_t R = p_.dims.size();
         for (auto& e : p_.exprs)
             if (e.kind == Expr::Load && e.access.stride.size() != R) return;
+        for (auto& o : p_.outs)
+            if (!o.stride.empty() && o.stride.size() != R) return;
         out_depth_.resize(p_.outs.size(), 0);
         for (size_t i = 0; i < p_.outs.size(); i++) {
             if (!p_.outs[i].reduce) continue;
@@ -347,6 +377,8 @@ private:
             p_.dims.erase(p_.dims.begin() + d);
             for (auto& e : p_.exprs)
                 if (e.kind == Expr::Load) e.access.stride.erase(e.access.stride.begin() + d);
+            for (auto& o : p_.outs)
+                if (!o.stride.empty()) o.stride.erase(o.stride.begin() + d);
         }
         const size_t rank = p_.dims.size();
         for (size_t i = 0; i < p_.outs.size(); i++) {
@@ -392,12 +424,19 @@ private:
         // Small tensors stay as they are: they live in the caches whatever the order, and rows that one wave folds
         // need no exchange between blocks, which at that size costs more than the strided reads.
         if (ir::num_elements(p_.dims) < fold_columns_threshold()) return;
+        // (full-size outputs may sit next to the reductions when they are stored by strides of their own)
         size_t depth = 0;
+        bool any_reduce = false;
         for (size_t i = 0; i < p_.outs.size(); i++) {
-            if (!p_.outs[i].reduce) return;
-            if (i && out_depth_[i] != out_depth_[0]) return;
+            if (!p_.outs[i].reduce) {
+                if (p_.outs[i].stride.size() != R) return;
+                continue;
+            }
+            if (any_reduce && out_depth_[i] != depth) return;
+            depth = out_depth_[i];
+            any_reduce = true;
         }
-        depth = out_depth_[0];
+        if (!any_reduce) return;
         if (depth >= R) return;
         const size_t K = R - depth, kl = K - 1;
         const Expr* big = nullptr;
@@ -423,11 +462,15 @@ private:
         permute(p_.dims);
         for (auto& e : p_.exprs)
             if (e.kind == Expr::Load) permute(e.access.stride);
+        for (auto& o : p_.outs)
+            if (!o.reduce) permute(o.stride);
         // merge neighbours among the folded dims (positions K-1 .. size-2) that every operand walks as one dim
         for (size_t i = K - 1; i + 2 < p_.dims.size();) {
             bool ok = true;
             for (auto& e : p_.exprs)
                 if (e.kind == Expr::Load && e.access.stride[i] != e.access.stride[i + 1] * p_.dims[i + 1]) ok = false;
+            for (auto& o : p_.outs)
+                if (!o.reduce && o.stride[i] != o.stride[i + 1] * p_.dims[i + 1]) ok = false;
             if (!ok) {
                 i++;
                 continue;
@@ -436,10 +479,13 @@ private:
             p_.dims.erase(p_.dims.begin() + i);
             for (auto& e : p_.exprs)
                 if (e.kind == Expr::Load) e.access.stride.erase(e.access.stride.begin() + i);
+            for (auto& o : p_.outs)
+                if (!o.reduce) o.stride.erase(o.stride.begin() + i);
         }
         int64_t b_div = 1;
         for (size_t i = K - 1; i + 2 < p_.dims.size(); i++) b_div *= p_.dims[i];
         for (auto& o : p_.outs) {
+            if (!o.reduce) continue;
             o.fold_n = false;
             o.fold_m = true;
             o.b_div = b_div;
@@ -505,8 +551,12 @@ private:
         const ir::Op& op = n.op;
         auto in_shape = [&](size_t i) -> const Shape& { return g_.get(op.inputs[i]).desc.shape; };
         switch (op.kind) {
-            case ir::OpKind::SwapDims:
-                return eval(op.inputs[0], through_swap(mp, p_.dims, n.desc.shape, in_shape(0), op.axis_a, op.axis_b));
+            case ir::OpKind::SwapDims: {
+                Mapping below = through_swap(mp, p_.dims, n.desc.shape, in_shape(0), op.axis_a, op.axis_b);
+                // (how the iteration space walks a tensor of the untransposed shape: kept for full-size outputs of it)
+                if (below.chain.empty() && g_.get(op.inputs[0]).op.kind != ir::OpKind::SwapDims) natural_.emplace(in_shape(0), below);
+                return eval(op.inputs[0], below);
+            }
             case ir::OpKind::Broadcast: {
                 std::vector<char> flags(n.desc.shape.size(), 0);
                 for (auto& a : op.broadcast_axes) flags[a.axis] = 1;
@@ -597,6 +647,8 @@ private:
     std::map<ir::NodeId, int> input_arg_;
     std::vector<Memo> memo_;
     std::vector<size_t> out_depth_;  // per output: the Reduce's depth (0 for full-size outputs)
+    std::map<Shape, Mapping> natural_;  // shape of a transposition's operand -> the affine mapping the iteration walks it with
+    size_t cur_out_ = 0;
 };
 
 // ---------------------------------------------------------------------------------------------------------
@@ -896,19 +948,37 @@ bool pointwise_supports(const ir::OpSubgraph& sg) {
     // tensor in memory order when every output of the kernel is such a reduction; any other output next to them (the
     // transposed tensor itself, or a tensor of the same extents in another order - a batch as large as the channel
     // count makes the two shapes equal) would be written element by element.
-    if (plan::rematerialize() && output_size >= fold_columns_threshold()) {
+    if (plan::rematerialize() && output_size >= fold_columns_threshold() && sg.nodes().size() > 1) {
+        // The one other output such a kernel may have: a full-size tensor of the shape the transpositions take (the
+        // untransposed tensor, or one computed element by element from it), provided every transposition is there for
+        // the reductions alone. It is stored through the same walk (tp::Out::stride), in memory order.
+        bool transposes = false, swaps_for_reductions = true, one_source_shape = true;
+        const Shape* source_shape = nullptr;
+        for (ir::NodeId node : sg.nodes()) {
+            const ir::Op& op = g.get(node).op;
+            if (op.kind != ir::OpKind::SwapDims) continue;
+            transposes = true;
+            swaps_for_reductions = swaps_for_reductions && plan::feeds_only_reductions(g, node, 64);
+            const ir::Node& in = g.get(op.inputs[0]);
+            if (in.kind == ir::Node::Intermediate && in.op.kind == ir::OpKind::SwapDims) continue;
+            if (source_shape && *source_shape != in.desc.shape) one_source_shape = false;
+            source_shape = &in.desc.shape;
+        }
         const Shape* shape = nullptr;
-        bool transposes = false, only_reductions = true;
-        for (ir::NodeId node : sg.nodes()) transposes = transposes || g.get(node).op.kind == ir::OpKind::SwapDims;
         for (ir::NodeId node : sg.leafs()) {
             const ir::Op& op = g.get(node).op;
             // (an output on its way to reductions that have not joined yet is let through: instructions fuse in pairs)
-            only_reductions = only_reductions && (op.kind == ir::OpKind::Reduce || plan::feeds_only_reductions(g, node, 64));
+            const bool for_reductions = op.kind == ir::OpKind::Reduce || plan::feeds_only_reductions(g, node, 64);
             const Shape& mine = g.get(op.kind == ir::OpKind::Reduce ? op.inputs[0] : node).desc.shape;
+            if (transposes && !for_reductions) {
+                if (!(swaps_for_reductions && one_source_shape && source_shape && *source_shape == mine && have_red &&
+                      g.get(node).desc.dtype != HE_BOOL))
+                    return false;
+                continue;
+            }
             if (shape && *shape != mine) return false;
             shape = &mine;
         }
-        if (transposes && !only_reductions && sg.nodes().size() > 1) return false;
     }
     return true;
 }

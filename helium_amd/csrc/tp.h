@@ -63,6 +63,10 @@ struct Out {
     bool fold_n = false, fold_m = false;
     int64_t b_div = 1;
     double mean_scale = 1.0;  // Mean multiplies every term by this (as a double, jit.rs:599-604)
+    // A full-size output that is not stored in iteration order: per iteration dim, the stride of its coordinate in the
+    // output (an untransposed tensor written by a kernel that iterates in the index space of its reductions). Empty:
+    // element i of the iteration space is element i of the output.
+    std::vector<int64_t> stride;
 };
 
 struct Arg {

@@ -269,6 +269,17 @@ def generated_cases():
     x = c.inp([6, 5, 4, 32], "f32", rng.standard_normal(6 * 5 * 4 * 32)); y = c.inp([32, 5, 4, 6], "f32", rng.standard_normal(6 * 5 * 4 * 32))
     c.out(c.op(c.g.reduce(c.op(c.g.binary(c.op(c.g.swap_dims(x, 0, 3)), y, "mul")), "sum", 3))); c.reduce_rel = 1e-3; cases.append(c)
 
+    # A full-size output next to reductions over its leading dims (the input gradient of a batch norm and the channel
+    # sums of the next one): the untransposed tensor is written through the same walk, in memory order.
+    c = Case("full_size_output_next_to_channel_sums"); c.env = FOLD_SMALL; c.admitted_by_fusion_rule = False
+    x = c.inp([3, 5, 4, 32], "f32", rng.standard_normal(3 * 5 * 4 * 32)); sc = c.inp([32], "f32", rng.uniform(0.5, 2.0, 32))
+    y = c.op(c.g.unary(c.op(c.g.binary(x, c.op(c.g.broadcast(sc, 4, [(0, 3), (1, 5), (2, 4)])), "mul")), "relu"))
+    yt = c.op(c.g.swap_dims(y, 0, 3))
+    c.out(y)
+    c.out(c.op(c.g.reduce(yt, "sum", 3)))
+    c.out(c.op(c.g.reduce(c.op(c.g.binary(yt, c.op(c.g.swap_dims(x, 0, 3)), "mul")), "sum", 3)))
+    c.reduce_rel = 1e-3; cases.append(c)
+
     return cases
 
 
