@@ -752,7 +752,9 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
         const int64_t TRv = (int64_t)TY * RPT;
         const bool ragged = M % TRv != 0 || N % ((int64_t)TX * NV) != 0;
         // UNROLL rows are in flight at a time: all RPT at once would keep every row's operands in registers
-        int unroll = std::min(RPT, 2);
+        // (one row where the expression count is large: two rows of a 75-expression kernel keep twice the registers and
+        // gain nothing; training step with the limit at none / 64 / 40 / 24 expressions: 5.34 / 5.31 / 5.30 / 5.28 ms)
+        int unroll = std::min(RPT, p.exprs.size() > 24 ? 1 : 2);
         if (const char* env = tuning::get("HELIUM_HIP_POINTWISE_UNROLL")) unroll = std::max(1, std::min(RPT, atoi(env)));
         while (RPT % unroll) unroll--;
         const std::string head = "#pragma unroll 1\nfor (u32 i0 = 0; i0 < RPT; i0 += " + std::to_string(unroll) + ") {\n#pragma unroll\nfor (u32 iu = 0; iu < " +
