@@ -890,7 +890,12 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
     if (any_finalize) {
         // The second launch: one block per 16 output columns (or per scalar output) folds that slice of the
         // partials, 16 thread groups sharing the blocks of the first launch between them, always in the same order.
-        const int FW = 16, FG = threads / FW;
+        // (fewer columns and more groups where a column has many partials: a thread then adds a few dozen of them, eight
+        // loads at a time, instead of a hundred one batch after the other - the launch is all latency)
+        auto fold_width = [&](const Out& o) {
+            const int64_t arrivals = gy * o.b_div;
+            return arrivals >= 512 ? 4 : arrivals >= 128 ? 8 : 16;
+        };
         struct Job {
             size_t oi;
             uint32_t first, blocks;
@@ -900,6 +905,7 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
         for (size_t oi = 0; oi < p.outs.size(); oi++) {
             if (!ws[oi].on || ws[oi].ticket) continue;
             const Out& o = p.outs[oi];
+            const int FW = fold_width(o);
             const uint32_t nb = o.fold_n ? (uint32_t)(B / o.b_div) : (uint32_t)((B / o.b_div) * ((N + FW - 1) / FW));
             jobs.push_back({oi, total, nb});
             total += nb;
@@ -916,6 +922,7 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
             s << "if (blockIdx.x >= " << jb.first << "u && blockIdx.x < " << jb.first + jb.blocks << "u) {\nconst u32 job = blockIdx.x - " << jb.first
               << "u;\nfloat acc = red_identity<" << rop << ">();\n";
             if (!o.fold_n) {
+                const int FW = fold_width(o), FG = threads / FW;
                 const int64_t arrivals = gy * o.b_div, slices = (N + FW - 1) / FW;
                 s << "const u32 q = job / " << slices << "u, n = (job % " << slices << "u) * " << FW << "u + threadIdx.x % " << FW
                   << "u, grp = threadIdx.x / " << FW << "u;\nconst u32 tile_x = n / (TX * NV), within = n % (TX * NV);\nif (n < DIM_N) {\n"
