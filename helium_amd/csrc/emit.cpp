@@ -679,7 +679,7 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
         }
     }
     std::ostringstream& main_stream = s;
-    auto row_body = [&](bool squares) {
+    auto row_body = [&](bool squares, bool from_raw) {
     std::ostringstream s;
     for (size_t oi = 0; oi < p.outs.size(); oi++)
         if (p.outs[oi].reduce && p.outs[oi].fold_n && !p.outs[oi].fold_m)
@@ -689,6 +689,8 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
     cx.nv = NV;
     cx.uniform_pow_is_square = squares;
     cx.row_part = hoist_rows ? 2 : 0;
+    cx.phase = from_raw ? 2 : 0;
+    cx.defer_row_varying_only = from_raw;
     s << emit_exprs(p, cx);
     // outputs
     Shape pst = ir::packed_strides(p.dims);
@@ -762,13 +764,43 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
         // (a launch of a few workgroups runs its code once or twice: a second form of the body without the bounds tests
         // costs more in instruction fetch than the tests do)
         const bool few_blocks = grid <= 16;
-        auto loops = [&](const std::string& body) {
+        // One row in flight per thread leaves a streaming kernel short of outstanding loads (three 8-byte loads per
+        // lane, four waves per SIMD: 24 KB per CU). The next row's operands are therefore requested before the current
+        // row is computed: they cost a few registers, where a second whole row in flight would double all of them.
+        bool any_deferred = false;
+        for (const Expr& e : p.exprs) any_deferred = any_deferred || is_deferred_load(p, e, NV, true);
+        bool pipelined = unroll == 1 && RPT >= 2 && any_deferred && !few_blocks;
+        int ahead = 1;  // rows requested ahead of the one being computed
+        if (const char* env = tuning::get("HELIUM_HIP_POINTWISE_PIPELINE")) ahead = atoi(env);
+        ahead = std::min(ahead, RPT - 1);
+        pipelined = pipelined && ahead >= 1;
+        std::string ahead_head, ahead_tail;
+        if (pipelined) {
+            EmitCtx lx;
+            lx.nv = NV;
+            lx.row_part = hoist_rows ? 2 : 0;
+            lx.phase = 1;
+            lx.defer_row_varying_only = true;
+            const std::string issue = emit_exprs(p, lx);
+            s << "struct RowRaw {\n" << emit_raw_members(p, NV, true) << "};\n";
+            auto name = [](int d) { return d == 0 ? std::string("R") : "R" + std::to_string(d); };
+            for (int d = 0; d < ahead; d++)
+                ahead_head += "RowRaw " + name(d) + ";\n{ const u32 m = tile_y * TR + " + std::to_string(d) + " * TY + ty;\n" +
+                              (d ? "RowRaw& R = " + name(d) + ";\n" : std::string()) + issue + "}\n";
+            ahead_head += "#pragma unroll 1\nfor (u32 i = 0; i < RPT; i++) {\nconst u32 m = tile_y * TR + i * TY + ty;\nRowRaw Rn;\n{ const u32 i1 = i + " +
+                          std::to_string(ahead) + " < RPT ? i + " + std::to_string(ahead) + " : RPT - 1;\nconst u32 m = tile_y * TR + i1 * TY + ty;\nRowRaw& R = Rn;\n" +
+                          issue + "}\n{\n";
+            for (int d = 0; d + 1 < ahead; d++) ahead_tail += name(d) + " = " + name(d + 1) + ";\n";
+            ahead_tail += name(ahead - 1) + " = Rn;\n";
+        }
+        auto loops = [&](const std::string& body, const std::string& body_from_raw) {
             if (ragged && few_blocks) {
                 s << head << "const bool ok = col_ok && m < DIM_M;\n" << body << "}\n}\n";
                 return;
             }
             if (ragged) s << "if ((tile_y + 1) * TR <= DIM_M && (tile_x + 1) * (TX * NV) <= DIM_N) {\n";
-            s << head << "const bool ok = true;\n" << body << "}\n}\n";
+            if (pipelined) s << ahead_head << "const bool ok = true;\n" << body_from_raw << "}\n" << ahead_tail << "}\n";
+            else s << head << "const bool ok = true;\n" << body << "}\n}\n";
             if (ragged) s << "} else {\n" << head << "const bool ok = col_ok && m < DIM_M;\n" << body << "}\n}\n}\n";
         };
         // `x.pow_scalar(2.0)` reaches the kernel as Pow with a broadcast 1-element operand. The exponents are read
@@ -780,14 +812,14 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
         std::sort(exps.begin(), exps.end());
         exps.erase(std::unique(exps.begin(), exps.end()), exps.end());
         if (exps.empty()) {
-            loops(row_body(false));
+            loops(row_body(false, false), pipelined ? row_body(false, true) : std::string());
         } else {
             s << "bool all_squares = true;\n";
             for (int a : exps) s << "all_squares = all_squares && ld_one(a" << a << ") == 2.0f;\n";
             s << "if (all_squares) {\n";
-            loops(row_body(true));
+            loops(row_body(true, false), pipelined ? row_body(true, true) : std::string());
             s << "} else {\n";
-            loops(row_body(false));
+            loops(row_body(false, false), pipelined ? row_body(false, true) : std::string());
             s << "}\n";
         }
     }
