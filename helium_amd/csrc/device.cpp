@@ -6,6 +6,7 @@
 #include <mutex>
 
 #include "common.h"
+#include "exec.h"
 #include "rtc.h"
 
 namespace he {
@@ -180,7 +181,10 @@ int he_device_arch(int device, char* buf, size_t buf_len) {
 }
 
 int he_device_synchronize(void) {
-    return he::guard([&] { HE_HIP(hipDeviceSynchronize()); });
+    return he::guard([&] {
+        HE_HIP(hipDeviceSynchronize());
+        he::exec::DevicePool::poll_if_created();
+    });
 }
 
 int he_stream_create(he_stream_t* stream) {
@@ -198,7 +202,10 @@ int he_stream_destroy(he_stream_t stream) {
     });
 }
 int he_stream_synchronize(he_stream_t stream) {
-    return he::guard([&] { HE_HIP(hipStreamSynchronize(raw(stream))); });
+    return he::guard([&] {
+        HE_HIP(hipStreamSynchronize(raw(stream)));
+        he::exec::DevicePool::poll_if_created();
+    });
 }
 namespace {
 struct HostCb {
@@ -245,7 +252,10 @@ int he_event_wait(he_event_t event, he_stream_t stream) {
     return he::guard([&] { HE_HIP(hipStreamWaitEvent(raw(stream), event->e, 0)); });
 }
 int he_event_synchronize(he_event_t event) {
-    return he::guard([&] { HE_HIP(hipEventSynchronize(event->e)); });
+    return he::guard([&] {
+        HE_HIP(hipEventSynchronize(event->e));
+        he::exec::DevicePool::poll_if_created();
+    });
 }
 int he_event_elapsed_ms(he_event_t start, he_event_t stop, float* ms) {
     return he::guard([&] { HE_HIP(hipEventElapsedTime(ms, start->e, stop->e)); });

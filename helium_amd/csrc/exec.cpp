@@ -2,6 +2,7 @@
 #include "exec.h"
 
 #include <algorithm>
+#include <atomic>
 #include <cstring>
 #include <future>
 #include <set>
@@ -11,9 +12,19 @@ namespace he::exec {
 // ---------------------------------------------------------------------------------------------------------
 // Device pool
 // ---------------------------------------------------------------------------------------------------------
+static std::atomic<DevicePool*> g_pool{nullptr};
+
 DevicePool& DevicePool::global() {
-    static DevicePool* pool = new DevicePool();  // never destroyed: tensors may outlive static destruction order
+    static DevicePool* pool = [] {
+        DevicePool* p = new DevicePool();  // never destroyed: tensors may outlive static destruction order
+        g_pool.store(p, std::memory_order_release);
+        return p;
+    }();
     return *pool;
+}
+
+void DevicePool::poll_if_created() {
+    if (DevicePool* p = g_pool.load(std::memory_order_acquire)) p->poll();
 }
 
 SharedEvent::~SharedEvent() {

@@ -49,6 +49,11 @@ public:
     // from allocate, so no host callback sits in any stream.
     void end_scope_after(uint64_t scope, EventRef done);
     void poll();
+    // The same, for callers that have just waited for the device (stream / event / device synchronize): retiring the
+    // executions that finished meanwhile is then part of the wait and not of the next execution's set-up (a host that
+    // ran 200 executions ahead found all of them to retire, 2.5 us each, at the head of its next call). No-op before
+    // the pool exists.
+    static void poll_if_created();
     Allocation allocate(size_t bytes, uint64_t scope);
     // `owner`: the scope the block was allocated in (0: none); `used`: every scope whose device work touches it. The
     // block is free again for whoever comes after all of those that are still live.

@@ -24,6 +24,10 @@ struct Dim3 { unsigned x = 0, y = 0, z = 0; };
 static thread_local Dim3 threadIdx, blockIdx;
 static Dim3 blockDim, gridDim;
 static pthread_barrier_t g_bar;
+// wave-level stand-ins (shuffles, matrix-core and transposing loads) meet on their own wave's barrier, so the waves of a
+// block need not run the same instruction stream (two groups of waves half a k-tile apart)
+static pthread_barrier_t g_wbar[16];
+#define WAVE_BAR() pthread_barrier_wait(&g_wbar[threadIdx.x >> 6])
 #define __global__
 #define __device__
 #define __forceinline__ inline
@@ -34,14 +38,14 @@ static pthread_barrier_t g_bar;
 #define __builtin_nontemporal_load(p) (*(p))
 #define __builtin_nontemporal_store(v, p) (*(p) = (v))
 #include <cmath>
-// wave shuffles: every thread of the block calls in lockstep, so a block-wide exchange through memory works
+// wave shuffles: every thread of a wave calls in lockstep, so an exchange through memory between wave barriers works
 static float g_shfl[1024];
 static inline float __shfl_xor(float v, int mask, int width) {
     unsigned tid = threadIdx.x;
     g_shfl[tid] = v;
-    pthread_barrier_wait(&g_bar);
+    WAVE_BAR();
     float r = g_shfl[(tid & ~63u) | ((tid & 63u) ^ (unsigned)mask)];
-    pthread_barrier_wait(&g_bar);
+    WAVE_BAR();
     return r;
 }
 static inline int __float_as_int(float f) { int i; memcpy(&i, &f, 4); return i; }
@@ -81,7 +85,7 @@ template <class V, bool BF> static inline emu_f32x16 emu_mfma(V a, V b, emu_f32x
     unsigned tid = threadIdx.x, base = tid & ~63u, lane = tid & 63u;
     g_mfa[tid] = __builtin_bit_cast(emu_s16x8, a);
     g_mfb[tid] = __builtin_bit_cast(emu_s16x8, b);
-    pthread_barrier_wait(&g_bar);
+    WAVE_BAR();
     for (int i = 0; i < 16; i++) {
         unsigned row = (i / 4) * 8 + (lane / 32) * 4 + i % 4, col = lane % 32;
         float sum = 0;
@@ -91,7 +95,7 @@ template <class V, bool BF> static inline emu_f32x16 emu_mfma(V a, V b, emu_f32x
         }
         c[i] += sum;
     }
-    pthread_barrier_wait(&g_bar);
+    WAVE_BAR();
     return c;
 }
 #define __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, x, y, z) emu_mfma<decltype(a), true>(a, b, c)
@@ -101,12 +105,12 @@ static inline emu_f32x16 emu_mfma_f32(float a, float b, emu_f32x16 c) {
     // v_mfma_f32_32x32x2_f32: lane l holds A[l%32][l/32] and B[l/32][l%32]
     unsigned tid = threadIdx.x, base = tid & ~63u, lane = tid & 63u;
     g_mfa32[tid] = a; g_mfb32[tid] = b;
-    pthread_barrier_wait(&g_bar);
+    WAVE_BAR();
     for (int i = 0; i < 16; i++) {
         unsigned row = (i / 4) * 8 + (lane / 32) * 4 + i % 4, col = lane % 32;
         c[i] += g_mfa32[base + row] * g_mfb32[base + col] + g_mfa32[base + 32 + row] * g_mfb32[base + 32 + col];
     }
-    pthread_barrier_wait(&g_bar);
+    WAVE_BAR();
     return c;
 }
 #define __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, x, y, z) emu_mfma_f32(a, b, c)
@@ -116,10 +120,10 @@ static inline emu_s16x4 emu_tr16(const emu_s16x4* p) {
     // four source lanes 4e + L/4 (e = 0..3)
     unsigned tid = threadIdx.x, gbase = tid & ~15u, L = tid & 15u;
     g_traddr[tid] = (const short*)p;
-    pthread_barrier_wait(&g_bar);
+    WAVE_BAR();
     emu_s16x4 r;
     for (int e = 0; e < 4; e++) r[e] = g_traddr[gbase + 4 * e + L / 4][L % 4];
-    pthread_barrier_wait(&g_bar);
+    WAVE_BAR();
     return r;
 }
 #define __builtin_amdgcn_ds_read_tr16_b64_v4i16(p) emu_tr16(p)
@@ -134,7 +138,8 @@ static inline emu_s16x4 emu_tr16(const emu_s16x4* p) {
 #define __builtin_amdgcn_sched_barrier(x)
 #define __builtin_amdgcn_sched_group_barrier(a, b, c)
 #define __builtin_amdgcn_s_setprio(x)
-#define __builtin_amdgcn_wave_barrier() pthread_barrier_wait(&g_bar)
+#define __builtin_amdgcn_wave_barrier() WAVE_BAR()
+#define __builtin_amdgcn_readfirstlane(x) (x)
 #define __expf expf
 #define HE_FAST_RCP(x) (1.0f / (x))
 #define HE_OPAQUE(x) (x)
@@ -179,6 +184,7 @@ int main(int argc, char** argv) {
     }
     g_bufs = bufs.data();
     pthread_barrier_init(&g_bar, nullptr, blockDim.x);
+    for (unsigned w = 0; w < (blockDim.x + 63) / 64; w++) pthread_barrier_init(&g_wbar[w], nullptr, blockDim.x - w * 64 < 64 ? blockDim.x - w * 64 : 64);
     std::vector<pthread_t> th(blockDim.x);
     for (unsigned t = 0; t < blockDim.x; t++) pthread_create(&th[t], nullptr, worker, (void*)(size_t)t);
     for (auto& t : th) pthread_join(t, nullptr);
