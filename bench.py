@@ -22,9 +22,25 @@ METRIC = "fused-GEMM TFLOP/s & permute/pointwise GB/s, % of MI355X roofline"
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 BF16_PEAK_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
 F32_PEAK_TFLOPS = 157.3      # MI355X dense fp32 matrix, published
-# Bytes that left the XCD L2s per launch of each workload's dominant kernel: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE,
-# each scaled by what the same counter reads for the COPY workload (profiles/<kernel>_<workload>.txt).
-TRAFFIC_BYTES = {"COPY": 268435456, "C2a": 205509374, "C2b": 67196580, "C2c": 12867962, "C3": 269743029, "C4": 370218917, "C5a-fused": 302134023, "C5a-planned": 335673461, "GEMM": 234914277, "C5b-bn": 313174768, "C5b-conv": 52383120}
+
+
+def _traffic_table():
+    """Bytes that leave the XCD L2s per launch of each workload's dominant kernel, from the committed counter summary
+    (profiles/traffic_per_launch.txt: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by the COPY workload); a workload
+    the file does not list reports null."""
+    table = {}
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "traffic_per_launch.txt")
+    try:
+        for line in open(path):
+            parts = line.split()
+            if len(parts) == 3 and not line.startswith("#"):
+                table[parts[0]] = int(parts[2])
+    except OSError:
+        pass
+    return table
+
+
+TRAFFIC_BYTES = _traffic_table()
 HEADLINE = "C4"              # the workload `value` is quoted on
 ROTATE_BYTES = 768 << 20     # rotate operand sets so repeated steps cannot live in the 256 MB Infinity Cache
 
@@ -53,6 +69,7 @@ class PermuteWorkload:
 
     def describe(self):
         return f"{self.name}: bf16 {list(self.shape)} permute {self.perm}"
+
 
     def setup(self):
         import helium_amd as ha
@@ -98,6 +115,70 @@ class PermuteWorkload:
     def free(self):
         for s, d in self.sets:
             s.free()
+            d.free()
+        self.sets = []
+
+
+class ReferencePermuteWorkload:
+    """The reference's own permute benchmark (helium/examples/permute_dim_benchmark.rs:13-41): f32 [2048,128,128,32],
+    swap_dims(0, 3), 4.3 GB in and 4.3 GB out, so every byte comes from HBM. Input element i holds the value i, which
+    makes every output element's expected value a closed form of its index."""
+
+    bound = "hbm"
+    unit = "GB/s"
+    dtype = "f32"
+    name = "PERM-ref"
+
+    def __init__(self):
+        from helium_amd import configs
+
+        self.shape, self.perm = configs.PERM_REF_SHAPE, configs.PERM_REF_PERM
+        self.numel = int(np.prod(self.shape))
+        self.work = 2 * self.numel * 4
+
+    def describe(self):
+        return f"PERM-ref: f32 {list(self.shape)} swap_dims(0, 3) (the reference's permute_dim_benchmark)"
+
+    def setup(self):
+        import helium_amd as ha
+
+        self.op = ha.PermuteDims(self.shape, "f32", perm=self.perm)
+        self.inverse = ha.PermuteDims(self.op.out_shape, "f32", perm=self.perm)  # swap_dims(0, 3) undoes itself
+        host = np.arange(self.numel, dtype=np.uint32)
+        self.sets = [(ha.DeviceBuffer.from_numpy(host), ha.DeviceBuffer(host.nbytes)) for _ in range(2)]
+        del host
+        log(f"[bench] {self.describe()} :: {self.op.description} :: 2 operand sets")
+
+    def step(self, stream, i):
+        src, dst = self.sets[i % 2]
+        self.op.execute(src, dst, stream)
+
+    def check(self):
+        from helium_amd import configs
+
+        src, dst = self.sets[0]
+        rng = np.random.default_rng(5)
+        row = self.shape[0]  # the output's innermost extent
+        for start in rng.integers(0, self.numel // row, size=256):
+            got = dst.read(int(start) * row * 4, np.uint32, row)
+            want = configs.perm_ref_expected(np.arange(int(start) * row, (int(start) + 1) * row, dtype=np.uint64))
+            if not np.array_equal(got, want):
+                raise SystemExit("[bench] PARITY FAILURE in PERM-ref: a sampled output row differs from the closed form")
+        # and back: the same permute applied to the output restores the input bit for bit (sampled rows of 1 MiB)
+        back = self.sets[1][1]
+        self.inverse.execute(dst, back)
+        for start in rng.integers(0, self.numel // (1 << 18), size=64):
+            got = back.read(int(start) * (1 << 20), np.uint32, 1 << 18)
+            if not np.array_equal(got, np.arange(int(start) << 18, (int(start) + 1) << 18, dtype=np.uint32)):
+                raise SystemExit("[bench] PARITY FAILURE in PERM-ref: permuting twice does not restore the input")
+        return "256 sampled output rows equal the closed form; permuting twice restores 64 sampled MiB of the input bit for bit"
+
+    def cpu_baseline(self, budget_s=10.0):
+        return None
+
+    def free(self):
+        for s_, d in self.sets:
+            s_.free()
             d.free()
         self.sets = []
 
@@ -266,7 +347,8 @@ class BatchNormWorkload:
 
     def setup(self):
         import helium_amd as ha
-        from helium_amd import configs, frontend
+        from helium_amd import configs
+        from harness import frontend
         from helium_amd.backend import Plan, Tensor
 
         g = ha.ir.OpGraph()
@@ -400,7 +482,8 @@ class ConvBatchNormWorkload(ConvWorkload):
 
     def setup(self):
         import helium_amd as ha
-        from helium_amd import configs, frontend
+        from helium_amd import configs
+        from harness import frontend
         from helium_amd.backend import Plan, Tensor
 
         g = ha.ir.OpGraph()
@@ -570,7 +653,8 @@ class SgdWorkload:
 
     def setup(self):
         import helium_amd as ha
-        from helium_amd import configs, frontend
+        from helium_amd import configs
+        from harness import frontend
         from helium_amd.backend import Plan, Tensor
 
         g = ha.ir.OpGraph()
@@ -640,7 +724,8 @@ class BasicBlockWorkload:
     @staticmethod
     def build(shape, seed):
         import helium_amd as ha
-        from helium_amd import configs, frontend
+        from helium_amd import configs
+        from harness import frontend
 
         g = ha.ir.OpGraph()
         rec = frontend.Recorder(g)
@@ -890,7 +975,7 @@ class TrainStepWorkload:
                 f"{self.image}x{self.image}x3 bf16 images, 1000 classes, via execute_graph")
 
     def setup(self):
-        from helium_amd import resnet
+        from harness import resnet
         from helium_amd.backend import Tensor, stats
 
         self.rec = resnet.record_training_step(self.batch, self.image)
@@ -1025,6 +1110,44 @@ class PlannedGemmWorkload(FusedGemmWorkload):
         self.sets = []
 
 
+CEILING_CHILD = r"""
+import json, sys
+import torch
+assert torch.cuda.is_available()
+n = 4096
+sets = [(torch.randn(n, n, device='cuda', dtype=torch.bfloat16) * 0.02, torch.randn(n, n, device='cuda', dtype=torch.bfloat16) * 0.02) for _ in range(8)]
+out = torch.empty(n, n, device='cuda', dtype=torch.bfloat16)
+def run(fn):
+    for i in range(200): fn(*sets[i % 8])
+    torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for i in range(100): fn(*sets[i % 8])
+    e.record(); torch.cuda.synchronize()
+    return 2 * n ** 3 / (s.elapsed_time(e) / 100 * 1e-3) / 1e12
+print("CEILINGS " + json.dumps({"hipblaslt_nn_TFLOPs": round(run(lambda a, b: torch.matmul(a, b, out=out)), 1),
+                                "hipblaslt_nt_TFLOPs": round(run(lambda a, b: torch.matmul(a, b.t(), out=out)), 1)}))
+"""
+
+
+def vendor_gemm_ceiling():
+    """The vendor library's bf16 4096^3 GEMM on the same box (torch.matmul -> hipBLASLt; NN, and NT = B stored [n][k]),
+    with the same warm-up and operand rotation as the GEMM workload: the analogue of the reference's benchmark printing
+    its kernel next to cuBLASLt (helium-kernel-generator/benches/src/main.rs:35-46). Measured in a child process of its
+    own before this process touches the device, so nothing of it lies inside a timed region. Returns the two figures, or
+    a reason string when torch is not usable."""
+    import subprocess
+
+    try:
+        r = subprocess.run([sys.executable, "-c", CEILING_CHILD], capture_output=True, text=True, timeout=420)
+    except Exception as e:  # noqa: BLE001
+        return {"skipped": f"child process failed: {e}"}
+    for line in r.stdout.splitlines():
+        if line.startswith("CEILINGS "):
+            return json.loads(line[9:])
+    return {"skipped": "torch not usable: " + (r.stderr.strip().splitlines() or ["no output"])[-1][:200]}
+
+
 def make_workloads():
     from helium_amd import configs
 
@@ -1033,6 +1156,7 @@ def make_workloads():
     # a plain copy of known size (identity permute): the measured ceiling the permute kernels are read against and
     # the scale for the FETCH_SIZE / WRITE_SIZE counters
     w["COPY"] = PermuteWorkload("COPY", (8192, 8192), (0, 1), 24)
+    w["PERM-ref"] = ReferencePermuteWorkload()
     w["C1"] = LinearLayerWorkload()
     w["C3"] = AuxChainWorkload()
     w["C5b-bn"] = BatchNormWorkload()
@@ -1102,10 +1226,14 @@ def main():
     ap.add_argument("--workload", default=None, help="headline workload (default: the best-covered BASELINE config)")
     ap.add_argument("--only", action="store_true", help="measure the headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-ceilings", action="store_true", help="skip the vendor-library GEMM measured on the same box")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
 
+    ceilings = {"skipped": "--only / --no-ceilings"} if (args.only or args.no_ceilings) else vendor_gemm_ceiling()
+    if "skipped" not in ceilings:
+        log(f"[bench] same-box ceilings: hipBLASLt bf16 4096^3 NN {ceilings['hipblaslt_nn_TFLOPs']} / NT {ceilings['hipblaslt_nt_TFLOPs']} TFLOP/s")
     import helium_amd as ha
 
     ha.device.init(0)
@@ -1161,6 +1289,10 @@ def main():
                    "host_cores": os.cpu_count(), "untimed_launches_before_timing": max(SETTLE_LAUNCHES, args.warmup)},
         "roofline": rl,
         "cpu_baseline": cpu,
+        # measured on this box in this run, outside every timed region: what a plain copy kernel of the permutes' design
+        # reaches (the permute and pointwise figures are to be read against it, the published 8 TB/s is not reachable by
+        # any copy) and the vendor library's GEMM
+        "ceilings": dict(ceilings, copy_GBps=kernels["COPY"]["roofline"]["achieved"] if "COPY" in kernels else None),
         "kernels": kernels,
     }
     print(json.dumps(line), flush=True)

@@ -13,7 +13,7 @@ import itertools
 
 import numpy as np
 
-from . import ir
+from helium_amd import ir
 
 FLOATS = ("f32", "bf16", "f16")
 

@@ -4,15 +4,15 @@ The model (fused_graph.cpp: mi355x_cost) is linear in seven terms per plan (fusi
 every plan the four search objectives produce for a list of graphs, takes the terms through the C ABI
 (he_fusion_plan_cost_terms) and the time per execution from HIP events, and solves the non-negative least squares
 problem. It prints a table (what profiles/cost_model_fit.txt holds) and the initialiser for
-Mi355xCoefficients::fitted(). Needs a GPU:  python -m helium_amd.cost_fit [--steps K]
+Mi355xCoefficients::fitted(). Needs a GPU:  python -m harness.cost_fit [--steps K]
 """
 import argparse
 import time
 
 import numpy as np
 
-from . import configs, device, fusion, fusion_search as fs
-from .device import DeviceBuffer, Event, Stream
+from helium_amd import configs, device, fusion, fusion_search as fs
+from helium_amd.device import DeviceBuffer, Event, Stream
 
 ITEMSIZE = {"bf16": 2, "f16": 2, "f32": 4}
 

@@ -2,9 +2,9 @@
 kernel cache, so that a GPU run starts without JIT latency. Needs no GPU."""
 import time
 
-from . import configs
-from .kernels import TileKernel
-from .permute import PermuteDims
+from helium_amd import configs
+from helium_amd.kernels import TileKernel
+from helium_amd.permute import PermuteDims
 
 
 def prebuild_kernels(verbose=True):
@@ -23,8 +23,9 @@ def prebuild_kernels(verbose=True):
         TileKernel.fused(g)
         n += 1
     # the plans the benchmark runs through execute_graph
-    from . import frontend, ir
-    from .backend import Plan
+    from helium_amd import ir
+    from helium_amd.backend import Plan
+    from . import frontend
 
     Plan(configs.c1_ir_graph()[0]).precompile()
     g = ir.OpGraph()
@@ -75,7 +76,7 @@ def prebuild_kernels(verbose=True):
     Plan(g).precompile()
     n += 1
     # C5a and C4m the way the fusion search plans them
-    from . import fusion_search as fs
+    from helium_amd import fusion_search as fs
 
     g, outs = configs.c4_graph(4096, mainloop=True, full_size_outputs=True)
     for node in ("loss", "db8", "db6"):

@@ -3,7 +3,7 @@ from ._ffi import HeliumError, lib  # noqa: F401  (raises ImportError when the l
 from . import device  # noqa: F401
 from .device import DeviceBuffer, Event, Stream  # noqa: F401
 from .permute import PermuteDims  # noqa: F401
-from . import allocator, autodiff, backend, configs, fusion, fusion_search, ir, kernels  # noqa: F401
+from . import allocator, backend, configs, fusion, fusion_search, ir, kernels  # noqa: F401
 from .kernels import TileKernel  # noqa: F401
 
 __all__ = ["HeliumError", "device", "DeviceBuffer", "Event", "Stream", "PermuteDims", "TileKernel", "ir", "fusion", "kernels", "backend", "configs", "fusion_search"]

@@ -1,8 +1,7 @@
 """Builds libhelium_hip.so (the C-ABI backend library) in-tree with hipcc.
 
 The library's GPU kernels are generated at run time and compiled with hiprtc for gfx950, so this step builds
-host code only; `prebuild_kernels()` then generates and compiles the kernels of the benchmark configurations
-into the on-disk kernel cache, which works on a machine without a GPU.
+host code only.
 """
 import os
 import subprocess
@@ -59,8 +58,3 @@ def _wait(procs):
 
 if __name__ == "__main__":
     build()
-    if "--prebuild" in sys.argv:
-        sys.path.insert(0, os.path.dirname(HERE))
-        from helium_amd import prebuild
-
-        prebuild.prebuild_kernels(verbose=True)

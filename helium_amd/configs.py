@@ -22,6 +22,23 @@ PERMUTES = {
 }
 
 
+# The reference's own permute benchmark (helium/examples/permute_dim_benchmark.rs:13-41): f32 [2048,128,128,32],
+# swap_dims(0, 3): 4.3 GB in, 4.3 GB out - a size no cache flatters.
+PERM_REF_SHAPE, PERM_REF_PERM = (2048, 128, 128, 32), (3, 1, 2, 0)
+
+
+def perm_ref_expected(out_index):
+    """With input element i holding the 32-bit value i, the value at linear index `out_index` (uint64 array) of
+    swap_dims(0, 3) of a [2048,128,128,32] tensor: output coordinates (i3, i1, i2, i0) read input (i0, i1, i2, i3)."""
+    n0, n1, n2, n3 = PERM_REF_SHAPE
+    j = np.asarray(out_index, dtype=np.uint64)
+    i0 = j % n0
+    i2 = (j // n0) % n2
+    i1 = (j // (n0 * n2)) % n1
+    i3 = j // (n0 * n2 * n1)
+    return (((i0 * n1 + i1) * n2 + i2) * n3 + i3).astype(np.uint32)
+
+
 def permute_input(name, seed=None):
     shape, _ = PERMUTES[name]
     seed = {"C2a": 21, "C2b": 22, "C2c": 23}[name] if seed is None else seed

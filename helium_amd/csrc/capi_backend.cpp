@@ -122,7 +122,7 @@ int he_execute_graph(he_graph_t graph, const uint32_t* input_nodes, const he_ten
         std::shared_ptr<const he::exec::Prepared> prepared;
         {
             std::lock_guard<std::mutex> lk(graph->mu);
-            const unsigned options = he::plan::option_mask();
+            const uint64_t options = he::plan::option_mask();
             if (!graph->prepared || graph->prepared_nodes != graph->g->num_nodes() || graph->prepared_options != options) {
                 graph->prepared = he::exec::prepare(*graph->g);
                 graph->prepared_nodes = graph->g->num_nodes();

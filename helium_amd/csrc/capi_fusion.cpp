@@ -101,6 +101,17 @@ extern "C" {
 namespace {
 void fusion_search(he_fgraph_t graph, int objective, bool subdivided, he_fusion_plan_t* plan) {
     HE_REQUIRE(graph && plan && objective >= 0 && objective <= 3, HE_ERR_INVALID, "bad argument");
+    {
+        // he_fusion_plan_execute hands every value to one caller buffer: a value that two Consumers read is refused here,
+        // before anything is compiled or launched
+        std::set<OpNode> consumed;
+        for (OpNode n : graph->g.nodes()) {
+            const fir::Op& op = graph->g.get(n);
+            if (op.kind != fir::OpKind::Consumer) continue;
+            HE_REQUIRE(consumed.insert(op.a).second, HE_ERR_UNSUPPORTED, "value %llu is read by two Consumers: a plan writes each value to one buffer",
+                       (unsigned long long)op.a);
+        }
+    }
     auto p = std::make_unique<he_fusion_plan_s>();
     p->g = std::make_shared<fir::OpGraph>(graph->g);
     const auto params = fsearch::CostParams::mi355x();
@@ -208,6 +219,7 @@ int he_fusion_plan_execute(he_fusion_plan_t plan, const uint64_t* producer_nodes
             if (!buffers.count(key)) buffers[key] = it->second;
             else copies.push_back({it->second, buffers[key]});
         }
+        HE_REQUIRE(copies.empty(), HE_ERR_INTERNAL, "a value with two Consumers passed the check of he_fusion_search");
         exec::DevicePool& pool = exec::DevicePool::global();
         const uint64_t scope = pool.begin_scope();
         std::vector<exec::TensorRef> temporaries;
@@ -227,11 +239,6 @@ int he_fusion_plan_execute(he_fusion_plan_t plan, const uint64_t* producer_nodes
                 ptrs[a] = it->second;
             }
             fk.kernel->execute(ptrs.data(), s);
-        }
-        for (auto& c : copies) {
-            // sized by the value's element count and the Consumer's dtype (equal to the buffer's by the dtype rule)
-            (void)c;
-            fail(HE_ERR_UNSUPPORTED, "two Consumers of one value");
         }
         exec::EventRef done = pool.take_event();
         HE_HIP(hipEventRecord(done->e, s));

@@ -15,7 +15,7 @@ struct he_graph_s {
     std::mutex mu;
     std::shared_ptr<const he::exec::Prepared> prepared;
     size_t prepared_nodes = 0;
-    unsigned prepared_options = 0;
+    uint64_t prepared_options = 0;
 };
 struct he_fgraph_s {
     he::fir::OpGraph g;

@@ -83,37 +83,40 @@ __device__ __forceinline__ u32 ld_one(const u32* p) { return *p; }
 __device__ __forceinline__ float ld_one(const bf16_t* p) { return __builtin_bit_cast(float, (u32)(*(const u16*)p) << 16); }
 __device__ __forceinline__ float ld_one(const f16_t* p) { return (float)*p; }
 
-template <int NV> __device__ __forceinline__ void st_vec(float* p, const float (&e)[NV]) {
+// STREAM: the store bypasses the caches' write allocation (a large output that nobody reads back before it has left L2
+// anyway: with plain stores the 32 MB output of a 4096^2 product cost 5 us more, and up to 26 us when the launch had
+// streamed its operands through L2 just before)
+template <int NV, bool STREAM = false> __device__ __forceinline__ void st_vec(float* p, const float (&e)[NV]) {
     typedef typename Vec<float, NV>::type V;
     V v;
     if constexpr (NV == 1) v = e[0]; else
 #pragma unroll
     for (int k = 0; k < NV; k++) v[k] = e[k];
-    *(V*)p = v;
+    if constexpr (STREAM) __builtin_nontemporal_store(v, (V*)p); else *(V*)p = v;
 }
-template <int NV> __device__ __forceinline__ void st_vec(u32* p, const u32 (&e)[NV]) {
+template <int NV, bool STREAM = false> __device__ __forceinline__ void st_vec(u32* p, const u32 (&e)[NV]) {
     typedef typename Vec<u32, NV>::type V;
     V v;
     if constexpr (NV == 1) v = e[0]; else
 #pragma unroll
     for (int k = 0; k < NV; k++) v[k] = e[k];
-    *(V*)p = v;
+    if constexpr (STREAM) __builtin_nontemporal_store(v, (V*)p); else *(V*)p = v;
 }
-template <int NV> __device__ __forceinline__ void st_vec(bf16_t* p, const float (&e)[NV]) {
+template <int NV, bool STREAM = false> __device__ __forceinline__ void st_vec(bf16_t* p, const float (&e)[NV]) {
     typedef typename Vec<bf16_t, NV>::type V;
     V v;
     if constexpr (NV == 1) v = (bf16_t)e[0]; else
 #pragma unroll
     for (int k = 0; k < NV; k++) v[k] = (bf16_t)e[k];   // round to nearest even
-    *(V*)p = v;
+    if constexpr (STREAM) __builtin_nontemporal_store(v, (V*)p); else *(V*)p = v;
 }
-template <int NV> __device__ __forceinline__ void st_vec(f16_t* p, const float (&e)[NV]) {
+template <int NV, bool STREAM = false> __device__ __forceinline__ void st_vec(f16_t* p, const float (&e)[NV]) {
     typedef typename Vec<f16_t, NV>::type V;
     V v;
     if constexpr (NV == 1) v = (f16_t)e[0]; else
 #pragma unroll
     for (int k = 0; k < NV; k++) v[k] = (f16_t)e[k];
-    *(V*)p = v;
+    if constexpr (STREAM) __builtin_nontemporal_store(v, (V*)p); else *(V*)p = v;
 }
 __device__ __forceinline__ void st_one(float* p, float v) { *p = v; }
 __device__ __forceinline__ void st_one(u32* p, u32 v) { *p = v; }
@@ -282,6 +285,11 @@ static void emit_generic_map(std::ostringstream& s, const GenericMap& g) {
         }
         s << " lin = in_index; }";
     }
+}
+
+bool streams_out(const Arg& a) {
+    if (tuning::get("HELIUM_HIP_NO_STREAM_STORES")) return false;
+    return a.is_output && storage_bytes(a.dtype, (size_t)a.numel) >= (size_t(4) << 20);
 }
 
 int pick_nv(const Program& p, int max_bytes) {
@@ -718,7 +726,7 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
                 s << "#pragma unroll\nfor (int k = 0; k < NV; k++) { const size_t l = o + k; if (" << v
                   << "[k]) atomicOr(a" << o.arg << " + (l >> 5), 1u << (l & 31)); }\n";
             } else {
-                s << "st_vec<NV>(a" << o.arg << " + o, " << v << ");\n";
+                s << "st_vec<NV, " << (streams_out(p.args[o.arg]) ? "true" : "false") << ">(a" << o.arg << " + o, " << v << ");\n";
             }
             s << "}\n";
             continue;

@@ -100,7 +100,7 @@ double analytical_cost(const FusedGraph& fg);                   // cost_model.rs
 
 // A cost model of the same purpose as the analytical one, for this backend's kernels on MI355X: the time of a plan
 // is a sum over its kernels, linear in seven terms whose coefficients are fitted to measured kernels
-// (helium_amd/cost_fit.py measures and fits; profiles/cost_model_fit.txt holds the data). The terms say what the
+// (harness/cost_fit.py measures and fits; profiles/cost_model_fit.txt holds the data). The terms say what the
 // hardware bounds: matrix-core work, the bytes a kernel moves to and from HBM, the vector work of epilogue / anchor-less
 // kernels, and - what makes a mainloop fusion lose on this chip - the operand traffic from L2 to the CUs, which every
 // tile column (for A) or tile row (for B) of a product repeats: a fused `relu(A0) * T` makes 16 workgroups per tile row

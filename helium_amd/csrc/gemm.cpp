@@ -138,11 +138,13 @@ typedef float mul_t;   /* multiplicand as stored in global memory */
 typedef bf16_t mul_t;  /* any two-byte multiplicand: only the element size matters to the address arithmetic */
 #endif
 
-// Operand fragments of k-step kk from one LDS stage (its A tile at `la`, its B tile at `lb`). Both are __restrict__ on purpose: after inlining, every LDS
+// Operand fragments of k-step kk from one LDS stage. `st` is __restrict__ on purpose: after inlining, every LDS
 // read carries alias-scope information that separates it from the direct global->LDS writes into the *other*
 // stage, so the compiler does not make the reads wait for those writes (vmcnt) before the MFMAs can start.
-__device__ __forceinline__ void load_frags(const unsigned char* __restrict__ la, const unsigned char* __restrict__ lb, int kk,
-                                           const WavePos& w, afrag_t (&af)[MB], bfrag_t (&bf)[NB]) {
+__device__ __forceinline__ void load_frags(const unsigned char* __restrict__ st, int kk, const WavePos& w,
+                                           afrag_t (&af)[MB], bfrag_t (&bf)[NB]) {
+    const unsigned char* la = st;
+    const unsigned char* lb = st + A_TILE_BYTES;
     const u32 lane = w.lane;
 #if MMA_F32
     // v_mfma_f32_32x32x2_f32: lane l supplies A[l % 32][l / 32] and B[l / 32][l % 32]. One k-step covers 8 k: each
@@ -169,10 +171,7 @@ __device__ __forceinline__ void load_frags(const unsigned char* __restrict__ la,
     }
 #else
     const u32 grp = lane >> 4, sub = lane & 15;
-#if GEMM_SKIP & 8
-#pragma unroll
-    for (int i = 0; i < MB; i++) af[i] = __builtin_bit_cast(afrag_t, u32x4{lane, lane, lane, lane});
-#elif A_KM
+#if A_KM
 #pragma unroll
     for (int i = 0; i < MB; i++) {
         const u32 k = kk * 16 + (grp >> 1) * 8 + (sub >> 2);
@@ -188,11 +187,7 @@ __device__ __forceinline__ void load_frags(const unsigned char* __restrict__ la,
         af[i] = *(const s16x8*)(la + a_off(row, kk * 2 + (lane >> 5)));
     }
 #endif
-#if GEMM_SKIP & 16
-    (void)grp; (void)sub;
-#pragma unroll
-    for (int j = 0; j < NB; j++) bf[j] = __builtin_bit_cast(bfrag_t, u32x4{lane, lane, lane, lane});
-#elif B_NK
+#if B_NK
     (void)grp; (void)sub;
 #pragma unroll
     for (int j = 0; j < NB; j++) {
@@ -253,11 +248,11 @@ __device__ __forceinline__ void mma_or_skip(f32x16 (&acc)[MB][NB], const afrag_t
 // fragment reads have been issued, so the LDS latency that follows the workgroup barrier hides behind them; this
 // tile's own last step is left in `fr` for the next call (or for finish_tiles after the last tile).
 template <class PerStep>
-__device__ __forceinline__ void compute_tile(const unsigned char* __restrict__ la, const unsigned char* __restrict__ lb,
-                                             f32x16 (&acc)[MB][NB], const WavePos& w, Frags& fr, PerStep&& per_step) {
+__device__ __forceinline__ void compute_tile(const unsigned char* __restrict__ st, f32x16 (&acc)[MB][NB], const WavePos& w,
+                                             Frags& fr, PerStep&& per_step) {
     static_assert(KK % 2 == 0, "the fragment double buffer assumes an even number of k-steps per tile");
 #if !(GEMM_SKIP & 2)
-    load_frags(la, lb, 0, w, fr.a[0], fr.b[0]);
+    load_frags(st, 0, w, fr.a[0], fr.b[0]);
 #endif
     // A slice (or all) of the next tile's global->LDS traffic. Issuing a direct load takes tens of cycles; the MFMAs
     // of the previous tile's step KK-1 (zero fragments before the first tile) need nothing from memory and are
@@ -271,7 +266,7 @@ __device__ __forceinline__ void compute_tile(const unsigned char* __restrict__ l
         for (int i = 0; i < MB; i++) fr.a[(kk + 1) & 1][i] = fr.a[kk & 1][i];
         for (int j = 0; j < NB; j++) fr.b[(kk + 1) & 1][j] = fr.b[kk & 1][j];
 #else
-        load_frags(la, lb, kk + 1, w, fr.a[(kk + 1) & 1], fr.b[(kk + 1) & 1]);
+        load_frags(st, kk + 1, w, fr.a[(kk + 1) & 1], fr.b[(kk + 1) & 1]);
 #endif
         mma_or_skip(acc, fr.a[kk & 1], fr.b[kk & 1]);
         SCHED_HINT
@@ -290,32 +285,21 @@ __device__ __forceinline__ void finish_tiles(f32x16 (&acc)[MB][NB], const Frags&
 // Operand tiles go from global memory straight into LDS (global_load_lds_dwordx4): a wave instruction fills
 // 1 KB of LDS in lane order, so each lane fetches the global chunk whose swizzled LDS slot is lane * 16.
 // `ga` / `gb` point at the tile's first A row / first B k-row (at this workgroup's columns).
-// LWAVES waves issue the direct loads, the youngest ones of the workgroup. With all of them loading (LWAVES == NWAVES)
-// every wave interleaves its share with its own MFMAs. With half of them (eight-wave tiles), the SIMD's older wave -
-// which the MFMA arbiter serves first - never touches the address path: a direct load occupies it for some 16 clocks,
-// a wave that finds it busy stalls at the load with its MFMAs queued behind, and 64 loads per tile keep it busy for
-// half a tile's time. The younger wave of each SIMD has no MFMA to issue in that half anyway, so it stalls for free.
-#define LOADER_FIRST (NWAVES - LWAVES)
-#define IS_LOADER(wave) (LWAVES == NWAVES || (wave) >= LOADER_FIRST)
-#define A_DPW (DIRECT_A ? A_TILE_BYTES / 1024 / LWAVES : 0)  /* direct-load instructions per loading wave and tile */
-// The address of a lane's chunk as (pointer that is the same for the whole wave) + (32-bit offset of the lane, in
-// multiplicands): where the wave's part is provably uniform the load takes it from scalar registers and keeps one
-// offset register per lane instead of a 64-bit address per load, and the k-loop advances scalars only.
-#define LANE_ADDR(uniform_ptr, lane_elems) ((const mul_t*)((const char*)(uniform_ptr) + (u32)((lane_elems) * ESZ)))
-#define B_DPW (DIRECT_B ? B_TILE_BYTES / 1024 / LWAVES : 0)
-__device__ __forceinline__ void direct_issue(unsigned char* __restrict__ sa, unsigned char* __restrict__ sb, const mul_t* __restrict__ ga,
+#define A_DPW (DIRECT_A ? A_TILE_BYTES / 1024 / NWAVES : 0)  /* direct-load instructions per wave and tile */
+#define B_DPW (DIRECT_B ? B_TILE_BYTES / 1024 / NWAVES : 0)
+__device__ __forceinline__ void direct_issue(unsigned char* __restrict__ st, const mul_t* __restrict__ ga,
                                              const mul_t* __restrict__ gb, const WavePos& w, int i) {
 #if GEMM_SKIP & 1
     return;
 #endif
-    const u32 lane = w.lane, wave = w.wave - LOADER_FIRST;
+    const u32 lane = w.lane, wave = w.wave;
     if (i < A_DPW) {
         const u32 blk = wave * A_DPW + i;
 #if A_KM
         const u32 krow = blk * (64 / AKM_CHUNKS) + lane / AKM_CHUNKS, pcm = lane % AKM_CHUNKS;
         const u32 mc = pcm ^ AKM_SWZ(krow);
-        const mul_t* gpm = LANE_ADDR(ga + (size_t)(blk * (64 / AKM_CHUNKS)) * GM, (lane / AKM_CHUNKS) * GM + mc * EPC);
-        __builtin_amdgcn_global_load_lds((GLOBAL_AS const void*)gpm, (LDS_AS void*)(sa + blk * 1024), 16, 0, 0);
+        const mul_t* gpm = ga + (size_t)krow * GM + mc * EPC;
+        __builtin_amdgcn_global_load_lds((GLOBAL_AS const void*)gpm, (LDS_AS void*)(st + blk * 1024), 16, 0, 0);
         return;
 #endif
         const u32 row = blk * (64 / A_CHUNKS) + lane / A_CHUNKS, pc = lane % A_CHUNKS;
@@ -334,15 +318,15 @@ __device__ __forceinline__ void direct_issue(unsigned char* __restrict__ sa, uns
         const bool inside = conv_tap(w.m0 + row, (u32)(ga - (const mul_t*)nullptr) + kc * EPC, at);
         const mul_t* gp = inside ? (const mul_t*)w.img + at : (const mul_t*)conv_zeros;
 #else
-        const mul_t* gp = LANE_ADDR(ga + (size_t)(blk * (64 / A_CHUNKS)) * GK, (lane / A_CHUNKS) * GK + kc * EPC);
+        const mul_t* gp = ga + (size_t)row * GK + kc * EPC;
 #endif
-        __builtin_amdgcn_global_load_lds((GLOBAL_AS const void*)gp, (LDS_AS void*)(sa + blk * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((GLOBAL_AS const void*)gp, (LDS_AS void*)(st + blk * 1024), 16, 0, 0);
     } else {
         const u32 blk = wave * B_DPW + (i - A_DPW);
 #if B_NK
         const u32 row = blk * (64 / A_CHUNKS) + lane / A_CHUNKS, pc = lane % A_CHUNKS;
         const u32 kc = pc ^ ((row >> A_SWZ_SHIFT) & (A_CHUNKS - 1));
-        const mul_t* gp = LANE_ADDR(gb + (size_t)(blk * (64 / A_CHUNKS)) * GK, (lane / A_CHUNKS) * GK + kc * EPC);
+        const mul_t* gp = gb + (size_t)row * GK + kc * EPC;
 #else
         const u32 krow = blk * (64 / B_CHUNKS) + lane / B_CHUNKS, pc = lane % B_CHUNKS;
         const u32 nc = pc ^ B_SWZ(krow);
@@ -356,21 +340,21 @@ __device__ __forceinline__ void direct_issue(unsigned char* __restrict__ sa, uns
         // `gb` carries the tile's first k as an element offset from null; row k of B starts at b_row_addr(k)
         const mul_t* gp = (const mul_t*)w.bsrc + b_row_addr((u32)(gb - (const mul_t*)nullptr) + krow) + w.n0 + nc * EPC;
 #else
-        const mul_t* gp = LANE_ADDR(gb + (size_t)(blk * (64 / B_CHUNKS)) * GN, (lane / B_CHUNKS) * GN + nc * EPC);
+        const mul_t* gp = gb + (size_t)krow * GN + nc * EPC;
 #endif
 #endif
-        __builtin_amdgcn_global_load_lds((GLOBAL_AS const void*)gp, (LDS_AS void*)(sb + blk * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((GLOBAL_AS const void*)gp, (LDS_AS void*)(st + A_TILE_BYTES + blk * 1024), 16, 0, 0);
     }
 }
 // Multiplies the tile in stage `rd` while requesting the tile that goes into stage `wr`.
 __device__ __forceinline__ void direct_tile(const unsigned char* __restrict__ rd, unsigned char* __restrict__ wr,
                                             const mul_t* __restrict__ ga, const mul_t* __restrict__ gb, bool more,
                                             f32x16 (&acc)[MB][NB], const WavePos& w, Frags& fr) {
-    compute_tile(rd, rd + A_TILE_BYTES, acc, w, fr, [&](int kk) {
+    compute_tile(rd, acc, w, fr, [&](int kk) {
         constexpr int per = ISSUE_FRONT ? (A_DPW + B_DPW) : (A_DPW + B_DPW + KK - 1) / KK;
-        if (more && IS_LOADER(w.wave)) {
+        if (more) {
 #pragma unroll
-            for (int i = kk * per; i < (kk + 1) * per && i < A_DPW + B_DPW; i++) direct_issue(wr, wr + A_TILE_BYTES, ga, gb, w, i);
+            for (int i = kk * per; i < (kk + 1) * per && i < A_DPW + B_DPW; i++) direct_issue(wr, ga, gb, w, i);
         }
     });
 }
@@ -383,18 +367,8 @@ __device__ __forceinline__ void direct_tile(const unsigned char* __restrict__ rd
 #endif
 extern "C" __global__ __launch_bounds__(NTHREADS) KERNEL_ATTRS
 void fused_matmul(KERNEL_PARAMS) {
-#if RING5
-    __shared__ __attribute__((aligned(16))) unsigned char lds[5 * A_TILE_BYTES];
-#else
     __shared__ __attribute__((aligned(16))) unsigned char lds[NSTAGES * STAGE_BYTES];
-#endif
-#if PINGPONG || LWAVES != NWAVES
-    // (the wave's index as a scalar: the two groups of waves branch on it, and the loads' addresses split into a
-    // scalar part per wave and an offset per lane)
-    const u32 tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-#else
     const u32 tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-#endif
     const u32 wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
     u32 tile_m, tile_n;
     TILE_ORDER
@@ -519,7 +493,7 @@ void fused_matmul(KERNEL_PARAMS) {
 #if CONV_A_FAST
     WavePos wpos = {lane, wave, wave_m, wave_n, m0, n0, (const void*)CONV_IMG_OR_NULL, (const void*)B_SRC_OR_NULL, {}, {}, {}};
 #pragma unroll
-    for (int i = 0; i < A_DPW_MAX; i++) conv_row_terms(m0 + ((wave - LOADER_FIRST) * A_DPW_MAX + i) * (64 / A_CHUNKS) + lane / A_CHUNKS, wpos.cbase[i], wpos.ch0[i], wpos.cw0[i]);
+    for (int i = 0; i < A_DPW_MAX; i++) conv_row_terms(m0 + (wave * A_DPW_MAX + i) * (64 / A_CHUNKS) + lane / A_CHUNKS, wpos.cbase[i], wpos.ch0[i], wpos.cw0[i]);
 #else
     const WavePos wpos = {lane, wave, wave_m, wave_n, m0, n0, (const void*)CONV_IMG_OR_NULL, (const void*)B_SRC_OR_NULL};
 #endif
@@ -551,154 +525,12 @@ void fused_matmul(KERNEL_PARAMS) {
     // wave only ever waits for loads issued NSTAGES - 2 tiles earlier.
 #pragma unroll
     for (int st = 0; st < NSTAGES - 1; st++)
-        if (st < KT && IS_LOADER(wave)) {
+        if (st < KT) {
 #pragma unroll
             for (int i = 0; i < A_DPW + B_DPW; i++)
-                direct_issue(lds + st * STAGE_BYTES, lds + st * STAGE_BYTES + A_TILE_BYTES, A_TILE_AT(k_tile(st) * BK), B_TILE_AT(k_tile(st) * BK), wpos, i);
+                direct_issue(lds + st * STAGE_BYTES, A_TILE_AT(k_tile(st) * BK), B_TILE_AT(k_tile(st) * BK), wpos, i);
         }
 #endif
-#if RING5
-    // A ring of five slots of one operand tile each (A and B tiles are the same size here), filled in the order A0 B0 A1
-    // B1 A2 ...: part p lives in slot p % 5. While tile t is multiplied out of slots 2t and 2t + 1, the slots of tile
-    // t - 1 are refilled with B of tile t + 1 and A of tile t + 2, so an A tile has two tiles' time to land and a B
-    // tile one; the B loads are asked for first, the A loads dealt out over the rest of the tile's MFMAs, where
-    // nobody waits for them. (Two stages of A + B ask for 64 KB at the head of every tile and need all of it at its end.)
-#define PART(p) (lds + ((p) % 5u) * A_TILE_BYTES)
-    if (IS_LOADER(wave)) {
-        if (KT > 0) {
-#pragma unroll
-            for (int i = 0; i < A_DPW; i++) direct_issue(PART(0u), PART(1u), A_TILE_AT(k_tile(0) * BK), B_TILE_AT(0), wpos, i);
-#pragma unroll
-            for (int i = A_DPW; i < A_DPW + B_DPW; i++) direct_issue(PART(0u), PART(1u), A_TILE_AT(0), B_TILE_AT(k_tile(0) * BK), wpos, i);
-        }
-        if (KT > 1) {
-#pragma unroll
-            for (int i = 0; i < A_DPW; i++) direct_issue(PART(2u), PART(3u), A_TILE_AT(k_tile(1) * BK), B_TILE_AT(0), wpos, i);
-        }
-    }
-    Frags frags;
-    init_frags(frags);
-    for (u32 kt = 0; kt < KT; kt++) {
-        // A and B of tile kt have landed when at most the youngest A tile (of tile kt + 1, if there is one) is in flight
-        if (kt + 1 < KT) __builtin_amdgcn_s_waitcnt(0x0070 | WAITCNT_VM(A_DPW));
-        else __builtin_amdgcn_s_waitcnt(0x0070);
-        __builtin_amdgcn_s_barrier();
-        const bool more_b = kt + 1 < KT, more_a = kt + 2 < KT;
-        const u32 kb = more_b ? k_tile(kt + 1) * BK : 0u, ka = more_a ? k_tile(kt + 2) * BK : 0u;
-        compute_tile(PART(2u * kt), PART(2u * kt + 1u), acc, wpos, frags, [&](int kk) {
-            if (kk == 0 && IS_LOADER(wpos.wave)) {
-                if (more_b) {
-#pragma unroll
-                    for (int i = A_DPW; i < A_DPW + B_DPW; i++) direct_issue(PART(0u), PART(2u * kt + 3u), A_TILE_AT(0), B_TILE_AT(kb), wpos, i);
-                }
-                if (more_a) {
-#pragma unroll
-                    for (int i = 0; i < A_DPW; i++) direct_issue(PART(2u * kt + 4u), PART(0u), A_TILE_AT(ka), B_TILE_AT(0), wpos, i);
-                }
-            }
-        });
-        __builtin_amdgcn_sched_barrier(0);
-    }
-    finish_tiles(acc, frags);
-    __syncthreads();
-#elif PINGPONG
-    // Two groups of four waves (one wave of each group per SIMD) run half a phase pair apart: while one group reads
-    // its fragments of a whole k-tile from LDS into registers (memory phase), the other multiplies out of registers
-    // (compute phase), then they swap. Every phase ends in a workgroup barrier; the late group takes one extra barrier
-    // up front, the early group one at the end, so the counts agree. Phases are numbered from 0: the early group
-    // reads tile t in phase 2t and multiplies it in phase 2t + 1, the late group reads it in phase 2t + 1 and
-    // multiplies it in phase 2t + 2. The slot of tile t is free when phase 2t + 1 has ended. Each group requests its
-    // share of a later tile during its compute phases (see there), and at the end of every odd phase 2v + 1 everybody
-    // has seen its own loads of tile v + 1 arrive (vmcnt: at most the NSTAGES - 2 younger tiles still in flight) - the
-    // barrier that follows precedes that tile's first reader. A tile's loads have 2 * NSTAGES - 4 whole phases to land.
-    {
-    const bool late = __builtin_amdgcn_readfirstlane(wave) >= NWAVES / 2;
-    afrag_t pa[KK][MB];
-    bfrag_t pb[KK][NB];
-    auto issue_tile = [&](u32 t) {
-        const u32 k0 = k_tile(t) * BK;
-#pragma unroll
-        for (int i = 0; i < A_DPW + B_DPW; i++) direct_issue(lds + (t % NSTAGES) * STAGE_BYTES, lds + (t % NSTAGES) * STAGE_BYTES + A_TILE_BYTES, A_TILE_AT(k0), B_TILE_AT(k0), wpos, i);
-    };
-#define PP_BARRIER() do { __builtin_amdgcn_sched_barrier(0); __builtin_amdgcn_s_barrier(); __builtin_amdgcn_sched_barrier(0); } while (0)
-#define PP_WAIT_LDS 0xC07F                                                   /* lgkmcnt(0), any number of loads in flight */
-#define PP_WAIT_LOADS(n) (0x0F70 | WAITCNT_VM((n) * (A_DPW + B_DPW)))        /* at most n tiles of this wave's loads in flight */
-#define PP_WAIT_BOTH(n) (0x0070 | WAITCNT_VM((n) * (A_DPW + B_DPW)))
-    // tile v + 1 has landed when at most the NSTAGES - 2 younger tiles are in flight (near the end: everything)
-#define PP_CONFIRM(v, WAIT) do { if ((v) + NSTAGES - 1 < KT) __builtin_amdgcn_s_waitcnt(WAIT(NSTAGES - 2)); else __builtin_amdgcn_s_waitcnt(WAIT(0)); } while (0)
-#pragma unroll
-    for (u32 t = 0; t < NSTAGES - 1; t++)
-        if (t < KT) issue_tile(t);
-    if (NSTAGES - 1 <= KT) __builtin_amdgcn_s_waitcnt(PP_WAIT_LOADS(NSTAGES - 2));
-    else __builtin_amdgcn_s_waitcnt(PP_WAIT_LOADS(0));
-    PP_BARRIER();
-    if (late) {  // phase 0 of the late group: nothing to multiply yet
-        if (NSTAGES - 1 < KT) issue_tile(NSTAGES - 1);
-        PP_BARRIER();
-    }
-    for (u32 kt = 0; kt < KT; kt++) {
-        // ---- memory phase (early group: phase 2 kt, late group: phase 2 kt + 1): fragment reads only
-        const unsigned char* rd = lds + (kt % NSTAGES) * STAGE_BYTES;
-#pragma unroll
-        for (int kk = 0; kk < KK; kk++) {
-#if !(GEMM_SKIP & 2)
-            load_frags(rd, rd + A_TILE_BYTES, kk, wpos, pa[kk], pb[kk]);
-#endif
-        }
-        if (late) PP_CONFIRM(kt, PP_WAIT_BOTH);
-        else __builtin_amdgcn_s_waitcnt(PP_WAIT_LDS);
-        PP_BARRIER();
-        // ---- compute phase (early group: phase 2 kt + 1, late group: phase 2 kt + 2). The wave's loads of one
-        // tile are dealt out evenly between its MFMAs: a direct load occupies the CU's one address path for some 16
-        // clocks, and a wave that finds it busy stalls at the load, MFMAs behind it included, so the four waves of
-        // the group ask for one load each per quarter of the phase instead of eight waves asking for everything at
-        // once. The early group fills the slot of tile kt - 1 (the late group still reads tile kt's), the late
-        // group the slot of tile kt.
-        const u32 fill = late ? kt + NSTAGES : kt + NSTAGES - 1;
-        const bool more = fill < KT;
-        const u32 kf = more ? k_tile(fill) * BK : 0u;
-        unsigned char* wr = lds + (fill % NSTAGES) * STAGE_BYTES;
-        __builtin_amdgcn_s_setprio(PP_PRIO);
-        {
-            constexpr int NM = KK * MB * NB, NL = A_DPW + B_DPW;
-#pragma unroll
-            for (int q = 0; q < NM; q++) {
-                // load l goes in front of MFMA number l * NM / NL
-#pragma unroll
-                for (int l = 0; l < NL; l++)
-                    if (q == (l * NM) / NL) {
-                        __builtin_amdgcn_sched_barrier(0);
-                        if (more) direct_issue(wr, wr + A_TILE_BYTES, A_TILE_AT(kf), B_TILE_AT(kf), wpos, l);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                const int kk = q / (MB * NB), i = (q / NB) % MB, j = q % NB;
-#if !(GEMM_SKIP & 4)
-#if MMA_F32
-#pragma unroll
-                for (int e = 0; e < 4; e++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(pa[kk][i][e], pb[kk][j][e], acc[i][j], 0, 0, 0);
-#elif MMA_BF16
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, pa[kk][i]), __builtin_bit_cast(bf16x8, pb[kk][j]), acc[i][j], 0, 0, 0);
-#else
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, pa[kk][i]), __builtin_bit_cast(f16x8, pb[kk][j]), acc[i][j], 0, 0, 0);
-#endif
-#else
-                if (q == 0) acc[0][0][0] += (float)pa[0][0][0] + (float)pb[0][0][0];
-#endif
-            }
-        }
-        __builtin_amdgcn_s_setprio(0);
-        if (!late) PP_CONFIRM(kt, PP_WAIT_LOADS);
-        PP_BARRIER();
-    }
-    }
-    // The early group is one phase ahead: it either waits here for the late group's last products, or (PP_EPI_OVERLAP)
-    // runs its epilogue strips meanwhile - every LDS read of the mainloop is over, the strips are private to a wave -
-    // and takes the barrier that evens out the count after them, so the two groups' epilogue traffic is spread out.
-    const bool late_group = __builtin_amdgcn_readfirstlane(wave) >= NWAVES / 2;
-#if !PP_EPI_OVERLAP
-    if (!late_group) PP_BARRIER();
-#endif
-#else
 #if STAGED
     stage_load(0);
     stage_store(0, 0);
@@ -736,7 +568,7 @@ void fused_matmul(KERNEL_PARAMS) {
         direct_tile(lds + (kt % NSTAGES) * STAGE_BYTES, lds + (next % NSTAGES) * STAGE_BYTES, A_TILE_AT(knext),
                     B_TILE_AT(knext), more, acc, wpos, frags);
 #else
-        compute_tile(lds + (kt % NSTAGES) * STAGE_BYTES, lds + (kt % NSTAGES) * STAGE_BYTES + A_TILE_BYTES, acc, wpos, frags, [](int) {});
+        compute_tile(lds + (kt % NSTAGES) * STAGE_BYTES, acc, wpos, frags, [](int) {});
 #endif
 #if STAGED
         STAGE_SCHED_BARRIER
@@ -746,7 +578,6 @@ void fused_matmul(KERNEL_PARAMS) {
     }
     finish_tiles(acc, frags);
     __syncthreads();
-#endif
 
     // ---- epilogue: accumulators -> wave-private LDS strip -> row-major NV-wide vectors -----------------------
     float* strip = (float*)lds + wave * (32 * EP);
@@ -781,9 +612,6 @@ void fused_matmul(KERNEL_PARAMS) {
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
-#if !RING5 && PINGPONG && PP_EPI_OVERLAP
-    if (!late_group) PP_BARRIER();
-#endif
     EPILOGUE_FINISH
 }
 )HIP";
@@ -1101,21 +929,6 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     const bool conv_a_fast = pr.conv_a.on && direct_a && pr.conv_a.C % t.bk == 0 && (t.bm * t.bk * esz / 1024) % (threads / 64) == 0 &&
                              (int64_t)pr.conv_a.N * pr.conv_a.H * pr.conv_a.W * pr.conv_a.C < (int64_t(1) << 32) &&
                              !tuning::get("HELIUM_HIP_GEMM_NO_CONV_FAST");
-    // Eight-wave tiles on direct loads: the younger wave of each SIMD issues all of them (see LWAVES in the template)
-    int loaders = threads / 64;
-    if (direct_a && direct_b && threads == 512 && !pr.conv_a.on && !pr.conv_b.on && (tuning::get_int("HELIUM_HIP_GEMM_LOADERS", 8) == 4 || tuning::get_int("HELIUM_HIP_GEMM_HALF_LOADERS", 0)) &&
-        (t.bm * t.bk * esz / 1024) % 4 == 0 && (t.bk * t.bn * esz / 1024) % 4 == 0)
-        loaders = 4;
-    if (tuning::get("HELIUM_HIP_GEMM_PINGPONG") && atoi(tuning::get("HELIUM_HIP_GEMM_PINGPONG")) != 0) loaders = threads / 64;  // (its loop deals loads to every wave)
-    // Eight waves whose operands both arrive by direct loads run as two groups half a k-tile apart (the template's
-    // PINGPONG loop); its LDS ring has two stages.
-    const bool pingpong = direct_a && direct_b && threads == 512 && pr.split_k == 1 && t.bk / (2 * epc) >= 1 &&
-                          (tuning::get("HELIUM_HIP_GEMM_PINGPONG") ? atoi(tuning::get("HELIUM_HIP_GEMM_PINGPONG")) != 0 : false);
-    if (pingpong) t.stages = std::min(4, std::max(2, tuning::get_int("HELIUM_HIP_GEMM_PP_STAGES", t.bk == 32 ? 4 : 2)));
-    // Square 256x256 tiles on direct loads keep a ring of five operand tiles instead of two stages (RING5 in the template)
-    const bool ring5 = direct_a && direct_b && !pingpong && t.bm == t.bn && 5 * t.bm * t.bk * esz <= 160 * 1024 && pr.split_k == 1 &&
-                       !fold_in_kernel && !pr.conv_a.on && !pr.conv_b.on && tuning::get_int("HELIUM_HIP_GEMM_RING5", 0) != 0;
-    if (ring5) t.stages = 2;
     if (!(direct_a && direct_b)) t.stages = 2;  // register staging is double-buffered only
     else if (!tuning::get("HELIUM_HIP_GEMM_TILE") && small) {
         // A grid that leaves CUs idle is bound by the latency of its k-loop: keep as many tiles in flight as LDS holds.
@@ -1153,13 +966,11 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
       << "\n#define WAVES_N " << t.wn << wgs_per_cu_attr << "\n#define NSTAGES " << t.stages << "\n#define NVE " << nve << "\n#define MMA_BF16 " << (pr.mma_dtype == HE_BF16 ? 1 : 0) << "\n#define MMA_F32 " << (f32 ? 1 : 0)
       << "\n#define STAGGER_EXPR " << (tuning::measuring() && tuning::get("HELIUM_HIP_GEMM_STAGGER") ? tuning::get("HELIUM_HIP_GEMM_STAGGER") : "0u")
       << "\n#define ISSUE_FRONT " << (issue_front ? 1 : 0)
-      << "\n#define RING5 " << (ring5 ? 1 : 0) << "\n#define LWAVES " << loaders << "\n#define PINGPONG " << (pingpong ? 1 : 0) << "\n#define PP_ORDER " << tuning::get_int("HELIUM_HIP_GEMM_PP_ORDER", 1)
-      << "\n#define PP_PRIO " << tuning::get_int("HELIUM_HIP_GEMM_PP_PRIO", 1) << "\n#define PP_EPI_OVERLAP " << tuning::get_int("HELIUM_HIP_GEMM_PP_EPI", 1)
       // measurement only (HELIUM_HIP_TUNING=measure): bit 0 drops the direct loads, bit 1 the fragment reads, bit 2 the
       // MFMAs - the kernel's results are then wrong, its timing tells what the rest costs
       << "\n#define GEMM_SKIP " << (tuning::measuring() ? tuning::get_int("HELIUM_HIP_GEMM_SKIP", 0) : 0)
       << "\n#define DIRECT_A " << (direct_a ? 1 : 0) << "\n#define DIRECT_B " << (direct_b ? 1 : 0)
-      << "\n#define CONV_A_FAST " << (conv_a_fast ? 1 : 0) << "\n#define A_DPW_MAX " << std::max(1, t.bm * t.bk * esz / 1024 / loaders)
+      << "\n#define CONV_A_FAST " << (conv_a_fast ? 1 : 0) << "\n#define A_DPW_MAX " << std::max(1, t.bm * t.bk * esz / 1024 / (threads / 64))
       << "\n#define A_KM " << (pr.a_km ? 1 : 0) << "\n#define B_NK " << (pr.b_nk ? 1 : 0) << "\n#define CONV_A " << (pr.conv_a.on ? 1 : 0) << "\n#define CONV_IMG p" << (pr.conv_a.on ? pr.map_a[0] : 0)
       << "\n#define CONV_IMG_OR_NULL " << (pr.conv_a.on ? "p" + std::to_string(pr.map_a[0]) : std::string("nullptr"))
       << "\n#define B_ROW_GATHER " << (pr.b_rows.on ? 1 : 0) << "\n#define CONV_B " << (pr.conv_b.on ? 1 : 0) << "\n#define SPLIT_K " << pr.split_k
@@ -1394,10 +1205,10 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
                     if (pr.out_rows.on) {
                         const auto& orow = pr.out_rows;
                         b << "{ const u32 on_ = m / " << orow.P * orow.Q << "u, opq = m % " << orow.P * orow.Q << "u, op_ = opq / " << orow.Q << "u, oq = opq % " << orow.Q
-                          << "u;\nst_vec<NVE>(a" << o.arg << " + (((size_t)on_ * " << orow.H << "u + op_ * " << orow.sh << "u + " << orow.a << "u) * " << orow.W << "u + oq * "
+                          << "u;\nst_vec<NVE, " << (tp::streams_out(pr.epi.args[o.arg]) ? "true" : "false") << ">(a" << o.arg << " + (((size_t)on_ * " << orow.H << "u + op_ * " << orow.sh << "u + " << orow.a << "u) * " << orow.W << "u + oq * "
                           << orow.sw << "u + " << orow.b << "u) * GN + nn, " << v << "); }\n";
                     } else
-                    b << "st_vec<NVE>(a" << o.arg << " + ((size_t)bz * GM + m) * GN + nn, " << v << ");\n";
+                    b << "st_vec<NVE, " << (tp::streams_out(pr.epi.args[o.arg]) ? "true" : "false") << ">(a" << o.arg << " + ((size_t)bz * GM + m) * GN + nn, " << v << ");\n";
                 } else if (o.fold_m && !o.fold_n) {
                     b << "#pragma unroll\nfor (int k = 0; k < NVE; k++) rc" << oi << "[step % " << colsets << "][k] += " << v << "[k];\n";
                 } else if (o.fold_m && o.fold_n) {
@@ -1558,45 +1369,29 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
             // per k-step the next step's reads between the first MFMAs (two per MFMA in mode 3, all before the
             // second MFMA in mode 4) so that they have landed when the step ends: while direct loads are in flight
             // the compiler can only wait for *all* outstanding LDS reads at once.
-            const int waves = loaders;
+            const int waves = threads / 64;
             const int dl = ((direct_a ? t.bm * t.bk * esz / 1024 : 0) + (direct_b ? t.bk * t.bn * esz / 1024 : 0)) / waves;
             const int per = issue_front ? dl : (dl + kk_steps - 1) / kk_steps;
             const int rate = mode == 3 ? 2 : nr;
-            // With all loads issued at the head of the tile (issue_front), they are dealt out over the first `spread`
-            // MFMAs: a direct load holds the CU's address path for some 16 clocks and the eight waves ask at the same
-            // time, so a wave gets a load accepted every 128 clocks or so; with one MFMA between two loads the matrix
-            // pipe is half idle for the 1000 clocks that 64 loads take, with two it stays full - and the last load
-            // still has half the tile's time to land.
-            const int spread = issue_front ? std::max(nm, std::min(nm * kk_steps, tuning::get_int("HELIUM_HIP_GEMM_LOAD_SPREAD", nm))) : nm;
-            int q = 0, done = 0;  // MFMAs planned so far, loads planned so far
-            const int dl_b = direct_b ? t.bk * t.bn * esz / 1024 / waves : 0;
-            const int a_spread = std::max(1, std::min(nm * (kk_steps - 1), tuning::get_int("HELIUM_HIP_GEMM_RING5_SPREAD", nm * (kk_steps - 1))));
-            auto loads_before_mfma = [&](int total) {
-                // (five-slot ring: the B tile's loads between the carried MFMAs, the A tile's over the MFMAs after them)
-                const int upto = ring5 ? (q < nm ? dl_b * (q + 1) / nm : std::min(total, dl_b + (total - dl_b) * (q + 1 - nm) / a_spread))
-                                       : q < spread ? total * (q + 1) / spread : total;
-                if (upto > done) plan << "__builtin_amdgcn_sched_group_barrier(0x020, " << (upto - done) << ", 0);\n";
-                done = std::max(done, upto);
-            };
             for (int g = 0; g < kk_steps; g++) {
                 int issue = std::max(0, std::min(per, dl - g * per));
                 if (g == 0) {
                     plan << "__builtin_amdgcn_sched_group_barrier(0x100, " << nr << ", 0);\n";
-                    for (int m = 0; m < nm; m++) {  // direct loads between the carried MFMAs
-                        loads_before_mfma(issue);
+                    int done = 0;
+                    for (int m = 0; m < nm; m++) {  // direct loads spread evenly between the carried MFMAs
+                        const int upto = issue * (m + 1) / nm;
+                        if (upto > done) plan << "__builtin_amdgcn_sched_group_barrier(0x020, " << (upto - done) << ", 0);\n";
+                        done = upto;
                         plan << "__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);\n";
-                        q++;
                     }
-                } else if (issue && !issue_front) {
+                } else if (issue) {
                     plan << "__builtin_amdgcn_sched_group_barrier(0x020, " << issue << ", 0);\n";
                 }
                 if (g + 1 == kk_steps) break;
                 // MFMAs of step g with the reads of step g + 1
                 int left = nr;
                 for (int m = 0; m < nm; m++) {
-                    if (issue_front) loads_before_mfma(dl);
                     plan << "__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);\n";
-                    q++;
                     const int r = std::min(left, rate);
                     if (r) plan << "__builtin_amdgcn_sched_group_barrier(0x100, " << r << ", 0);\n";
                     left -= r;
@@ -1605,7 +1400,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         } else if (mode == 2) {
             // reads of step kk+1 are spread between the MFMAs of step kk
             plan << "__builtin_amdgcn_sched_group_barrier(0x100, " << nr << ", 0);\n";
-            const int waves = loaders;
+            const int waves = threads / 64;
             const int dl = ((direct_a ? t.bm * t.bk * esz / 1024 : 0) + (direct_b ? t.bk * t.bn * esz / 1024 : 0)) / waves;
             const int per = issue_front ? dl : (dl + kk_steps - 1) / kk_steps;
             for (int kk = 0; kk < kk_steps; kk++) {
@@ -1692,9 +1487,9 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     std::string reduce_args;
     for (int a : reduce_outs_) reduce_args += (reduce_args.empty() ? "" : ",") + std::to_string(a);
     describe_ = strfmt("gemm [%lld,%lld,%lld]x[%lld] tile=%dx%dx%d stages=%d waves=%dx%d threads=%d grid=%ux%u rawA=%d rawB=%d NVA=%d NVB=%d NVE=%d "
-                       "direct=%d%d pingpong=%d ring5=%d loaders=%d mma=%s epilogue_exprs=%zu outs=%zu split_k=%d reduce_ws=%llu reduce_grid=%u reduce_args=[%s] reduce_counters=%llu",
+                       "direct=%d%d mma=%s epilogue_exprs=%zu outs=%zu split_k=%d reduce_ws=%llu reduce_grid=%u reduce_args=[%s] reduce_counters=%llu",
                        (long long)pr.batch, (long long)pr.M, (long long)pr.K, (long long)pr.N, t.bm, t.bn, t.bk, t.stages, t.wm, t.wn, threads,
-                       grid_[0], grid_[1], (int)raw_a, (int)raw_b, nva, nvb, nve, (int)direct_a, (int)direct_b, (int)pingpong, (int)ring5, loaders, dtype_name(pr.mma_dtype), pr.epi.exprs.size(),
+                       grid_[0], grid_[1], (int)raw_a, (int)raw_b, nva, nvb, nve, (int)direct_a, (int)direct_b, dtype_name(pr.mma_dtype), pr.epi.exprs.size(),
                        pr.epi.outs.size(), pr.split_k, (unsigned long long)reduce_floats_, reduce_grid_, reduce_args.c_str(), (unsigned long long)reduce_counters_);
     kernel_.reset(new JitKernel(source_, "fused_matmul", {"-ffp-contract=fast", "-munsafe-fp-atomics"}));
     if (pr.split_k > 1) finalize_.reset(new JitKernel(source_, "fused_matmul_finalize", {"-ffp-contract=fast", "-munsafe-fp-atomics"}));
@@ -1715,10 +1510,12 @@ void GemmKernel::load() {
     kernel_->load();
     if (finalize_) finalize_->load();
     if (reduce_) reduce_->load();
+    if (reduce_counters_) load_fill_kernel();  // execute_in_scratch clears the arrival counters with it
 }
 
 bool GemmKernel::loaded() const {
-    return kernel_->loaded() && (!finalize_ || finalize_->loaded()) && (!reduce_ || reduce_->loaded());
+    return kernel_->loaded() && (!finalize_ || finalize_->loaded()) && (!reduce_ || reduce_->loaded()) &&
+           (!reduce_counters_ || fill_kernel_loaded());
 }
 
 void GemmKernel::execute(void* const* ptrs, hipStream_t stream) {
@@ -1790,7 +1587,8 @@ void CompositeKernel::zero_outputs(void* const* ptrs, hipStream_t stream) const 
     std::vector<std::pair<void*, std::pair<uint32_t, uint32_t>>> fills;
     const auto& a = args();
     for (size_t i = 0; i < a.size(); i++)
-        if (a[i].is_output) fills.push_back({ptrs[i], {(uint32_t)(storage_bytes(a[i].dtype, (size_t)a[i].numel) / 4), 0u}});
+        // (whole words, rounded up: an odd count of 16-bit elements ends in half a word, and blocks are 256-byte granules)
+        if (a[i].is_output) fills.push_back({ptrs[i], {(uint32_t)((storage_bytes(a[i].dtype, (size_t)a[i].numel) + 3) / 4), 0u}});
     if (!fills.empty()) fill_buffers(fills, stream);
 }
 

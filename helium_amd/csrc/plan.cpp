@@ -76,9 +76,9 @@ bool feeds_only_reductions(const ir::OpGraph& g, NodeId node, int budget) {
 }
 void set_fuse_matmul_epilogue(bool on) { g_fuse_matmul_epilogue.store(on); }
 bool fuse_matmul_epilogue() { return g_fuse_matmul_epilogue.load(); }
-unsigned option_mask() {
+uint64_t option_mask() {
     // the hash of the tuning overrides (0 unless tuning is on) rides along: plans keep their kernels
-    return (fuse_matmul_epilogue() ? 1u : 0u) | (g_fold_swap_into_reduce.load() ? 2u : 0u) | (g_rematerialize.load() ? 4u : 0u) | (g_cancel_transposes.load() ? 8u : 0u) | (g_hoist_broadcasts.load() ? 16u : 0u) | (tuning::hash() << 5);
+    return (fuse_matmul_epilogue() ? 1u : 0u) | (g_fold_swap_into_reduce.load() ? 2u : 0u) | (g_rematerialize.load() ? 4u : 0u) | (g_cancel_transposes.load() ? 8u : 0u) | (g_hoist_broadcasts.load() ? 16u : 0u) | ((uint64_t)tuning::hash() << 5);
 }
 void set_fold_swap_into_reduce(bool on) { g_fold_swap_into_reduce.store(on); }
 void set_rematerialize(bool on) { g_rematerialize.store(on); }
@@ -670,7 +670,7 @@ std::shared_ptr<const ir::OpGraph> graph_for_execution(const std::shared_ptr<con
 // ---------------------------------------------------------------------------------------------------------
 namespace {
 struct CacheEntry {
-    unsigned options;
+    uint64_t options;
     uint64_t hash;
     std::shared_ptr<const ir::OpGraph> graph;
     std::shared_ptr<const Plan> plan;

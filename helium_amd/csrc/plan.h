@@ -71,7 +71,7 @@ void set_fuse_matmul_epilogue(bool on);
 bool fuse_matmul_epilogue();
 // Whether a large SwapDims whose values all end in reductions stays in the pointwise instruction instead of becoming
 // a permute instruction of its own (on by default). Off gives the reference's choice by element count alone.
-unsigned option_mask();  // the options above as bits: what a generated plan depends on besides the graph
+uint64_t option_mask();  // the options above as bits: what a generated plan depends on besides the graph
 void set_fold_swap_into_reduce(bool on);
 bool fold_swap_into_reduce();
 

@@ -1,6 +1,7 @@
 // hiprtc compilation with a memory + disk cache, and a loaded-kernel wrapper
 // (the counterpart of KernelBuilder::build_ptx / JitKernel in helium/src/cuda/kernel_jit.rs).
 #pragma once
+#include <atomic>
 #include <memory>
 #include <string>
 #include <vector>
@@ -46,7 +47,7 @@ public:
     int vgprs();
     // Loads the code object onto the current device (allocates device memory for the code); launch does it on demand.
     void load() { ensure_loaded(); }
-    bool loaded() const { return func_ != nullptr; }
+    bool loaded() const { return func_.load(std::memory_order_acquire) != nullptr; }
 
 private:
     void ensure_loaded();
@@ -54,7 +55,7 @@ private:
     std::vector<std::string> options_;
     std::shared_ptr<const std::vector<char>> code_;
     hipModule_t module_ = nullptr;
-    hipFunction_t func_ = nullptr;
+    std::atomic<hipFunction_t> func_{nullptr};  // written under the load mutex, read without it
 };
 
 }  // namespace he

@@ -164,6 +164,9 @@ std::string emit_raw_members(const Program& p, int nv, bool row_varying_only = f
 std::string emit_exprs(const Program& p, const EmitCtx& cx);
 // Largest vector width (elements) legal for every full-row access and store of the program.
 int pick_nv(const Program& p, int max_bytes);
+// Whether an output tensor is written with streaming stores (st_vec<NV, true>): 4 MiB or more, i.e. too large to be
+// read back out of L2 by whoever comes next.
+bool streams_out(const Arg& a);
 std::string emit_prelude(const Program& p);
 const char* c_type(int dtype);
 

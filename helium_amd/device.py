@@ -139,6 +139,17 @@ class DeviceBuffer:
             check(lib.he_stream_synchronize(_h(stream)))
         return out if shape is None else out.reshape(shape)
 
+    def read(self, byte_offset, dtype, count, stream=None):
+        """`count` elements of `dtype` starting `byte_offset` bytes into the buffer (a sampled download)."""
+        dtype = np.dtype(dtype)
+        out = np.empty(int(count), dtype=dtype)
+        assert 0 <= byte_offset and byte_offset + out.nbytes <= self.nbytes, (byte_offset, out.nbytes, self.nbytes)
+        if out.nbytes:
+            src = C.c_void_p(self.ptr.value + int(byte_offset))
+            check(lib.he_memcpy_d2h_async(out.ctypes.data_as(C.c_void_p), src, out.nbytes, _h(stream)))
+            check(lib.he_stream_synchronize(_h(stream)))
+        return out
+
     def fill_u32(self, value, stream=None):
         check(lib.he_memset_d32_async(self.ptr, value, self.nbytes // 4, _h(stream)))
 

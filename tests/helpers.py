@@ -9,7 +9,7 @@ from oracle import numerics as nm
 
 
 # ---- front-end lowerings (helium/src/raw_tensor.rs) live in the package; the tests use the same ones
-from helium_amd.frontend import broadcast_to, div, scalar_tensor, sub  # noqa: E402,F401
+from harness.frontend import broadcast_to, div, scalar_tensor, sub  # noqa: E402,F401
 
 
 # ---- runners -----------------------------------------------------------------------------------------------

@@ -6,7 +6,7 @@ import os
 
 import numpy as np
 
-from helium_amd import autodiff as ad
+from harness import autodiff as ad
 from oracle import helium_ir as oracle_ir
 from oracle import numerics as nm
 

@@ -282,7 +282,7 @@ def test_batch_norm_train_step(gpu, fold):
     """BatchNorm2d::forward in Train mode + Relu (helium/src/modules/batch_norm.rs:32-72) above the 1M-element
     SwapDims threshold, planned both ways: with the transposition folded into the statistics kernel and as the
     reference plans it (permute, then two reductions)."""
-    from helium_amd import frontend
+    from harness import frontend
     from helium_amd.backend import OPT_FOLD_SWAP_INTO_REDUCE, set_option
 
     shape = [8, 36, 36, 128]  # 1.3M elements
@@ -320,7 +320,7 @@ def test_batch_norm_train_step(gpu, fold):
 def test_residual_block_forward(gpu):
     """BasicBlock::forward in Train mode (resnet-train/src/model.rs:155-165) through execute_graph: the first convolution's
     instruction takes its bias and the second batch norm's statistics, the second one its bias and the shortcut add."""
-    from helium_amd import frontend
+    from harness import frontend
 
     shape = [4, 12, 10, 64]
     c = shape[3]
@@ -361,7 +361,7 @@ def test_convolution_takes_the_batch_norm_statistics_of_its_output(gpu, image, o
     """conv -> BatchNorm2d(train) -> relu through execute_graph: the convolution's kernel also folds its output per
     channel (mean of y and of y^2, written SwapDims + Reduce), the rest of the batch norm runs as pointwise kernels.
     The last case has batch = channels: the Reduce's input then has the output's own shape."""
-    from helium_amd import frontend
+    from harness import frontend
 
     rng = np.random.default_rng(31)
     g = ha.ir.OpGraph()
@@ -424,6 +424,8 @@ def test_convolution_runs_as_an_implicit_gemm(gpu, image, oc, kernel, stride, mo
     ((2, 30, 30, 64), 128, (3, 3), (2, 2), "bf16"),
     ((2, 30, 30, 64), 128, (1, 1), (2, 2), "bf16"),
     ((1, 17, 19, 16), 24, (3, 3), (1, 1), "f32"),
+    # classes of pixels that no tap reaches (zeroed by the fill), the last pixel among them
+    ((1, 7, 7, 8), 8, (3, 3), (4, 4), "bf16"),
 ])
 def test_convolution_backward_data_runs_as_an_implicit_gemm(gpu, image, oc, kernel, stride, dtype):
     """Op::ConvBackwardData through execute_graph against the oracle's adjoint of the forward convolution, and the

@@ -267,7 +267,7 @@ def test_random_graphs_searched_by_subdivision(seed):
 
 
 # ---- the MI355X cost model (no counterpart in the reference beyond its fitted constants, cost_model.rs:200-207) ------
-# Times measured on an MI355X with `python -m helium_amd.cost_fit` (profiles/cost_model_fit.txt), microseconds.
+# Times measured on an MI355X with `python -m harness.cost_fit` (profiles/cost_model_fit.txt), microseconds.
 MEASURED_US = {
     ("C5a", "core[m2,e3]"): 164.7, ("C5a", "aux[2]+core[m0,e3]"): 133.3, ("C5a", "aux[1]+aux[2]+core[m0,e2]"): 148.1,
     ("C4m", "core[m2,e39]"): 199.3, ("C4m", "aux[2]+core[m0,e39]"): 171.4,
@@ -283,7 +283,7 @@ def _kinds(plan):
 
 
 def test_mi355x_model_ranks_the_measured_plans_the_way_the_gpu_did():
-    from helium_amd import cost_fit
+    from harness import cost_fit
 
     graphs = cost_fit.graphs()
     for name in sorted({k[0] for k in MEASURED_US}):
@@ -321,3 +321,15 @@ def test_mi355x_model_materialises_a_mainloop_chain_that_many_tile_columns_would
     a0, t, b = narrow.producer([1, 4096, 4096]), narrow.producer([1, 4096, 4096]), narrow.producer([1, 4096, 256])
     narrow.consumer(narrow.matmul(narrow.binary(narrow.unary(a0, "relu"), t, "mul"), b))
     assert _kinds(fs.FusionPlan(narrow, fs.MIN_MI355X_COST)) == "core[m2,e0]"
+
+
+def test_a_value_with_two_consumers_is_refused_when_the_plan_is_made():
+    """he_fusion_plan_execute writes every value to one caller buffer, so the search refuses such a graph up front
+    (nothing has been compiled or launched by then)."""
+    g = ha.fusion.OpGraph()
+    x = g.unary(g.producer([1, 64, 64], "f32"), "relu")
+    g.consumer(x, "f32")
+    g.consumer(x, "f32")
+    for objective in (fs.MAXIMAL, fs.MIN_MI355X_COST):
+        with pytest.raises(ha.HeliumError, match="two Consumers"):
+            fs.FusionPlan(g, objective)

@@ -5,12 +5,13 @@ where a reduction walks its operand in another order - and the transpositions th
 
 The recorded graphs are what the reference's front end writes for these computations: a reduction over leading dims as
 SwapDims + Reduce (batch_norm.rs:41-46), a SwapDims answered by a SwapDims in the backward pass and the gradient of a
-broadcast as a chain of swaps in front of a Reduce (tensor.rs; helium_amd/autodiff.py restates them)."""
+broadcast as a chain of swaps in front of a Reduce (tensor.rs; harness/autodiff.py restates them)."""
 import numpy as np
 import pytest
 
-from helium_amd import autodiff as ad
-from helium_amd import ir, resnet
+from harness import autodiff as ad
+from helium_amd import ir
+from harness import resnet
 from helium_amd.backend import OPT_CANCEL_TRANSPOSES, OPT_HOIST_BROADCASTS, OPT_REMATERIALIZE, Plan, set_option
 from oracle import helium_ir as oracle_ir
 from oracle import numerics as nm

@@ -93,3 +93,36 @@ def test_f16_and_u32_take_the_same_path(gpu):
 def test_empty_tensor_is_a_no_op(gpu):
     p = PermuteDims((0, 5), "f32", perm=(1, 0))
     p.execute(DeviceBuffer(16), DeviceBuffer(16))
+
+
+def test_the_reference_benchmark_at_full_size(gpu):
+    """helium/examples/permute_dim_benchmark.rs:13-41: f32 [2048,128,128,32], swap_dims(0, 3) - 4.3 GB in, 4.3 GB out.
+    Input element i holds the value i, so the whole output is checked against the closed form of its index, slices of
+    it against the oracle's permute of the same slices of the input, and permuting twice must restore the input."""
+    from helium_amd import configs
+
+    shape, perm = configs.PERM_REF_SHAPE, configs.PERM_REF_PERM
+    numel = int(np.prod(shape))
+    p = PermuteDims(shape, "f32", perm=perm)
+    print(f"permute {shape} f32 perm={perm}: {p.description}", flush=True)
+    x = np.arange(numel, dtype=np.uint32)
+    src = DeviceBuffer.from_numpy(x)
+    dst = DeviceBuffer(x.nbytes)
+    dst.fill_u8(0xEE)
+    p.execute(src, dst)
+    chunk = 1 << 24
+    for start in range(0, numel, chunk):  # the whole output, 64 MiB at a time
+        got = dst.read(start * 4, np.uint32, chunk)
+        assert np.array_equal(got, configs.perm_ref_expected(np.arange(start, start + chunk, dtype=np.uint64))), start
+    # slices against the oracle: output[:, a, b, :] is the permute of input[:, a, b, :] (dims 1 and 2 stay in place)
+    xs = x.reshape(shape)
+    rng = np.random.default_rng(9)
+    for a, b in rng.integers(0, 128, size=(6, 2)):
+        want = oracle.permute(np.ascontiguousarray(xs[:, a:a + 1, b:b + 1, :]), perm)[:, 0, 0, :]
+        rows = [dst.read((((i3 * 128 + int(a)) * 128 + int(b)) * 2048) * 4, np.uint32, 2048) for i3 in range(32)]
+        assert np.array_equal(np.stack(rows), want), (a, b)
+    del xs
+    back = DeviceBuffer(x.nbytes)
+    PermuteDims(p.out_shape, "f32", perm=perm).execute(dst, back)   # swap_dims(0, 3) undoes itself
+    for start in range(0, numel, chunk):
+        assert np.array_equal(back.read(start * 4, np.uint32, chunk), x[start:start + chunk]), start

@@ -212,7 +212,7 @@ def test_plan_cache_returns_the_same_plan_for_an_equal_graph():
 
 
 def batch_norm_graph(shape):
-    from helium_amd import frontend
+    from harness import frontend
 
     g = ha.ir.OpGraph()
     rec = frontend.Recorder(g)
@@ -250,7 +250,7 @@ def test_batch_norm_statistics_join_the_convolution_that_feeds_them():
     """conv -> BatchNorm2d (a resnet block's first half): the per-channel means of y and y^2 are column reductions of the
     implicit GEMM, so the convolution's instruction takes the SwapDims, the square and both reductions; the rest of
     the batch norm needs the finished statistics and stays outside."""
-    from helium_amd import frontend
+    from harness import frontend
 
     g = ha.ir.OpGraph()
     rec = frontend.Recorder(g)

@@ -13,7 +13,7 @@ but for rounding, in any arithmetic - those are checked to be small, not equal."
 import numpy as np
 import pytest
 
-from helium_amd import resnet
+from harness import resnet
 from helium_amd.backend import Plan, Tensor, execute_graph
 from oracle import helium_ir as oracle_ir
 from oracle import numerics as nm
@@ -120,12 +120,13 @@ def test_training_step_in_bf16_matches_the_oracle_as_far_as_the_arithmetic_pins_
             assert _rel(_f64(got[o], "f32"), _f64(want[o], "f32")) <= 0.1, (kind,)
 
 
-def test_training_step_at_the_reference_size_has_the_invariants_of_a_first_step(gpu):
-    """Batch 64 of 256 x 256 images (train.rs:33,286-287), 1000 classes, random He-initialised weights: the loss is
-    ln(1000) within a few percent, every row of the probabilities sums to one, the running statistics have moved a
-    tenth of the way from (0, 1) towards the batch statistics, and every new parameter is finite."""
-    batch = 64
-    r = resnet.record_training_step(batch, 256)
+@pytest.mark.parametrize("batch,image", [(64, 256), (128, 224)], ids=["reference_64x256", "baseline_128x224"])
+def test_training_step_at_full_size_has_the_invariants_of_a_first_step(gpu, batch, image):
+    """Batch 64 of 256 x 256 images (the reference's own size, train.rs:33,286-287) and batch 128 of 224 x 224 (the size
+    the benchmark configuration names), 1000 classes, random He-initialised weights: the loss is ln(1000) within a few
+    percent, every row of the probabilities sums to one, the running statistics have moved a tenth of the way from
+    (0, 1) towards the batch statistics, and every new parameter is finite."""
+    r = resnet.record_training_step(batch, image)
     G = r["graph"]
     by_id = {n["id"]: n for n in G.g.nodes}
     tensors = {i: Tensor.from_numpy(a, by_id[i]["dtype"], int(np.prod(by_id[i]["shape"]))) for i, a in G.feeds.items()}

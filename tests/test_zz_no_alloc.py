@@ -51,6 +51,25 @@ def test_outputs_equal_the_allocating_entry_point_call_after_call(gpu):
                 assert np.array_equal(a, b), (k.description, round_)
 
 
+def test_first_call_on_a_gemm_with_arrival_counters_loads_nothing(gpu):
+    """A small fused GEMM folds its column sums inside the kernel (arrival counters, cleared by the library's fill kernel
+    at the head of every allocation-free call). Created after he_init, its first call must find every code object
+    loaded - the fill kernel's included - so the call neither compiles nor looks anything up."""
+    import gemm_cases
+    from helium_amd import device
+
+    g, inputs, _ = gemm_cases.bias_relu_colsum(192, 320, 128)
+    k = ha.TileKernel.fused(g)
+    assert int(re.search(r"reduce_counters=(\d+)", k.description).group(1)) > 0, k.description
+    before = device.rtc_stats()
+    got = _run(k, inputs, noalloc=True)   # the allocation-free entry point first: nothing was launched before
+    assert device.rtc_stats() == before
+    want = _run(k, inputs, noalloc=False)
+    assert len(got) == len(want) >= 2
+    for a, b in zip(got, want):
+        assert np.array_equal(a, b), k.description
+
+
 def test_a_kernel_that_needs_more_scratch_is_refused(gpu):
     g, _, _ = configs.c3_chain(16384, 16384, make_inputs=False)
     k = ha.TileKernel.auxiliary(g)
