@@ -326,6 +326,15 @@ int pick_nv(const Program& p, int max_bytes) {
     return nv;
 }
 
+// A load whose value is one element per row (a [.., M, 1] operand broadcast along the columns): deferred as a scalar
+// when only row-varying loads are (the GEMM epilogue's pipelined form, where a load left inline would be younger than
+// the next step's requests and make the step wait for them).
+static bool is_deferred_row_scalar(const Program& p, const Expr& e, bool row_varying_only) {
+    if (!row_varying_only || e.kind != Expr::Load || !e.access.chain.empty() || e.access.dtype == HE_BOOL) return false;
+    const int n = (int)p.dims.size();
+    if (n < 2 || p.dims[n - 2] <= 1 || e.access.stride[n - 2] == 0) return false;
+    return p.dims[n - 1] <= 1 || e.access.stride[n - 1] == 0;
+}
 static bool is_deferred_load(const Program& p, const Expr& e, int nv, bool row_varying_only = false) {
     if (e.kind != Expr::Load || nv < 2 || !e.access.chain.empty() || e.access.dtype == HE_BOOL) return false;
     const int n = (int)p.dims.size();
@@ -340,6 +349,7 @@ std::string emit_raw_members(const Program& p, int nv, bool row_varying_only) {
     std::ostringstream s;
     for (size_t i = 0; i < p.exprs.size(); i++)
         if (is_deferred_load(p, p.exprs[i], nv, row_varying_only)) s << raw_type(p.exprs[i].access.dtype, nv) << " raw" << i << ";\n";
+        else if (is_deferred_row_scalar(p, p.exprs[i], row_varying_only)) s << cls_type(p.exprs[i].cls) << " raw" << i << ";\n";
     return s.str();
 }
 
@@ -393,6 +403,11 @@ std::string emit_exprs(const Program& p, const EmitCtx& cx) {
         const char* T = cls_type(e.cls);
         if (cx.row_part == 1 && !invariant[i]) continue;
         if (cx.row_part == 2 && invariant[i]) continue;
+        if (cx.phase != 0 && is_deferred_row_scalar(p, e, cx.defer_row_varying_only)) {
+            if (cx.phase == 1) s << "R.raw" << i << " = ld_one(a" << e.access.arg << " + " << coord_sum(e.access.stride) << ");\n";
+            else s << T << " " << v << "[" << NV << "];\n#pragma unroll\nfor (int k = 0; k < " << NV << "; k++) " << v << "[k] = R.raw" << i << ";\n";
+            continue;
+        }
         if (cx.phase != 0) {
             const bool deferred = is_deferred_load(p, e, NV, cx.defer_row_varying_only);
             if (cx.phase == 1) {

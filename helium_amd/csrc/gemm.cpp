@@ -1127,26 +1127,33 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
 
     // epilogue pieces
     std::ostringstream setup, body, finish, prefetch;
-    // Optional (HELIUM_HIP_GEMM_EPIPIPE=1): full-size tensors the epilogue reads are requested one step ahead of the
-    // step that uses them. Measured within run-to-run noise of the compiler's own placement on the 40-op epilogue
-    // (162.5 vs 162.6 us over three alternating runs each), so off.
+    // The tensors an epilogue reads row by row (full-size operands, per-row vectors) are requested EPI_DEPTH steps ahead
+    // of the step that uses them, into registers; what does not depend on the row (per-column vectors, constants and
+    // what is computed from those alone) is loaded and computed once per wave, ahead of the strips. Left to itself
+    // the compiler requests a step's operands inside the step, in two dependent groups, so that a wave's sixteen steps
+    // were thirty-two memory round trips one after the other (the 40-op epilogue: 30 us on top of the product). A load
+    // left inside the step would also be younger than the requests for the next step, and waiting for it waits for
+    // them: hence everything row-varying is requested ahead, and everything else hoisted.
     const std::string raw_members = tp::emit_raw_members(pr.epi, nve, true);
-    const char* epipipe = tuning::get("HELIUM_HIP_GEMM_EPIPIPE");
-    const bool pipelined = !raw_members.empty() && epipipe && atoi(epipipe) != 0;
+    const int epi_depth = std::max(0, std::min(3, tuning::get_int("HELIUM_HIP_GEMM_EPIPIPE", 1)));
+    const bool pipelined = !raw_members.empty() && epi_depth > 0 && pr.split_k == 1;
+    // hoisting needs a lane's columns to be the same in every step: steps that cover whole rows of the strip
+    bool hoisted = pipelined && colsets == 1 && (64 * nve) % wtn == 0 && !tuning::get("HELIUM_HIP_GEMM_NO_EPI_HOIST");
+    for (size_t i = 0; i < pr.epi.exprs.size(); i++) hoisted = hoisted && !tp::is_uniform_pow(pr.epi, (int)i);
     if (pipelined) {
         tp::EmitCtx lx;
         lx.nv = nve;
         lx.phase = 1;
         lx.defer_row_varying_only = true;
-        s << "struct RawE {\n" << raw_members << "};\n__device__ __forceinline__ void epi_load(";
+        s << "#define EPI_DEPTH " << epi_depth << "\nstruct RawE {\n" << raw_members << "};\n__device__ __forceinline__ void epi_load(";
         for (size_t a = 0; a < pr.epi.args.size(); a++)
             s << (pr.epi.args[a].is_output ? "" : "const ") << tp::c_type(pr.epi.args[a].dtype) << "* __restrict__ a" << a << ", ";
         s << "u32 cB0, u32 m, u32 n0, RawE& R) {\n(void)cB0; (void)m; (void)n0;\n" << tp::emit_exprs(pr.epi, lx) << "}\n";
         std::string pass;
         for (size_t a = 0; a < pr.epi.args.size(); a++) pass += "a" + std::to_string(a) + ", ";
-        prefetch << "{ const int q1 = i * EPI_STEPS + step + 1;\nif (q1 < MB * EPI_STEPS) {\nconst int i1 = q1 / EPI_STEPS, s1 = q1 % EPI_STEPS;\n"
+        prefetch << "{ const int q1 = i * EPI_STEPS + step + EPI_DEPTH;\nif (q1 < MB * EPI_STEPS) {\nconst int i1 = q1 / EPI_STEPS, s1 = q1 % EPI_STEPS;\n"
                  << "const u32 idx1 = (s1 * 64 + lane) * NVE;\nconst u32 m1 = m0 + wave_m * WTM + i1 * 32 + idx1 / WTN, nn1 = n0 + wave_n * WTN + idx1 % WTN;\n"
-                 << "if (m1 < GM && nn1 < GN) epi_load(" << pass << "bz, m1, nn1, Rb[q1 & 1]);\n} }\n";
+                 << "if (m1 < GM && nn1 < GN) epi_load(" << pass << "bz, m1, nn1, Rb[q1 % (EPI_DEPTH + 1)]);\n} }\n";
     }
     for (size_t a = 0; a < pr.epi.args.size(); a++)
         setup << "auto* a" << a << " = p" << pr.map_e[a] << "; (void)a" << a << ";\n";
@@ -1154,8 +1161,26 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     if (pipelined) {
         std::string pass;
         for (size_t a = 0; a < pr.epi.args.size(); a++) pass += "a" + std::to_string(a) + ", ";
-        setup << "RawE Rb[2];\n{ const u32 idx1 = lane * NVE;\nconst u32 m1 = m0 + wave_m * WTM + idx1 / WTN, nn1 = n0 + wave_n * WTN + idx1 % WTN;\n"
-              << "if (m1 < GM && nn1 < GN) epi_load(" << pass << "bz, m1, nn1, Rb[0]);\n}\n";
+        setup << "RawE Rb[EPI_DEPTH + 1];\n#pragma unroll\nfor (int q1 = 0; q1 < EPI_DEPTH && q1 < MB * EPI_STEPS; q1++) {\nconst int i1 = q1 / EPI_STEPS, s1 = q1 % EPI_STEPS;\n"
+              << "const u32 idx1 = (s1 * 64 + lane) * NVE;\nconst u32 m1 = m0 + wave_m * WTM + i1 * 32 + idx1 / WTN, nn1 = n0 + wave_n * WTN + idx1 % WTN;\n"
+              << "if (m1 < GM && nn1 < GN) epi_load(" << pass << "bz, m1, nn1, Rb[q1]);\n}\n";
+    }
+    if (hoisted) {
+        // the emitter names the first of a lane's columns `n0`, which is the tile's origin out here
+        tp::EmitCtx hx;
+        hx.nv = nve;
+        hx.row_part = 1;
+        std::string text = tp::emit_exprs(pr.epi, hx), renamed;
+        for (size_t i = 0; i < text.size();) {
+            const bool word_start = i == 0 || !(isalnum((unsigned char)text[i - 1]) || text[i - 1] == '_');
+            if (word_start && text.compare(i, 2, "n0") == 0 && (i + 2 == text.size() || !(isalnum((unsigned char)text[i + 2]) || text[i + 2] == '_'))) {
+                renamed += "n0_lane";
+                i += 2;
+            } else {
+                renamed += text[i++];
+            }
+        }
+        setup << "const u32 n0_lane = n0 + wave_n * WTN + (lane * NVE) % WTN; const bool col_ok = n0_lane < GN; (void)col_ok;\n" << renamed;
     }
     for (size_t oi = 0; oi < pr.epi.outs.size(); oi++) {
         const tp::Out& o = pr.epi.outs[oi];
@@ -1194,8 +1219,9 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
             if (pipelined) {
                 cx.phase = 2;
                 cx.defer_row_varying_only = true;
-                b << "const RawE& R = Rb[(i * EPI_STEPS + step) & 1]; (void)R;\n";
+                b << "const RawE& R = Rb[(i * EPI_STEPS + step) % (EPI_DEPTH + 1)]; (void)R;\n";
             }
+            if (hoisted) cx.row_part = 2;
             // the emitter names the first of the NV columns `n0`; the tile origin of the same name is shadowed here
             b << tp::emit_exprs(pr.epi, cx);
             for (size_t oi = 0; oi < pr.epi.outs.size(); oi++) {
