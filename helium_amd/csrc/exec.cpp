@@ -436,6 +436,7 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
         double us;
         int64_t bytes;
         const plan::Instr* instr;
+        size_t order;  // position in the execution
     };
     std::vector<InstrTime> instr_times;
     // Whatever happens below, the scope must end, and only after the work already queued: a failing instruction leaves
@@ -507,7 +508,7 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
                 int64_t bytes = 0;
                 for (NodeId n : instr.inputs()) bytes += (int64_t)tensors.at(n)->bytes;
                 for (NodeId n : instr.outputs()) bytes += (int64_t)tensors.at(n)->bytes;
-                instr_times.push_back({us, bytes, &instr});
+                instr_times.push_back({us, bytes, &instr, instr_times.size()});
             }
             // taken by the instruction's last launch, or still pending (a launch too large for that entry point)
             if (&instr == closing) done_recorded = take_pending_stop_event() == nullptr;
@@ -558,7 +559,7 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
             const int top = atoi(getenv("HELIUM_HIP_INSTR_TIMING"));
             for (int i = 0; i < top && i < (int)instr_times.size(); i++) {
                 const std::string d = instr_times[i].instr->describe();
-                fprintf(stderr, "  %8.1f us %8.1f MB %6.2f TB/s  %s\n", instr_times[i].us, instr_times[i].bytes / 1e6,
+                fprintf(stderr, "  #%-4zu %8.1f us %8.1f MB %6.2f TB/s  %s\n", instr_times[i].order, instr_times[i].us, instr_times[i].bytes / 1e6,
                         instr_times[i].bytes / instr_times[i].us / 1e6, d.substr(0, 200).c_str());
             }
         }

@@ -105,7 +105,7 @@ def all_reductions(m, n, k, batch=2, seed=2):
 MATMUL_DTYPES = ("f32", "bf16", "f16")
 # helium-kernel-generator/tests/matmul.rs:171-181: the precisions of matmul_no_fusion (the four F8 mode pairs share one
 # entry here: the modes change nothing on hardware whose F8 products run as bf16)
-MATMUL_PRECISIONS = ("f32_f32", "tf32_f32", "bf16_f32", "f16_f32", "f16_f16", "f8_f32")
+MATMUL_PRECISIONS = ("f32_f32", "tf32_f32", "bf16_f32", "f16_f32", "f16_f16", "f8_f32", "f8_f16")
 
 
 def ir_matmul(m, n, k, dtype_a, dtype_b, precision, out_dtype, seed=7):
