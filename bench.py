@@ -25,7 +25,7 @@ F32_PEAK_TFLOPS = 157.3      # MI355X dense fp32 matrix, published
 
 
 def _traffic_table():
-    """Bytes that leave the XCD L2s per launch of each workload's dominant kernel, from the committed counter summary
+    """Bytes that leave the XCD L2s per step of each workload (all launches of the step), from the committed counter summary
     (profiles/traffic_per_launch.txt: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by the COPY workload); a workload
     the file does not list reports null."""
     table = {}

@@ -280,6 +280,41 @@ def generated_cases():
     c.out(c.op(c.g.reduce(c.op(c.g.binary(yt, c.op(c.g.swap_dims(x, 0, 3)), "mul")), "sum", 3)))
     c.reduce_rel = 1e-3; cases.append(c)
 
+    # 16-bit activations seen as [rows, channels] next to f32 per-channel vectors (a batch norm's backward pass): the
+    # per-channel operands are loaded once ahead of the rows; with few expressions two rows are in flight.
+    TALL = dict(FOLD_SMALL, HELIUM_HIP_POINTWISE_RPT="2")
+    c = Case("channel_vectors_hoisted_two_rows_in_flight"); c.env = TALL; c.admitted_by_fusion_rule = False
+    x = c.inp([1100, 64], "bf16", rng.standard_normal(1100 * 64)); sc = c.inp([64], "f32", rng.uniform(0.5, 2.0, 64))
+    sh = c.inp([64], "f32", rng.standard_normal(64))
+    bc = lambda v: c.op(c.g.broadcast(v, 2, [(0, 1100)]))
+    y = c.op(c.g.unary(c.op(c.g.binary(c.op(c.g.binary(x, bc(sc), "mul")), bc(sh), "add")), "relu"))
+    c.out(c.op(c.g.change_data_type(y, "bf16")))
+    c.out(c.op(c.g.reduce(c.op(c.g.swap_dims(y, 0, 1)), "sum", 1)))
+    c.reduce_rel = 1e-3; cases.append(c)
+
+    # The same with more than 24 expressions: one row is in flight and the next row's raw vectors are requested ahead of
+    # its arithmetic.
+    c = Case("many_expressions_rows_requested_ahead"); c.env = TALL; c.admitted_by_fusion_rule = False
+    x = c.inp([1100, 64], "bf16", rng.standard_normal(1100 * 64)); f = c.inp([1100, 64], "bf16", rng.standard_normal(1100 * 64))
+    sc = c.inp([64], "f32", rng.uniform(0.5, 2.0, 64)); sh = c.inp([64], "f32", rng.standard_normal(64))
+    var = c.inp([64], "f32", rng.uniform(0.5, 2.0, 64))
+    bc = lambda v: c.op(c.g.broadcast(v, 2, [(0, 1100)]))
+    inv = c.op(c.g.unary(c.op(c.g.unary(c.op(c.g.binary(bc(var), c.scalar(1e-3, [1100, 64]), "add")), "sqrt")), "recip"))  # the same in every row
+    xh = c.op(c.g.binary(c.op(c.g.binary(x, bc(sh), "add")), inv, "mul"))
+    y = c.op(c.g.binary(c.op(c.g.binary(xh, bc(sc), "mul")), bc(sh), "add"))
+    zero = c.op(c.g.constant(0.0, "f32", [1100, 64]))
+    mask = c.op(c.g.compare(y, zero, "gt"))
+    g1 = c.op(c.g.select(zero, f, mask))
+    t = g1
+    for fn in ("tanh", "neg", "sigmoid", "neg", "relu", "neg", "tanh", "neg"):
+        t = c.op(c.g.binary(c.op(c.g.unary(t, fn)), g1, "add"))
+    dx = c.op(c.g.binary(c.op(c.g.binary(t, bc(sc), "mul")), inv, "mul"))
+    c.out(c.op(c.g.change_data_type(dx, "bf16")))
+    c.out(c.op(c.g.change_data_type(mask, "bf16")))
+    c.out(c.op(c.g.reduce(c.op(c.g.swap_dims(t, 0, 1)), "sum", 1)))
+    c.out(c.op(c.g.reduce(c.op(c.g.swap_dims(c.op(c.g.binary(t, xh, "mul")), 0, 1)), "sum", 1)))
+    c.reduce_rel = 1e-3; cases.append(c)
+
     return cases
 
 
