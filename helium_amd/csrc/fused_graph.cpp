@@ -797,7 +797,7 @@ CostTerms mi355x_cost_terms(const FusedGraph& fg) {
 Mi355xCoefficients Mi355xCoefficients::fitted() {
     // seconds per: launch, matrix-core FLOP, L2->CU byte of extra operands, weighted mainloop op, HBM byte, weighted
     // epilogue op, weighted op of an anchor-less kernel. Non-negative least squares over the 30 measured plans listed in
-    // profiles/cost_model_fit.txt (helium_amd/cost_fit.py): mean relative error 5%, worst 12%. The launch term carries
+    // profiles/cost_model_fit.txt (harness/cost_fit.py): mean relative error 5%, worst 12%. The launch term carries
     // the host's time per kernel of he_fusion_plan_execute; the extra-operand bytes and the mainloop ops of the measured
     // plans grow together, and the fit puts all of their weight on the ops.
     return {1.467e-05, 6.998e-16, 0.0, 1.022e-13, 6.747e-14, 8.514e-15, 3.356e-14};
