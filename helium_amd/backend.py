@@ -21,6 +21,7 @@ _ffi._sig("he_plan_graph", C.c_void_p, C.POINTER(C.c_void_p))
 _ffi._sig("he_plan_describe_planned", C.c_void_p, restype=C.c_char_p)
 _ffi._sig("he_plan_destroy", C.c_void_p)
 _ffi._sig("he_plan_precompile", C.c_void_p)
+_ffi._sig("he_plan_instruction_kernel", C.c_void_p, C.c_int, C.POINTER(C.c_void_p))
 _ffi._sig("he_execute_graph", C.c_void_p, C.POINTER(C.c_uint32), C.POINTER(C.c_void_p), C.c_int, C.POINTER(C.c_uint32),
           C.POINTER(C.c_void_p), C.c_int, C.POINTER(C.c_int))
 _ffi._sig("he_backend_stats", C.POINTER(C.c_uint64))
@@ -123,6 +124,15 @@ class Plan:
         handle = C.c_void_p()
         check(lib.he_plan_graph(self.handle, C.byref(handle)))
         return ir.OpGraph.from_handle(handle)
+
+    def kernel(self, index):
+        """The compiled kernel of the index-th instruction (he_plan_instruction_kernel), as a kernels.TileKernel whose
+        argument nodes are nodes of `graph()`."""
+        from .kernels import TileKernel
+
+        h = C.c_void_p()
+        check(lib.he_plan_instruction_kernel(self.handle, index, C.byref(h)))
+        return TileKernel(h)
 
     def precompile(self):
         """Compiles the kernels of all instructions (in parallel) into the kernel caches; needs no device."""

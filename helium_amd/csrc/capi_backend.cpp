@@ -82,6 +82,23 @@ int he_plan_num_steps(he_plan_t plan, int* steps) {
 }
 const char* he_plan_describe(he_plan_t plan) { return plan ? plan->text.c_str() : ""; }
 const char* he_plan_describe_planned(he_plan_t plan) { return plan ? plan->text_planned.c_str() : ""; }
+int he_plan_instruction_kernel(he_plan_t plan, int index, he_tile_kernel_t* kernel) {
+    return he::guard([&] {
+        HE_REQUIRE(plan && kernel && index >= 0, HE_ERR_INVALID, "bad argument");
+        int at = 0;
+        for (auto& step : plan->plan->steps)
+            for (auto& instr : step.instrs)
+                if (at++ == index) {
+                    HE_REQUIRE(!instr->absorbed(), HE_ERR_INVALID, "instruction %d launches nothing: the kernel of an earlier instruction does its work", index);
+                    auto k = std::make_unique<he_tile_kernel_s>();
+                    k->k = instr->kernel();
+                    HE_REQUIRE(k->k, HE_ERR_INVALID, "instruction %d is a permute instruction", index);
+                    *kernel = k.release();
+                    return;
+                }
+        he::fail(HE_ERR_INVALID, "the plan has " + std::to_string(at) + " instructions");
+    });
+}
 int he_plan_precompile(he_plan_t plan) {
     return he::guard([&] {
         HE_REQUIRE(plan, HE_ERR_INVALID, "bad argument");

@@ -21,5 +21,5 @@ struct he_fgraph_s {
     he::fir::OpGraph g;
 };
 struct he_tile_kernel_s {
-    std::unique_ptr<he::KernelBase> k;
+    std::shared_ptr<he::KernelBase> k;  // shared with the plan when the handle came from he_plan_instruction_kernel
 };

@@ -122,6 +122,13 @@ __device__ __forceinline__ void st_one(float* p, float v) { *p = v; }
 __device__ __forceinline__ void st_one(u32* p, u32 v) { *p = v; }
 __device__ __forceinline__ void st_one(bf16_t* p, float v) { *p = (bf16_t)v; }
 __device__ __forceinline__ void st_one(f16_t* p, float v) { *p = (f16_t)v; }
+// stores v and returns what a load of that element would give back (the value rounded to the element type)
+template <class T> __device__ __forceinline__ float store_and_keep(T* p, float v) {
+    T t;
+    st_one(&t, v);
+    st_one(p, v);
+    return ld_one((const T*)&t);
+}
 
 // Reduction operators: 0 Sum, 1 Mean (terms are pre-scaled), 2 Max, 3 Min.
 template <int OP> __device__ __forceinline__ float red_op(float a, float b) {
@@ -326,6 +333,48 @@ int pick_nv(const Program& p, int max_bytes) {
     return nv;
 }
 
+bool attach_post(Program* main, const Program& post) {
+    if (main->post || main->acc_expr >= 0 || post.acc_expr >= 0 || post.post || post.dims.empty()) return false;
+    // one thread per column evaluates it: a program over [columns] and nothing else
+    const int64_t cols = post.N();
+    if (ir::num_elements(post.dims) != cols || cols != main->N() || post.exprs.empty() || post.outs.empty()) return false;
+    for (const Out& o : post.outs)
+        if (o.reduce || o.dtype == HE_BOOL || !o.stride.empty()) return false;
+    for (const Expr& e : post.exprs)
+        if (e.kind == Expr::Load && (!e.access.chain.empty() || e.access.dtype == HE_BOOL)) return false;
+    // its arguments among main's: a column reduction that yields one row of `cols` values, or a tensor both only read
+    std::vector<int> to_main(post.args.size(), -1);
+    std::vector<Arg> args = main->args;
+    bool reads_a_reduction = false;
+    for (size_t a = 0; a < post.args.size(); a++) {
+        const Arg& pa = post.args[a];
+        for (size_t m = 0; m < main->args.size() && to_main[a] < 0; m++)
+            if (main->args[m].node == pa.node) to_main[a] = (int)m;
+        if (to_main[a] < 0) {
+            to_main[a] = (int)args.size();
+            args.push_back(pa);
+            continue;
+        }
+        const Arg& ma = main->args[to_main[a]];
+        if (pa.is_output) return false;  // writes what main reads or writes
+        if (!ma.is_output) continue;
+        const Out* out = nullptr;
+        for (const Out& o : main->outs)
+            if (o.arg == to_main[a]) out = &o;
+        if (!out || !out->reduce || !out->fold_m || out->fold_n || main->B() / out->b_div != 1) return false;
+        reads_a_reduction = true;
+    }
+    if (!reads_a_reduction) return false;
+    Program carried = post;
+    carried.args.clear();  // indices refer to main's list
+    for (Expr& e : carried.exprs)
+        if (e.kind == Expr::Load) e.access.arg = to_main[e.access.arg];
+    for (Out& o : carried.outs) o.arg = to_main[o.arg];
+    main->args = std::move(args);
+    main->post = std::make_shared<const Program>(std::move(carried));
+    return true;
+}
+
 // A load whose value is one element per row (a [.., M, 1] operand broadcast along the columns): deferred as a scalar
 // when only row-varying loads are (the GEMM epilogue's pipelined form, where a load left inline would be younger than
 // the next step's requests and make the step wait for them).
@@ -432,6 +481,10 @@ std::string emit_exprs(const Program& p, const EmitCtx& cx) {
         switch (e.kind) {
             case Expr::Load: {
                 const Access& a = e.access;
+                if (cx.arg_values && cx.arg_values->count(a.arg)) {
+                    each(cx.arg_values->at(a.arg));
+                    break;
+                }
                 const int64_t sn = p.dims[n - 1] > 1 ? a.stride[n - 1] : 0;
                 const std::string ptr = "a" + std::to_string(a.arg);
                 if (cx.row_part == 1) s << T << " " << v << "[" << NV << "] = {};\nif (col_ok) { const size_t o = " << coord_sum(a.stride) << ";\n";
@@ -957,8 +1010,31 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
         };
         std::vector<Job> jobs;
         uint32_t total = 0;
+        // The column reductions a carried program reads are folded by the same blocks, FW columns each: the threads that
+        // end up with a column's sums go on to evaluate that program for the column.
+        std::vector<size_t> carried;  // outs
+        int64_t carried_arrivals = 0;
+        if (p.post) {
+            bool ok = true;
+            std::vector<char> read(p.args.size(), 0);
+            for (const Expr& e : p.post->exprs)
+                if (e.kind == Expr::Load) read[e.access.arg] = 1;
+            for (size_t oi = 0; oi < p.outs.size() && ok; oi++) {
+                const Out& o = p.outs[oi];
+                if (!o.reduce || !read[o.arg]) continue;
+                ok = ws[oi].on && !ws[oi].ticket && o.fold_m && !o.fold_n && B / o.b_div == 1 &&
+                     (carried.empty() || carried_arrivals == gy * o.b_div);
+                carried_arrivals = gy * o.b_div;
+                carried.push_back(oi);
+            }
+            if (!ok || carried.empty()) carried.clear();
+            L.post_carried = !carried.empty();
+        }
+        auto is_carried = [&](size_t oi) { return std::find(carried.begin(), carried.end(), oi) != carried.end(); };
+        const int CFW = carried.empty() ? 0 : fold_width(p.outs[carried[0]]);
+        if (!carried.empty()) total = (uint32_t)((N + CFW - 1) / CFW);
         for (size_t oi = 0; oi < p.outs.size(); oi++) {
-            if (!ws[oi].on || ws[oi].ticket) continue;
+            if (!ws[oi].on || ws[oi].ticket || is_carried(oi)) continue;
             const Out& o = p.outs[oi];
             const int FW = fold_width(o);
             const uint32_t nb = o.fold_n ? (uint32_t)(B / o.b_div) : (uint32_t)((B / o.b_div) * ((N + FW - 1) / FW));
@@ -971,6 +1047,41 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
         for (size_t a = 0; a < p.args.size(); a++)
             s << (a ? ", " : "") << (p.args[a].is_output ? "" : "const ") << c_type(p.args[a].dtype) << "* __restrict__ a" << a;
         s << ", const float* __restrict__ wsf) {\n__shared__ float fin_red[" << threads << "];\n";
+        if (!carried.empty()) {
+            const int FW = CFW, FG = threads / FW;
+            const int64_t arrivals = carried_arrivals, slices = (N + FW - 1) / FW;
+            s << "if (blockIdx.x < " << slices << "u) {\nconst u32 n = blockIdx.x * " << FW << "u + threadIdx.x % " << FW
+              << "u, grp = threadIdx.x / " << FW << "u;\nconst u32 tile_x = n / (TX * NV), within = n % (TX * NV);\n";
+            std::map<int, std::string> values;
+            // every reduction's partials are requested before any is added up: the launch is all latency
+            for (size_t oi : carried)
+                s << "float red" << oi << " = 0.0f, acc" << oi << " = red_identity<" << (int)p.outs[oi].rop << ">();\n";
+            s << "if (n < DIM_N) {\nfor (u32 j0 = grp; j0 < " << arrivals << "u; j0 += " << FG * 8 << "u) {\n";
+            for (size_t oi : carried) {
+                const int rop = (int)p.outs[oi].rop;
+                s << "float pv" << oi << "[8];\n#pragma unroll\nfor (u32 c = 0; c < 8; c++) {\nconst u32 j = j0 + c * " << FG << "u;\npv" << oi << "[c] = j < "
+                  << arrivals << "u ? wsf[" << ws[oi].foff << "ull + (size_t)(j * " << gx << "u + tile_x) * (TX * NV) + within] : red_identity<" << rop << ">();\n}\n";
+            }
+            for (size_t oi : carried)
+                s << "#pragma unroll\nfor (u32 c = 0; c < 8; c++) acc" << oi << " = red_op<" << (int)p.outs[oi].rop << ">(acc" << oi << ", pv" << oi << "[c]);\n";
+            s << "}\n}\n";
+            for (size_t oi : carried) {
+                const Out& o = p.outs[oi];
+                const int rop = (int)o.rop;
+                s << "__syncthreads();\nfin_red[threadIdx.x] = acc" << oi << ";\n__syncthreads();\nif (grp == 0 && n < DIM_N) {\nfloat acc = acc" << oi
+                  << ";\nfor (u32 g = 1; g < " << FG << "u; g++) acc = red_op<" << rop << ">(acc, fin_red[g * " << FW << "u + threadIdx.x]);\nred" << oi
+                  << " = store_and_keep(a" << o.arg << " + n, " << scaled(o, "acc") << ");\n}\n";
+                values[o.arg] = "red" + std::to_string(oi);
+            }
+            // the carried program, one column per thread
+            const Program& q = *p.post;
+            EmitCtx cx;
+            cx.nv = 1;
+            cx.arg_values = &values;
+            s << "if (grp == 0 && n < DIM_N) {\nconst u32 n0 = n, m = 0u; (void)m;\n" << emit_exprs(q, cx);
+            for (const Out& o : q.outs) s << "st_one(a" << o.arg << " + n0, e" << o.expr << "[0]);\n";
+            s << "}\nreturn;\n}\n";
+        }
         for (auto& jb : jobs) {
             const Out& o = p.outs[jb.oi];
             const int rop = (int)o.rop;
@@ -1017,7 +1128,9 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
     d << "dims=[";
     for (int i = 0; i < n; i++) d << (i ? "x" : "") << p.dims[i];
     d << "] NV=" << NV << " TX=" << TX << " TY=" << TY << " RPT=" << RPT << " grid=" << L.grid << " threads=" << threads
-      << " exprs=" << p.exprs.size() << " outs=" << p.outs.size() << " ws_floats=" << L.ws_floats << " ws_counters=" << L.ws_counters << " finalize_grid=" << L.finalize_grid << " fills=[";
+      << " exprs=" << p.exprs.size() << " outs=" << p.outs.size() << " ws_floats=" << L.ws_floats << " ws_counters=" << L.ws_counters << " finalize_grid=" << L.finalize_grid;
+    if (L.post_carried) d << " carries=" << p.post->exprs.size() << "exprs/" << p.post->outs.size() << "outs";
+    d << " fills=[";
     for (size_t i = 0; i < L.fills.size(); i++) d << (i ? "," : "") << L.fills[i].first << ":" << L.fills[i].second;
     d << "]";
     L.describe = d.str();

@@ -417,7 +417,7 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
     const int fan_mode = g_fan_out.load();
     auto step_width = [&](size_t k) {
         const plan::Step& step = plan->steps[k];
-        const bool fan = fan_mode == 2 || (fan_mode == 1 && prepared.fan_out[k]);
+        const bool fan = !step.in_order && (fan_mode == 2 || (fan_mode == 1 && prepared.fan_out[k]));
         return fan ? std::min(step.instrs.size(), st.s.size()) : std::min<size_t>(step.instrs.size(), 1);
     };
     const plan::Instr* closing = nullptr;
@@ -426,7 +426,8 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
         for (size_t k = 0; k < plan->steps.size(); k++) {
             auto& step = plan->steps[k];
             one_stream = one_stream && step_width(k) <= 1;
-            if (!step.instrs.empty()) closing = step.instrs.back().get();
+            for (auto& instr : step.instrs)
+                if (!instr->absorbed()) closing = instr.get();  // (an absorbed instruction launches nothing)
         }
         if (!one_stream || getenv("HELIUM_HIP_NO_LAUNCH_EVENTS")) closing = nullptr;
     }
@@ -458,16 +459,17 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
         ht.lap(6);
         for (size_t i = 0; i < step.instrs.size(); i++) {
             const plan::Instr& instr = *step.instrs[i];
+            if (instr.absorbed()) continue;  // run, and its outputs allocated, by the instruction that carries it
             hipStream_t stream = st.s[i % width];
             // a stream's first work of this execution comes after the end of the thread's previous execution
             // (stream 0 carried that end itself)
             if (used_streams.insert(i % width).second && i % width != 0 && st.has_run)
                 HE_HIP(hipStreamWaitEvent(stream, st.exec_end->e, 0));
-            for (NodeId out : instr.outputs()) {
+            for (NodeId out : instr.all_outputs()) {
                 const ir::Descriptor& d = graph->get(out).desc;
                 tensors[out] = allocate_tensor(d.dtype, (size_t)ir::num_elements(d.shape), scope);
             }
-            for (NodeId in : instr.inputs()) {
+            for (NodeId in : instr.all_inputs()) {
                 auto it = tensors.find(in);
                 HE_REQUIRE(it != tensors.end(), HE_ERR_INTERNAL, "missing storage for node %u", in);
                 // tensors made outside this execution carry a ready event (uploads, earlier graphs)
@@ -506,8 +508,8 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
                 HE_HIP(hipDeviceSynchronize());
                 const double us = std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t_instr).count();
                 int64_t bytes = 0;
-                for (NodeId n : instr.inputs()) bytes += (int64_t)tensors.at(n)->bytes;
-                for (NodeId n : instr.outputs()) bytes += (int64_t)tensors.at(n)->bytes;
+                for (NodeId n : instr.all_inputs()) bytes += (int64_t)tensors.at(n)->bytes;
+                for (NodeId n : instr.all_outputs()) bytes += (int64_t)tensors.at(n)->bytes;
                 instr_times.push_back({us, bytes, &instr, instr_times.size()});
             }
             // taken by the instruction's last launch, or still pending (a launch too large for that entry point)

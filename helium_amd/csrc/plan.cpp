@@ -187,14 +187,36 @@ KernelCache<KernelBase> g_tile_kernels(1024);  // pointwise.rs:45, permute_dims.
 KernelCache<Permute> g_permutes(1024);
 }  // namespace
 
+std::vector<NodeId> Instr::all_inputs() const {
+    std::vector<NodeId> in = sg_.inputs();
+    if (carried_) {
+        const std::vector<NodeId> own = sg_.leafs();
+        for (NodeId n : carried_->sg_.inputs())
+            if (std::find(own.begin(), own.end(), n) == own.end() && std::find(in.begin(), in.end(), n) == in.end()) in.push_back(n);
+    }
+    return in;
+}
+
+std::vector<NodeId> Instr::all_outputs() const {
+    std::vector<NodeId> out = sg_.leafs();
+    if (carried_)
+        for (NodeId n : carried_->sg_.leafs()) out.push_back(n);
+    return out;
+}
+
 void Instr::precompile() const {
     std::lock_guard<std::mutex> lk(mu_);
-    if (kernel_ || permute_) return;
+    if (kernel_ || permute_ || absorbed_) return;
     switch (kind_) {
         case InstrKind::Pointwise:
-            kernel_ = g_tile_kernels.get_or_insert(tuning::key() + "pw:" + sg_.cache_key(), [&] {
-                return std::shared_ptr<KernelBase>(new TileKernel(tp::lower_pointwise(sg_), "pointwise_kernel"));
-            });
+            kernel_ = g_tile_kernels.get_or_insert(
+                tuning::key() + "pw:" + sg_.cache_key() + (carried_ ? "+carries:" + carried_->sg_.cache_key() : std::string()), [&] {
+                    tp::Program prog = tp::lower_pointwise(sg_);
+                    if (carried_)
+                        HE_REQUIRE(tp::attach_post(&prog, tp::lower_pointwise(carried_->sg_)), HE_ERR_INTERNAL,
+                                   "the carried instruction does not fit the fold launch any more");
+                    return std::shared_ptr<KernelBase>(new TileKernel(std::move(prog), "pointwise_kernel"));
+                });
             break;
         case InstrKind::Gemm:
             kernel_ = g_tile_kernels.get_or_insert(tuning::key() + "mm:" + sg_.cache_key(), [&] {
@@ -218,6 +240,7 @@ void Instr::precompile() const {
 }
 
 void Instr::execute(const std::function<void*(NodeId)>& storage, hipStream_t stream) const {
+    if (absorbed_) return;  // the instruction that carries it has done the work
     precompile();
     if (kind_ == InstrKind::Permute) {
         permute_->execute(storage(sg_.inputs()[0]), storage(sg_.leafs()[0]), stream);
@@ -539,6 +562,63 @@ std::shared_ptr<const Plan> generate_plan(const std::shared_ptr<const ir::OpGrap
                     }
                 }
             }
+        }
+    }
+
+    // Beyond the reference: a small pointwise instruction that reads column reductions of a large pointwise instruction
+    // (a batch norm's per-channel arithmetic behind its sums) rides on the launch that folds those reductions instead of
+    // being a launch of its own, when everything else it reads exists by then. The plan keeps both instructions where
+    // they are; the large one carries the small one (Instr::carry).
+    if (rematerialize() && !tuning::get("HELIUM_HIP_NO_CARRY")) {
+        std::map<NodeId, std::pair<size_t, size_t>> made_at;  // leaf -> (step, position in the step)
+        size_t carried_count = 0;
+        std::map<std::string, int> why;
+        for (size_t i = 0; i < plan->steps.size(); i++)
+            for (size_t j = 0; j < plan->steps[i].instrs.size(); j++)
+                for (NodeId leaf : plan->steps[i].instrs[j]->outputs()) made_at[leaf] = {i, j};
+        for (size_t i2 = 0; i2 < plan->steps.size(); i2++) {
+            for (auto& small : plan->steps[i2].instrs) {
+                if (small->kind() != InstrKind::Pointwise || small->carried() || small->absorbed()) continue;
+                bool is_small = true;
+                for (NodeId n : small->subgraph().nodes()) is_small = is_small && ir::num_elements(g->get(n).desc.shape) <= (1 << 16);
+                if (!is_small) continue;
+                // the producer that runs last must be the one whose reductions are read (the others are done before it: earlier
+                // steps, or earlier in a step that then runs in order)
+                bool have = false, reads_reduction = false;
+                std::pair<size_t, size_t> last{0, 0};
+                for (NodeId in : small->inputs()) {
+                    auto it = made_at.find(in);
+                    if (it == made_at.end()) continue;  // an input of the graph
+                    if (!have || it->second > last) last = it->second;
+                    have = true;
+                }
+                if (!have || last.first >= i2) { why["no producer before"]++; continue; }
+                Instr& large = *plan->steps[last.first].instrs[last.second];
+                if (large.kind() != InstrKind::Pointwise || large.carried() || large.absorbed()) { why[large.kind() != InstrKind::Pointwise ? "last producer is a product" : "last producer taken"]++; continue; }
+                bool same_step = false;  // another producer in the large one's step (ahead of it, `last` being the last)
+                for (NodeId in : small->inputs()) {
+                    auto it = made_at.find(in);
+                    if (it == made_at.end()) continue;
+                    if (it->second == last) reads_reduction = reads_reduction || g->get(in).op.kind == ir::OpKind::Reduce;
+                    else same_step = same_step || it->second.first == last.first;
+                }
+                if (!reads_reduction) { why["reads no reduction of it"]++; continue; }
+                try {
+                    tp::Program prog = tp::lower_pointwise(large.subgraph());
+                    if (!tp::attach_post(&prog, tp::lower_pointwise(small->subgraph()))) { why["does not attach"]++; continue; }
+                    if (!tp::emit_pointwise(prog, "pointwise_kernel").post_carried) { why["no fold launch"]++; continue; }
+                } catch (const Error&) {
+                    continue;
+                }
+                large.carry(small);
+                if (same_step) plan->steps[last.first].in_order = true;
+                carried_count++;
+            }
+        }
+        if (getenv("HELIUM_HIP_PLAN_DEBUG") && carried_count) {
+            fprintf(stderr, "[plan] %zu small instructions ride on fold launches", carried_count);
+            for (auto& kv : why) fprintf(stderr, "; %s: %d", kv.first.c_str(), kv.second);
+            fprintf(stderr, "\n");
         }
     }
 

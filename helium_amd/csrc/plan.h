@@ -36,13 +36,34 @@ public:
     void precompile() const;
     bool compiled() const {
         std::lock_guard<std::mutex> lk(mu_);
-        return kernel_ || permute_;
+        return kernel_ || permute_ || absorbed_;
     }
     // execute (instr.rs:27-42): `storage(node)` returns the device address of a tensor.
     void execute(const std::function<void*(NodeId)>& storage, hipStream_t stream) const;
     std::string describe(bool origins = true) const;  // origins: name nodes by OpGraph::origin
 
+    // Beyond the reference: `small` (a pointwise instruction over the columns of this instruction's column reductions:
+    // the per-channel arithmetic behind a batch norm's sums) is evaluated by the launch that folds those reductions.
+    // It stays in the plan where it was and launches nothing; this instruction's execution needs its inputs and
+    // writes its outputs as well.
+    void carry(const std::shared_ptr<Instr>& small) {
+        carried_ = small;
+        small->absorbed_ = true;
+    }
+    const std::shared_ptr<Instr>& carried() const { return carried_; }
+    bool absorbed() const { return absorbed_; }
+    // The compiled kernel (compiling it if need be); null for a permute instruction and an absorbed one.
+    std::shared_ptr<KernelBase> kernel() const {
+        precompile();
+        std::lock_guard<std::mutex> lk(mu_);
+        return kernel_;
+    }
+    std::vector<NodeId> all_inputs() const;   // inputs() plus what the carried instruction reads from elsewhere
+    std::vector<NodeId> all_outputs() const;  // outputs() plus the carried instruction's
+
 private:
+    std::shared_ptr<Instr> carried_;
+    bool absorbed_ = false;
     InstrKind kind_;
     ir::OpSubgraph sg_;
     mutable std::shared_ptr<KernelBase> kernel_;   // Gemm / Pointwise
@@ -59,6 +80,9 @@ Instr make_instr_for_op(const std::shared_ptr<const ir::OpGraph>& g, NodeId node
 struct Step {
     std::vector<std::shared_ptr<Instr>> instrs;
     std::vector<NodeId> tensors_to_release;
+    // The instructions must run one after the other, in this order: one of them carries an instruction that reads what
+    // an earlier one of the same step writes.
+    bool in_order = false;
 };
 struct Plan {
     std::vector<Step> steps;

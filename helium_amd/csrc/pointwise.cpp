@@ -73,6 +73,7 @@ TileKernel::~TileKernel() { scratch_.release(); }
 
 TileKernel::TileKernel(tp::Program prog, const std::string& entry) : prog_(std::move(prog)) {
     launch_ = tp::emit_pointwise(prog_, entry);
+    HE_REQUIRE(!prog_.post || launch_.post_carried, HE_ERR_INTERNAL, "the program's carried part has no fold launch to ride on");
     if (launch_.grid > 0) kernel_.reset(new JitKernel(launch_.source, launch_.entry, launch_.options));
     if (launch_.grid > 0 && launch_.finalize_grid > 0)
         finalize_.reset(new JitKernel(launch_.source, launch_.finalize_entry, launch_.options));

@@ -5,6 +5,8 @@
 // instruction (helium/src/cuda/instr/pointwise/jit.rs), the anchor-less "auxiliary" fusions and the epilogue of
 // the fused GEMM (helium-playground/src/kernel_generator.rs), which differ only in the loop that drives it.
 #pragma once
+#include <map>
+#include <memory>
 #include <string>
 #include <vector>
 
@@ -83,6 +85,11 @@ struct Program {
     std::vector<Arg> args;
     bool fast_math = false;   // GEMM epilogues use the fast intrinsics (helium-kernel-generator/src/pointwise.rs:53-98)
     int acc_expr = -1;        // id of the Acc expression when the program is a GEMM epilogue
+    // A second, small program over [columns] that the launch which folds this program's column reductions evaluates once
+    // per column (the per-channel arithmetic behind a batch norm's sums, which would otherwise be a launch of its own):
+    // its Loads of arguments that are column reductions of this program read the folded values, everything else comes
+    // from memory. Its argument indices refer to this program's `args`. Set by attach_post.
+    std::shared_ptr<const Program> post;
 
     int64_t N() const { return dims.empty() ? 1 : dims.back(); }
     int64_t M() const { return dims.size() >= 2 ? dims[dims.size() - 2] : 1; }
@@ -117,6 +124,11 @@ Program lower_epilogue(const fir::OpGraph& g, fir::OpNode anchor);
 // `transposed`: the same values iterated as [batch, cols, rows] (vector accesses then run along the value's rows).
 Program lower_operand(const fir::OpGraph& g, fir::OpNode value, int* root_expr, bool transposed = false);
 
+// Makes `post` (a program over the columns of main's column reductions: no reductions, Bool values or index maps of its
+// own) ride on the launch that folds them: its arguments are merged into main->args (shared tensors once, the rest
+// appended) and main->post is set. False, with *main untouched, when it cannot.
+bool attach_post(Program* main, const Program& post);
+
 // ---- emission -----------------------------------------------------------------------------------------------
 struct PointwiseLaunch {
     std::string source, entry;
@@ -134,6 +146,9 @@ struct PointwiseLaunch {
     uint32_t finalize_grid = 0;
     std::vector<std::string> options;
     std::string describe;
+    // Whether the program's `post` is evaluated by the fold launch. False (and `post` ignored) when the column reductions
+    // it reads do not all fold in a second launch over the same partial blocks.
+    bool post_carried = false;
 };
 PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry);
 
@@ -154,6 +169,9 @@ struct EmitCtx {
     // broadcast along the rows, and what is computed from them alone); their loads are issued only `if (col_ok)`.
     // 2: the others, which read the former from the enclosing scope.
     int row_part = 0;
+    // Loads of these arguments take the given expression (a value the surrounding code holds in a register) instead of
+    // reading memory.
+    const std::map<int, std::string>* arg_values = nullptr;
 };
 // Per expression: whether its value ignores the row coordinate `m`.
 std::vector<char> row_invariant_exprs(const Program& p);

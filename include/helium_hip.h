@@ -311,6 +311,13 @@ int he_plan_num_steps(he_plan_t plan, int* steps);
 const char* he_plan_describe(he_plan_t plan);
 /* The same text with the node ids of the graph he_plan_graph returns. */
 const char* he_plan_describe_planned(he_plan_t plan);
+/* The compiled kernel of instruction `index` of the plan (instructions counted in the order he_plan_describe lists them),
+ * for inspection and tests: its arguments name nodes of the graph he_plan_graph returns. An instruction whose kernel also
+ * does the work of a later, small one (the per-channel arithmetic behind a batch norm's sums rides on the launch that
+ * folds them) lists that one's tensors among its arguments; the later one, like a permute instruction, has no kernel of
+ * this kind and gives HE_ERR_INVALID. The handle shares the kernel with the plan; destroy it like any other. No
+ * counterpart in the reference (its instructions are not inspectable). */
+int he_plan_instruction_kernel(he_plan_t plan, int index, he_tile_kernel_t* kernel);
 /* Compiles the kernels of every instruction of the plan, in parallel, into the kernel caches: what begin_execute does
  * on first sight of a plan (cuda.rs:98-139, parallel_compile_kernels :262-270). Needs no device. */
 int he_plan_precompile(he_plan_t plan);

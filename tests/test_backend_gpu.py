@@ -277,15 +277,16 @@ def test_four_threads_execute_concurrently(gpu):
     assert s["plan_cache_misses"] == misses_before and s["pool_reuses"] > 0
 
 
-@pytest.mark.parametrize("fold", [1, 0], ids=["statistics_without_permute", "reference_grouping"])
-def test_batch_norm_train_step(gpu, fold):
+@pytest.mark.parametrize("fold, shape", [(1, [8, 36, 36, 128]), (0, [8, 36, 36, 128]), (1, [16, 48, 48, 128])],
+                         ids=["statistics_without_permute", "reference_grouping", "channel_arithmetic_rides_on_the_fold_launch"])
+def test_batch_norm_train_step(gpu, fold, shape):
     """BatchNorm2d::forward in Train mode + Relu (helium/src/modules/batch_norm.rs:32-72) above the 1M-element
     SwapDims threshold, planned both ways: with the transposition folded into the statistics kernel and as the
-    reference plans it (permute, then two reductions)."""
+    reference plans it (permute, then two reductions). Above 2M elements (the third case: 4.7M) the statistics fold in a
+    second launch, which then also does the per-channel arithmetic behind them."""
     from harness import frontend
     from helium_amd.backend import OPT_FOLD_SWAP_INTO_REDUCE, set_option
 
-    shape = [8, 36, 36, 128]  # 1.3M elements
     g = ha.ir.OpGraph()
     rec = frontend.Recorder(g)
     x = g.new_input(shape, "bf16")
@@ -306,6 +307,11 @@ def test_batch_norm_train_step(gpu, fold):
         set_option(OPT_FOLD_SWAP_INTO_REDUCE, 1)
     kinds = [k for instrs, _ in steps for k, _ in instrs]
     assert ("permute" in kinds) == (fold == 0), steps
+    if int(np.prod(shape)) > (1 << 21):
+        plan = Plan(g)
+        assert "carries=" in plan.kernel(0).description, plan.kernel(0).description
+        with pytest.raises(ha.HeliumError, match="launches nothing"):
+            plan.kernel(1)
     want = oracle_ir.plan_outputs(g.nodes, host, steps)
     _, desc = oracle_ir.evaluate(g.nodes, host)
     for o in want:
