@@ -1181,27 +1181,33 @@ def make_workloads():
 SETTLE_LAUNCHES = 200  # launches after which the device's clock has settled (see --warmup's comment in main)
 
 
-def time_workload(wl, stream, steps, warmup):
+def time_workload(wl, stream, steps, warmup, batches=1):
     """Returns (ms_per_step from HIP events on the launch stream, wall ms per step). When fewer warm-up steps are asked
-    for than the clock needs to settle, the difference is run first, untimed like the warm-up itself."""
+    for than the clock needs to settle, the difference is run first, untimed like the warm-up itself. `batches` > 1:
+    that many timed regions of `steps` steps each, one after the other, and the median of them (a region of twenty
+    launches of a few microseconds is at the mercy of one hiccup of the host)."""
     import helium_amd as ha
 
     for i in range(max(0, SETTLE_LAUNCHES - warmup)):
         wl.step(stream, i)
     for i in range(warmup):
         wl.step(stream, i)
-    stream.synchronize()
-    ha.device.synchronize()
-    start, stop = ha.Event(), ha.Event()
-    t0 = time.perf_counter()
-    start.record(stream)
-    for i in range(steps):
-        wl.step(stream, warmup + i)
-    stop.record(stream)
-    stop.synchronize()
-    ha.device.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    return start.elapsed_ms(stop) / steps, wall_ms
+    results = []
+    for b in range(batches):
+        stream.synchronize()
+        ha.device.synchronize()
+        start, stop = ha.Event(), ha.Event()
+        t0 = time.perf_counter()
+        start.record(stream)
+        for i in range(steps):
+            wl.step(stream, warmup + b * steps + i)
+        stop.record(stream)
+        stop.synchronize()
+        ha.device.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+        results.append((start.elapsed_ms(stop) / steps, wall_ms))
+    results.sort(key=lambda r: (r[1] if getattr(wl, "wall_timed", False) else r[0]))
+    return results[len(results) // 2]
 
 
 def roofline(wl, ms):
@@ -1256,7 +1262,10 @@ def main():
         wl.step(stream, 0)
         stream.synchronize()
         parity = wl.check()
-        ms, wall = time_workload(wl, stream, args.steps, args.warmup)
+        # the headline is timed over exactly --steps steps; the other workloads, when --steps is small, over five such
+        # regions of which the median is reported
+        batches = 1 if name == headline or args.steps >= 100 else 5
+        ms, wall = time_workload(wl, stream, args.steps, args.warmup, batches)
         if getattr(wl, "wall_timed", False):
             ms = wall  # launched on the executor's own streams: only the host clock brackets them
         rl = roofline(wl, ms)
