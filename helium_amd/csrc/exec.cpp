@@ -561,8 +561,9 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
             const int top = atoi(getenv("HELIUM_HIP_INSTR_TIMING"));
             for (int i = 0; i < top && i < (int)instr_times.size(); i++) {
                 const std::string d = instr_times[i].instr->describe();
-                fprintf(stderr, "  #%-4zu %8.1f us %8.1f MB %6.2f TB/s  %s\n", instr_times[i].order, instr_times[i].us, instr_times[i].bytes / 1e6,
-                        instr_times[i].bytes / instr_times[i].us / 1e6, d.substr(0, 200).c_str());
+                const auto k = instr_times[i].instr->kernel();
+                fprintf(stderr, "  #%-4zu %8.1f us %8.1f MB %6.2f TB/s  %s  %s\n", instr_times[i].order, instr_times[i].us, instr_times[i].bytes / 1e6,
+                        instr_times[i].bytes / instr_times[i].us / 1e6, d.substr(0, 60).c_str(), k ? k->describe().substr(0, 260).c_str() : "");
             }
         }
     }

@@ -819,6 +819,27 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
             t.wm = t.wn = 2;
             if (pr.split_k > 1 && pr.N >= 256) t.wn = 4;
             small = true;
+        } else if (!f32 && pr.M <= 128 && pr.M > 64 && pr.N >= 512 && pr.conv_b.on && pr.conv_b.C % epc == 0 && pr.split_k > 1 &&
+                   !tuning::get("HELIUM_HIP_GEMM_NO_WIDE_CONV_TILES")) {
+            // a filter gradient with 128 output channels: tiles as tall as M and 256 wide, so that the image's pixels
+            // travel to half as many workgroups (plan.cpp deals the k range to one workgroup per CU)
+            t.bm = 128;
+            t.bn = 256;
+            t.wm = 2;
+            t.wn = 4;
+            small = true;
+        } else if (!f32 && pr.conv_a.on && pr.conv_a.C % epc == 0 && pr.N >= 256 && pr.N % 256 == 0 && pr.split_k == 1 &&
+                   ((pr.M + 255) / 256) * (pr.N / 256) * pr.batch < 128 && ((pr.M + 127) / 128) * (pr.N / 256) * pr.batch >= 192 &&
+                   !tuning::get("HELIUM_HIP_GEMM_NO_WIDE_CONV_TILES")) {
+            // a convolution (or data gradient) into a multiple of 256 channels whose 256x256 tiles would leave half the chip
+            // idle while 128x256 tiles fill three quarters of it or more: the filter travels to half as many workgroups
+            // as with 128x128 tiles (the 14x14x256 layer at batch 128: forward 45.4 -> 41.4 us, data gradient 46.1 -> 42.5;
+            // the 7x7x512 layer has 98 such tiles and loses: 47.8 -> 65.2)
+            t.bm = 128;
+            t.bn = 256;
+            t.wm = 2;
+            t.wn = 4;
+            small = true;
         } else
         // Smaller problems take smaller tiles so that every CU gets work.
         // (a split k range multiplies the workgroups: the filter gradients of 256 and 512 channels keep the large tile,

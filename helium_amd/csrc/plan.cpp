@@ -1066,6 +1066,22 @@ int filter_gradient_split_k(const GemmProblem& pr, bool element_gather) {
     // the 56x56x64 layer 102 -> 87 us; few shares are rounded up: 3 instead of 4 leave a quarter of the chip idle)
     const int64_t shares = 512 / tiles >= 32 ? 512 / tiles : (512 + tiles - 1) / tiles;
     int split = (int)std::max<int64_t>(1, std::min<int64_t>({shares, k_tiles / 4, 1024}));
+    // Measured at batch 128 on the resnet-train layers (us per graph, fold launch included), and kept where batch 64 and the
+    // stride-2 layers do not lose:
+    //  - 128 output channels take 128x256 tiles (gemm.cpp), one workgroup per CU: the 28x28x128 layer 73.7 -> 61.8
+    //    (5 tiles x 50 shares against 9 x 56 of 128x128), at batch 64 45.8 -> 43.6, the stride-2 56x56x64 -> 128 layer 50.8 -> 44.5;
+    //  - 512 output channels keep 256x256 tiles, whose count, not that of 128x128 tiles, decides the shares as long as a
+    //    share keeps 12 k-tiles: the 7x7x512 layer 36 x 4 = 144 workgroups 77.4 us, 36 x 7 = 252 workgroups 70.3.
+    if (tuning::get("HELIUM_HIP_GEMM_NO_WIDE_CONV_TILES")) {
+        // (the shares as they were, for comparison)
+    } else if (!element_gather && pr.M > 64 && pr.M <= 128 && pr.N >= 512) {
+        const int64_t wide = (pr.N + 255) / 256;
+        split = (int)std::max<int64_t>(1, std::min<int64_t>({256 / wide, k_tiles / 4, 1024}));
+    } else if (!element_gather && pr.M >= 512 && pr.N >= 512) {
+        const int64_t large = ((pr.M + 255) / 256) * ((pr.N + 255) / 256);
+        const int64_t s256 = std::min<int64_t>(256 / large, k_tiles / 12);
+        if (s256 * large >= 192) split = (int)s256;
+    }
     // (an image whose channels do not fill 16-byte chunks is gathered element by element, by 32x64 tiles of two waves: six
     // workgroups per CU, one round of them over the chip)
     if (element_gather && pr.M <= 32 && pr.M > 16 && pr.N >= 128)

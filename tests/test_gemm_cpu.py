@@ -450,6 +450,8 @@ BWD_FILTER_CASES = [
     ("thirty_two_rows_tile_direct_loads", (2, 12, 12, 16), 32, (3, 3), "bf16", (1, 1), (1, 1), "same", "32,128,64,1,4"),
     ("five_channels_3x3_f16", (1, 7, 9, 5), 8, (3, 3), "f16", (1, 1), (1, 1), "same", "64,64,64,2,2"),
     ("three_channels_f32_full", (1, 6, 5, 3), 8, (3, 3), "f32", (1, 1), (1, 2), "full", "64,64,32,2,2"),
+    # 128 output channels: tiles as tall as M and 256 wide (what the generator picks for this shape when the k range is split)
+    ("tall_wide_tile_128_channels", (2, 16, 16, 64), 128, (3, 3), "bf16", (1, 1), (1, 1), "same", "128,256,64,2,4"),
 ]
 
 
@@ -481,6 +483,17 @@ def test_conv_backward_filter_on_cpu(name, image, oc, kernel, dtype, stride, dil
     tol = 1e-4 if dtype == "f32" else 2e-2
     assert np.abs(got[dw] - want).max() <= tol * max(1.0, np.abs(want).max()), (k.description, np.abs(got[dw] - want).max())
     assert k.description.startswith("repacked") == repacks(image, kernel, dtype, stride, dilation), k.description
+
+
+def test_filter_gradient_of_128_channels_takes_tall_wide_tiles():
+    """Without an override: a [128 x 576] gradient over 512 pixels gets 128x256 tiles and a split k range."""
+    g = ha.ir.OpGraph()
+    params = {"in_channels": 64, "out_channels": 128, "kernel_size": [3, 3], "stride": [1, 1], "dilation": [1, 1], "padding_mode": "same"}
+    dy = g.new_input([2, 16, 16, 128], "bf16"); x = g.new_input([2, 16, 16, 64], "bf16")
+    dw = g.conv_backward_filter(dy, x, params)
+    g.new_output(dw)
+    d = ha.backend.matmul_kernel(g, [dw]).description
+    assert "tile=128x256x64" in d and "split_k=2" in d, d
 
 
 def test_conv_backward_filter_with_many_partial_tiles_on_cpu(monkeypatch):
