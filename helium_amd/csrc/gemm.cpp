@@ -956,7 +956,10 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
         // With more than one workgroup per CU (a split k range) the LDS is better spent on a second and third
         // workgroup, whose loads hide each other's waits (filter gradient of a 64-channel layer: 66 -> 56 us).
         const int64_t workgroups = ((pr.M + t.bm - 1) / t.bm) * ((pr.N + t.bn - 1) / t.bn) * pr.batch * pr.split_k;
-        while (workgroups <= 256 && t.stages < 4 && (t.stages + 1) * (t.bm + t.bn) * t.bk * esz <= 128 * 1024) t.stages++;
+        // (not for a data gradient's gather: at batch 128 the 7x7x512 layer takes 54.2 us with four stages, 49.7 with three,
+        // 48.9 with two, the 14x14x256 layer at batch 64 29.3 / 27.5 / 27.8; the forward gather does not care)
+        const bool deeper = !(pr.conv_a.on && pr.conv_a.bwd);
+        while (deeper && workgroups <= 256 && t.stages < 4 && (t.stages + 1) * (t.bm + t.bn) * t.bk * esz <= 128 * 1024) t.stages++;
     }
     // All direct loads of the next tile are issued at the start of a tile's MFMAs (the round trip needs the whole
     // tile to hide); HELIUM_HIP_GEMM_ISSUE=0 spreads them over the k-steps instead.
