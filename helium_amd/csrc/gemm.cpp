@@ -381,6 +381,7 @@ void fused_matmul(KERNEL_PARAMS) {
     constexpr u32 KT = KT_ALL;
 #endif
     const u32 m0 = tile_m * BM, n0 = tile_n * BN;
+    EPILOGUE_EARLY
     // Optional rotation of the k loop per workgroup (tuning knob, off by default: workgroups that share an A or B
     // panel read the same k range at the same time, which is what lets them share it through L2).
     const u32 k_shift = KT ? (STAGGER_EXPR) % KT : 0u;
@@ -1150,7 +1151,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     else emit_fetch("b", pr.op_b, pr.root_b, pr.map_b, raw_b, nvb, "GK", "GN", pr.K % t.bk == 0 && pr.N % t.bn == 0);
 
     // epilogue pieces
-    std::ostringstream setup, body, finish, prefetch;
+    std::ostringstream setup, body, finish, prefetch, early;
     // The tensors an epilogue reads row by row (full-size operands, per-row vectors) are requested EPI_DEPTH steps ahead
     // of the step that uses them, into registers; what does not depend on the row (per-column vectors, constants and
     // what is computed from those alone) is loaded and computed once per wave, ahead of the strips. Left to itself
@@ -1231,9 +1232,11 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
             if (tp::is_uniform_pow(pr.epi, (int)i)) exps.push_back(pr.epi.exprs[pr.epi.exprs[i].b].access.arg);
         std::sort(exps.begin(), exps.end());
         exps.erase(std::unique(exps.begin(), exps.end()), exps.end());
+        // (read ahead of the k-loop: at the head of the epilogue the load's round trip, a microsecond, would stand between
+        // the last k-tile and the first strip of every workgroup)
         if (!exps.empty()) {
-            setup << "bool all_squares = true;\n";
-            for (int a : exps) setup << "all_squares = all_squares && ld_one(a" << a << ") == 2.0f;\n";
+            early << "bool all_squares = true;\n";
+            for (int a : exps) early << "all_squares = all_squares && ld_one(p" << pr.map_e[a] << ") == 2.0f;\n";
         }
         auto element_body = [&](bool squares) {
             std::ostringstream b;
@@ -1471,6 +1474,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     splice("EPILOGUE_PREFETCH", prefetch.str());
     splice("EPILOGUE_BODY", body.str());
     splice("EPILOGUE_FINISH", finish.str());
+    splice("EPILOGUE_EARLY", early.str());
     s << body_text;
     if (pr.split_k > 1) {
         // second launch of a split-k product: the output element is the sum of its partials, rounded once
