@@ -334,7 +334,7 @@ int pick_nv(const Program& p, int max_bytes) {
 }
 
 bool attach_post(Program* main, const Program& post) {
-    if (main->post || main->acc_expr >= 0 || post.acc_expr >= 0 || post.post || post.dims.empty()) return false;
+    if (main->post || post.acc_expr >= 0 || post.post || post.dims.empty()) return false;
     // one thread per column evaluates it: a program over [columns] and nothing else
     const int64_t cols = post.N();
     if (ir::num_elements(post.dims) != cols || cols != main->N() || post.exprs.empty() || post.outs.empty()) return false;

@@ -916,7 +916,9 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     // per graph). A large product is better off with the second launch: its workgroups all end together, the tickets and
     // the loads of the partials are three dependent round trips at the very end of the kernel, and a 4096^3 product with
     // the README's epilogue took 155 us this way against 141. Row sums keep the second launch as well.
-    bool fold_in_kernel = !reds.empty() && pr.split_k == 1 && tiles_m * tiles_n * pr.batch <= 64 && !tuning::get("HELIUM_HIP_GEMM_NO_TICKET_FOLD");
+    // (a program that rides on the fold launch needs that launch)
+    bool fold_in_kernel = !reds.empty() && pr.split_k == 1 && tiles_m * tiles_n * pr.batch <= 64 && !pr.epi.post &&
+                          !tuning::get("HELIUM_HIP_GEMM_NO_TICKET_FOLD");
     for (auto& r : reds) {
         const tp::Out& o = pr.epi.outs[r.out];
         fold_in_kernel = fold_in_kernel && o.fold_m && (!o.fold_n || r.parts <= 4096);
@@ -1510,10 +1512,61 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
              "for (u32 p = pg; p < parts; p += PG) acc += src[(size_t)p * inner];\n}\n"
              "part[e * PG + pg] = acc;\n__syncthreads();\n"
              "if (pg == 0 && j < n) {\nfloat r = 0.0f;\nfor (int q = 0; q < PG; q++) r += part[e * PG + q];\nout[j] = r * scale;\n}\n}\n";
+        // The column sums that a carried program reads (tp::Program::post: the per-channel arithmetic behind a batch norm's
+        // statistics) are folded by the same blocks, EB columns each, and the threads that end up with a column's sums
+        // evaluate the program for that column. The kernel then takes every argument of the epilogue program.
+        std::vector<size_t> carried;  // indices into reds
+        if (pr.epi.post) {
+            std::vector<char> read(pr.epi.args.size(), 0);
+            for (const tp::Expr& e : pr.epi.post->exprs)
+                if (e.kind == tp::Expr::Load) read[e.access.arg] = 1;
+            for (size_t i = 0; i < reds.size(); i++) {
+                const tp::Out& o = pr.epi.outs[reds[i].out];
+                if (!read[o.arg]) continue;
+                HE_REQUIRE(o.fold_m && !o.fold_n && pr.batch == 1, HE_ERR_INTERNAL, "a carried program reads column sums of an unbatched product");
+                carried.push_back(i);
+            }
+            HE_REQUIRE(!carried.empty(), HE_ERR_INTERNAL, "the carried program reads no reduction of this product");
+            reduce_all_args_ = true;
+        }
         s << "extern \"C\" __global__ __launch_bounds__(256) void fused_matmul_reduce(const float* __restrict__ ws";
-        for (size_t i = 0; i < reds.size(); i++) s << ", float* __restrict__ o" << i;
+        if (reduce_all_args_) {
+            for (size_t a = 0; a < pr.epi.args.size(); a++)
+                s << ", " << (pr.epi.args[a].is_output ? "" : "const ") << tp::c_type(pr.epi.args[a].dtype) << "* __restrict__ a" << a;
+        } else {
+            for (size_t i = 0; i < reds.size(); i++) s << ", float* __restrict__ o" << i;
+        }
         s << ") {\n__shared__ float part[256];\nu32 blk = blockIdx.x;\n";
+        if (!carried.empty()) {
+            const RedOut& r0 = reds[carried[0]];
+            int eb = 16;
+            while (eb > 1 && (r0.elems < eb || (r0.elems / eb < 64 && r0.parts > 256 / eb))) eb /= 2;
+            const int pg = 256 / eb;
+            const uint32_t blocks = (uint32_t)((r0.elems + eb - 1) / eb);
+            s << "if (blk < " << blocks << "u) {\nconst u32 tid = threadIdx.x, e = tid % " << eb << "u, pg = tid / " << eb << "u, j = blk * " << eb << "u + e;\n";
+            std::map<int, std::string> values;
+            for (size_t i : carried) s << "float red" << i << " = 0.0f, acc" << i << " = 0.0f;\n";
+            s << "if (j < " << r0.elems << "u) {\n#pragma unroll 8\nfor (u32 p = pg; p < " << r0.parts << "u; p += " << pg << "u) {\n";
+            for (size_t i : carried) s << "acc" << i << " += ws[" << reds[i].off << "ull + (size_t)p * " << reds[i].inner << "u + j];\n";
+            s << "}\n}\n";
+            for (size_t i : carried) {
+                const tp::Out& o = pr.epi.outs[reds[i].out];
+                char scale[64];
+                snprintf(scale, sizeof scale, "%.9ef", o.rop == tp::ROp::Mean ? (float)o.mean_scale : 1.0f);
+                s << "__syncthreads();\npart[pg * " << eb << "u + e] = acc" << i << ";\n__syncthreads();\nif (pg == 0 && j < " << r0.elems << "u) {\nfloat r = 0.0f;\nfor (int q = 0; q < "
+                  << pg << "; q++) r += part[q * " << eb << " + e];\nred" << i << " = store_and_keep(a" << o.arg << " + j, r * " << scale << ");\n}\n";
+                values[o.arg] = "red" + std::to_string(i);
+            }
+            tp::EmitCtx cx;
+            cx.nv = 1;
+            cx.arg_values = &values;
+            s << "if (pg == 0 && j < " << r0.elems << "u) {\nconst u32 n0 = j, m = 0u; (void)m;\n" << tp::emit_exprs(*pr.epi.post, cx);
+            for (const tp::Out& o : pr.epi.post->outs) s << "st_one(a" << o.arg << " + n0, e" << o.expr << "[0]);\n";
+            s << "}\nreturn;\n}\nblk -= " << blocks << "u;\n";
+            reduce_grid_ += blocks;
+        }
         for (size_t i = 0; i < reds.size(); i++) {
+            if (std::find(carried.begin(), carried.end(), i) != carried.end()) continue;
             const RedOut& r = reds[i];
             const tp::Out& o = pr.epi.outs[r.out];
             // elements per workgroup: 16 where there are many elements with few partials each, fewer (more threads per
@@ -1523,7 +1576,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
             const uint32_t blocks = (uint32_t)((r.elems + eb - 1) / eb);
             char scale[64];
             snprintf(scale, sizeof scale, "%.9ef", o.rop == tp::ROp::Mean ? (float)o.mean_scale : 1.0f);
-            s << "if (blk < " << blocks << "u) { fold_partials<" << eb << ", " << (r.inner == 1 ? "true" : "false") << ">(ws + " << r.off << "ull, o" << i << ", "
+            s << "if (blk < " << blocks << "u) { fold_partials<" << eb << ", " << (r.inner == 1 ? "true" : "false") << ">(ws + " << r.off << "ull, " << (reduce_all_args_ ? "(float*)a" + std::to_string(o.arg) : "o" + std::to_string(i)) << ", "
               << r.elems << "u, " << r.parts << "u, " << r.inner << "u, " << scale << ", blk, part); return; }\nblk -= " << blocks << "u;\n";
             reduce_grid_ += blocks;
         }
@@ -1539,7 +1592,7 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
     for (auto& r : reds) reduce_outs_.push_back(pr.map_e[pr.epi.outs[r.out].arg]);
     reduce_floats_ = red_floats;
     std::string reduce_args;
-    for (int a : reduce_outs_) reduce_args += (reduce_args.empty() ? "" : ",") + std::to_string(a);
+    for (int a : reduce_all_args_ ? pr.map_e : reduce_outs_) reduce_args += (reduce_args.empty() ? "" : ",") + std::to_string(a);
     describe_ = strfmt("gemm [%lld,%lld,%lld]x[%lld] tile=%dx%dx%d stages=%d waves=%dx%d threads=%d grid=%ux%u rawA=%d rawB=%d NVA=%d NVB=%d NVE=%d "
                        "direct=%d%d mma=%s epilogue_exprs=%zu outs=%zu split_k=%d reduce_ws=%llu reduce_grid=%u reduce_args=[%s] reduce_counters=%llu",
                        (long long)pr.batch, (long long)pr.M, (long long)pr.K, (long long)pr.N, t.bm, t.bn, t.bk, t.stages, t.wm, t.wn, threads,
@@ -1547,7 +1600,9 @@ GemmKernel::GemmKernel(GemmProblem prob) : prob_(std::move(prob)) {
                        pr.epi.outs.size(), pr.split_k, (unsigned long long)reduce_floats_, reduce_grid_, reduce_args.c_str(), (unsigned long long)reduce_counters_);
     kernel_.reset(new JitKernel(source_, "fused_matmul", {"-ffp-contract=fast", "-munsafe-fp-atomics"}));
     if (pr.split_k > 1) finalize_.reset(new JitKernel(source_, "fused_matmul_finalize", {"-ffp-contract=fast", "-munsafe-fp-atomics"}));
-    if (reduce_grid_) reduce_.reset(new JitKernel(source_, "fused_matmul_reduce", {"-ffp-contract=fast"}));
+    if (pr.epi.post) describe_ += strfmt(" carries=%zuexprs/%zuouts", pr.epi.post->exprs.size(), pr.epi.post->outs.size());
+    // (a carried program is a pointwise instruction's: no contraction into fused multiply-adds, as when it runs alone)
+    if (reduce_grid_) reduce_.reset(new JitKernel(source_, "fused_matmul_reduce", {reduce_all_args_ ? "-ffp-contract=off" : "-ffp-contract=fast"}));
 }
 
 GemmKernel::~GemmKernel() { scratch_.release(); }
@@ -1617,7 +1672,10 @@ void GemmKernel::run(void* const* ptrs, hipStream_t stream, float* ws, uint32_t*
     }
     if (reduce_) {
         std::vector<void*> rh{ws};
-        for (int a : reduce_outs_) rh.push_back(ptrs[a]);
+        if (reduce_all_args_)
+            for (int a : prob_.map_e) rh.push_back(ptrs[a]);
+        else
+            for (int a : reduce_outs_) rh.push_back(ptrs[a]);
         std::vector<void*> rargv(rh.size());
         for (size_t i = 0; i < rh.size(); i++) rargv[i] = &rh[i];
         const uint32_t rgrid[3] = {reduce_grid_, 1, 1}, rblock[3] = {256, 1, 1};

@@ -169,6 +169,7 @@ private:
     uint64_t reduce_floats_ = 0;
     uint64_t reduce_counters_ = 0;  // arrival counters of reductions that fold inside the kernel (no reduce_ launch then)
     std::vector<int> reduce_outs_;  // kernel arguments the reduce launch writes, in its parameter order
+    bool reduce_all_args_ = false;  // the reduce launch carries a program and takes every epilogue argument instead
     ReduceScratch scratch_;
 };
 

@@ -43,7 +43,8 @@ bool enumerate_swaps(const ir::OpSubgraph& sg, std::vector<std::pair<int, int>>*
     return true;
 }
 
-std::unique_ptr<KernelBase> make_gemm_kernel(const ir::OpSubgraph& sg);
+std::unique_ptr<KernelBase> make_gemm_kernel(const ir::OpSubgraph& sg, const ir::OpSubgraph* carried);
+bool gemm_can_carry(const ir::OpSubgraph& large, const ir::OpSubgraph& small);
 namespace {
 std::atomic<bool> g_fuse_matmul_epilogue{true};
 std::atomic<bool> g_fold_swap_into_reduce{true};
@@ -219,9 +220,9 @@ void Instr::precompile() const {
                 });
             break;
         case InstrKind::Gemm:
-            kernel_ = g_tile_kernels.get_or_insert(tuning::key() + "mm:" + sg_.cache_key(), [&] {
-                return std::shared_ptr<KernelBase>(make_gemm_kernel(sg_));
-            });
+            kernel_ = g_tile_kernels.get_or_insert(
+                tuning::key() + "mm:" + sg_.cache_key() + (carried_ ? "+carries:" + carried_->sg_.cache_key() : std::string()),
+                [&] { return std::shared_ptr<KernelBase>(make_gemm_kernel(sg_, carried_ ? &carried_->sg_ : nullptr)); });
             break;
         case InstrKind::Permute: {
             std::vector<std::pair<int, int>> swaps;
@@ -594,7 +595,7 @@ std::shared_ptr<const Plan> generate_plan(const std::shared_ptr<const ir::OpGrap
                 }
                 if (!have || last.first >= i2) { why["no producer before"]++; continue; }
                 Instr& large = *plan->steps[last.first].instrs[last.second];
-                if (large.kind() != InstrKind::Pointwise || large.carried() || large.absorbed()) { why[large.kind() != InstrKind::Pointwise ? "last producer is a product" : "last producer taken"]++; continue; }
+                if (large.kind() == InstrKind::Permute || large.carried() || large.absorbed()) { why["last producer taken"]++; continue; }
                 bool same_step = false;  // another producer in the large one's step (ahead of it, `last` being the last)
                 for (NodeId in : small->inputs()) {
                     auto it = made_at.find(in);
@@ -604,6 +605,13 @@ std::shared_ptr<const Plan> generate_plan(const std::shared_ptr<const ir::OpGrap
                 }
                 if (!reads_reduction) { why["reads no reduction of it"]++; continue; }
                 try {
+                    if (large.kind() == InstrKind::Gemm) {
+                        if (!gemm_can_carry(large.subgraph(), small->subgraph())) { why["does not attach to the product"]++; continue; }
+                        large.carry(small);
+                        if (same_step) plan->steps[last.first].in_order = true;
+                        carried_count++;
+                        continue;
+                    }
                     tp::Program prog = tp::lower_pointwise(large.subgraph());
                     if (!tp::attach_post(&prog, tp::lower_pointwise(small->subgraph()))) { why["does not attach"]++; continue; }
                     if (!tp::emit_pointwise(prog, "pointwise_kernel").post_carried) { why["no fold launch"]++; continue; }
@@ -1143,7 +1151,26 @@ bool over_repacked_image(const GemmProblem& pr, GemmProblem* packed, ConvRepack*
 }
 }  // namespace
 
-std::unique_ptr<KernelBase> make_gemm_kernel(const ir::OpSubgraph& sg) {
+// Whether the launch that folds the epilogue reductions of the product `large` can also evaluate the small pointwise
+// instruction `small` (tp::attach_post): a plain product (no classes of a strided data gradient, no repacked image, a
+// whole k range) whose column sums the small program reads.
+bool gemm_can_carry(const ir::OpSubgraph& large, const ir::OpSubgraph& small) {
+    bool any_empty = false;
+    if (!strided_data_gradient_classes(large, &any_empty).empty()) return false;
+    GemmProblem pr = gemm_problem_from_ir(large);
+    ConvRepack geometry;
+    GemmProblem packed;
+    if (over_repacked_image(pr, &packed, &geometry) || pr.split_k != 1 || pr.batch != 1) return false;
+    return tp::attach_post(&pr.epi, tp::lower_pointwise(small));
+}
+
+std::unique_ptr<KernelBase> make_gemm_kernel(const ir::OpSubgraph& sg, const ir::OpSubgraph* carried) {
+    if (carried) {
+        GemmProblem pr = gemm_problem_from_ir(sg);
+        HE_REQUIRE(tp::attach_post(&pr.epi, tp::lower_pointwise(*carried)), HE_ERR_INTERNAL, "the carried instruction does not fit the fold launch any more");
+        assemble_gemm_args(pr);
+        return std::unique_ptr<KernelBase>(new GemmKernel(std::move(pr)));
+    }
     // The data gradient of a strided convolution is one product per class of pixels (row and column modulo the
     // stride): each multiplies only the taps that reach its pixels.
     bool any_empty = false;

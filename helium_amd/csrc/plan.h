@@ -131,6 +131,6 @@ GemmProblem gemm_problem_from_ir(const ir::OpSubgraph& sg);
 // no tap, so its pixels have to be zeroed.
 std::vector<GemmProblem> strided_data_gradient_classes(const ir::OpSubgraph& sg, bool* any_empty);
 // The kernel of a Gemm instruction: one fused GEMM, or the classes of a strided data gradient one after the other.
-std::unique_ptr<KernelBase> make_gemm_kernel(const ir::OpSubgraph& sg);
+std::unique_ptr<KernelBase> make_gemm_kernel(const ir::OpSubgraph& sg, const ir::OpSubgraph* carried = nullptr);
 
 }  // namespace he::plan

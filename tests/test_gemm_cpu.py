@@ -36,12 +36,14 @@ def launch_gemm(k, bufs):
     res = run_kernel(k.source, "fused_matmul", gx, threads, bufs + [(np.full(ws_floats, np.nan, dtype=np.float32), 2)], grid_y=gy)
     ws, res = res[-1], res[:-1]
     out_args = [i for i, a in enumerate(k.args) if a["is_output"]]
-    # the reduce launch takes the reduction outputs in the order the description lists their kernel arguments
-    listed = re.search(r"reduce_args=\[([\d,]*)\]", k.description).group(1)
-    reduced = [out_args.index(int(i)) for i in listed.split(",")]
-    folded = run_kernel(k.source, "fused_matmul_reduce", reduce_grid, 256, [(ws, 0)] + [(res[j], 1) for j in reduced])
-    for j, r in zip(reduced, folded):
-        res[j] = r
+    # the reduce launch takes the kernel arguments the description lists, in that order: the reduction outputs, or - when
+    # it also evaluates a carried program - every argument of the epilogue, inputs included
+    listed = [int(i) for i in re.search(r"reduce_args=\[([\d,]*)\]", k.description).group(1).split(",")]
+    again = [(res[out_args.index(i)], 2) if k.args[i]["is_output"] else bufs[i] for i in listed]
+    folded = iter(run_kernel(k.source, "fused_matmul_reduce", reduce_grid, 256, [(ws, 0)] + again))
+    for i in listed:
+        if k.args[i]["is_output"]:
+            res[out_args.index(i)] = next(folded)
     return res
 
 

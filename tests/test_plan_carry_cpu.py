@@ -98,3 +98,66 @@ def test_without_the_option_every_instruction_launches_for_itself(monkeypatch):
                 assert "permute" in str(e)
     finally:
         set_option(OPT_REMATERIALIZE, 1)
+
+
+def product_with_statistics(rows, inner, channels, rng):
+    """y = x w with the per-channel sums of y and y*y in the product's epilogue, the arithmetic behind them, and the pass
+    that applies it."""
+    g = ha.ir.OpGraph()
+    inputs = {}
+
+    def inp(shape, dt, values):
+        i = g.new_input(list(shape), dt)
+        inputs[i] = nm.to_storage(np.asarray(values).reshape(shape), dt)
+        return i
+
+    x = inp([rows, inner], "f32", rng.standard_normal(rows * inner) * 0.5)
+    w = inp([inner, channels], "f32", rng.standard_normal(inner * channels) * 0.2)
+    gamma = inp([channels, 1], "f32", rng.uniform(0.5, 2.0, channels))
+    y = g.matmul(x, w, "f32_f32")
+    yt = g.swap_dims(y, 0, 1)
+    s1 = g.reduce(yt, "sum", 1)
+    s2 = g.reduce(g.binary(yt, yt, "mul"), "sum", 1)
+
+    def scalar(value):
+        b, s, host = scalar_tensor(g, value, [channels, 1])
+        inputs[s] = host
+        return b
+
+    mean = g.binary(s1, scalar(1.0 / rows), "mul")
+    ex2 = g.binary(s2, scalar(1.0 / rows), "mul")
+    var = g.binary(ex2, g.unary(g.binary(mean, mean, "mul"), "neg"), "add")
+    inv = g.unary(g.unary(g.binary(var, scalar(1e-3), "add"), "sqrt"), "recip")
+    scale = g.binary(gamma, inv, "mul")
+    z = g.binary(y, broadcast_to(g, g.reshape(scale, [channels]), [channels], [rows, channels]), "mul")
+    g.new_output(z)
+    g.new_output(mean)
+    return g, inputs, dict(y=y, s1=s1, s2=s2, mean=mean)
+
+
+def test_per_channel_arithmetic_rides_on_a_products_fold_launch():
+    import test_gemm_cpu as gemm
+
+    rng = np.random.default_rng(3)
+    g, inputs, names = product_with_statistics(300, 64, 72, rng)
+    g.optimize()
+    plan = Plan(g)
+    instrs = [i for step, _ in plan.planned_steps() for i in step]
+    assert [kind for kind, _ in instrs] == ["gemm", "pointwise", "pointwise"], plan.text
+    pg = plan.graph()
+    origin = {n["id"]: n["origin"] for n in pg.nodes}
+    k = plan.kernel(0)
+    assert k.description.startswith("gemm") and "carries=" in k.description and "reduce_counters=0" in k.description, k.description
+    with pytest.raises(ha.HeliumError, match="launches nothing"):
+        plan.kernel(1)
+    planned_inputs = {n["id"]: inputs[origin[n["id"]]] for n in pg.nodes if n["node"] == "input"}
+    got = gemm._run_one_product(k, planned_inputs)
+    val, _ = oracle_ir.evaluate(g.nodes, inputs)
+    by_id = {n["id"]: n for n in g.nodes}
+    seen = {origin[node] for node in got}
+    assert {names["y"], names["s1"], names["s2"], names["mean"]} <= seen and len(seen) >= 5, (seen, names)
+    for node, data in got.items():
+        o = origin[node]
+        want = np.asarray(val[o], dtype=np.float32).reshape(-1)
+        g32 = nm.from_storage(data, by_id[o]["dtype"], want.shape).reshape(-1)
+        assert np.allclose(g32, want, rtol=1e-4, atol=1e-4 * np.abs(want).max()), (o, g32[:4], want[:4])
