@@ -4,6 +4,7 @@
 #include <algorithm>
 #include <atomic>
 #include <cstring>
+#include <functional>
 #include <future>
 #include <set>
 
@@ -321,6 +322,102 @@ bool fan_out_pays(const plan::Step& step, const ir::OpGraph& g) {
     const double gain = wide ? narrow_sum : narrow_sum - narrow_max;
     return gain > 2 * kJoinUs;
 }
+
+// The side stream. A training step ends in many chains that nothing else waits for: a filter gradient, the launch that
+// adds up its partial tiles, the optimizer's update of that filter. On one stream each of them holds up the chain
+// that everything else hangs on (the data gradients); on a second stream they run beside it - matrix-core work under
+// the memory-bound kernels of the next layers, and the other way round. The split: the instruction that nothing reads
+// and that the most work leads up to ends the main chain; every instruction it does not depend on, directly or
+// indirectly, may run on the side (no main instruction reads what a side instruction writes, by construction). Small
+// side instructions that read main results only stay on the main stream - a join costs more than they do.
+// HELIUM_HIP_SIDE_STREAM=0 switches the side stream off, =1 on for plans of any size.
+void side_stream_split(Prepared* pr) {
+    const char* env = tuning::get("HELIUM_HIP_SIDE_STREAM");
+    if (env && atoi(env) == 0) return;
+    const bool forced = env && atoi(env) != 0;
+    for (uint8_t f : pr->fan_out)
+        if (f) return;  // a plan whose steps fan out keeps to that scheme
+    Prepared::Side S;
+    for (auto& step : pr->plan->steps)
+        for (auto& instr : step.instrs)
+            if (!instr->absorbed()) {
+                S.index[instr.get()] = S.order.size();
+                S.order.push_back(instr.get());
+            }
+    const size_t n = S.order.size();
+    if (n < 3) return;
+    const ir::OpGraph& g = *pr->graph;
+    auto bytes_of = [&](NodeId id) { return (double)storage_bytes(g.get(id).desc.dtype, (size_t)ir::num_elements(g.get(id).desc.shape)); };
+    constexpr double kLaunchUs = 4, kBytesPerUs = 2e6, kWorthUs = 200;
+    const double kSmallUs = tuning::get("HELIUM_HIP_SIDE_SMALL_US") ? atof(tuning::get("HELIUM_HIP_SIDE_SMALL_US")) : 10;
+    std::map<NodeId, uint32_t> made_by;
+    std::vector<double> cost(n);
+    S.deps.resize(n);
+    S.dependents.resize(n);
+    for (size_t i = 0; i < n; i++) {
+        double bytes = 0;
+        std::set<uint32_t> from;
+        for (NodeId in : S.order[i]->all_inputs()) {
+            bytes += bytes_of(in);
+            auto it = made_by.find(in);
+            if (it != made_by.end() && it->second != i) from.insert(it->second);
+        }
+        for (uint32_t d : from) {
+            S.deps[i].push_back(d);
+            S.dependents[d].push_back((uint32_t)i);
+        }
+        for (NodeId out : S.order[i]->all_outputs()) {
+            bytes += bytes_of(out);
+            made_by[out] = (uint32_t)i;
+        }
+        cost[i] = kLaunchUs + bytes / kBytesPerUs;
+    }
+    auto ancestors = [&](size_t of) {
+        std::vector<uint8_t> in(n, 0);
+        std::vector<uint32_t> stack{(uint32_t)of};
+        in[of] = 1;
+        while (!stack.empty()) {
+            const uint32_t cur = stack.back();
+            stack.pop_back();
+            for (uint32_t d : S.deps[cur])
+                if (!in[d]) {
+                    in[d] = 1;
+                    stack.push_back(d);
+                }
+        }
+        return in;
+    };
+    std::vector<uint8_t> main_set;
+    double main_cost = -1;
+    for (size_t s = 0; s < n; s++) {
+        if (!S.dependents[s].empty()) continue;
+        std::vector<uint8_t> in = ancestors(s);
+        double c = 0;
+        for (size_t i = 0; i < n; i++)
+            if (in[i]) c += cost[i];
+        if (c >= main_cost) {
+            main_cost = c;
+            main_set.swap(in);
+        }
+    }
+    S.side.assign(n, 0);
+    double side_cost = 0;
+    for (size_t i = 0; i < n; i++) {
+        if (main_set[i]) continue;
+        bool reads_side = false;
+        for (uint32_t d : S.deps[i]) reads_side = reads_side || S.side[d];
+        if (!reads_side && cost[i] < kSmallUs && !forced) continue;  // (deps come earlier in the order: one pass is enough)
+        S.side[i] = 1;
+        side_cost += cost[i];
+    }
+    if (getenv("HELIUM_HIP_PLAN_DEBUG")) {
+        size_t count = 0;
+        for (uint8_t f : S.side) count += f;
+        fprintf(stderr, "[plan] side stream: %zu of %zu launching instructions, about %.0f us beside %.0f us\n", count, n, side_cost, main_cost);
+    }
+    if (side_cost == 0 || (!forced && side_cost < kWorthUs)) return;
+    pr->side = std::move(S);
+}
 }  // namespace
 
 void set_stream_fan_out(int mode) {
@@ -351,6 +448,7 @@ std::shared_ptr<const Prepared> prepare(const ir::OpGraph& graph_in) {
         for (NodeId r : step.tensors_to_release) pr->alive.erase(r);
         pr->fan_out.push_back(fan_out_pays(step, *pr->graph));
     }
+    side_stream_split(pr.get());
     if (getenv("HELIUM_HIP_PLAN_DEBUG")) {
         size_t fanned = 0, multi = 0;
         for (size_t k = 0; k < pr->plan->steps.size(); k++) {
@@ -431,6 +529,19 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
         }
         if (!one_stream || getenv("HELIUM_HIP_NO_LAUNCH_EVENTS")) closing = nullptr;
     }
+    // The side stream (side_stream_split): stream 1 runs the chains that nothing on the main stream waits for.
+    const Prepared::Side& S = prepared.side;
+    const bool side_mode = fan_mode == 1 && !S.side.empty() && st.s.size() >= 2;
+    // (the end event follows the join of the two streams: the last launch carries it only if it runs on the main stream)
+    if (side_mode && (getenv("HELIUM_HIP_NO_LAUNCH_EVENTS") || S.side.back())) closing = nullptr;
+    if (side_mode && !getenv("HELIUM_HIP_NO_LAUNCH_EVENTS") && !S.side.back()) closing = S.order.back();
+    std::vector<uint8_t> issued(side_mode ? S.order.size() : 0, 0);
+    std::vector<TensorRef> held;           // what side instructions touch stays allocated until the streams have joined
+    std::set<const Tensor*> synced_side;   // input tensors whose ready event the side stream waited on
+    bool main_dirty = false;               // the main stream has taken work since the side stream last waited for it
+    bool side_joined = false;              // the main stream has waited for the end of the side stream's work
+    std::vector<EventRef> launch_events;   // completion events of main-stream launches that a side instruction follows
+    bool main_end_known = false;           // ... and whether the last of them marks the main stream's latest launch
     EventRef done = pool.take_event();
     bool done_recorded = false;
     struct InstrTime {
@@ -440,6 +551,99 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
         size_t order;  // position in the execution
     };
     std::vector<InstrTime> instr_times;
+    static const int instr_timing = getenv("HELIUM_HIP_INSTR_TIMING") ? atoi(getenv("HELIUM_HIP_INSTR_TIMING")) : 0;
+    // One instruction on stream `w` of the thread's pool: storage for what it writes, waits for inputs made outside
+    // this execution, its launches.
+    auto run_instr = [&](const plan::Instr& instr, size_t w, bool on_side, std::vector<const Tensor*>& waited) {
+        hipStream_t stream = st.s[w];
+        // a stream's first work of this execution comes after the end of the thread's previous execution
+        // (stream 0 carried that end itself)
+        if (used_streams.insert(w).second && w != 0 && st.has_run)
+            HE_HIP(hipStreamWaitEvent(stream, st.exec_end->e, 0));
+        for (NodeId out : instr.all_outputs()) {
+            const ir::Descriptor& d = graph->get(out).desc;
+            tensors[out] = allocate_tensor(d.dtype, (size_t)ir::num_elements(d.shape), scope);
+        }
+        for (NodeId in : instr.all_inputs()) {
+            auto it = tensors.find(in);
+            HE_REQUIRE(it != tensors.end(), HE_ERR_INTERNAL, "missing storage for node %u", in);
+            // tensors made outside this execution carry a ready event (uploads, earlier graphs); a wait of the main
+            // stream also covers the side stream, which waits for the main stream before every instruction it takes
+            if (inputs.count(in) && !synced.count(it->second.get()) && !(on_side && synced_side.count(it->second.get()))) {
+                Tensor& t = *it->second;
+                // a producer seen finished once stays finished: no wait is queued for it again
+                if (t.ready && !t.ready_seen.load(std::memory_order_acquire)) {
+                    if (hipEventQuery(t.ready->e) == hipSuccess) {
+                        t.ready_seen.store(true, std::memory_order_release);
+                    } else {
+                        HE_HIP(hipStreamWaitEvent(stream, t.ready->e, 0));
+                        local.event_waits++;
+                    }
+                }
+                waited.push_back(it->second.get());
+            }
+        }
+        ht.lap(3);
+        if (&instr == closing) set_pending_stop_event(done->e);
+        // HELIUM_HIP_INSTR_TIMING=<n>: every instruction is timed on its own (the device is drained before and after
+        // it), and the n slowest of the execution are listed with the bytes they read and write. A debugging aid:
+        // the execution is serialised while it is on.
+        std::chrono::steady_clock::time_point t_instr;
+        if (instr_timing) {
+            HE_HIP(hipDeviceSynchronize());
+            t_instr = std::chrono::steady_clock::now();
+        }
+        try {
+            instr.execute([&](NodeId n) -> void* { return tensors.at(n)->ptr; }, stream);
+        } catch (...) {
+            (void)take_pending_stop_event();
+            throw;
+        }
+        if (instr_timing) {
+            HE_HIP(hipDeviceSynchronize());
+            const double us = std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t_instr).count();
+            int64_t bytes = 0;
+            for (NodeId n : instr.all_inputs()) bytes += (int64_t)tensors.at(n)->bytes;
+            for (NodeId n : instr.all_outputs()) bytes += (int64_t)tensors.at(n)->bytes;
+            instr_times.push_back({us, bytes, &instr, instr_times.size()});
+        }
+        // taken by the instruction's last launch, or still pending (a launch too large for that entry point)
+        if (&instr == closing) done_recorded = take_pending_stop_event() == nullptr;
+        ht.lap(4);
+        local.instrs++;
+    };
+    // A side instruction waits for everything the main stream has taken so far: for the results it reads, and because
+    // the blocks it is given may have been freed by the main stream just now. What it touches is held until the
+    // streams join, so the main stream is never handed a block the side stream still uses. The side instructions that
+    // read its results alone follow at once (a filter gradient's update), which saves them a wait of their own.
+    std::function<void(size_t)> issue_side = [&](size_t idx) {
+        const plan::Instr& instr = *S.order[idx];
+        if (main_dirty) {
+            hipEvent_t e;
+            if (main_end_known) {
+                e = launch_events.back()->e;
+            } else {
+                HE_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+                events.push_back(e);
+                HE_HIP(hipEventRecord(e, st.s[0]));
+            }
+            HE_HIP(hipStreamWaitEvent(st.s[1], e, 0));
+            local.event_waits++;
+            main_dirty = false;
+        }
+        std::vector<const Tensor*> waited_side;
+        run_instr(instr, 1, true, waited_side);
+        synced_side.insert(waited_side.begin(), waited_side.end());
+        for (NodeId n : instr.all_inputs()) held.push_back(tensors.at(n));
+        for (NodeId n : instr.all_outputs()) held.push_back(tensors.at(n));
+        issued[idx] = 1;
+        for (uint32_t d : S.dependents[idx]) {
+            if (issued[d] || !S.side[d]) continue;
+            bool ready = true;
+            for (uint32_t dep : S.deps[d]) ready = ready && issued[dep];
+            if (ready) issue_side(d);
+        }
+    };
     // Whatever happens below, the scope must end, and only after the work already queued: a failing instruction leaves
     // earlier launches running on up to four streams. On failure stream 0 is ordered after every stream this execution
     // used, the end event is recorded there as usual, and the error goes on to the caller.
@@ -460,62 +664,38 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
         for (size_t i = 0; i < step.instrs.size(); i++) {
             const plan::Instr& instr = *step.instrs[i];
             if (instr.absorbed()) continue;  // run, and its outputs allocated, by the instruction that carries it
-            hipStream_t stream = st.s[i % width];
-            // a stream's first work of this execution comes after the end of the thread's previous execution
-            // (stream 0 carried that end itself)
-            if (used_streams.insert(i % width).second && i % width != 0 && st.has_run)
-                HE_HIP(hipStreamWaitEvent(stream, st.exec_end->e, 0));
-            for (NodeId out : instr.all_outputs()) {
-                const ir::Descriptor& d = graph->get(out).desc;
-                tensors[out] = allocate_tensor(d.dtype, (size_t)ir::num_elements(d.shape), scope);
-            }
-            for (NodeId in : instr.all_inputs()) {
-                auto it = tensors.find(in);
-                HE_REQUIRE(it != tensors.end(), HE_ERR_INTERNAL, "missing storage for node %u", in);
-                // tensors made outside this execution carry a ready event (uploads, earlier graphs)
-                if (inputs.count(in) && !synced.count(it->second.get())) {
-                    Tensor& t = *it->second;
-                    // a producer seen finished once stays finished: no wait is queued for it again
-                    if (t.ready && !t.ready_seen.load(std::memory_order_acquire)) {
-                        if (hipEventQuery(t.ready->e) == hipSuccess) {
-                            t.ready_seen.store(true, std::memory_order_release);
-                        } else {
-                            HE_HIP(hipStreamWaitEvent(stream, t.ready->e, 0));
-                            local.event_waits++;
-                        }
+            if (side_mode) {
+                const size_t idx = S.index.at(&instr);
+                if (issued[idx]) continue;  // went out early, behind the side instruction it reads
+                if (S.side[idx]) {
+                    issue_side(idx);
+                    continue;
+                }
+                issued[idx] = 1;
+                main_dirty = true;
+                main_end_known = false;
+                if (&instr == closing) {
+                    if (used_streams.count(1)) {
+                        prev_streams = {1};
+                        join({0});
+                        prev_streams = {0};
                     }
-                    waited.push_back(it->second.get());
+                    side_joined = true;
+                } else if (!instr_timing && !getenv("HELIUM_HIP_NO_LAUNCH_EVENTS")) {
+                    // when a side instruction comes next, this instruction's last launch carries the event it will wait
+                    // for, which saves the main stream a record of its own
+                    size_t next = idx + 1;
+                    while (next < issued.size() && issued[next]) next++;
+                    if (next < issued.size() && S.side[next]) {
+                        launch_events.push_back(pool.take_event());
+                        set_pending_stop_event(launch_events.back()->e);
+                        run_instr(instr, i % width, false, waited);
+                        main_end_known = take_pending_stop_event() == nullptr;
+                        continue;
+                    }
                 }
             }
-            ht.lap(3);
-            if (&instr == closing) set_pending_stop_event(done->e);
-            // HELIUM_HIP_INSTR_TIMING=<n>: every instruction is timed on its own (the device is drained before and after
-            // it), and the n slowest of the execution are listed with the bytes they read and write. A debugging aid:
-            // the execution is serialised while it is on.
-            static const int instr_timing = getenv("HELIUM_HIP_INSTR_TIMING") ? atoi(getenv("HELIUM_HIP_INSTR_TIMING")) : 0;
-            std::chrono::steady_clock::time_point t_instr;
-            if (instr_timing) {
-                HE_HIP(hipDeviceSynchronize());
-                t_instr = std::chrono::steady_clock::now();
-            }
-            try {
-                instr.execute([&](NodeId n) -> void* { return tensors.at(n)->ptr; }, stream);
-            } catch (...) {
-                (void)take_pending_stop_event();
-                throw;
-            }
-            if (instr_timing) {
-                HE_HIP(hipDeviceSynchronize());
-                const double us = std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t_instr).count();
-                int64_t bytes = 0;
-                for (NodeId n : instr.all_inputs()) bytes += (int64_t)tensors.at(n)->bytes;
-                for (NodeId n : instr.all_outputs()) bytes += (int64_t)tensors.at(n)->bytes;
-                instr_times.push_back({us, bytes, &instr, instr_times.size()});
-            }
-            // taken by the instruction's last launch, or still pending (a launch too large for that entry point)
-            if (&instr == closing) done_recorded = take_pending_stop_event() == nullptr;
-            ht.lap(4);
-            local.instrs++;
+            run_instr(instr, i % width, false, waited);
         }
         // every stream of the next steps is ordered after this step's streams, so one wait per tensor is enough
         synced.insert(waited.begin(), waited.end());
@@ -537,6 +717,7 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
         throw;
     }
     ht.lap(3);
+    if (side_mode && used_streams.count(1) && !side_joined) prev_streams = {0, 1};
     // Drop of the executor (cuda.rs:232-260): when everything queued above has run, the scope's freed blocks
     // become available to everyone. Stream 0 joins the last step and carries the event the pool polls.
     join({0});

@@ -114,6 +114,14 @@ struct Prepared {
     // of the caller's, and the caller's Output node for each of its own. Empty when the ids are the caller's.
     std::map<NodeId, NodeId> input_of, caller_output;
     std::vector<uint8_t> fan_out;  // per step of the plan: whether its instructions are worth a stream each
+    // The side stream (see side_stream_split in exec.cpp): the instructions that launch something, in plan order, which of
+    // them run beside the main chain, and who reads whose results. `side` is empty when nothing runs on the side.
+    struct Side {
+        std::vector<const plan::Instr*> order;
+        std::map<const plan::Instr*, size_t> index;
+        std::vector<uint8_t> side;
+        std::vector<std::vector<uint32_t>> deps, dependents;
+    } side;
 };
 // 0: every instruction runs on one stream; 1 (default): the instructions of a step fan out over the thread's streams
 // where the work that can overlap outweighs the joins; 2: every step with several instructions fans out, as

@@ -23,7 +23,11 @@ pytestmark = pytest.mark.gpu
 BATCH, IMAGE, WIDTH, CLASSES = 8, 64, 8, 16
 
 
-def _run(dtype, fan_out=1):
+def _run(dtype, fan_out=1, side=False):
+    """fan_out: the executor's stream option; side: the chains nothing waits for go to a second stream whatever their
+    size (at the size of this test the executor would not bother)."""
+    import os
+
     from helium_amd.backend import OPT_STREAM_FAN_OUT, set_option, stats
 
     r = resnet.record_training_step(BATCH, IMAGE, width=WIDTH, num_classes=CLASSES, dtype=dtype)
@@ -31,11 +35,19 @@ def _run(dtype, fan_out=1):
     by_id = {n["id"]: n for n in G.g.nodes}
     tensors = {i: Tensor.from_numpy(a, by_id[i]["dtype"], int(np.prod(by_id[i]["shape"]))) for i, a in G.feeds.items()}
     set_option(OPT_STREAM_FAN_OUT, fan_out)
+    before = os.environ.get("HELIUM_HIP_SIDE_STREAM")
+    os.environ["HELIUM_HIP_SIDE_STREAM"] = "1" if side else "0"
     try:
-        got = {o: t.to_numpy() for o, t in execute_graph(G.g, tensors).items()}
-        assert (stats()["streams_used"] > 1) == (fan_out == 2)
+        for _ in range(2 if side else 1):  # (twice: the second execution's side stream starts behind the first one's end)
+            got = {o: t.to_numpy() for o, t in execute_graph(G.g, tensors).items()}
+            used = stats()["streams_used"]
+            assert used == 2 if side else used > 1 if fan_out == 2 else used == 1, used
     finally:
         set_option(OPT_STREAM_FAN_OUT, 1)
+        if before is None:
+            del os.environ["HELIUM_HIP_SIDE_STREAM"]
+        else:
+            os.environ["HELIUM_HIP_SIDE_STREAM"] = before
     # the executor plans the pruned graph: the oracle follows the plan of the same
     G.g.optimize()
     steps = Plan(G.g).steps
@@ -68,9 +80,10 @@ def _rel(a, b):
     return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
 
 
-@pytest.mark.parametrize("fan_out", [1, 2], ids=["streams_where_they_pay", "a_stream_per_instruction_of_a_step"])
-def test_training_step_in_f32_matches_the_oracle_everywhere(gpu, fan_out):
-    r, got, steps = _run("f32", fan_out)
+@pytest.mark.parametrize("fan_out,side", [(1, False), (2, False), (1, True)],
+                         ids=["one_stream", "a_stream_per_instruction_of_a_step", "side_stream"])
+def test_training_step_in_f32_matches_the_oracle_everywhere(gpu, fan_out, side):
+    r, got, steps = _run("f32", fan_out, side)
     G = r["graph"]
     want = oracle_ir.plan_outputs(G.g.nodes, G.feeds, steps)
     _, desc = oracle_ir.evaluate(G.g.nodes, G.feeds)
