@@ -627,6 +627,15 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
         while (RPT < (tall ? 32 : 16) && blocks1 / (RPT * 2) >= (tall ? 512 : 2048) &&
                (!tall || row_bytes * TY * RPT * 2 <= (256 << 10)))
             RPT *= 2;
+        // A column reduction over few rows (a mean over the 7x7 pixels of a pooled image): when one more doubling or two
+        // let a block span all of them and a block per CU is still left, no partial results are written and no second
+        // launch folds them.
+        if (any_col && !any_scalar)
+            for (int r = RPT * 2; r <= 32; r *= 2)
+                if ((int64_t)TY * r >= M) {
+                    if ((int64_t)TY * RPT < M && gx * B >= 256 && row_bytes * TY * r <= (256 << 10)) RPT = r;
+                    break;
+                }
     }
     RPT = (int)std::min<int64_t>(RPT, std::max<int64_t>(1, gy1));
     const int TR = TY * RPT;
@@ -715,6 +724,14 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
     s << ") {\n";
     if (any_col && TY > 1) s << "__shared__ float col_red[TY * TX * NV];\n";
     if (any_scalar) s << "__shared__ float blk_red[" << threads / 64 << "];\n";
+    // rows that one block spans with two or four waves: the waves' parts of a row meet in LDS (two sets taking turns, so
+    // one barrier per row is enough), and no atomics - and no fill launch ahead of the kernel - are needed
+    const bool rows_meet_in_lds = gx == 1 && TX > 64 && !tuning::get("HELIUM_HIP_NO_ROW_LDS");
+    if (rows_meet_in_lds) {
+        size_t row_outs = 0;
+        for (auto& o : p.outs) row_outs += o.reduce && o.fold_n && !o.fold_m;
+        if (row_outs) s << "__shared__ float row_red[" << row_outs << "][2][" << threads / 64 << "];\n";
+    }
     if (any_ticket) s << "__shared__ u32 ticket_s[" << p.outs.size() << "];\n";
     s << "u32 t = blockIdx.x;\nconst u32 tile_x = t % " << gx << "u; t /= " << gx << "u;\nconst u32 tile_y = t % " << gy
       << "u; t /= " << gy << "u;\nconst u32 b = t;\n";
@@ -812,6 +829,7 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
     }
     s << "}\n";  // if (ok)
     // per-row reductions: every lane takes part in the butterfly
+    size_t row_out = 0;
     for (size_t oi = 0; oi < p.outs.size(); oi++) {
         const Out& o = p.outs[oi];
         if (!(o.reduce && o.fold_n && !o.fold_m)) continue;
@@ -819,7 +837,14 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
         s << "{ float r = wave_reduce<" << (int)o.rop << ", " << width << ">(rr" << oi << ");\n";
         if (gx == 1 && TX <= 64)  // one wave segment holds the whole row
             s << "if ((threadIdx.x % " << width << ") == 0 && m < DIM_M && col_ok) a" << o.arg << "[(size_t)b * " << M << "ull + m] = " << scaled(o, "r") << "; }\n";
-        else
+        else if (rows_meet_in_lds) {
+            // (lanes past the row's end hold the identity; the row's first lane is in range whenever the row is)
+            s << "if ((threadIdx.x & 63u) == 0) row_red[" << row_out << "][i & 1u][threadIdx.x >> 6] = r;\n__syncthreads();\n"
+              << "if ((threadIdx.x % " << TX << "u) == 0 && m < DIM_M) {\nfloat acc = r;\nfor (u32 w = 1; w < " << TX / 64
+              << "u; w++) acc = red_op<" << (int)o.rop << ">(acc, row_red[" << row_out << "][i & 1u][(threadIdx.x >> 6) + w]);\na" << o.arg << "[(size_t)b * "
+              << M << "ull + m] = " << scaled(o, "acc") << ";\n} }\n";
+            row_out++;
+        } else
             s << "if ((threadIdx.x % " << width << ") == 0 && m < DIM_M && col_ok) atomic_red<" << (int)o.rop << ">(a" << o.arg
               << " + (size_t)b * " << M << "ull + m, " << scaled(o, "r") << "); }\n";
     }
@@ -1115,7 +1140,7 @@ PointwiseLaunch emit_pointwise(const Program& p, const std::string& entry) {
         const Out& o = p.outs[oi];
         if (o.reduce) {
             // rows wider than a block accumulate with atomics, from the operator's identity
-            if (!(o.fold_n && !o.fold_m) || (gx == 1 && TX <= 64)) continue;
+            if (!(o.fold_n && !o.fold_m) || (gx == 1 && TX <= 64) || rows_meet_in_lds) continue;
             uint32_t bits = 0;
             float f = o.rop == ROp::Max ? -INFINITY : o.rop == ROp::Min ? INFINITY : 0.0f;
             memcpy(&bits, &f, 4);

@@ -23,6 +23,7 @@ class Case:
         self.reduce_rel = None
         self.admitted_by_fusion_rule = True
         self.env = {}  # environment overrides the kernel is generated under
+        self.describes = None  # text the kernel's description has to hold
 
     def inp(self, shape, dtype, values):
         i = self.g.new_input(list(shape), dtype)
@@ -314,6 +315,23 @@ def generated_cases():
     c.out(c.op(c.g.reduce(c.op(c.g.swap_dims(t, 0, 1)), "sum", 1)))
     c.out(c.op(c.g.reduce(c.op(c.g.swap_dims(c.op(c.g.binary(t, xh, "mul")), 0, 1)), "sum", 1)))
     c.reduce_rel = 1e-3; cases.append(c)
+
+    # A mean over few rows per batch entry (global average pooling: 7 x 7 pixels per image and channel): a block spans
+    # all 49 rows, so the kernel writes the means itself - no partial results, no second launch.
+    c = Case("pooling_rows_fit_one_block"); c.env = FOLD_SMALL
+    x = c.inp([64, 49, 1000], "f32", rng.standard_normal(64 * 49 * 1000))
+    c.out(c.op(c.g.reduce(c.op(c.g.swap_dims(x, 1, 2)), "mean", 1))); c.reduce_rel = 1e-3
+    c.describes = "grid=256 threads=256 exprs=1 outs=1 ws_floats=0 ws_counters=0 finalize_grid=0"; cases.append(c)
+
+    # Rows that a block spans with four (two) waves: the waves' parts of a row meet in LDS, nothing is accumulated with
+    # atomics and nothing has to be filled ahead of the launch (a softmax over 1000 classes).
+    for rows, cols, tx in ((37, 1000, 256), (9, 500, 128)):
+        c = Case(f"rows_spanning_{tx // 64}_waves")
+        x = c.inp([rows, cols], "f32", rng.standard_normal(rows * cols))
+        c.out(c.op(c.g.reduce(x, "max", 1)))
+        c.out(c.op(c.g.reduce(c.op(c.g.unary(x, "exp")), "sum", 1))); c.reduce_rel = 1e-4
+        c.describes = f" TX={tx} TY={256 // tx} RPT=1 grid={(rows + 256 // tx - 1) // (256 // tx)} threads=256 exprs=2 outs=2 ws_floats=0 ws_counters=0 finalize_grid=0 fills=[]"
+        cases.append(c)
 
     return cases
 

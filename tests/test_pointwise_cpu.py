@@ -43,6 +43,7 @@ def test_generated_kernel_on_cpu_matches_oracle(case, monkeypatch):
     assert ha.kernels.pointwise_supports(case.g, case.nodes), case.name
     kernel = ha.TileKernel.pointwise(case.g, case.nodes)
     assert [a["node"] for a in kernel.args if a["is_output"]] == sorted(case.leaves)
+    assert case.describes is None or case.describes in kernel.description, kernel.description
     want = oracle_ir.kernel_outputs(case.g.nodes, case.inputs, case.leaves)
     got = run_tile_kernel_cpu(kernel, case.inputs, "pointwise_kernel", reduction_fills(case.g.nodes, case.leaves))
     by_id = {n["id"]: n for n in case.g.nodes}
