@@ -156,3 +156,36 @@ def test_training_step_at_full_size_has_the_invariants_of_a_first_step(gpu, batc
             assert (v > 0.85).all() and (v < 2.0).all(), (mi, v.min(), v.max())   # 0.9 * 1 + 0.1 * batch variance
         if kind == "mean":
             assert np.abs(v).max() < 1.0, (mi,)
+
+
+def test_two_threads_with_side_streams_give_what_one_stream_gives(gpu, monkeypatch):
+    """Each host thread has its own pair of streams; blocks of the device pool go round between the threads. The step's
+    kernels are the same whichever stream they run on, so every output is bit for bit what one stream gives."""
+    import threading
+
+    def tensors_of(G):
+        by_id = {n["id"]: n for n in G.g.nodes}
+        return {i: Tensor.from_numpy(a, by_id[i]["dtype"], int(np.prod(by_id[i]["shape"]))) for i, a in G.feeds.items()}
+
+    monkeypatch.setenv("HELIUM_HIP_SIDE_STREAM", "0")
+    G = resnet.record_training_step(BATCH, IMAGE, width=WIDTH, num_classes=CLASSES, dtype="f32")["graph"]
+    ref = {o: t.to_numpy() for o, t in execute_graph(G.g, tensors_of(G)).items()}
+    monkeypatch.setenv("HELIUM_HIP_SIDE_STREAM", "1")
+    S = resnet.record_training_step(BATCH, IMAGE, width=WIDTH, num_classes=CLASSES, dtype="f32")["graph"]  # (a handle keeps its plan)
+    errors = []
+
+    def worker():
+        try:
+            tensors = tensors_of(S)
+            for _ in range(4):
+                got = {o: t.to_numpy() for o, t in execute_graph(S.g, tensors).items()}
+                assert sorted(got) == sorted(ref)
+                for o in ref:
+                    assert np.array_equal(got[o], ref[o]), o
+        except BaseException as e:  # noqa: BLE001 - reported by the test's own thread
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker) for _ in range(2)]
+    [t.start() for t in threads]
+    [t.join() for t in threads]
+    assert not errors, errors[0]
