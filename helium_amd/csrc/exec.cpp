@@ -406,10 +406,31 @@ void side_stream_split(Prepared* pr) {
         S.side[i] = 1;
         side_cost += cost[i];
     }
+    // Early instructions (side value 2): small main-chain instructions that read nothing but the graph's inputs (or each
+    // other) - a filter converted to the multiplicands' type ahead of its convolution - and whose first reader comes
+    // well into the execution. Each would hold the main stream for a launch's latency; the side stream runs them all at
+    // the start instead, and the main stream waits for them once, ahead of the first instruction that reads one.
+    size_t early = 0;
+    if (!tuning::get("HELIUM_HIP_NO_EARLY_INSTRS")) {
+        constexpr double kEarlyUs = 20, kLeadUs = 100;
+        std::vector<double> before(n + 1, 0);  // main-stream work ahead of each position
+        for (size_t i = 0; i < n; i++) before[i + 1] = before[i] + (S.side[i] ? 0 : cost[i]);
+        for (size_t i = 0; i < n; i++) {
+            if (S.side[i] || cost[i] >= kEarlyUs || S.dependents[i].empty()) continue;
+            bool sources_only = true;
+            for (uint32_t d : S.deps[i]) sources_only = sources_only && S.side[d] == 2;
+            uint32_t first_reader = (uint32_t)n;
+            for (uint32_t d : S.dependents[i]) first_reader = std::min(first_reader, d);
+            if (!sources_only || (!forced && before[first_reader] < kLeadUs)) continue;
+            S.side[i] = 2;
+            early++;
+        }
+    }
     if (getenv("HELIUM_HIP_PLAN_DEBUG")) {
         size_t count = 0;
-        for (uint8_t f : S.side) count += f;
-        fprintf(stderr, "[plan] side stream: %zu of %zu launching instructions, about %.0f us beside %.0f us\n", count, n, side_cost, main_cost);
+        for (uint8_t f : S.side) count += f == 1;
+        fprintf(stderr, "[plan] side stream: %zu of %zu launching instructions, about %.0f us beside %.0f us; %zu early instructions\n", count, n, side_cost,
+                main_cost, early);
     }
     if (side_cost == 0 || (!forced && side_cost < kWorthUs)) return;
     pr->side = std::move(S);
@@ -634,7 +655,7 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
         for (NodeId n : instr.all_outputs()) held.push_back(tensors.at(n));
         issued[idx] = 1;
         for (uint32_t d : S.dependents[idx]) {
-            if (issued[d] || !S.side[d]) continue;
+            if (issued[d] || S.side[d] != 1) continue;
             bool ready = true;
             for (uint32_t dep : S.deps[d]) ready = ready && issued[dep];
             if (ready) issue_side(d);
@@ -643,7 +664,21 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
     // Whatever happens below, the scope must end, and only after the work already queued: a failing instruction leaves
     // earlier launches running on up to four streams. On failure stream 0 is ordered after every stream this execution
     // used, the end event is recorded there as usual, and the error goes on to the caller.
+    EventRef early_done;  // the early instructions' end on the side stream, until the main stream has waited for it
     try {
+    if (side_mode && !instr_timing) {
+        for (size_t idx = 0; idx < S.order.size(); idx++) {
+            if (S.side[idx] != 2) continue;
+            std::vector<const Tensor*> waited_side;
+            run_instr(*S.order[idx], 1, true, waited_side);
+            synced_side.insert(waited_side.begin(), waited_side.end());
+            for (NodeId n : S.order[idx]->all_inputs()) held.push_back(tensors.at(n));
+            for (NodeId n : S.order[idx]->all_outputs()) held.push_back(tensors.at(n));
+            issued[idx] = 1;
+            if (!early_done) early_done = pool.take_event();
+        }
+        if (early_done) HE_HIP(hipEventRecord(early_done->e, st.s[1]));
+    }
     for (size_t step_no = 0; step_no < plan->steps.size(); step_no++) {
         auto& step = plan->steps[step_no];
         for (NodeId r : step.tensors_to_release) tensors.erase(r);
@@ -663,11 +698,20 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
             if (side_mode) {
                 const size_t idx = S.index.at(&instr);
                 if (issued[idx]) continue;  // went out early, behind the side instruction it reads
-                if (S.side[idx]) {
+                if (S.side[idx] == 1) {
                     issue_side(idx);
                     continue;
                 }
-                issued[idx] = 1;
+                issued[idx] = 1;  // (an early instruction left for here - under instruction timing - runs on the main stream)
+                if (early_done) {
+                    bool reads_early = false;
+                    for (uint32_t d : S.deps[idx]) reads_early = reads_early || S.side[d] == 2;
+                    if (reads_early) {
+                        HE_HIP(hipStreamWaitEvent(st.s[0], early_done->e, 0));
+                        local.event_waits++;
+                        early_done.reset();
+                    }
+                }
                 main_dirty = true;
                 main_end_known = false;
                 if (&instr == closing) {
@@ -682,7 +726,7 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
                     // for, which saves the main stream a record of its own
                     size_t next = idx + 1;
                     while (next < issued.size() && issued[next]) next++;
-                    if (next < issued.size() && S.side[next]) {
+                    if (next < issued.size() && S.side[next] == 1) {
                         launch_events.push_back(pool.take_event());
                         set_pending_stop_event(launch_events.back()->e);
                         run_instr(instr, i % width, false, waited);
