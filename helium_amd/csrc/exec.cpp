@@ -452,12 +452,6 @@ std::shared_ptr<const Prepared> prepare(const ir::OpGraph& graph_in) {
         for (NodeId out : pr->graph->outputs()) pr->caller_output[out] = pr->graph->origin(out);
     }
     pr->plan = plan::generate_cached_plan(pr->graph);
-    // begin_execute (cuda.rs:98-139): compile every kernel of the plan up front, in parallel (cuda.rs:262-270)
-    std::vector<std::future<void>> jobs;
-    for (auto& step : pr->plan->steps)
-        for (auto& instr : step.instrs)
-            if (!instr->compiled()) jobs.push_back(std::async(std::launch::async, [instr] { instr->precompile(); }));
-    for (auto& j : jobs) j.get();
     // tensors that survive the plan get their ready event recorded (enumerate_output_tensors, cuda.rs:142-153)
     for (auto& step : pr->plan->steps) {
         for (auto& instr : step.instrs)
@@ -465,7 +459,16 @@ std::shared_ptr<const Prepared> prepare(const ir::OpGraph& graph_in) {
         for (NodeId r : step.tensors_to_release) pr->alive.erase(r);
         pr->fan_out.push_back(fan_out_pays(step, *pr->graph));
     }
+    // (ahead of the kernels: a product that will run beside the main chain is built for that)
     side_stream_split(pr.get());
+    for (size_t i = 0; i < pr->side.order.size(); i++)
+        if (pr->side.side[i] == 1 && pr->side.order[i]->kind() == plan::InstrKind::Gemm) pr->side.order[i]->runs_beside_main_chain();
+    // begin_execute (cuda.rs:98-139): compile every kernel of the plan up front, in parallel (cuda.rs:262-270)
+    std::vector<std::future<void>> jobs;
+    for (auto& step : pr->plan->steps)
+        for (auto& instr : step.instrs)
+            if (!instr->compiled()) jobs.push_back(std::async(std::launch::async, [instr] { instr->precompile(); }));
+    for (auto& j : jobs) j.get();
     if (getenv("HELIUM_HIP_PLAN_DEBUG")) {
         size_t fanned = 0, multi = 0;
         for (size_t k = 0; k < pr->plan->steps.size(); k++) {

@@ -45,7 +45,7 @@ bool enumerate_swaps(const ir::OpSubgraph& sg, std::vector<std::pair<int, int>>*
     return true;
 }
 
-std::unique_ptr<KernelBase> make_gemm_kernel(const ir::OpSubgraph& sg, const ir::OpSubgraph* carried);
+std::unique_ptr<KernelBase> make_gemm_kernel(const ir::OpSubgraph& sg, const ir::OpSubgraph* carried, bool beside_main_chain);
 bool gemm_can_carry(const ir::OpSubgraph& large, const ir::OpSubgraph& small);
 namespace {
 std::atomic<bool> g_fuse_matmul_epilogue{true};
@@ -223,8 +223,8 @@ void Instr::precompile() const {
             break;
         case InstrKind::Gemm:
             kernel_ = g_tile_kernels.get_or_insert(
-                tuning::key() + "mm:" + sg_.cache_key() + (carried_ ? "+carries:" + carried_->sg_.cache_key() : std::string()),
-                [&] { return std::shared_ptr<KernelBase>(make_gemm_kernel(sg_, carried_ ? &carried_->sg_ : nullptr)); });
+                tuning::key() + (beside_main_chain() ? "mm-beside:" : "mm:") + sg_.cache_key() + (carried_ ? "+carries:" + carried_->sg_.cache_key() : std::string()),
+                [&] { return std::shared_ptr<KernelBase>(make_gemm_kernel(sg_, carried_ ? &carried_->sg_ : nullptr, beside_main_chain())); });
             break;
         case InstrKind::Permute: {
             std::vector<std::pair<int, int>> swaps;
@@ -1175,7 +1175,7 @@ bool gemm_can_carry(const ir::OpSubgraph& large, const ir::OpSubgraph& small) {
     return tp::attach_post(&pr.epi, tp::lower_pointwise(small));
 }
 
-std::unique_ptr<KernelBase> make_gemm_kernel(const ir::OpSubgraph& sg, const ir::OpSubgraph* carried) {
+std::unique_ptr<KernelBase> make_gemm_kernel(const ir::OpSubgraph& sg, const ir::OpSubgraph* carried, bool beside_main_chain) {
     if (carried) {
         GemmProblem pr = gemm_problem_from_ir(sg);
         HE_REQUIRE(tp::attach_post(&pr.epi, tp::lower_pointwise(*carried)), HE_ERR_INTERNAL, "the carried instruction does not fit the fold launch any more");
@@ -1192,6 +1192,15 @@ std::unique_ptr<KernelBase> make_gemm_kernel(const ir::OpSubgraph& sg, const ir:
         return std::unique_ptr<KernelBase>(new CompositeKernel(std::move(parts), any_empty));
     }
     GemmProblem pr = gemm_problem_from_ir(sg);
+    // A filter gradient that runs beside the main chain takes 0.4 of the workgroups it would take alone: four in ten of
+    // the CUs are then busy with it and the main chain's kernels keep the rest, where a launch that fills the chip
+    // holds every main-chain kernel back until its workgroups retire. Measured on the training step at batch 128
+    // (shares of 1 / 0.5 / 0.4 / 0.33 / 0.25 / 0.2: 4.49 / 4.42 / 4.39 / 4.40 / 4.39 / 4.67 ms - below a quarter the side
+    // stream becomes the longer chain); fewer shares also write and re-read fewer partial tiles.
+    if (beside_main_chain && pr.conv_b.on && pr.split_k > 1) {
+        const double share = tuning::get("HELIUM_HIP_SIDE_SPLIT_SCALE") ? atof(tuning::get("HELIUM_HIP_SIDE_SPLIT_SCALE")) : 0.4;
+        pr.split_k = std::max(1, (int)(pr.split_k * share + 0.5));
+    }
     ConvRepack geometry;
     GemmProblem packed;
     if (over_repacked_image(pr, &packed, &geometry)) {

@@ -2,6 +2,7 @@
 // scheduling and tensor lifetimes — helium/src/backend/plan_generation.rs, with the HIP backend's op -> instruction
 // mapping (helium/src/cuda.rs:33-60) and its instruction kinds (helium/src/cuda/instr.rs).
 #pragma once
+#include <atomic>
 #include <functional>
 #include <memory>
 #include <mutex>
@@ -58,12 +59,18 @@ public:
         std::lock_guard<std::mutex> lk(mu_);
         return kernel_;
     }
+    // Beyond the reference: the executor runs this instruction on its side stream, beside the chain of instructions
+    // that everything else waits for (exec.cpp: side_stream_split). Told before the kernel is made, a filter gradient
+    // then splits its k range over fewer workgroups: it has time, and the CUs it leaves alone keep the main chain going.
+    void runs_beside_main_chain() const { beside_main_.store(true); }
+    bool beside_main_chain() const { return beside_main_.load(); }
     std::vector<NodeId> all_inputs() const;   // inputs() plus what the carried instruction reads from elsewhere
     std::vector<NodeId> all_outputs() const;  // outputs() plus the carried instruction's
 
 private:
     std::shared_ptr<Instr> carried_;
     bool absorbed_ = false;
+    mutable std::atomic<bool> beside_main_{false};
     InstrKind kind_;
     ir::OpSubgraph sg_;
     mutable std::shared_ptr<KernelBase> kernel_;   // Gemm / Pointwise
@@ -131,6 +138,6 @@ GemmProblem gemm_problem_from_ir(const ir::OpSubgraph& sg);
 // no tap, so its pixels have to be zeroed.
 std::vector<GemmProblem> strided_data_gradient_classes(const ir::OpSubgraph& sg, bool* any_empty);
 // The kernel of a Gemm instruction: one fused GEMM, or the classes of a strided data gradient one after the other.
-std::unique_ptr<KernelBase> make_gemm_kernel(const ir::OpSubgraph& sg, const ir::OpSubgraph* carried = nullptr);
+std::unique_ptr<KernelBase> make_gemm_kernel(const ir::OpSubgraph& sg, const ir::OpSubgraph* carried = nullptr, bool beside_main_chain = false);
 
 }  // namespace he::plan
