@@ -102,6 +102,13 @@ int he_plan_instruction_kernel(he_plan_t plan, int index, he_tile_kernel_t* kern
 int he_plan_precompile(he_plan_t plan) {
     return he::guard([&] {
         HE_REQUIRE(plan, HE_ERR_INVALID, "bad argument");
+        {
+            // the kernels the executor would run: its assignment of instructions to streams shapes some of them
+            he::exec::Prepared as_executed;
+            as_executed.graph = plan->graph;
+            as_executed.plan = plan->plan;
+            he::exec::assign_streams(&as_executed);
+        }
         std::vector<std::future<void>> jobs;
         for (auto& step : plan->plan->steps)
             for (auto& instr : step.instrs)

@@ -437,6 +437,13 @@ void side_stream_split(Prepared* pr) {
 }
 }  // namespace
 
+void assign_streams(Prepared* pr) {
+    for (auto& step : pr->plan->steps) pr->fan_out.push_back(fan_out_pays(step, *pr->graph));
+    side_stream_split(pr);
+    for (size_t i = 0; i < pr->side.order.size(); i++)
+        if (pr->side.side[i] == 1 && pr->side.order[i]->kind() == plan::InstrKind::Gemm) pr->side.order[i]->runs_beside_main_chain();
+}
+
 void set_stream_fan_out(int mode) {
     HE_REQUIRE(mode >= 0 && mode <= 2, HE_ERR_INVALID, "stream fan-out is 0 (never), 1 (where it pays) or 2 (always)");
     g_fan_out.store(mode);
@@ -457,12 +464,9 @@ std::shared_ptr<const Prepared> prepare(const ir::OpGraph& graph_in) {
         for (auto& instr : step.instrs)
             for (NodeId o : instr->outputs()) pr->alive.insert(o);
         for (NodeId r : step.tensors_to_release) pr->alive.erase(r);
-        pr->fan_out.push_back(fan_out_pays(step, *pr->graph));
     }
     // (ahead of the kernels: a product that will run beside the main chain is built for that)
-    side_stream_split(pr.get());
-    for (size_t i = 0; i < pr->side.order.size(); i++)
-        if (pr->side.side[i] == 1 && pr->side.order[i]->kind() == plan::InstrKind::Gemm) pr->side.order[i]->runs_beside_main_chain();
+    assign_streams(pr.get());
     // begin_execute (cuda.rs:98-139): compile every kernel of the plan up front, in parallel (cuda.rs:262-270)
     std::vector<std::future<void>> jobs;
     for (auto& step : pr->plan->steps)

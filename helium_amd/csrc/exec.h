@@ -127,6 +127,9 @@ struct Prepared {
 // where the work that can overlap outweighs the joins; 2: every step with several instructions fans out, as
 // cuda.rs:190-221 does.
 void set_stream_fan_out(int mode);
+// Which instructions of pr->plan (a plan of pr->graph) run on which stream of an execution; the products that will run
+// beside the main chain are told so (plan::Instr::runs_beside_main_chain), which has to happen before their kernels are made.
+void assign_streams(Prepared* pr);
 std::shared_ptr<const Prepared> prepare(const ir::OpGraph& graph);
 std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std::map<NodeId, TensorRef>& inputs,
                                              ExecStats* stats = nullptr);
