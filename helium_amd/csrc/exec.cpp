@@ -348,7 +348,7 @@ void side_stream_split(Prepared* pr) {
     if (n < 3) return;
     const ir::OpGraph& g = *pr->graph;
     auto bytes_of = [&](NodeId id) { return (double)storage_bytes(g.get(id).desc.dtype, (size_t)ir::num_elements(g.get(id).desc.shape)); };
-    constexpr double kLaunchUs = 4, kBytesPerUs = 2e6, kWorthUs = 200;
+    constexpr double kLaunchUs = 4, kBytesPerUs = 2e6, kWorthUs = 200, kDeviceBoundUs = 14;
     std::map<NodeId, uint32_t> made_by;
     std::vector<double> cost(n);
     S.deps.resize(n);
@@ -433,6 +433,11 @@ void side_stream_split(Prepared* pr) {
                 main_cost, early);
     }
     if (side_cost == 0 || (!forced && side_cost < kWorthUs)) return;
+    // An execution that the host cannot keep ahead of (it needs 8-10 us per launch, and 15-20 more per wait between
+    // streams) gains nothing from a second stream and loses the waits: the training step at batch 4 to 32, where the
+    // estimate is 6 to 11 us of device time per launch, ran up to 1.5x slower with it, at 18 and 26 us per launch (the
+    // reference's size and batch 128) 7-10% faster.
+    if (!forced && (main_cost + side_cost) / (double)n < kDeviceBoundUs) return;
     pr->side = std::move(S);
 }
 }  // namespace
