@@ -348,7 +348,7 @@ void side_stream_split(Prepared* pr) {
     if (n < 3) return;
     const ir::OpGraph& g = *pr->graph;
     auto bytes_of = [&](NodeId id) { return (double)storage_bytes(g.get(id).desc.dtype, (size_t)ir::num_elements(g.get(id).desc.shape)); };
-    constexpr double kLaunchUs = 4, kBytesPerUs = 2e6, kWorthUs = 200, kDeviceBoundUs = 14;
+    constexpr double kLaunchUs = 4, kBytesPerUs = 2e6, kWorthUs = 200, kDeviceBoundUs = 10;
     std::map<NodeId, uint32_t> made_by;
     std::vector<double> cost(n);
     S.deps.resize(n);
@@ -434,9 +434,9 @@ void side_stream_split(Prepared* pr) {
     }
     if (side_cost == 0 || (!forced && side_cost < kWorthUs)) return;
     // An execution that the host cannot keep ahead of (it needs 8-10 us per launch, and 15-20 more per wait between
-    // streams) gains nothing from a second stream and loses the waits: the training step at batch 4 to 32, where the
-    // estimate is 6 to 11 us of device time per launch, ran up to 1.5x slower with it, at 18 and 26 us per launch (the
-    // reference's size and batch 128) 7-10% faster.
+    // streams) gains nothing from a second stream and loses the waits: the training step at batch 4 to 16, where the
+    // estimate is 6 to 8 us of device time per launch, ran up to 1.5x slower with it; at 11 us (batch 32) and above it
+    // gains 7-12%.
     if (!forced && (main_cost + side_cost) / (double)n < kDeviceBoundUs) return;
     pr->side = std::move(S);
 }
@@ -520,6 +520,7 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
     std::set<const Tensor*> synced;        // input tensors whose ready event a stream already waited on
     std::vector<size_t> prev_streams;      // streams the previous step ran on
     std::vector<hipEvent_t> events;        // join events of this execution
+    std::map<size_t, std::set<hipEvent_t>> waited_for;  // per stream: the events it has been made to wait for
     std::set<size_t> used_streams;
     // Every stream in `cur` waits for the end of the previous step on every other stream it ran on. The events are
     // recorded here, before the new step enqueues anything, so they mark exactly the end of that step.
@@ -587,8 +588,10 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
         hipStream_t stream = st.s[w];
         // a stream's first work of this execution comes after the end of the thread's previous execution
         // (stream 0 carried that end itself)
-        if (used_streams.insert(w).second && w != 0 && st.has_run)
+        if (used_streams.insert(w).second && w != 0 && st.has_run) {
             HE_HIP(hipStreamWaitEvent(stream, st.exec_end->e, 0));
+            waited_for[w].insert(st.exec_end->e);
+        }
         for (NodeId out : instr.all_outputs()) {
             const ir::Descriptor& d = graph->get(out).desc;
             tensors[out] = allocate_tensor(d.dtype, (size_t)ir::num_elements(d.shape), scope);
@@ -604,7 +607,9 @@ std::map<NodeId, TensorRef> execute_prepared(const Prepared& prepared, const std
                 if (t.ready && !t.ready_seen.load(std::memory_order_acquire)) {
                     if (hipEventQuery(t.ready->e) == hipSuccess) {
                         t.ready_seen.store(true, std::memory_order_release);
-                    } else {
+                    } else if (waited_for[w].insert(t.ready->e).second) {
+                        // (one wait per event and stream: the tensors a previous execution returned share its end event,
+                        // and a wait costs the host 15-20 us on a stream other than the one that recorded the event)
                         HE_HIP(hipStreamWaitEvent(stream, t.ready->e, 0));
                         local.event_waits++;
                     }
