@@ -333,7 +333,8 @@ std::string OpSubgraph::cache_key() const {
 
 namespace he::ir {
 
-std::shared_ptr<OpGraph> rematerialized(const OpGraph& g, const std::set<NodeId>& keep_single) {
+std::shared_ptr<OpGraph> rematerialized(const OpGraph& g, const std::set<NodeId>& keep_single,
+                                        const std::set<std::vector<NodeId>>& two_sources) {
     const size_t cap = g.capacity();
     // 1. Ops that compute the same thing are one op. The reference's tape records a forward op again when the backward
     //    pass needs its value (tensor/tape.rs:93-158 recomputes from the last checkpoint), so every batch norm's
@@ -425,7 +426,8 @@ std::shared_ptr<OpGraph> rematerialized(const OpGraph& g, const std::set<NodeId>
         I.cost = std::min(I.cost, kMaxCost + 1);
         // (a node with one consumer is copied as well when that consumer is: its copies' inputs must not meet in one
         // shared node, which would then have several consumers and travel through memory after all)
-        I.remat = numel >= kMinElements && I.anchors.size() <= kMaxAnchors && I.cost <= kMaxCost && !keep_single.count(id);
+        I.remat = numel >= kMinElements && (I.anchors.size() <= kMaxAnchors || (I.anchors.size() == 2 && two_sources.count(I.anchors))) &&
+                  I.cost <= kMaxCost && !keep_single.count(id);
         // A value that only reductions read (through transpositions and pointwise ops) may depend on one tensor more:
         // written out and read back it moves as many bytes as its two operands do, and the reductions of one backward
         // pass (a batch norm's four) then share one pass over those operands instead of reading a tensor each.

@@ -126,7 +126,8 @@ private:
     std::vector<std::vector<NodeId>> in_, out_;
     std::vector<NodeId> origin_;
     std::vector<uint8_t> for_consumer_;
-    friend std::shared_ptr<OpGraph> rematerialized(const OpGraph& g, const std::set<NodeId>& keep_single);
+    friend std::shared_ptr<OpGraph> rematerialized(const OpGraph& g, const std::set<NodeId>& keep_single,
+                                                   const std::set<std::vector<NodeId>>& two_sources);
     friend std::shared_ptr<OpGraph> transposes_cancelled(const OpGraph& g);
     friend std::shared_ptr<OpGraph> broadcasts_hoisted(const OpGraph& g);
 };
@@ -141,7 +142,10 @@ private:
 // when the backward pass needs its value). A consumer that reads its operands from memory whatever happens (a product, a
 // large permute, an Output) shares one copy. `keep_single`: nodes of `g` that are not to be duplicated. Node ids are new
 // (in dataflow order); `origin` maps them back to `g`. Returns null when nothing changes.
-std::shared_ptr<OpGraph> rematerialized(const OpGraph& g, const std::set<NodeId>& keep_single = {});
+// `two_sources`: sorted pairs of tensors (nodes of `g`) from which a value may be recomputed by every kernel that uses
+// it, although a value that depends on two tensors of its size is otherwise written once and read back.
+std::shared_ptr<OpGraph> rematerialized(const OpGraph& g, const std::set<NodeId>& keep_single = {},
+                                        const std::set<std::vector<NodeId>>& two_sources = {});
 
 // A copy of `g` without the transpositions that undo each other. The reference's front end writes a reduction over
 // leading dims as SwapDims + Reduce and its gradient rules answer a SwapDims with a SwapDims (tensor.rs), so a recorded

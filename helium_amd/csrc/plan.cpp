@@ -756,6 +756,56 @@ std::shared_ptr<const ir::OpGraph> graph_for_execution(const std::shared_ptr<con
             other = ir::rematerialized(*base, keep_single);
         }
         other = best;  // (a round that takes copies back usually moves fewer bytes, not always)
+        // A value that depends on two tensors of its size is written once and read back - unless the kernel that reads
+        // it reads those two tensors anyway, or all but one of them: then it computes the value itself, the kernel that
+        // made it (a batch norm's backward sums, which need it too) no longer writes it, and a pass or two over a
+        // full-size tensor goes. The plan tells which values those are; the graph is rewritten with their source
+        // pairs admitted, planned again, and kept when it moves fewer bytes.
+        if (other && !tuning::get("HELIUM_HIP_NO_TWO_SOURCE_REMAT")) {
+            std::set<std::vector<ir::NodeId>> two_sources;
+            for (int round = 0; round < 3; round++) {
+                const auto plan = generate_plan(other);
+                const size_t known = two_sources.size();
+                auto large_inputs = [&](const Instr& instr, int64_t numel) {
+                    std::vector<ir::NodeId> v;
+                    for (ir::NodeId in : instr.inputs())
+                        if (ir::num_elements(other->get(in).desc.shape) * 8 >= numel) v.push_back(in);
+                    return v;
+                };
+                std::map<ir::NodeId, std::vector<const Instr*>> readers;
+                for (auto& st : plan->steps)
+                    for (auto& instr : st.instrs)
+                        for (ir::NodeId in : instr->inputs()) readers[in].push_back(instr.get());
+                for (auto& st : plan->steps)
+                    for (auto& maker : st.instrs) {
+                        if (maker->kind() != InstrKind::Pointwise) continue;
+                        for (ir::NodeId x : maker->outputs()) {
+                            const ir::Node& xn = other->get(x);
+                            const int64_t numel = ir::num_elements(xn.desc.shape);
+                            if (numel < (1 << 16) || xn.op.kind == ir::OpKind::Reduce || other->feeds_output(x)) continue;
+                            auto rd = readers.find(x);
+                            if (rd == readers.end() || rd->second.size() != 1 || rd->second[0]->kind() != InstrKind::Pointwise) continue;
+                            std::vector<ir::NodeId> sources = large_inputs(*maker, numel);
+                            if (sources.size() != 2) continue;
+                            const std::vector<ir::NodeId> theirs = large_inputs(*rd->second[0], numel);
+                            int fresh = 0;
+                            for (ir::NodeId s : sources) fresh += std::find(theirs.begin(), theirs.end(), s) == theirs.end();
+                            if (fresh > 1) continue;
+                            std::vector<ir::NodeId> pair{other->origin(sources[0]), other->origin(sources[1])};
+                            std::sort(pair.begin(), pair.end());
+                            two_sources.insert(pair);
+                        }
+                    }
+                if (two_sources.size() == known) break;
+                auto again = ir::rematerialized(*base, keep_single, two_sources);
+                if (!again) break;
+                const int64_t bytes = plan_traffic_bytes(*generate_plan(again));
+                if (debug) fprintf(stderr, "[plan] two-source round %d: %zu pairs, %lld -> %lld bytes\n", round, two_sources.size(), (long long)best_bytes, (long long)bytes);
+                if (bytes >= best_bytes) break;
+                other = again;
+                best_bytes = bytes;
+            }
+        }
     }
     if (!other) return base;
     if (base != g) other->rebase_origins(*base);
